@@ -1,0 +1,233 @@
+#!/usr/bin/env python3
+"""SpMM benchmark: GFLOPS (2*nnz*K / t) and fraction of the HBM-traffic roofline on one MI355X.
+
+One *step* is one pass of the hot path over the benchmark's synthetic inputs:
+one C = A*B for every (graph, K) workload of configurations 1-4
+(citation 20k x {32,64,128}, social 233k x {32,64,128}, co-purchase 2.4M x 64,
+R-MAT scale 22 x 128).  Inputs are generated on the host (seeded), copied to
+HBM once, and every timed region starts with them resident.
+
+    value        geometric mean of the per-workload GFLOPS
+    ms_per_step  sum of the per-workload mean SpMM times
+    roofline     social graph, K=128 (the longest-running launch of a step):
+                 algorithmic bytes 4(M+1) + 8 nnz + 4 K nnz + 4 K M per SpMM
+                 divided by the mean SpMM time, against 8 TB/s
+    cpu_baseline the FP32 CPU oracle on a bounded row sample of the same
+                 social-graph workload, on this machine's host cores
+
+Times are HIP-event times on the stream the kernels are launched on, over
+exactly --steps back-to-back launches after --warmup untimed ones (the
+reference's protocol: include/spmm/utils/timer_cuda.h:3-40,
+spmm/mm/spmm_kernel.cu:404-424; GFLOPS formula spmm/mm/spmm_common.cpp:24-31).
+"""
+import argparse
+import importlib
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = [
+    ("c1_citation", 32), ("c1_citation", 64), ("c1_citation", 128),
+    ("c2_social", 32), ("c2_social", 64), ("c2_social", 128),
+    ("c3_copurchase", 64),
+    ("c4_rmat", 128),
+]
+ROOFLINE_WORKLOAD = ("c2_social", 128)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def algorithmic_bytes(rows, nnz, k):
+    """rowptr + (col, val) stream + B gather counted per nonzero + C write."""
+    return 4 * (rows + 1) + 8 * nnz + 4 * k * nnz + 4 * k * rows
+
+
+def unique_bytes(rows, cols, nnz, k):
+    """Lower bound if every B row were fetched from HBM only once."""
+    return 4 * (rows + 1) + 8 * nnz + 4 * k * cols + 4 * k * rows
+
+
+def ensure_built():
+    pkg_dir = os.path.join(ROOT, "hp-spmm-sddmm_amd")
+    needed = [os.path.join(pkg_dir, "libhpspmm.so"), os.path.join(pkg_dir, "libhpspmm_graphgen.so")]
+    if not all(os.path.exists(p) for p in needed):
+        import __graft_entry__
+        __graft_entry__.build()
+
+
+def cpu_baseline(graphs, g, B, k, C_gpu_host_rows, budget_nnz):
+    """Time the CPU oracle (FP32, OpenMP, all host threads) on the first rows of the
+    workload holding about budget_nnz nonzeros; also use it to check those GPU rows."""
+    import numpy as np
+    from oracle import oracle as o
+    o.lib()
+    r_end = int(np.searchsorted(g.rowptr, min(budget_nnz, g.nnz), side="left"))
+    r_end = max(1, min(g.rows, r_end))
+    nnz_s = int(g.rowptr[r_end])
+    out = np.empty((r_end, k), dtype=np.float32)
+    o.csr_spmm_f32_rows(g.rowptr, g.col, g.val, B, 0, r_end, out=out)  # warm-up
+    reps = 2
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        o.csr_spmm_f32_rows(g.rowptr, g.col, g.val, B, 0, r_end, out=out)
+    dt = (time.perf_counter() - t0) / reps
+    C64, S64 = o.csr_spmm_f64_rows(g.rowptr, g.col, g.val, B, 0, min(r_end, 4096))
+    err, _ = o.max_norm_err(C_gpu_host_rows[: C64.shape[0]], C64, S64)
+    return {
+        "value": 2.0 * nnz_s * k / dt / 1e9,
+        "unit": "GFLOPS",
+        "cores": o.num_threads(),
+        "kind": "port",
+        "sample": f"rows [0,{r_end}) of c2_social K={k}: {nnz_s} nnz, {reps} timed passes after 1 warm-up, "
+                  f"{dt * 1e3:.1f} ms per pass",
+        "gpu_rows_max_normalised_err": err,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink every graph (debugging only; <1 is not the benchmark)")
+    ap.add_argument("--only", default="", help="comma list of config names to run (debugging only)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-budget-nnz", type=int, default=24_000_000)
+    ap.add_argument("--plan-flags", type=int, default=0)
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path runs on a single MI355X and no multi-GPU "
+              "figure exists for it; run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+    ensure_built()
+    pkg = importlib.import_module("hp-spmm-sddmm_amd")
+    capi, graphs = pkg.capi, pkg.graphs
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no CPU fallback for the measured path)", file=sys.stderr)
+        return 2
+    capi.lib()
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream()
+
+    workloads = WORKLOADS
+    if args.only:
+        keep = set(args.only.split(","))
+        workloads = [w for w in WORKLOADS if w[0] in keep]
+    names = []
+    for n, _ in workloads:
+        if n not in names:
+            names.append(n)
+
+    results = []
+    cpu = None
+    roofline = None
+    for name in names:
+        t0 = time.perf_counter()
+        g = graphs.make_graph(name, args.scale)
+        st = graphs.degree_stats(g.rowptr)
+        log(f"[{name}] generated in {time.perf_counter() - t0:.1f}s: rows={g.rows} nnz={g.nnz} "
+            f"mean_deg={st['mean_degree']:.1f} max_deg={st['max_degree']} empty={st['empty_row_fraction']:.3f} cv={st['cv']:.2f}")
+        d_rp = torch.from_numpy(g.rowptr).to(dev)
+        d_ci = torch.from_numpy(g.col).to(dev)
+        d_v = torch.from_numpy(g.val).to(dev)
+        for wname, k in workloads:
+            if wname != name:
+                continue
+            B = graphs.make_dense(name, g.cols, k)
+            d_B = torch.from_numpy(B).to(dev)
+            d_C = torch.empty((g.rows, k), device=dev, dtype=torch.float32)
+            t0 = time.perf_counter()
+            plan = capi.Plan(g.rows, g.cols, d_rp, d_ci, k, args.plan_flags)
+            torch.cuda.synchronize()
+            plan_ms = (time.perf_counter() - t0) * 1e3
+            info = plan.info
+            for _ in range(args.warmup):
+                capi.csr_spmm(plan, d_rp, d_ci, d_v, d_B, d_C, stream)
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            w0 = time.perf_counter()
+            e0.record(stream)
+            for _ in range(args.steps):
+                capi.csr_spmm(plan, d_rp, d_ci, d_v, d_B, d_C, stream)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            wall_ms = (time.perf_counter() - w0) * 1e3 / args.steps
+            ms = e0.elapsed_time(e1) / args.steps
+            gflops = 2.0 * g.nnz * k / (ms * 1e-3) / 1e9
+            abytes = algorithmic_bytes(g.rows, g.nnz, k)
+            gbs = abytes / (ms * 1e-3) / 1e9
+            rec = {
+                "workload": name, "k": k, "rows": g.rows, "nnz": g.nnz, "ms": ms, "wall_ms": wall_ms,
+                "gflops": gflops, "algorithmic_gb": abytes / 1e9, "achieved_gbs": gbs,
+                "roofline_frac": gbs / HBM_PEAK_GBS,
+                "unique_bytes_gb": unique_bytes(g.rows, g.cols, g.nnz, k) / 1e9,
+                "strategy": info["strategy"], "segment_length": info["segment_length"],
+                "launches_per_spmm": info["launches_per_spmm"], "plan_ms": plan_ms,
+                "plan_workspace_mb": info["workspace_bytes"] / 1e6,
+                "max_degree": st["max_degree"], "cv": st["cv"],
+            }
+            results.append(rec)
+            log(f"[{name} K={k}] {ms:.4f} ms  {gflops:.1f} GFLOPS  {gbs:.0f} GB/s algorithmic "
+                f"({100 * gbs / HBM_PEAK_GBS:.1f}% of 8 TB/s)  strategy={info['strategy']} seg={info['segment_length']} plan={plan_ms:.1f} ms")
+            if (name, k) == ROOFLINE_WORKLOAD:
+                roofline = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                            "kernel": "spmm_segments_kernel<128> + spmm_fixup_kernel<128> (one SpMM)",
+                            "workload": f"{name} K={k}", "algorithmic_bytes_per_launch": abytes,
+                            "mean_launch_ms": ms}
+                if not args.no_cpu_baseline:
+                    rows_chk = min(g.rows, 4096)
+                    c_rows = d_C[:rows_chk].cpu().numpy()
+                    t0 = time.perf_counter()
+                    cpu = cpu_baseline(graphs, g, B, k, c_rows, args.cpu_budget_nnz)
+                    log(f"[cpu baseline] {cpu['value']:.2f} GFLOPS on {cpu['cores']} threads "
+                        f"({time.perf_counter() - t0:.1f}s); GPU rows err {cpu['gpu_rows_max_normalised_err']:.2e}")
+            plan.destroy()
+            del d_B, d_C, B
+        del d_rp, d_ci, d_v, g
+        torch.cuda.empty_cache()
+
+    if not results:
+        print("no workload selected", file=sys.stderr)
+        return 2
+    geo = math.exp(sum(math.log(r["gflops"]) for r in results) / len(results))
+    line = {
+        "metric": "SpMM GFLOPS (2*nnz*K/s), geometric mean over configs[1..4] x K, FP32 CSR, 1 MI355X",
+        "value": geo,
+        "unit": "GFLOPS",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": sum(r["ms"] for r in results),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic (seeded generators, see hp-spmm-sddmm_amd/graphs.py)",
+        "config": {"workload": "configs[1..4]: " + ", ".join(f"{r['workload']}/K={r['k']}" for r in results),
+                   "scale": args.scale},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "per_workload": results,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,75 @@
+"""In-tree build of the native libraries (no cmake: three compiler lines).
+
+  libhpspmm.so           HIP kernels + C ABI (include/hpspmm.h), hipcc, gfx950
+  libhpspmm_graphgen.so  seeded synthetic graph generators, g++ / OpenMP
+  libhpspmm_host.so      C++ host layer with the reference's entry-point shapes
+  spmm_test_all          command-line driver with the reference's argv
+
+Run as a script (`python hp-spmm-sddmm_amd/build.py`) or call build_all().
+"""
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+HOST = os.path.join(HERE, "host")
+INCLUDE = os.path.join(ROOT, "include")
+
+HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+CXX = os.environ.get("CXX") or "g++"
+
+# packed FP32 VALU ops are disabled for all device code in this build
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wextra",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+CXX_FLAGS = ["-O3", "-march=x86-64-v2", "-std=c++17", "-fPIC", "-fopenmp", "-Wall", "-Wextra"]
+
+
+def _run(cmd, verbose):
+    if verbose:
+        print("+", " ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build_kernels(verbose=False):
+    out = os.path.join(HERE, "libhpspmm.so")
+    _run([HIPCC, *HIP_FLAGS, "-shared", "-I", INCLUDE, "-I", CSRC,
+          os.path.join(CSRC, "hpspmm.hip"), "-o", out], verbose)
+    return out
+
+
+def build_graphgen(verbose=False):
+    out = os.path.join(HERE, "libhpspmm_graphgen.so")
+    _run([CXX, *CXX_FLAGS, "-shared", os.path.join(CSRC, "graphgen.cpp"), "-o", out], verbose)
+    return out
+
+
+def build_host(verbose=False):
+    """C++ host layer + CLI driver (needs libhpspmm.so and libhpspmm_graphgen.so)."""
+    if not os.path.isdir(HOST):
+        return None
+    srcs = sorted(os.path.join(HOST, "src", f) for f in os.listdir(os.path.join(HOST, "src"))
+                  if f.endswith(".cpp"))
+    lib = os.path.join(HERE, "libhpspmm_host.so")
+    common = [*HIP_FLAGS[1:], "-fopenmp", "-I", INCLUDE, "-I", os.path.join(HOST, "include")]
+    link = ["-L", HERE, "-lhpspmm", "-lhpspmm_graphgen", "-Wl,-rpath,$ORIGIN"]
+    _run([HIPCC, "-x", "hip", "--offload-arch=gfx950", *common, "-shared", *srcs, "-o", lib, *link], verbose)
+    exe = os.path.join(HERE, "spmm_test_all")
+    _run([HIPCC, *common, os.path.join(HOST, "test_all.cpp"), "-o", exe,
+          "-L", HERE, "-lhpspmm_host", "-lhpspmm", "-lhpspmm_graphgen", "-Wl,-rpath,$ORIGIN"], verbose)
+    return lib
+
+
+def build_all(verbose=False):
+    build_kernels(verbose)
+    build_graphgen(verbose)
+    build_host(verbose)
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)
+    sys.exit(0)

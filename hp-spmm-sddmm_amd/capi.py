@@ -1,0 +1,206 @@
+"""ctypes binding of libhpspmm.so (the C ABI declared in include/hpspmm.h).
+
+PyTorch is used only to hold device memory and to name the stream; every
+compute call goes through the C ABI into the HIP kernels.  There is no CPU or
+PyTorch fallback: if the library is missing or no GPU is present the calls
+raise.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhpspmm.so")
+HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "hpspmm.h")
+
+OK = 0
+ERR_INVALID_ARG = 1
+ERR_BAD_CSR = 2
+ERR_HIP = 3
+ERR_NO_DEVICE = 4
+ERR_ALLOC = 5
+
+PLAN_DEFAULT = 0
+PLAN_NO_VALIDATE = 1
+PLAN_FORCE_ROWS = 2
+PLAN_FORCE_SEGMENTS = 4
+PLAN_NO_XCD_REMAP = 8
+
+
+def plan_segment_shift(log2_len):
+    return (int(log2_len) & 0xFF) << 8
+
+
+STRATEGY_ROWS = 1
+STRATEGY_SEGMENTS = 2
+STRATEGY_GENERIC_K = 3
+
+# every symbol include/hpspmm.h declares
+EXPORTS = (
+    "hpspmm_version", "hpspmm_last_error", "hpspmm_plan_create", "hpspmm_plan_get_info",
+    "hpspmm_plan_destroy", "hpspmm_csr_spmm", "hpspmm_csr_spmm_noplan", "hpspmm_coo_spmm_accumulate",
+    "hpspmm_fill_f32", "hpspmm_csr_spmm_timed",
+)
+
+_i64 = ctypes.c_int64
+_p = ctypes.c_void_p
+
+
+class PlanInfo(ctypes.Structure):
+    _fields_ = [
+        ("rows", _i64), ("cols", _i64), ("nnz", _i64), ("k", _i64),
+        ("strategy", ctypes.c_int32), ("segment_length", ctypes.c_int32),
+        ("num_segments", _i64), ("max_row_nnz", _i64), ("empty_rows", _i64),
+        ("workspace_bytes", _i64), ("launches_per_spmm", ctypes.c_int32), ("reserved", ctypes.c_int32),
+    ]
+
+    def as_dict(self):
+        return {name: getattr(self, name) for name, _ in self._fields_ if name != "reserved"}
+
+
+class HpSpmmError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"hpspmm status {code}: {message}")
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    """Load libhpspmm.so (raises if it has not been built)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing; build it with hp-spmm-sddmm_amd/build.py "
+                               "(there is no fallback path)")
+        L = ctypes.CDLL(LIB_PATH)
+        L.hpspmm_version.restype = ctypes.c_int
+        L.hpspmm_last_error.restype = ctypes.c_char_p
+        L.hpspmm_plan_create.argtypes = [_i64, _i64, _i64, _p, _p, _i64, ctypes.c_uint32, _p,
+                                         ctypes.POINTER(_p)]
+        L.hpspmm_plan_get_info.argtypes = [_p, ctypes.POINTER(PlanInfo)]
+        L.hpspmm_plan_destroy.argtypes = [_p]
+        L.hpspmm_csr_spmm.argtypes = [_p, _p, _p, _p, _p, _p, _p]
+        L.hpspmm_csr_spmm_noplan.argtypes = [_i64, _i64, _i64, _p, _p, _p, _p, _i64, _p, _p]
+        L.hpspmm_coo_spmm_accumulate.argtypes = [_i64, _i64, _i64, _p, _p, _p, _p, _i64, _p, _p]
+        L.hpspmm_fill_f32.argtypes = [_p, _i64, ctypes.c_float, _p]
+        L.hpspmm_csr_spmm_timed.argtypes = [_p, _p, _p, _p, _p, _p, _p, ctypes.c_int, ctypes.c_int,
+                                            ctypes.POINTER(ctypes.c_float)]
+        _lib = L
+    return _lib
+
+
+def check(code):
+    if code != OK:
+        raise HpSpmmError(code, lib().hpspmm_last_error().decode())
+
+
+def _ptr(t):
+    """Device pointer of a torch tensor (None -> NULL)."""
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(stream):
+    if stream is None:
+        import torch
+        stream = torch.cuda.current_stream()
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def _dev(t, dtype, name):
+    import torch
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError(f"{name} must be a torch tensor in GPU memory")
+    if t.dtype != dtype or not t.is_contiguous():
+        raise TypeError(f"{name} must be contiguous {dtype}")
+    return t
+
+
+class Plan:
+    """Owns an hpspmm_plan (see hpspmm_plan_create in include/hpspmm.h)."""
+
+    def __init__(self, rows, cols, rowptr, col, k, flags=PLAN_DEFAULT, stream=None):
+        import torch
+        _dev(rowptr, torch.int32, "rowptr")
+        _dev(col, torch.int32, "col")
+        if rowptr.numel() != rows + 1:
+            raise ValueError("rowptr must have rows + 1 entries")
+        self._h = ctypes.c_void_p()
+        self.rows, self.cols, self.nnz, self.k = int(rows), int(cols), int(col.numel()), int(k)
+        check(lib().hpspmm_plan_create(rows, cols, self.nnz, _ptr(rowptr), _ptr(col), k, flags,
+                                       _stream(stream), ctypes.byref(self._h)))
+
+    @property
+    def info(self):
+        out = PlanInfo()
+        check(lib().hpspmm_plan_get_info(self._h, ctypes.byref(out)))
+        return out.as_dict()
+
+    def destroy(self):
+        if getattr(self, "_h", None):
+            lib().hpspmm_plan_destroy(self._h)
+            self._h = None
+
+    __del__ = destroy
+
+
+def _check_operands(rows, cols, nnz, k, rowptr, col, val, B, C):
+    import torch
+    if rowptr is not None:
+        _dev(rowptr, torch.int32, "rowptr")
+        if rowptr.numel() != rows + 1:
+            raise ValueError("rowptr must have rows + 1 entries")
+    _dev(col, torch.int32, "col")
+    _dev(val, torch.float32, "val")
+    _dev(B, torch.float32, "B")
+    _dev(C, torch.float32, "C")
+    if col.numel() != nnz or val.numel() != nnz:
+        raise ValueError("col / val length differs from nnz")
+    if tuple(B.shape) != (cols, k) or tuple(C.shape) != (rows, k):
+        raise ValueError(f"B must be {(cols, k)} and C {(rows, k)}; got {tuple(B.shape)}, {tuple(C.shape)}")
+
+
+def csr_spmm(plan, rowptr, col, val, B, C, stream=None):
+    """C = A @ B through hpspmm_csr_spmm."""
+    _check_operands(plan.rows, plan.cols, plan.nnz, plan.k, rowptr, col, val, B, C)
+    check(lib().hpspmm_csr_spmm(plan._h, _ptr(rowptr), _ptr(col), _ptr(val), _ptr(B), _ptr(C),
+                                _stream(stream)))
+    return C
+
+
+def csr_spmm_noplan(rows, cols, rowptr, col, val, B, C, stream=None):
+    """C = A @ B through hpspmm_csr_spmm_noplan."""
+    k = int(B.shape[1])
+    _check_operands(rows, cols, int(col.numel()), k, rowptr, col, val, B, C)
+    check(lib().hpspmm_csr_spmm_noplan(rows, cols, int(col.numel()), _ptr(rowptr), _ptr(col), _ptr(val),
+                                       _ptr(B), k, _ptr(C), _stream(stream)))
+    return C
+
+
+def coo_spmm_accumulate(rows, cols, row, col, val, B, C, stream=None):
+    """C += A @ B through hpspmm_coo_spmm_accumulate."""
+    import torch
+    k = int(B.shape[1])
+    _dev(row, torch.int32, "row")
+    _check_operands(rows, cols, int(col.numel()), k, None, col, val, B, C)
+    if row.numel() != col.numel():
+        raise ValueError("row / col length differs")
+    check(lib().hpspmm_coo_spmm_accumulate(rows, cols, int(col.numel()), _ptr(row), _ptr(col), _ptr(val),
+                                           _ptr(B), k, _ptr(C), _stream(stream)))
+    return C
+
+
+def fill_f32(x, value, stream=None):
+    import torch
+    _dev(x, torch.float32, "x")
+    check(lib().hpspmm_fill_f32(_ptr(x), x.numel(), float(value), _stream(stream)))
+    return x
+
+
+def csr_spmm_timed(plan, rowptr, col, val, B, C, warmup=20, iters=200, stream=None):
+    """Mean milliseconds per SpMM over `iters` back-to-back launches (HIP events on the launch stream)."""
+    _check_operands(plan.rows, plan.cols, plan.nnz, plan.k, rowptr, col, val, B, C)
+    ms = ctypes.c_float(0.0)
+    check(lib().hpspmm_csr_spmm_timed(plan._h, _ptr(rowptr), _ptr(col), _ptr(val), _ptr(B), _ptr(C),
+                                      _stream(stream), warmup, iters, ctypes.byref(ms)))
+    return float(ms.value)

@@ -1,0 +1,372 @@
+// Host side of libhpspmm.so: the C ABI declared in include/hpspmm.h, the plan
+// (device-side work assignment) and the kernel launches.
+#include "hpspmm.h"
+
+#include <hip/hip_runtime.h>
+
+#include <climits>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+
+#include "spmm_kernels.hpp"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+#define HPSPMM_HIP(call)                                                                       \
+  do {                                                                                         \
+    hipError_t e_ = (call);                                                                    \
+    if (e_ != hipSuccess)                                                                      \
+      return fail(e_ == hipErrorNoDevice ? HPSPMM_ERR_NO_DEVICE : HPSPMM_ERR_HIP, "%s: %s",    \
+                  #call, hipGetErrorString(e_));                                               \
+  } while (0)
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+inline bool fast_k(int64_t k) { return k == 32 || k == 64 || k == 128; }
+
+int check_dims(int64_t rows, int64_t cols, int64_t nnz, int64_t k) {
+  if (rows < 0 || cols < 0 || nnz < 0) return fail(HPSPMM_ERR_INVALID_ARG, "negative dimension (rows=%lld cols=%lld nnz=%lld)",
+                                                   (long long)rows, (long long)cols, (long long)nnz);
+  if (rows >= INT32_MAX || cols > INT32_MAX || nnz > INT32_MAX)
+    return fail(HPSPMM_ERR_INVALID_ARG, "dimension exceeds the int32 index range (rows=%lld cols=%lld nnz=%lld)",
+                (long long)rows, (long long)cols, (long long)nnz);
+  if (k <= 0 || k > (1 << 20)) return fail(HPSPMM_ERR_INVALID_ARG, "k must be in [1, 2^20], got %lld", (long long)k);
+  if (nnz > 0 && cols == 0) return fail(HPSPMM_ERR_INVALID_ARG, "nnz > 0 with cols == 0");
+  return HPSPMM_OK;
+}
+
+int grid_for(int64_t items, int64_t cap = 1 << 20) {
+  int64_t b = ceil_div(items, hpspmm::kBlock);
+  if (b < 1) b = 1;
+  if (b > cap) b = cap;
+  return (int)b;
+}
+
+}  // namespace
+
+struct hpspmm_plan {
+  int64_t rows = 0, cols = 0, nnz = 0, k = 0;
+  int strategy = 0;
+  int shift = 0;  // log2(segment length)
+  int64_t nseg = 0;
+  int64_t max_row_nnz = 0, empty_rows = 0;
+  bool xcd_remap = true;
+  int32_t* d_nnz_row = nullptr;  // [nnz]
+  float* d_carry = nullptr;      // [2 * nseg * k]
+  int64_t workspace_bytes = 0;
+};
+
+namespace {
+
+// Launch geometry of the kernels that run one sub-wave per row.
+inline int64_t row_blocks(int64_t rows, int64_t k) {
+  const int64_t per_wave = 64 / (k / 4);
+  return ceil_div(ceil_div(rows, per_wave), hpspmm::kWavesPerBlock);
+}
+
+template <int K>
+int launch_rows(int64_t rows, const int32_t* rp, const int32_t* ci, const float* v, const float* B, float* C,
+                hipStream_t st) {
+  const int64_t blocks = row_blocks(rows, K);
+  if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  hipLaunchKernelGGL(hpspmm::spmm_rows_kernel<K>, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rows, rp, ci,
+                     v, B, C);
+  return HPSPMM_OK;
+}
+
+int launch_rows_any(int64_t rows, int64_t k, const int32_t* rp, const int32_t* ci, const float* v,
+                    const float* B, float* C, hipStream_t st) {
+  if (rows == 0) return HPSPMM_OK;
+  switch (k) {
+    case 32: return launch_rows<32>(rows, rp, ci, v, B, C, st);
+    case 64: return launch_rows<64>(rows, rp, ci, v, B, C, st);
+    case 128: return launch_rows<128>(rows, rp, ci, v, B, C, st);
+    default: {
+      const int64_t blocks = ceil_div(rows, hpspmm::kWavesPerBlock);
+      hipLaunchKernelGGL(hpspmm::spmm_rows_generic_kernel, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st,
+                         rows, k, rp, ci, v, B, C);
+      return HPSPMM_OK;
+    }
+  }
+}
+
+template <int K>
+int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, const float* v,
+                    const float* B, float* C, hipStream_t st) {
+  constexpr int P = 64 / (K / 4);
+  const int64_t nblocks = ceil_div(ceil_div(p->nseg, P), hpspmm::kWavesPerBlock);
+  const int64_t grid = p->xcd_remap ? ceil_div(nblocks, hpspmm::kXcds) * hpspmm::kXcds : nblocks;
+  if (grid > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  if (p->nnz > 0)
+    hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, false>), dim3((unsigned)grid), dim3(hpspmm::kBlock), 0, st,
+                       rp, ci, v, p->d_nnz_row, B, C, p->d_carry, p->nnz, p->shift, p->nseg, nblocks,
+                       p->xcd_remap);
+  hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)row_blocks(p->rows, K)), dim3(hpspmm::kBlock), 0,
+                     st, p->rows, rp, p->d_carry, C, p->shift);
+  return HPSPMM_OK;
+}
+
+template <int K>
+int launch_coo(int64_t nnz, const int32_t* ri, const int32_t* ci, const float* v, const float* B, float* C,
+               hipStream_t st) {
+  constexpr int P = 64 / (K / 4);
+  // 64 nonzeros per sub-wave: short enough to balance, long enough that the
+  // one flush per segment end is amortised
+  const int shift = 6;
+  const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
+  const int64_t nblocks = ceil_div(ceil_div(nseg, P), hpspmm::kWavesPerBlock);
+  if (nblocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, true>), dim3((unsigned)nblocks), dim3(hpspmm::kBlock), 0, st,
+                     (const int32_t*)nullptr, ci, v, ri, B, C, (float*)nullptr, nnz, shift, nseg, nblocks, false);
+  return HPSPMM_OK;
+}
+
+// Segment length: long enough that the carry traffic (two K-float partials per
+// segment, against S*(K+2) floats of gather) is small, short enough that there
+// are several waves of work per SIMD.
+int choose_shift(int64_t nnz, int64_t k) {
+  const int64_t subwaves = 64 / (k / 4);
+  const int64_t target_waves = 256 /*CUs*/ * 4 /*SIMDs*/ * 16;
+  int shift = 5;
+  while (shift < 9 && (nnz >> (shift + 1)) / subwaves >= target_waves) ++shift;
+  return shift;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hpspmm_version(void) { return 100; }
+
+const char* hpspmm_last_error(void) { return g_last_error.c_str(); }
+
+int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr, const int32_t* d_col,
+                       int64_t k, uint32_t flags, void* stream, hpspmm_plan** plan_out) {
+  if (!plan_out) return fail(HPSPMM_ERR_INVALID_ARG, "plan_out is NULL");
+  *plan_out = nullptr;
+  if (int rc = check_dims(rows, cols, nnz, k)) return rc;
+  if (!d_rowptr) return fail(HPSPMM_ERR_INVALID_ARG, "d_rowptr is NULL");
+  if (nnz > 0 && !d_col) return fail(HPSPMM_ERR_INVALID_ARG, "d_col is NULL with nnz > 0");
+  hipStream_t st = (hipStream_t)stream;
+
+  int ndev = 0;
+  if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
+    (void)hipGetLastError();
+    return fail(HPSPMM_ERR_NO_DEVICE, "no HIP device available");
+  }
+
+  // validation flags + row statistics, one small device buffer
+  int32_t* d_meta = nullptr;
+  HPSPMM_HIP(hipMalloc(&d_meta, 4 * sizeof(int32_t)));
+  struct MetaGuard {
+    int32_t* p;
+    ~MetaGuard() { (void)hipFree(p); }
+  } meta_guard{d_meta};
+  HPSPMM_HIP(hipMemsetAsync(d_meta, 0, 4 * sizeof(int32_t), st));
+  if (!(flags & HPSPMM_PLAN_NO_VALIDATE)) {
+    const int64_t work = rows > nnz ? rows : nnz;
+    hipLaunchKernelGGL(hpspmm::validate_csr_kernel, dim3(grid_for(work, 8192)), dim3(hpspmm::kBlock), 0, st, rows,
+                       cols, nnz, d_rowptr, d_col, d_meta);
+    int32_t bad = 0;
+    HPSPMM_HIP(hipMemcpyAsync(&bad, d_meta, sizeof bad, hipMemcpyDeviceToHost, st));
+    HPSPMM_HIP(hipStreamSynchronize(st));
+    if (bad)
+      return fail(HPSPMM_ERR_BAD_CSR, "invalid CSR:%s%s%s%s", (bad & 1) ? " rowptr[0] != 0;" : "",
+                  (bad & 2) ? " rowptr decreases;" : "", (bad & 4) ? " rowptr[rows] != nnz;" : "",
+                  (bad & 8) ? " column index out of range;" : "");
+  }
+  int32_t stats[2] = {0, 0};
+  if (rows > 0) {
+    hipLaunchKernelGGL(hpspmm::row_stats_kernel, dim3(grid_for(rows, 4096)), dim3(hpspmm::kBlock), 0, st, rows,
+                       d_rowptr, d_meta + 1);
+    HPSPMM_HIP(hipMemcpyAsync(stats, d_meta + 1, sizeof stats, hipMemcpyDeviceToHost, st));
+    HPSPMM_HIP(hipStreamSynchronize(st));
+  }
+
+  hpspmm_plan* p = new (std::nothrow) hpspmm_plan;
+  if (!p) return fail(HPSPMM_ERR_ALLOC, "out of host memory");
+  p->rows = rows;
+  p->cols = cols;
+  p->nnz = nnz;
+  p->k = k;
+  p->max_row_nnz = stats[0];
+  p->empty_rows = stats[1];
+  p->xcd_remap = !(flags & HPSPMM_PLAN_NO_XCD_REMAP);
+
+  if (!fast_k(k)) {
+    p->strategy = HPSPMM_STRATEGY_GENERIC_K;
+  } else if (flags & HPSPMM_PLAN_FORCE_ROWS) {
+    p->strategy = HPSPMM_STRATEGY_ROWS;
+  } else if (flags & HPSPMM_PLAN_FORCE_SEGMENTS) {
+    p->strategy = HPSPMM_STRATEGY_SEGMENTS;
+  } else {
+    // Whole rows when no row is long enough to unbalance the sub-waves and the
+    // matrix is small enough that a second (fix-up) launch would be felt.
+    const bool small = nnz < (1 << 21);
+    p->strategy = (nnz == 0 || (small && p->max_row_nnz <= 512)) ? HPSPMM_STRATEGY_ROWS : HPSPMM_STRATEGY_SEGMENTS;
+  }
+
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS) {
+    int forced = (int)((flags >> 8) & 0xFFu);
+    if (forced && (forced < 3 || forced > 20)) {
+      delete p;
+      return fail(HPSPMM_ERR_INVALID_ARG, "forced segment shift %d outside [3, 20]", forced);
+    }
+    p->shift = forced ? forced : choose_shift(nnz, k);
+    p->nseg = ceil_div(nnz, (int64_t)1 << p->shift);
+    const size_t row_bytes = (size_t)(nnz > 0 ? nnz : 1) * sizeof(int32_t);
+    const size_t carry_bytes = (size_t)(p->nseg > 0 ? p->nseg : 1) * 2 * (size_t)k * sizeof(float);
+    if (hipMalloc(&p->d_nnz_row, row_bytes) != hipSuccess || hipMalloc(&p->d_carry, carry_bytes) != hipSuccess) {
+      (void)hipGetLastError();
+      hpspmm_plan_destroy(p);
+      return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the plan failed", row_bytes + carry_bytes);
+    }
+    p->workspace_bytes = (int64_t)(row_bytes + carry_bytes);
+    if (nnz > 0) {
+      hipLaunchKernelGGL(hpspmm::expand_rows_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)),
+                         dim3(hpspmm::kBlock), 0, st, rows, nnz, d_rowptr, p->d_nnz_row);
+      hipError_t e = hipStreamSynchronize(st);
+      if (e != hipSuccess) {
+        hpspmm_plan_destroy(p);
+        return fail(HPSPMM_ERR_HIP, "row expansion failed: %s", hipGetErrorString(e));
+      }
+    }
+  }
+  *plan_out = p;
+  return HPSPMM_OK;
+}
+
+int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
+  if (!plan || !out) return fail(HPSPMM_ERR_INVALID_ARG, "plan or info_out is NULL");
+  std::memset(out, 0, sizeof *out);
+  out->rows = plan->rows;
+  out->cols = plan->cols;
+  out->nnz = plan->nnz;
+  out->k = plan->k;
+  out->strategy = plan->strategy;
+  out->segment_length = plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? (1 << plan->shift) : 0;
+  out->num_segments = plan->nseg;
+  out->max_row_nnz = plan->max_row_nnz;
+  out->empty_rows = plan->empty_rows;
+  out->workspace_bytes = plan->workspace_bytes;
+  out->launches_per_spmm = plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? 2 : 1;
+  return HPSPMM_OK;
+}
+
+int hpspmm_plan_destroy(hpspmm_plan* plan) {
+  if (!plan) return HPSPMM_OK;
+  if (plan->d_nnz_row) (void)hipFree(plan->d_nnz_row);
+  if (plan->d_carry) (void)hipFree(plan->d_carry);
+  delete plan;
+  return HPSPMM_OK;
+}
+
+int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d_col, const float* d_val,
+                    const float* d_B, float* d_C, void* stream) {
+  if (!plan) return fail(HPSPMM_ERR_INVALID_ARG, "plan is NULL");
+  if (plan->rows == 0) return HPSPMM_OK;
+  if (!d_rowptr || !d_C) return fail(HPSPMM_ERR_INVALID_ARG, "d_rowptr or d_C is NULL");
+  if (plan->nnz > 0 && (!d_col || !d_val || !d_B))
+    return fail(HPSPMM_ERR_INVALID_ARG, "d_col, d_val or d_B is NULL with nnz > 0");
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  if (plan->strategy == HPSPMM_STRATEGY_SEGMENTS) {
+    switch (plan->k) {
+      case 32: rc = launch_segments<32>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;
+      case 64: rc = launch_segments<64>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;
+      default: rc = launch_segments<128>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;
+    }
+  } else {
+    rc = launch_rows_any(plan->rows, plan->k, d_rowptr, d_col, d_val, d_B, d_C, st);
+  }
+  if (rc) return rc;
+  HPSPMM_HIP(hipGetLastError());
+  return HPSPMM_OK;
+}
+
+int hpspmm_csr_spmm_noplan(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr,
+                           const int32_t* d_col, const float* d_val, const float* d_B, int64_t k, float* d_C,
+                           void* stream) {
+  if (int rc = check_dims(rows, cols, nnz, k)) return rc;
+  if (rows == 0) return HPSPMM_OK;
+  if (!d_rowptr || !d_C) return fail(HPSPMM_ERR_INVALID_ARG, "d_rowptr or d_C is NULL");
+  if (nnz > 0 && (!d_col || !d_val || !d_B))
+    return fail(HPSPMM_ERR_INVALID_ARG, "d_col, d_val or d_B is NULL with nnz > 0");
+  if (int rc = launch_rows_any(rows, k, d_rowptr, d_col, d_val, d_B, d_C, (hipStream_t)stream)) return rc;
+  HPSPMM_HIP(hipGetLastError());
+  return HPSPMM_OK;
+}
+
+int hpspmm_coo_spmm_accumulate(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_row,
+                               const int32_t* d_col, const float* d_val, const float* d_B, int64_t k, float* d_C,
+                               void* stream) {
+  if (int rc = check_dims(rows, cols, nnz, k)) return rc;
+  if (nnz == 0) return HPSPMM_OK;
+  if (rows == 0) return fail(HPSPMM_ERR_INVALID_ARG, "nnz > 0 with rows == 0");
+  if (!d_row || !d_col || !d_val || !d_B || !d_C) return fail(HPSPMM_ERR_INVALID_ARG, "NULL device pointer");
+  hipStream_t st = (hipStream_t)stream;
+  int rc = HPSPMM_OK;
+  switch (k) {
+    case 32: rc = launch_coo<32>(nnz, d_row, d_col, d_val, d_B, d_C, st); break;
+    case 64: rc = launch_coo<64>(nnz, d_row, d_col, d_val, d_B, d_C, st); break;
+    case 128: rc = launch_coo<128>(nnz, d_row, d_col, d_val, d_B, d_C, st); break;
+    default:
+      hipLaunchKernelGGL(hpspmm::spmm_coo_generic_kernel, dim3(grid_for(nnz * k, 1 << 16)), dim3(hpspmm::kBlock), 0,
+                         st, nnz, k, d_row, d_col, d_val, d_B, d_C);
+  }
+  if (rc) return rc;
+  HPSPMM_HIP(hipGetLastError());
+  return HPSPMM_OK;
+}
+
+int hpspmm_fill_f32(float* d_x, int64_t n, float value, void* stream) {
+  if (n < 0) return fail(HPSPMM_ERR_INVALID_ARG, "negative length");
+  if (n == 0) return HPSPMM_OK;
+  if (!d_x) return fail(HPSPMM_ERR_INVALID_ARG, "d_x is NULL");
+  hipLaunchKernelGGL(hpspmm::fill_f32_kernel, dim3(grid_for(n, 1 << 16)), dim3(hpspmm::kBlock), 0,
+                     (hipStream_t)stream, d_x, n, value);
+  HPSPMM_HIP(hipGetLastError());
+  return HPSPMM_OK;
+}
+
+int hpspmm_csr_spmm_timed(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d_col, const float* d_val,
+                          const float* d_B, float* d_C, void* stream, int warmup, int iters, float* mean_ms_out) {
+  if (!mean_ms_out || iters <= 0 || warmup < 0) return fail(HPSPMM_ERR_INVALID_ARG, "bad timing arguments");
+  hipStream_t st = (hipStream_t)stream;
+  for (int i = 0; i < warmup; ++i)
+    if (int rc = hpspmm_csr_spmm(plan, d_rowptr, d_col, d_val, d_B, d_C, stream)) return rc;
+  hipEvent_t t0, t1;
+  HPSPMM_HIP(hipEventCreate(&t0));
+  HPSPMM_HIP(hipEventCreate(&t1));
+  int rc = HPSPMM_OK;
+  hipError_t e = hipEventRecord(t0, st);
+  for (int i = 0; i < iters && rc == HPSPMM_OK && e == hipSuccess; ++i)
+    rc = hpspmm_csr_spmm(plan, d_rowptr, d_col, d_val, d_B, d_C, stream);
+  if (e == hipSuccess) e = hipEventRecord(t1, st);
+  if (e == hipSuccess) e = hipEventSynchronize(t1);
+  float ms = 0.f;
+  if (e == hipSuccess && rc == HPSPMM_OK) e = hipEventElapsedTime(&ms, t0, t1);
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  if (rc) return rc;
+  if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "timing failed: %s", hipGetErrorString(e));
+  *mean_ms_out = ms / (float)iters;
+  return HPSPMM_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,152 @@
+/*
+ * hpspmm.h - C ABI of the gfx950 (MI355X) FP32 CSR SpMM library, libhpspmm.so.
+ *
+ *   C = A * B     A: sparse, CSR, int32 zero-based indices, FP32 values
+ *                 B: dense  cols x k, FP32, row-major, leading dimension k
+ *                 C: dense  rows x k, FP32, row-major, leading dimension k
+ *                 alpha = 1, beta = 0 (C is overwritten), A not transposed.
+ *
+ * These are the operand conventions of the reference's SpMM entry points
+ * (include/spmm/mm/spmm_kernel.h:17-21; descriptors at
+ * spmm/mm/spmm_kernel.cu:82-108; indexing col*k + cid at :269).  Each entry
+ * point below names the reference interface it stands in for.
+ *
+ * Conventions
+ *   - Every pointer whose name starts with d_ is a DEVICE pointer owned by the
+ *     caller; the library never frees or reallocates caller memory.
+ *   - Sizes and counts are int64_t; index arrays are int32_t as in the
+ *     reference's CSR container (include/spmm/mm/spmm_common.h:58-82), so
+ *     rows, cols and nnz must each be <= INT32_MAX.  Byte offsets are computed
+ *     in 64 bits (the reference's int byte counts overflow at 2^31 bytes,
+ *     spmm/starml/operators/cuda/copy_kernel.cu:12,30).
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *     Launches are asynchronous; nothing synchronises with the host except
+ *     hpspmm_plan_create (which reads back validation flags and statistics).
+ *   - Every function returns HPSPMM_OK (0) or a positive hpspmm_status; after
+ *     a failure hpspmm_last_error() gives a message for the calling thread.
+ *     The reference has no error convention on this path (statuses are
+ *     dropped, failed checks abort through loguru, loguru.h:1535); a status
+ *     code replaces the abort.
+ *   - A plan may be used from one stream at a time: it owns the scratch
+ *     buffer that split rows are reduced through.
+ */
+#ifndef HPSPMM_H_
+#define HPSPMM_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum hpspmm_status {
+  HPSPMM_OK = 0,
+  HPSPMM_ERR_INVALID_ARG = 1, /* null pointer, negative size, size > INT32_MAX, k <= 0 */
+  HPSPMM_ERR_BAD_CSR = 2,     /* rowptr not monotone / rowptr[0] != 0 / rowptr[rows] != nnz / col out of range */
+  HPSPMM_ERR_HIP = 3,         /* a HIP runtime call failed (message carries hipGetErrorString) */
+  HPSPMM_ERR_NO_DEVICE = 4,   /* no usable GPU */
+  HPSPMM_ERR_ALLOC = 5        /* device allocation for the plan failed */
+} hpspmm_status;
+
+/* hpspmm_plan_create flags */
+#define HPSPMM_PLAN_DEFAULT 0u
+#define HPSPMM_PLAN_NO_VALIDATE 1u    /* skip the device-side CSR check */
+#define HPSPMM_PLAN_FORCE_ROWS 2u     /* always use the whole-row kernel */
+#define HPSPMM_PLAN_FORCE_SEGMENTS 4u /* always use the nnz-segment kernel + carry fix-up */
+#define HPSPMM_PLAN_NO_XCD_REMAP 8u   /* keep the hardware's round-robin workgroup->XCD order */
+/* bits 8..15: log2 of the segment length to force (0 = choose automatically) */
+#define HPSPMM_PLAN_SEGMENT_SHIFT(log2_len) (((uint32_t)(log2_len) & 0xFFu) << 8)
+
+/* strategy reported by hpspmm_plan_get_info */
+#define HPSPMM_STRATEGY_ROWS 1
+#define HPSPMM_STRATEGY_SEGMENTS 2
+#define HPSPMM_STRATEGY_GENERIC_K 3
+
+typedef struct hpspmm_plan hpspmm_plan;
+
+typedef struct hpspmm_plan_info {
+  int64_t rows, cols, nnz, k;
+  int32_t strategy;        /* HPSPMM_STRATEGY_* */
+  int32_t segment_length;  /* nonzeros per sub-wave segment (segments strategy), else 0 */
+  int64_t num_segments;
+  int64_t max_row_nnz;
+  int64_t empty_rows;
+  int64_t workspace_bytes; /* device memory owned by the plan */
+  int32_t launches_per_spmm;
+  int32_t reserved;
+} hpspmm_plan_info;
+
+/* Library version, major*10000 + minor*100 + patch. */
+int hpspmm_version(void);
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char *hpspmm_last_error(void);
+
+/*
+ * Analyse the sparsity structure of A for a given k and build the device-side
+ * work assignment (row-of-nonzero map, segment length, carry buffer).
+ * Replaces the host-side preprocessing the reference does before timing:
+ * CSR->COO expansion (spmm/mm/spmm_common.cpp:185-235) and the choice of
+ * nnz_per_warp (spmm/mm/spmm_kernel.cu:749-751).  Synchronises `stream`.
+ * Values are not read: the plan stays valid when d_val or B change, and must
+ * be rebuilt when rowptr / col change.
+ */
+int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
+                       const int32_t *d_col, int64_t k, uint32_t flags, void *stream,
+                       hpspmm_plan **plan_out);
+
+int hpspmm_plan_get_info(const hpspmm_plan *plan, hpspmm_plan_info *info_out);
+
+/* Frees the plan's device memory.  NULL is accepted. */
+int hpspmm_plan_destroy(hpspmm_plan *plan);
+
+/*
+ * C = A * B with a plan.  One call = one SpMM = the body of one iteration of
+ * the reference's launch loop in GESpMM (spmm/mm/spmm_kernel.cu:405-422) /
+ * one cusparseSpMM call (spmm/mm/spmm_kernel.cu:129-141).  C need not be
+ * zeroed beforehand; every element of C, empty rows included, is written.
+ * The result is deterministic (no atomics).
+ */
+int hpspmm_csr_spmm(hpspmm_plan *plan, const int32_t *d_rowptr, const int32_t *d_col,
+                    const float *d_val, const float *d_B, float *d_C, void *stream);
+
+/*
+ * C = A * B without a plan: whole-row kernel, no preprocessing, no device
+ * allocation.  Same contract as GESpMM's single launch
+ * (spmm/mm/spmm_kernel.cu:406-421), for callers that cannot keep a plan.
+ */
+int hpspmm_csr_spmm_noplan(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
+                           const int32_t *d_col, const float *d_val, const float *d_B, int64_t k,
+                           float *d_C, void *stream);
+
+/*
+ * C += A * B for A in COO (row-index per nonzero), the contract of one launch
+ * of LBSpMM (spmm/mm/spmm_kernel.cu:733-768: accumulates with atomics,
+ * :463-476).  Entries of one row need not be contiguous, `nnz` may include
+ * zero-valued padding entries (spmm/mm/spmm_common.cpp:220-226), and entries
+ * may arrive in a permuted row order (spmm/mm/spmm_common.cpp:269-277).
+ * The caller zeroes C first if it wants C = A * B.  Uses FP32 atomics, so the
+ * summation order (not the set of terms) can differ between runs.
+ */
+int hpspmm_coo_spmm_accumulate(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_row,
+                               const int32_t *d_col, const float *d_val, const float *d_B, int64_t k,
+                               float *d_C, void *stream);
+
+/* d_x[i] = value for i in [0, n): fill_matrix (spmm/mm/spmm_kernel.cu:23-34). */
+int hpspmm_fill_f32(float *d_x, int64_t n, float value, void *stream);
+
+/*
+ * Time `iters` back-to-back hpspmm_csr_spmm launches on `stream` with HIP
+ * events after `warmup` untimed ones and return the mean in milliseconds:
+ * the measurement protocol of GESpMM / cusparseCSRSpMM
+ * (include/spmm/utils/timer_cuda.h:3-40, spmm/mm/spmm_kernel.cu:128-145,
+ * 404-424).  Synchronises `stream`.
+ */
+int hpspmm_csr_spmm_timed(hpspmm_plan *plan, const int32_t *d_rowptr, const int32_t *d_col,
+                          const float *d_val, const float *d_B, float *d_C, void *stream,
+                          int warmup, int iters, float *mean_ms_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HPSPMM_H_ */

@@ -104,6 +104,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget-nnz", type=int, default=24_000_000)
     ap.add_argument("--plan-flags", type=int, default=0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run three 1 GiB device-to-device copies (a kernel of known traffic, "
+                         "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -122,6 +125,15 @@ def main():
     capi.lib()
     dev = torch.device("cuda:0")
     stream = torch.cuda.current_stream()
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, device=dev, dtype=torch.float32).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     workloads = WORKLOADS
     if args.only:

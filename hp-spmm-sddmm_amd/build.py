@@ -20,6 +20,7 @@ INCLUDE = os.path.join(ROOT, "include")
 
 HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 CXX = os.environ.get("CXX") or "g++"
+ROCM = os.environ.get("ROCM_PATH") or "/opt/rocm"
 
 # packed FP32 VALU ops are disabled for all device code in this build
 HIP_FLAGS = [
@@ -49,18 +50,19 @@ def build_graphgen(verbose=False):
 
 
 def build_host(verbose=False):
-    """C++ host layer + CLI driver (needs libhpspmm.so and libhpspmm_graphgen.so)."""
-    if not os.path.isdir(HOST):
-        return None
+    """C++ host layer + CLI driver + CPU self-test (needs libhpspmm.so and libhpspmm_graphgen.so)."""
     srcs = sorted(os.path.join(HOST, "src", f) for f in os.listdir(os.path.join(HOST, "src"))
                   if f.endswith(".cpp"))
     lib = os.path.join(HERE, "libhpspmm_host.so")
-    common = [*HIP_FLAGS[1:], "-fopenmp", "-I", INCLUDE, "-I", os.path.join(HOST, "include")]
-    link = ["-L", HERE, "-lhpspmm", "-lhpspmm_graphgen", "-Wl,-rpath,$ORIGIN"]
-    _run([HIPCC, "-x", "hip", "--offload-arch=gfx950", *common, "-shared", *srcs, "-o", lib, *link], verbose)
-    exe = os.path.join(HERE, "spmm_test_all")
-    _run([HIPCC, *common, os.path.join(HOST, "test_all.cpp"), "-o", exe,
-          "-L", HERE, "-lhpspmm_host", "-lhpspmm", "-lhpspmm_graphgen", "-Wl,-rpath,$ORIGIN"], verbose)
+    common = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-I", INCLUDE,
+              "-I", os.path.join(HOST, "include")]
+    link = ["-L", HERE, "-lhpspmm", "-lhpspmm_graphgen", "-L", os.path.join(ROCM, "lib"), "-lrocsparse",
+            "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(ROCM, "lib")]
+    _run([HIPCC, *common, "-shared", *srcs, "-o", lib, *link], verbose)
+    for name in ("test_all", "host_selftest"):
+        exe = os.path.join(HERE, "spmm_" + name)
+        _run([HIPCC, *common, os.path.join(HOST, name + ".cpp"), "-o", exe, "-L", HERE, "-lhpspmm_host",
+              *link], verbose)
     return lib
 
 

@@ -403,6 +403,46 @@ hpspmm_graph* hpspmm_gen_rmat(int scale, int64_t n_edges, double a, double b, do
   return (hpspmm_graph*)build_symmetric((int64_t)1 << scale, n_edges, smp, false, kValSymUniformPM1, seed);
 }
 
+// The benchmark configurations by name.  scale < 1 shrinks vertex and edge
+// counts together (tests); scale = 1 is the benchmark size.  Parameters were
+// calibrated so that the full-size graphs land on the configured statistics:
+//   c1_citation   20,000 vertices, mean degree ~5, max ~170-190
+//   c2_social     232,965 vertices, ~114.6 M nonzeros, max degree ~21,000
+//   c3_copurchase 2,449,029 vertices, ~123.7 M nonzeros (80 % of the edge
+//                 samples are intra-community; communities of ~37 vertices
+//                 saturate, so more samples than stored edges are drawn)
+//   c4_rmat       R-MAT scale 22, edge factor 16
+hpspmm_graph* hpspmm_gen_named(const char* name, double scale) {
+  const std::string n = name ? name : "";
+  if (!(scale > 0)) {
+    g_err = "gen_named: scale must be positive";
+    return nullptr;
+  }
+  auto scaled = [&](double full, int64_t floor_) {
+    return std::max<int64_t>(floor_, (int64_t)std::llround(full * scale));
+  };
+  if (n == "c0_uniform") {
+    const int64_t v = scaled(4096, 16);
+    return hpspmm_gen_uniform_rows(v, v, 16, 0);
+  }
+  if (n == "c1_citation") {
+    const int64_t v = scaled(20000, 64);
+    return hpspmm_gen_citation(v, 2.5, 70, (int64_t)std::llround(2.05 * (double)v), 1);
+  }
+  if (n == "c2_social")
+    return hpspmm_gen_powerlaw(scaled(232965, 64), 2.1, std::max(4.0, 520.0 * scale),
+                               (int64_t)std::llround(60.45e6 * scale), kValSymUniform01, 2);
+  if (n == "c3_copurchase")
+    return hpspmm_gen_community(scaled(2449029, 64), 3.5, 1.0, scaled(65536, 1), 0.8,
+                                (int64_t)std::llround(165.4e6 * scale), 3);
+  if (n == "c4_rmat") {
+    const int sc = scale >= 1 ? 22 : std::max(6, 22 + (int)std::floor(std::log2(scale)));
+    return hpspmm_gen_rmat(sc, (int64_t)16 << sc, 0.57, 0.19, 0.19, 4);
+  }
+  g_err = "gen_named: unknown configuration '" + n + "'";
+  return nullptr;
+}
+
 // out[i] ~ N(0,1), Box-Muller on pairs (2p, 2p+1).
 void hpspmm_gen_dense_normal(uint64_t seed, int64_t count, float* out) {
   const int64_t pairs = (count + 1) / 2;

@@ -49,6 +49,7 @@ def lib():
         L.hpspmm_gen_community.argtypes = [_i64, _dbl, _dbl, _i64, _dbl, _i64, _u64]
         L.hpspmm_gen_community.restype = _p
         L.hpspmm_gen_rmat.argtypes, L.hpspmm_gen_rmat.restype = [ctypes.c_int, _i64, _dbl, _dbl, _dbl, _u64], _p
+        L.hpspmm_gen_named.argtypes, L.hpspmm_gen_named.restype = [ctypes.c_char_p, _dbl], _p
         L.hpspmm_gen_dense_normal.argtypes = [_u64, _i64, _p]
         L.hpspmm_gen_dense_uniform.argtypes = [_u64, _i64, ctypes.c_float, ctypes.c_float, _p]
         _lib = L
@@ -141,31 +142,11 @@ CONFIG_SEED = {"c0_uniform": 0, "c1_citation": 1, "c2_social": 2, "c3_copurchase
 
 
 def make_graph(name, scale=1.0):
-    """Build the sparse operand of a named benchmark configuration."""
-    seed = CONFIG_SEED[name]
-    if name == "c0_uniform":
-        n = max(16, int(round(4096 * scale)))
-        return uniform_rows(n, n, 16, seed)
-    if name == "c1_citation":
-        n = max(64, int(round(20000 * scale)))
-        return citation(n, 2.5, 70, int(round(2.05 * n)), seed)
-    if name == "c2_social":
-        n = max(64, int(round(232965 * scale)))
-        # i0 fixes the hub / mean weight ratio (max degree), n_edges the mean degree
-        return powerlaw(n, 2.1, max(4.0, 520.0 * scale), int(round(60.45e6 * scale)), seed)
-    if name == "c3_copurchase":
-        n = max(64, int(round(2449029 * scale)))
-        n_comm = max(1, int(round(65536 * scale)))
-        # 80 % of the edge *samples* are intra-community; communities of ~37
-        # vertices saturate, so more samples than stored edges are needed
-        return community(n, 3.5, 1.0, n_comm, 0.8, int(round(165.4e6 * scale)), seed)
-    if name == "c4_rmat":
-        if scale >= 1:
-            sc = 22
-        else:
-            sc = max(6, 22 + int(np.floor(np.log2(scale))))
-        return rmat(sc, 16 * (1 << sc), 0.57, 0.19, 0.19, seed)
-    raise KeyError(name)
+    """Build the sparse operand of a named benchmark configuration (parameters live in
+    hpspmm_gen_named, csrc/graphgen.cpp, shared with the C++ host layer)."""
+    if name not in CONFIG_SEED:
+        raise KeyError(name)
+    return _take(lib().hpspmm_gen_named(name.encode(), float(scale)))
 
 
 def make_dense(name, rows, k):

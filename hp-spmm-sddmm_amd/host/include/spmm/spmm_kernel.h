@@ -1,0 +1,25 @@
+// SpMM entry points of the host layer, with the signatures of
+// include/spmm/mm/spmm_kernel.h:17-21 of the reference.  Operands live in device
+// memory (Matrix on kHIP); `time` receives the mean milliseconds per launch over
+// EXE_NUM_CUDA back-to-back launches (spmm/mm/spmm_kernel.cu:404-424).
+#pragma once
+
+#include "spmm/spmm_common.h"
+#include "spmm/timer.h"
+
+// C = A * B for CSR A.  Stands in for GESpMM (spmm_kernel.cu:389-426): same
+// arguments, C overwritten.  Builds a plan (untimed, like the reference's host
+// preprocessing), runs WARMUP_NUM_CUDA + EXE_NUM_CUDA launches, frees the plan.
+void GESpMM(const CSR_Matrix& mat1, const Matrix& mat2, Matrix& result, float& time);
+// The same operation under the name of this library's own method.
+void HPSpMM(const CSR_Matrix& mat1, const Matrix& mat2, Matrix& result, float& time);
+// C += A * B for COO A, EXE_NUM_CUDA launches without re-zeroing, i.e. C ends up
+// as C0 + EXE_NUM_CUDA * A * B exactly like LBSpMM (spmm_kernel.cu:733-768).
+void LBSpMM(const COO_Matrix& mat1, const Matrix& mat2, Matrix& result, float& time);
+// Vendor comparator in the role of cusparseCSRSpMM (spmm_kernel.cu:36-151):
+// rocSPARSE CSR SpMM, alpha = 1, beta = 0, row-major B and C.  algid as in the
+// reference: 2, 3 or -1 (default).  Returns false (time = 0) when the library
+// call is not available.
+bool rocsparseCSRSpMM(const CSR_Matrix& mat1, const Matrix& mat2, Matrix& result, int algid, float& time);
+// x[i] = val on the device (spmm_kernel.cu:23-34).
+void fill_matrix(starml::Matrix& a, float val);

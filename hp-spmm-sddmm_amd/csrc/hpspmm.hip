@@ -68,6 +68,9 @@ struct hpspmm_plan {
   bool xcd_remap = true;
   int32_t* d_nnz_row = nullptr;  // [nnz]
   float* d_carry = nullptr;      // [2 * nseg * k]
+  int32_t* d_long_rows = nullptr;  // rows strategy: rows longer than long_threshold
+  int64_t n_long = 0;
+  int32_t long_threshold = INT32_MAX;
   int64_t workspace_bytes = 0;
 };
 
@@ -79,23 +82,28 @@ inline int64_t row_blocks(int64_t rows, int64_t k) {
   return ceil_div(ceil_div(rows, per_wave), hpspmm::kWavesPerBlock);
 }
 
+// Rows longer than this are handled by a whole wavefront in the rows strategy.
+constexpr int32_t kLongRowThreshold = 32;
+
 template <int K>
 int launch_rows(int64_t rows, const int32_t* rp, const int32_t* ci, const float* v, const float* B, float* C,
-                hipStream_t st) {
-  const int64_t blocks = row_blocks(rows, K);
+                int32_t long_threshold, const int32_t* long_rows, int64_t n_long, hipStream_t st) {
+  const int64_t short_blocks = row_blocks(rows, K);
+  const int64_t blocks = short_blocks + ceil_div(n_long, hpspmm::kWavesPerBlock);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   hipLaunchKernelGGL(hpspmm::spmm_rows_kernel<K>, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rows, rp, ci,
-                     v, B, C);
+                     v, B, C, short_blocks, long_threshold, long_rows, n_long);
   return HPSPMM_OK;
 }
 
 int launch_rows_any(int64_t rows, int64_t k, const int32_t* rp, const int32_t* ci, const float* v,
-                    const float* B, float* C, hipStream_t st) {
+                    const float* B, float* C, int32_t long_threshold, const int32_t* long_rows, int64_t n_long,
+                    hipStream_t st) {
   if (rows == 0) return HPSPMM_OK;
   switch (k) {
-    case 32: return launch_rows<32>(rows, rp, ci, v, B, C, st);
-    case 64: return launch_rows<64>(rows, rp, ci, v, B, C, st);
-    case 128: return launch_rows<128>(rows, rp, ci, v, B, C, st);
+    case 32: return launch_rows<32>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+    case 64: return launch_rows<64>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+    case 128: return launch_rows<128>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
     default: {
       const int64_t blocks = ceil_div(rows, hpspmm::kWavesPerBlock);
       hipLaunchKernelGGL(hpspmm::spmm_rows_generic_kernel, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st,
@@ -116,8 +124,9 @@ int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, 
     hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, false>), dim3((unsigned)grid), dim3(hpspmm::kBlock), 0, st,
                        rp, ci, v, p->d_nnz_row, B, C, p->d_carry, p->nnz, p->shift, p->nseg, nblocks,
                        p->xcd_remap);
-  hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)row_blocks(p->rows, K)), dim3(hpspmm::kBlock), 0,
-                     st, p->rows, rp, p->d_carry, C, p->shift);
+  const int64_t fix_blocks = ceil_div(ceil_div(p->rows, 64), hpspmm::kWavesPerBlock);
+  hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st, p->rows,
+                     rp, p->d_carry, C, p->shift);
   return HPSPMM_OK;
 }
 
@@ -215,10 +224,11 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d
   } else if (flags & HPSPMM_PLAN_FORCE_SEGMENTS) {
     p->strategy = HPSPMM_STRATEGY_SEGMENTS;
   } else {
-    // Whole rows when no row is long enough to unbalance the sub-waves and the
-    // matrix is small enough that a second (fix-up) launch would be felt.
+    // Whole rows (one launch; long rows get a wavefront each) when the matrix is
+    // small enough that a second (fix-up) launch would be felt and no row is so
+    // long that a single wavefront would be the critical path.
     const bool small = nnz < (1 << 21);
-    p->strategy = (nnz == 0 || (small && p->max_row_nnz <= 512)) ? HPSPMM_STRATEGY_ROWS : HPSPMM_STRATEGY_SEGMENTS;
+    p->strategy = (nnz == 0 || (small && p->max_row_nnz <= 4096)) ? HPSPMM_STRATEGY_ROWS : HPSPMM_STRATEGY_SEGMENTS;
   }
 
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS) {
@@ -247,6 +257,27 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d
       }
     }
   }
+  if (p->strategy == HPSPMM_STRATEGY_ROWS && p->max_row_nnz > kLongRowThreshold) {
+    // list of the rows that get a whole wavefront; d_meta[3] counts them
+    p->long_threshold = kLongRowThreshold;
+    const int64_t cap = nnz / (kLongRowThreshold + 1) + 1;  // cannot be more rows than that
+    if (hipMalloc(&p->d_long_rows, (size_t)cap * sizeof(int32_t)) != hipSuccess) {
+      (void)hipGetLastError();
+      hpspmm_plan_destroy(p);
+      return fail(HPSPMM_ERR_ALLOC, "device allocation of the long-row list failed");
+    }
+    p->workspace_bytes += cap * (int64_t)sizeof(int32_t);
+    hipLaunchKernelGGL(hpspmm::collect_long_rows_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)),
+                       dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, p->long_threshold, p->d_long_rows, d_meta + 3);
+    int32_t n_long = 0;
+    hipError_t e = hipMemcpyAsync(&n_long, d_meta + 3, sizeof n_long, hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess || n_long < 0 || n_long > cap) {
+      hpspmm_plan_destroy(p);
+      return fail(HPSPMM_ERR_HIP, "long-row collection failed: %s", hipGetErrorString(e));
+    }
+    p->n_long = n_long;
+  }
   *plan_out = p;
   return HPSPMM_OK;
 }
@@ -272,6 +303,7 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
   if (!plan) return HPSPMM_OK;
   if (plan->d_nnz_row) (void)hipFree(plan->d_nnz_row);
   if (plan->d_carry) (void)hipFree(plan->d_carry);
+  if (plan->d_long_rows) (void)hipFree(plan->d_long_rows);
   delete plan;
   return HPSPMM_OK;
 }
@@ -292,7 +324,8 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
       default: rc = launch_segments<128>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;
     }
   } else {
-    rc = launch_rows_any(plan->rows, plan->k, d_rowptr, d_col, d_val, d_B, d_C, st);
+    rc = launch_rows_any(plan->rows, plan->k, d_rowptr, d_col, d_val, d_B, d_C, plan->long_threshold,
+                         plan->d_long_rows, plan->n_long, st);
   }
   if (rc) return rc;
   HPSPMM_HIP(hipGetLastError());
@@ -307,7 +340,9 @@ int hpspmm_csr_spmm_noplan(int64_t rows, int64_t cols, int64_t nnz, const int32_
   if (!d_rowptr || !d_C) return fail(HPSPMM_ERR_INVALID_ARG, "d_rowptr or d_C is NULL");
   if (nnz > 0 && (!d_col || !d_val || !d_B))
     return fail(HPSPMM_ERR_INVALID_ARG, "d_col, d_val or d_B is NULL with nnz > 0");
-  if (int rc = launch_rows_any(rows, k, d_rowptr, d_col, d_val, d_B, d_C, (hipStream_t)stream)) return rc;
+  if (int rc = launch_rows_any(rows, k, d_rowptr, d_col, d_val, d_B, d_C, INT32_MAX, nullptr, 0,
+                               (hipStream_t)stream))
+    return rc;
   HPSPMM_HIP(hipGetLastError());
   return HPSPMM_OK;
 }

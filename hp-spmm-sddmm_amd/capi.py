@@ -24,6 +24,12 @@ PLAN_NO_VALIDATE = 1
 PLAN_FORCE_ROWS = 2
 PLAN_FORCE_SEGMENTS = 4
 PLAN_NO_XCD_REMAP = 8
+PLAN_HUB_CACHE = 16
+PLAN_NO_HUB_CACHE = 32
+
+
+def plan_hub_log2(log2_rows):
+    return (int(log2_rows) & 0xFF) << 16
 
 
 def plan_segment_shift(log2_len):
@@ -51,6 +57,7 @@ class PlanInfo(ctypes.Structure):
         ("strategy", ctypes.c_int32), ("segment_length", ctypes.c_int32),
         ("num_segments", _i64), ("max_row_nnz", _i64), ("empty_rows", _i64),
         ("workspace_bytes", _i64), ("launches_per_spmm", ctypes.c_int32), ("reserved", ctypes.c_int32),
+        ("hub_rows", _i64),
     ]
 
     def as_dict(self):

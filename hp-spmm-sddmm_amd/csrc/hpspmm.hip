@@ -4,12 +4,14 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <climits>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
 #include <new>
 #include <string>
+#include <vector>
 
 #include "spmm_kernels.hpp"
 
@@ -68,6 +70,11 @@ struct hpspmm_plan {
   bool xcd_remap = true;
   int32_t* d_nnz_row = nullptr;  // [nnz]
   float* d_carry = nullptr;      // [2 * nseg * k]
+  // hub cache (segments strategy, optional): the n_hub most referenced rows of B
+  int32_t* d_hub_ids = nullptr;  // [n_hub] column index of every cached row
+  int32_t* d_hub_col = nullptr;  // [nnz] column indices with cached columns rewritten as ~slot
+  float* d_bhot = nullptr;       // [n_hub * k]
+  int64_t n_hub = 0;
   int32_t* d_long_rows = nullptr;  // rows strategy: rows longer than long_threshold
   int64_t n_long = 0;
   int32_t long_threshold = INT32_MAX;
@@ -120,10 +127,20 @@ int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, 
   const int64_t nblocks = ceil_div(ceil_div(p->nseg, P), hpspmm::kWavesPerBlock);
   const int64_t grid = p->xcd_remap ? ceil_div(nblocks, hpspmm::kXcds) * hpspmm::kXcds : nblocks;
   if (grid > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
-  if (p->nnz > 0)
-    hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, false>), dim3((unsigned)grid), dim3(hpspmm::kBlock), 0, st,
-                       rp, ci, v, p->d_nnz_row, B, C, p->d_carry, p->nnz, p->shift, p->nseg, nblocks,
-                       p->xcd_remap);
+  if (p->nnz > 0) {
+    if (p->n_hub > 0) {
+      const int64_t threads = p->n_hub * (K / 4);
+      hipLaunchKernelGGL(hpspmm::gather_hub_rows_kernel<K>, dim3((unsigned)ceil_div(threads, hpspmm::kBlock)),
+                         dim3(hpspmm::kBlock), 0, st, p->n_hub, p->d_hub_ids, B, p->d_bhot);
+      hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, false, true>), dim3((unsigned)grid), dim3(hpspmm::kBlock),
+                         0, st, rp, p->d_hub_col, v, p->d_nnz_row, B, p->d_bhot, C, p->d_carry, p->nnz, p->shift,
+                         p->nseg, nblocks, p->xcd_remap);
+    } else {
+      hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, false, false>), dim3((unsigned)grid),
+                         dim3(hpspmm::kBlock), 0, st, rp, ci, v, p->d_nnz_row, B, (const float*)nullptr, C,
+                         p->d_carry, p->nnz, p->shift, p->nseg, nblocks, p->xcd_remap);
+    }
+  }
   const int64_t fix_blocks = ceil_div(ceil_div(p->rows, 64), hpspmm::kWavesPerBlock);
   hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st, p->rows,
                      rp, p->d_carry, C, p->shift);
@@ -140,8 +157,9 @@ int launch_coo(int64_t nnz, const int32_t* ri, const int32_t* ci, const float* v
   const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
   const int64_t nblocks = ceil_div(ceil_div(nseg, P), hpspmm::kWavesPerBlock);
   if (nblocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
-  hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, true>), dim3((unsigned)nblocks), dim3(hpspmm::kBlock), 0, st,
-                     (const int32_t*)nullptr, ci, v, ri, B, C, (float*)nullptr, nnz, shift, nseg, nblocks, false);
+  hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, true, false>), dim3((unsigned)nblocks), dim3(hpspmm::kBlock),
+                     0, st, (const int32_t*)nullptr, ci, v, ri, B, (const float*)nullptr, C, (float*)nullptr, nnz,
+                     shift, nseg, nblocks, false);
   return HPSPMM_OK;
 }
 
@@ -154,6 +172,61 @@ int choose_shift(int64_t nnz, int64_t k) {
   int shift = 5;
   while (shift < 9 && (nnz >> (shift + 1)) / subwaves >= target_waves) ++shift;
   return shift;
+}
+
+// Automatic hub cache: only when the cached rows would serve at least this share of the nonzeros.
+constexpr double kHubMinShare = 0.25;
+
+// Picks the most referenced columns of A (by nonzero count; ties by lower index, so
+// the choice is reproducible), gives each a slot in a compact copy of B and
+// rewrites the column array accordingly.  log2_hubs = 0 picks the default size.
+int build_hub_cache(hpspmm_plan* p, const int32_t* d_col, int log2_hubs, bool forced, hipStream_t st) {
+  if (log2_hubs == 0) log2_hubs = 16;
+  if (log2_hubs < 4 || log2_hubs > 24) return fail(HPSPMM_ERR_INVALID_ARG, "hub cache size 2^%d outside [2^4, 2^24]", log2_hubs);
+  const int64_t want = std::min<int64_t>((int64_t)1 << log2_hubs, p->cols);
+  int32_t* d_count = nullptr;
+  HPSPMM_HIP(hipMalloc(&d_count, (size_t)p->cols * sizeof(int32_t)));
+  struct Guard {
+    int32_t* q;
+    ~Guard() { (void)hipFree(q); }
+  } guard{d_count};
+  HPSPMM_HIP(hipMemsetAsync(d_count, 0, (size_t)p->cols * sizeof(int32_t), st));
+  hipLaunchKernelGGL(hpspmm::count_columns_kernel, dim3(grid_for(p->nnz, 1 << 16)), dim3(hpspmm::kBlock), 0, st,
+                     p->nnz, d_col, d_count);
+  std::vector<int32_t> count((size_t)p->cols);
+  HPSPMM_HIP(hipMemcpyAsync(count.data(), d_count, count.size() * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+
+  std::vector<int32_t> ids((size_t)p->cols);
+  for (int64_t i = 0; i < p->cols; ++i) ids[i] = (int32_t)i;
+  auto hotter = [&](int32_t a, int32_t b) { return count[a] != count[b] ? count[a] > count[b] : a < b; };
+  std::nth_element(ids.begin(), ids.begin() + (want - 1), ids.end(), hotter);
+  ids.resize((size_t)want);
+  std::sort(ids.begin(), ids.end(), hotter);
+  while (!ids.empty() && count[ids.back()] < 2) ids.pop_back();  // a row read once gains nothing
+  if (ids.empty()) return HPSPMM_OK;
+  if (!forced) {
+    // worth the extra column array only when the cached rows serve a good part of the gathers
+    int64_t served = 0;
+    for (int32_t c : ids) served += count[c];
+    if ((double)served < kHubMinShare * (double)p->nnz) return HPSPMM_OK;
+  }
+  std::vector<int32_t> colmap((size_t)p->cols, -1);
+  for (size_t s = 0; s < ids.size(); ++s) colmap[ids[s]] = (int32_t)s;
+
+  const int64_t n_hub = (int64_t)ids.size();
+  HPSPMM_HIP(hipMalloc(&p->d_hub_ids, (size_t)n_hub * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&p->d_hub_col, (size_t)p->nnz * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&p->d_bhot, (size_t)n_hub * (size_t)p->k * sizeof(float)));
+  p->workspace_bytes += n_hub * 4 + p->nnz * 4 + n_hub * p->k * 4;
+  HPSPMM_HIP(hipMemcpyAsync(p->d_hub_ids, ids.data(), (size_t)n_hub * sizeof(int32_t), hipMemcpyHostToDevice, st));
+  // the column-count buffer is reused for the column -> slot map
+  HPSPMM_HIP(hipMemcpyAsync(d_count, colmap.data(), colmap.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
+  hipLaunchKernelGGL(hpspmm::remap_columns_kernel, dim3(grid_for(p->nnz, 1 << 16)), dim3(hpspmm::kBlock), 0, st,
+                     p->nnz, d_col, d_count, p->d_hub_col);
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  p->n_hub = n_hub;
+  return HPSPMM_OK;
 }
 
 }  // namespace
@@ -257,6 +330,12 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d
       }
     }
   }
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && !(flags & HPSPMM_PLAN_NO_HUB_CACHE) && nnz > 0) {
+    if (int rc = build_hub_cache(p, d_col, (int)((flags >> 16) & 0xFFu), (flags & HPSPMM_PLAN_HUB_CACHE) != 0, st)) {
+      hpspmm_plan_destroy(p);
+      return rc;
+    }
+  }
   if (p->strategy == HPSPMM_STRATEGY_ROWS && p->max_row_nnz > kLongRowThreshold) {
     // list of the rows that get a whole wavefront; d_meta[3] counts them
     p->long_threshold = kLongRowThreshold;
@@ -295,7 +374,8 @@ int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
   out->max_row_nnz = plan->max_row_nnz;
   out->empty_rows = plan->empty_rows;
   out->workspace_bytes = plan->workspace_bytes;
-  out->launches_per_spmm = plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? 2 : 1;
+  out->launches_per_spmm = plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? (plan->n_hub > 0 ? 3 : 2) : 1;
+  out->hub_rows = plan->n_hub;
   return HPSPMM_OK;
 }
 
@@ -304,6 +384,9 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
   if (plan->d_nnz_row) (void)hipFree(plan->d_nnz_row);
   if (plan->d_carry) (void)hipFree(plan->d_carry);
   if (plan->d_long_rows) (void)hipFree(plan->d_long_rows);
+  if (plan->d_hub_ids) (void)hipFree(plan->d_hub_ids);
+  if (plan->d_hub_col) (void)hipFree(plan->d_hub_col);
+  if (plan->d_bhot) (void)hipFree(plan->d_bhot);
   delete plan;
   return HPSPMM_OK;
 }

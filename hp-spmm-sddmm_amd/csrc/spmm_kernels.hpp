@@ -58,6 +58,22 @@ __device__ __forceinline__ float4 load_b(const float* __restrict__ B, int32_t c,
   return *reinterpret_cast<const float4*>(B + (uint64_t)(uint32_t)c * (uint64_t)K + (uint32_t)(4 * l));
 }
 
+// Hub cache: the plan may keep the most referenced rows of B in a compact
+// buffer (refreshed at the start of every SpMM) and rewrite their column
+// indices as ~slot (negative).  A negative index reads the compact buffer.
+template <int K, bool kHub>
+__device__ __forceinline__ float4 load_b_hub(const float* __restrict__ B, const float* __restrict__ Bhot, int32_t c,
+                                             int l) {
+  if constexpr (kHub) {
+    const bool hot = c < 0;
+    const float* base = hot ? Bhot : B;
+    const uint32_t idx = hot ? (uint32_t)~c : (uint32_t)c;
+    return *reinterpret_cast<const float4*>(base + (uint64_t)idx * (uint64_t)K + (uint32_t)(4 * l));
+  } else {
+    return load_b<K>(B, c, l);
+  }
+}
+
 // Workgroups are dealt to the XCDs round-robin (workgroup b runs on XCD
 // b % 8).  Remapping so that XCD x receives the x-th contiguous eighth of the
 // logical workgroups keeps neighbouring rows (similar column sets) behind one
@@ -232,11 +248,12 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_generic_kernel(int64_t rows,
 // kAtomic = true is the COO "accumulate" form: no carry buffer, every flush is
 // an FP32 atomic add into C, rows may come in any order.
 // ---------------------------------------------------------------------------
-template <int K, bool kAtomic>
+template <int K, bool kAtomic, bool kHub>
 __global__ __launch_bounds__(kBlock) void spmm_segments_kernel(
     const int32_t* __restrict__ rowptr, const int32_t* __restrict__ col, const float* __restrict__ val,
-    const int32_t* __restrict__ nnz_row, const float* __restrict__ B, float* __restrict__ C,
-    float* __restrict__ carry, int64_t nnz, int shift, int64_t nseg, int64_t nblocks, bool remap) {
+    const int32_t* __restrict__ nnz_row, const float* __restrict__ B, const float* __restrict__ Bhot,
+    float* __restrict__ C, float* __restrict__ carry, int64_t nnz, int shift, int64_t nseg, int64_t nblocks,
+    bool remap) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
   constexpr int U = G < kBatch ? G : kBatch;
@@ -298,7 +315,7 @@ __global__ __launch_bounds__(kBlock) void spmm_segments_kernel(
         r[i] = s_row[base + u + i];
       }
 #pragma unroll
-      for (int i = 0; i < U; ++i) b[i] = load_b<K>(B, c[i], l);
+      for (int i = 0; i < U; ++i) b[i] = load_b_hub<K, kHub>(B, Bhot, c[i], l);
 #pragma unroll
       for (int i = 0; i < U; ++i) {
         if (r[i] != cur) {
@@ -311,7 +328,7 @@ __global__ __launch_bounds__(kBlock) void spmm_segments_kernel(
     }
     for (; u < cnt; ++u) {
       const int32_t r = s_row[base + u];
-      const float4 b = load_b<K>(B, s_col[base + u], l);
+      const float4 b = load_b_hub<K, kHub>(B, Bhot, s_col[base + u], l);
       if (r != cur) {
         flush(false);
         acc = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -466,6 +483,38 @@ __global__ __launch_bounds__(kBlock) void collect_long_rows_kernel(int64_t rows,
   if (lane == 0) base = atomicAdd(count, (int32_t)__popcll(mask));
   base = __shfl(base, 0);
   if (is_long) list[base + __popcll(mask & ((1ull << lane) - 1ull))] = (int32_t)i;
+}
+
+// count[c] = number of nonzeros in column c (count[] zeroed by the caller).
+__global__ __launch_bounds__(kBlock) void count_columns_kernel(int64_t nnz, const int32_t* __restrict__ col,
+                                                               int32_t* __restrict__ count) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < nnz; j += stride) atomicAdd(&count[col[j]], 1);
+}
+
+// out[j] = ~slot if column col[j] is cached in slot colmap[col[j]] >= 0, else col[j].
+__global__ __launch_bounds__(kBlock) void remap_columns_kernel(int64_t nnz, const int32_t* __restrict__ col,
+                                                               const int32_t* __restrict__ colmap,
+                                                               int32_t* __restrict__ out) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < nnz; j += stride) {
+    const int32_t c = col[j];
+    const int32_t slot = colmap[c];
+    out[j] = slot >= 0 ? ~slot : c;
+  }
+}
+
+// Bhot[s, :] = B[hub_ids[s], :] for s in [0, n_hub): one sub-wave per row.
+template <int K>
+__global__ __launch_bounds__(kBlock) void gather_hub_rows_kernel(int64_t n_hub, const int32_t* __restrict__ hub_ids,
+                                                                 const float* __restrict__ B,
+                                                                 float* __restrict__ Bhot) {
+  constexpr int G = K / 4;
+  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t s = t / G;
+  const int l = (int)(t % G);
+  if (s >= n_hub) return;
+  *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) = load_b<K>(B, hub_ids[s], l);
 }
 
 // nnz_row[j] = the row r with rowptr[r] <= j < rowptr[r+1] (CSR -> COO row

@@ -54,6 +54,11 @@ typedef enum hpspmm_status {
 #define HPSPMM_PLAN_FORCE_ROWS 2u     /* always use the whole-row kernel */
 #define HPSPMM_PLAN_FORCE_SEGMENTS 4u /* always use the nnz-segment kernel + carry fix-up */
 #define HPSPMM_PLAN_NO_XCD_REMAP 8u   /* keep the hardware's round-robin workgroup->XCD order */
+#define HPSPMM_PLAN_HUB_CACHE 16u     /* segments strategy: always keep the most referenced rows of B in a compact
+                                         copy (default: only when they serve >= 25 % of the nonzeros) */
+#define HPSPMM_PLAN_NO_HUB_CACHE 32u  /* never build the hub cache */
+/* bits 16..23: log2 of the number of cached rows (0 = default, 2^16) */
+#define HPSPMM_PLAN_HUB_LOG2(log2_rows) (((uint32_t)(log2_rows) & 0xFFu) << 16)
 /* bits 8..15: log2 of the segment length to force (0 = choose automatically) */
 #define HPSPMM_PLAN_SEGMENT_SHIFT(log2_len) (((uint32_t)(log2_len) & 0xFFu) << 8)
 
@@ -74,6 +79,7 @@ typedef struct hpspmm_plan_info {
   int64_t workspace_bytes; /* device memory owned by the plan */
   int32_t launches_per_spmm;
   int32_t reserved;
+  int64_t hub_rows;        /* rows of B kept in the hub cache (0 = none) */
 } hpspmm_plan_info;
 
 /* Library version, major*10000 + minor*100 + patch. */

@@ -49,8 +49,11 @@ def _check(oracle, g, B, C, what=""):
 def _strategies(capi):
     return [("auto", capi.PLAN_DEFAULT), ("rows", capi.PLAN_FORCE_ROWS),
             ("seg", capi.PLAN_FORCE_SEGMENTS),
-            ("seg8", capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(3)),
-            ("seg64_noremap", capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(6) | capi.PLAN_NO_XCD_REMAP)]
+            ("seg8_nohub", capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(3) | capi.PLAN_NO_HUB_CACHE),
+            ("seg64_noremap", capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(6) | capi.PLAN_NO_XCD_REMAP),
+            ("seg_hub", capi.PLAN_FORCE_SEGMENTS | capi.PLAN_HUB_CACHE | capi.plan_hub_log2(8)),
+            ("seg16_hub_all", capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(4) | capi.PLAN_HUB_CACHE
+             | capi.plan_hub_log2(24))]
 
 
 @pytest.mark.parametrize("k", [32, 64, 128])

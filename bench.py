@@ -204,7 +204,11 @@ def main():
             if (name, k) == ROOFLINE_WORKLOAD:
                 roofline = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                             "frac": gbs / HBM_PEAK_GBS, "traffic": None,
-                            "kernel": "spmm_segments_kernel<128> + spmm_fixup_kernel<128> (one SpMM)",
+                            "kernel": {1: "spmm_rows_kernel<128>",
+                                       2: "spmm_segments_kernel<128> + spmm_fixup_kernel<128>",
+                                       4: "routed_gather_hub_kernel<128> + spmm_routed_kernel<128> + "
+                                          "spmm_routed_final_kernel<128>"}.get(info["strategy"], "?")
+                                      + " (all launches of one SpMM)",
                             "workload": f"{name} K={k}", "algorithmic_bytes_per_launch": abytes,
                             "mean_launch_ms": ms}
                 if not args.no_cpu_baseline:

@@ -26,6 +26,8 @@ PLAN_FORCE_SEGMENTS = 4
 PLAN_NO_XCD_REMAP = 8
 PLAN_HUB_CACHE = 16
 PLAN_NO_HUB_CACHE = 32
+PLAN_FORCE_ROUTED = 64
+PLAN_NO_ROUTED = 128
 
 
 def plan_hub_log2(log2_rows):
@@ -39,6 +41,7 @@ def plan_segment_shift(log2_len):
 STRATEGY_ROWS = 1
 STRATEGY_SEGMENTS = 2
 STRATEGY_GENERIC_K = 3
+STRATEGY_ROUTED = 4
 
 # every symbol include/hpspmm.h declares
 EXPORTS = (

@@ -13,6 +13,7 @@
 #include <string>
 #include <vector>
 
+#include "routed_kernels.hpp"
 #include "spmm_kernels.hpp"
 
 namespace {
@@ -40,6 +41,10 @@ int fail(int code, const char* fmt, ...) {
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 inline bool fast_k(int64_t k) { return k == 32 || k == 64 || k == 128; }
+
+inline bool aligned16(const void* a, const void* b, const void* c) {
+  return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15u) == 0;
+}
 
 int check_dims(int64_t rows, int64_t cols, int64_t nnz, int64_t k) {
   if (rows < 0 || cols < 0 || nnz < 0) return fail(HPSPMM_ERR_INVALID_ARG, "negative dimension (rows=%lld cols=%lld nnz=%lld)",
@@ -75,6 +80,17 @@ struct hpspmm_plan {
   int32_t* d_hub_col = nullptr;  // [nnz] column indices with cached columns rewritten as ~slot
   float* d_bhot = nullptr;       // [n_hub * k]
   int64_t n_hub = 0;
+  // routed strategy
+  hpspmm::RoutedLayout lay{};
+  int32_t* d_vptr = nullptr;      // [9 * (rows + 1)]
+  int32_t* d_vcol = nullptr;      // [vtotal] column, or compact-buffer row for hub classes
+  int32_t* d_vsrc = nullptr;      // [vtotal] index into the caller's value array
+  int32_t* d_vrow = nullptr;      // [vtotal]
+  int32_t* d_bhot_src = nullptr;  // [n_bhot] source column of every compact-buffer row (-1 = unused)
+  uint8_t* d_action = nullptr;    // [rows] what the final kernel does with each row
+  float* d_partial = nullptr;     // [9 * rows * k]
+  int64_t n_bhot = 0;
+  int64_t routed_grid = 0;
   int32_t* d_long_rows = nullptr;  // rows strategy: rows longer than long_threshold
   int64_t n_long = 0;
   int32_t long_threshold = INT32_MAX;
@@ -134,11 +150,12 @@ int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, 
                          dim3(hpspmm::kBlock), 0, st, p->n_hub, p->d_hub_ids, B, p->d_bhot);
       hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, false, true>), dim3((unsigned)grid), dim3(hpspmm::kBlock),
                          0, st, rp, p->d_hub_col, v, p->d_nnz_row, B, p->d_bhot, C, p->d_carry, p->nnz, p->shift,
-                         p->nseg, nblocks, p->xcd_remap);
+                         p->nseg, nblocks, p->xcd_remap, aligned16(p->d_hub_col, v, p->d_nnz_row));
     } else {
       hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, false, false>), dim3((unsigned)grid),
                          dim3(hpspmm::kBlock), 0, st, rp, ci, v, p->d_nnz_row, B, (const float*)nullptr, C,
-                         p->d_carry, p->nnz, p->shift, p->nseg, nblocks, p->xcd_remap);
+                         p->d_carry, p->nnz, p->shift, p->nseg, nblocks, p->xcd_remap,
+                         aligned16(ci, v, p->d_nnz_row));
     }
   }
   const int64_t fix_blocks = ceil_div(ceil_div(p->rows, 64), hpspmm::kWavesPerBlock);
@@ -159,7 +176,7 @@ int launch_coo(int64_t nnz, const int32_t* ri, const int32_t* ci, const float* v
   if (nblocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, true, false>), dim3((unsigned)nblocks), dim3(hpspmm::kBlock),
                      0, st, (const int32_t*)nullptr, ci, v, ri, B, (const float*)nullptr, C, (float*)nullptr, nnz,
-                     shift, nseg, nblocks, false);
+                     shift, nseg, nblocks, false, aligned16(ci, v, ri));
   return HPSPMM_OK;
 }
 
@@ -174,16 +191,11 @@ int choose_shift(int64_t nnz, int64_t k) {
   return shift;
 }
 
-// Automatic hub cache: only when the cached rows would serve at least this share of the nonzeros.
-constexpr double kHubMinShare = 0.25;
-
-// Picks the most referenced columns of A (by nonzero count; ties by lower index, so
-// the choice is reproducible), gives each a slot in a compact copy of B and
-// rewrites the column array accordingly.  log2_hubs = 0 picks the default size.
-int build_hub_cache(hpspmm_plan* p, const int32_t* d_col, int log2_hubs, bool forced, hipStream_t st) {
-  if (log2_hubs == 0) log2_hubs = 16;
-  if (log2_hubs < 4 || log2_hubs > 24) return fail(HPSPMM_ERR_INVALID_ARG, "hub cache size 2^%d outside [2^4, 2^24]", log2_hubs);
-  const int64_t want = std::min<int64_t>((int64_t)1 << log2_hubs, p->cols);
+// Column popularity: count[c] = nonzeros in column c, and the `want` most
+// referenced columns in order of decreasing count (ties by lower index, so the
+// choice is reproducible); columns referenced fewer than twice are dropped.
+int rank_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t want, hipStream_t st,
+                 std::vector<int32_t>& count, std::vector<int32_t>& ids) {
   int32_t* d_count = nullptr;
   HPSPMM_HIP(hipMalloc(&d_count, (size_t)p->cols * sizeof(int32_t)));
   struct Guard {
@@ -193,17 +205,189 @@ int build_hub_cache(hpspmm_plan* p, const int32_t* d_col, int log2_hubs, bool fo
   HPSPMM_HIP(hipMemsetAsync(d_count, 0, (size_t)p->cols * sizeof(int32_t), st));
   hipLaunchKernelGGL(hpspmm::count_columns_kernel, dim3(grid_for(p->nnz, 1 << 16)), dim3(hpspmm::kBlock), 0, st,
                      p->nnz, d_col, d_count);
-  std::vector<int32_t> count((size_t)p->cols);
+  count.resize((size_t)p->cols);
   HPSPMM_HIP(hipMemcpyAsync(count.data(), d_count, count.size() * sizeof(int32_t), hipMemcpyDeviceToHost, st));
   HPSPMM_HIP(hipStreamSynchronize(st));
-
-  std::vector<int32_t> ids((size_t)p->cols);
+  want = std::min<int64_t>(want, p->cols);
+  ids.resize((size_t)p->cols);
   for (int64_t i = 0; i < p->cols; ++i) ids[i] = (int32_t)i;
   auto hotter = [&](int32_t a, int32_t b) { return count[a] != count[b] ? count[a] > count[b] : a < b; };
-  std::nth_element(ids.begin(), ids.begin() + (want - 1), ids.end(), hotter);
+  if (want < p->cols) std::nth_element(ids.begin(), ids.begin() + (want - 1), ids.end(), hotter);
   ids.resize((size_t)want);
   std::sort(ids.begin(), ids.end(), hotter);
-  while (!ids.empty() && count[ids.back()] < 2) ids.pop_back();  // a row read once gains nothing
+  while (!ids.empty() && count[ids.back()] < 2) ids.pop_back();
+  return HPSPMM_OK;
+}
+
+// Device exclusive scan of n uint32 values (three passes, tile sums in between).
+int exclusive_scan_u32(const uint32_t* d_in, uint32_t* d_out, int64_t n, hipStream_t st) {
+  const int64_t ntiles = ceil_div(n, hpspmm::kScanTile);
+  if (ntiles > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "scan too large");
+  uint32_t* d_tiles = nullptr;
+  HPSPMM_HIP(hipMalloc(&d_tiles, (size_t)ntiles * sizeof(uint32_t)));
+  hipLaunchKernelGGL(hpspmm::scan_tile_sums_kernel, dim3((unsigned)ntiles), dim3(hpspmm::kBlock), 0, st, n, d_in,
+                     d_tiles);
+  hipLaunchKernelGGL(hpspmm::scan_tile_offsets_kernel, dim3(1), dim3(hpspmm::kBlock), 0, st, ntiles, d_tiles);
+  hipLaunchKernelGGL(hpspmm::scan_apply_kernel, dim3((unsigned)ntiles), dim3(hpspmm::kBlock), 0, st, n, d_in, d_tiles,
+                     d_out);
+  hipError_t e = hipStreamSynchronize(st);
+  (void)hipFree(d_tiles);
+  if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "scan failed: %s", hipGetErrorString(e));
+  return HPSPMM_OK;
+}
+
+// Rows of B kept in the compact buffer by the routed strategy (all slices together).
+constexpr int kRoutedLog2Cached = 16;
+// Automatic choice of the routed strategy (thresholds from measurements on the
+// benchmark graphs: it pays on the 233k-vertex social graph at K = 64 and 128
+// (2.95 -> 2.31 ms, 6.6 -> 4.5 ms) and on the R-MAT graph (8.6 -> 7.9 ms); not at
+// K = 32 on the social graph, where B already fits the L2s, and not on the
+// co-purchase graph, whose columns are too evenly used (4.5 -> 5.5 ms)).
+constexpr int64_t kRoutedMinNnz = (int64_t)1 << 22;
+constexpr int64_t kRoutedMinBBytes = (int64_t)48 << 20;  // B must overflow the 8 x 4 MB of L2
+constexpr double kRoutedMinShare = 0.35;     // of the nonzeros in the 64k most referenced columns
+constexpr double kRoutedMinRowNnz = 32.0;    // mean nonzeros per non-empty row
+constexpr int32_t kRoutedRowThreshold = 64;  // rows shorter than this are not split over the classes
+
+// Builds the routed layout.  Returns HPSPMM_OK with p->strategy left at
+// SEGMENTS when the graph does not qualify (and `forced` is false).
+int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, int log2_hubs,
+                 hipStream_t st) {
+  const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
+  if (!forced && (nnz < kRoutedMinNnz || p->cols * k * 4 < kRoutedMinBBytes)) return HPSPMM_OK;
+  // cached rows per class
+  const int64_t h =
+      std::max<int64_t>(1, ((int64_t)1 << (log2_hubs ? log2_hubs : kRoutedLog2Cached)) / hpspmm::kHubClasses);
+  std::vector<int32_t> count, ids;
+  if (int rc = rank_columns(p, d_col, h * hpspmm::kHubClasses, st, count, ids)) return rc;
+  int64_t served = 0;
+  for (int32_t c : ids) served += count[c];
+  const int64_t nonempty = std::max<int64_t>(1, rows - p->empty_rows);
+  if (!forced && ((double)served < kRoutedMinShare * (double)nnz ||
+                  (double)nnz / (double)nonempty < kRoutedMinRowNnz))
+    return HPSPMM_OK;
+  if (nnz > INT32_MAX - ((int64_t)1 << 24)) return HPSPMM_OK;  // virtual indices stay int32
+
+  // popularity rank s -> class s % 8, compact-buffer row (s % 8) * h + s / 8
+  const int64_t n_bhot = h * hpspmm::kHubClasses;
+  std::vector<int32_t> colmap((size_t)p->cols, -1), bhot_src((size_t)n_bhot, -1);
+  for (size_t s2 = 0; s2 < ids.size(); ++s2) {
+    const int64_t slot = (int64_t)(s2 % hpspmm::kHubClasses) * h + (int64_t)(s2 / hpspmm::kHubClasses);
+    colmap[ids[s2]] = (int32_t)slot;
+    bhot_src[(size_t)slot] = ids[s2];
+  }
+
+  int32_t* d_colmap = nullptr;
+  uint32_t* d_cnt = nullptr;
+  uint32_t* d_scan = nullptr;
+  struct Guard {
+    void** q[3];
+    ~Guard() {
+      for (void** x : q)
+        if (*x) (void)hipFree(*x);
+    }
+  } guard{{(void**)&d_colmap, (void**)&d_cnt, (void**)&d_scan}};
+  const int64_t ncnt = rows * hpspmm::kClasses;
+  HPSPMM_HIP(hipMalloc(&d_colmap, (size_t)std::max<int64_t>(1, p->cols) * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&d_cnt, (size_t)ncnt * sizeof(uint32_t)));
+  HPSPMM_HIP(hipMalloc(&d_scan, (size_t)ncnt * sizeof(uint32_t)));
+  HPSPMM_HIP(hipMemcpyAsync(d_colmap, colmap.data(), colmap.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
+  const unsigned row_grid = (unsigned)ceil_div(rows, hpspmm::kWavesPerBlock);
+  const int32_t min_row_nnz = forced && log2_hubs ? 2 : kRoutedRowThreshold;  // forced small hub sets: tests
+  hipLaunchKernelGGL(hpspmm::routed_count_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col,
+                     d_colmap, (int32_t)h, min_row_nnz, d_cnt);
+  if (int rc = exclusive_scan_u32(d_cnt, d_scan, ncnt, st)) return rc;
+
+  // class sizes = differences of the scan at the class origins
+  uint32_t origin[hpspmm::kClasses];
+  for (int x = 0; x < hpspmm::kClasses; ++x)
+    HPSPMM_HIP(hipMemcpyAsync(&origin[x], d_scan + (int64_t)x * rows, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+
+  hpspmm::RoutedLayout& lay = p->lay;
+  lay.rows = rows;
+  lay.shift = p->shift;
+  const int64_t subwaves = 64 / (k / 4);
+  const int64_t quantum = ((int64_t)1 << p->shift) * subwaves * hpspmm::kWavesPerBlock;  // nonzeros per workgroup
+  int64_t at = 0, hub_blocks = 0;
+  for (int x = 0; x < hpspmm::kClasses; ++x) {
+    const int64_t n_x = (x + 1 < hpspmm::kClasses ? (int64_t)origin[x + 1] : nnz) - (int64_t)origin[x];
+    lay.cls_begin[x] = at;
+    lay.cls_end[x] = at + n_x;
+    lay.cls_blocks[x] = ceil_div(n_x, quantum);
+    at += lay.cls_blocks[x] * quantum;
+    if (x < hpspmm::kHubClasses) hub_blocks = std::max(hub_blocks, lay.cls_blocks[x]);
+  }
+  const int64_t vtotal = std::max<int64_t>(at, 1);
+  lay.hub_grid = hub_blocks * hpspmm::kHubClasses;
+  p->routed_grid = lay.hub_grid + lay.cls_blocks[hpspmm::kColdClass];
+  if (vtotal >= INT32_MAX || p->routed_grid > INT32_MAX) return HPSPMM_OK;
+
+  const int64_t nseg = vtotal >> p->shift;
+  const size_t vptr_bytes = (size_t)hpspmm::kClasses * (size_t)(rows + 1) * sizeof(int32_t);
+  const size_t v_bytes = (size_t)vtotal * sizeof(int32_t);
+  const size_t partial_bytes = (size_t)hpspmm::kClasses * (size_t)rows * (size_t)k * sizeof(float);
+  const size_t carry_bytes = (size_t)std::max<int64_t>(nseg, 1) * 2 * (size_t)k * sizeof(float);
+  const size_t bhot_bytes = (size_t)n_bhot * (size_t)k * sizeof(float);
+  // the segments strategy's buffers are not needed any more
+  if (p->d_nnz_row) { (void)hipFree(p->d_nnz_row); p->d_nnz_row = nullptr; }
+  if (p->d_carry) { (void)hipFree(p->d_carry); p->d_carry = nullptr; }
+  if (hipMalloc(&p->d_vptr, vptr_bytes) != hipSuccess || hipMalloc(&p->d_vcol, v_bytes) != hipSuccess ||
+      hipMalloc(&p->d_vsrc, v_bytes) != hipSuccess || hipMalloc(&p->d_vrow, v_bytes) != hipSuccess ||
+      hipMalloc(&p->d_partial, partial_bytes) != hipSuccess || hipMalloc(&p->d_carry, carry_bytes) != hipSuccess ||
+      hipMalloc(&p->d_bhot, bhot_bytes) != hipSuccess ||
+      hipMalloc(&p->d_bhot_src, (size_t)n_bhot * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&p->d_action, (size_t)rows) != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(HPSPMM_ERR_ALLOC, "device allocation for the routed plan failed (%zu bytes)",
+                vptr_bytes + 3 * v_bytes + partial_bytes + carry_bytes + bhot_bytes);
+  }
+  p->workspace_bytes = (int64_t)(vptr_bytes + 3 * v_bytes + partial_bytes + carry_bytes + bhot_bytes + n_bhot * 4);
+  HPSPMM_HIP(hipMemcpyAsync(p->d_bhot_src, bhot_src.data(), bhot_src.size() * sizeof(int32_t),
+                            hipMemcpyHostToDevice, st));
+  // unused compact-buffer rows are never read; keep them defined anyway
+  HPSPMM_HIP(hipMemsetAsync(p->d_bhot, 0, bhot_bytes, st));
+  const int64_t nvptr = (int64_t)hpspmm::kClasses * (rows + 1);
+  hipLaunchKernelGGL(hpspmm::routed_vptr_kernel, dim3((unsigned)ceil_div(nvptr, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, lay, d_scan, p->d_vptr);
+  hipLaunchKernelGGL(hpspmm::routed_fill_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col,
+                     d_colmap, (int32_t)h, min_row_nnz, p->d_vptr, p->d_vcol, p->d_vsrc, p->d_vrow, p->d_action,
+                     p->shift);
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  HPSPMM_HIP(hipGetLastError());
+  p->n_bhot = n_bhot;
+  p->n_hub = (int64_t)ids.size();
+  p->nseg = nseg;
+  p->strategy = HPSPMM_STRATEGY_ROUTED;
+  return HPSPMM_OK;
+}
+
+template <int K>
+int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
+  const int64_t threads = p->n_bhot * (K / 4);
+  hipLaunchKernelGGL(hpspmm::routed_gather_hub_kernel<K>, dim3((unsigned)ceil_div(threads, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, p->n_bhot, p->d_bhot_src, B, p->d_bhot);
+  if (p->routed_grid > 0)
+    hipLaunchKernelGGL(hpspmm::spmm_routed_kernel<K>, dim3((unsigned)p->routed_grid), dim3(hpspmm::kBlock), 0, st,
+                       p->lay, p->d_vptr, p->d_vcol, p->d_vsrc, p->d_vrow, v, B, p->d_bhot, p->d_partial,
+                       p->d_carry, C);
+  const int64_t fin_blocks = ceil_div(ceil_div(p->rows, 64), hpspmm::kWavesPerBlock);
+  hipLaunchKernelGGL(hpspmm::spmm_routed_final_kernel<K>, dim3((unsigned)fin_blocks), dim3(hpspmm::kBlock), 0, st,
+                     p->lay, p->d_vptr, p->d_action, p->d_partial, p->d_carry, C);
+  return HPSPMM_OK;
+}
+
+// Automatic hub cache: only when the cached rows would serve at least this share of the nonzeros.
+constexpr double kHubMinShare = 0.25;
+
+// Picks the most referenced columns of A (by nonzero count; ties by lower index, so
+// the choice is reproducible), gives each a slot in a compact copy of B and
+// rewrites the column array accordingly.  log2_hubs = 0 picks the default size.
+int build_hub_cache(hpspmm_plan* p, const int32_t* d_col, int log2_hubs, bool forced, hipStream_t st) {
+  if (log2_hubs == 0) log2_hubs = 16;
+  if (log2_hubs < 4 || log2_hubs > 24) return fail(HPSPMM_ERR_INVALID_ARG, "hub cache size 2^%d outside [2^4, 2^24]", log2_hubs);
+  std::vector<int32_t> count, ids;
+  if (int rc = rank_columns(p, d_col, (int64_t)1 << log2_hubs, st, count, ids)) return rc;
   if (ids.empty()) return HPSPMM_OK;
   if (!forced) {
     // worth the extra column array only when the cached rows serve a good part of the gathers
@@ -220,11 +404,16 @@ int build_hub_cache(hpspmm_plan* p, const int32_t* d_col, int log2_hubs, bool fo
   HPSPMM_HIP(hipMalloc(&p->d_bhot, (size_t)n_hub * (size_t)p->k * sizeof(float)));
   p->workspace_bytes += n_hub * 4 + p->nnz * 4 + n_hub * p->k * 4;
   HPSPMM_HIP(hipMemcpyAsync(p->d_hub_ids, ids.data(), (size_t)n_hub * sizeof(int32_t), hipMemcpyHostToDevice, st));
-  // the column-count buffer is reused for the column -> slot map
-  HPSPMM_HIP(hipMemcpyAsync(d_count, colmap.data(), colmap.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
-  hipLaunchKernelGGL(hpspmm::remap_columns_kernel, dim3(grid_for(p->nnz, 1 << 16)), dim3(hpspmm::kBlock), 0, st,
-                     p->nnz, d_col, d_count, p->d_hub_col);
-  HPSPMM_HIP(hipStreamSynchronize(st));
+  int32_t* d_colmap = nullptr;
+  HPSPMM_HIP(hipMalloc(&d_colmap, colmap.size() * sizeof(int32_t)));
+  hipError_t e = hipMemcpyAsync(d_colmap, colmap.data(), colmap.size() * sizeof(int32_t), hipMemcpyHostToDevice, st);
+  if (e == hipSuccess) {
+    hipLaunchKernelGGL(hpspmm::remap_columns_kernel, dim3(grid_for(p->nnz, 1 << 16)), dim3(hpspmm::kBlock), 0, st,
+                       p->nnz, d_col, d_colmap, p->d_hub_col);
+    e = hipStreamSynchronize(st);
+  }
+  (void)hipFree(d_colmap);
+  if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "column remap failed: %s", hipGetErrorString(e));
   p->n_hub = n_hub;
   return HPSPMM_OK;
 }
@@ -294,8 +483,8 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d
     p->strategy = HPSPMM_STRATEGY_GENERIC_K;
   } else if (flags & HPSPMM_PLAN_FORCE_ROWS) {
     p->strategy = HPSPMM_STRATEGY_ROWS;
-  } else if (flags & HPSPMM_PLAN_FORCE_SEGMENTS) {
-    p->strategy = HPSPMM_STRATEGY_SEGMENTS;
+  } else if (flags & (HPSPMM_PLAN_FORCE_SEGMENTS | HPSPMM_PLAN_FORCE_ROUTED)) {
+    p->strategy = HPSPMM_STRATEGY_SEGMENTS;  // the routed layout is built on top of it below
   } else {
     // Whole rows (one launch; long rows get a wavefront each) when the matrix is
     // small enough that a second (fix-up) launch would be felt and no row is so
@@ -328,6 +517,14 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d
         hpspmm_plan_destroy(p);
         return fail(HPSPMM_ERR_HIP, "row expansion failed: %s", hipGetErrorString(e));
       }
+    }
+  }
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && !(flags & HPSPMM_PLAN_NO_ROUTED) && nnz > 0 &&
+      !(flags & HPSPMM_PLAN_FORCE_SEGMENTS && !(flags & HPSPMM_PLAN_FORCE_ROUTED))) {
+    if (int rc = build_routed(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_ROUTED) != 0,
+                              (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 16) & 0xFFu) : 0, st)) {
+      hpspmm_plan_destroy(p);
+      return rc;
     }
   }
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && !(flags & HPSPMM_PLAN_NO_HUB_CACHE) && nnz > 0) {
@@ -369,12 +566,14 @@ int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
   out->nnz = plan->nnz;
   out->k = plan->k;
   out->strategy = plan->strategy;
-  out->segment_length = plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? (1 << plan->shift) : 0;
+  const bool segmented = plan->strategy == HPSPMM_STRATEGY_SEGMENTS || plan->strategy == HPSPMM_STRATEGY_ROUTED;
+  out->segment_length = segmented ? (1 << plan->shift) : 0;
   out->num_segments = plan->nseg;
   out->max_row_nnz = plan->max_row_nnz;
   out->empty_rows = plan->empty_rows;
   out->workspace_bytes = plan->workspace_bytes;
-  out->launches_per_spmm = plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? (plan->n_hub > 0 ? 3 : 2) : 1;
+  out->launches_per_spmm = plan->strategy == HPSPMM_STRATEGY_ROUTED ? 3
+                           : plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? (plan->n_hub > 0 ? 3 : 2) : 1;
   out->hub_rows = plan->n_hub;
   return HPSPMM_OK;
 }
@@ -387,6 +586,9 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
   if (plan->d_hub_ids) (void)hipFree(plan->d_hub_ids);
   if (plan->d_hub_col) (void)hipFree(plan->d_hub_col);
   if (plan->d_bhot) (void)hipFree(plan->d_bhot);
+  for (void* q : {(void*)plan->d_vptr, (void*)plan->d_vcol, (void*)plan->d_vsrc, (void*)plan->d_vrow,
+                  (void*)plan->d_bhot_src, (void*)plan->d_partial, (void*)plan->d_action})
+    if (q) (void)hipFree(q);
   delete plan;
   return HPSPMM_OK;
 }
@@ -400,7 +602,13 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
     return fail(HPSPMM_ERR_INVALID_ARG, "d_col, d_val or d_B is NULL with nnz > 0");
   hipStream_t st = (hipStream_t)stream;
   int rc;
-  if (plan->strategy == HPSPMM_STRATEGY_SEGMENTS) {
+  if (plan->strategy == HPSPMM_STRATEGY_ROUTED) {
+    switch (plan->k) {
+      case 32: rc = launch_routed<32>(plan, d_val, d_B, d_C, st); break;
+      case 64: rc = launch_routed<64>(plan, d_val, d_B, d_C, st); break;
+      default: rc = launch_routed<128>(plan, d_val, d_B, d_C, st); break;
+    }
+  } else if (plan->strategy == HPSPMM_STRATEGY_SEGMENTS) {
     switch (plan->k) {
       case 32: rc = launch_segments<32>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;
       case 64: rc = launch_segments<64>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;

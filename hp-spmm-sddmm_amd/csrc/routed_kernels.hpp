@@ -1,0 +1,413 @@
+// gfx950 device code of the *routed* strategy for FP32 CSR SpMM.
+//
+// On power-law graphs a few thousand columns receive most of the nonzeros, yet
+// with eight XCDs each seeing an eighth of a mixed stream those rows of B do
+// not survive in any 4 MB L2 (measured: ~15 % L2 hits, the gather runs at the
+// fabric's ~7.4 TB/s while an L2-resident gather runs at ~22 TB/s).  The routed
+// strategy makes the hot rows L2-resident by construction:
+//
+//   * every column belongs to one of 8 slices: the most referenced columns by
+//     popularity rank, round robin, so that the slices carry equal load, the
+//     rest by a hash of the index.  Slice x of B is only ever read by
+//     workgroups running on XCD x (workgroup b runs on XCD b % 8), so each L2
+//     sees an eighth of the columns and keeps the hot ones (measured on the
+//     233k-vertex social graph, K=128: 6.6 ms -> 4.5 ms);
+//   * the most referenced rows of B are additionally copied, slice by slice,
+//     into a compact buffer at the start of every SpMM, which takes them off
+//     whatever memory channels their original addresses collide on;
+//   * degree binning: only rows with at least `min_row_nnz` nonzeros are
+//     routed - a short row would pay one partial-result row per class it
+//     touches for a handful of gathers.  A nonzero of a routed row belongs to
+//     the class of its column's slice, all nonzeros of a short row to class 8.
+//     The plan lays the nonzeros out class by class, each class in row order,
+//     as three arrays: column (~compact-buffer row if the column is cached),
+//     source index into the caller's value array, and row;
+//   * inside a class the work is cut into fixed-length segments exactly as in
+//     the segments strategy; a (row, class) run that lies inside one segment is
+//     stored to a per-class partial-result buffer, runs that cross a segment
+//     boundary go through the carry slots;
+//   * a final kernel adds, for every row, its class partials in class order
+//     and writes C (zeros for empty rows).  No atomics; results are
+//     bit-reproducible for a given plan.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "spmm_kernels.hpp"
+
+namespace hpspmm {
+
+constexpr int kHubClasses = 8;             // one per XCD
+constexpr int kClasses = kHubClasses + 1;  // + the cold class
+constexpr int kColdClass = kHubClasses;
+
+// What the final kernel does with a row.
+constexpr uint8_t kActionNone = 0;    // the main kernel stored the row to C itself
+constexpr uint8_t kActionZero = 1;    // no nonzeros: write zeros
+constexpr uint8_t kActionReduce = 2;  // add the class results
+
+struct RoutedLayout {
+  int64_t cls_begin[kClasses];   // first virtual index of the class (multiple of the workgroup quantum)
+  int64_t cls_end[kClasses];     // one past its last real entry
+  int64_t cls_blocks[kClasses];  // workgroups needed by the class
+  int64_t hub_grid;              // 8 * max(cls_blocks[0..7]): hub workgroups are interleaved by class
+  int64_t rows;
+  int shift;                     // log2(segment length)
+};
+
+// ---- plan-time kernels -----------------------------------------------------
+
+// Class of a nonzero in column c: mapped = colmap[c] is the compact-buffer row
+// of a cached column (slice = row / hub_rows_per_class) or -1, in which case
+// a multiplicative hash of c picks the slice; rows shorter than the routing
+// threshold send everything to class 8.
+__device__ __forceinline__ int class_of(int32_t c, int32_t mapped, int32_t hub_rows_per_class, bool routed_row) {
+  if (!routed_row) return kColdClass;
+  return mapped >= 0 ? mapped / hub_rows_per_class : (int)(((uint32_t)c * 0x9E3779B1u) >> 29);
+}
+
+// cnt[x * rows + r] = number of nonzeros of row r in class x.  One wavefront per row.
+__global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                              const int32_t* __restrict__ col,
+                                                              const int32_t* __restrict__ colmap,
+                                                              int32_t hub_rows_per_class, int32_t min_row_nnz,
+                                                              uint32_t* __restrict__ cnt) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int32_t lb = rowptr[row];
+  const int32_t hb = rowptr[row + 1];
+  const bool routed_row = hb - lb >= min_row_nnz;
+  uint32_t mine = 0;  // lane x < kClasses accumulates the count of class x
+  for (int32_t j0 = lb; j0 < hb; j0 += 64) {
+    const int32_t j = j0 + lane;
+    int cls = -1;
+    if (j < hb) {
+      const int32_t c = col[j];
+      cls = class_of(c, colmap[c], hub_rows_per_class, routed_row);
+    }
+#pragma unroll
+    for (int x = 0; x < kClasses; ++x) {
+      const uint64_t m = __ballot(cls == x);
+      if (lane == x) mine += (uint32_t)__popcll(m);
+    }
+  }
+  if (lane < kClasses) cnt[(int64_t)lane * rows + row] = mine;
+}
+
+// Three-pass exclusive scan of uint32 (n up to 2^32, total < 2^32).
+constexpr int kScanItems = 16;  // per thread
+constexpr int kScanTile = kBlock * kScanItems;
+
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s_wave, uint32_t& block_total) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  uint32_t incl = v;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t o = __shfl_up(incl, off);
+    if (lane >= off) incl += o;
+  }
+  if (lane == 63) s_wave[wave] = incl;
+  __syncthreads();
+  uint32_t wave_off = 0;
+  uint32_t total = 0;
+#pragma unroll
+  for (int w = 0; w < kWavesPerBlock; ++w) {
+    if (w < wave) wave_off += s_wave[w];
+    total += s_wave[w];
+  }
+  __syncthreads();
+  block_total = total;
+  return wave_off + incl - v;
+}
+
+__global__ __launch_bounds__(kBlock) void scan_tile_sums_kernel(int64_t n, const uint32_t* __restrict__ in,
+                                                                uint32_t* __restrict__ tile_sums) {
+  __shared__ uint32_t s_wave[kWavesPerBlock];
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+  uint32_t sum = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i)
+    if (base + i < n) sum += in[base + i];
+  uint32_t total;
+  (void)block_exclusive_scan(sum, s_wave, total);
+  if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+// Exclusive scan of the tile sums in place, by one workgroup.
+__global__ __launch_bounds__(kBlock) void scan_tile_offsets_kernel(int64_t ntiles, uint32_t* __restrict__ tile_sums) {
+  __shared__ uint32_t s_wave[kWavesPerBlock];
+  uint32_t carry = 0;
+  for (int64_t base = 0; base < ntiles; base += kBlock) {
+    const int64_t i = base + threadIdx.x;
+    const uint32_t v = i < ntiles ? tile_sums[i] : 0u;
+    uint32_t total;
+    const uint32_t ex = block_exclusive_scan(v, s_wave, total);
+    if (i < ntiles) tile_sums[i] = carry + ex;
+    carry += total;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void scan_apply_kernel(int64_t n, const uint32_t* __restrict__ in,
+                                                            const uint32_t* __restrict__ tile_offsets,
+                                                            uint32_t* __restrict__ out) {
+  __shared__ uint32_t s_wave[kWavesPerBlock];
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+  uint32_t v[kScanItems];
+  uint32_t sum = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    v[i] = base + i < n ? in[base + i] : 0u;
+    sum += v[i];
+  }
+  uint32_t total;
+  uint32_t run = tile_offsets[blockIdx.x] + block_exclusive_scan(sum, s_wave, total);
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    if (base + i < n) out[base + i] = run;
+    run += v[i];
+  }
+}
+
+// vptr[x * (rows + 1) + r] = virtual index of the first class-x nonzero of row r
+// (r = rows: one past the class), from the exclusive scan of the class-major
+// counts and the padded class origins.
+__global__ __launch_bounds__(kBlock) void routed_vptr_kernel(RoutedLayout lay, const uint32_t* __restrict__ scanned,
+                                                             int32_t* __restrict__ vptr) {
+  const int64_t per = lay.rows + 1;
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= per * kClasses) return;
+  const int x = (int)(i / per);
+  const int64_t r = i - (int64_t)x * per;
+  const int64_t first = scanned[(int64_t)x * lay.rows];
+  const int64_t local = r < lay.rows ? (int64_t)scanned[(int64_t)x * lay.rows + r] - first
+                                     : lay.cls_end[x] - lay.cls_begin[x];
+  vptr[i] = (int32_t)(lay.cls_begin[x] + local);
+}
+
+// Scatter the nonzeros into class-major order, keeping the stored order inside
+// every (row, class) run.  One wavefront per row; positions from ballots.
+__global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                             const int32_t* __restrict__ col,
+                                                             const int32_t* __restrict__ colmap,
+                                                             int32_t hub_rows_per_class, int32_t min_row_nnz,
+                                                             const int32_t* __restrict__ vptr,
+                                                             int32_t* __restrict__ vcol, int32_t* __restrict__ vsrc,
+                                                             int32_t* __restrict__ vrow,
+                                                             uint8_t* __restrict__ action, int shift) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int32_t lb = rowptr[row];
+  const int32_t hb = rowptr[row + 1];
+  const bool routed_row = hb - lb >= min_row_nnz;
+  int32_t cursor = lane < kClasses ? vptr[(int64_t)lane * (rows + 1) + row] : 0;  // lane x: next slot of class x
+  const int32_t cls_last = lane < kClasses ? vptr[(int64_t)lane * (rows + 1) + row + 1] : 0;
+  const uint64_t below = (1ull << lane) - 1ull;
+  // A row without hub-class entries is "direct": its cold run is stored straight to
+  // C (flagged by the sign bit of vrow) unless it crosses a segment boundary.
+  const bool direct = __ballot(lane < kHubClasses && cls_last > cursor) == 0;
+  if (lane == kColdClass) {
+    uint8_t a = kActionReduce;
+    if (direct) {
+      if (cls_last == cursor) a = kActionZero;
+      else if (((int64_t)cursor >> shift) == ((int64_t)(cls_last - 1) >> shift)) a = kActionNone;
+    }
+    action[row] = a;
+  }
+  const int32_t row_tag = direct ? (int32_t)((uint32_t)row | 0x80000000u) : (int32_t)row;
+  for (int32_t j0 = lb; j0 < hb; j0 += 64) {
+    const int32_t j = j0 + lane;
+    const bool valid = j < hb;
+    const int32_t c = valid ? col[j] : 0;
+    const int32_t mapped = valid ? colmap[c] : -1;
+    const int cls = valid ? class_of(c, mapped, hub_rows_per_class, routed_row) : -1;
+#pragma unroll
+    for (int x = 0; x < kClasses; ++x) {
+      const uint64_t m = __ballot(cls == x);
+      const int32_t start = __shfl(cursor, x);
+      if (cls == x) {
+        const int32_t pos = start + (int32_t)__popcll(m & below);
+        vcol[pos] = mapped >= 0 ? ~mapped : c;  // ~compact-buffer row if the column is cached
+        vsrc[pos] = j;
+        vrow[pos] = row_tag;
+      }
+      if (lane == x) cursor += (int32_t)__popcll(m);
+    }
+  }
+}
+
+// Bhot[s, :] = B[src[s], :] for every compact-buffer row with a source column (src[s] >= 0).
+template <int K>
+__global__ __launch_bounds__(kBlock) void routed_gather_hub_kernel(int64_t n, const int32_t* __restrict__ src,
+                                                                   const float* __restrict__ B,
+                                                                   float* __restrict__ Bhot) {
+  constexpr int G = K / 4;
+  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t s = t / G;
+  const int l = (int)(t % G);
+  if (s >= n) return;
+  const int32_t c = src[s];
+  if (c < 0) return;
+  *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) = load_b<K>(B, c, l);
+}
+
+// ---- SpMM kernels ----------------------------------------------------------
+
+// Workgroups [0, hub_grid): workgroup b serves column class b % 8 (and runs on
+// XCD b % 8), its b / 8-th workgroup.  Workgroups [hub_grid, ...): class 8, the
+// short rows.
+// Each sub-wave owns one segment of its class; see the carry rule of the
+// segments kernel - here "stored to C" becomes "stored to the class's
+// partial-result buffer".
+template <int K>
+__global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, const int32_t* __restrict__ vptr,
+                                                             const int32_t* __restrict__ vcol,
+                                                             const int32_t* __restrict__ vsrc,
+                                                             const int32_t* __restrict__ vrow,
+                                                             const float* __restrict__ val,
+                                                             const float* __restrict__ B,
+                                                             const float* __restrict__ Bhot,
+                                                             float* __restrict__ partial,
+                                                             float* __restrict__ carry, float* __restrict__ C) {
+  constexpr int G = K / 4;
+  constexpr int P = 64 / G;
+  constexpr int TL = kTile / G;
+  __shared__ __attribute__((aligned(16))) int32_t s_col[kWavesPerBlock * P * kTileStride];
+  __shared__ __attribute__((aligned(16))) float s_val[kWavesPerBlock * P * kTileStride];
+  __shared__ __attribute__((aligned(16))) int32_t s_row[kWavesPerBlock * P * kTileStride];
+
+  int x;
+  int64_t i;
+  if ((int64_t)blockIdx.x < lay.hub_grid) {
+    x = (int)(blockIdx.x % kHubClasses);
+    i = blockIdx.x / kHubClasses;
+  } else {
+    x = kColdClass;
+    i = (int64_t)blockIdx.x - lay.hub_grid;
+  }
+  if (i >= lay.cls_blocks[x]) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int l = lane % G;
+  const int shift = lay.shift;
+  const int64_t g = (lay.cls_begin[x] >> shift) + (i * kWavesPerBlock + (tid >> 6)) * P + lane / G;
+  const int64_t s = g << shift;
+  const int64_t cls_end = lay.cls_end[x];
+  if (s >= cls_end) return;
+  const int64_t e = (s + ((int64_t)1 << shift)) < cls_end ? (s + ((int64_t)1 << shift)) : cls_end;
+  const int sbase = ((tid >> 6) * P + lane / G) * kTileStride;
+  const int32_t* vp = vptr + (int64_t)x * (lay.rows + 1);
+  float* pout = partial + (uint64_t)x * (uint64_t)lay.rows * K;
+
+  // the sign bit of a row entry marks a row that is stored straight to C
+  int32_t cur = vrow[s];
+  bool head_pending = (int64_t)vp[cur & 0x7FFFFFFF] < s;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+
+  auto flush_to = [&](bool is_tail) {
+    const uint32_t row = (uint32_t)cur & 0x7FFFFFFFu;
+    float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
+                              : (is_tail ? carry + (uint64_t)(2 * g + 1) * K
+                                         : (cur < 0 ? C + (uint64_t)row * K : pout + (uint64_t)row * K));
+    head_pending = false;
+    *reinterpret_cast<float4*>(dst + 4 * l) = acc;
+  };
+  auto flush = [&]() { flush_to(false); };
+  auto loadb = [&](int32_t c) { return load_b_hub<K, true>(B, Bhot, c, l); };
+
+  // Two-deep prefetch: the source indices of tile t+2 and, through the indices
+  // fetched one iteration earlier, the values of tile t+1 (the plan's arrays
+  // are allocated by the library, hence always aligned for the vector loads).
+  TileRegs<TL> m;
+  int32_t src[TL];
+  const int64_t q0 = s + l * TL;
+  load_run<TL>(src, vsrc, q0, e, true);
+  load_run<TL>(m.c, vcol, q0, e, true);
+  load_run<TL>(m.r, vrow, q0, e, true);
+#pragma unroll
+  for (int j = 0; j < TL; ++j) m.v[j] = q0 + j < e ? val[src[j]] : 0.f;
+  if (s + kTile < e) load_run<TL>(src, vsrc, q0 + kTile, e, true);
+
+  for (int64_t t = s; t < e; t += kTile) {
+    stage_tile<TL>(m, sbase + l * TL, s_col, s_val, s_row);
+    wave_lds_fence();
+    if (t + kTile < e) {
+      const int64_t q = t + kTile + l * TL;
+      load_run<TL>(m.c, vcol, q, e, true);
+      load_run<TL>(m.r, vrow, q, e, true);
+#pragma unroll
+      for (int j = 0; j < TL; ++j) m.v[j] = q + j < e ? val[src[j]] : 0.f;
+      if (t + 2 * kTile < e) load_run<TL>(src, vsrc, q + kTile, e, true);
+    }
+    const int cnt = (e - t) < kTile ? (int)(e - t) : kTile;
+    consume_tile(cnt, sbase, s_col, s_val, s_row, cur, acc, loadb, flush);
+    wave_lds_fence();
+  }
+  flush_to((int64_t)vp[(cur & 0x7FFFFFFF) + 1] > e);
+}
+
+// Final pass.  A wavefront takes 64 consecutive rows, reads their action bytes
+// and lets its sub-waves serve the rows that need work: zeros for empty rows;
+// for kActionReduce rows the sum over the classes, in class order, of the
+// class result - the partial-buffer row if the (row, class) run lies in one
+// segment, else tail[ga] + head[ga+1] + ... + head[gb] from the carry slots.
+template <int K>
+__global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout lay,
+                                                                   const int32_t* __restrict__ vptr,
+                                                                   const uint8_t* __restrict__ action,
+                                                                   const float* __restrict__ partial,
+                                                                   const float* __restrict__ carry,
+                                                                   float* __restrict__ C) {
+  constexpr int G = K / 4;
+  constexpr int P = 64 / G;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int l = lane % G;
+  const int sub = lane / G;
+  const int64_t r0 = ((int64_t)blockIdx.x * kWavesPerBlock + (tid >> 6)) * 64;
+  if (r0 >= lay.rows) return;
+  const uint8_t a = r0 + lane < lay.rows ? action[r0 + lane] : kActionNone;
+  const uint64_t m_zero = __ballot(a == kActionZero);
+  const uint64_t m_reduce = __ballot(a == kActionReduce);
+  if ((m_zero | m_reduce) == 0) return;
+  const int shift = lay.shift;
+
+  for (int i = sub; i < 64; i += P) {
+    const bool zero = (m_zero >> i) & 1ull;
+    const bool reduce = (m_reduce >> i) & 1ull;
+    if (!zero && !reduce) continue;
+    const int64_t row = r0 + i;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (reduce) {
+      auto add = [&](const float* src) {
+        const float4 t = *reinterpret_cast<const float4*>(src + 4 * l);
+        acc.x += t.x;
+        acc.y += t.y;
+        acc.z += t.z;
+        acc.w += t.w;
+      };
+#pragma unroll 1
+      for (int x = 0; x < kClasses; ++x) {
+        const int32_t* vp = vptr + (int64_t)x * (lay.rows + 1);
+        const int64_t lb = vp[row];
+        const int64_t hb = vp[row + 1];
+        if (lb == hb) continue;
+        const int64_t ga = lb >> shift;
+        const int64_t gb = (hb - 1) >> shift;
+        if (ga == gb) {
+          add(partial + ((uint64_t)x * (uint64_t)lay.rows + (uint64_t)row) * K);
+        } else {
+          add(carry + (uint64_t)(2 * ga + 1) * K);
+          for (int64_t g = ga + 1; g <= gb; ++g) add(carry + (uint64_t)(2 * g) * K);
+        }
+      }
+    }
+    *reinterpret_cast<float4*>(C + (uint64_t)row * K + 4 * l) = acc;
+  }
+}
+
+}  // namespace hpspmm

@@ -235,6 +235,110 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_generic_kernel(int64_t rows,
 }
 
 // ---------------------------------------------------------------------------
+// Tile engine of the segment-type kernels.
+//
+// A sub-wave consumes its segment in tiles of kTile = 32 entries.  Lane l holds
+// TL = 32 / G consecutive entries of the *next* tile in registers (one 16/8/4
+// byte load per array), so that the metadata fetch of tile t+1 overlaps the B
+// gathers of tile t (the role cp.async double buffering plays in the
+// reference, spmm/mm/spmm_kernel.cu:650-702).  At the top of an iteration the
+// registers are written to the sub-wave's LDS region and read back as
+// broadcasts, 8 entries (8 B-row fragments in flight per lane) at a time.
+// LDS regions are 36 entries apart: 16-byte aligned for the vector stores and
+// on distinct banks for the broadcast reads of the P sub-waves.
+// ---------------------------------------------------------------------------
+constexpr int kTile = 32;
+constexpr int kTileStride = 36;
+
+template <int TL>
+struct TileRegs {
+  int32_t c[TL];
+  float v[TL];
+  int32_t r[TL];
+};
+
+// dst[0..TL) = src[q .. q+TL): one vector load when allowed and the tile is full, else guarded scalars.
+template <int TL, typename T>
+__device__ __forceinline__ void load_run(T (&dst)[TL], const T* __restrict__ src, int64_t q, int64_t e, bool vec_ok) {
+  if (TL > 1 && vec_ok && q + TL <= e) {
+    if constexpr (TL == 4) {
+      const int4 w = *reinterpret_cast<const int4*>(src + q);
+      dst[0] = __builtin_bit_cast(T, w.x);
+      dst[1] = __builtin_bit_cast(T, w.y);
+      dst[2] = __builtin_bit_cast(T, w.z);
+      dst[3] = __builtin_bit_cast(T, w.w);
+    } else if constexpr (TL == 2) {
+      const int2 w = *reinterpret_cast<const int2*>(src + q);
+      dst[0] = __builtin_bit_cast(T, w.x);
+      dst[1] = __builtin_bit_cast(T, w.y);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < TL; ++i) dst[i] = q + i < e ? src[q + i] : T(0);
+  }
+}
+
+template <int TL>
+__device__ __forceinline__ void stage_tile(const TileRegs<TL>& m, int slot, int32_t* s_col, float* s_val,
+                                           int32_t* s_row) {
+  if constexpr (TL == 4) {
+    *reinterpret_cast<int4*>(s_col + slot) = make_int4(m.c[0], m.c[1], m.c[2], m.c[3]);
+    *reinterpret_cast<float4*>(s_val + slot) = make_float4(m.v[0], m.v[1], m.v[2], m.v[3]);
+    *reinterpret_cast<int4*>(s_row + slot) = make_int4(m.r[0], m.r[1], m.r[2], m.r[3]);
+  } else if constexpr (TL == 2) {
+    *reinterpret_cast<int2*>(s_col + slot) = make_int2(m.c[0], m.c[1]);
+    *reinterpret_cast<float2*>(s_val + slot) = make_float2(m.v[0], m.v[1]);
+    *reinterpret_cast<int2*>(s_row + slot) = make_int2(m.r[0], m.r[1]);
+  } else {
+    s_col[slot] = m.c[0];
+    s_val[slot] = m.v[0];
+    s_row[slot] = m.r[0];
+  }
+}
+
+// Accumulate the first `cnt` staged entries of a sub-wave's tile; a change of
+// row calls flush() (which stores the finished row and is told nothing else).
+template <class LoadB, class Flush>
+__device__ __forceinline__ void consume_tile(int cnt, int sbase, const int32_t* s_col, const float* s_val,
+                                             const int32_t* s_row, int32_t& cur, float4& acc, LoadB loadb,
+                                             Flush flush) {
+  constexpr int U = kBatch;
+  int u = 0;
+  for (; u + U <= cnt; u += U) {
+    int32_t c[U], r[U];
+    float v[U];
+    float4 b[U];
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      c[i] = s_col[sbase + u + i];
+      v[i] = s_val[sbase + u + i];
+      r[i] = s_row[sbase + u + i];
+    }
+#pragma unroll
+    for (int i = 0; i < U; ++i) b[i] = loadb(c[i]);
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      if (r[i] != cur) {
+        flush();
+        acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        cur = r[i];
+      }
+      fma4(acc, v[i], b[i]);
+    }
+  }
+  for (; u < cnt; ++u) {
+    const int32_t r = s_row[sbase + u];
+    const float4 b = loadb(s_col[sbase + u]);
+    if (r != cur) {
+      flush();
+      acc = make_float4(0.f, 0.f, 0.f, 0.f);
+      cur = r;
+    }
+    fma4(acc, s_val[sbase + u], b);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // segments kernel.
 //
 // Segment g covers nonzeros [g << shift, min((g+1) << shift, nnz)).  nnz_row[j]
@@ -253,13 +357,13 @@ __global__ __launch_bounds__(kBlock) void spmm_segments_kernel(
     const int32_t* __restrict__ rowptr, const int32_t* __restrict__ col, const float* __restrict__ val,
     const int32_t* __restrict__ nnz_row, const float* __restrict__ B, const float* __restrict__ Bhot,
     float* __restrict__ C, float* __restrict__ carry, int64_t nnz, int shift, int64_t nseg, int64_t nblocks,
-    bool remap) {
+    bool remap, bool vec_ok) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
-  constexpr int U = G < kBatch ? G : kBatch;
-  __shared__ int32_t s_col[kBlock];
-  __shared__ float s_val[kBlock];
-  __shared__ int32_t s_row[kBlock];
+  constexpr int TL = kTile / G;
+  __shared__ __attribute__((aligned(16))) int32_t s_col[kWavesPerBlock * P * kTileStride];
+  __shared__ __attribute__((aligned(16))) float s_val[kWavesPerBlock * P * kTileStride];
+  __shared__ __attribute__((aligned(16))) int32_t s_row[kWavesPerBlock * P * kTileStride];
 
   const int64_t blk = xcd_remap(blockIdx.x, nblocks, remap);
   if (blk < 0) return;
@@ -271,14 +375,14 @@ __global__ __launch_bounds__(kBlock) void spmm_segments_kernel(
 
   const int64_t s = g << shift;
   const int64_t e = (s + ((int64_t)1 << shift)) < nnz ? (s + ((int64_t)1 << shift)) : nnz;
-  const int base = tid - l;
+  const int sbase = ((tid >> 6) * P + lane / G) * kTileStride;
 
   int32_t cur = nnz_row[s];
   bool head_pending = false;
   if constexpr (!kAtomic) head_pending = (int64_t)rowptr[cur] < s;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 
-  auto flush = [&](bool is_tail) {
+  auto flush_to = [&](bool is_tail) {
     if constexpr (kAtomic) {
       float* dst = C + (uint64_t)(uint32_t)cur * K + 4 * l;
       unsafeAtomicAdd(dst + 0, acc.x);
@@ -293,54 +397,28 @@ __global__ __launch_bounds__(kBlock) void spmm_segments_kernel(
       *reinterpret_cast<float4*>(dst + 4 * l) = acc;
     }
   };
+  auto flush = [&]() { flush_to(false); };
+  auto loadb = [&](int32_t c) { return load_b_hub<K, kHub>(B, Bhot, c, l); };
+  auto fetch = [&](TileRegs<TL>& m, int64_t t) {
+    const int64_t q = t + l * TL;
+    load_run<TL>(m.c, col, q, e, vec_ok);
+    load_run<TL>(m.v, val, q, e, vec_ok);
+    load_run<TL>(m.r, nnz_row, q, e, vec_ok);
+  };
 
-  for (int64_t t = s; t < e; t += G) {
-    const int64_t p = t + l;
-    if (p < e) {
-      s_col[tid] = col[p];
-      s_val[tid] = val[p];
-      s_row[tid] = nnz_row[p];
-    }
+  TileRegs<TL> m;
+  fetch(m, s);
+  for (int64_t t = s; t < e; t += kTile) {
+    stage_tile<TL>(m, sbase + l * TL, s_col, s_val, s_row);
     wave_lds_fence();
-    const int cnt = (e - t) < G ? (int)(e - t) : G;
-    int u = 0;
-    for (; u + U <= cnt; u += U) {
-      int32_t c[U], r[U];
-      float v[U];
-      float4 b[U];
-#pragma unroll
-      for (int i = 0; i < U; ++i) {
-        c[i] = s_col[base + u + i];
-        v[i] = s_val[base + u + i];
-        r[i] = s_row[base + u + i];
-      }
-#pragma unroll
-      for (int i = 0; i < U; ++i) b[i] = load_b_hub<K, kHub>(B, Bhot, c[i], l);
-#pragma unroll
-      for (int i = 0; i < U; ++i) {
-        if (r[i] != cur) {
-          flush(false);
-          acc = make_float4(0.f, 0.f, 0.f, 0.f);
-          cur = r[i];
-        }
-        fma4(acc, v[i], b[i]);
-      }
-    }
-    for (; u < cnt; ++u) {
-      const int32_t r = s_row[base + u];
-      const float4 b = load_b_hub<K, kHub>(B, Bhot, s_col[base + u], l);
-      if (r != cur) {
-        flush(false);
-        acc = make_float4(0.f, 0.f, 0.f, 0.f);
-        cur = r;
-      }
-      fma4(acc, s_val[base + u], b);
-    }
+    if (t + kTile < e) fetch(m, t + kTile);
+    const int cnt = (e - t) < kTile ? (int)(e - t) : kTile;
+    consume_tile(cnt, sbase, s_col, s_val, s_row, cur, acc, loadb, flush);
     wave_lds_fence();
   }
   bool continues = false;
   if constexpr (!kAtomic) continues = (int64_t)rowptr[cur + 1] > e;
-  flush(continues);
+  flush_to(continues);
 }
 
 // Fix-up after the segments kernel.  A wavefront scans 64 consecutive rows (one

@@ -57,6 +57,9 @@ typedef enum hpspmm_status {
 #define HPSPMM_PLAN_HUB_CACHE 16u     /* segments strategy: always keep the most referenced rows of B in a compact
                                          copy (default: only when they serve >= 25 % of the nonzeros) */
 #define HPSPMM_PLAN_NO_HUB_CACHE 32u  /* never build the hub cache */
+#define HPSPMM_PLAN_FORCE_ROUTED 64u  /* always use the routed strategy (hub columns pinned to one XCD each);
+                                         bits 16..23 then give log2 of the total number of hub rows (0 = auto) */
+#define HPSPMM_PLAN_NO_ROUTED 128u    /* never use the routed strategy */
 /* bits 16..23: log2 of the number of cached rows (0 = default, 2^16) */
 #define HPSPMM_PLAN_HUB_LOG2(log2_rows) (((uint32_t)(log2_rows) & 0xFFu) << 16)
 /* bits 8..15: log2 of the segment length to force (0 = choose automatically) */
@@ -66,6 +69,7 @@ typedef enum hpspmm_status {
 #define HPSPMM_STRATEGY_ROWS 1
 #define HPSPMM_STRATEGY_SEGMENTS 2
 #define HPSPMM_STRATEGY_GENERIC_K 3
+#define HPSPMM_STRATEGY_ROUTED 4
 
 typedef struct hpspmm_plan hpspmm_plan;
 

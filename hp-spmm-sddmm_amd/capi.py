@@ -34,6 +34,10 @@ def plan_hub_log2(log2_rows):
     return (int(log2_rows) & 0xFF) << 16
 
 
+def plan_routed_row_log2(log2_nnz):
+    return (int(log2_nnz) & 0x1F) << 24
+
+
 def plan_segment_shift(log2_len):
     return (int(log2_len) & 0xFF) << 8
 

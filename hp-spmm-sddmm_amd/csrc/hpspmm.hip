@@ -108,25 +108,50 @@ inline int64_t row_blocks(int64_t rows, int64_t k) {
 // Rows longer than this are handled by a whole wavefront in the rows strategy.
 constexpr int32_t kLongRowThreshold = 32;
 
-template <int K>
-int launch_rows(int64_t rows, const int32_t* rp, const int32_t* ci, const float* v, const float* B, float* C,
-                int32_t long_threshold, const int32_t* long_rows, int64_t n_long, hipStream_t st) {
-  const int64_t short_blocks = row_blocks(rows, K);
-  const int64_t blocks = short_blocks + ceil_div(n_long, hpspmm::kWavesPerBlock);
+// Column-tile width of the rows kernel: the widest tile of B (cols x KT floats)
+// that still fits one XCD's L2 next to the streamed arrays, so that a B too big
+// for one L2 is split over the XCDs by columns of B instead of thrashing all
+// eight.  Measured on the 20k-vertex citation graph at K=128 (B = 10 MB):
+// 14.3 us with one 128-wide tile, 11.9 us with two 64-wide, 11.2 us with four
+// 32-wide tiles; at K=64 (B = 5 MB) tiling does not pay (6.8 vs 7.2 us).
+constexpr int64_t kRowsUntiledBytes = 6 << 20;  // B up to this size is left in one tile
+constexpr int64_t kRowsTileBytes = 3 << 20;     // else: the widest tile of B not larger than this
+
+template <int K, int KT>
+int launch_rows_tiled(int64_t rows, const int32_t* rp, const int32_t* ci, const float* v, const float* B, float* C,
+                      int32_t long_threshold, const int32_t* long_rows, int64_t n_long, hipStream_t st) {
+  const int64_t short_blocks = row_blocks(rows, KT);
+  const int64_t blocks = (short_blocks + ceil_div(n_long, hpspmm::kWavesPerBlock)) * (K / KT);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
-  hipLaunchKernelGGL(hpspmm::spmm_rows_kernel<K>, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rows, rp, ci,
-                     v, B, C, short_blocks, long_threshold, long_rows, n_long);
+  hipLaunchKernelGGL((hpspmm::spmm_rows_kernel<K, KT>), dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rows, rp,
+                     ci, v, B, C, short_blocks, long_threshold, long_rows, n_long);
   return HPSPMM_OK;
 }
 
-int launch_rows_any(int64_t rows, int64_t k, const int32_t* rp, const int32_t* ci, const float* v,
+template <int K>
+int launch_rows(int64_t rows, int64_t cols, const int32_t* rp, const int32_t* ci, const float* v, const float* B,
+                float* C, int32_t long_threshold, const int32_t* long_rows, int64_t n_long, hipStream_t st) {
+  if constexpr (K >= 64) {
+    if (cols * K * 4 > kRowsUntiledBytes) {
+      if constexpr (K == 128) {
+        if (cols * 64 * 4 <= kRowsTileBytes)
+          return launch_rows_tiled<K, 64>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+      }
+      if (cols * 32 * 4 <= kRowsTileBytes)
+        return launch_rows_tiled<K, 32>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+    }
+  }
+  return launch_rows_tiled<K, K>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+}
+
+int launch_rows_any(int64_t rows, int64_t cols, int64_t k, const int32_t* rp, const int32_t* ci, const float* v,
                     const float* B, float* C, int32_t long_threshold, const int32_t* long_rows, int64_t n_long,
                     hipStream_t st) {
   if (rows == 0) return HPSPMM_OK;
   switch (k) {
-    case 32: return launch_rows<32>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
-    case 64: return launch_rows<64>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
-    case 128: return launch_rows<128>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+    case 32: return launch_rows<32>(rows, cols, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+    case 64: return launch_rows<64>(rows, cols, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+    case 128: return launch_rows<128>(rows, cols, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
     default: {
       const int64_t blocks = ceil_div(rows, hpspmm::kWavesPerBlock);
       hipLaunchKernelGGL(hpspmm::spmm_rows_generic_kernel, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st,
@@ -247,12 +272,12 @@ constexpr int64_t kRoutedMinNnz = (int64_t)1 << 22;
 constexpr int64_t kRoutedMinBBytes = (int64_t)48 << 20;  // B must overflow the 8 x 4 MB of L2
 constexpr double kRoutedMinShare = 0.35;     // of the nonzeros in the 64k most referenced columns
 constexpr double kRoutedMinRowNnz = 32.0;    // mean nonzeros per non-empty row
-constexpr int32_t kRoutedRowThreshold = 64;  // rows shorter than this are not split over the classes
+constexpr int32_t kRoutedRowThreshold = 128;  // rows shorter than this are not split over the classes
 
 // Builds the routed layout.  Returns HPSPMM_OK with p->strategy left at
 // SEGMENTS when the graph does not qualify (and `forced` is false).
 int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, int log2_hubs,
-                 hipStream_t st) {
+                 int log2_row_threshold, hipStream_t st) {
   const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
   if (!forced && (nnz < kRoutedMinNnz || p->cols * k * 4 < kRoutedMinBBytes)) return HPSPMM_OK;
   // cached rows per class
@@ -293,7 +318,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   HPSPMM_HIP(hipMalloc(&d_scan, (size_t)ncnt * sizeof(uint32_t)));
   HPSPMM_HIP(hipMemcpyAsync(d_colmap, colmap.data(), colmap.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
   const unsigned row_grid = (unsigned)ceil_div(rows, hpspmm::kWavesPerBlock);
-  const int32_t min_row_nnz = forced && log2_hubs ? 2 : kRoutedRowThreshold;  // forced small hub sets: tests
+  const int32_t min_row_nnz = forced && log2_row_threshold ? (1 << log2_row_threshold) : kRoutedRowThreshold;
   hipLaunchKernelGGL(hpspmm::routed_count_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col,
                      d_colmap, (int32_t)h, min_row_nnz, d_cnt);
   if (int rc = exclusive_scan_u32(d_cnt, d_scan, ncnt, st)) return rc;
@@ -522,7 +547,8 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && !(flags & HPSPMM_PLAN_NO_ROUTED) && nnz > 0 &&
       !(flags & HPSPMM_PLAN_FORCE_SEGMENTS && !(flags & HPSPMM_PLAN_FORCE_ROUTED))) {
     if (int rc = build_routed(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_ROUTED) != 0,
-                              (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 16) & 0xFFu) : 0, st)) {
+                              (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 16) & 0xFFu) : 0,
+                              (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 24) & 0x1Fu) : 0, st)) {
       hpspmm_plan_destroy(p);
       return rc;
     }
@@ -615,7 +641,7 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
       default: rc = launch_segments<128>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;
     }
   } else {
-    rc = launch_rows_any(plan->rows, plan->k, d_rowptr, d_col, d_val, d_B, d_C, plan->long_threshold,
+    rc = launch_rows_any(plan->rows, plan->cols, plan->k, d_rowptr, d_col, d_val, d_B, d_C, plan->long_threshold,
                          plan->d_long_rows, plan->n_long, st);
   }
   if (rc) return rc;
@@ -631,7 +657,7 @@ int hpspmm_csr_spmm_noplan(int64_t rows, int64_t cols, int64_t nnz, const int32_
   if (!d_rowptr || !d_C) return fail(HPSPMM_ERR_INVALID_ARG, "d_rowptr or d_C is NULL");
   if (nnz > 0 && (!d_col || !d_val || !d_B))
     return fail(HPSPMM_ERR_INVALID_ARG, "d_col, d_val or d_B is NULL with nnz > 0");
-  if (int rc = launch_rows_any(rows, k, d_rowptr, d_col, d_val, d_B, d_C, INT32_MAX, nullptr, 0,
+  if (int rc = launch_rows_any(rows, cols, k, d_rowptr, d_col, d_val, d_B, d_C, INT32_MAX, nullptr, 0,
                                (hipStream_t)stream))
     return rc;
   HPSPMM_HIP(hipGetLastError());

@@ -58,6 +58,12 @@ __device__ __forceinline__ float4 load_b(const float* __restrict__ B, int32_t c,
   return *reinterpret_cast<const float4*>(B + (uint64_t)(uint32_t)c * (uint64_t)K + (uint32_t)(4 * l));
 }
 
+// Fragment l of a KT-wide column tile starting at column k0 of row c (leading dimension K).
+template <int K>
+__device__ __forceinline__ float4 load_b_tile(const float* __restrict__ B, int32_t c, int k0, int l) {
+  return *reinterpret_cast<const float4*>(B + (uint64_t)(uint32_t)c * (uint64_t)K + (uint32_t)(k0 + 4 * l));
+}
+
 // Hub cache: the plan may keep the most referenced rows of B in a compact
 // buffer (refreshed at the start of every SpMM) and rewrite their column
 // indices as ~slot (negative).  A negative index reads the compact buffer.
@@ -92,11 +98,12 @@ __device__ __forceinline__ int64_t xcd_remap(int64_t b, int64_t nblocks, bool re
 
 // acc += sum over nonzeros [lb, hb) of val[j] * B[col[j], 4l .. 4l+4), executed by
 // one sub-wave.  `base` is the LDS slot of the sub-wave's lane 0.
-template <int K>
+template <int K, int KT>
 __device__ __forceinline__ void accumulate_range(float4& acc, int32_t lb, int32_t hb, int l, int tid, int base,
                                                  int32_t* s_col, float* s_val, const int32_t* __restrict__ col,
-                                                 const float* __restrict__ val, const float* __restrict__ B) {
-  constexpr int G = K / 4;
+                                                 const float* __restrict__ val, const float* __restrict__ B,
+                                                 int k0) {
+  constexpr int G = KT / 4;
   constexpr int U = G < kBatch ? G : kBatch;
   for (int32_t jj = lb; jj < hb; jj += G) {
     const int32_t p = jj + l;
@@ -117,7 +124,7 @@ __device__ __forceinline__ void accumulate_range(float4& acc, int32_t lb, int32_
         v[i] = s_val[base + u + i];
       }
 #pragma unroll
-      for (int i = 0; i < U; ++i) b[i] = load_b<K>(B, c[i], l);
+      for (int i = 0; i < U; ++i) b[i] = load_b_tile<K>(B, c[i], k0, l);
 #pragma unroll
       for (int i = 0; i < U; ++i) fma4(acc, v[i], b[i]);
     }
@@ -139,7 +146,7 @@ __device__ __forceinline__ void accumulate_range(float4& acc, int32_t lb, int32_
           ok[i] = u + i < cnt;
           const int slot = base + (ok[i] ? u + i : cnt - 1);
           v[i] = s_val[slot];
-          b[i] = load_b<K>(B, s_col[slot], l);
+          b[i] = load_b_tile<K>(B, s_col[slot], k0, l);
         }
 #pragma unroll
         for (int i = 0; i < R; ++i) {
@@ -153,7 +160,7 @@ __device__ __forceinline__ void accumulate_range(float4& acc, int32_t lb, int32_
       }
     } else {
       for (; u < cnt; ++u) {
-        const float4 b = load_b<K>(B, s_col[base + u], l);
+        const float4 b = load_b_tile<K>(B, s_col[base + u], k0, l);
         fma4(acc, s_val[base + u], b);
       }
     }
@@ -161,11 +168,14 @@ __device__ __forceinline__ void accumulate_range(float4& acc, int32_t lb, int32_
   }
 }
 
-// Workgroups [0, short_blocks): one sub-wave per row, rows longer than
-// long_threshold skipped.  Workgroups [short_blocks, ...): one wavefront per
-// entry of long_rows[]; the row's nonzeros are dealt in contiguous runs to the
-// P sub-waves and the partial sums are combined with wavefront shuffles.
-template <int K>
+// Workgroups come in groups of T = K / KT, one per KT-wide column tile of B
+// and C (workgroup b serves tile b % T; T divides 8, so an XCD always sees the
+// same tile and its L2 only has to hold cols * KT floats of B).  Within a tile:
+// workgroup groups [0, short_blocks) run one sub-wave per row and skip rows
+// longer than long_threshold; the remaining groups run one wavefront per entry
+// of long_rows[], the row's nonzeros dealt in contiguous runs to the sub-waves
+// and the partial sums combined with wavefront shuffles.
+template <int K, int KT>
 __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                            const int32_t* __restrict__ col,
                                                            const float* __restrict__ val,
@@ -173,7 +183,8 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(int64_t rows, const i
                                                            int64_t short_blocks, int32_t long_threshold,
                                                            const int32_t* __restrict__ long_rows,
                                                            int64_t n_long) {
-  constexpr int G = K / 4;
+  constexpr int T = K / KT;
+  constexpr int G = KT / 4;
   constexpr int P = 64 / G;
   __shared__ int32_t s_col[kBlock];
   __shared__ float s_val[kBlock];
@@ -182,18 +193,20 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(int64_t rows, const i
   const int lane = tid & 63;
   const int l = lane % G;
   const int base = tid - l;
+  const int k0 = (int)(blockIdx.x % T) * KT;
+  const int64_t blk = blockIdx.x / T;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 
-  if ((int64_t)blockIdx.x < short_blocks) {
-    const int64_t row = ((int64_t)blockIdx.x * kWavesPerBlock + (tid >> 6)) * P + lane / G;
+  if (blk < short_blocks) {
+    const int64_t row = (blk * kWavesPerBlock + (tid >> 6)) * P + lane / G;
     if (row >= rows) return;
     const int32_t lb = rowptr[row];
     const int32_t hb = rowptr[row + 1];
     if (hb - lb > long_threshold) return;
-    accumulate_range<K>(acc, lb, hb, l, tid, base, s_col, s_val, col, val, B);
-    *reinterpret_cast<float4*>(C + (uint64_t)row * K + 4 * l) = acc;
+    accumulate_range<K, KT>(acc, lb, hb, l, tid, base, s_col, s_val, col, val, B, k0);
+    *reinterpret_cast<float4*>(C + (uint64_t)row * K + k0 + 4 * l) = acc;
   } else {
-    const int64_t w = ((int64_t)blockIdx.x - short_blocks) * kWavesPerBlock + (tid >> 6);
+    const int64_t w = (blk - short_blocks) * kWavesPerBlock + (tid >> 6);
     if (w >= n_long) return;
     const int32_t row = long_rows[w];
     const int32_t lb = rowptr[row];
@@ -202,7 +215,7 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(int64_t rows, const i
     const int32_t per = ((hb - lb + P * G - 1) / (P * G)) * G;
     const int32_t my_lb = lb + (lane / G) * per;
     const int32_t my_hb = (my_lb + per) < hb ? (my_lb + per) : hb;
-    accumulate_range<K>(acc, my_lb, my_hb, l, tid, base, s_col, s_val, col, val, B);
+    accumulate_range<K, KT>(acc, my_lb, my_hb, l, tid, base, s_col, s_val, col, val, B, k0);
 #pragma unroll
     for (int off = G; off < 64; off <<= 1) {
       acc.x += __shfl_xor(acc.x, off);
@@ -210,7 +223,7 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(int64_t rows, const i
       acc.z += __shfl_xor(acc.z, off);
       acc.w += __shfl_xor(acc.w, off);
     }
-    if (lane < G) *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)row * K + 4 * l) = acc;
+    if (lane < G) *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)row * K + k0 + 4 * l) = acc;
   }
 }
 

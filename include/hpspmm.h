@@ -60,6 +60,8 @@ typedef enum hpspmm_status {
 #define HPSPMM_PLAN_FORCE_ROUTED 64u  /* always use the routed strategy (hub columns pinned to one XCD each);
                                          bits 16..23 then give log2 of the total number of hub rows (0 = auto) */
 #define HPSPMM_PLAN_NO_ROUTED 128u    /* never use the routed strategy */
+/* bits 24..28, with FORCE_ROUTED: log2 of the shortest row that is routed (0 = default, 128) */
+#define HPSPMM_PLAN_ROUTED_ROW_LOG2(log2_nnz) (((uint32_t)(log2_nnz) & 0x1Fu) << 24)
 /* bits 16..23: log2 of the number of cached rows (0 = default, 2^16) */
 #define HPSPMM_PLAN_HUB_LOG2(log2_rows) (((uint32_t)(log2_rows) & 0xFFu) << 16)
 /* bits 8..15: log2 of the segment length to force (0 = choose automatically) */

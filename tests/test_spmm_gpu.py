@@ -55,8 +55,10 @@ def _strategies(capi):
             ("seg16_hub_all", capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(4) | capi.PLAN_HUB_CACHE
              | capi.plan_hub_log2(24)),
             ("routed", capi.PLAN_FORCE_ROUTED),
-            ("routed_tiny", capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(3) | capi.plan_segment_shift(3)),
-            ("routed_s16", capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(10) | capi.plan_segment_shift(4))]
+            ("routed_tiny", capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(3) | capi.plan_segment_shift(3)
+             | capi.plan_routed_row_log2(1)),
+            ("routed_s16", capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(10) | capi.plan_segment_shift(4)
+             | capi.plan_routed_row_log2(3))]
 
 
 @pytest.mark.parametrize("k", [32, 64, 128])
@@ -97,8 +99,9 @@ def test_deterministic_and_strategies_agree(pkg, oracle, gpu):
     ref, _ = _run(pkg, gpu, g, B, pkg.capi.PLAN_FORCE_SEGMENTS)
     again, _ = _run(pkg, gpu, g, B, pkg.capi.PLAN_FORCE_SEGMENTS)
     assert np.array_equal(ref, again), "segments strategy must be bit-reproducible"
-    r1, info = _run(pkg, gpu, g, B, pkg.capi.PLAN_FORCE_ROUTED | pkg.capi.plan_hub_log2(9))
-    r2, _ = _run(pkg, gpu, g, B, pkg.capi.PLAN_FORCE_ROUTED | pkg.capi.plan_hub_log2(9))
+    fl = pkg.capi.PLAN_FORCE_ROUTED | pkg.capi.plan_hub_log2(9) | pkg.capi.plan_routed_row_log2(2)
+    r1, info = _run(pkg, gpu, g, B, fl)
+    r2, _ = _run(pkg, gpu, g, B, fl)
     assert info["strategy"] == pkg.capi.STRATEGY_ROUTED and info["hub_rows"] > 0
     assert np.array_equal(r1, r2), "routed strategy must be bit-reproducible"
     rows, _ = _run(pkg, gpu, g, B, pkg.capi.PLAN_FORCE_ROWS)

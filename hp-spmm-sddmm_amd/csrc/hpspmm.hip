@@ -132,14 +132,9 @@ template <int K>
 int launch_rows(int64_t rows, int64_t cols, const int32_t* rp, const int32_t* ci, const float* v, const float* B,
                 float* C, int32_t long_threshold, const int32_t* long_rows, int64_t n_long, hipStream_t st) {
   if constexpr (K >= 64) {
-    if (cols * K * 4 > kRowsUntiledBytes) {
-      if constexpr (K == 128) {
-        if (cols * 64 * 4 <= kRowsTileBytes)
-          return launch_rows_tiled<K, 64>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
-      }
-      if (cols * 32 * 4 <= kRowsTileBytes)
-        return launch_rows_tiled<K, 32>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
-    }
+    // 32-wide tiles only: a 64-wide tile of a B beyond kRowsUntiledBytes can never be within kRowsTileBytes
+    if (cols * K * 4 > kRowsUntiledBytes && cols * 32 * 4 <= kRowsTileBytes)
+      return launch_rows_tiled<K, 32>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
   }
   return launch_rows_tiled<K, K>(rows, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
 }

@@ -288,3 +288,56 @@ def test_error_codes(pkg, gpu):
     plan = capi.Plan(3, 3, rp, ci, 32)
     assert plan.info["rows"] == 3
     plan.destroy()
+
+
+def _sample_check(oracle, g, B, C_dev, ranges, what):
+    """Oracle check on contiguous row ranges of a large result held on the GPU."""
+    for lo, hi in ranges:
+        got = C_dev[lo:hi].cpu().numpy()
+        C64, S64 = oracle.csr_spmm_f64_rows(g.rowptr, g.col, g.val, B, lo, hi)
+        err, pos = oracle.max_norm_err(got, C64, S64)
+        assert err <= TOL, f"{what}: rows [{lo},{hi}) normalised error {err:.3e} at {pos}"
+        deg = np.diff(g.rowptr[lo:hi + 1])
+        assert not got[deg == 0].any()
+
+
+@pytest.mark.parametrize("name,k", [("c2_social", 128), ("c2_social", 64), ("c4_rmat", 128), ("c3_copurchase", 64),
+                                    ("c2_social", 32)])
+def test_full_size_configs(pkg, oracle, gpu, name, k):
+    """The benchmark configurations at full size, default plan (the strategy the benchmark times):
+    oracle on row samples, agreement between strategies, NaN-poisoned C fully overwritten."""
+    import torch
+    capi = pkg.capi
+    g = pkg.graphs.make_graph(name)
+    B = pkg.graphs.make_dense(name, g.cols, k)
+    rp, ci, v, Bd = _to_dev(gpu, g.rowptr, g.col, g.val, B)
+    out = {}
+    for tag, flags in (("auto", capi.PLAN_DEFAULT),
+                       ("plain", capi.PLAN_FORCE_SEGMENTS | capi.PLAN_NO_HUB_CACHE | capi.PLAN_NO_ROUTED)):
+        C = torch.full((g.rows, k), float("nan"), device=gpu)
+        plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
+        info = plan.info
+        capi.csr_spmm(plan, rp, ci, v, Bd, C)
+        torch.cuda.synchronize()
+        plan.destroy()
+        assert not torch.isnan(C).any().item(), f"{name} K={k} {tag}: C not fully written"
+        out[tag] = (C, info)
+    expect = {("c2_social", 128): capi.STRATEGY_ROUTED, ("c2_social", 64): capi.STRATEGY_ROUTED,
+              ("c4_rmat", 128): capi.STRATEGY_ROUTED, ("c3_copurchase", 64): capi.STRATEGY_SEGMENTS,
+              ("c2_social", 32): capi.STRATEGY_SEGMENTS}[(name, k)]
+    assert out["auto"][1]["strategy"] == expect
+    # the two strategies sum in different orders: they agree to rounding, scaled by |A| |B|
+    plan = capi.Plan(g.rows, g.cols, rp, ci, k, capi.PLAN_FORCE_SEGMENTS | capi.PLAN_NO_HUB_CACHE | capi.PLAN_NO_ROUTED)
+    S = torch.empty((g.rows, k), device=gpu)
+    capi.csr_spmm(plan, rp, ci, v.abs(), Bd.abs(), S)
+    torch.cuda.synchronize()
+    plan.destroy()
+    diff = (out["auto"][0] - out["plain"][0]).abs()
+    assert torch.all(diff <= TOL * S).item(), f"{name} K={k}: strategies disagree by {float((diff / S.clamp_min(1e-30)).max()):.3e}"
+    del S, diff
+    # oracle on three row ranges, including the heaviest rows
+    deg = np.diff(g.rowptr)
+    top = int(np.argmax(deg))
+    lo = max(0, min(top - 50, g.rows - 200))
+    ranges = [(0, 300), (lo, lo + 200), (g.rows - 300, g.rows)]
+    _sample_check(oracle, g, B, out["auto"][0], ranges, f"{name} K={k}")

@@ -42,6 +42,13 @@ WORKLOADS = [
 ]
 ROOFLINE_WORKLOAD = ("c2_social", 128)
 
+# L2<->fabric bytes per SpMM (all launches) of the roofline workload, from two rocprofv3 --pmc
+# runs (FETCH_SIZE, WRITE_SIZE, each scaled by what a 1 GiB copy kernel reads on the same
+# counter); summary in profiles/spmm_routed_kernel__c2_social.txt.  Counters cannot be read
+# from inside this process, so the figure is carried here and only reported for the exact
+# configuration it was measured on: (workload, K, strategy) at scale 1.
+MEASURED_TRAFFIC_BYTES = {("c2_social", 128, 4): 31.739e9 + 1.120e9 + 0.07e9}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -203,7 +210,9 @@ def main():
                 f"({100 * gbs / HBM_PEAK_GBS:.1f}% of 8 TB/s)  strategy={info['strategy']} seg={info['segment_length']} plan={plan_ms:.1f} ms")
             if (name, k) == ROOFLINE_WORKLOAD:
                 roofline = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                            "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                            "frac": gbs / HBM_PEAK_GBS,
+                            "traffic": MEASURED_TRAFFIC_BYTES.get((name, k, info["strategy"]))
+                            if args.scale == 1.0 and args.plan_flags == 0 else None,
                             "kernel": {1: "spmm_rows_kernel<128>",
                                        2: "spmm_segments_kernel<128> + spmm_fixup_kernel<128>",
                                        4: "routed_gather_hub_kernel<128> + spmm_routed_kernel<128> + "

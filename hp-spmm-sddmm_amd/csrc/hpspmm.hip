@@ -88,6 +88,9 @@ struct hpspmm_plan {
   int32_t* d_vrow = nullptr;      // [vtotal]
   int32_t* d_bhot_src = nullptr;  // [n_bhot] source column of every compact-buffer row (-1 = unused)
   uint8_t* d_action = nullptr;    // [rows] what the final kernel does with each row
+  int32_t* d_reduce_rows = nullptr;  // rows whose class results must be added
+  int32_t* d_zero_rows = nullptr;    // rows without nonzeros
+  int64_t n_reduce = 0, n_zero = 0;
   float* d_partial = nullptr;     // [9 * rows * k]
   int64_t n_bhot = 0;
   int64_t routed_grid = 0;
@@ -375,6 +378,32 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
                      p->shift);
   HPSPMM_HIP(hipStreamSynchronize(st));
   HPSPMM_HIP(hipGetLastError());
+  // compact lists of the rows the final kernel has to visit
+  {
+    int32_t* d_counts = nullptr;
+    HPSPMM_HIP(hipMalloc(&d_counts, 2 * sizeof(int32_t)));
+    struct CountGuard {
+      int32_t* q;
+      ~CountGuard() { (void)hipFree(q); }
+    } cg{d_counts};
+    HPSPMM_HIP(hipMemsetAsync(d_counts, 0, 2 * sizeof(int32_t), st));
+    if (hipMalloc(&p->d_reduce_rows, (size_t)rows * sizeof(int32_t)) != hipSuccess ||
+        hipMalloc(&p->d_zero_rows, (size_t)rows * sizeof(int32_t)) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(HPSPMM_ERR_ALLOC, "device allocation for the routed row lists failed");
+    }
+    p->workspace_bytes += 2 * rows * (int64_t)sizeof(int32_t);
+    const unsigned cgrid = (unsigned)ceil_div(rows, hpspmm::kBlock);
+    hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(cgrid), dim3(hpspmm::kBlock), 0, st, rows, p->d_action,
+                       hpspmm::kActionReduce, p->d_reduce_rows, d_counts);
+    hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(cgrid), dim3(hpspmm::kBlock), 0, st, rows, p->d_action,
+                       hpspmm::kActionZero, p->d_zero_rows, d_counts + 1);
+    int32_t counts[2] = {0, 0};
+    HPSPMM_HIP(hipMemcpyAsync(counts, d_counts, sizeof counts, hipMemcpyDeviceToHost, st));
+    HPSPMM_HIP(hipStreamSynchronize(st));
+    p->n_reduce = counts[0];
+    p->n_zero = counts[1];
+  }
   p->n_bhot = n_bhot;
   p->n_hub = (int64_t)ids.size();
   p->nseg = nseg;
@@ -391,9 +420,12 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
     hipLaunchKernelGGL(hpspmm::spmm_routed_kernel<K>, dim3((unsigned)p->routed_grid), dim3(hpspmm::kBlock), 0, st,
                        p->lay, p->d_vptr, p->d_vcol, p->d_vsrc, p->d_vrow, v, B, p->d_bhot, p->d_partial,
                        p->d_carry, C);
-  const int64_t fin_blocks = ceil_div(ceil_div(p->rows, 64), hpspmm::kWavesPerBlock);
-  hipLaunchKernelGGL(hpspmm::spmm_routed_final_kernel<K>, dim3((unsigned)fin_blocks), dim3(hpspmm::kBlock), 0, st,
-                     p->lay, p->d_vptr, p->d_action, p->d_partial, p->d_carry, C);
+  const int64_t reduce_blocks = row_blocks(p->n_reduce, K);
+  const int64_t fin_blocks = reduce_blocks + row_blocks(p->n_zero, K);
+  if (fin_blocks > 0)
+    hipLaunchKernelGGL(hpspmm::spmm_routed_final_kernel<K>, dim3((unsigned)fin_blocks), dim3(hpspmm::kBlock), 0, st,
+                       p->lay, p->d_vptr, p->d_reduce_rows, p->n_reduce, reduce_blocks, p->d_zero_rows, p->n_zero,
+                       p->d_partial, p->d_carry, C);
   return HPSPMM_OK;
 }
 
@@ -608,7 +640,8 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
   if (plan->d_hub_col) (void)hipFree(plan->d_hub_col);
   if (plan->d_bhot) (void)hipFree(plan->d_bhot);
   for (void* q : {(void*)plan->d_vptr, (void*)plan->d_vcol, (void*)plan->d_vsrc, (void*)plan->d_vrow,
-                  (void*)plan->d_bhot_src, (void*)plan->d_partial, (void*)plan->d_action})
+                  (void*)plan->d_bhot_src, (void*)plan->d_partial, (void*)plan->d_action,
+                  (void*)plan->d_reduce_rows, (void*)plan->d_zero_rows})
     if (q) (void)hipFree(q);
   delete plan;
   return HPSPMM_OK;

@@ -350,15 +350,35 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
   flush_to((int64_t)vp[(cur & 0x7FFFFFFF) + 1] > e);
 }
 
-// Final pass.  A wavefront takes 64 consecutive rows, reads their action bytes
-// and lets its sub-waves serve the rows that need work: zeros for empty rows;
-// for kActionReduce rows the sum over the classes, in class order, of the
-// class result - the partial-buffer row if the (row, class) run lies in one
-// segment, else tail[ga] + head[ga+1] + ... + head[gb] from the carry slots.
+// list[] <- every row whose action byte equals `which` (order unspecified); *count must be zero on entry.
+__global__ __launch_bounds__(kBlock) void routed_collect_rows_kernel(int64_t rows, const uint8_t* __restrict__ action,
+                                                                     uint8_t which, int32_t* __restrict__ list,
+                                                                     int32_t* __restrict__ count) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const bool hit = i < rows && action[i] == which;
+  const uint64_t mask = __ballot(hit);
+  if (mask == 0) return;
+  const int lane = threadIdx.x & 63;
+  int32_t base = 0;
+  if (lane == 0) base = atomicAdd(count, (int32_t)__popcll(mask));
+  base = __shfl(base, 0);
+  if (hit) list[base + __popcll(mask & ((1ull << lane) - 1ull))] = (int32_t)i;
+}
+
+// Final pass, one sub-wave per listed row.  Workgroups [0, reduce_blocks): rows
+// whose class results must be added - in class order, the partial-buffer row if
+// the (row, class) run lies in one segment, else tail[ga] + head[ga+1] + ... +
+// head[gb] from the carry slots.  Remaining workgroups: rows without nonzeros,
+// which get zeros.  Rows in neither list were stored by the main kernel.
+// (Lists rather than a scan over all rows: on R-MAT the rows that need a
+// reduction sit together at low indices and serialised inside a few waves.)
 template <int K>
 __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout lay,
                                                                    const int32_t* __restrict__ vptr,
-                                                                   const uint8_t* __restrict__ action,
+                                                                   const int32_t* __restrict__ reduce_rows,
+                                                                   int64_t n_reduce, int64_t reduce_blocks,
+                                                                   const int32_t* __restrict__ zero_rows,
+                                                                   int64_t n_zero,
                                                                    const float* __restrict__ partial,
                                                                    const float* __restrict__ carry,
                                                                    float* __restrict__ C) {
@@ -367,47 +387,66 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
-  const int sub = lane / G;
-  const int64_t r0 = ((int64_t)blockIdx.x * kWavesPerBlock + (tid >> 6)) * 64;
-  if (r0 >= lay.rows) return;
-  const uint8_t a = r0 + lane < lay.rows ? action[r0 + lane] : kActionNone;
-  const uint64_t m_zero = __ballot(a == kActionZero);
-  const uint64_t m_reduce = __ballot(a == kActionReduce);
-  if ((m_zero | m_reduce) == 0) return;
   const int shift = lay.shift;
-
-  for (int i = sub; i < 64; i += P) {
-    const bool zero = (m_zero >> i) & 1ull;
-    const bool reduce = (m_reduce >> i) & 1ull;
-    if (!zero && !reduce) continue;
-    const int64_t row = r0 + i;
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (reduce) {
-      auto add = [&](const float* src) {
-        const float4 t = *reinterpret_cast<const float4*>(src + 4 * l);
-        acc.x += t.x;
-        acc.y += t.y;
-        acc.z += t.z;
-        acc.w += t.w;
-      };
-#pragma unroll 1
-      for (int x = 0; x < kClasses; ++x) {
-        const int32_t* vp = vptr + (int64_t)x * (lay.rows + 1);
-        const int64_t lb = vp[row];
-        const int64_t hb = vp[row + 1];
-        if (lb == hb) continue;
-        const int64_t ga = lb >> shift;
-        const int64_t gb = (hb - 1) >> shift;
-        if (ga == gb) {
-          add(partial + ((uint64_t)x * (uint64_t)lay.rows + (uint64_t)row) * K);
-        } else {
-          add(carry + (uint64_t)(2 * ga + 1) * K);
-          for (int64_t g = ga + 1; g <= gb; ++g) add(carry + (uint64_t)(2 * g) * K);
-        }
-      }
-    }
-    *reinterpret_cast<float4*>(C + (uint64_t)row * K + 4 * l) = acc;
+  if ((int64_t)blockIdx.x >= reduce_blocks) {
+    const int64_t idx = (((int64_t)blockIdx.x - reduce_blocks) * kWavesPerBlock + (tid >> 6)) * P + lane / G;
+    if (idx >= n_zero) return;
+    *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * K + 4 * l) = make_float4(0.f, 0.f, 0.f, 0.f);
+    return;
   }
+  const int64_t idx = ((int64_t)blockIdx.x * kWavesPerBlock + (tid >> 6)) * P + lane / G;
+  if (idx >= n_reduce) return;
+  const int64_t row = reduce_rows[idx];
+
+  // all class bounds first, then all single-segment partials, so that the loads
+  // of a row are in flight together; the adds stay in class order
+  int64_t lb[kClasses], hb[kClasses];
+#pragma unroll
+  for (int x = 0; x < kClasses; ++x) {
+    const int32_t* vp = vptr + (int64_t)x * (lay.rows + 1);
+    lb[x] = vp[row];
+    hb[x] = vp[row + 1];
+  }
+  float4 part[kClasses];
+  bool single[kClasses];
+#pragma unroll
+  for (int x = 0; x < kClasses; ++x) {
+    single[x] = lb[x] != hb[x] && (lb[x] >> shift) == ((hb[x] - 1) >> shift);
+    part[x] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (single[x])
+      part[x] =
+          *reinterpret_cast<const float4*>(partial + ((uint64_t)x * (uint64_t)lay.rows + (uint64_t)row) * K + 4 * l);
+  }
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  auto add = [&](const float4& t) {
+    acc.x += t.x;
+    acc.y += t.y;
+    acc.z += t.z;
+    acc.w += t.w;
+  };
+#pragma unroll
+  for (int x = 0; x < kClasses; ++x) {
+    if (lb[x] == hb[x]) continue;
+    if (single[x]) {
+      add(part[x]);
+    } else {
+      // a hub row spans hundreds of segments: fetch the carry slots 8 at a time, add them in segment order
+      const int64_t ga = lb[x] >> shift;
+      const int64_t gb = (hb[x] - 1) >> shift;
+      add(*reinterpret_cast<const float4*>(carry + (uint64_t)(2 * ga + 1) * K + 4 * l));
+      int64_t g = ga + 1;
+      for (; g + kBatch <= gb + 1; g += kBatch) {
+        float4 slot[kBatch];
+#pragma unroll
+        for (int q = 0; q < kBatch; ++q)
+          slot[q] = *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * (g + q)) * K + 4 * l);
+#pragma unroll
+        for (int q = 0; q < kBatch; ++q) add(slot[q]);
+      }
+      for (; g <= gb; ++g) add(*reinterpret_cast<const float4*>(carry + (uint64_t)(2 * g) * K + 4 * l));
+    }
+  }
+  *reinterpret_cast<float4*>(C + (uint64_t)row * K + 4 * l) = acc;
 }
 
 }  // namespace hpspmm

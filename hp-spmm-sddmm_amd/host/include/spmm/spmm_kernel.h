@@ -21,5 +21,9 @@ void LBSpMM(const COO_Matrix& mat1, const Matrix& mat2, Matrix& result, float& t
 // reference: 2, 3 or -1 (default).  Returns false (time = 0) when the library
 // call is not available.
 bool rocsparseCSRSpMM(const CSR_Matrix& mat1, const Matrix& mat2, Matrix& result, int algid, float& time);
+// Vendor comparator in the role of cusparseCOOSpMM (spmm_kernel.cu:154-238): rocSPARSE COO SpMM
+// (segmented algorithm), alpha = 1, beta = 0, row-major.  The COO arrays must hold the rows in
+// ascending order (the plain loader's output, not the reordered one).
+bool rocsparseCOOSpMM(const COO_Matrix& mat1, const Matrix& mat2, Matrix& result, float& time);
 // x[i] = val on the device (spmm_kernel.cu:23-34).
 void fill_matrix(starml::Matrix& a, float val);

@@ -78,25 +78,16 @@ void fill_matrix(starml::Matrix& a, float val) {
   check_status(hpspmm_fill_f32(a.mutable_data<float>(), a.size(), val, nullptr), "fill_matrix");
 }
 
-bool rocsparseCSRSpMM(const CSR_Matrix& mat1, const Matrix& mat2, Matrix& result, int algid, float& time) {
-  time = 0.f;
-  const Matrix rp = mat1.row_offsets(), ci = mat1.column_indices(), va = mat1.values();
-  const Dims d = check_operands(mat1.num_rows(), mat1.num_cols(), rp, ci, va, mat2, result, "rocsparseCSRSpMM");
-  rocsparse_spmm_alg alg = rocsparse_spmm_alg_default;
-  if (algid == 2) alg = rocsparse_spmm_alg_csr_row_split;
-  if (algid == 3) alg = rocsparse_spmm_alg_csr_nnz_split;
-  if (algid == 4) alg = rocsparse_spmm_alg_csr_merge_path;
+namespace {
 
-  rocsparse_handle handle = nullptr;
-  rocsparse_spmat_descr A = nullptr;
+// Shared body of the two vendor comparators: descriptors for B and C, buffer,
+// preprocess, WARMUP_NUM_CUDA + EXE_NUM_CUDA timed compute calls.
+bool rocsparse_spmm_timed(rocsparse_spmat_descr A, const Dims& d, const Matrix& mat2, Matrix& result,
+                          rocsparse_spmm_alg alg, rocsparse_handle handle, float& time) {
   rocsparse_dnmat_descr B = nullptr, C = nullptr;
   void* buffer = nullptr;
-  bool ok = rocsparse_create_handle(&handle) == rocsparse_status_success;
-  ok = ok && rocsparse_create_csr_descr(&A, d.m, d.n, d.nnz, rp.raw_mutable_data(), ci.raw_mutable_data(),
-                                        va.raw_mutable_data(), rocsparse_indextype_i32, rocsparse_indextype_i32,
-                                        rocsparse_index_base_zero, rocsparse_datatype_f32_r) == rocsparse_status_success;
-  ok = ok && rocsparse_create_dnmat_descr(&B, d.n, d.k, d.k, mat2.raw_mutable_data(), rocsparse_datatype_f32_r,
-                                          rocsparse_order_row) == rocsparse_status_success;
+  bool ok = rocsparse_create_dnmat_descr(&B, d.n, d.k, d.k, mat2.raw_mutable_data(), rocsparse_datatype_f32_r,
+                                         rocsparse_order_row) == rocsparse_status_success;
   ok = ok && rocsparse_create_dnmat_descr(&C, d.m, d.k, d.k, result.raw_mutable_data(), rocsparse_datatype_f32_r,
                                           rocsparse_order_row) == rocsparse_status_success;
   const float alpha = 1.0f, beta = 0.0f;
@@ -119,8 +110,45 @@ bool rocsparseCSRSpMM(const CSR_Matrix& mat1, const Matrix& mat2, Matrix& result
   if (buffer) (void)hipFree(buffer);
   if (C) rocsparse_destroy_dnmat_descr(C);
   if (B) rocsparse_destroy_dnmat_descr(B);
+  return ok;
+}
+
+}  // namespace
+
+bool rocsparseCSRSpMM(const CSR_Matrix& mat1, const Matrix& mat2, Matrix& result, int algid, float& time) {
+  time = 0.f;
+  const Matrix rp = mat1.row_offsets(), ci = mat1.column_indices(), va = mat1.values();
+  const Dims d = check_operands(mat1.num_rows(), mat1.num_cols(), rp, ci, va, mat2, result, "rocsparseCSRSpMM");
+  rocsparse_spmm_alg alg = rocsparse_spmm_alg_default;
+  if (algid == 2) alg = rocsparse_spmm_alg_csr_row_split;
+  if (algid == 3) alg = rocsparse_spmm_alg_csr_nnz_split;
+  if (algid == 4) alg = rocsparse_spmm_alg_csr_merge_path;
+  rocsparse_handle handle = nullptr;
+  rocsparse_spmat_descr A = nullptr;
+  bool ok = rocsparse_create_handle(&handle) == rocsparse_status_success;
+  ok = ok && rocsparse_create_csr_descr(&A, d.m, d.n, d.nnz, rp.raw_mutable_data(), ci.raw_mutable_data(),
+                                        va.raw_mutable_data(), rocsparse_indextype_i32, rocsparse_indextype_i32,
+                                        rocsparse_index_base_zero, rocsparse_datatype_f32_r) == rocsparse_status_success;
+  ok = ok && rocsparse_spmm_timed(A, d, mat2, result, alg, handle, time);
   if (A) rocsparse_destroy_spmat_descr(A);
   if (handle) rocsparse_destroy_handle(handle);
   if (ok) std::cout << "rocSPARSE CSR SpMM (alg " << algid << ") time: " << time << " ms " << std::endl;
+  return ok;
+}
+
+bool rocsparseCOOSpMM(const COO_Matrix& mat1, const Matrix& mat2, Matrix& result, float& time) {
+  time = 0.f;
+  const Matrix ri = mat1.row_indices(), ci = mat1.column_indices(), va = mat1.values();
+  const Dims d = check_operands(mat1.num_rows(), mat1.num_cols(), ri, ci, va, mat2, result, "rocsparseCOOSpMM");
+  rocsparse_handle handle = nullptr;
+  rocsparse_spmat_descr A = nullptr;
+  bool ok = rocsparse_create_handle(&handle) == rocsparse_status_success;
+  ok = ok && rocsparse_create_coo_descr(&A, d.m, d.n, d.nnz, ri.raw_mutable_data(), ci.raw_mutable_data(),
+                                        va.raw_mutable_data(), rocsparse_indextype_i32, rocsparse_index_base_zero,
+                                        rocsparse_datatype_f32_r) == rocsparse_status_success;
+  ok = ok && rocsparse_spmm_timed(A, d, mat2, result, rocsparse_spmm_alg_coo_segmented, handle, time);
+  if (A) rocsparse_destroy_spmat_descr(A);
+  if (handle) rocsparse_destroy_handle(handle);
+  if (ok) std::cout << "rocSPARSE COO SpMM time: " << time << " ms " << std::endl;
   return ok;
 }

@@ -43,7 +43,7 @@ int main(int argc, char** argv) {
     ResInfo info;
     int64_t num = 0, dim = 0, nnz = 0;
     CSR_Matrix h_csr;
-    COO_Matrix h_coo_reorder;
+    COO_Matrix h_coo_reorder, h_coo;
     if (synthetic) {
       info.filename_ = pos[0] + "@" + pos[1];
       h_csr = make_synthetic_csr(pos[0], std::stod(pos[1]));
@@ -54,10 +54,12 @@ int main(int argc, char** argv) {
       std::vector<int32_t> order((size_t)num);
       std::iota(order.begin(), order.end(), 0);
       h_coo_reorder = csr_to_coo_reorder(h_csr, order, 32);
+      h_coo = csr_to_coo(h_csr, 1);
     } else {
       info.filename_ = pos[0];
       info.stdv = get_standard_CV(pos[0]);
       h_csr = get_csr_mat_from_smtx(pos[0], num, dim, nnz);
+      h_coo = get_coo_mat_from_smtx(pos[0], num, dim, nnz, 1);  // unpadded: the vendor routine wants sorted rows
       h_coo_reorder = pos[1] == "-" ? get_coo_mat_from_smtx(pos[0], num, dim, nnz, 32)
                                     : get_coo_mat_from_smtx_reorder(pos[0], pos[1], num, dim, nnz, 32);
     }
@@ -78,6 +80,12 @@ int main(int argc, char** argv) {
     bool have_ref = rocsparseCSRSpMM(d_csr, d_B, d_ref, 2, info.spmm_cs_csralg2_time_);
     have_ref = rocsparseCSRSpMM(d_csr, d_B, d_ref, 3, info.spmm_cs_csralg3_time_) || have_ref;
     have_ref = rocsparseCSRSpMM(d_csr, d_B, d_ref, -1, info.spmm_cs_csrdef_time_) || have_ref;
+    {
+      // vendor COO baseline on the row-ordered, unpadded COO
+      COO_Matrix d_coo_plain = coo_to_cuda(h_coo);
+      Matrix d_tmp = full({num, k}, Device(kHIP), DataType(kFloat), 0.0);
+      rocsparseCOOSpMM(d_coo_plain, d_B, d_tmp, info.spmm_cs_coo_time_);
+    }
     (void)hipDeviceSynchronize();
 
     fill_matrix(d_csr_out, 0.0f);

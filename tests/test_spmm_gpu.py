@@ -341,3 +341,63 @@ def test_full_size_configs(pkg, oracle, gpu, name, k):
     lo = max(0, min(top - 50, g.rows - 200))
     ranges = [(0, 300), (lo, lo + 200), (g.rows - 300, g.rows)]
     _sample_check(oracle, g, B, out["auto"][0], ranges, f"{name} K={k}")
+
+
+def _random_csr(rng, rows, cols, mean_deg, skew, empty_frac, sorted_unique=True):
+    """Random CSR with a heavy-tailed degree sequence; optionally unsorted columns with duplicates."""
+    deg = np.minimum((rng.pareto(skew, rows) + 0.2) * mean_deg, cols * (1 if sorted_unique else 3)).astype(np.int64)
+    deg[rng.random(rows) < empty_frac] = 0
+    rowptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    parts = []
+    for d in deg:
+        if sorted_unique:
+            parts.append(np.sort(rng.choice(cols, size=int(d), replace=False)))
+        else:
+            parts.append(rng.integers(0, cols, size=int(d)))
+    col = (np.concatenate(parts) if parts else np.zeros(0)).astype(np.int32)
+    val = rng.uniform(-1, 1, col.size).astype(np.float32)
+    return rowptr, col, val
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_matrices_all_strategies(pkg, oracle, gpu, seed):
+    """Randomised shapes, degree skews, empty rows; every strategy against scipy float64
+    (independent of the oracle) at the benchmark tolerance."""
+    import scipy.sparse as sp
+    rng = np.random.default_rng(1000 + seed)
+    rows = int(rng.integers(1, 3000))
+    cols = int(rng.integers(1, 3000))
+    k = int(rng.choice([32, 64, 128]))
+    rowptr, col, val = _random_csr(rng, rows, cols, mean_deg=float(rng.uniform(0.5, 40)),
+                                   skew=float(rng.uniform(0.8, 3.0)), empty_frac=float(rng.uniform(0, 0.6)),
+                                   sorted_unique=(seed % 3 != 2))
+    g = pkg.graphs.CSR(rows, cols, rowptr, col, val)
+    B = rng.standard_normal((cols, k)).astype(np.float32)
+    # copies: scipy canonicalises (sorts, merges duplicates) in place on the arrays it is given
+    A = sp.csr_matrix((val.astype(np.float64), col.copy(), rowptr.copy()), shape=(rows, cols))
+    Aabs = sp.csr_matrix((np.abs(val).astype(np.float64), col.copy(), rowptr.copy()), shape=(rows, cols))
+    want = A @ B.astype(np.float64)
+    S = Aabs @ np.abs(B).astype(np.float64)
+    for name, flags in _strategies(pkg.capi):
+        C, _ = _run(pkg, gpu, g, B, flags)
+        bad = np.abs(C - want) > TOL * S
+        assert not bad.any(), f"seed {seed} rows={rows} cols={cols} k={k} {name}: {int(bad.sum())} elements off"
+        assert not C[np.diff(rowptr) == 0].any()
+
+
+def test_non_finite_values_stay_in_their_rows(pkg, oracle, gpu):
+    """An inf / NaN in B reaches exactly the rows that reference that row of B (no 0 * inf leaks
+    from padding or predication)."""
+    g = pkg.graphs.make_graph("c1_citation", 0.1)
+    for k in (32, 64, 128):
+        B = pkg.graphs.dense_normal(g.cols, k, 5)
+        B[7, 3] = np.inf
+        B[11, 0] = np.nan
+        rows = np.repeat(np.arange(g.rows), np.diff(g.rowptr))
+        touched = np.zeros(g.rows, dtype=bool)
+        touched[rows[(g.col == 7) | (g.col == 11)]] = True
+        for name, flags in _strategies(pkg.capi):
+            C, _ = _run(pkg, gpu, g, B, flags)
+            finite_rows = np.isfinite(C).all(axis=1)
+            assert finite_rows[~touched].all(), f"k={k} {name}: non-finite value leaked into an unrelated row"
+            assert (~finite_rows[touched]).all(), f"k={k} {name}: a referencing row lost the non-finite value"

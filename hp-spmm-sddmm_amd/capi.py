@@ -38,6 +38,10 @@ def plan_routed_row_log2(log2_nnz):
     return (int(log2_nnz) & 0x1F) << 24
 
 
+def plan_routed_phases(n):
+    return (int(n) & 0x7) << 29
+
+
 def plan_segment_shift(log2_len):
     return (int(log2_len) & 0xFF) << 8
 

@@ -82,16 +82,17 @@ struct hpspmm_plan {
   int64_t n_hub = 0;
   // routed strategy
   hpspmm::RoutedLayout lay{};
-  int32_t* d_vptr = nullptr;      // [9 * (rows + 1)]
+  int32_t* d_vptr = nullptr;      // [(rows + 1) * ncls]
   int32_t* d_vcol = nullptr;      // [vtotal] column, or compact-buffer row for hub classes
-  int32_t* d_vsrc = nullptr;      // [vtotal] index into the caller's value array
+  int32_t* d_vpos = nullptr;      // [nnz] position of every stored nonzero in the class-major order
+  float* d_vval = nullptr;        // [vtotal] the values in that order, rewritten by every SpMM
   int32_t* d_vrow = nullptr;      // [vtotal]
   int32_t* d_bhot_src = nullptr;  // [n_bhot] source column of every compact-buffer row (-1 = unused)
   uint8_t* d_action = nullptr;    // [rows] what the final kernel does with each row
   int32_t* d_reduce_rows = nullptr;  // rows whose class results must be added
   int32_t* d_zero_rows = nullptr;    // rows without nonzeros
   int64_t n_reduce = 0, n_zero = 0;
-  float* d_partial = nullptr;     // [9 * rows * k]
+  float* d_partial = nullptr;     // [rows * ncls * k]
   int64_t n_bhot = 0;
   int64_t routed_grid = 0;
   int32_t* d_long_rows = nullptr;  // rows strategy: rows longer than long_threshold
@@ -271,18 +272,23 @@ constexpr int64_t kRoutedMinBBytes = (int64_t)48 << 20;  // B must overflow the 
 constexpr double kRoutedMinShare = 0.35;     // of the nonzeros in the 64k most referenced columns
 constexpr double kRoutedMinRowNnz = 32.0;    // mean nonzeros per non-empty row
 constexpr int32_t kRoutedRowThreshold = 128;  // rows shorter than this are not split over the classes
+// Phases: a slice of B larger than this is worked through in several phases.  Every phase
+// adds a partial-result row per routed row, so on the 233k-vertex social graph only
+// K = 128 (15 MB a slice) gains, and only from two phases: 4.16 -> 4.06 ms, three: 4.38 ms;
+// at K = 64 (7.5 MB a slice) one phase 2.18 ms, two 2.34 ms.
+constexpr int64_t kRoutedPhaseBytes = (int64_t)8 << 20;
 
 // Builds the routed layout.  Returns HPSPMM_OK with p->strategy left at
 // SEGMENTS when the graph does not qualify (and `forced` is false).
 int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, int log2_hubs,
-                 int log2_row_threshold, hipStream_t st) {
+                 int log2_row_threshold, int want_sub, hipStream_t st) {
   const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
   if (!forced && (nnz < kRoutedMinNnz || p->cols * k * 4 < kRoutedMinBBytes)) return HPSPMM_OK;
   // cached rows per class
   const int64_t h =
-      std::max<int64_t>(1, ((int64_t)1 << (log2_hubs ? log2_hubs : kRoutedLog2Cached)) / hpspmm::kHubClasses);
+      std::max<int64_t>(1, ((int64_t)1 << (log2_hubs ? log2_hubs : kRoutedLog2Cached)) / hpspmm::kSlices);
   std::vector<int32_t> count, ids;
-  if (int rc = rank_columns(p, d_col, h * hpspmm::kHubClasses, st, count, ids)) return rc;
+  if (int rc = rank_columns(p, d_col, h * hpspmm::kSlices, st, count, ids)) return rc;
   int64_t served = 0;
   for (int32_t c : ids) served += count[c];
   const int64_t nonempty = std::max<int64_t>(1, rows - p->empty_rows);
@@ -291,11 +297,19 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
     return HPSPMM_OK;
   if (nnz > INT32_MAX - ((int64_t)1 << 24)) return HPSPMM_OK;  // virtual indices stay int32
 
-  // popularity rank s -> class s % 8, compact-buffer row (s % 8) * h + s / 8
-  const int64_t n_bhot = h * hpspmm::kHubClasses;
+  // Phases: as many as bring one phase's share of a slice of B down to kRoutedPhaseBytes,
+  // at most 2 (see above); a B far beyond what phases could make L2-sized gets one.
+  const int64_t slice_bytes = p->cols * k * 4 / hpspmm::kSlices;
+  int nsub = (int)std::min<int64_t>(2, std::max<int64_t>(1, ceil_div(slice_bytes, kRoutedPhaseBytes)));
+  if (slice_bytes > kRoutedPhaseBytes * 4) nsub = 1;
+  if (want_sub) nsub = std::min(want_sub, hpspmm::kMaxSub);
+  const int ncls = hpspmm::kSlices * nsub + 1;
+
+  // popularity rank s -> slice s % 8, compact-buffer row (s % 8) * h + s / 8
+  const int64_t n_bhot = h * hpspmm::kSlices;
   std::vector<int32_t> colmap((size_t)p->cols, -1), bhot_src((size_t)n_bhot, -1);
   for (size_t s2 = 0; s2 < ids.size(); ++s2) {
-    const int64_t slot = (int64_t)(s2 % hpspmm::kHubClasses) * h + (int64_t)(s2 / hpspmm::kHubClasses);
+    const int64_t slot = (int64_t)(s2 % hpspmm::kSlices) * h + (int64_t)(s2 / hpspmm::kSlices);
     colmap[ids[s2]] = (int32_t)slot;
     bhot_src[(size_t)slot] = ids[s2];
   }
@@ -310,7 +324,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
         if (*x) (void)hipFree(*x);
     }
   } guard{{(void**)&d_colmap, (void**)&d_cnt, (void**)&d_scan}};
-  const int64_t ncnt = rows * hpspmm::kClasses;
+  const int64_t ncnt = rows * ncls;
   HPSPMM_HIP(hipMalloc(&d_colmap, (size_t)std::max<int64_t>(1, p->cols) * sizeof(int32_t)));
   HPSPMM_HIP(hipMalloc(&d_cnt, (size_t)ncnt * sizeof(uint32_t)));
   HPSPMM_HIP(hipMalloc(&d_scan, (size_t)ncnt * sizeof(uint32_t)));
@@ -318,45 +332,56 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   const unsigned row_grid = (unsigned)ceil_div(rows, hpspmm::kWavesPerBlock);
   const int32_t min_row_nnz = forced && log2_row_threshold ? (1 << log2_row_threshold) : kRoutedRowThreshold;
   hipLaunchKernelGGL(hpspmm::routed_count_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col,
-                     d_colmap, (int32_t)h, min_row_nnz, d_cnt);
+                     d_colmap, (int32_t)h, nsub, min_row_nnz, d_cnt);
   if (int rc = exclusive_scan_u32(d_cnt, d_scan, ncnt, st)) return rc;
 
   // class sizes = differences of the scan at the class origins
-  uint32_t origin[hpspmm::kClasses];
-  for (int x = 0; x < hpspmm::kClasses; ++x)
+  uint32_t origin[hpspmm::kMaxClasses];
+  for (int x = 0; x < ncls; ++x)
     HPSPMM_HIP(hipMemcpyAsync(&origin[x], d_scan + (int64_t)x * rows, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
   HPSPMM_HIP(hipStreamSynchronize(st));
 
   hpspmm::RoutedLayout& lay = p->lay;
+  lay = hpspmm::RoutedLayout{};
   lay.rows = rows;
   lay.shift = p->shift;
+  lay.nsub = nsub;
+  lay.ncls = ncls;
   const int64_t subwaves = 64 / (k / 4);
   const int64_t quantum = ((int64_t)1 << p->shift) * subwaves * hpspmm::kWavesPerBlock;  // nonzeros per workgroup
-  int64_t at = 0, hub_blocks = 0;
-  for (int x = 0; x < hpspmm::kClasses; ++x) {
-    const int64_t n_x = (x + 1 < hpspmm::kClasses ? (int64_t)origin[x + 1] : nnz) - (int64_t)origin[x];
+  int64_t at = 0;
+  for (int x = 0; x < ncls; ++x) {
+    const int64_t n_x = (x + 1 < ncls ? (int64_t)origin[x + 1] : nnz) - (int64_t)origin[x];
     lay.cls_begin[x] = at;
     lay.cls_end[x] = at + n_x;
     lay.cls_blocks[x] = ceil_div(n_x, quantum);
     at += lay.cls_blocks[x] * quantum;
-    if (x < hpspmm::kHubClasses) hub_blocks = std::max(hub_blocks, lay.cls_blocks[x]);
   }
   const int64_t vtotal = std::max<int64_t>(at, 1);
-  lay.hub_grid = hub_blocks * hpspmm::kHubClasses;
-  p->routed_grid = lay.hub_grid + lay.cls_blocks[hpspmm::kColdClass];
+  // a phase's workgroups are interleaved by slice, so it takes 8 x its largest class
+  int64_t grid = 0;
+  for (int ph = 0; ph < nsub; ++ph) {
+    lay.phase_begin[ph] = grid;
+    int64_t most = 0;
+    for (int x = 0; x < hpspmm::kSlices; ++x) most = std::max(most, lay.cls_blocks[ph * hpspmm::kSlices + x]);
+    grid += most * hpspmm::kSlices;
+  }
+  lay.phase_begin[nsub] = grid;
+  p->routed_grid = grid + lay.cls_blocks[ncls - 1];
   if (vtotal >= INT32_MAX || p->routed_grid > INT32_MAX) return HPSPMM_OK;
 
   const int64_t nseg = vtotal >> p->shift;
-  const size_t vptr_bytes = (size_t)hpspmm::kClasses * (size_t)(rows + 1) * sizeof(int32_t);
+  const size_t vptr_bytes = (size_t)ncls * (size_t)(rows + 1) * sizeof(int32_t);
   const size_t v_bytes = (size_t)vtotal * sizeof(int32_t);
-  const size_t partial_bytes = (size_t)hpspmm::kClasses * (size_t)rows * (size_t)k * sizeof(float);
+  const size_t partial_bytes = (size_t)ncls * (size_t)rows * (size_t)k * sizeof(float);
   const size_t carry_bytes = (size_t)std::max<int64_t>(nseg, 1) * 2 * (size_t)k * sizeof(float);
   const size_t bhot_bytes = (size_t)n_bhot * (size_t)k * sizeof(float);
   // the segments strategy's buffers are not needed any more
   if (p->d_nnz_row) { (void)hipFree(p->d_nnz_row); p->d_nnz_row = nullptr; }
   if (p->d_carry) { (void)hipFree(p->d_carry); p->d_carry = nullptr; }
   if (hipMalloc(&p->d_vptr, vptr_bytes) != hipSuccess || hipMalloc(&p->d_vcol, v_bytes) != hipSuccess ||
-      hipMalloc(&p->d_vsrc, v_bytes) != hipSuccess || hipMalloc(&p->d_vrow, v_bytes) != hipSuccess ||
+      hipMalloc(&p->d_vval, v_bytes) != hipSuccess || hipMalloc(&p->d_vrow, v_bytes) != hipSuccess ||
+      hipMalloc(&p->d_vpos, (size_t)std::max<int64_t>(nnz, 1) * sizeof(int32_t)) != hipSuccess ||
       hipMalloc(&p->d_partial, partial_bytes) != hipSuccess || hipMalloc(&p->d_carry, carry_bytes) != hipSuccess ||
       hipMalloc(&p->d_bhot, bhot_bytes) != hipSuccess ||
       hipMalloc(&p->d_bhot_src, (size_t)n_bhot * sizeof(int32_t)) != hipSuccess ||
@@ -365,16 +390,18 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
     return fail(HPSPMM_ERR_ALLOC, "device allocation for the routed plan failed (%zu bytes)",
                 vptr_bytes + 3 * v_bytes + partial_bytes + carry_bytes + bhot_bytes);
   }
-  p->workspace_bytes = (int64_t)(vptr_bytes + 3 * v_bytes + partial_bytes + carry_bytes + bhot_bytes + n_bhot * 4);
+  p->workspace_bytes =
+      (int64_t)(vptr_bytes + 3 * v_bytes + (size_t)nnz * 4 + partial_bytes + carry_bytes + bhot_bytes + n_bhot * 4);
   HPSPMM_HIP(hipMemcpyAsync(p->d_bhot_src, bhot_src.data(), bhot_src.size() * sizeof(int32_t),
                             hipMemcpyHostToDevice, st));
-  // unused compact-buffer rows are never read; keep them defined anyway
+  // unused compact-buffer rows and the padding between the classes are never used; keep them defined anyway
   HPSPMM_HIP(hipMemsetAsync(p->d_bhot, 0, bhot_bytes, st));
-  const int64_t nvptr = (int64_t)hpspmm::kClasses * (rows + 1);
+  HPSPMM_HIP(hipMemsetAsync(p->d_vval, 0, v_bytes, st));
+  const int64_t nvptr = (int64_t)ncls * (rows + 1);
   hipLaunchKernelGGL(hpspmm::routed_vptr_kernel, dim3((unsigned)ceil_div(nvptr, hpspmm::kBlock)),
                      dim3(hpspmm::kBlock), 0, st, lay, d_scan, p->d_vptr);
   hipLaunchKernelGGL(hpspmm::routed_fill_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col,
-                     d_colmap, (int32_t)h, min_row_nnz, p->d_vptr, p->d_vcol, p->d_vsrc, p->d_vrow, p->d_action,
+                     d_colmap, (int32_t)h, nsub, min_row_nnz, p->d_vptr, p->d_vcol, p->d_vpos, p->d_vrow, p->d_action,
                      p->shift);
   HPSPMM_HIP(hipStreamSynchronize(st));
   HPSPMM_HIP(hipGetLastError());
@@ -413,13 +440,15 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
 
 template <int K>
 int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
-  const int64_t threads = p->n_bhot * (K / 4);
-  hipLaunchKernelGGL(hpspmm::routed_gather_hub_kernel<K>, dim3((unsigned)ceil_div(threads, hpspmm::kBlock)),
-                     dim3(hpspmm::kBlock), 0, st, p->n_bhot, p->d_bhot_src, B, p->d_bhot);
+  const int64_t gather_blocks = ceil_div(p->n_bhot * (K / 4), hpspmm::kBlock);
+  const int64_t prep_blocks = gather_blocks + ceil_div(ceil_div(p->nnz, 4), hpspmm::kBlock);
+  if (prep_blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  hipLaunchKernelGGL(hpspmm::routed_prepare_kernel<K>, dim3((unsigned)prep_blocks), dim3(hpspmm::kBlock), 0, st,
+                     p->n_bhot, gather_blocks, p->d_bhot_src, B, p->d_bhot, p->nnz, v, p->d_vpos, p->d_vval,
+                     aligned16(v, v, v));
   if (p->routed_grid > 0)
     hipLaunchKernelGGL(hpspmm::spmm_routed_kernel<K>, dim3((unsigned)p->routed_grid), dim3(hpspmm::kBlock), 0, st,
-                       p->lay, p->d_vptr, p->d_vcol, p->d_vsrc, p->d_vrow, v, B, p->d_bhot, p->d_partial,
-                       p->d_carry, C);
+                       p->lay, p->d_vptr, p->d_vcol, p->d_vval, p->d_vrow, B, p->d_bhot, p->d_partial, p->d_carry, C);
   const int64_t reduce_blocks = row_blocks(p->n_reduce, K);
   const int64_t fin_blocks = reduce_blocks + row_blocks(p->n_zero, K);
   if (fin_blocks > 0)
@@ -575,7 +604,8 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d
       !(flags & HPSPMM_PLAN_FORCE_SEGMENTS && !(flags & HPSPMM_PLAN_FORCE_ROUTED))) {
     if (int rc = build_routed(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_ROUTED) != 0,
                               (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 16) & 0xFFu) : 0,
-                              (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 24) & 0x1Fu) : 0, st)) {
+                              (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 24) & 0x1Fu) : 0,
+                              (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 29) & 0x7u) : 0, st)) {
       hpspmm_plan_destroy(p);
       return rc;
     }
@@ -639,7 +669,7 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
   if (plan->d_hub_ids) (void)hipFree(plan->d_hub_ids);
   if (plan->d_hub_col) (void)hipFree(plan->d_hub_col);
   if (plan->d_bhot) (void)hipFree(plan->d_bhot);
-  for (void* q : {(void*)plan->d_vptr, (void*)plan->d_vcol, (void*)plan->d_vsrc, (void*)plan->d_vrow,
+  for (void* q : {(void*)plan->d_vptr, (void*)plan->d_vcol, (void*)plan->d_vpos, (void*)plan->d_vval, (void*)plan->d_vrow,
                   (void*)plan->d_bhot_src, (void*)plan->d_partial, (void*)plan->d_action,
                   (void*)plan->d_reduce_rows, (void*)plan->d_zero_rows})
     if (q) (void)hipFree(q);

@@ -11,21 +11,26 @@
 //     rest by a hash of the index.  Slice x of B is only ever read by
 //     workgroups running on XCD x (workgroup b runs on XCD b % 8), so each L2
 //     sees an eighth of the columns and keeps the hot ones (measured on the
-//     233k-vertex social graph, K=128: 6.6 ms -> 4.5 ms);
+//     233k-vertex social graph, K=128: 6.6 ms -> 4.5 ms).  A slice can further
+//     be cut into up to 7 phases that an XCD works through one after the other,
+//     each with the same mix of hot and cold columns;
 //   * the most referenced rows of B are additionally copied, slice by slice,
 //     into a compact buffer at the start of every SpMM, which takes them off
 //     whatever memory channels their original addresses collide on;
 //   * degree binning: only rows with at least `min_row_nnz` nonzeros are
 //     routed - a short row would pay one partial-result row per class it
 //     touches for a handful of gathers.  A nonzero of a routed row belongs to
-//     the class of its column's slice, all nonzeros of a short row to class 8.
-//     The plan lays the nonzeros out class by class, each class in row order,
-//     as three arrays: column (~compact-buffer row if the column is cached),
-//     source index into the caller's value array, and row;
+//     the class (phase, slice) of its column, all nonzeros of a short row to
+//     the last class.  The plan lays the nonzeros out class by class, each
+//     class in row order, as column (~compact-buffer row if the column is
+//     cached) and row arrays, plus the position of every stored nonzero in
+//     that order; every SpMM first scatters the caller's values into the same
+//     order (reading them in place would fetch each line of the value array
+//     once per class: 3.7 GB instead of 0.46 GB on the social graph);
 //   * inside a class the work is cut into fixed-length segments exactly as in
 //     the segments strategy; a (row, class) run that lies inside one segment is
-//     stored to a per-class partial-result buffer, runs that cross a segment
-//     boundary go through the carry slots;
+//     stored to the row's partial-result slot of the class, runs that cross a
+//     segment boundary go through the carry slots;
 //   * a final kernel adds, for every row, its class partials in class order
 //     and writes C (zeros for empty rows).  No atomics; results are
 //     bit-reproducible for a given plan.
@@ -38,62 +43,82 @@
 
 namespace hpspmm {
 
-constexpr int kHubClasses = 8;             // one per XCD
-constexpr int kClasses = kHubClasses + 1;  // + the cold class
-constexpr int kColdClass = kHubClasses;
+constexpr int kSlices = 8;                          // column slices, one per XCD
+constexpr int kMaxSub = 7;                          // sub-slices (phases) per slice, at most
+constexpr int kMaxClasses = kSlices * kMaxSub + 1;  // + the class of the short rows; fits one wavefront's lanes
 
 // What the final kernel does with a row.
 constexpr uint8_t kActionNone = 0;    // the main kernel stored the row to C itself
 constexpr uint8_t kActionZero = 1;    // no nonzeros: write zeros
 constexpr uint8_t kActionReduce = 2;  // add the class results
 
+// Class x < 8 * nsub is (phase x / 8, slice x % 8); class 8 * nsub holds the short rows.
 struct RoutedLayout {
-  int64_t cls_begin[kClasses];   // first virtual index of the class (multiple of the workgroup quantum)
-  int64_t cls_end[kClasses];     // one past its last real entry
-  int64_t cls_blocks[kClasses];  // workgroups needed by the class
-  int64_t hub_grid;              // 8 * max(cls_blocks[0..7]): hub workgroups are interleaved by class
+  int64_t cls_begin[kMaxClasses];    // first virtual index of the class (multiple of the workgroup quantum)
+  int64_t cls_end[kMaxClasses];      // one past its last real entry
+  int64_t cls_blocks[kMaxClasses];   // workgroups needed by the class
+  int64_t phase_begin[kMaxSub + 1];  // first workgroup of phase p (a multiple of 8); [nsub]: of the short-row class
   int64_t rows;
-  int shift;                     // log2(segment length)
+  int shift;  // log2(segment length)
+  int nsub;   // phases
+  int ncls;   // 8 * nsub + 1
 };
 
 // ---- plan-time kernels -----------------------------------------------------
 
 // Class of a nonzero in column c: mapped = colmap[c] is the compact-buffer row
-// of a cached column (slice = row / hub_rows_per_class) or -1, in which case
-// a multiplicative hash of c picks the slice; rows shorter than the routing
-// threshold send everything to class 8.
-__device__ __forceinline__ int class_of(int32_t c, int32_t mapped, int32_t hub_rows_per_class, bool routed_row) {
-  if (!routed_row) return kColdClass;
-  return mapped >= 0 ? mapped / hub_rows_per_class : (int)(((uint32_t)c * 0x9E3779B1u) >> 29);
+// of a cached column or -1.  A cached column of popularity rank s sits in
+// compact-buffer row (s % 8) * hub_rows_per_slice + s / 8 and belongs to slice
+// s % 8, phase (s / 8) % nsub, so that every (slice, phase) gets the same mix
+// of hot and cold columns; the other columns are spread by a multiplicative
+// hash.  Rows shorter than the routing threshold send everything to the last
+// class.
+__device__ __forceinline__ int class_of(int32_t c, int32_t mapped, int32_t hub_rows_per_slice, int nsub,
+                                        bool routed_row) {
+  if (!routed_row) return kSlices * nsub;
+  int slice, sub;
+  if (mapped >= 0) {
+    slice = mapped / hub_rows_per_slice;
+    sub = (mapped - slice * hub_rows_per_slice) % nsub;
+  } else {
+    const uint32_t h = (uint32_t)c * 0x9E3779B1u;
+    slice = (int)(h >> 29);
+    sub = (int)((((h >> 13) & 0xFFFFu) * (uint32_t)nsub) >> 16);
+  }
+  return sub * kSlices + slice;
 }
 
 // cnt[x * rows + r] = number of nonzeros of row r in class x.  One wavefront per row.
 __global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                               const int32_t* __restrict__ col,
                                                               const int32_t* __restrict__ colmap,
-                                                              int32_t hub_rows_per_class, int32_t min_row_nnz,
-                                                              uint32_t* __restrict__ cnt) {
+                                                              int32_t hub_rows_per_slice, int nsub,
+                                                              int32_t min_row_nnz, uint32_t* __restrict__ cnt) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   if (row >= rows) return;
+  const int ncls = kSlices * nsub + 1;
   const int32_t lb = rowptr[row];
   const int32_t hb = rowptr[row + 1];
   const bool routed_row = hb - lb >= min_row_nnz;
-  uint32_t mine = 0;  // lane x < kClasses accumulates the count of class x
-  for (int32_t j0 = lb; j0 < hb; j0 += 64) {
-    const int32_t j = j0 + lane;
-    int cls = -1;
-    if (j < hb) {
-      const int32_t c = col[j];
-      cls = class_of(c, colmap[c], hub_rows_per_class, routed_row);
-    }
-#pragma unroll
-    for (int x = 0; x < kClasses; ++x) {
-      const uint64_t m = __ballot(cls == x);
-      if (lane == x) mine += (uint32_t)__popcll(m);
+  uint32_t mine = 0;  // lane x < ncls accumulates the count of class x
+  if (!routed_row) {
+    if (lane == ncls - 1) mine = (uint32_t)(hb - lb);
+  } else {
+    for (int32_t j0 = lb; j0 < hb; j0 += 64) {
+      const int32_t j = j0 + lane;
+      int cls = -1;
+      if (j < hb) {
+        const int32_t c = col[j];
+        cls = class_of(c, colmap[c], hub_rows_per_slice, nsub, true);
+      }
+      for (int x = 0; x < ncls - 1; ++x) {
+        const uint64_t m = __ballot(cls == x);
+        if (lane == x) mine += (uint32_t)__popcll(m);
+      }
     }
   }
-  if (lane < kClasses) cnt[(int64_t)lane * rows + row] = mine;
+  if (lane < ncls) cnt[(int64_t)lane * rows + row] = mine;
 }
 
 // Three-pass exclusive scan of uint32 (n up to 2^32, total < 2^32).
@@ -171,16 +196,16 @@ __global__ __launch_bounds__(kBlock) void scan_apply_kernel(int64_t n, const uin
   }
 }
 
-// vptr[x * (rows + 1) + r] = virtual index of the first class-x nonzero of row r
+// vptr[r * ncls + x] = virtual index of the first class-x nonzero of row r
 // (r = rows: one past the class), from the exclusive scan of the class-major
-// counts and the padded class origins.
+// counts and the padded class origins.  The end of the (r, x) run is
+// vptr[(r + 1) * ncls + x].
 __global__ __launch_bounds__(kBlock) void routed_vptr_kernel(RoutedLayout lay, const uint32_t* __restrict__ scanned,
                                                              int32_t* __restrict__ vptr) {
-  const int64_t per = lay.rows + 1;
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (i >= per * kClasses) return;
-  const int x = (int)(i / per);
-  const int64_t r = i - (int64_t)x * per;
+  if (i >= (lay.rows + 1) * lay.ncls) return;
+  const int64_t r = i / lay.ncls;
+  const int x = (int)(i - r * lay.ncls);
   const int64_t first = scanned[(int64_t)x * lay.rows];
   const int64_t local = r < lay.rows ? (int64_t)scanned[(int64_t)x * lay.rows + r] - first
                                      : lay.cls_end[x] - lay.cls_begin[x];
@@ -192,24 +217,25 @@ __global__ __launch_bounds__(kBlock) void routed_vptr_kernel(RoutedLayout lay, c
 __global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                              const int32_t* __restrict__ col,
                                                              const int32_t* __restrict__ colmap,
-                                                             int32_t hub_rows_per_class, int32_t min_row_nnz,
-                                                             const int32_t* __restrict__ vptr,
-                                                             int32_t* __restrict__ vcol, int32_t* __restrict__ vsrc,
+                                                             int32_t hub_rows_per_slice, int nsub,
+                                                             int32_t min_row_nnz, const int32_t* __restrict__ vptr,
+                                                             int32_t* __restrict__ vcol, int32_t* __restrict__ vpos,
                                                              int32_t* __restrict__ vrow,
                                                              uint8_t* __restrict__ action, int shift) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   if (row >= rows) return;
+  const int ncls = kSlices * nsub + 1;
   const int32_t lb = rowptr[row];
   const int32_t hb = rowptr[row + 1];
   const bool routed_row = hb - lb >= min_row_nnz;
-  int32_t cursor = lane < kClasses ? vptr[(int64_t)lane * (rows + 1) + row] : 0;  // lane x: next slot of class x
-  const int32_t cls_last = lane < kClasses ? vptr[(int64_t)lane * (rows + 1) + row + 1] : 0;
+  int32_t cursor = lane < ncls ? vptr[row * ncls + lane] : 0;  // lane x: next slot of class x
+  const int32_t cls_last = lane < ncls ? vptr[(row + 1) * ncls + lane] : 0;
   const uint64_t below = (1ull << lane) - 1ull;
-  // A row without hub-class entries is "direct": its cold run is stored straight to
-  // C (flagged by the sign bit of vrow) unless it crosses a segment boundary.
-  const bool direct = __ballot(lane < kHubClasses && cls_last > cursor) == 0;
-  if (lane == kColdClass) {
+  // A row without entries outside the last class is "direct": its run is stored
+  // straight to C (flagged by the sign bit of vrow) unless it crosses a segment boundary.
+  const bool direct = __ballot(lane < ncls - 1 && cls_last > cursor) == 0;
+  if (lane == ncls - 1) {
     uint8_t a = kActionReduce;
     if (direct) {
       if (cls_last == cursor) a = kActionZero;
@@ -218,20 +244,33 @@ __global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const
     action[row] = a;
   }
   const int32_t row_tag = direct ? (int32_t)((uint32_t)row | 0x80000000u) : (int32_t)row;
+  if (!routed_row) {
+    // everything goes to the last class, in stored order
+    const int32_t start = __shfl(cursor, ncls - 1);
+    for (int32_t j = lb + lane; j < hb; j += 64) {
+      const int32_t c = col[j];
+      const int32_t mapped = colmap[c];
+      const int32_t pos = start + (j - lb);
+      vcol[pos] = mapped >= 0 ? ~mapped : c;
+      vpos[j] = pos;
+      vrow[pos] = row_tag;
+    }
+    return;
+  }
   for (int32_t j0 = lb; j0 < hb; j0 += 64) {
     const int32_t j = j0 + lane;
     const bool valid = j < hb;
     const int32_t c = valid ? col[j] : 0;
     const int32_t mapped = valid ? colmap[c] : -1;
-    const int cls = valid ? class_of(c, mapped, hub_rows_per_class, routed_row) : -1;
-#pragma unroll
-    for (int x = 0; x < kClasses; ++x) {
+    const int cls = valid ? class_of(c, mapped, hub_rows_per_slice, nsub, true) : -1;
+    for (int x = 0; x < ncls - 1; ++x) {
       const uint64_t m = __ballot(cls == x);
+      if (m == 0) continue;
       const int32_t start = __shfl(cursor, x);
       if (cls == x) {
         const int32_t pos = start + (int32_t)__popcll(m & below);
         vcol[pos] = mapped >= 0 ? ~mapped : c;  // ~compact-buffer row if the column is cached
-        vsrc[pos] = j;
+        vpos[j] = pos;
         vrow[pos] = row_tag;
       }
       if (lane == x) cursor += (int32_t)__popcll(m);
@@ -239,35 +278,59 @@ __global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const
   }
 }
 
-// Bhot[s, :] = B[src[s], :] for every compact-buffer row with a source column (src[s] >= 0).
+// Start of every SpMM, two jobs in one launch.  Workgroups [0, gather_blocks):
+// Bhot[s, :] = B[src[s], :] for every compact-buffer row with a source column
+// (src[s] >= 0).  The others: vval[vpos[j]] = val[j], the caller's values
+// brought into the plan's class-major order by a scatter in stored order (a
+// gather in class order would fetch every line of val once per class).
 template <int K>
-__global__ __launch_bounds__(kBlock) void routed_gather_hub_kernel(int64_t n, const int32_t* __restrict__ src,
-                                                                   const float* __restrict__ B,
-                                                                   float* __restrict__ Bhot) {
+__global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, int64_t gather_blocks,
+                                                                const int32_t* __restrict__ src,
+                                                                const float* __restrict__ B,
+                                                                float* __restrict__ Bhot, int64_t nnz,
+                                                                const float* __restrict__ val,
+                                                                const int32_t* __restrict__ vpos,
+                                                                float* __restrict__ vval, bool val_vec_ok) {
   constexpr int G = K / 4;
-  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int64_t s = t / G;
-  const int l = (int)(t % G);
-  if (s >= n) return;
-  const int32_t c = src[s];
-  if (c < 0) return;
-  *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) = load_b<K>(B, c, l);
+  if ((int64_t)blockIdx.x < gather_blocks) {
+    const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t s = t / G;
+    const int l = (int)(t % G);
+    if (s >= n_bhot) return;
+    const int32_t c = src[s];
+    if (c < 0) return;
+    *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) = load_b<K>(B, c, l);
+    return;
+  }
+  const int64_t j = (((int64_t)blockIdx.x - gather_blocks) * kBlock + threadIdx.x) * 4;
+  if (j >= nnz) return;
+  if (val_vec_ok && j + 4 <= nnz) {
+    const int4 q = *reinterpret_cast<const int4*>(vpos + j);
+    const float4 v = *reinterpret_cast<const float4*>(val + j);
+    vval[q.x] = v.x;
+    vval[q.y] = v.y;
+    vval[q.z] = v.z;
+    vval[q.w] = v.w;
+  } else {
+    for (int64_t i = j; i < j + 4 && i < nnz; ++i) vval[vpos[i]] = val[i];
+  }
 }
 
 // ---- SpMM kernels ----------------------------------------------------------
 
-// Workgroups [0, hub_grid): workgroup b serves column class b % 8 (and runs on
-// XCD b % 8), its b / 8-th workgroup.  Workgroups [hub_grid, ...): class 8, the
-// short rows.
+// Workgroups [phase_begin[p], phase_begin[p + 1]): phase p; its workgroup number
+// i serves class (p, i % 8) - and runs on XCD i % 8 - as that class's i / 8-th
+// workgroup.  Workgroups from phase_begin[nsub] on: the short rows.  The
+// hardware starts workgroups in index order, so every XCD works through its
+// slice one phase, i.e. one L2-sized set of B rows, at a time.
 // Each sub-wave owns one segment of its class; see the carry rule of the
-// segments kernel - here "stored to C" becomes "stored to the class's
-// partial-result buffer".
+// segments kernel - here "stored to C" becomes "stored to the row's
+// partial-result slot of the class".
 template <int K>
 __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, const int32_t* __restrict__ vptr,
                                                              const int32_t* __restrict__ vcol,
-                                                             const int32_t* __restrict__ vsrc,
+                                                             const float* __restrict__ vval,
                                                              const int32_t* __restrict__ vrow,
-                                                             const float* __restrict__ val,
                                                              const float* __restrict__ B,
                                                              const float* __restrict__ Bhot,
                                                              float* __restrict__ partial,
@@ -279,14 +342,18 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
   __shared__ __attribute__((aligned(16))) float s_val[kWavesPerBlock * P * kTileStride];
   __shared__ __attribute__((aligned(16))) int32_t s_row[kWavesPerBlock * P * kTileStride];
 
+  const int ncls = lay.ncls;
+  int p = 0;
+  while (p < lay.nsub && (int64_t)blockIdx.x >= lay.phase_begin[p + 1]) ++p;
+  const int64_t rel = (int64_t)blockIdx.x - lay.phase_begin[p];
   int x;
   int64_t i;
-  if ((int64_t)blockIdx.x < lay.hub_grid) {
-    x = (int)(blockIdx.x % kHubClasses);
-    i = blockIdx.x / kHubClasses;
+  if (p < lay.nsub) {
+    x = p * kSlices + (int)(rel % kSlices);
+    i = rel / kSlices;
   } else {
-    x = kColdClass;
-    i = (int64_t)blockIdx.x - lay.hub_grid;
+    x = ncls - 1;
+    i = rel;
   }
   if (i >= lay.cls_blocks[x]) return;
 
@@ -300,54 +367,43 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
   if (s >= cls_end) return;
   const int64_t e = (s + ((int64_t)1 << shift)) < cls_end ? (s + ((int64_t)1 << shift)) : cls_end;
   const int sbase = ((tid >> 6) * P + lane / G) * kTileStride;
-  const int32_t* vp = vptr + (int64_t)x * (lay.rows + 1);
-  float* pout = partial + (uint64_t)x * (uint64_t)lay.rows * K;
+  const int32_t* vp = vptr + x;
+  float* pout = partial + (uint64_t)x * K;
 
   // the sign bit of a row entry marks a row that is stored straight to C
   int32_t cur = vrow[s];
-  bool head_pending = (int64_t)vp[cur & 0x7FFFFFFF] < s;
+  bool head_pending = (int64_t)vp[(int64_t)(cur & 0x7FFFFFFF) * ncls] < s;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 
   auto flush_to = [&](bool is_tail) {
     const uint32_t row = (uint32_t)cur & 0x7FFFFFFFu;
     float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
                               : (is_tail ? carry + (uint64_t)(2 * g + 1) * K
-                                         : (cur < 0 ? C + (uint64_t)row * K : pout + (uint64_t)row * K));
+                                         : (cur < 0 ? C + (uint64_t)row * K : pout + (uint64_t)row * ncls * K));
     head_pending = false;
     *reinterpret_cast<float4*>(dst + 4 * l) = acc;
   };
   auto flush = [&]() { flush_to(false); };
   auto loadb = [&](int32_t c) { return load_b_hub<K, true>(B, Bhot, c, l); };
 
-  // Two-deep prefetch: the source indices of tile t+2 and, through the indices
-  // fetched one iteration earlier, the values of tile t+1 (the plan's arrays
-  // are allocated by the library, hence always aligned for the vector loads).
+  // the plan's arrays are allocated by the library, hence always aligned for the vector loads
+  auto fetch = [&](TileRegs<TL>& m, int64_t t) {
+    const int64_t q = t + l * TL;
+    load_run<TL>(m.c, vcol, q, e, true);
+    load_run<TL>(m.v, vval, q, e, true);
+    load_run<TL>(m.r, vrow, q, e, true);
+  };
   TileRegs<TL> m;
-  int32_t src[TL];
-  const int64_t q0 = s + l * TL;
-  load_run<TL>(src, vsrc, q0, e, true);
-  load_run<TL>(m.c, vcol, q0, e, true);
-  load_run<TL>(m.r, vrow, q0, e, true);
-#pragma unroll
-  for (int j = 0; j < TL; ++j) m.v[j] = q0 + j < e ? val[src[j]] : 0.f;
-  if (s + kTile < e) load_run<TL>(src, vsrc, q0 + kTile, e, true);
-
+  fetch(m, s);
   for (int64_t t = s; t < e; t += kTile) {
     stage_tile<TL>(m, sbase + l * TL, s_col, s_val, s_row);
     wave_lds_fence();
-    if (t + kTile < e) {
-      const int64_t q = t + kTile + l * TL;
-      load_run<TL>(m.c, vcol, q, e, true);
-      load_run<TL>(m.r, vrow, q, e, true);
-#pragma unroll
-      for (int j = 0; j < TL; ++j) m.v[j] = q + j < e ? val[src[j]] : 0.f;
-      if (t + 2 * kTile < e) load_run<TL>(src, vsrc, q + kTile, e, true);
-    }
+    if (t + kTile < e) fetch(m, t + kTile);
     const int cnt = (e - t) < kTile ? (int)(e - t) : kTile;
     consume_tile(cnt, sbase, s_col, s_val, s_row, cur, acc, loadb, flush);
     wave_lds_fence();
   }
-  flush_to((int64_t)vp[(cur & 0x7FFFFFFF) + 1] > e);
+  flush_to((int64_t)vp[(int64_t)((cur & 0x7FFFFFFF) + 1) * ncls] > e);
 }
 
 // list[] <- every row whose action byte equals `which` (order unspecified); *count must be zero on entry.
@@ -366,10 +422,10 @@ __global__ __launch_bounds__(kBlock) void routed_collect_rows_kernel(int64_t row
 }
 
 // Final pass, one sub-wave per listed row.  Workgroups [0, reduce_blocks): rows
-// whose class results must be added - in class order, the partial-buffer row if
-// the (row, class) run lies in one segment, else tail[ga] + head[ga+1] + ... +
-// head[gb] from the carry slots.  Remaining workgroups: rows without nonzeros,
-// which get zeros.  Rows in neither list were stored by the main kernel.
+// whose class results must be added - in class order, the row's partial-result
+// slot if the (row, class) run lies in one segment, else tail[ga] + head[ga+1]
+// + ... + head[gb] from the carry slots.  Remaining workgroups: rows without
+// nonzeros, which get zeros.  Rows in neither list were stored by the main kernel.
 // (Lists rather than a scan over all rows: on R-MAT the rows that need a
 // reduction sit together at low indices and serialised inside a few waves.)
 template <int K>
@@ -384,10 +440,12 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout 
                                                                    float* __restrict__ C) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
+  constexpr int kGroup = 8;  // classes whose loads are in flight together
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
   const int shift = lay.shift;
+  const int ncls = lay.ncls;
   if ((int64_t)blockIdx.x >= reduce_blocks) {
     const int64_t idx = (((int64_t)blockIdx.x - reduce_blocks) * kWavesPerBlock + (tid >> 6)) * P + lane / G;
     if (idx >= n_zero) return;
@@ -397,26 +455,10 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout 
   const int64_t idx = ((int64_t)blockIdx.x * kWavesPerBlock + (tid >> 6)) * P + lane / G;
   if (idx >= n_reduce) return;
   const int64_t row = reduce_rows[idx];
+  const int32_t* vlo = vptr + row * ncls;
+  const int32_t* vhi = vlo + ncls;
+  const float* prow = partial + (uint64_t)row * ncls * K + 4 * l;
 
-  // all class bounds first, then all single-segment partials, so that the loads
-  // of a row are in flight together; the adds stay in class order
-  int64_t lb[kClasses], hb[kClasses];
-#pragma unroll
-  for (int x = 0; x < kClasses; ++x) {
-    const int32_t* vp = vptr + (int64_t)x * (lay.rows + 1);
-    lb[x] = vp[row];
-    hb[x] = vp[row + 1];
-  }
-  float4 part[kClasses];
-  bool single[kClasses];
-#pragma unroll
-  for (int x = 0; x < kClasses; ++x) {
-    single[x] = lb[x] != hb[x] && (lb[x] >> shift) == ((hb[x] - 1) >> shift);
-    part[x] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (single[x])
-      part[x] =
-          *reinterpret_cast<const float4*>(partial + ((uint64_t)x * (uint64_t)lay.rows + (uint64_t)row) * K + 4 * l);
-  }
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   auto add = [&](const float4& t) {
     acc.x += t.x;
@@ -424,24 +466,54 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout 
     acc.z += t.z;
     acc.w += t.w;
   };
+  for (int x0 = 0; x0 < ncls; x0 += kGroup) {
+    // all bounds of the group first, then all single-segment partials, so that
+    // the loads are in flight together; the adds stay in class order
+    int32_t lb[kGroup], hb[kGroup];
 #pragma unroll
-  for (int x = 0; x < kClasses; ++x) {
-    if (lb[x] == hb[x]) continue;
-    if (single[x]) {
-      add(part[x]);
-    } else {
+    for (int q = 0; q < kGroup; ++q) {
+      const bool in = x0 + q < ncls;
+      const int x = in ? x0 + q : ncls - 1;
+      lb[q] = vlo[x];
+      hb[q] = in ? vhi[x] : lb[q];
+    }
+    float4 part[kGroup];
+    bool split = false;  // some run of the group crosses a segment boundary
+#pragma unroll
+    for (int q = 0; q < kGroup; ++q) {
+      const bool some = lb[q] != hb[q];
+      const bool single = some && (lb[q] >> shift) == ((hb[q] - 1) >> shift);
+      split |= some && !single;
+      part[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (single) part[q] = *reinterpret_cast<const float4*>(prow + (uint64_t)(x0 + q) * K);
+    }
+    if (!split) {
+#pragma unroll
+      for (int q = 0; q < kGroup; ++q)
+        if (lb[q] != hb[q]) add(part[q]);
+      continue;
+    }
+    // rare: walk the group again class by class (bounds and partials come from the caches)
+#pragma unroll 1
+    for (int x = x0; x < x0 + kGroup && x < ncls; ++x) {
+      const int32_t lo = vlo[x], hi = vhi[x];
+      if (lo == hi) continue;
+      const int64_t ga = lo >> shift;
+      const int64_t gb = (hi - 1) >> shift;
+      if (ga == gb) {
+        add(*reinterpret_cast<const float4*>(prow + (uint64_t)x * K));
+        continue;
+      }
       // a hub row spans hundreds of segments: fetch the carry slots 8 at a time, add them in segment order
-      const int64_t ga = lb[x] >> shift;
-      const int64_t gb = (hb[x] - 1) >> shift;
       add(*reinterpret_cast<const float4*>(carry + (uint64_t)(2 * ga + 1) * K + 4 * l));
       int64_t g = ga + 1;
       for (; g + kBatch <= gb + 1; g += kBatch) {
         float4 slot[kBatch];
 #pragma unroll
-        for (int q = 0; q < kBatch; ++q)
-          slot[q] = *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * (g + q)) * K + 4 * l);
+        for (int t = 0; t < kBatch; ++t)
+          slot[t] = *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * (g + t)) * K + 4 * l);
 #pragma unroll
-        for (int q = 0; q < kBatch; ++q) add(slot[q]);
+        for (int t = 0; t < kBatch; ++t) add(slot[t]);
       }
       for (; g <= gb; ++g) add(*reinterpret_cast<const float4*>(carry + (uint64_t)(2 * g) * K + 4 * l));
     }

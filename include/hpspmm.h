@@ -62,6 +62,8 @@ typedef enum hpspmm_status {
 #define HPSPMM_PLAN_NO_ROUTED 128u    /* never use the routed strategy */
 /* bits 24..28, with FORCE_ROUTED: log2 of the shortest row that is routed (0 = default, 128) */
 #define HPSPMM_PLAN_ROUTED_ROW_LOG2(log2_nnz) (((uint32_t)(log2_nnz) & 0x1Fu) << 24)
+/* bits 29..31, with FORCE_ROUTED: number of phases every XCD cuts its slice of the columns into, 1..7 (0 = auto) */
+#define HPSPMM_PLAN_ROUTED_PHASES(n) (((uint32_t)(n) & 0x7u) << 29)
 /* bits 16..23: log2 of the number of cached rows (0 = default, 2^16) */
 #define HPSPMM_PLAN_HUB_LOG2(log2_rows) (((uint32_t)(log2_rows) & 0xFFu) << 16)
 /* bits 8..15: log2 of the segment length to force (0 = choose automatically) */

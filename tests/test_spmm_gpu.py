@@ -58,7 +58,10 @@ def _strategies(capi):
             ("routed_tiny", capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(3) | capi.plan_segment_shift(3)
              | capi.plan_routed_row_log2(1)),
             ("routed_s16", capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(10) | capi.plan_segment_shift(4)
-             | capi.plan_routed_row_log2(3))]
+             | capi.plan_routed_row_log2(3)),
+            ("routed_3phases", capi.PLAN_FORCE_ROUTED | capi.plan_routed_phases(3) | capi.plan_routed_row_log2(4)),
+            ("routed_7phases_tiny", capi.PLAN_FORCE_ROUTED | capi.plan_routed_phases(7) | capi.plan_hub_log2(5)
+             | capi.plan_segment_shift(3) | capi.plan_routed_row_log2(1))]
 
 
 @pytest.mark.parametrize("k", [32, 64, 128])
@@ -401,3 +404,28 @@ def test_non_finite_values_stay_in_their_rows(pkg, oracle, gpu):
             finite_rows = np.isfinite(C).all(axis=1)
             assert finite_rows[~touched].all(), f"k={k} {name}: non-finite value leaked into an unrelated row"
             assert (~finite_rows[touched]).all(), f"k={k} {name}: a referencing row lost the non-finite value"
+
+
+def test_unaligned_arrays_and_new_values_per_call(pkg, oracle, gpu):
+    """Caller arrays that are only 4-byte aligned (views one element into a buffer), and a plan reused
+    with different values: the plan holds structure only, so the second call must see the new values."""
+    import torch
+    capi = pkg.capi
+    g = pkg.graphs.make_graph("c4_rmat", 0.004)
+    for k in (32, 128):
+        B = pkg.graphs.make_dense("c4_rmat", g.cols, k)
+        Bd, = _to_dev(gpu, B)
+        pad = lambda a: torch.from_numpy(np.concatenate([np.zeros(1, a.dtype), a])).to(gpu)[1:]
+        rp, ci, v = pad(g.rowptr), pad(g.col), pad(g.val)
+        assert v.data_ptr() % 16 == 4
+        val2 = (g.val * np.float32(-0.5) + np.float32(0.25)).astype(np.float32)
+        v2 = pad(val2)
+        g2 = pkg.graphs.CSR(g.rows, g.cols, g.rowptr, g.col, val2)
+        for name, flags in _strategies(capi):
+            plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
+            C = torch.full((g.rows, k), float("nan"), device=gpu)
+            capi.csr_spmm(plan, rp, ci, v, Bd, C)
+            _check(oracle, g, B, C.cpu().numpy(), f"unaligned k={k} {name}")
+            capi.csr_spmm(plan, rp, ci, v2, Bd, C)
+            _check(oracle, g2, B, C.cpu().numpy(), f"unaligned, new values k={k} {name}")
+            plan.destroy()

@@ -441,7 +441,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
 template <int K>
 int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
   const int64_t gather_blocks = ceil_div(p->n_bhot * (K / 4), hpspmm::kBlock);
-  const int64_t prep_blocks = gather_blocks + ceil_div(ceil_div(p->nnz, 4), hpspmm::kBlock);
+  const int64_t prep_blocks = gather_blocks + ceil_div(p->nnz, hpspmm::kBlock * hpspmm::kPermutePerThread);
   if (prep_blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   hipLaunchKernelGGL(hpspmm::routed_prepare_kernel<K>, dim3((unsigned)prep_blocks), dim3(hpspmm::kBlock), 0, st,
                      p->n_bhot, gather_blocks, p->d_bhot_src, B, p->d_bhot, p->nnz, v, p->d_vpos, p->d_vval,

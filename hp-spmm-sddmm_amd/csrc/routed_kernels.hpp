@@ -283,6 +283,8 @@ __global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const
 // (src[s] >= 0).  The others: vval[vpos[j]] = val[j], the caller's values
 // brought into the plan's class-major order by a scatter in stored order (a
 // gather in class order would fetch every line of val once per class).
+constexpr int kPermutePerThread = 4;
+
 template <int K>
 __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, int64_t gather_blocks,
                                                                 const int32_t* __restrict__ src,
@@ -302,7 +304,9 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
     *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) = load_b<K>(B, c, l);
     return;
   }
-  const int64_t j = (((int64_t)blockIdx.x - gather_blocks) * kBlock + threadIdx.x) * 4;
+  // four consecutive nonzeros per thread (measured against one instruction per
+  // 64 consecutive nonzeros of a wavefront: 0.28 vs 0.31 ms on the social graph)
+  const int64_t j = (((int64_t)blockIdx.x - gather_blocks) * kBlock + threadIdx.x) * kPermutePerThread;
   if (j >= nnz) return;
   if (val_vec_ok && j + 4 <= nnz) {
     const int4 q = *reinterpret_cast<const int4*>(vpos + j);
@@ -428,6 +432,12 @@ __global__ __launch_bounds__(kBlock) void routed_collect_rows_kernel(int64_t row
 // nonzeros, which get zeros.  Rows in neither list were stored by the main kernel.
 // (Lists rather than a scan over all rows: on R-MAT the rows that need a
 // reduction sit together at low indices and serialised inside a few waves.)
+//
+// With segments of 512 nonzeros and runs of some tens, about one run in eight
+// crosses a segment boundary, i.e. most rows have one: the first two slots of
+// every run (partial or tail, then the next head) are therefore fetched
+// together for a group of classes, and only a run over three or more segments
+// (a hub row) takes the loop over the remaining heads.
 template <int K>
 __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout lay,
                                                                    const int32_t* __restrict__ vptr,
@@ -440,7 +450,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout 
                                                                    float* __restrict__ C) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
-  constexpr int kGroup = 8;  // classes whose loads are in flight together
+  constexpr int kGroup = 4;  // classes whose loads are in flight together
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
@@ -458,6 +468,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout 
   const int32_t* vlo = vptr + row * ncls;
   const int32_t* vhi = vlo + ncls;
   const float* prow = partial + (uint64_t)row * ncls * K + 4 * l;
+  const float* cbase = carry + 4 * l;
 
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   auto add = [&](const float4& t) {
@@ -466,10 +477,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout 
     acc.z += t.z;
     acc.w += t.w;
   };
-  for (int x0 = 0; x0 < ncls; x0 += kGroup) {
-    // all bounds of the group first, then all single-segment partials, so that
-    // the loads are in flight together; the adds stay in class order
-    int32_t lb[kGroup], hb[kGroup];
+  auto bounds = [&](int x0, int32_t (&lb)[kGroup], int32_t (&hb)[kGroup]) {
 #pragma unroll
     for (int q = 0; q < kGroup; ++q) {
       const bool in = x0 + q < ncls;
@@ -477,45 +485,55 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout 
       lb[q] = vlo[x];
       hb[q] = in ? vhi[x] : lb[q];
     }
-    float4 part[kGroup];
-    bool split = false;  // some run of the group crosses a segment boundary
+  };
+  int32_t nlb[kGroup], nhb[kGroup];
+  bounds(0, nlb, nhb);
+  for (int x0 = 0; x0 < ncls; x0 += kGroup) {
+    int32_t lb[kGroup], hb[kGroup];
+    float4 first[kGroup], second[kGroup];
+    bool some[kGroup], two[kGroup];
+    bool longer = false;  // some run of the group covers three or more segments
 #pragma unroll
     for (int q = 0; q < kGroup; ++q) {
-      const bool some = lb[q] != hb[q];
-      const bool single = some && (lb[q] >> shift) == ((hb[q] - 1) >> shift);
-      split |= some && !single;
-      part[q] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (single) part[q] = *reinterpret_cast<const float4*>(prow + (uint64_t)(x0 + q) * K);
+      lb[q] = nlb[q];
+      hb[q] = nhb[q];
+      some[q] = lb[q] != hb[q];
+      const int64_t ga = lb[q] >> shift;
+      const int64_t gb = (hb[q] - 1) >> shift;
+      two[q] = some[q] && gb > ga;
+      longer |= some[q] && gb > ga + 1;
+      const float* pa = two[q] ? cbase + (uint64_t)(2 * ga + 1) * K : prow + (uint64_t)(x0 + q) * K;
+      first[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+      second[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (some[q]) first[q] = *reinterpret_cast<const float4*>(pa);
+      if (two[q]) second[q] = *reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * (ga + 1)) * K);
     }
-    if (!split) {
+    if (x0 + kGroup < ncls) bounds(x0 + kGroup, nlb, nhb);  // in flight together with the slots above
+    if (!longer) {
 #pragma unroll
-      for (int q = 0; q < kGroup; ++q)
-        if (lb[q] != hb[q]) add(part[q]);
+      for (int q = 0; q < kGroup; ++q) {
+        if (some[q]) add(first[q]);
+        if (two[q]) add(second[q]);
+      }
       continue;
     }
-    // rare: walk the group again class by class (bounds and partials come from the caches)
-#pragma unroll 1
-    for (int x = x0; x < x0 + kGroup && x < ncls; ++x) {
-      const int32_t lo = vlo[x], hi = vhi[x];
-      if (lo == hi) continue;
-      const int64_t ga = lo >> shift;
-      const int64_t gb = (hi - 1) >> shift;
-      if (ga == gb) {
-        add(*reinterpret_cast<const float4*>(prow + (uint64_t)x * K));
-        continue;
-      }
-      // a hub row spans hundreds of segments: fetch the carry slots 8 at a time, add them in segment order
-      add(*reinterpret_cast<const float4*>(carry + (uint64_t)(2 * ga + 1) * K + 4 * l));
-      int64_t g = ga + 1;
+#pragma unroll
+    for (int q = 0; q < kGroup; ++q) {
+      if (some[q]) add(first[q]);
+      if (!two[q]) continue;
+      add(second[q]);
+      // a hub row spans hundreds of segments: fetch the remaining heads 8 at a time, add them in segment order
+      const int64_t gb = (hb[q] - 1) >> shift;
+      int64_t g = (lb[q] >> shift) + 2;
       for (; g + kBatch <= gb + 1; g += kBatch) {
         float4 slot[kBatch];
 #pragma unroll
         for (int t = 0; t < kBatch; ++t)
-          slot[t] = *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * (g + t)) * K + 4 * l);
+          slot[t] = *reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * (g + t)) * K);
 #pragma unroll
         for (int t = 0; t < kBatch; ++t) add(slot[t]);
       }
-      for (; g <= gb; ++g) add(*reinterpret_cast<const float4*>(carry + (uint64_t)(2 * g) * K + 4 * l));
+      for (; g <= gb; ++g) add(*reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * g) * K));
     }
   }
   *reinterpret_cast<float4*>(C + (uint64_t)row * K + 4 * l) = acc;

@@ -82,17 +82,18 @@ struct hpspmm_plan {
   int64_t n_hub = 0;
   // routed strategy
   hpspmm::RoutedLayout lay{};
-  int32_t* d_vptr = nullptr;      // [(rows + 1) * ncls]
-  int32_t* d_vcol = nullptr;      // [vtotal] column, or compact-buffer row for hub classes
+  int32_t* d_rvptr = nullptr;     // [(n_routed + 1) * nhub] run starts of the routed rows in the hub classes
+  int32_t* d_coldptr = nullptr;   // [rows + 1] run starts in the cold class
+  int32_t* d_vcol = nullptr;      // [vtotal] column, or ~compact-buffer row
   int32_t* d_vpos = nullptr;      // [nnz] position of every stored nonzero in the class-major order
   float* d_vval = nullptr;        // [vtotal] the values in that order, rewritten by every SpMM
-  int32_t* d_vrow = nullptr;      // [vtotal]
+  int32_t* d_vrow = nullptr;      // [vtotal] routed-row number (hub classes) or row (cold class)
   int32_t* d_bhot_src = nullptr;  // [n_bhot] source column of every compact-buffer row (-1 = unused)
-  uint8_t* d_action = nullptr;    // [rows] what the final kernel does with each row
-  int32_t* d_reduce_rows = nullptr;  // rows whose class results must be added
+  int32_t* d_routed_rows = nullptr;  // [n_routed] row of every routed-row number
+  int32_t* d_cross_rows = nullptr;   // short rows whose run crosses a segment boundary
   int32_t* d_zero_rows = nullptr;    // rows without nonzeros
-  int64_t n_reduce = 0, n_zero = 0;
-  float* d_partial = nullptr;     // [rows * ncls * k]
+  int64_t n_cross = 0, n_zero = 0;
+  float* d_partial = nullptr;     // [n_routed * nhub * k]
   int64_t n_bhot = 0;
   int64_t routed_grid = 0;
   int32_t* d_long_rows = nullptr;  // rows strategy: rows longer than long_threshold
@@ -243,7 +244,7 @@ int rank_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t want, hipSt
   return HPSPMM_OK;
 }
 
-// Device exclusive scan of n uint32 values (three passes, tile sums in between).
+// Device exclusive scan of n uint32 values (three passes, tile sums in between); d_out may be d_in.
 int exclusive_scan_u32(const uint32_t* d_in, uint32_t* d_out, int64_t n, hipStream_t st) {
   const int64_t ntiles = ceil_div(n, hpspmm::kScanTile);
   if (ntiles > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "scan too large");
@@ -303,7 +304,6 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   int nsub = (int)std::min<int64_t>(2, std::max<int64_t>(1, ceil_div(slice_bytes, kRoutedPhaseBytes)));
   if (slice_bytes > kRoutedPhaseBytes * 4) nsub = 1;
   if (want_sub) nsub = std::min(want_sub, hpspmm::kMaxSub);
-  const int ncls = hpspmm::kSlices * nsub + 1;
 
   // popularity rank s -> slice s % 8, compact-buffer row (s % 8) * h + s / 8
   const int64_t n_bhot = h * hpspmm::kSlices;
@@ -314,44 +314,72 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
     bhot_src[(size_t)slot] = ids[s2];
   }
 
+  const int nhub = hpspmm::kSlices * nsub;
+  const int32_t min_row_nnz =
+      std::max<int32_t>(1, forced && log2_row_threshold ? (1 << log2_row_threshold) : kRoutedRowThreshold);
+
+  // temporaries of the layout construction
   int32_t* d_colmap = nullptr;
-  uint32_t* d_cnt = nullptr;
-  uint32_t* d_scan = nullptr;
+  uint32_t* d_ridx = nullptr;     // [rows + 1] routed flag, then (scanned in place) routed-row number
+  uint32_t* d_cnt = nullptr;      // [nhub * n_routed + 1] class-major counts, then their scan
+  uint32_t* d_coldcnt = nullptr;  // [rows + 1] cold-class count per row, then its scan
+  uint8_t* d_action = nullptr;    // [rows]
+  int32_t* d_counts = nullptr;    // [2] list lengths
   struct Guard {
-    void** q[3];
+    void** q[6];
     ~Guard() {
       for (void** x : q)
         if (*x) (void)hipFree(*x);
     }
-  } guard{{(void**)&d_colmap, (void**)&d_cnt, (void**)&d_scan}};
-  const int64_t ncnt = rows * ncls;
+  } guard{{(void**)&d_colmap, (void**)&d_ridx, (void**)&d_cnt, (void**)&d_coldcnt, (void**)&d_action,
+           (void**)&d_counts}};
   HPSPMM_HIP(hipMalloc(&d_colmap, (size_t)std::max<int64_t>(1, p->cols) * sizeof(int32_t)));
-  HPSPMM_HIP(hipMalloc(&d_cnt, (size_t)ncnt * sizeof(uint32_t)));
-  HPSPMM_HIP(hipMalloc(&d_scan, (size_t)ncnt * sizeof(uint32_t)));
+  HPSPMM_HIP(hipMalloc(&d_ridx, (size_t)(rows + 1) * sizeof(uint32_t)));
+  HPSPMM_HIP(hipMalloc(&d_coldcnt, (size_t)(rows + 1) * sizeof(uint32_t)));
+  HPSPMM_HIP(hipMalloc(&d_action, (size_t)rows));
+  HPSPMM_HIP(hipMalloc(&d_counts, 2 * sizeof(int32_t)));
   HPSPMM_HIP(hipMemcpyAsync(d_colmap, colmap.data(), colmap.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
+
+  // number the routed rows
+  hipLaunchKernelGGL(hpspmm::routed_flag_kernel, dim3((unsigned)ceil_div(rows + 1, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, min_row_nnz, d_ridx);
+  if (int rc = exclusive_scan_u32(d_ridx, d_ridx, rows + 1, st)) return rc;
+  uint32_t n_routed_u = 0;
+  HPSPMM_HIP(hipMemcpyAsync(&n_routed_u, d_ridx + rows, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  const int64_t n_routed = n_routed_u;
+
+  // per-row class counts and their scans
+  const int64_t ncnt = (int64_t)nhub * n_routed + 1;
+  HPSPMM_HIP(hipMalloc(&d_cnt, (size_t)ncnt * sizeof(uint32_t)));
   const unsigned row_grid = (unsigned)ceil_div(rows, hpspmm::kWavesPerBlock);
-  const int32_t min_row_nnz = forced && log2_row_threshold ? (1 << log2_row_threshold) : kRoutedRowThreshold;
-  hipLaunchKernelGGL(hpspmm::routed_count_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col,
-                     d_colmap, (int32_t)h, nsub, min_row_nnz, d_cnt);
-  if (int rc = exclusive_scan_u32(d_cnt, d_scan, ncnt, st)) return rc;
+  hipLaunchKernelGGL(hpspmm::routed_count_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, n_routed,
+                     d_rowptr, d_col, d_colmap, d_ridx, (int32_t)h, nsub, min_row_nnz, d_cnt, d_coldcnt);
+  if (int rc = exclusive_scan_u32(d_cnt, d_cnt, ncnt, st)) return rc;
+  if (int rc = exclusive_scan_u32(d_coldcnt, d_coldcnt, rows + 1, st)) return rc;
 
   // class sizes = differences of the scan at the class origins
-  uint32_t origin[hpspmm::kMaxClasses];
-  for (int x = 0; x < ncls; ++x)
-    HPSPMM_HIP(hipMemcpyAsync(&origin[x], d_scan + (int64_t)x * rows, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+  uint32_t origin[hpspmm::kMaxHub + 1];
+  for (int x = 0; x <= nhub; ++x)
+    HPSPMM_HIP(hipMemcpyAsync(&origin[x], d_cnt + (int64_t)x * n_routed, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+  uint32_t cold_total = 0;
+  HPSPMM_HIP(hipMemcpyAsync(&cold_total, d_coldcnt + rows, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
   HPSPMM_HIP(hipStreamSynchronize(st));
+  if ((int64_t)origin[nhub] + (int64_t)cold_total != nnz)
+    return fail(HPSPMM_ERR_HIP, "routed plan: class counts do not add up to nnz");
 
   hpspmm::RoutedLayout& lay = p->lay;
   lay = hpspmm::RoutedLayout{};
   lay.rows = rows;
+  lay.n_routed = n_routed;
   lay.shift = p->shift;
   lay.nsub = nsub;
-  lay.ncls = ncls;
+  lay.nhub = nhub;
   const int64_t subwaves = 64 / (k / 4);
   const int64_t quantum = ((int64_t)1 << p->shift) * subwaves * hpspmm::kWavesPerBlock;  // nonzeros per workgroup
   int64_t at = 0;
-  for (int x = 0; x < ncls; ++x) {
-    const int64_t n_x = (x + 1 < ncls ? (int64_t)origin[x + 1] : nnz) - (int64_t)origin[x];
+  for (int x = 0; x <= nhub; ++x) {
+    const int64_t n_x = x < nhub ? (int64_t)origin[x + 1] - (int64_t)origin[x] : (int64_t)cold_total;
     lay.cls_begin[x] = at;
     lay.cls_end[x] = at + n_x;
     lay.cls_blocks[x] = ceil_div(n_x, quantum);
@@ -367,70 +395,62 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
     grid += most * hpspmm::kSlices;
   }
   lay.phase_begin[nsub] = grid;
-  p->routed_grid = grid + lay.cls_blocks[ncls - 1];
+  p->routed_grid = grid + lay.cls_blocks[nhub];
   if (vtotal >= INT32_MAX || p->routed_grid > INT32_MAX) return HPSPMM_OK;
 
   const int64_t nseg = vtotal >> p->shift;
-  const size_t vptr_bytes = (size_t)ncls * (size_t)(rows + 1) * sizeof(int32_t);
+  const size_t rvptr_bytes = (size_t)(n_routed + 1) * (size_t)nhub * sizeof(int32_t);
+  const size_t coldptr_bytes = (size_t)(rows + 1) * sizeof(int32_t);
   const size_t v_bytes = (size_t)vtotal * sizeof(int32_t);
-  const size_t partial_bytes = (size_t)ncls * (size_t)rows * (size_t)k * sizeof(float);
+  const size_t vpos_bytes = (size_t)std::max<int64_t>(nnz, 1) * sizeof(int32_t);
+  const size_t partial_bytes = (size_t)std::max<int64_t>(n_routed, 1) * (size_t)nhub * (size_t)k * sizeof(float);
   const size_t carry_bytes = (size_t)std::max<int64_t>(nseg, 1) * 2 * (size_t)k * sizeof(float);
   const size_t bhot_bytes = (size_t)n_bhot * (size_t)k * sizeof(float);
+  const size_t list_bytes = (size_t)std::max<int64_t>(rows, 1) * sizeof(int32_t);
+  const size_t routed_rows_bytes = (size_t)std::max<int64_t>(n_routed, 1) * sizeof(int32_t);
   // the segments strategy's buffers are not needed any more
   if (p->d_nnz_row) { (void)hipFree(p->d_nnz_row); p->d_nnz_row = nullptr; }
   if (p->d_carry) { (void)hipFree(p->d_carry); p->d_carry = nullptr; }
-  if (hipMalloc(&p->d_vptr, vptr_bytes) != hipSuccess || hipMalloc(&p->d_vcol, v_bytes) != hipSuccess ||
-      hipMalloc(&p->d_vval, v_bytes) != hipSuccess || hipMalloc(&p->d_vrow, v_bytes) != hipSuccess ||
-      hipMalloc(&p->d_vpos, (size_t)std::max<int64_t>(nnz, 1) * sizeof(int32_t)) != hipSuccess ||
+  const size_t total_bytes = rvptr_bytes + coldptr_bytes + 3 * v_bytes + vpos_bytes + partial_bytes + carry_bytes +
+                             bhot_bytes + (size_t)n_bhot * 4 + 2 * list_bytes + routed_rows_bytes;
+  if (hipMalloc(&p->d_rvptr, rvptr_bytes) != hipSuccess || hipMalloc(&p->d_coldptr, coldptr_bytes) != hipSuccess ||
+      hipMalloc(&p->d_vcol, v_bytes) != hipSuccess || hipMalloc(&p->d_vval, v_bytes) != hipSuccess ||
+      hipMalloc(&p->d_vrow, v_bytes) != hipSuccess || hipMalloc(&p->d_vpos, vpos_bytes) != hipSuccess ||
       hipMalloc(&p->d_partial, partial_bytes) != hipSuccess || hipMalloc(&p->d_carry, carry_bytes) != hipSuccess ||
       hipMalloc(&p->d_bhot, bhot_bytes) != hipSuccess ||
       hipMalloc(&p->d_bhot_src, (size_t)n_bhot * sizeof(int32_t)) != hipSuccess ||
-      hipMalloc(&p->d_action, (size_t)rows) != hipSuccess) {
+      hipMalloc(&p->d_routed_rows, routed_rows_bytes) != hipSuccess ||
+      hipMalloc(&p->d_cross_rows, list_bytes) != hipSuccess || hipMalloc(&p->d_zero_rows, list_bytes) != hipSuccess) {
     (void)hipGetLastError();
-    return fail(HPSPMM_ERR_ALLOC, "device allocation for the routed plan failed (%zu bytes)",
-                vptr_bytes + 3 * v_bytes + partial_bytes + carry_bytes + bhot_bytes);
+    return fail(HPSPMM_ERR_ALLOC, "device allocation for the routed plan failed (%zu bytes)", total_bytes);
   }
-  p->workspace_bytes =
-      (int64_t)(vptr_bytes + 3 * v_bytes + (size_t)nnz * 4 + partial_bytes + carry_bytes + bhot_bytes + n_bhot * 4);
+  p->workspace_bytes = (int64_t)total_bytes;
   HPSPMM_HIP(hipMemcpyAsync(p->d_bhot_src, bhot_src.data(), bhot_src.size() * sizeof(int32_t),
                             hipMemcpyHostToDevice, st));
   // unused compact-buffer rows and the padding between the classes are never used; keep them defined anyway
   HPSPMM_HIP(hipMemsetAsync(p->d_bhot, 0, bhot_bytes, st));
   HPSPMM_HIP(hipMemsetAsync(p->d_vval, 0, v_bytes, st));
-  const int64_t nvptr = (int64_t)ncls * (rows + 1);
-  hipLaunchKernelGGL(hpspmm::routed_vptr_kernel, dim3((unsigned)ceil_div(nvptr, hpspmm::kBlock)),
-                     dim3(hpspmm::kBlock), 0, st, lay, d_scan, p->d_vptr);
+  HPSPMM_HIP(hipMemsetAsync(d_counts, 0, 2 * sizeof(int32_t), st));
+  const int64_t nrv = (n_routed + 1) * nhub;
+  hipLaunchKernelGGL(hpspmm::routed_vptr_kernel, dim3((unsigned)ceil_div(nrv, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                     0, st, lay, d_cnt, p->d_rvptr);
+  hipLaunchKernelGGL(hpspmm::routed_coldptr_kernel, dim3((unsigned)ceil_div(rows + 1, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, rows, lay.cls_begin[nhub], d_coldcnt, p->d_coldptr);
   hipLaunchKernelGGL(hpspmm::routed_fill_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col,
-                     d_colmap, (int32_t)h, nsub, min_row_nnz, p->d_vptr, p->d_vcol, p->d_vpos, p->d_vrow, p->d_action,
-                     p->shift);
+                     d_colmap, d_ridx, (int32_t)h, nsub, min_row_nnz, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vpos,
+                     p->d_vrow, p->d_routed_rows, d_action, p->shift);
+  // compact lists of the short rows the final kernel has to visit
+  const unsigned cgrid = (unsigned)ceil_div(rows, hpspmm::kBlock);
+  hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(cgrid), dim3(hpspmm::kBlock), 0, st, rows, d_action,
+                     hpspmm::kActionCross, p->d_cross_rows, d_counts);
+  hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(cgrid), dim3(hpspmm::kBlock), 0, st, rows, d_action,
+                     hpspmm::kActionZero, p->d_zero_rows, d_counts + 1);
+  int32_t counts[2] = {0, 0};
+  HPSPMM_HIP(hipMemcpyAsync(counts, d_counts, sizeof counts, hipMemcpyDeviceToHost, st));
   HPSPMM_HIP(hipStreamSynchronize(st));
   HPSPMM_HIP(hipGetLastError());
-  // compact lists of the rows the final kernel has to visit
-  {
-    int32_t* d_counts = nullptr;
-    HPSPMM_HIP(hipMalloc(&d_counts, 2 * sizeof(int32_t)));
-    struct CountGuard {
-      int32_t* q;
-      ~CountGuard() { (void)hipFree(q); }
-    } cg{d_counts};
-    HPSPMM_HIP(hipMemsetAsync(d_counts, 0, 2 * sizeof(int32_t), st));
-    if (hipMalloc(&p->d_reduce_rows, (size_t)rows * sizeof(int32_t)) != hipSuccess ||
-        hipMalloc(&p->d_zero_rows, (size_t)rows * sizeof(int32_t)) != hipSuccess) {
-      (void)hipGetLastError();
-      return fail(HPSPMM_ERR_ALLOC, "device allocation for the routed row lists failed");
-    }
-    p->workspace_bytes += 2 * rows * (int64_t)sizeof(int32_t);
-    const unsigned cgrid = (unsigned)ceil_div(rows, hpspmm::kBlock);
-    hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(cgrid), dim3(hpspmm::kBlock), 0, st, rows, p->d_action,
-                       hpspmm::kActionReduce, p->d_reduce_rows, d_counts);
-    hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(cgrid), dim3(hpspmm::kBlock), 0, st, rows, p->d_action,
-                       hpspmm::kActionZero, p->d_zero_rows, d_counts + 1);
-    int32_t counts[2] = {0, 0};
-    HPSPMM_HIP(hipMemcpyAsync(counts, d_counts, sizeof counts, hipMemcpyDeviceToHost, st));
-    HPSPMM_HIP(hipStreamSynchronize(st));
-    p->n_reduce = counts[0];
-    p->n_zero = counts[1];
-  }
+  p->n_cross = counts[0];
+  p->n_zero = counts[1];
   p->n_bhot = n_bhot;
   p->n_hub = (int64_t)ids.size();
   p->nseg = nseg;
@@ -448,13 +468,15 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
                      aligned16(v, v, v));
   if (p->routed_grid > 0)
     hipLaunchKernelGGL(hpspmm::spmm_routed_kernel<K>, dim3((unsigned)p->routed_grid), dim3(hpspmm::kBlock), 0, st,
-                       p->lay, p->d_vptr, p->d_vcol, p->d_vval, p->d_vrow, B, p->d_bhot, p->d_partial, p->d_carry, C);
-  const int64_t reduce_blocks = row_blocks(p->n_reduce, K);
-  const int64_t fin_blocks = reduce_blocks + row_blocks(p->n_zero, K);
+                       p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval, p->d_vrow, B, p->d_bhot, p->d_partial,
+                       p->d_carry, C);
+  const int64_t routed_blocks = row_blocks(p->lay.n_routed, K);
+  const int64_t cross_blocks = row_blocks(p->n_cross, K);
+  const int64_t fin_blocks = routed_blocks + cross_blocks + row_blocks(p->n_zero, K);
   if (fin_blocks > 0)
     hipLaunchKernelGGL(hpspmm::spmm_routed_final_kernel<K>, dim3((unsigned)fin_blocks), dim3(hpspmm::kBlock), 0, st,
-                       p->lay, p->d_vptr, p->d_reduce_rows, p->n_reduce, reduce_blocks, p->d_zero_rows, p->n_zero,
-                       p->d_partial, p->d_carry, C);
+                       p->lay, p->d_rvptr, p->d_coldptr, p->d_routed_rows, routed_blocks, p->d_cross_rows, p->n_cross,
+                       cross_blocks, p->d_zero_rows, p->n_zero, p->d_partial, p->d_carry, C);
   return HPSPMM_OK;
 }
 
@@ -669,9 +691,9 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
   if (plan->d_hub_ids) (void)hipFree(plan->d_hub_ids);
   if (plan->d_hub_col) (void)hipFree(plan->d_hub_col);
   if (plan->d_bhot) (void)hipFree(plan->d_bhot);
-  for (void* q : {(void*)plan->d_vptr, (void*)plan->d_vcol, (void*)plan->d_vpos, (void*)plan->d_vval, (void*)plan->d_vrow,
-                  (void*)plan->d_bhot_src, (void*)plan->d_partial, (void*)plan->d_action,
-                  (void*)plan->d_reduce_rows, (void*)plan->d_zero_rows})
+  for (void* q : {(void*)plan->d_rvptr, (void*)plan->d_coldptr, (void*)plan->d_vcol, (void*)plan->d_vpos,
+                  (void*)plan->d_vval, (void*)plan->d_vrow, (void*)plan->d_bhot_src, (void*)plan->d_partial,
+                  (void*)plan->d_routed_rows, (void*)plan->d_cross_rows, (void*)plan->d_zero_rows})
     if (q) (void)hipFree(q);
   delete plan;
   return HPSPMM_OK;

@@ -19,21 +19,26 @@
 //     whatever memory channels their original addresses collide on;
 //   * degree binning: only rows with at least `min_row_nnz` nonzeros are
 //     routed - a short row would pay one partial-result row per class it
-//     touches for a handful of gathers.  A nonzero of a routed row belongs to
-//     the class (phase, slice) of its column, all nonzeros of a short row to
-//     the last class.  The plan lays the nonzeros out class by class, each
+//     touches for a handful of gathers.  Routed rows are numbered 0 ..
+//     n_routed-1 in row order; a nonzero of a routed row belongs to the hub
+//     class (phase, slice) of its column, all nonzeros of a short row to the
+//     last ("cold") class.  The plan lays the nonzeros out class by class, each
 //     class in row order, as column (~compact-buffer row if the column is
-//     cached) and row arrays, plus the position of every stored nonzero in
-//     that order; every SpMM first scatters the caller's values into the same
-//     order (reading them in place would fetch each line of the value array
-//     once per class: 3.7 GB instead of 0.46 GB on the social graph);
+//     cached) and row arrays (routed-row number in the hub classes, row in the
+//     cold class), plus the position of every stored nonzero in that order;
+//     every SpMM first scatters the caller's values into the same order
+//     (reading them in place would fetch each line of the value array once per
+//     class: 3.7 GB instead of 0.46 GB on the social graph);
 //   * inside a class the work is cut into fixed-length segments exactly as in
-//     the segments strategy; a (row, class) run that lies inside one segment is
-//     stored to the row's partial-result slot of the class, runs that cross a
+//     the segments strategy.  A run (the nonzeros of one row in one class)
+//     that lies inside one segment is complete: in a hub class it is stored to
+//     the routed row's partial-result slot of the class, in the cold class
+//     straight to C (a short row has no other class).  Runs that cross a
 //     segment boundary go through the carry slots;
-//   * a final kernel adds, for every row, its class partials in class order
-//     and writes C (zeros for empty rows).  No atomics; results are
-//     bit-reproducible for a given plan.
+//   * a final kernel adds, for every routed row, its class results in class
+//     order and writes C; it also finishes the short rows whose run crossed a
+//     segment boundary and writes zeros for empty rows.  No atomics; results
+//     are bit-reproducible for a given plan.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -43,39 +48,37 @@
 
 namespace hpspmm {
 
-constexpr int kSlices = 8;                          // column slices, one per XCD
-constexpr int kMaxSub = 7;                          // sub-slices (phases) per slice, at most
-constexpr int kMaxClasses = kSlices * kMaxSub + 1;  // + the class of the short rows; fits one wavefront's lanes
+constexpr int kSlices = 8;                 // column slices, one per XCD
+constexpr int kMaxSub = 7;                 // phases per slice, at most
+constexpr int kMaxHub = kSlices * kMaxSub;  // hub classes, at most: fits one wavefront's lanes
+constexpr int kMaxClasses = kMaxHub + 1;   // + the cold class
 
-// What the final kernel does with a row.
-constexpr uint8_t kActionNone = 0;    // the main kernel stored the row to C itself
-constexpr uint8_t kActionZero = 1;    // no nonzeros: write zeros
-constexpr uint8_t kActionReduce = 2;  // add the class results
+// What the final kernel does with a short row.
+constexpr uint8_t kActionNone = 0;   // the main kernel stored it (or it is routed)
+constexpr uint8_t kActionZero = 1;   // no nonzeros: write zeros
+constexpr uint8_t kActionCross = 2;  // its run crosses a segment boundary: add the carry slots
 
-// Class x < 8 * nsub is (phase x / 8, slice x % 8); class 8 * nsub holds the short rows.
+// Class x < nhub = 8 * nsub is (phase x / 8, slice x % 8); class nhub is the cold class.
 struct RoutedLayout {
   int64_t cls_begin[kMaxClasses];    // first virtual index of the class (multiple of the workgroup quantum)
   int64_t cls_end[kMaxClasses];      // one past its last real entry
   int64_t cls_blocks[kMaxClasses];   // workgroups needed by the class
-  int64_t phase_begin[kMaxSub + 1];  // first workgroup of phase p (a multiple of 8); [nsub]: of the short-row class
+  int64_t phase_begin[kMaxSub + 1];  // first workgroup of phase p (a multiple of 8); [nsub]: of the cold class
   int64_t rows;
+  int64_t n_routed;
   int shift;  // log2(segment length)
   int nsub;   // phases
-  int ncls;   // 8 * nsub + 1
+  int nhub;   // 8 * nsub
 };
 
 // ---- plan-time kernels -----------------------------------------------------
 
-// Class of a nonzero in column c: mapped = colmap[c] is the compact-buffer row
-// of a cached column or -1.  A cached column of popularity rank s sits in
+// Hub class of a nonzero in column c: mapped = colmap[c] is the compact-buffer
+// row of a cached column or -1.  A cached column of popularity rank s sits in
 // compact-buffer row (s % 8) * hub_rows_per_slice + s / 8 and belongs to slice
 // s % 8, phase (s / 8) % nsub, so that every (slice, phase) gets the same mix
-// of hot and cold columns; the other columns are spread by a multiplicative
-// hash.  Rows shorter than the routing threshold send everything to the last
-// class.
-__device__ __forceinline__ int class_of(int32_t c, int32_t mapped, int32_t hub_rows_per_slice, int nsub,
-                                        bool routed_row) {
-  if (!routed_row) return kSlices * nsub;
+// of hot and cold columns; the other columns are spread by a multiplicative hash.
+__device__ __forceinline__ int hub_class_of(int32_t c, int32_t mapped, int32_t hub_rows_per_slice, int nsub) {
   int slice, sub;
   if (mapped >= 0) {
     slice = mapped / hub_rows_per_slice;
@@ -88,37 +91,55 @@ __device__ __forceinline__ int class_of(int32_t c, int32_t mapped, int32_t hub_r
   return sub * kSlices + slice;
 }
 
-// cnt[x * rows + r] = number of nonzeros of row r in class x.  One wavefront per row.
-__global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+// flag[r] = 1 if row r is routed (r < rows), flag[rows] = 0.
+__global__ __launch_bounds__(kBlock) void routed_flag_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                             int32_t min_row_nnz, uint32_t* __restrict__ flag) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r > rows) return;
+  flag[r] = r < rows && rowptr[r + 1] - rowptr[r] >= min_row_nnz ? 1u : 0u;
+}
+
+// One wavefront per row.  Routed row (number ridx[r]): cnt[x * n_routed +
+// ridx[r]] = its nonzeros in hub class x, coldcnt[r] = 0.  Short row:
+// coldcnt[r] = its nonzeros.  coldcnt[rows] = 0 and cnt[nhub * n_routed] = 0
+// (the scans' total slots) are written by the first wavefront.
+__global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t rows, int64_t n_routed,
+                                                              const int32_t* __restrict__ rowptr,
                                                               const int32_t* __restrict__ col,
                                                               const int32_t* __restrict__ colmap,
+                                                              const uint32_t* __restrict__ ridx,
                                                               int32_t hub_rows_per_slice, int nsub,
-                                                              int32_t min_row_nnz, uint32_t* __restrict__ cnt) {
+                                                              int32_t min_row_nnz, uint32_t* __restrict__ cnt,
+                                                              uint32_t* __restrict__ coldcnt) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   if (row >= rows) return;
-  const int ncls = kSlices * nsub + 1;
+  const int nhub = kSlices * nsub;
+  if (row == 0 && lane == 0) {
+    coldcnt[rows] = 0;
+    cnt[(int64_t)nhub * n_routed] = 0;
+  }
   const int32_t lb = rowptr[row];
   const int32_t hb = rowptr[row + 1];
-  const bool routed_row = hb - lb >= min_row_nnz;
-  uint32_t mine = 0;  // lane x < ncls accumulates the count of class x
-  if (!routed_row) {
-    if (lane == ncls - 1) mine = (uint32_t)(hb - lb);
-  } else {
-    for (int32_t j0 = lb; j0 < hb; j0 += 64) {
-      const int32_t j = j0 + lane;
-      int cls = -1;
-      if (j < hb) {
-        const int32_t c = col[j];
-        cls = class_of(c, colmap[c], hub_rows_per_slice, nsub, true);
-      }
-      for (int x = 0; x < ncls - 1; ++x) {
-        const uint64_t m = __ballot(cls == x);
-        if (lane == x) mine += (uint32_t)__popcll(m);
-      }
+  if (hb - lb < min_row_nnz) {
+    if (lane == 0) coldcnt[row] = (uint32_t)(hb - lb);
+    return;
+  }
+  if (lane == 0) coldcnt[row] = 0;
+  uint32_t mine = 0;  // lane x < nhub accumulates the count of class x
+  for (int32_t j0 = lb; j0 < hb; j0 += 64) {
+    const int32_t j = j0 + lane;
+    int cls = -1;
+    if (j < hb) {
+      const int32_t c = col[j];
+      cls = hub_class_of(c, colmap[c], hub_rows_per_slice, nsub);
+    }
+    for (int x = 0; x < nhub; ++x) {
+      const uint64_t m = __ballot(cls == x);
+      if (lane == x) mine += (uint32_t)__popcll(m);
     }
   }
-  if (lane < ncls) cnt[(int64_t)lane * rows + row] = mine;
+  if (lane < nhub) cnt[(int64_t)lane * n_routed + ridx[row]] = mine;
 }
 
 // Three-pass exclusive scan of uint32 (n up to 2^32, total < 2^32).
@@ -175,9 +196,10 @@ __global__ __launch_bounds__(kBlock) void scan_tile_offsets_kernel(int64_t ntile
   }
 }
 
-__global__ __launch_bounds__(kBlock) void scan_apply_kernel(int64_t n, const uint32_t* __restrict__ in,
+// (`out` may be `in`: every thread reads its items before it writes them.)
+__global__ __launch_bounds__(kBlock) void scan_apply_kernel(int64_t n, const uint32_t* in,
                                                             const uint32_t* __restrict__ tile_offsets,
-                                                            uint32_t* __restrict__ out) {
+                                                            uint32_t* out) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
   const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
   uint32_t v[kScanItems];
@@ -196,82 +218,91 @@ __global__ __launch_bounds__(kBlock) void scan_apply_kernel(int64_t n, const uin
   }
 }
 
-// vptr[r * ncls + x] = virtual index of the first class-x nonzero of row r
-// (r = rows: one past the class), from the exclusive scan of the class-major
-// counts and the padded class origins.  The end of the (r, x) run is
-// vptr[(r + 1) * ncls + x].
+// rvptr[r * nhub + x] = virtual index of the first class-x nonzero of routed
+// row number r (r = n_routed: one past the class), from the exclusive scan of
+// the class-major counts and the padded class origins.  The end of the (r, x)
+// run is rvptr[(r + 1) * nhub + x].
 __global__ __launch_bounds__(kBlock) void routed_vptr_kernel(RoutedLayout lay, const uint32_t* __restrict__ scanned,
-                                                             int32_t* __restrict__ vptr) {
+                                                             int32_t* __restrict__ rvptr) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (i >= (lay.rows + 1) * lay.ncls) return;
-  const int64_t r = i / lay.ncls;
-  const int x = (int)(i - r * lay.ncls);
-  const int64_t first = scanned[(int64_t)x * lay.rows];
-  const int64_t local = r < lay.rows ? (int64_t)scanned[(int64_t)x * lay.rows + r] - first
-                                     : lay.cls_end[x] - lay.cls_begin[x];
-  vptr[i] = (int32_t)(lay.cls_begin[x] + local);
+  if (i >= (lay.n_routed + 1) * lay.nhub) return;
+  const int64_t r = i / lay.nhub;
+  const int x = (int)(i - r * lay.nhub);
+  const int64_t first = scanned[(int64_t)x * lay.n_routed];
+  const int64_t local = r < lay.n_routed ? (int64_t)scanned[(int64_t)x * lay.n_routed + r] - first
+                                         : lay.cls_end[x] - lay.cls_begin[x];
+  rvptr[i] = (int32_t)(lay.cls_begin[x] + local);
+}
+
+// coldptr[r] = virtual index of the first cold-class nonzero of row r (r = rows: one past the class).
+__global__ __launch_bounds__(kBlock) void routed_coldptr_kernel(int64_t rows, int64_t cold_begin,
+                                                                const uint32_t* __restrict__ scanned,
+                                                                int32_t* __restrict__ coldptr) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r > rows) return;
+  coldptr[r] = (int32_t)(cold_begin + (int64_t)scanned[r]);
 }
 
 // Scatter the nonzeros into class-major order, keeping the stored order inside
-// every (row, class) run.  One wavefront per row; positions from ballots.
+// every run.  One wavefront per row; positions in the hub classes from ballots.
 __global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                              const int32_t* __restrict__ col,
                                                              const int32_t* __restrict__ colmap,
+                                                             const uint32_t* __restrict__ ridx,
                                                              int32_t hub_rows_per_slice, int nsub,
-                                                             int32_t min_row_nnz, const int32_t* __restrict__ vptr,
+                                                             int32_t min_row_nnz, const int32_t* __restrict__ rvptr,
+                                                             const int32_t* __restrict__ coldptr,
                                                              int32_t* __restrict__ vcol, int32_t* __restrict__ vpos,
                                                              int32_t* __restrict__ vrow,
+                                                             int32_t* __restrict__ routed_rows,
                                                              uint8_t* __restrict__ action, int shift) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   if (row >= rows) return;
-  const int ncls = kSlices * nsub + 1;
+  const int nhub = kSlices * nsub;
   const int32_t lb = rowptr[row];
   const int32_t hb = rowptr[row + 1];
-  const bool routed_row = hb - lb >= min_row_nnz;
-  int32_t cursor = lane < ncls ? vptr[row * ncls + lane] : 0;  // lane x: next slot of class x
-  const int32_t cls_last = lane < ncls ? vptr[(row + 1) * ncls + lane] : 0;
-  const uint64_t below = (1ull << lane) - 1ull;
-  // A row without entries outside the last class is "direct": its run is stored
-  // straight to C (flagged by the sign bit of vrow) unless it crosses a segment boundary.
-  const bool direct = __ballot(lane < ncls - 1 && cls_last > cursor) == 0;
-  if (lane == ncls - 1) {
-    uint8_t a = kActionReduce;
-    if (direct) {
-      if (cls_last == cursor) a = kActionZero;
-      else if (((int64_t)cursor >> shift) == ((int64_t)(cls_last - 1) >> shift)) a = kActionNone;
+  if (hb - lb < min_row_nnz) {
+    // everything goes to the cold class, in stored order
+    const int32_t start = coldptr[row];
+    if (lane == 0) {
+      uint8_t a = kActionNone;
+      if (hb == lb) a = kActionZero;
+      else if (((int64_t)start >> shift) != ((int64_t)(start + (hb - lb) - 1) >> shift)) a = kActionCross;
+      action[row] = a;
     }
-    action[row] = a;
-  }
-  const int32_t row_tag = direct ? (int32_t)((uint32_t)row | 0x80000000u) : (int32_t)row;
-  if (!routed_row) {
-    // everything goes to the last class, in stored order
-    const int32_t start = __shfl(cursor, ncls - 1);
     for (int32_t j = lb + lane; j < hb; j += 64) {
       const int32_t c = col[j];
       const int32_t mapped = colmap[c];
       const int32_t pos = start + (j - lb);
-      vcol[pos] = mapped >= 0 ? ~mapped : c;
+      vcol[pos] = mapped >= 0 ? ~mapped : c;  // ~compact-buffer row if the column is cached
       vpos[j] = pos;
-      vrow[pos] = row_tag;
+      vrow[pos] = (int32_t)row;
     }
     return;
   }
+  const int32_t r = (int32_t)ridx[row];
+  if (lane == 0) {
+    action[row] = kActionNone;
+    routed_rows[r] = (int32_t)row;
+  }
+  int32_t cursor = lane < nhub ? rvptr[(int64_t)r * nhub + lane] : 0;  // lane x: next slot of class x
+  const uint64_t below = (1ull << lane) - 1ull;
   for (int32_t j0 = lb; j0 < hb; j0 += 64) {
     const int32_t j = j0 + lane;
     const bool valid = j < hb;
     const int32_t c = valid ? col[j] : 0;
     const int32_t mapped = valid ? colmap[c] : -1;
-    const int cls = valid ? class_of(c, mapped, hub_rows_per_slice, nsub, true) : -1;
-    for (int x = 0; x < ncls - 1; ++x) {
+    const int cls = valid ? hub_class_of(c, mapped, hub_rows_per_slice, nsub) : -1;
+    for (int x = 0; x < nhub; ++x) {
       const uint64_t m = __ballot(cls == x);
       if (m == 0) continue;
       const int32_t start = __shfl(cursor, x);
       if (cls == x) {
         const int32_t pos = start + (int32_t)__popcll(m & below);
-        vcol[pos] = mapped >= 0 ? ~mapped : c;  // ~compact-buffer row if the column is cached
+        vcol[pos] = mapped >= 0 ? ~mapped : c;
         vpos[j] = pos;
-        vrow[pos] = row_tag;
+        vrow[pos] = r;
       }
       if (lane == x) cursor += (int32_t)__popcll(m);
     }
@@ -324,14 +355,15 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
 
 // Workgroups [phase_begin[p], phase_begin[p + 1]): phase p; its workgroup number
 // i serves class (p, i % 8) - and runs on XCD i % 8 - as that class's i / 8-th
-// workgroup.  Workgroups from phase_begin[nsub] on: the short rows.  The
+// workgroup.  Workgroups from phase_begin[nsub] on: the cold class.  The
 // hardware starts workgroups in index order, so every XCD works through its
-// slice one phase, i.e. one L2-sized set of B rows, at a time.
+// slice one phase, i.e. one set of B rows, at a time.
 // Each sub-wave owns one segment of its class; see the carry rule of the
-// segments kernel - here "stored to C" becomes "stored to the row's
-// partial-result slot of the class".
+// segments kernel - in a hub class "stored to C" becomes "stored to the routed
+// row's partial-result slot of the class".
 template <int K>
-__global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, const int32_t* __restrict__ vptr,
+__global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, const int32_t* __restrict__ rvptr,
+                                                             const int32_t* __restrict__ coldptr,
                                                              const int32_t* __restrict__ vcol,
                                                              const float* __restrict__ vval,
                                                              const int32_t* __restrict__ vrow,
@@ -346,17 +378,18 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
   __shared__ __attribute__((aligned(16))) float s_val[kWavesPerBlock * P * kTileStride];
   __shared__ __attribute__((aligned(16))) int32_t s_row[kWavesPerBlock * P * kTileStride];
 
-  const int ncls = lay.ncls;
+  const int nhub = lay.nhub;
   int p = 0;
   while (p < lay.nsub && (int64_t)blockIdx.x >= lay.phase_begin[p + 1]) ++p;
   const int64_t rel = (int64_t)blockIdx.x - lay.phase_begin[p];
+  const bool hub = p < lay.nsub;
   int x;
   int64_t i;
-  if (p < lay.nsub) {
+  if (hub) {
     x = p * kSlices + (int)(rel % kSlices);
     i = rel / kSlices;
   } else {
-    x = ncls - 1;
+    x = nhub;
     i = rel;
   }
   if (i >= lay.cls_blocks[x]) return;
@@ -371,19 +404,19 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
   if (s >= cls_end) return;
   const int64_t e = (s + ((int64_t)1 << shift)) < cls_end ? (s + ((int64_t)1 << shift)) : cls_end;
   const int sbase = ((tid >> 6) * P + lane / G) * kTileStride;
-  const int32_t* vp = vptr + x;
-  float* pout = partial + (uint64_t)x * K;
+  // first index of a run: rvptr[number * nhub + x] in a hub class, coldptr[row] in the cold class
+  const int32_t* vp = hub ? rvptr + x : coldptr;
+  const int64_t vstride = hub ? nhub : 1;
+  float* out = hub ? partial + (uint64_t)x * K : C;
+  const uint64_t ostride = hub ? (uint64_t)nhub * K : (uint64_t)K;
 
-  // the sign bit of a row entry marks a row that is stored straight to C
   int32_t cur = vrow[s];
-  bool head_pending = (int64_t)vp[(int64_t)(cur & 0x7FFFFFFF) * ncls] < s;
+  bool head_pending = (int64_t)vp[(int64_t)cur * vstride] < s;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 
   auto flush_to = [&](bool is_tail) {
-    const uint32_t row = (uint32_t)cur & 0x7FFFFFFFu;
     float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
-                              : (is_tail ? carry + (uint64_t)(2 * g + 1) * K
-                                         : (cur < 0 ? C + (uint64_t)row * K : pout + (uint64_t)row * ncls * K));
+                              : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : out + (uint64_t)(uint32_t)cur * ostride);
     head_pending = false;
     *reinterpret_cast<float4*>(dst + 4 * l) = acc;
   };
@@ -407,7 +440,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
     consume_tile(cnt, sbase, s_col, s_val, s_row, cur, acc, loadb, flush);
     wave_lds_fence();
   }
-  flush_to((int64_t)vp[(int64_t)((cur & 0x7FFFFFFF) + 1) * ncls] > e);
+  flush_to((int64_t)vp[(int64_t)(cur + 1) * vstride] > e);
 }
 
 // list[] <- every row whose action byte equals `which` (order unspecified); *count must be zero on entry.
@@ -425,29 +458,25 @@ __global__ __launch_bounds__(kBlock) void routed_collect_rows_kernel(int64_t row
   if (hit) list[base + __popcll(mask & ((1ull << lane) - 1ull))] = (int32_t)i;
 }
 
-// Final pass, one sub-wave per listed row.  Workgroups [0, reduce_blocks): rows
-// whose class results must be added - in class order, the row's partial-result
-// slot if the (row, class) run lies in one segment, else tail[ga] + head[ga+1]
-// + ... + head[gb] from the carry slots.  Remaining workgroups: rows without
-// nonzeros, which get zeros.  Rows in neither list were stored by the main kernel.
-// (Lists rather than a scan over all rows: on R-MAT the rows that need a
-// reduction sit together at low indices and serialised inside a few waves.)
-//
-// With segments of 512 nonzeros and runs of some tens, about one run in eight
-// crosses a segment boundary, i.e. most rows have one: the first two slots of
-// every run (partial or tail, then the next head) are therefore fetched
-// together for a group of classes, and only a run over three or more segments
-// (a hub row) takes the loop over the remaining heads.
+// Final pass, one sub-wave per listed row, three parts.
+// Workgroups [0, routed_blocks): routed row number i gets the sum of its class
+// results in class order - per class the partial-result slot if the run lies
+// in one segment, else tail[ga] + head[ga+1] + ... + head[gb] from the carry
+// slots.  With segments of 512 nonzeros and runs of some tens, about one run
+// in eight crosses a segment boundary, i.e. most rows have one: the first two
+// slots of every run are therefore fetched together for a group of classes,
+// and only a run over three or more segments (a hub row) takes the loop over
+// the remaining heads.
+// Workgroups [routed_blocks, routed_blocks + cross_blocks): short rows whose
+// cold-class run crossed a segment boundary, from the carry slots alone.
+// The rest: rows without nonzeros, which get zeros.
+// Rows in none of the lists were stored by the main kernel.
 template <int K>
-__global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout lay,
-                                                                   const int32_t* __restrict__ vptr,
-                                                                   const int32_t* __restrict__ reduce_rows,
-                                                                   int64_t n_reduce, int64_t reduce_blocks,
-                                                                   const int32_t* __restrict__ zero_rows,
-                                                                   int64_t n_zero,
-                                                                   const float* __restrict__ partial,
-                                                                   const float* __restrict__ carry,
-                                                                   float* __restrict__ C) {
+__global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
+    RoutedLayout lay, const int32_t* __restrict__ rvptr, const int32_t* __restrict__ coldptr,
+    const int32_t* __restrict__ routed_rows, int64_t routed_blocks, const int32_t* __restrict__ cross_rows,
+    int64_t n_cross, int64_t cross_blocks, const int32_t* __restrict__ zero_rows, int64_t n_zero,
+    const float* __restrict__ partial, const float* __restrict__ carry, float* __restrict__ C) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
   constexpr int kGroup = 4;  // classes whose loads are in flight together
@@ -455,20 +484,9 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout 
   const int lane = tid & 63;
   const int l = lane % G;
   const int shift = lay.shift;
-  const int ncls = lay.ncls;
-  if ((int64_t)blockIdx.x >= reduce_blocks) {
-    const int64_t idx = (((int64_t)blockIdx.x - reduce_blocks) * kWavesPerBlock + (tid >> 6)) * P + lane / G;
-    if (idx >= n_zero) return;
-    *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * K + 4 * l) = make_float4(0.f, 0.f, 0.f, 0.f);
-    return;
-  }
-  const int64_t idx = ((int64_t)blockIdx.x * kWavesPerBlock + (tid >> 6)) * P + lane / G;
-  if (idx >= n_reduce) return;
-  const int64_t row = reduce_rows[idx];
-  const int32_t* vlo = vptr + row * ncls;
-  const int32_t* vhi = vlo + ncls;
-  const float* prow = partial + (uint64_t)row * ncls * K + 4 * l;
+  const int nhub = lay.nhub;
   const float* cbase = carry + 4 * l;
+  const int64_t sub = (int64_t)(tid >> 6) * P + lane / G;  // sub-wave within the workgroup
 
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   auto add = [&](const float4& t) {
@@ -477,18 +495,56 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout 
     acc.z += t.z;
     acc.w += t.w;
   };
+  // acc += head[g] for g in [g0, gb], 8 slots in flight at a time, added in segment order
+  auto add_heads = [&](int64_t g0, int64_t gb) {
+    int64_t g = g0;
+    for (; g + kBatch <= gb + 1; g += kBatch) {
+      float4 slot[kBatch];
+#pragma unroll
+      for (int t = 0; t < kBatch; ++t)
+        slot[t] = *reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * (g + t)) * K);
+#pragma unroll
+      for (int t = 0; t < kBatch; ++t) add(slot[t]);
+    }
+    for (; g <= gb; ++g) add(*reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * g) * K));
+  };
+
+  if ((int64_t)blockIdx.x >= routed_blocks + cross_blocks) {
+    const int64_t idx = ((int64_t)blockIdx.x - routed_blocks - cross_blocks) * (kWavesPerBlock * P) + sub;
+    if (idx >= n_zero) return;
+    *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * K + 4 * l) = acc;
+    return;
+  }
+  if ((int64_t)blockIdx.x >= routed_blocks) {
+    const int64_t idx = ((int64_t)blockIdx.x - routed_blocks) * (kWavesPerBlock * P) + sub;
+    if (idx >= n_cross) return;
+    const int64_t row = cross_rows[idx];
+    const int64_t ga = coldptr[row] >> shift;
+    const int64_t gb = (coldptr[row + 1] - 1) >> shift;
+    add(*reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * ga + 1) * K));
+    add_heads(ga + 1, gb);
+    *reinterpret_cast<float4*>(C + (uint64_t)row * K + 4 * l) = acc;
+    return;
+  }
+  const int64_t idx = (int64_t)blockIdx.x * (kWavesPerBlock * P) + sub;
+  if (idx >= lay.n_routed) return;
+  const int64_t row = routed_rows[idx];
+  const int32_t* vlo = rvptr + idx * nhub;
+  const int32_t* vhi = vlo + nhub;
+  const float* prow = partial + (uint64_t)idx * nhub * K + 4 * l;
+
   auto bounds = [&](int x0, int32_t (&lb)[kGroup], int32_t (&hb)[kGroup]) {
 #pragma unroll
     for (int q = 0; q < kGroup; ++q) {
-      const bool in = x0 + q < ncls;
-      const int x = in ? x0 + q : ncls - 1;
+      const bool in = x0 + q < nhub;
+      const int x = in ? x0 + q : nhub - 1;
       lb[q] = vlo[x];
       hb[q] = in ? vhi[x] : lb[q];
     }
   };
   int32_t nlb[kGroup], nhb[kGroup];
   bounds(0, nlb, nhb);
-  for (int x0 = 0; x0 < ncls; x0 += kGroup) {
+  for (int x0 = 0; x0 < nhub; x0 += kGroup) {
     int32_t lb[kGroup], hb[kGroup];
     float4 first[kGroup], second[kGroup];
     bool some[kGroup], two[kGroup];
@@ -508,7 +564,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout 
       if (some[q]) first[q] = *reinterpret_cast<const float4*>(pa);
       if (two[q]) second[q] = *reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * (ga + 1)) * K);
     }
-    if (x0 + kGroup < ncls) bounds(x0 + kGroup, nlb, nhb);  // in flight together with the slots above
+    if (x0 + kGroup < nhub) bounds(x0 + kGroup, nlb, nhb);  // in flight together with the slots above
     if (!longer) {
 #pragma unroll
       for (int q = 0; q < kGroup; ++q) {
@@ -522,18 +578,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(RoutedLayout 
       if (some[q]) add(first[q]);
       if (!two[q]) continue;
       add(second[q]);
-      // a hub row spans hundreds of segments: fetch the remaining heads 8 at a time, add them in segment order
-      const int64_t gb = (hb[q] - 1) >> shift;
-      int64_t g = (lb[q] >> shift) + 2;
-      for (; g + kBatch <= gb + 1; g += kBatch) {
-        float4 slot[kBatch];
-#pragma unroll
-        for (int t = 0; t < kBatch; ++t)
-          slot[t] = *reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * (g + t)) * K);
-#pragma unroll
-        for (int t = 0; t < kBatch; ++t) add(slot[t]);
-      }
-      for (; g <= gb; ++g) add(*reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * g) * K));
+      add_heads((lb[q] >> shift) + 2, (hb[q] - 1) >> shift);
     }
   }
   *reinterpret_cast<float4*>(C + (uint64_t)row * K + 4 * l) = acc;

@@ -273,10 +273,11 @@ constexpr int64_t kRoutedMinBBytes = (int64_t)48 << 20;  // B must overflow the 
 constexpr double kRoutedMinShare = 0.35;     // of the nonzeros in the 64k most referenced columns
 constexpr double kRoutedMinRowNnz = 32.0;    // mean nonzeros per non-empty row
 constexpr int32_t kRoutedRowThreshold = 128;  // rows shorter than this are not split over the classes
-// Phases: a slice of B larger than this is worked through in several phases.  Every phase
-// adds a partial-result row per routed row, so on the 233k-vertex social graph only
-// K = 128 (15 MB a slice) gains, and only from two phases: 4.16 -> 4.06 ms, three: 4.38 ms;
-// at K = 64 (7.5 MB a slice) one phase 2.18 ms, two 2.34 ms.
+// Phases: a slice of B larger than this is worked through in two phases, which halves the
+// set of hot rows an L2 has to hold at a time.  Every phase adds a partial-result row per
+// routed row, and more than two never paid: 233k-vertex social graph, K = 128 (15 MB a
+// slice) 4.11 / 4.01 / 4.34 ms with 1 / 2 / 3 phases, K = 64 (7.5 MB a slice) 2.14 / 2.28 /
+// 2.51 ms; R-MAT scale 22, K = 128 (268 MB a slice) 6.63 / 6.23 / 6.32 ms.
 constexpr int64_t kRoutedPhaseBytes = (int64_t)8 << 20;
 
 // Builds the routed layout.  Returns HPSPMM_OK with p->strategy left at
@@ -298,11 +299,8 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
     return HPSPMM_OK;
   if (nnz > INT32_MAX - ((int64_t)1 << 24)) return HPSPMM_OK;  // virtual indices stay int32
 
-  // Phases: as many as bring one phase's share of a slice of B down to kRoutedPhaseBytes,
-  // at most 2 (see above); a B far beyond what phases could make L2-sized gets one.
   const int64_t slice_bytes = p->cols * k * 4 / hpspmm::kSlices;
-  int nsub = (int)std::min<int64_t>(2, std::max<int64_t>(1, ceil_div(slice_bytes, kRoutedPhaseBytes)));
-  if (slice_bytes > kRoutedPhaseBytes * 4) nsub = 1;
+  int nsub = slice_bytes > kRoutedPhaseBytes ? 2 : 1;
   if (want_sub) nsub = std::min(want_sub, hpspmm::kMaxSub);
 
   // popularity rank s -> slice s % 8, compact-buffer row (s % 8) * h + s / 8

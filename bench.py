@@ -47,7 +47,7 @@ ROOFLINE_WORKLOAD = ("c2_social", 128)
 # counter); summary in profiles/spmm_routed_kernel__c2_social.txt.  Counters cannot be read
 # from inside this process, so the figure is carried here and only reported for the exact
 # configuration it was measured on: (workload, K, strategy) at scale 1.
-MEASURED_TRAFFIC_BYTES = {("c2_social", 128, 4): 31.739e9 + 1.120e9 + 0.07e9}
+MEASURED_TRAFFIC_BYTES = {("c2_social", 128, 4): 1.495e9 + 17.649e9 + 1.870e9}
 
 
 def log(*a):
@@ -215,7 +215,7 @@ def main():
                             if args.scale == 1.0 and args.plan_flags == 0 else None,
                             "kernel": {1: "spmm_rows_kernel<128>",
                                        2: "spmm_segments_kernel<128> + spmm_fixup_kernel<128>",
-                                       4: "routed_gather_hub_kernel<128> + spmm_routed_kernel<128> + "
+                                       4: "routed_prepare_kernel<128> + spmm_routed_kernel<128> + "
                                           "spmm_routed_final_kernel<128>"}.get(info["strategy"], "?")
                                       + " (all launches of one SpMM)",
                             "workload": f"{name} K={k}", "algorithmic_bytes_per_launch": abytes,

@@ -55,7 +55,7 @@ STRATEGY_ROUTED = 4
 EXPORTS = (
     "hpspmm_version", "hpspmm_last_error", "hpspmm_plan_create", "hpspmm_plan_get_info",
     "hpspmm_plan_destroy", "hpspmm_csr_spmm", "hpspmm_csr_spmm_noplan", "hpspmm_coo_spmm_accumulate",
-    "hpspmm_fill_f32", "hpspmm_csr_spmm_timed",
+    "hpspmm_fill_f32", "hpspmm_csr_spmm_timed", "hpspmm_plan_bind_values",
 )
 
 _i64 = ctypes.c_int64
@@ -98,6 +98,7 @@ def lib():
                                          ctypes.POINTER(_p)]
         L.hpspmm_plan_get_info.argtypes = [_p, ctypes.POINTER(PlanInfo)]
         L.hpspmm_plan_destroy.argtypes = [_p]
+        L.hpspmm_plan_bind_values.argtypes = [_p, _p, _p]
         L.hpspmm_csr_spmm.argtypes = [_p, _p, _p, _p, _p, _p, _p]
         L.hpspmm_csr_spmm_noplan.argtypes = [_i64, _i64, _i64, _p, _p, _p, _p, _i64, _p, _p]
         L.hpspmm_coo_spmm_accumulate.argtypes = [_i64, _i64, _i64, _p, _p, _p, _p, _i64, _p, _p]
@@ -153,6 +154,15 @@ class Plan:
         out = PlanInfo()
         check(lib().hpspmm_plan_get_info(self._h, ctypes.byref(out)))
         return out.as_dict()
+
+    def bind_values(self, val, stream=None):
+        """hpspmm_plan_bind_values: `val` (or None to unbind) stays unchanged until the next bind."""
+        import torch
+        if val is not None:
+            _dev(val, torch.float32, "val")
+            if val.numel() != self.nnz:
+                raise ValueError("val must have nnz entries")
+        check(lib().hpspmm_plan_bind_values(self._h, _ptr(val) if val is not None else None, _stream(stream)))
 
     def destroy(self):
         if getattr(self, "_h", None):

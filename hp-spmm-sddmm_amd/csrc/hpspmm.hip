@@ -96,6 +96,7 @@ struct hpspmm_plan {
   float* d_partial = nullptr;     // [n_routed * nhub * k]
   int64_t n_bhot = 0;
   int64_t routed_grid = 0;
+  const float* bound_val = nullptr;  // value array whose class-major copy d_vval currently holds (or NULL)
   int32_t* d_long_rows = nullptr;  // rows strategy: rows longer than long_threshold
   int64_t n_long = 0;
   int32_t long_threshold = INT32_MAX;
@@ -458,12 +459,15 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
 
 template <int K>
 int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
+  // values bound to the plan are already in class-major order: only the hub rows of B are refreshed
+  const int64_t permute_nnz = (p->bound_val && p->bound_val == v) ? 0 : p->nnz;
   const int64_t gather_blocks = ceil_div(p->n_bhot * (K / 4), hpspmm::kBlock);
-  const int64_t prep_blocks = gather_blocks + ceil_div(p->nnz, hpspmm::kBlock * hpspmm::kPermutePerThread);
+  const int64_t prep_blocks = gather_blocks + ceil_div(permute_nnz, hpspmm::kBlock * hpspmm::kPermutePerThread);
   if (prep_blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
-  hipLaunchKernelGGL(hpspmm::routed_prepare_kernel<K>, dim3((unsigned)prep_blocks), dim3(hpspmm::kBlock), 0, st,
-                     p->n_bhot, gather_blocks, p->d_bhot_src, B, p->d_bhot, p->nnz, v, p->d_vpos, p->d_vval,
-                     aligned16(v, v, v));
+  if (prep_blocks > 0)
+    hipLaunchKernelGGL(hpspmm::routed_prepare_kernel<K>, dim3((unsigned)prep_blocks), dim3(hpspmm::kBlock), 0, st,
+                       p->n_bhot, gather_blocks, p->d_bhot_src, B, p->d_bhot, permute_nnz, v, p->d_vpos, p->d_vval,
+                       aligned16(v, v, v));
   if (p->routed_grid > 0)
     hipLaunchKernelGGL(hpspmm::spmm_routed_kernel<K>, dim3((unsigned)p->routed_grid), dim3(hpspmm::kBlock), 0, st,
                        p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval, p->d_vrow, B, p->d_bhot, p->d_partial,
@@ -697,6 +701,24 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
   return HPSPMM_OK;
 }
 
+int hpspmm_plan_bind_values(hpspmm_plan* plan, const float* d_val, void* stream) {
+  if (!plan) return fail(HPSPMM_ERR_INVALID_ARG, "plan is NULL");
+  plan->bound_val = nullptr;
+  if (!d_val || plan->nnz == 0) return HPSPMM_OK;
+  if (plan->strategy == HPSPMM_STRATEGY_ROUTED) {
+    hipStream_t st = (hipStream_t)stream;
+    // the value half of routed_prepare_kernel alone (its template argument only shapes the other half)
+    const int64_t blocks = ceil_div(plan->nnz, hpspmm::kBlock * hpspmm::kPermutePerThread);
+    if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+    hipLaunchKernelGGL(hpspmm::routed_prepare_kernel<32>, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st,
+                       (int64_t)0, (int64_t)0, (const int32_t*)nullptr, (const float*)nullptr, (float*)nullptr,
+                       plan->nnz, d_val, plan->d_vpos, plan->d_vval, aligned16(d_val, d_val, d_val));
+    HPSPMM_HIP(hipGetLastError());
+  }
+  plan->bound_val = d_val;
+  return HPSPMM_OK;
+}
+
 int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d_col, const float* d_val,
                     const float* d_B, float* d_C, void* stream) {
   if (!plan) return fail(HPSPMM_ERR_INVALID_ARG, "plan is NULL");
@@ -706,6 +728,8 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
     return fail(HPSPMM_ERR_INVALID_ARG, "d_col, d_val or d_B is NULL with nnz > 0");
   hipStream_t st = (hipStream_t)stream;
   int rc;
+  // another value array overwrites the plan's copy of the bound one
+  if (plan->bound_val && plan->bound_val != d_val) plan->bound_val = nullptr;
   if (plan->strategy == HPSPMM_STRATEGY_ROUTED) {
     switch (plan->k) {
       case 32: rc = launch_routed<32>(plan, d_val, d_B, d_C, st); break;

@@ -11,7 +11,10 @@
 // arguments, C overwritten.  Builds a plan (untimed, like the reference's host
 // preprocessing), runs WARMUP_NUM_CUDA + EXE_NUM_CUDA launches, frees the plan.
 void GESpMM(const CSR_Matrix& mat1, const Matrix& mat2, Matrix& result, float& time);
-// The same operation under the name of this library's own method.
+// The same operation under the name of this library's own method, with the
+// values bound to the plan before the timed loop: the reference's HP-SpMM also
+// lays its values out during preprocessing (spmm/mm/spmm_common.cpp:269-277),
+// while GESpMM above is handed the CSR arrays as they are on every launch.
 void HPSpMM(const CSR_Matrix& mat1, const Matrix& mat2, Matrix& result, float& time);
 // C += A * B for COO A, EXE_NUM_CUDA launches without re-zeroing, i.e. C ends up
 // as C0 + EXE_NUM_CUDA * A * B exactly like LBSpMM (spmm_kernel.cu:733-768).

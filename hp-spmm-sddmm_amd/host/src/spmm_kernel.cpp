@@ -32,7 +32,8 @@ void check_status(int rc, const char* who) {
   if (rc != HPSPMM_OK) throw Error(std::string(who) + ": " + hpspmm_last_error());
 }
 
-void csr_spmm_timed(const CSR_Matrix& a, const Matrix& mat2, Matrix& result, float& time, const char* who) {
+void csr_spmm_timed(const CSR_Matrix& a, const Matrix& mat2, Matrix& result, float& time, const char* who,
+                    bool bind_values) {
   const Matrix rp = a.row_offsets(), ci = a.column_indices(), va = a.values();
   if (rp.size() != a.num_rows() + 1) throw Error(std::string(who) + ": row_offsets must have num_rows + 1 entries");
   const Dims d = check_operands(a.num_rows(), a.num_cols(), rp, ci, va, mat2, result, who);
@@ -40,6 +41,13 @@ void csr_spmm_timed(const CSR_Matrix& a, const Matrix& mat2, Matrix& result, flo
   check_status(hpspmm_plan_create(d.m, d.n, d.nnz, rp.data<int32_t>(), ci.data<int32_t>(), d.k, HPSPMM_PLAN_DEFAULT,
                                   nullptr, &plan),
                who);
+  if (bind_values) {
+    const int rb = hpspmm_plan_bind_values(plan, va.data<float>(), nullptr);
+    if (rb != HPSPMM_OK) {
+      hpspmm_plan_destroy(plan);
+      check_status(rb, who);
+    }
+  }
   const int rc = hpspmm_csr_spmm_timed(plan, rp.data<int32_t>(), ci.data<int32_t>(), va.data<float>(),
                                        mat2.data<float>(), result.mutable_data<float>(), nullptr, WARMUP_NUM_CUDA,
                                        EXE_NUM_CUDA, &time);
@@ -51,11 +59,11 @@ void csr_spmm_timed(const CSR_Matrix& a, const Matrix& mat2, Matrix& result, flo
 }  // namespace
 
 void GESpMM(const CSR_Matrix& mat1, const Matrix& mat2, Matrix& result, float& time) {
-  csr_spmm_timed(mat1, mat2, result, time, "GESpMM");
+  csr_spmm_timed(mat1, mat2, result, time, "GESpMM", false);
 }
 
 void HPSpMM(const CSR_Matrix& mat1, const Matrix& mat2, Matrix& result, float& time) {
-  csr_spmm_timed(mat1, mat2, result, time, "HPSpMM");
+  csr_spmm_timed(mat1, mat2, result, time, "HPSpMM", true);
 }
 
 void LBSpMM(const COO_Matrix& mat1, const Matrix& mat2, Matrix& result, float& time) {

@@ -115,6 +115,22 @@ int hpspmm_plan_get_info(const hpspmm_plan *plan, hpspmm_plan_info *info_out);
 int hpspmm_plan_destroy(hpspmm_plan *plan);
 
 /*
+ * Optional: declare that the nnz values at d_val will not change until the
+ * next call of this function (or the destruction of the plan).  Strategies
+ * that keep the nonzeros in an order of their own then bring the values into
+ * that order once, here, instead of at the start of every SpMM; later
+ * hpspmm_csr_spmm calls that pass this same d_val use the stored copy; a call
+ * with any other pointer works as if nothing was bound and drops the binding.
+ * d_val = NULL unbinds.
+ * This is where the reference's HP-SpMM does the same work: its preprocessing
+ * emits the values in its own processing order before the timed loop
+ * (spmm/mm/spmm_common.cpp:269-277, test/test_all.cpp:38-40).  A caller that
+ * overwrites the array in place must bind again (or unbind); otherwise SpMM
+ * keeps using the values it copied.  Asynchronous on `stream`.
+ */
+int hpspmm_plan_bind_values(hpspmm_plan *plan, const float *d_val, void *stream);
+
+/*
  * C = A * B with a plan.  One call = one SpMM = the body of one iteration of
  * the reference's launch loop in GESpMM (spmm/mm/spmm_kernel.cu:405-422) /
  * one cusparseSpMM call (spmm/mm/spmm_kernel.cu:129-141).  C need not be

@@ -429,3 +429,35 @@ def test_unaligned_arrays_and_new_values_per_call(pkg, oracle, gpu):
             capi.csr_spmm(plan, rp, ci, v2, Bd, C)
             _check(oracle, g2, B, C.cpu().numpy(), f"unaligned, new values k={k} {name}")
             plan.destroy()
+
+
+def test_bound_values(pkg, oracle, gpu):
+    """hpspmm_plan_bind_values: same bits as the unbound call, another pointer drops the binding,
+    binding again picks up values changed in place."""
+    import torch
+    capi = pkg.capi
+    g = pkg.graphs.make_graph("c4_rmat", 0.004)
+    k = 64
+    B = pkg.graphs.make_dense("c4_rmat", g.cols, k)
+    val2 = (g.val * np.float32(0.75) - np.float32(0.125)).astype(np.float32)
+    g2 = pkg.graphs.CSR(g.rows, g.cols, g.rowptr, g.col, val2)
+    rp, ci, v, vb, Bd = _to_dev(gpu, g.rowptr, g.col, g.val, val2, B)
+    for name, flags in _strategies(capi):
+        plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
+        run = lambda vals: (lambda C: (capi.csr_spmm(plan, rp, ci, vals, Bd, C), C.cpu().numpy())[1])(
+            torch.full((g.rows, k), float("nan"), device=gpu))
+        unbound = run(v)
+        plan.bind_values(v)
+        assert np.array_equal(run(v), unbound), f"{name}: bound result differs from the unbound one"
+        assert np.array_equal(run(v), unbound), f"{name}: second bound call differs"
+        other = run(vb)                      # another array: used as given, binding dropped
+        _check(oracle, g2, B, other, f"bound, other pointer {name}")
+        assert np.array_equal(run(v), unbound), f"{name}: first array after the binding was dropped"
+        plan.bind_values(v)
+        v.copy_(vb)                          # changed in place ...
+        plan.bind_values(v)                  # ... and bound again
+        assert np.array_equal(run(v), other), f"{name}: binding again must pick up the new values"
+        plan.bind_values(None)
+        assert np.array_equal(run(v), other), f"{name}: unbound call after unbinding"
+        v.copy_(torch.from_numpy(g.val).to(gpu))
+        plan.destroy()

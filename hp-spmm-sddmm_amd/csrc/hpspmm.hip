@@ -85,7 +85,9 @@ struct hpspmm_plan {
   int32_t* d_rvptr = nullptr;     // [(n_routed + 1) * nhub] run starts of the routed rows in the hub classes
   int32_t* d_coldptr = nullptr;   // [rows + 1] run starts in the cold class
   int32_t* d_vcol = nullptr;      // [vtotal] column, or ~compact-buffer row
-  int32_t* d_vpos = nullptr;      // [nnz] position of every stored nonzero in the class-major order
+  uint16_t* d_lslot = nullptr;    // [nnz] rank of every stored nonzero within its chunk sorted by class-major position
+  int32_t* d_chunk_base = nullptr;  // [nchunks * ncls] first class-major position of the chunk's run in each class
+  int32_t* d_chunk_pref = nullptr;  // [nchunks * ncls] nonzeros of the chunk in lower classes
   float* d_vval = nullptr;        // [vtotal] the values in that order, rewritten by every SpMM
   int32_t* d_vrow = nullptr;      // [vtotal] routed-row number (hub classes) or row (cold class)
   int32_t* d_bhot_src = nullptr;  // [n_bhot] source column of every compact-buffer row (-1 = unused)
@@ -265,12 +267,12 @@ int exclusive_scan_u32(const uint32_t* d_in, uint32_t* d_out, int64_t n, hipStre
 // Rows of B kept in the compact buffer by the routed strategy (all slices together).
 constexpr int kRoutedLog2Cached = 16;
 // Automatic choice of the routed strategy (thresholds from measurements on the
-// benchmark graphs: it pays on the 233k-vertex social graph at K = 64 and 128
-// (2.95 -> 2.31 ms, 6.6 -> 4.5 ms) and on the R-MAT graph (8.6 -> 7.9 ms); not at
-// K = 32 on the social graph, where B already fits the L2s, and not on the
-// co-purchase graph, whose columns are too evenly used (4.5 -> 5.5 ms)).
+// benchmark graphs: it pays on the 233k-vertex social graph at K = 32, 64 and
+// 128 (1.34 -> 1.25 ms, 2.95 -> 2.05 ms, 6.6 -> 3.9 ms) and on the R-MAT graph
+// (8.6 -> 6.1 ms); not on the co-purchase graph, whose columns are too evenly
+// used (4.5 -> 5.5 ms)).
 constexpr int64_t kRoutedMinNnz = (int64_t)1 << 22;
-constexpr int64_t kRoutedMinBBytes = (int64_t)48 << 20;  // B must overflow the 8 x 4 MB of L2
+constexpr int64_t kRoutedMinBBytes = (int64_t)24 << 20;  // a B that one or two L2s hold needs no routing
 constexpr double kRoutedMinShare = 0.35;     // of the nonzeros in the 64k most referenced columns
 constexpr double kRoutedMinRowNnz = 32.0;    // mean nonzeros per non-empty row
 constexpr int32_t kRoutedRowThreshold = 128;  // rows shorter than this are not split over the classes
@@ -324,14 +326,15 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   uint32_t* d_coldcnt = nullptr;  // [rows + 1] cold-class count per row, then its scan
   uint8_t* d_action = nullptr;    // [rows]
   int32_t* d_counts = nullptr;    // [2] list lengths
+  int32_t* d_vpos = nullptr;      // [nnz] position of every stored nonzero in the class-major order
   struct Guard {
-    void** q[6];
+    void** q[7];
     ~Guard() {
       for (void** x : q)
         if (*x) (void)hipFree(*x);
     }
   } guard{{(void**)&d_colmap, (void**)&d_ridx, (void**)&d_cnt, (void**)&d_coldcnt, (void**)&d_action,
-           (void**)&d_counts}};
+           (void**)&d_counts, (void**)&d_vpos}};
   HPSPMM_HIP(hipMalloc(&d_colmap, (size_t)std::max<int64_t>(1, p->cols) * sizeof(int32_t)));
   HPSPMM_HIP(hipMalloc(&d_ridx, (size_t)(rows + 1) * sizeof(uint32_t)));
   HPSPMM_HIP(hipMalloc(&d_coldcnt, (size_t)(rows + 1) * sizeof(uint32_t)));
@@ -402,6 +405,9 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   const size_t coldptr_bytes = (size_t)(rows + 1) * sizeof(int32_t);
   const size_t v_bytes = (size_t)vtotal * sizeof(int32_t);
   const size_t vpos_bytes = (size_t)std::max<int64_t>(nnz, 1) * sizeof(int32_t);
+  const int64_t nchunks = ceil_div(nnz, hpspmm::kPermChunk);
+  const size_t lslot_bytes = (size_t)std::max<int64_t>(nnz, 1) * sizeof(uint16_t);
+  const size_t chunk_bytes = (size_t)std::max<int64_t>(nchunks, 1) * (size_t)(nhub + 1) * sizeof(int32_t);
   const size_t partial_bytes = (size_t)std::max<int64_t>(n_routed, 1) * (size_t)nhub * (size_t)k * sizeof(float);
   const size_t carry_bytes = (size_t)std::max<int64_t>(nseg, 1) * 2 * (size_t)k * sizeof(float);
   const size_t bhot_bytes = (size_t)n_bhot * (size_t)k * sizeof(float);
@@ -410,11 +416,14 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   // the segments strategy's buffers are not needed any more
   if (p->d_nnz_row) { (void)hipFree(p->d_nnz_row); p->d_nnz_row = nullptr; }
   if (p->d_carry) { (void)hipFree(p->d_carry); p->d_carry = nullptr; }
-  const size_t total_bytes = rvptr_bytes + coldptr_bytes + 3 * v_bytes + vpos_bytes + partial_bytes + carry_bytes +
-                             bhot_bytes + (size_t)n_bhot * 4 + 2 * list_bytes + routed_rows_bytes;
+  const size_t total_bytes = rvptr_bytes + coldptr_bytes + 3 * v_bytes + lslot_bytes + 2 * chunk_bytes +
+                             partial_bytes + carry_bytes + bhot_bytes + (size_t)n_bhot * 4 + 2 * list_bytes +
+                             routed_rows_bytes;
   if (hipMalloc(&p->d_rvptr, rvptr_bytes) != hipSuccess || hipMalloc(&p->d_coldptr, coldptr_bytes) != hipSuccess ||
       hipMalloc(&p->d_vcol, v_bytes) != hipSuccess || hipMalloc(&p->d_vval, v_bytes) != hipSuccess ||
-      hipMalloc(&p->d_vrow, v_bytes) != hipSuccess || hipMalloc(&p->d_vpos, vpos_bytes) != hipSuccess ||
+      hipMalloc(&p->d_vrow, v_bytes) != hipSuccess || hipMalloc(&d_vpos, vpos_bytes) != hipSuccess ||
+      hipMalloc(&p->d_lslot, lslot_bytes) != hipSuccess || hipMalloc(&p->d_chunk_base, chunk_bytes) != hipSuccess ||
+      hipMalloc(&p->d_chunk_pref, chunk_bytes) != hipSuccess ||
       hipMalloc(&p->d_partial, partial_bytes) != hipSuccess || hipMalloc(&p->d_carry, carry_bytes) != hipSuccess ||
       hipMalloc(&p->d_bhot, bhot_bytes) != hipSuccess ||
       hipMalloc(&p->d_bhot_src, (size_t)n_bhot * sizeof(int32_t)) != hipSuccess ||
@@ -436,8 +445,12 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   hipLaunchKernelGGL(hpspmm::routed_coldptr_kernel, dim3((unsigned)ceil_div(rows + 1, hpspmm::kBlock)),
                      dim3(hpspmm::kBlock), 0, st, rows, lay.cls_begin[nhub], d_coldcnt, p->d_coldptr);
   hipLaunchKernelGGL(hpspmm::routed_fill_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col,
-                     d_colmap, d_ridx, (int32_t)h, nsub, min_row_nnz, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vpos,
+                     d_colmap, d_ridx, (int32_t)h, nsub, min_row_nnz, p->d_rvptr, p->d_coldptr, p->d_vcol, d_vpos,
                      p->d_vrow, p->d_routed_rows, d_action, p->shift);
+  // chunk tables of the value scatter
+  if (nchunks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  hipLaunchKernelGGL(hpspmm::routed_chunk_kernel, dim3((unsigned)nchunks), dim3(hpspmm::kBlock), 0, st, lay, nnz, d_vpos,
+                     p->d_lslot, p->d_chunk_base, p->d_chunk_pref);
   // compact lists of the short rows the final kernel has to visit
   const unsigned cgrid = (unsigned)ceil_div(rows, hpspmm::kBlock);
   hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(cgrid), dim3(hpspmm::kBlock), 0, st, rows, d_action,
@@ -462,12 +475,12 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
   // values bound to the plan are already in class-major order: only the hub rows of B are refreshed
   const int64_t permute_nnz = (p->bound_val && p->bound_val == v) ? 0 : p->nnz;
   const int64_t gather_blocks = ceil_div(p->n_bhot * (K / 4), hpspmm::kBlock);
-  const int64_t prep_blocks = gather_blocks + ceil_div(permute_nnz, hpspmm::kBlock * hpspmm::kPermutePerThread);
+  const int64_t prep_blocks = gather_blocks + ceil_div(permute_nnz, hpspmm::kPermChunk);
   if (prep_blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   if (prep_blocks > 0)
     hipLaunchKernelGGL(hpspmm::routed_prepare_kernel<K>, dim3((unsigned)prep_blocks), dim3(hpspmm::kBlock), 0, st,
-                       p->n_bhot, gather_blocks, p->d_bhot_src, B, p->d_bhot, permute_nnz, v, p->d_vpos, p->d_vval,
-                       aligned16(v, v, v));
+                       p->n_bhot, gather_blocks, p->d_bhot_src, B, p->d_bhot, p->nnz, p->lay.nhub + 1, v, p->d_lslot,
+                       p->d_chunk_base, p->d_chunk_pref, p->d_vval);
   if (p->routed_grid > 0)
     hipLaunchKernelGGL(hpspmm::spmm_routed_kernel<K>, dim3((unsigned)p->routed_grid), dim3(hpspmm::kBlock), 0, st,
                        p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval, p->d_vrow, B, p->d_bhot, p->d_partial,
@@ -693,7 +706,8 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
   if (plan->d_hub_ids) (void)hipFree(plan->d_hub_ids);
   if (plan->d_hub_col) (void)hipFree(plan->d_hub_col);
   if (plan->d_bhot) (void)hipFree(plan->d_bhot);
-  for (void* q : {(void*)plan->d_rvptr, (void*)plan->d_coldptr, (void*)plan->d_vcol, (void*)plan->d_vpos,
+  for (void* q : {(void*)plan->d_rvptr, (void*)plan->d_coldptr, (void*)plan->d_vcol, (void*)plan->d_lslot,
+                  (void*)plan->d_chunk_base, (void*)plan->d_chunk_pref,
                   (void*)plan->d_vval, (void*)plan->d_vrow, (void*)plan->d_bhot_src, (void*)plan->d_partial,
                   (void*)plan->d_routed_rows, (void*)plan->d_cross_rows, (void*)plan->d_zero_rows})
     if (q) (void)hipFree(q);
@@ -708,11 +722,12 @@ int hpspmm_plan_bind_values(hpspmm_plan* plan, const float* d_val, void* stream)
   if (plan->strategy == HPSPMM_STRATEGY_ROUTED) {
     hipStream_t st = (hipStream_t)stream;
     // the value half of routed_prepare_kernel alone (its template argument only shapes the other half)
-    const int64_t blocks = ceil_div(plan->nnz, hpspmm::kBlock * hpspmm::kPermutePerThread);
+    const int64_t blocks = ceil_div(plan->nnz, hpspmm::kPermChunk);
     if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
     hipLaunchKernelGGL(hpspmm::routed_prepare_kernel<32>, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st,
                        (int64_t)0, (int64_t)0, (const int32_t*)nullptr, (const float*)nullptr, (float*)nullptr,
-                       plan->nnz, d_val, plan->d_vpos, plan->d_vval, aligned16(d_val, d_val, d_val));
+                       plan->nnz, plan->lay.nhub + 1, d_val, plan->d_lslot, plan->d_chunk_base, plan->d_chunk_pref,
+                       plan->d_vval);
     HPSPMM_HIP(hipGetLastError());
   }
   plan->bound_val = d_val;

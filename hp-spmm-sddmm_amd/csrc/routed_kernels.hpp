@@ -309,22 +309,88 @@ __global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const
   }
 }
 
+// Chunk tables for the value scatter.  The stored nonzeros are cut into chunks
+// of kPermChunk consecutive ones.  Inside a chunk the nonzeros of one class
+// occupy consecutive positions of the class-major order (both orders keep the
+// stored order within a class), so a chunk maps to at most one run per class:
+// chunk_base[c * ncls + x] = first position of class x's run, chunk_pref[c *
+// ncls + x] = number of the chunk's nonzeros in classes < x, and lslot[j] =
+// chunk_pref + (position - chunk_base) = rank of nonzero j when its chunk is
+// sorted by position.  One workgroup per chunk.
+constexpr int kPermChunk = 4096;
+
+__global__ __launch_bounds__(kBlock) void routed_chunk_kernel(RoutedLayout lay, int64_t nnz,
+                                                              const int32_t* __restrict__ vpos,
+                                                              uint16_t* __restrict__ lslot,
+                                                              int32_t* __restrict__ chunk_base,
+                                                              int32_t* __restrict__ chunk_pref) {
+  __shared__ int32_t s_min[kMaxClasses];
+  __shared__ int32_t s_cnt[kMaxClasses];
+  __shared__ int32_t s_pref[kMaxClasses];
+  const int ncls = lay.nhub + 1;
+  const int64_t j0 = (int64_t)blockIdx.x * kPermChunk;
+  for (int x = threadIdx.x; x < ncls; x += kBlock) {
+    s_min[x] = INT32_MAX;
+    s_cnt[x] = 0;
+  }
+  __syncthreads();
+  auto class_of_position = [&](int32_t p) {
+    int x = 0;
+    while (x + 1 < ncls && (int64_t)p >= lay.cls_begin[x + 1]) ++x;
+    return x;
+  };
+  for (int i = threadIdx.x; i < kPermChunk; i += kBlock) {
+    const int64_t j = j0 + i;
+    if (j >= nnz) break;
+    const int32_t p = vpos[j];
+    const int x = class_of_position(p);
+    atomicMin(&s_min[x], p);
+    atomicAdd(&s_cnt[x], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t run = 0;
+    for (int x = 0; x < ncls; ++x) {
+      s_pref[x] = run;
+      run += s_cnt[x];
+    }
+  }
+  __syncthreads();
+  for (int x = threadIdx.x; x < ncls; x += kBlock) {
+    chunk_base[(int64_t)blockIdx.x * ncls + x] = s_cnt[x] ? s_min[x] : 0;
+    chunk_pref[(int64_t)blockIdx.x * ncls + x] = s_pref[x];
+  }
+  for (int i = threadIdx.x; i < kPermChunk; i += kBlock) {
+    const int64_t j = j0 + i;
+    if (j >= nnz) break;
+    const int32_t p = vpos[j];
+    const int x = class_of_position(p);
+    lslot[j] = (uint16_t)(s_pref[x] + (p - s_min[x]));
+  }
+}
+
 // Start of every SpMM, two jobs in one launch.  Workgroups [0, gather_blocks):
 // Bhot[s, :] = B[src[s], :] for every compact-buffer row with a source column
-// (src[s] >= 0).  The others: vval[vpos[j]] = val[j], the caller's values
-// brought into the plan's class-major order by a scatter in stored order (a
-// gather in class order would fetch every line of val once per class).
-constexpr int kPermutePerThread = 4;
-
+// (src[s] >= 0).  The others, one per chunk of kPermChunk stored nonzeros:
+// the caller's values are brought into the plan's class-major order.  A gather
+// in class order would fetch every line of val once per class, a scatter of
+// single values costs one L2 transaction for every two or three of them; so
+// the chunk is sorted by destination in LDS (lslot) and written out run by
+// run in full lines (233k-vertex social graph: 0.28 ms for the plain scatter).
 template <int K>
 __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, int64_t gather_blocks,
                                                                 const int32_t* __restrict__ src,
                                                                 const float* __restrict__ B,
-                                                                float* __restrict__ Bhot, int64_t nnz,
+                                                                float* __restrict__ Bhot, int64_t nnz, int ncls,
                                                                 const float* __restrict__ val,
-                                                                const int32_t* __restrict__ vpos,
-                                                                float* __restrict__ vval, bool val_vec_ok) {
+                                                                const uint16_t* __restrict__ lslot,
+                                                                const int32_t* __restrict__ chunk_base,
+                                                                const int32_t* __restrict__ chunk_pref,
+                                                                float* __restrict__ vval) {
   constexpr int G = K / 4;
+  __shared__ float s_buf[kPermChunk];
+  __shared__ int32_t s_base[kMaxClasses];
+  __shared__ int32_t s_pref[kMaxClasses + 1];
   if ((int64_t)blockIdx.x < gather_blocks) {
     const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     const int64_t s = t / G;
@@ -335,19 +401,35 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
     *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) = load_b<K>(B, c, l);
     return;
   }
-  // four consecutive nonzeros per thread (measured against one instruction per
-  // 64 consecutive nonzeros of a wavefront: 0.28 vs 0.31 ms on the social graph)
-  const int64_t j = (((int64_t)blockIdx.x - gather_blocks) * kBlock + threadIdx.x) * kPermutePerThread;
-  if (j >= nnz) return;
-  if (val_vec_ok && j + 4 <= nnz) {
-    const int4 q = *reinterpret_cast<const int4*>(vpos + j);
-    const float4 v = *reinterpret_cast<const float4*>(val + j);
-    vval[q.x] = v.x;
-    vval[q.y] = v.y;
-    vval[q.z] = v.z;
-    vval[q.w] = v.w;
-  } else {
-    for (int64_t i = j; i < j + 4 && i < nnz; ++i) vval[vpos[i]] = val[i];
+  const int64_t chunk = (int64_t)blockIdx.x - gather_blocks;
+  const int64_t j0 = chunk * kPermChunk;
+  const int n = nnz - j0 < kPermChunk ? (int)(nnz - j0) : kPermChunk;
+  for (int x = threadIdx.x; x < ncls; x += kBlock) {
+    s_base[x] = chunk_base[chunk * ncls + x];
+    s_pref[x] = chunk_pref[chunk * ncls + x];
+  }
+  if (threadIdx.x == 0) s_pref[ncls] = n;
+  constexpr int kPer = kPermChunk / kBlock;
+  float v[kPer];
+  uint16_t q[kPer];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int t = i * kBlock + threadIdx.x;
+    v[i] = t < n ? val[j0 + t] : 0.f;
+    q[i] = t < n ? lslot[j0 + t] : (uint16_t)0;
+  }
+#pragma unroll
+  for (int i = 0; i < kPer; ++i)
+    if (i * kBlock + (int)threadIdx.x < n) s_buf[q[i]] = v[i];
+  __syncthreads();
+  // thread t of every pass writes sorted element t: consecutive threads, consecutive addresses within a run
+  int x = 0;
+#pragma unroll 1
+  for (int i = 0; i < kPer; ++i) {
+    const int t = i * kBlock + threadIdx.x;
+    if (t >= n) break;
+    while (s_pref[x + 1] <= t) ++x;  // t grows with i, so the class only moves forward
+    vval[s_base[x] + (t - s_pref[x])] = s_buf[t];
   }
 }
 

@@ -327,7 +327,7 @@ def test_full_size_configs(pkg, oracle, gpu, name, k):
         out[tag] = (C, info)
     expect = {("c2_social", 128): capi.STRATEGY_ROUTED, ("c2_social", 64): capi.STRATEGY_ROUTED,
               ("c4_rmat", 128): capi.STRATEGY_ROUTED, ("c3_copurchase", 64): capi.STRATEGY_SEGMENTS,
-              ("c2_social", 32): capi.STRATEGY_SEGMENTS}[(name, k)]
+              ("c2_social", 32): capi.STRATEGY_ROUTED}[(name, k)]
     assert out["auto"][1]["strategy"] == expect
     # the two strategies sum in different orders: they agree to rounding, scaled by |A| |B|
     plan = capi.Plan(g.rows, g.cols, rp, ci, k, capi.PLAN_FORCE_SEGMENTS | capi.PLAN_NO_HUB_CACHE | capi.PLAN_NO_ROUTED)

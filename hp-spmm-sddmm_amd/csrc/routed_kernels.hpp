@@ -542,13 +542,18 @@ __global__ __launch_bounds__(kBlock) void routed_collect_rows_kernel(int64_t row
 
 // Final pass, one sub-wave per listed row, three parts.
 // Workgroups [0, routed_blocks): routed row number i gets the sum of its class
-// results in class order - per class the partial-result slot if the run lies
-// in one segment, else tail[ga] + head[ga+1] + ... + head[gb] from the carry
-// slots.  With segments of 512 nonzeros and runs of some tens, about one run
-// in eight crosses a segment boundary, i.e. most rows have one: the first two
-// slots of every run are therefore fetched together for a group of classes,
-// and only a run over three or more segments (a hub row) takes the loop over
-// the remaining heads.
+// results - per class the partial-result slot if the run lies in one segment,
+// else tail[ga] + head[ga+1] + ... + head[gb] from the carry slots.  The
+// kernel is a chain of dependent loads per row, so it is built to have few
+// links: the row's 2 * nhub run bounds come in with one coalesced load and are
+// kept in wave-local LDS; then, eight classes at a time, the first slot of
+// every run (partial or tail); then the second slot of the runs that have one
+// (with segments of 512 nonzeros and runs of some tens about one run in eight
+// crosses a segment boundary, i.e. most rows have one); then, for a hub row's
+// runs over three or more segments, the remaining heads.  The order of the
+// additions is therefore: all first slots in class order, all second slots in
+// class order, the remaining heads in class and segment order - fixed by the
+// plan, so results stay bit-reproducible.
 // Workgroups [routed_blocks, routed_blocks + cross_blocks): short rows whose
 // cold-class run crossed a segment boundary, from the carry slots alone.
 // The rest: rows without nonzeros, which get zeros.
@@ -561,14 +566,15 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
     const float* __restrict__ partial, const float* __restrict__ carry, float* __restrict__ C) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
-  constexpr int kGroup = 4;  // classes whose loads are in flight together
+  constexpr int kGroup = kSlices;  // classes whose loads are in flight together; divides nhub
+  __shared__ int32_t s_bounds[kWavesPerBlock * P][2 * kMaxHub];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
   const int shift = lay.shift;
   const int nhub = lay.nhub;
   const float* cbase = carry + 4 * l;
-  const int64_t sub = (int64_t)(tid >> 6) * P + lane / G;  // sub-wave within the workgroup
+  const int sub = (tid >> 6) * P + lane / G;  // sub-wave within the workgroup
 
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   auto add = [&](const float4& t) {
@@ -611,56 +617,57 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
   const int64_t idx = (int64_t)blockIdx.x * (kWavesPerBlock * P) + sub;
   if (idx >= lay.n_routed) return;
   const int64_t row = routed_rows[idx];
-  const int32_t* vlo = rvptr + idx * nhub;
-  const int32_t* vhi = vlo + nhub;
+  // bounds of the row's runs: lo[x] = sb[x], hi[x] = sb[nhub + x] (the next routed row's lo)
+  int32_t* sb = s_bounds[sub];
+  for (int t = l; t < 2 * nhub; t += G) sb[t] = rvptr[idx * nhub + t];
+  wave_lds_fence();
   const float* prow = partial + (uint64_t)idx * nhub * K + 4 * l;
 
-  auto bounds = [&](int x0, int32_t (&lb)[kGroup], int32_t (&hb)[kGroup]) {
-#pragma unroll
-    for (int q = 0; q < kGroup; ++q) {
-      const bool in = x0 + q < nhub;
-      const int x = in ? x0 + q : nhub - 1;
-      lb[q] = vlo[x];
-      hb[q] = in ? vhi[x] : lb[q];
-    }
-  };
-  int32_t nlb[kGroup], nhb[kGroup];
-  bounds(0, nlb, nhb);
+  bool any_two = false, any_longer = false;
   for (int x0 = 0; x0 < nhub; x0 += kGroup) {
-    int32_t lb[kGroup], hb[kGroup];
-    float4 first[kGroup], second[kGroup];
-    bool some[kGroup], two[kGroup];
-    bool longer = false;  // some run of the group covers three or more segments
+    float4 slot[kGroup];
+    bool some[kGroup];
 #pragma unroll
     for (int q = 0; q < kGroup; ++q) {
-      lb[q] = nlb[q];
-      hb[q] = nhb[q];
-      some[q] = lb[q] != hb[q];
-      const int64_t ga = lb[q] >> shift;
-      const int64_t gb = (hb[q] - 1) >> shift;
-      two[q] = some[q] && gb > ga;
-      longer |= some[q] && gb > ga + 1;
-      const float* pa = two[q] ? cbase + (uint64_t)(2 * ga + 1) * K : prow + (uint64_t)(x0 + q) * K;
-      first[q] = make_float4(0.f, 0.f, 0.f, 0.f);
-      second[q] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (some[q]) first[q] = *reinterpret_cast<const float4*>(pa);
-      if (two[q]) second[q] = *reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * (ga + 1)) * K);
+      const int32_t lo = sb[x0 + q], hi = sb[nhub + x0 + q];
+      some[q] = lo != hi;
+      const int64_t ga = lo >> shift;
+      const int64_t gb = (hi - 1) >> shift;
+      const bool two = some[q] && gb > ga;
+      any_two |= two;
+      any_longer |= some[q] && gb > ga + 1;
+      const float* pa = two ? cbase + (uint64_t)(2 * ga + 1) * K : prow + (uint64_t)(x0 + q) * K;
+      slot[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (some[q]) slot[q] = *reinterpret_cast<const float4*>(pa);
     }
-    if (x0 + kGroup < nhub) bounds(x0 + kGroup, nlb, nhb);  // in flight together with the slots above
-    if (!longer) {
+#pragma unroll
+    for (int q = 0; q < kGroup; ++q)
+      if (some[q]) add(slot[q]);
+  }
+  if (any_two) {
+    for (int x0 = 0; x0 < nhub; x0 += kGroup) {
+      float4 slot[kGroup];
+      bool two[kGroup];
 #pragma unroll
       for (int q = 0; q < kGroup; ++q) {
-        if (some[q]) add(first[q]);
-        if (two[q]) add(second[q]);
+        const int32_t lo = sb[x0 + q], hi = sb[nhub + x0 + q];
+        const int64_t ga = lo >> shift;
+        two[q] = lo != hi && ((hi - 1) >> shift) > ga;
+        slot[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (two[q]) slot[q] = *reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * (ga + 1)) * K);
       }
-      continue;
-    }
 #pragma unroll
-    for (int q = 0; q < kGroup; ++q) {
-      if (some[q]) add(first[q]);
-      if (!two[q]) continue;
-      add(second[q]);
-      add_heads((lb[q] >> shift) + 2, (hb[q] - 1) >> shift);
+      for (int q = 0; q < kGroup; ++q)
+        if (two[q]) add(slot[q]);
+    }
+  }
+  if (any_longer) {
+    for (int x = 0; x < nhub; ++x) {
+      const int32_t lo = sb[x], hi = sb[nhub + x];
+      if (lo == hi) continue;
+      const int64_t ga = lo >> shift;
+      const int64_t gb = (hi - 1) >> shift;
+      if (gb > ga + 1) add_heads(ga + 2, gb);
     }
   }
   *reinterpret_cast<float4*>(C + (uint64_t)row * K + 4 * l) = acc;

@@ -49,7 +49,7 @@ ROOFLINE_WORKLOAD = ("c2_social", 128)
 # counter); summary in profiles/spmm_routed_kernel__c2_social.txt.  Counters cannot be read
 # from inside this process, so the figure is carried here and only reported for the exact
 # configuration it was measured on: (workload, K, strategy) at scale 1.
-MEASURED_TRAFFIC_BYTES = {("c2_social", 128, 4): 1.495e9 + 17.649e9 + 1.870e9}
+MEASURED_TRAFFIC_BYTES = {("c2_social", 128, 4): 1.238e9 + 17.641e9 + 1.868e9}
 
 
 def log(*a):
@@ -118,6 +118,9 @@ def main():
     ap.add_argument("--cpu-budget-nnz", type=int, default=0,
                     help="nonzeros in the CPU-baseline row sample (0 = the whole social graph)")
     ap.add_argument("--plan-flags", type=int, default=0)
+    ap.add_argument("--no-values-bound", action="store_true",
+                    help="skip the additional timing with hpspmm_plan_bind_values (keeps a profile of this "
+                         "run to the launches of the figure of merit)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three 1 GiB device-to-device copies (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -199,9 +202,11 @@ def main():
             ms, wall_ms = timed(args.warmup, args.steps)
             # for information: values declared constant once (hpspmm_plan_bind_values), which is how
             # the reference's HP-SpMM is timed (values laid out during its preprocessing)
-            plan.bind_values(d_v, stream)
-            ms_bound, _ = timed(min(args.warmup, 3), args.steps)
-            plan.bind_values(None, stream)
+            ms_bound = ms
+            if not args.no_values_bound:
+                plan.bind_values(d_v, stream)
+                ms_bound, _ = timed(min(args.warmup, 3), args.steps)
+                plan.bind_values(None, stream)
             gflops = 2.0 * g.nnz * k / (ms * 1e-3) / 1e9
             abytes = algorithmic_bytes(g.rows, g.nnz, k)
             gbs = abytes / (ms * 1e-3) / 1e9

@@ -567,7 +567,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
   constexpr int kGroup = kSlices;  // classes whose loads are in flight together; divides nhub
-  __shared__ int32_t s_bounds[kWavesPerBlock * P][2 * kMaxHub];
+  __shared__ int32_t s_bounds[kWavesPerBlock * P][2 * kMaxHub + 1];  // odd stride: sub-waves on different banks
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;

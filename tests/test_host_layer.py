@@ -50,7 +50,7 @@ def test_driver_on_smtx_with_reorder(pkg, gpu, tmp_path, k):
     out = subprocess.run([_exe(pkg, "spmm_test_all"), str(smtx), str(tmp_path / "g.reorder"), str(k),
                           "--check", "--csv", str(csv)], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-3000:]
-    assert out.stdout.count("PASSed!!") == 2, out.stdout[-3000:]
+    assert out.stdout.count("PASSed!!") == 3, out.stdout[-3000:]
     line = csv.read_text().strip().splitlines()[-1]
     assert line.startswith(f"{smtx},{g.rows},{g.cols},{g.nnz},{k},")
     assert "GE-SpMM: ," in line and "HP-SpMM ," in line
@@ -64,5 +64,5 @@ def test_driver_on_synthetic(pkg, gpu, tmp_path):
     out = subprocess.run([_exe(pkg, "spmm_test_all"), "--synthetic", "c1_citation", "1.0", "64", "--check",
                           "--csv", str(csv)], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-3000:]
-    assert out.stdout.count("PASSed!!") == 2
+    assert out.stdout.count("PASSed!!") == 3
     assert csv.read_text().startswith("c1_citation@1.0,20000,20000,101878,64,")

@@ -500,7 +500,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
     float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
                               : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : out + (uint64_t)(uint32_t)cur * ostride);
     head_pending = false;
-    *reinterpret_cast<float4*>(dst + 4 * l) = acc;
+    store_result(dst + 4 * l, acc);
   };
   auto flush = [&]() { flush_to(false); };
   auto loadb = [&](int32_t c) { return load_b_hub<K, true>(B, Bhot, c, l); };

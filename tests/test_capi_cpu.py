@@ -80,3 +80,15 @@ def test_product_does_not_import_the_oracle(pkg):
             if f.endswith((".py", ".cpp", ".hip", ".hpp", ".h")):
                 text = open(os.path.join(dirpath, f), errors="replace").read()
                 assert "oracle" not in text.lower(), f"{f} mentions the oracle"
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU and says so instead of producing a figure for several."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                         capture_output=True, text=True, timeout=120)
+    assert out.returncode != 0
+    assert "one GPU" in out.stderr and out.stdout.strip() == ""

@@ -135,7 +135,9 @@ int hpspmm_plan_bind_values(hpspmm_plan *plan, const float *d_val, void *stream)
  * the reference's launch loop in GESpMM (spmm/mm/spmm_kernel.cu:405-422) /
  * one cusparseSpMM call (spmm/mm/spmm_kernel.cu:129-141).  C need not be
  * zeroed beforehand; every element of C, empty rows included, is written.
- * The result is deterministic (no atomics).
+ * The result is deterministic (no atomics).  The call only launches kernels (no
+ * allocation, no memset, no host synchronisation), so it may be captured in a
+ * HIP graph; a replay reads d_val and d_B as they are then.
  */
 int hpspmm_csr_spmm(hpspmm_plan *plan, const int32_t *d_rowptr, const int32_t *d_col,
                     const float *d_val, const float *d_B, float *d_C, void *stream);

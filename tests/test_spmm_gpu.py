@@ -461,3 +461,38 @@ def test_bound_values(pkg, oracle, gpu):
         assert np.array_equal(run(v), other), f"{name}: unbound call after unbinding"
         v.copy_(torch.from_numpy(g.val).to(gpu))
         plan.destroy()
+
+
+def test_hip_graph_capture_and_replay(pkg, oracle, gpu):
+    """One SpMM is kernel launches only (no allocation, no memset, no host synchronisation), so it can
+    be captured in a HIP graph; every replay must see the current contents of val and B."""
+    import torch
+    capi = pkg.capi
+    g = pkg.graphs.make_graph("c4_rmat", 0.004)
+    k = 64
+    B = pkg.graphs.make_dense("c4_rmat", g.cols, k)
+    rp, ci, v, Bd = _to_dev(gpu, g.rowptr, g.col, g.val, B)
+    for name, flags in _strategies(capi):
+        plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
+        C = torch.full((g.rows, k), float("nan"), device=gpu)
+        eager = torch.empty_like(C)
+        capi.csr_spmm(plan, rp, ci, v, Bd, eager)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                capi.csr_spmm(plan, rp, ci, v, Bd, C, side)
+        torch.cuda.current_stream().wait_stream(side)
+        for scale in (1.0, -0.5, 2.0):
+            v.copy_(torch.from_numpy(g.val).to(gpu) * scale)
+            capi.csr_spmm(plan, rp, ci, v, Bd, eager)      # the program's own eager work between replays
+            torch.cuda.synchronize()
+            C.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(C, eager), f"{name}: replay with values x{scale} differs from the eager call"
+        v.copy_(torch.from_numpy(g.val).to(gpu))
+        del graph
+        plan.destroy()

@@ -496,3 +496,30 @@ def test_hip_graph_capture_and_replay(pkg, oracle, gpu):
         v.copy_(torch.from_numpy(g.val).to(gpu))
         del graph
         plan.destroy()
+
+
+def test_auto_strategy_leaves_short_rows_unrouted(pkg, oracle, gpu):
+    """Popular columns but no long rows: routing would move nothing, so the plan must stay with the
+    segments strategy; forced routing of the same matrix still gives the right result."""
+    import torch
+    capi = pkg.capi
+    rng = np.random.default_rng(77)
+    rows, cols, per_row, k = 120_000, 150_000, 40, 64
+    pop = rng.zipf(1.6, size=rows * per_row) % cols               # heavy-tailed column popularity
+    col = np.sort(pop.reshape(rows, per_row), axis=1).astype(np.int32).ravel()
+    rowptr = (np.arange(rows + 1, dtype=np.int64) * per_row).astype(np.int32)
+    val = rng.uniform(-1, 1, col.size).astype(np.float32)
+    g = pkg.graphs.CSR(rows, cols, rowptr, col, val)
+    B = rng.standard_normal((cols, k)).astype(np.float32)
+    C, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+    assert info["strategy"] == capi.STRATEGY_SEGMENTS
+    lo, hi = 50_000, 54_000
+    C64, S64 = oracle.csr_spmm_f64_rows(g.rowptr, g.col, g.val, B, lo, hi)
+    err, _ = oracle.max_norm_err(C[lo:hi], C64, S64)
+    assert err <= TOL
+    Cr, info_r = _run(pkg, gpu, g, B, capi.PLAN_FORCE_ROUTED)
+    assert info_r["strategy"] == capi.STRATEGY_ROUTED
+    err, _ = oracle.max_norm_err(Cr[lo:hi], C64, S64)
+    assert err <= TOL
+    # the two strategies add every row's products in the same (stored) order here: no row is routed
+    assert np.array_equal(C, Cr)

@@ -197,8 +197,10 @@ int launch_coo(int64_t nnz, const int32_t* ri, const int32_t* ci, const float* v
                hipStream_t st) {
   constexpr int P = 64 / (K / 4);
   // 64 nonzeros per sub-wave: short enough to balance, long enough that the
-  // one flush per segment end is amortised
-  const int shift = 6;
+  // one flush per segment end is amortised; shorter segments when that would
+  // leave most of the 1024 SIMDs without a wavefront
+  int shift = 6;
+  while (shift > 4 && (nnz >> shift) / P < 4096) --shift;
   const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
   const int64_t nblocks = ceil_div(ceil_div(nseg, P), hpspmm::kWavesPerBlock);
   if (nblocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");

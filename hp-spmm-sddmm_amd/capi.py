@@ -28,6 +28,8 @@ PLAN_HUB_CACHE = 16
 PLAN_NO_HUB_CACHE = 32
 PLAN_FORCE_ROUTED = 64
 PLAN_NO_ROUTED = 128
+PLAN_CLUSTER = 4096
+PLAN_NO_CLUSTER = 8192
 
 
 def plan_hub_log2(log2_rows):
@@ -43,19 +45,20 @@ def plan_routed_phases(n):
 
 
 def plan_segment_shift(log2_len):
-    return (int(log2_len) & 0xFF) << 8
+    return (int(log2_len) & 0xF) << 8
 
 
 STRATEGY_ROWS = 1
 STRATEGY_SEGMENTS = 2
 STRATEGY_GENERIC_K = 3
 STRATEGY_ROUTED = 4
+STRATEGY_ORDERED = 5
 
 # every symbol include/hpspmm.h declares
 EXPORTS = (
     "hpspmm_version", "hpspmm_last_error", "hpspmm_plan_create", "hpspmm_plan_get_info",
     "hpspmm_plan_destroy", "hpspmm_csr_spmm", "hpspmm_csr_spmm_noplan", "hpspmm_coo_spmm_accumulate",
-    "hpspmm_fill_f32", "hpspmm_csr_spmm_timed", "hpspmm_plan_bind_values",
+    "hpspmm_fill_f32", "hpspmm_csr_spmm_timed", "hpspmm_plan_bind_values", "hpspmm_plan_create_ordered",
 )
 
 _i64 = ctypes.c_int64
@@ -68,7 +71,7 @@ class PlanInfo(ctypes.Structure):
         ("strategy", ctypes.c_int32), ("segment_length", ctypes.c_int32),
         ("num_segments", _i64), ("max_row_nnz", _i64), ("empty_rows", _i64),
         ("workspace_bytes", _i64), ("launches_per_spmm", ctypes.c_int32), ("reserved", ctypes.c_int32),
-        ("hub_rows", _i64),
+        ("hub_rows", _i64), ("lds_served_nnz", _i64),
     ]
 
     def as_dict(self):
@@ -96,6 +99,8 @@ def lib():
         L.hpspmm_last_error.restype = ctypes.c_char_p
         L.hpspmm_plan_create.argtypes = [_i64, _i64, _i64, _p, _p, _i64, ctypes.c_uint32, _p,
                                          ctypes.POINTER(_p)]
+        L.hpspmm_plan_create_ordered.argtypes = [_i64, _i64, _i64, _p, _p, _i64, ctypes.c_uint32, _p, _p,
+                                                 ctypes.POINTER(_p)]
         L.hpspmm_plan_get_info.argtypes = [_p, ctypes.POINTER(PlanInfo)]
         L.hpspmm_plan_destroy.argtypes = [_p]
         L.hpspmm_plan_bind_values.argtypes = [_p, _p, _p]
@@ -138,7 +143,7 @@ def _dev(t, dtype, name):
 class Plan:
     """Owns an hpspmm_plan (see hpspmm_plan_create in include/hpspmm.h)."""
 
-    def __init__(self, rows, cols, rowptr, col, k, flags=PLAN_DEFAULT, stream=None):
+    def __init__(self, rows, cols, rowptr, col, k, flags=PLAN_DEFAULT, stream=None, row_order=None):
         import torch
         _dev(rowptr, torch.int32, "rowptr")
         _dev(col, torch.int32, "col")
@@ -146,8 +151,15 @@ class Plan:
             raise ValueError("rowptr must have rows + 1 entries")
         self._h = ctypes.c_void_p()
         self.rows, self.cols, self.nnz, self.k = int(rows), int(cols), int(col.numel()), int(k)
-        check(lib().hpspmm_plan_create(rows, cols, self.nnz, _ptr(rowptr), _ptr(col), k, flags,
-                                       _stream(stream), ctypes.byref(self._h)))
+        if row_order is None:
+            check(lib().hpspmm_plan_create(rows, cols, self.nnz, _ptr(rowptr), _ptr(col), k, flags,
+                                           _stream(stream), ctypes.byref(self._h)))
+        else:
+            _dev(row_order, torch.int32, "row_order")
+            if row_order.numel() != rows:
+                raise ValueError("row_order must have rows entries")
+            check(lib().hpspmm_plan_create_ordered(rows, cols, self.nnz, _ptr(rowptr), _ptr(col), k, flags,
+                                                   _ptr(row_order), _stream(stream), ctypes.byref(self._h)))
 
     @property
     def info(self):

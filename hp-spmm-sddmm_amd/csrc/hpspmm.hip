@@ -13,6 +13,7 @@
 #include <string>
 #include <vector>
 
+#include "ordered_kernels.hpp"
 #include "routed_kernels.hpp"
 #include "spmm_kernels.hpp"
 
@@ -99,6 +100,15 @@ struct hpspmm_plan {
   int64_t n_bhot = 0;
   int64_t routed_grid = 0;
   const float* bound_val = nullptr;  // value array whose class-major copy d_vval currently holds (or NULL)
+  // ordered strategy
+  int32_t* d_ostart = nullptr;  // [rows] first position of every row in processing order
+  int32_t* d_ocol = nullptr;    // [nnz] column, or ~slot of the window's LDS copy of B
+  int32_t* d_osrc = nullptr;    // [nnz] original index of the nonzero
+  int32_t* d_orow = nullptr;    // [nnz] row of the nonzero
+  int32_t* d_wcols = nullptr;   // [windows * ocap] columns held in LDS by each window's workgroup
+  int ocap = 0;
+  int64_t owindows = 0;
+  int64_t oserved = 0;          // nonzeros that read B from LDS
   int32_t* d_long_rows = nullptr;  // rows strategy: rows longer than long_threshold
   int64_t n_long = 0;
   int32_t long_threshold = INT32_MAX;
@@ -188,7 +198,26 @@ int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, 
   }
   const int64_t fix_blocks = ceil_div(ceil_div(p->rows, 64), hpspmm::kWavesPerBlock);
   hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st, p->rows,
-                     rp, p->d_carry, C, p->shift);
+                     rp, (const int32_t*)nullptr, p->d_carry, C, p->shift);
+  return HPSPMM_OK;
+}
+
+// LDS bytes for a window's rows of B in the ordered strategy.
+constexpr int kOrderedLdsBytes = 32 << 10;
+
+template <int K>
+int launch_ordered(const hpspmm_plan* p, const int32_t* rp, const float* v, const float* B, float* C,
+                   hipStream_t st) {
+  const int64_t nblocks = p->owindows;
+  const int64_t grid = p->xcd_remap ? ceil_div(nblocks, hpspmm::kXcds) * hpspmm::kXcds : nblocks;
+  if (grid > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  if (p->nnz > 0)
+    hipLaunchKernelGGL(hpspmm::spmm_ordered_kernel<K>, dim3((unsigned)grid), dim3(hpspmm::kBlock),
+                       (size_t)p->ocap * K * sizeof(float), st, rp, p->d_ostart, p->d_ocol, p->d_osrc, p->d_orow, v,
+                       p->d_wcols, p->ocap, B, C, p->d_carry, p->nnz, p->shift, nblocks, p->xcd_remap);
+  const int64_t fix_blocks = ceil_div(ceil_div(p->rows, 64), hpspmm::kWavesPerBlock);
+  hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st, p->rows,
+                     rp, p->d_ostart, p->d_carry, C, p->shift);
   return HPSPMM_OK;
 }
 
@@ -500,6 +529,163 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
   return HPSPMM_OK;
 }
 
+// Builds the ordered layout for the processing order d_order (a permutation of
+// the row numbers, in device memory).  p->shift is chosen here.
+// With min_served > 0 the layout is kept only if at least that share of the nonzeros reads B from
+// LDS; otherwise everything built here is freed again and the plan is left as it was.
+int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, const int32_t* d_order,
+                  double min_served, hipStream_t st) {
+  const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
+  const int64_t subwaves = 64 / (k / 4);
+  // window = one workgroup's segments, at most kOrderedMaxWindow nonzeros
+  int shift = 9;
+  while (((int64_t)hpspmm::kWavesPerBlock * subwaves << shift) > hpspmm::kOrderedMaxWindow) --shift;
+  const int window = (int)((int64_t)hpspmm::kWavesPerBlock * subwaves << shift);
+  const int cap = (int)(kOrderedLdsBytes / (k * 4));
+  const int64_t windows = ceil_div(nnz, window);
+  const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
+
+  uint32_t* d_len = nullptr;   // [rows + 1] row lengths in processing order, then their scan
+  int32_t* d_seen = nullptr;   // [rows] + [1]: permutation check
+  unsigned long long* d_served = nullptr;
+  struct Guard {
+    void** q[3];
+    ~Guard() {
+      for (void** x : q)
+        if (*x) (void)hipFree(*x);
+    }
+  } guard{{(void**)&d_len, (void**)&d_seen, (void**)&d_served}};
+  HPSPMM_HIP(hipMalloc(&d_len, (size_t)(rows + 1) * sizeof(uint32_t)));
+  HPSPMM_HIP(hipMalloc(&d_seen, (size_t)(rows + 1) * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&d_served, sizeof(unsigned long long)));
+  HPSPMM_HIP(hipMemsetAsync(d_seen, 0, (size_t)(rows + 1) * sizeof(int32_t), st));
+  HPSPMM_HIP(hipMemsetAsync(d_served, 0, sizeof(unsigned long long), st));
+  const unsigned rgrid = (unsigned)ceil_div(rows + 1, hpspmm::kBlock);
+  hipLaunchKernelGGL(hpspmm::ordered_mark_kernel, dim3(rgrid), dim3(hpspmm::kBlock), 0, st, rows, d_order, d_seen,
+                     d_seen + rows);
+  int32_t bad = 0;
+  HPSPMM_HIP(hipMemcpyAsync(&bad, d_seen + rows, sizeof bad, hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  if (bad) return fail(HPSPMM_ERR_INVALID_ARG, "row order is not a permutation of [0, rows)");
+  hipLaunchKernelGGL(hpspmm::ordered_len_kernel, dim3(rgrid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_order,
+                     d_len);
+  if (int rc = exclusive_scan_u32(d_len, d_len, rows + 1, st)) return rc;
+
+  const size_t n_bytes = (size_t)std::max<int64_t>(nnz, 1) * sizeof(int32_t);
+  const size_t start_bytes = (size_t)std::max<int64_t>(rows, 1) * sizeof(int32_t);
+  const size_t wcols_bytes = (size_t)std::max<int64_t>(windows, 1) * (size_t)cap * sizeof(int32_t);
+  const size_t carry_bytes = (size_t)std::max<int64_t>(nseg, 1) * 2 * (size_t)k * sizeof(float);
+  float* d_new_carry = nullptr;
+  auto drop = [&]() {
+    for (void** q : {(void**)&p->d_ostart, (void**)&p->d_ocol, (void**)&p->d_osrc, (void**)&p->d_orow,
+                     (void**)&p->d_wcols, (void**)&d_new_carry}) {
+      if (*q) (void)hipFree(*q);
+      *q = nullptr;
+    }
+  };
+  if (hipMalloc(&p->d_ostart, start_bytes) != hipSuccess || hipMalloc(&p->d_ocol, n_bytes) != hipSuccess ||
+      hipMalloc(&p->d_osrc, n_bytes) != hipSuccess || hipMalloc(&p->d_orow, n_bytes) != hipSuccess ||
+      hipMalloc(&p->d_wcols, wcols_bytes) != hipSuccess || hipMalloc(&d_new_carry, carry_bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    drop();
+    return fail(HPSPMM_ERR_ALLOC, "device allocation for the ordered plan failed");
+  }
+  hipLaunchKernelGGL(hpspmm::ordered_fill_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
+                     dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_order, d_len, p->d_ostart, p->d_ocol,
+                     p->d_osrc, p->d_orow);
+  if (windows > INT32_MAX) {
+    drop();
+    return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  }
+  if (nnz > 0)
+    hipLaunchKernelGGL(hpspmm::ordered_hot_kernel, dim3((unsigned)windows), dim3(hpspmm::kBlock), 0, st, nnz, window,
+                       cap, p->d_ocol, p->d_wcols, d_served);
+  hipLaunchKernelGGL(hpspmm::ordered_partition_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
+                     dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, p->d_ostart, window, p->d_ocol, p->d_osrc);
+  unsigned long long served = 0;
+  hipError_t e = hipMemcpyAsync(&served, d_served, sizeof served, hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e == hipSuccess) e = hipGetLastError();
+  if (e != hipSuccess) {
+    drop();
+    return fail(HPSPMM_ERR_HIP, "construction of the ordered plan failed: %s", hipGetErrorString(e));
+  }
+  if ((double)served < min_served * (double)nnz) {
+    drop();
+    return HPSPMM_OK;
+  }
+  // accepted: the segments strategy's buffers are not needed any more
+  if (p->d_nnz_row) { (void)hipFree(p->d_nnz_row); p->d_nnz_row = nullptr; }
+  if (p->d_carry) (void)hipFree(p->d_carry);
+  p->d_carry = d_new_carry;
+  p->workspace_bytes = (int64_t)(start_bytes + 3 * n_bytes + wcols_bytes + carry_bytes);
+  p->shift = shift;
+  p->nseg = nseg;
+  p->ocap = cap;
+  p->owindows = windows;
+  p->oserved = (int64_t)served;
+  p->strategy = HPSPMM_STRATEGY_ORDERED;
+  return HPSPMM_OK;
+}
+
+// Automatic clustering is tried for graphs of at least this size ...
+constexpr int64_t kClusterMinNnz = (int64_t)1 << 22;
+constexpr int64_t kClusterMinBBytes = (int64_t)64 << 20;
+constexpr int64_t kClusterMinMeanNnz = 8;
+// ... and its order is kept if this share of the nonzeros then reads B from LDS.
+constexpr double kClusterMinServed = 0.15;
+
+// Finds a processing order for a square matrix by label propagation on its graph: rows of one
+// label next to each other, labels in increasing order, rows of a label in increasing order.
+// d_order_out receives a device array of `rows` entries (caller frees).
+constexpr int kClusterMaxSweeps = 10;
+
+int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st,
+                 int32_t** d_order_out) {
+  const int64_t rows = p->rows;
+  *d_order_out = nullptr;
+  int32_t* d_label = nullptr;
+  unsigned long long* d_changed = nullptr;
+  struct Guard {
+    void** q[2];
+    ~Guard() {
+      for (void** x : q)
+        if (*x) (void)hipFree(*x);
+    }
+  } guard{{(void**)&d_label, (void**)&d_changed}};
+  HPSPMM_HIP(hipMalloc(&d_label, (size_t)rows * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&d_changed, sizeof(unsigned long long)));
+  hipLaunchKernelGGL(hpspmm::cluster_init_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                     0, st, rows, d_label);
+  for (int sweep = 0; sweep < kClusterMaxSweeps; ++sweep) {
+    HPSPMM_HIP(hipMemsetAsync(d_changed, 0, sizeof(unsigned long long), st));
+    hipLaunchKernelGGL(hpspmm::cluster_sweep_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
+                       dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_label, (uint32_t)sweep, d_changed);
+    unsigned long long changed = 0;
+    HPSPMM_HIP(hipMemcpyAsync(&changed, d_changed, sizeof changed, hipMemcpyDeviceToHost, st));
+    HPSPMM_HIP(hipStreamSynchronize(st));
+    if ((int64_t)changed * 200 < rows) break;
+  }
+  // counting sort by label on the host: stable, hence the same order on every run
+  std::vector<int32_t> label((size_t)rows), order((size_t)rows);
+  HPSPMM_HIP(hipMemcpyAsync(label.data(), d_label, label.size() * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  std::vector<int32_t> first((size_t)rows + 1, 0);
+  for (int64_t r = 0; r < rows; ++r) first[(size_t)label[(size_t)r] + 1]++;
+  for (int64_t l = 0; l < rows; ++l) first[(size_t)l + 1] += first[(size_t)l];
+  for (int64_t r = 0; r < rows; ++r) order[(size_t)first[(size_t)label[(size_t)r]]++] = (int32_t)r;
+  int32_t* d_order = nullptr;
+  HPSPMM_HIP(hipMalloc(&d_order, (size_t)rows * sizeof(int32_t)));
+  hipError_t e = hipMemcpyAsync(d_order, order.data(), order.size() * sizeof(int32_t), hipMemcpyHostToDevice, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e != hipSuccess) {
+    (void)hipFree(d_order);
+    return fail(HPSPMM_ERR_HIP, "upload of the row order failed: %s", hipGetErrorString(e));
+  }
+  *d_order_out = d_order;
+  return HPSPMM_OK;
+}
+
 // Automatic hub cache: only when the cached rows would serve at least this share of the nonzeros.
 constexpr double kHubMinShare = 0.25;
 
@@ -549,8 +735,9 @@ int hpspmm_version(void) { return 100; }
 
 const char* hpspmm_last_error(void) { return g_last_error.c_str(); }
 
-int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr, const int32_t* d_col,
-                       int64_t k, uint32_t flags, void* stream, hpspmm_plan** plan_out) {
+static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr, const int32_t* d_col,
+                            int64_t k, uint32_t flags, const int32_t* d_order, void* stream,
+                            hpspmm_plan** plan_out) {
   if (!plan_out) return fail(HPSPMM_ERR_INVALID_ARG, "plan_out is NULL");
   *plan_out = nullptr;
   if (int rc = check_dims(rows, cols, nnz, k)) return rc;
@@ -604,6 +791,13 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d
 
   if (!fast_k(k)) {
     p->strategy = HPSPMM_STRATEGY_GENERIC_K;
+  } else if (d_order && nnz > 0) {
+    if (int rc = build_ordered(p, d_rowptr, d_col, d_order, 0.0, st)) {
+      hpspmm_plan_destroy(p);
+      return rc;
+    }
+    *plan_out = p;
+    return HPSPMM_OK;
   } else if (flags & HPSPMM_PLAN_FORCE_ROWS) {
     p->strategy = HPSPMM_STRATEGY_ROWS;
   } else if (flags & (HPSPMM_PLAN_FORCE_SEGMENTS | HPSPMM_PLAN_FORCE_ROUTED)) {
@@ -617,10 +811,10 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d
   }
 
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS) {
-    int forced = (int)((flags >> 8) & 0xFFu);
-    if (forced && (forced < 3 || forced > 20)) {
+    int forced = (int)((flags >> 8) & 0xFu);
+    if (forced && (forced < 3 || forced > 15)) {
       delete p;
-      return fail(HPSPMM_ERR_INVALID_ARG, "forced segment shift %d outside [3, 20]", forced);
+      return fail(HPSPMM_ERR_INVALID_ARG, "forced segment shift %d outside [3, 15]", forced);
     }
     p->shift = forced ? forced : choose_shift(nnz, k);
     p->nseg = ceil_div(nnz, (int64_t)1 << p->shift);
@@ -658,6 +852,22 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d
       return rc;
     }
   }
+  // Community structure: neither hot columns nor anything else to exploit so far, the matrix is a
+  // graph (square) and B does not fit the L2s - look for clusters of rows that share columns.
+  const bool want_cluster = (flags & HPSPMM_PLAN_CLUSTER) != 0;
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && p->n_hub == 0 && rows == cols && nnz > 0 &&
+      !(flags & HPSPMM_PLAN_NO_CLUSTER) &&
+      (want_cluster || (!(flags & HPSPMM_PLAN_FORCE_SEGMENTS) && nnz >= kClusterMinNnz &&
+                        cols * k * 4 >= kClusterMinBBytes && nnz >= rows * kClusterMinMeanNnz))) {
+    int32_t* d_order = nullptr;
+    int rc = cluster_rows(p, d_rowptr, d_col, st, &d_order);
+    if (rc == HPSPMM_OK) rc = build_ordered(p, d_rowptr, d_col, d_order, want_cluster ? 0.0 : kClusterMinServed, st);
+    if (d_order) (void)hipFree(d_order);
+    if (rc) {
+      hpspmm_plan_destroy(p);
+      return rc;
+    }
+  }
   if (p->strategy == HPSPMM_STRATEGY_ROWS && p->max_row_nnz > kLongRowThreshold) {
     // list of the rows that get a whole wavefront; d_meta[3] counts them
     p->long_threshold = kLongRowThreshold;
@@ -683,6 +893,18 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d
   return HPSPMM_OK;
 }
 
+int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr, const int32_t* d_col,
+                       int64_t k, uint32_t flags, void* stream, hpspmm_plan** plan_out) {
+  return plan_create_impl(rows, cols, nnz, d_rowptr, d_col, k, flags, nullptr, stream, plan_out);
+}
+
+int hpspmm_plan_create_ordered(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr,
+                               const int32_t* d_col, int64_t k, uint32_t flags, const int32_t* d_row_order,
+                               void* stream, hpspmm_plan** plan_out) {
+  if (rows > 0 && !d_row_order) return fail(HPSPMM_ERR_INVALID_ARG, "d_row_order is NULL");
+  return plan_create_impl(rows, cols, nnz, d_rowptr, d_col, k, flags, d_row_order, stream, plan_out);
+}
+
 int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
   if (!plan || !out) return fail(HPSPMM_ERR_INVALID_ARG, "plan or info_out is NULL");
   std::memset(out, 0, sizeof *out);
@@ -691,15 +913,19 @@ int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
   out->nnz = plan->nnz;
   out->k = plan->k;
   out->strategy = plan->strategy;
-  const bool segmented = plan->strategy == HPSPMM_STRATEGY_SEGMENTS || plan->strategy == HPSPMM_STRATEGY_ROUTED;
+  const bool segmented = plan->strategy == HPSPMM_STRATEGY_SEGMENTS || plan->strategy == HPSPMM_STRATEGY_ROUTED ||
+                         plan->strategy == HPSPMM_STRATEGY_ORDERED;
   out->segment_length = segmented ? (1 << plan->shift) : 0;
   out->num_segments = plan->nseg;
   out->max_row_nnz = plan->max_row_nnz;
   out->empty_rows = plan->empty_rows;
   out->workspace_bytes = plan->workspace_bytes;
-  out->launches_per_spmm = plan->strategy == HPSPMM_STRATEGY_ROUTED ? 3
-                           : plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? (plan->n_hub > 0 ? 3 : 2) : 1;
+  out->launches_per_spmm = plan->strategy == HPSPMM_STRATEGY_ROUTED    ? 3
+                           : plan->strategy == HPSPMM_STRATEGY_ORDERED ? 2
+                           : plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? (plan->n_hub > 0 ? 3 : 2)
+                                                                        : 1;
   out->hub_rows = plan->n_hub;
+  out->lds_served_nnz = plan->oserved;
   return HPSPMM_OK;
 }
 
@@ -714,7 +940,9 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
   for (void* q : {(void*)plan->d_rvptr, (void*)plan->d_coldptr, (void*)plan->d_vcol, (void*)plan->d_lslot,
                   (void*)plan->d_chunk_base, (void*)plan->d_chunk_pref,
                   (void*)plan->d_vval, (void*)plan->d_vrow, (void*)plan->d_bhot_src, (void*)plan->d_partial,
-                  (void*)plan->d_routed_rows, (void*)plan->d_cross_rows, (void*)plan->d_zero_rows})
+                  (void*)plan->d_routed_rows, (void*)plan->d_cross_rows, (void*)plan->d_zero_rows,
+                  (void*)plan->d_ostart, (void*)plan->d_ocol, (void*)plan->d_osrc, (void*)plan->d_orow,
+                  (void*)plan->d_wcols})
     if (q) (void)hipFree(q);
   delete plan;
   return HPSPMM_OK;
@@ -750,7 +978,13 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
   int rc;
   // another value array overwrites the plan's copy of the bound one
   if (plan->bound_val && plan->bound_val != d_val) plan->bound_val = nullptr;
-  if (plan->strategy == HPSPMM_STRATEGY_ROUTED) {
+  if (plan->strategy == HPSPMM_STRATEGY_ORDERED) {
+    switch (plan->k) {
+      case 32: rc = launch_ordered<32>(plan, d_rowptr, d_val, d_B, d_C, st); break;
+      case 64: rc = launch_ordered<64>(plan, d_rowptr, d_val, d_B, d_C, st); break;
+      default: rc = launch_ordered<128>(plan, d_rowptr, d_val, d_B, d_C, st); break;
+    }
+  } else if (plan->strategy == HPSPMM_STRATEGY_ROUTED) {
     switch (plan->k) {
       case 32: rc = launch_routed<32>(plan, d_val, d_B, d_C, st); break;
       case 64: rc = launch_routed<64>(plan, d_val, d_B, d_C, st); break;

@@ -1,0 +1,392 @@
+// gfx950 device code of the *ordered* strategy for FP32 CSR SpMM.
+//
+// Graphs with community structure reuse rows of B only among the few dozen
+// rows of A of one community.  Processing those rows next to each other is not
+// enough on this machine: a sub-wave returns to the same row of B one row of A
+// later, i.e. after some 50 gathers or ~9 us, and under full-rate streaming an
+// L2 of 4 MB is turned over every ~4 us (measured on the 2.4M-vertex
+// co-purchase graph with its rows grouped by community: L2 hits rise from 3 %
+// to 12 % only).  The ordered strategy therefore makes the reuse explicit:
+//
+//   * the rows of A are processed in a given order (a permutation of the row
+//     numbers, supplied by the caller - the reference's HP-SpMM reads one from
+//     a .cugraph_reorder file, spmm/mm/spmm_common.cpp:237-296 - or found by
+//     the plan's own clustering); C is written at the original row numbers;
+//   * the nonzeros, laid out in that order, are cut into windows of
+//     kWavesPerBlock * P segments, one workgroup each.  The plan finds, per
+//     window, the columns that occur at least twice in it and gives the most
+//     frequent ones a slot in a workgroup-local LDS copy of B (their column
+//     index is rewritten as ~slot);
+//   * the workgroup first fetches those rows of B into LDS, once, then runs
+//     the tile engine of the segments kernel, reading a slotted column from
+//     LDS and every other one from memory.
+//
+// The values are read in place through the nonzeros' original indices (a row's
+// nonzeros stay contiguous, so these loads remain coalesced).  Rows cut by a
+// segment boundary go through the carry slots exactly as in the segments
+// strategy; the fix-up kernel is shared.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "spmm_kernels.hpp"
+
+namespace hpspmm {
+
+// ---- plan-time kernels -----------------------------------------------------
+
+// Label propagation, one sweep: every row takes the label that is most frequent
+// among (a sample of at most 64 of) its neighbours' labels - the rows whose
+// indices are its column indices; the matrix is taken as a graph, which is
+// meant for square, structurally symmetric A.  Ties are broken by a hash that
+// changes with the sweep, except that a row keeps its label when that is among
+// the most frequent.  Labels are updated in place (asynchronous propagation,
+// which does not oscillate the way the synchronous form does).  One wavefront
+// per row; the 64 sampled labels are sorted by a bitonic network of
+// wavefront shuffles.  changed[0] += rows whose label changed.
+__global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                               const int32_t* __restrict__ col,
+                                                               int32_t* __restrict__ label, uint32_t sweep,
+                                                               unsigned long long* __restrict__ changed) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const int32_t lb = rowptr[r];
+  const int32_t n = rowptr[r + 1] - lb;
+  if (n == 0) return;
+  const int32_t stride = (n + 63) / 64;
+  const bool valid = lane * stride < n;
+  int32_t lab = INT32_MAX;  // sorts behind every label
+  if (valid) {
+    const int32_t c = col[lb + lane * stride];
+    if ((int64_t)c < rows) lab = label[c];
+  }
+  const int32_t mine = label[r];
+  const int self_count = (int)__popcll(__ballot(lab == mine));
+#pragma unroll
+  for (int size = 2; size <= 64; size <<= 1) {
+#pragma unroll
+    for (int j = size >> 1; j > 0; j >>= 1) {
+      const int32_t other = __shfl_xor(lab, j);
+      const bool up = (lane & size) == 0;
+      const bool lower = (lane & j) == 0;
+      const int32_t lo = lab < other ? lab : other;
+      const int32_t hi = lab < other ? other : lab;
+      lab = (lower == up) ? lo : hi;
+    }
+  }
+  const int32_t prev = __shfl_up(lab, 1);
+  const bool real = lab != INT32_MAX;
+  const bool head = real && (lane == 0 || lab != prev);
+  const uint64_t heads = __ballot(head);
+  const int n_real = (int)__popcll(__ballot(real));
+  if (n_real == 0) return;
+  unsigned long long key = 0;
+  if (head) {
+    const uint64_t later = lane < 63 ? (heads >> (lane + 1)) : 0ull;
+    const int next = later ? lane + 1 + (int)__ffsll((long long)later) - 1 : n_real;
+    const uint32_t h = ((uint32_t)lab * 0x9E3779B1u) ^ (sweep * 0x85EBCA6Bu) ^ ((uint32_t)r * 0xC2B2AE35u);
+    key = ((unsigned long long)(uint32_t)(next - lane) << 32) | (h >> 1);
+  }
+  unsigned long long best = key;
+  int32_t best_lab = lab;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned long long o = __shfl_xor(best, off);
+    const int32_t ol = __shfl_xor(best_lab, off);
+    if (o > best) {
+      best = o;
+      best_lab = ol;
+    }
+  }
+  const int best_count = (int)(best >> 32);
+  if (lane == 0 && self_count < best_count && best_lab != mine) {
+    label[r] = best_lab;
+    atomicAdd(changed, 1ull);
+  }
+}
+
+// label[r] = r.
+__global__ __launch_bounds__(kBlock) void cluster_init_kernel(int64_t rows, int32_t* __restrict__ label) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r < rows) label[r] = (int32_t)r;
+}
+
+// len[i] = number of nonzeros of the i-th row in processing order; len[rows] = 0.
+__global__ __launch_bounds__(kBlock) void ordered_len_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                             const int32_t* __restrict__ order,
+                                                             uint32_t* __restrict__ len) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i > rows) return;
+  uint32_t n = 0;
+  if (i < rows) {
+    const int32_t r = order[i];
+    n = (uint32_t)(rowptr[r + 1] - rowptr[r]);
+  }
+  len[i] = n;
+}
+
+// seen[order[i]] += 1: a permutation leaves every counter at exactly one.
+__global__ __launch_bounds__(kBlock) void ordered_mark_kernel(int64_t rows, const int32_t* __restrict__ order,
+                                                              int32_t* __restrict__ seen,
+                                                              int32_t* __restrict__ bad) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= rows) return;
+  const int32_t r = order[i];
+  if (r < 0 || (int64_t)r >= rows) {
+    atomicOr(bad, 1);
+    return;
+  }
+  if (atomicAdd(&seen[r], 1) != 0) atomicOr(bad, 2);
+}
+
+// Lays the nonzeros out in processing order.  One wavefront per position i:
+// row r = order[i] starts at pstart[i]; start[r] = pstart[i];
+// ocol / osrc / orow = column, original index and row of every nonzero.
+__global__ __launch_bounds__(kBlock) void ordered_fill_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                              const int32_t* __restrict__ col,
+                                                              const int32_t* __restrict__ order,
+                                                              const uint32_t* __restrict__ pstart,
+                                                              int32_t* __restrict__ start,
+                                                              int32_t* __restrict__ ocol, int32_t* __restrict__ osrc,
+                                                              int32_t* __restrict__ orow) {
+  const int lane = threadIdx.x & 63;
+  const int64_t i = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (i >= rows) return;
+  const int32_t r = order[i];
+  const int32_t lb = rowptr[r];
+  const int32_t hb = rowptr[r + 1];
+  const int32_t p0 = (int32_t)pstart[i];
+  if (lane == 0) start[r] = p0;
+  for (int32_t j = lb + lane; j < hb; j += 64) {
+    const int32_t p = p0 + (j - lb);
+    ocol[p] = col[j];
+    osrc[p] = j;
+    orow[p] = r;
+  }
+}
+
+// Per window of `window` consecutive nonzeros (in processing order; window <=
+// kOrderedMaxWindow): the columns that occur at least twice, the `cap` most
+// frequent of them (ties: an occurrence count is either kept whole or dropped
+// whole), in increasing column order -> wcols[w * cap + slot] (-1 = unused
+// slot); the nonzeros of those columns get ocol = ~slot.  One workgroup per
+// window: bitonic sort of the window's columns in LDS, run lengths, a
+// threshold on the run length, compaction.  served[0] += rewritten nonzeros.
+constexpr int kOrderedMaxWindow = 8192;
+constexpr int kOrderedHistMax = 65;  // run lengths are told apart up to this one
+
+__global__ __launch_bounds__(kBlock) void ordered_hot_kernel(int64_t nnz, int window, int cap,
+                                                             int32_t* __restrict__ ocol,
+                                                             int32_t* __restrict__ wcols,
+                                                             unsigned long long* __restrict__ served) {
+  __shared__ int32_t s_key[kOrderedMaxWindow];   // the window's columns, sorted (INT32_MAX pads)
+  __shared__ int32_t s_sel[kOrderedMaxWindow / 2];  // selected columns (each occurs >= 2 times)
+  __shared__ int32_t s_count;
+  __shared__ int32_t s_hist[kOrderedHistMax + 1];  // s_hist[t] = runs of length >= t, t in [2, kOrderedHistMax]
+  const int tid = threadIdx.x;
+  const int64_t w = blockIdx.x;
+  const int64_t p0 = w * window;
+  const int n = nnz - p0 < window ? (int)(nnz - p0) : window;
+  int npow = 1;
+  while (npow < n) npow <<= 1;
+  for (int i = tid; i < npow; i += kBlock) s_key[i] = i < n ? ocol[p0 + i] : INT32_MAX;
+  for (int i = tid; i <= kOrderedHistMax; i += kBlock) s_hist[i] = 0;
+  if (tid == 0) s_count = 0;
+  __syncthreads();
+  for (int size = 2; size <= npow; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int i = tid; i < npow / 2; i += kBlock) {
+        const int lo = ((i / stride) * stride * 2) + (i % stride);
+        const int hi = lo + stride;
+        const bool up = ((lo & size) == 0);
+        const int32_t a = s_key[lo], b = s_key[hi];
+        if ((a > b) == up) {
+          s_key[lo] = b;
+          s_key[hi] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  // run heads: position i starts a run if it differs from its predecessor
+  auto run_length = [&](int i) {
+    int len = 1;
+    while (i + len < n && s_key[i + len] == s_key[i]) ++len;
+    return len;
+  };
+  for (int i = tid; i < n; i += kBlock) {
+    if (i > 0 && s_key[i] == s_key[i - 1]) continue;
+    const int len = run_length(i);
+    if (len >= 2) {
+      const int top = len < kOrderedHistMax ? len : kOrderedHistMax;
+      for (int t = 2; t <= top; ++t) atomicAdd(&s_hist[t], 1);
+    }
+  }
+  __syncthreads();
+  int threshold = 2;
+  while (threshold < kOrderedHistMax && s_hist[threshold] > cap) ++threshold;
+  const bool fits = s_hist[threshold] <= cap;  // always, as long as cap >= window / kOrderedHistMax
+  __syncthreads();
+  // selection in column order: one thread walks the run heads (windows are small and this is plan time)
+  if (tid == 0) {
+    int m = 0;
+    for (int i = 0; i < n && fits;) {
+      const int len = run_length(i);
+      if (len >= threshold && m < cap) s_sel[m++] = s_key[i];
+      i += len;
+    }
+    s_count = m;
+  }
+  __syncthreads();
+  const int m = s_count;
+  for (int i = tid; i < cap; i += kBlock) wcols[w * cap + i] = i < m ? s_sel[i] : -1;
+  unsigned long long mine = 0;
+  for (int i = tid; i < n; i += kBlock) {
+    const int32_t c = ocol[p0 + i];
+    int lo = 0, hi = m;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (s_sel[mid] < c) lo = mid + 1;
+      else hi = mid;
+    }
+    if (lo < m && s_sel[lo] == c) {
+      ocol[p0 + i] = ~lo;
+      ++mine;
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) mine += __shfl_down(mine, off);
+  if ((tid & 63) == 0 && mine) atomicAdd(served, mine);
+}
+
+// Within every row, the nonzeros that read B from memory first, those that read
+// it from LDS last (each group in its previous order): the gathers are issued
+// in batches, and a batch is as slow as its slowest load.  One wavefront per
+// row; a row cut by a window boundary is left as it is (its slots belong to
+// two different windows).
+__global__ __launch_bounds__(kBlock) void ordered_partition_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                                   const int32_t* __restrict__ start, int window,
+                                                                   int32_t* __restrict__ ocol,
+                                                                   int32_t* __restrict__ osrc) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const int32_t n = rowptr[r + 1] - rowptr[r];
+  if (n < 2) return;
+  const int32_t p0 = start[r];
+  if (p0 / window != (p0 + n - 1) / window) return;
+  // count the memory group, then place both groups; chunks of 64 keep their relative order
+  int32_t n_mem = 0;
+  for (int32_t i0 = 0; i0 < n; i0 += 64) {
+    const int32_t i = i0 + lane;
+    const bool mem = i < n && ocol[p0 + i] >= 0;
+    n_mem += (int32_t)__popcll(__ballot(mem));
+  }
+  if (n_mem == 0 || n_mem == n) return;
+  // rows longer than 64 would be overwritten while still being read: stage them through registers in
+  // chunks only when the whole row fits one chunk, else leave the row unchanged
+  if (n > 64) return;
+  const bool valid = lane < n;
+  const int32_t c = valid ? ocol[p0 + lane] : 0;
+  const int32_t sidx = valid ? osrc[p0 + lane] : 0;
+  const bool mem = valid && c >= 0;
+  const uint64_t m_mem = __ballot(mem);
+  const uint64_t m_lds = __ballot(valid && !mem);
+  const uint64_t below = (1ull << lane) - 1ull;
+  if (valid) {
+    const int32_t dst = mem ? (int32_t)__popcll(m_mem & below) : n_mem + (int32_t)__popcll(m_lds & below);
+    ocol[p0 + dst] = c;
+    osrc[p0 + dst] = sidx;
+  }
+}
+
+// ---- SpMM kernel -----------------------------------------------------------
+
+// One workgroup per window = kWavesPerBlock * P segments of 2^shift nonzeros.
+// Dynamic LDS: cap * K floats, the window's slotted rows of B.
+template <int K>
+__global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
+    const int32_t* __restrict__ rowptr, const int32_t* __restrict__ start, const int32_t* __restrict__ ocol,
+    const int32_t* __restrict__ osrc, const int32_t* __restrict__ orow, const float* __restrict__ val,
+    const int32_t* __restrict__ wcols, int cap, const float* __restrict__ B, float* __restrict__ C,
+    float* __restrict__ carry, int64_t nnz, int shift, int64_t nblocks, bool remap) {
+  constexpr int G = K / 4;
+  constexpr int P = 64 / G;
+  constexpr int TL = kTile / G;
+  __shared__ __attribute__((aligned(16))) int32_t s_col[kWavesPerBlock * P * kTileStride];
+  __shared__ __attribute__((aligned(16))) float s_val[kWavesPerBlock * P * kTileStride];
+  __shared__ __attribute__((aligned(16))) int32_t s_row[kWavesPerBlock * P * kTileStride];
+  extern __shared__ __attribute__((aligned(16))) float s_b[];  // [cap][K]
+
+  const int64_t blk = xcd_remap(blockIdx.x, nblocks, remap);
+  if (blk < 0) return;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int l = lane % G;
+
+  // the window's rows of B; every thread of the workgroup reaches the barrier
+  for (int i = tid; i < cap * G; i += kBlock) {
+    const int slot = i / G;
+    const int32_t c = wcols[blk * cap + slot];
+    if (c >= 0) *reinterpret_cast<float4*>(s_b + slot * K + 4 * (i % G)) = load_b<K>(B, c, i % G);
+  }
+  __syncthreads();
+
+  const int64_t g = (blk * kWavesPerBlock + (tid >> 6)) * P + lane / G;
+  const int64_t s = g << shift;
+  if (s >= nnz) return;
+  const int64_t e = (s + ((int64_t)1 << shift)) < nnz ? (s + ((int64_t)1 << shift)) : nnz;
+  const int sbase = ((tid >> 6) * P + lane / G) * kTileStride;
+
+  int32_t cur = orow[s];
+  bool head_pending = (int64_t)start[cur] < s;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+
+  auto flush_to = [&](bool is_tail) {
+    float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
+                              : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : C + (uint64_t)(uint32_t)cur * K);
+    head_pending = false;
+    store_result(dst + 4 * l, acc);
+  };
+  auto flush = [&]() { flush_to(false); };
+  // One flat load per gather, its address selected between the LDS copy and memory: a branch
+  // per gather would make every load of a batch wait for the one before it.
+  const float* lds_b = s_b;
+  auto loadb = [&](int32_t c) {
+    const float* row = c < 0 ? lds_b + (uint32_t)(~c) * (uint32_t)K : B + (uint64_t)(uint32_t)c * (uint64_t)K;
+    return *reinterpret_cast<const float4*>(row + 4 * l);
+  };
+
+  // Two-deep prefetch: the original indices of tile t+2 and, through the indices
+  // fetched one iteration earlier, the values of tile t+1 (the plan's arrays
+  // are allocated by the library, hence always aligned for the vector loads).
+  TileRegs<TL> m;
+  int32_t src[TL];
+  const int64_t q0 = s + l * TL;
+  load_run<TL>(src, osrc, q0, e, true);
+  load_run<TL>(m.c, ocol, q0, e, true);
+  load_run<TL>(m.r, orow, q0, e, true);
+#pragma unroll
+  for (int j = 0; j < TL; ++j) m.v[j] = q0 + j < e ? val[src[j]] : 0.f;
+  if (s + kTile < e) load_run<TL>(src, osrc, q0 + kTile, e, true);
+
+  for (int64_t t = s; t < e; t += kTile) {
+    stage_tile<TL>(m, sbase + l * TL, s_col, s_val, s_row);
+    wave_lds_fence();
+    if (t + kTile < e) {
+      const int64_t q = t + kTile + l * TL;
+      load_run<TL>(m.c, ocol, q, e, true);
+      load_run<TL>(m.r, orow, q, e, true);
+#pragma unroll
+      for (int j = 0; j < TL; ++j) m.v[j] = q + j < e ? val[src[j]] : 0.f;
+      if (t + 2 * kTile < e) load_run<TL>(src, osrc, q + kTile, e, true);
+    }
+    const int cnt = (e - t) < kTile ? (int)(e - t) : kTile;
+    consume_tile(cnt, sbase, s_col, s_val, s_row, cur, acc, loadb, flush);
+    wave_lds_fence();
+  }
+  flush_to((int64_t)start[cur] + (rowptr[cur + 1] - rowptr[cur]) > e);
+}
+
+}  // namespace hpspmm

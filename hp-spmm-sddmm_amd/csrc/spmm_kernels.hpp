@@ -450,8 +450,11 @@ __global__ __launch_bounds__(kBlock) void spmm_segments_kernel(
 // rowptr pair per lane, coalesced) and classifies them by ballot; its sub-waves
 // then zero the empty rows and, for rows that cross a segment boundary, add the
 // carry slots in segment order.  All other rows were already stored.
+// `start` (may be NULL): first position of every row when the nonzeros were
+// processed in an order of the plan's own; NULL = stored order (rowptr).
 template <int K>
 __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                            const int32_t* __restrict__ start,
                                                             const float* __restrict__ carry,
                                                             float* __restrict__ C, int shift) {
   constexpr int G = K / 4;
@@ -464,8 +467,12 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
   if (r0 >= rows) return;
   const int64_t r = r0 + lane;
   const bool valid = r < rows;
-  const int32_t lb = valid ? rowptr[r] : 0;
-  const int32_t hb = valid ? rowptr[r + 1] : 0;
+  int32_t lb = valid ? rowptr[r] : 0;
+  int32_t hb = valid ? rowptr[r + 1] : 0;
+  if (start != nullptr && valid) {
+    hb = start[r] + (hb - lb);
+    lb = start[r];
+  }
   const bool empty = valid && lb == hb;
   const bool split = valid && lb != hb && ((int64_t)lb >> shift) != ((int64_t)(hb - 1) >> shift);
   const uint64_t m_empty = __ballot(empty);

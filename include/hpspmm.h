@@ -66,14 +66,20 @@ typedef enum hpspmm_status {
 #define HPSPMM_PLAN_ROUTED_PHASES(n) (((uint32_t)(n) & 0x7u) << 29)
 /* bits 16..23: log2 of the number of cached rows (0 = default, 2^16) */
 #define HPSPMM_PLAN_HUB_LOG2(log2_rows) (((uint32_t)(log2_rows) & 0xFFu) << 16)
-/* bits 8..15: log2 of the segment length to force (0 = choose automatically) */
-#define HPSPMM_PLAN_SEGMENT_SHIFT(log2_len) (((uint32_t)(log2_len) & 0xFFu) << 8)
+/* bits 8..11: log2 of the segment length to force (0 = choose automatically) */
+#define HPSPMM_PLAN_SEGMENT_SHIFT(log2_len) (((uint32_t)(log2_len) & 0xFu) << 8)
+#define HPSPMM_PLAN_CLUSTER 4096u     /* square A: always look for clusters of rows that share columns and use the
+                                         ordered strategy on the order found (default: only for large graphs
+                                         without hot columns, and only if >= 15 % of the nonzeros then read B
+                                         from LDS) */
+#define HPSPMM_PLAN_NO_CLUSTER 8192u  /* never */
 
 /* strategy reported by hpspmm_plan_get_info */
 #define HPSPMM_STRATEGY_ROWS 1
 #define HPSPMM_STRATEGY_SEGMENTS 2
 #define HPSPMM_STRATEGY_GENERIC_K 3
 #define HPSPMM_STRATEGY_ROUTED 4
+#define HPSPMM_STRATEGY_ORDERED 5
 
 typedef struct hpspmm_plan hpspmm_plan;
 
@@ -88,6 +94,7 @@ typedef struct hpspmm_plan_info {
   int32_t launches_per_spmm;
   int32_t reserved;
   int64_t hub_rows;        /* rows of B kept in the hub cache (0 = none) */
+  int64_t lds_served_nnz;  /* ordered strategy: nonzeros whose row of B comes from a workgroup's LDS copy */
 } hpspmm_plan_info;
 
 /* Library version, major*10000 + minor*100 + patch. */
@@ -108,6 +115,21 @@ const char *hpspmm_last_error(void);
 int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
                        const int32_t *d_col, int64_t k, uint32_t flags, void *stream,
                        hpspmm_plan **plan_out);
+
+/*
+ * hpspmm_plan_create for a caller-chosen processing order of the rows:
+ * d_row_order[i] = the row handled i-th (a permutation of 0..rows-1, device
+ * memory, read only here).  Rows that share many columns should be neighbours
+ * in it: every workgroup keeps the rows of B that its stretch of nonzeros uses
+ * more than once in LDS.  C is written at the original row numbers, so the
+ * result is that of hpspmm_plan_create up to summation order.  The role of the
+ * row permutation that the reference reads from a .cugraph_reorder file for
+ * HP-SpMM (spmm/mm/spmm_common.cpp:237-296: nonzeros emitted in that row
+ * order, row indices kept).  K must be 32, 64 or 128 for the order to be used.
+ */
+int hpspmm_plan_create_ordered(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
+                               const int32_t *d_col, int64_t k, uint32_t flags,
+                               const int32_t *d_row_order, void *stream, hpspmm_plan **plan_out);
 
 int hpspmm_plan_get_info(const hpspmm_plan *plan, hpspmm_plan_info *info_out);
 

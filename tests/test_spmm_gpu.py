@@ -59,6 +59,8 @@ def _strategies(capi):
              | capi.plan_routed_row_log2(1)),
             ("routed_s16", capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(10) | capi.plan_segment_shift(4)
              | capi.plan_routed_row_log2(3)),
+            ("cluster", capi.PLAN_CLUSTER),
+            ("cluster_seg", capi.PLAN_CLUSTER | capi.PLAN_FORCE_SEGMENTS | capi.PLAN_NO_HUB_CACHE),
             ("routed_3phases", capi.PLAN_FORCE_ROUTED | capi.plan_routed_phases(3) | capi.plan_routed_row_log2(4)),
             ("routed_7phases_tiny", capi.PLAN_FORCE_ROUTED | capi.plan_routed_phases(7) | capi.plan_hub_log2(5)
              | capi.plan_segment_shift(3) | capi.plan_routed_row_log2(1))]
@@ -326,7 +328,7 @@ def test_full_size_configs(pkg, oracle, gpu, name, k):
         assert not torch.isnan(C).any().item(), f"{name} K={k} {tag}: C not fully written"
         out[tag] = (C, info)
     expect = {("c2_social", 128): capi.STRATEGY_ROUTED, ("c2_social", 64): capi.STRATEGY_ROUTED,
-              ("c4_rmat", 128): capi.STRATEGY_ROUTED, ("c3_copurchase", 64): capi.STRATEGY_SEGMENTS,
+              ("c4_rmat", 128): capi.STRATEGY_ROUTED, ("c3_copurchase", 64): capi.STRATEGY_ORDERED,
               ("c2_social", 32): capi.STRATEGY_ROUTED}[(name, k)]
     assert out["auto"][1]["strategy"] == expect
     # the two strategies sum in different orders: they agree to rounding, scaled by |A| |B|
@@ -523,3 +525,36 @@ def test_auto_strategy_leaves_short_rows_unrouted(pkg, oracle, gpu):
     assert err <= TOL
     # the two strategies add every row's products in the same (stored) order here: no row is routed
     assert np.array_equal(C, Cr)
+
+
+@pytest.mark.parametrize("k", [32, 64, 128])
+def test_caller_supplied_row_order(pkg, oracle, gpu, k):
+    """hpspmm_plan_create_ordered: any permutation of the rows gives the product at the original row
+    numbers; identity, reversed, random and rows sorted by length; rectangular A included."""
+    import torch
+    capi = pkg.capi
+    rng = np.random.default_rng(11)
+    g = pkg.graphs.make_graph("c4_rmat", 0.004)
+    rowptr, col, val = _random_csr(rng, 1500, 700, mean_deg=12.0, skew=2.0, empty_frac=0.3, sorted_unique=True)
+    rect = pkg.graphs.CSR(1500, 700, rowptr, col, val)
+    for graph in (g, rect):
+        B = rng.standard_normal((graph.cols, k)).astype(np.float32)
+        rp, ci, v, Bd = _to_dev(gpu, graph.rowptr, graph.col, graph.val, B)
+        deg = np.diff(graph.rowptr)
+        orders = {"identity": np.arange(graph.rows), "reversed": np.arange(graph.rows)[::-1],
+                  "random": rng.permutation(graph.rows), "by length": np.argsort(-deg, kind="stable")}
+        for name, order in orders.items():
+            od, = _to_dev(gpu, order.astype(np.int32))
+            plan = capi.Plan(graph.rows, graph.cols, rp, ci, k, 0, row_order=od)
+            assert plan.info["strategy"] == capi.STRATEGY_ORDERED
+            C = torch.full((graph.rows, k), float("nan"), device=gpu)
+            capi.csr_spmm(plan, rp, ci, v, Bd, C)
+            again = torch.full_like(C, float("nan"))
+            capi.csr_spmm(plan, rp, ci, v, Bd, again)
+            plan.destroy()
+            assert torch.equal(C, again), f"{name}: not reproducible"
+            _check(oracle, graph, B, C.cpu().numpy(), f"ordered {name} k={k}")
+        bad = torch.zeros(graph.rows, dtype=torch.int32, device=gpu)          # not a permutation
+        with pytest.raises(capi.HpSpmmError) as ei:
+            capi.Plan(graph.rows, graph.cols, rp, ci, k, 0, row_order=bad)
+        assert ei.value.code == capi.ERR_INVALID_ARG

@@ -202,8 +202,10 @@ int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, 
   return HPSPMM_OK;
 }
 
-// LDS bytes for a window's rows of B in the ordered strategy.
-constexpr int kOrderedLdsBytes = 32 << 10;
+// LDS of one workgroup of the ordered strategy, staging tiles included: the most that still lets
+// three workgroups share a CU's 160 KB (measured on the co-purchase graph, K = 64: 3.14 ms with
+// 32 KB for the rows of B, 2.92 ms with 45 KB, 3.39 ms with 46 KB, where only two fit).
+constexpr int kOrderedBlockLdsBytes = 52992;
 
 template <int K>
 int launch_ordered(const hpspmm_plan* p, const int32_t* rp, const float* v, const float* B, float* C,
@@ -541,7 +543,8 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
   int shift = 9;
   while (((int64_t)hpspmm::kWavesPerBlock * subwaves << shift) > hpspmm::kOrderedMaxWindow) --shift;
   const int window = (int)((int64_t)hpspmm::kWavesPerBlock * subwaves << shift);
-  const int cap = (int)(kOrderedLdsBytes / (k * 4));
+  const int64_t staging_bytes = 3 * hpspmm::kWavesPerBlock * subwaves * hpspmm::kTileStride * 4;
+  const int cap = (int)((kOrderedBlockLdsBytes - staging_bytes) / (k * 4));
   const int64_t windows = ceil_div(nnz, window);
   const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
 
@@ -645,7 +648,7 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
   const int64_t rows = p->rows;
   *d_order_out = nullptr;
   int32_t* d_label = nullptr;
-  unsigned long long* d_changed = nullptr;
+  uint32_t* d_changed = nullptr;
   struct Guard {
     void** q[2];
     ~Guard() {
@@ -654,17 +657,20 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
     }
   } guard{{(void**)&d_label, (void**)&d_changed}};
   HPSPMM_HIP(hipMalloc(&d_label, (size_t)rows * sizeof(int32_t)));
-  HPSPMM_HIP(hipMalloc(&d_changed, sizeof(unsigned long long)));
+  HPSPMM_HIP(hipMalloc(&d_changed, hpspmm::kClusterCounters * sizeof(uint32_t)));
+  std::vector<uint32_t> counters((size_t)hpspmm::kClusterCounters);
   hipLaunchKernelGGL(hpspmm::cluster_init_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock),
                      0, st, rows, d_label);
   for (int sweep = 0; sweep < kClusterMaxSweeps; ++sweep) {
-    HPSPMM_HIP(hipMemsetAsync(d_changed, 0, sizeof(unsigned long long), st));
+    HPSPMM_HIP(hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st));
     hipLaunchKernelGGL(hpspmm::cluster_sweep_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
                        dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_label, (uint32_t)sweep, d_changed);
-    unsigned long long changed = 0;
-    HPSPMM_HIP(hipMemcpyAsync(&changed, d_changed, sizeof changed, hipMemcpyDeviceToHost, st));
+    HPSPMM_HIP(hipMemcpyAsync(counters.data(), d_changed, counters.size() * sizeof(uint32_t), hipMemcpyDeviceToHost,
+                              st));
     HPSPMM_HIP(hipStreamSynchronize(st));
-    if ((int64_t)changed * 200 < rows) break;
+    int64_t changed = 0;
+    for (uint32_t c : counters) changed += c;
+    if (changed * 200 < rows) break;
   }
   // counting sort by label on the host: stable, hence the same order on every run
   std::vector<int32_t> label((size_t)rows), order((size_t)rows);

@@ -44,11 +44,13 @@ namespace hpspmm {
 // the most frequent.  Labels are updated in place (asynchronous propagation,
 // which does not oscillate the way the synchronous form does).  One wavefront
 // per row; the 64 sampled labels are sorted by a bitonic network of
-// wavefront shuffles.  changed[0] += rows whose label changed.
+// wavefront shuffles.  The kClusterCounters entries of changed[] together
+// count the rows whose label changed.
+constexpr int kClusterCounters = 1024;
 __global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                const int32_t* __restrict__ col,
                                                                int32_t* __restrict__ label, uint32_t sweep,
-                                                               unsigned long long* __restrict__ changed) {
+                                                               uint32_t* __restrict__ changed) {
   const int lane = threadIdx.x & 63;
   const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   if (r >= rows) return;
@@ -103,7 +105,7 @@ __global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, con
   const int best_count = (int)(best >> 32);
   if (lane == 0 && self_count < best_count && best_lab != mine) {
     label[r] = best_lab;
-    atomicAdd(changed, 1ull);
+    atomicAdd(&changed[r & (kClusterCounters - 1)], 1u);  // spread: one counter would serialise the first sweep
   }
 }
 
@@ -184,6 +186,7 @@ __global__ __launch_bounds__(kBlock) void ordered_hot_kernel(int64_t nnz, int wi
   __shared__ int32_t s_key[kOrderedMaxWindow];   // the window's columns, sorted (INT32_MAX pads)
   __shared__ int32_t s_sel[kOrderedMaxWindow / 2];  // selected columns (each occurs >= 2 times)
   __shared__ int32_t s_count;
+  __shared__ int32_t s_scan[kBlock];
   __shared__ int32_t s_hist[kOrderedHistMax + 1];  // s_hist[t] = runs of length >= t, t in [2, kOrderedHistMax]
   const int tid = threadIdx.x;
   const int64_t w = blockIdx.x;
@@ -216,29 +219,42 @@ __global__ __launch_bounds__(kBlock) void ordered_hot_kernel(int64_t nnz, int wi
     while (i + len < n && s_key[i + len] == s_key[i]) ++len;
     return len;
   };
-  for (int i = tid; i < n; i += kBlock) {
+  // every thread owns a contiguous stretch of the sorted window
+  const int per = (npow + kBlock - 1) / kBlock;
+  const int i_begin = tid * per < n ? tid * per : n;
+  const int i_end = i_begin + per < n ? i_begin + per : n;
+  for (int i = i_begin; i < i_end; ++i) {
     if (i > 0 && s_key[i] == s_key[i - 1]) continue;
     const int len = run_length(i);
-    if (len >= 2) {
-      const int top = len < kOrderedHistMax ? len : kOrderedHistMax;
-      for (int t = 2; t <= top; ++t) atomicAdd(&s_hist[t], 1);
-    }
+    if (len >= 2) atomicAdd(&s_hist[len < kOrderedHistMax ? len : kOrderedHistMax], 1);
   }
+  __syncthreads();
+  if (tid == 0)  // s_hist[t] = runs of exactly t  ->  runs of at least t
+    for (int t = kOrderedHistMax - 1; t >= 2; --t) s_hist[t] += s_hist[t + 1];
   __syncthreads();
   int threshold = 2;
   while (threshold < kOrderedHistMax && s_hist[threshold] > cap) ++threshold;
   const bool fits = s_hist[threshold] <= cap;  // always, as long as cap >= window / kOrderedHistMax
-  __syncthreads();
-  // selection in column order: one thread walks the run heads (windows are small and this is plan time)
-  if (tid == 0) {
-    int m = 0;
-    for (int i = 0; i < n && fits;) {
-      const int len = run_length(i);
-      if (len >= threshold && m < cap) s_sel[m++] = s_key[i];
-      i += len;
-    }
-    s_count = m;
+  // selection in column order: count per stretch, exclusive scan over the threads, write
+  int mine_sel = 0;
+  for (int i = i_begin; i < i_end && fits; ++i) {
+    if (i > 0 && s_key[i] == s_key[i - 1]) continue;
+    if (run_length(i) >= threshold) ++mine_sel;
   }
+  s_scan[tid] = mine_sel;
+  __syncthreads();
+  for (int off = 1; off < kBlock; off <<= 1) {
+    const int add = tid >= off ? s_scan[tid - off] : 0;
+    __syncthreads();
+    s_scan[tid] += add;
+    __syncthreads();
+  }
+  int at = s_scan[tid] - mine_sel;
+  for (int i = i_begin; i < i_end && fits; ++i) {
+    if (i > 0 && s_key[i] == s_key[i - 1]) continue;
+    if (run_length(i) >= threshold) s_sel[at++] = s_key[i];
+  }
+  if (tid == kBlock - 1) s_count = s_scan[tid];
   __syncthreads();
   const int m = s_count;
   for (int i = tid; i < cap; i += kBlock) wcols[w * cap + i] = i < m ? s_sel[i] : -1;

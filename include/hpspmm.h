@@ -105,10 +105,16 @@ const char *hpspmm_last_error(void);
 
 /*
  * Analyse the sparsity structure of A for a given k and build the device-side
- * work assignment (row-of-nonzero map, segment length, carry buffer).
+ * work assignment.  The plan picks a strategy (reported by
+ * hpspmm_plan_get_info): whole rows for small matrices; fixed-length segments
+ * of nonzeros with a carry buffer; the same inside column slices pinned to
+ * one XCD each when a few columns take most of the nonzeros ("routed"); or
+ * segments over a clustered row order with the reused rows of B held in LDS
+ * when the matrix is a graph with communities ("ordered").
  * Replaces the host-side preprocessing the reference does before timing:
- * CSR->COO expansion (spmm/mm/spmm_common.cpp:185-235) and the choice of
- * nnz_per_warp (spmm/mm/spmm_kernel.cu:749-751).  Synchronises `stream`.
+ * CSR->COO expansion (spmm/mm/spmm_common.cpp:185-235), the row re-ordering
+ * (:237-296) and the choice of nnz_per_warp (spmm/mm/spmm_kernel.cu:749-751).
+ * Synchronises `stream`.
  * Values are not read: the plan stays valid when d_val or B change, and must
  * be rebuilt when rowptr / col change.
  */

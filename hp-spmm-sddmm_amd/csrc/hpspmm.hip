@@ -255,8 +255,23 @@ int choose_shift(int64_t nnz, int64_t k) {
 // Column popularity: count[c] = nonzeros in column c, and the `want` most
 // referenced columns in order of decreasing count (ties by lower index, so the
 // choice is reproducible); columns referenced fewer than twice are dropped.
+// The result of the last call is kept per thread and handed out again for the same plan and
+// `want`: the routed and the hub-cache decisions of one plan ask for the same ranking.
+struct RankCache {
+  const hpspmm_plan* plan = nullptr;
+  int64_t want = 0;
+  std::vector<int32_t> count, ids;
+};
+thread_local RankCache g_rank_cache;
+
 int rank_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t want, hipStream_t st,
                  std::vector<int32_t>& count, std::vector<int32_t>& ids) {
+  if (g_rank_cache.plan == p && g_rank_cache.want == want) {
+    count = g_rank_cache.count;
+    ids = g_rank_cache.ids;
+    return HPSPMM_OK;
+  }
+  const int64_t asked = want;
   int32_t* d_count = nullptr;
   HPSPMM_HIP(hipMalloc(&d_count, (size_t)p->cols * sizeof(int32_t)));
   struct Guard {
@@ -277,6 +292,10 @@ int rank_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t want, hipSt
   ids.resize((size_t)want);
   std::sort(ids.begin(), ids.end(), hotter);
   while (!ids.empty() && count[ids.back()] < 2) ids.pop_back();
+  g_rank_cache.plan = p;
+  g_rank_cache.want = asked;
+  g_rank_cache.count = count;
+  g_rank_cache.ids = ids;
   return HPSPMM_OK;
 }
 
@@ -901,14 +920,18 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
 
 int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr, const int32_t* d_col,
                        int64_t k, uint32_t flags, void* stream, hpspmm_plan** plan_out) {
-  return plan_create_impl(rows, cols, nnz, d_rowptr, d_col, k, flags, nullptr, stream, plan_out);
+  const int rc = plan_create_impl(rows, cols, nnz, d_rowptr, d_col, k, flags, nullptr, stream, plan_out);
+  g_rank_cache = RankCache{};  // a later plan may get the same address
+  return rc;
 }
 
 int hpspmm_plan_create_ordered(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr,
                                const int32_t* d_col, int64_t k, uint32_t flags, const int32_t* d_row_order,
                                void* stream, hpspmm_plan** plan_out) {
   if (rows > 0 && !d_row_order) return fail(HPSPMM_ERR_INVALID_ARG, "d_row_order is NULL");
-  return plan_create_impl(rows, cols, nnz, d_rowptr, d_col, k, flags, d_row_order, stream, plan_out);
+  const int rc = plan_create_impl(rows, cols, nnz, d_rowptr, d_col, k, flags, d_row_order, stream, plan_out);
+  g_rank_cache = RankCache{};
+  return rc;
 }
 
 int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {

@@ -35,6 +35,7 @@ constexpr int kBlock = 256;         // threads per workgroup = 4 wavefronts
 constexpr int kWavesPerBlock = 4;
 constexpr int kBatch = 8;           // B-row fragments in flight per lane
 constexpr int kXcds = 8;            // accelerator complex dies, each with its own L2
+constexpr int kLongChain = 32;      // fix-up: a row over this many segments is added up by a whole wavefront
 
 // LDS written by some lanes of a wavefront and read by others: LDS operations
 // of one wavefront complete in issue order, so only the compiler has to be
@@ -475,9 +476,32 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
   }
   const bool empty = valid && lb == hb;
   const bool split = valid && lb != hb && ((int64_t)lb >> shift) != ((int64_t)(hb - 1) >> shift);
+  // a row over many segments is put together by the whole wavefront, see below
+  const bool chain = split && (((int64_t)(hb - 1) >> shift) - ((int64_t)lb >> shift)) >= kLongChain;
   const uint64_t m_empty = __ballot(empty);
-  const uint64_t m_split = __ballot(split);
-  if ((m_empty | m_split) == 0) return;
+  const uint64_t m_split = __ballot(split && !chain);
+  uint64_t m_chain = __ballot(chain);
+  if ((m_empty | m_split | m_chain) == 0) return;
+
+  auto add = [](float4& a, const float4& b) {
+    a.x += b.x;
+    a.y += b.y;
+    a.z += b.z;
+    a.w += b.w;
+  };
+  // acc += head[g0] + head[g0 + step] + ... (g <= gb), 8 slots in flight at a time, in that order
+  auto add_heads = [&](float4& acc, int64_t g0, int64_t gb, int64_t step) {
+    int64_t g = g0;
+    for (; g + (kBatch - 1) * step <= gb; g += kBatch * step) {
+      float4 part[kBatch];
+#pragma unroll
+      for (int q = 0; q < kBatch; ++q)
+        part[q] = *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * (g + q * step)) * K + 4 * l);
+#pragma unroll
+      for (int q = 0; q < kBatch; ++q) add(acc, part[q]);
+    }
+    for (; g <= gb; g += step) add(acc, *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * g) * K + 4 * l));
+  };
 
   for (int i = sub; i < 64; i += P) {
     // every lane takes part in the shuffles; only then do the sub-waves diverge
@@ -490,29 +514,33 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
       const int64_t ga = (int64_t)lb_i >> shift;
       const int64_t gb = (int64_t)(hb_i - 1) >> shift;
       float4 acc = *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * ga + 1) * K + 4 * l);
-      int64_t g = ga + 1;
-      for (; g + kBatch <= gb + 1; g += kBatch) {
-        float4 part[kBatch];
-#pragma unroll
-        for (int q = 0; q < kBatch; ++q)
-          part[q] = *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * (g + q)) * K + 4 * l);
-#pragma unroll
-        for (int q = 0; q < kBatch; ++q) {
-          acc.x += part[q].x;
-          acc.y += part[q].y;
-          acc.z += part[q].z;
-          acc.w += part[q].w;
-        }
-      }
-      for (; g <= gb; ++g) {
-        const float4 part = *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * g) * K + 4 * l);
-        acc.x += part.x;
-        acc.y += part.y;
-        acc.z += part.z;
-        acc.w += part.w;
-      }
+      add_heads(acc, ga + 1, gb, 1);
       *out = acc;
     }
+  }
+  // Long chains, one row at a time, all P sub-waves together: sub-wave s adds the heads ga+1+s,
+  // ga+1+s+P, ...; sub-wave 0 then adds tail[ga] and the P partial sums in the order of s.  (A
+  // single dense row of 100k nonzeros cut into 1500 segments: 80 us for one sub-wave alone.)
+  while (m_chain) {
+    const int i = __ffsll((long long)m_chain) - 1;
+    m_chain &= m_chain - 1;
+    const int32_t lb_i = __shfl(lb, i);
+    const int32_t hb_i = __shfl(hb, i);
+    const int64_t ga = (int64_t)lb_i >> shift;
+    const int64_t gb = (int64_t)(hb_i - 1) >> shift;
+    float4 part = make_float4(0.f, 0.f, 0.f, 0.f);
+    add_heads(part, ga + 1 + sub, gb, P);
+    float4 acc = *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * ga + 1) * K + 4 * l);
+#pragma unroll
+    for (int s = 0; s < P; ++s) {
+      float4 t;
+      t.x = __shfl(part.x, s * G + l);
+      t.y = __shfl(part.y, s * G + l);
+      t.z = __shfl(part.z, s * G + l);
+      t.w = __shfl(part.w, s * G + l);
+      add(acc, t);
+    }
+    if (sub == 0) *reinterpret_cast<float4*>(C + (uint64_t)(r0 + i) * K + 4 * l) = acc;
   }
 }
 

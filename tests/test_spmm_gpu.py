@@ -580,3 +580,32 @@ def test_clustering_finds_planted_communities(pkg, oracle, gpu):
     C, info = _run(pkg, gpu, sq, Bs, flags)
     assert info["strategy"] == capi.STRATEGY_ORDERED
     _check(oracle, sq, Bs, C, "clustered unsymmetric square matrix")
+
+
+def test_extreme_shapes(pkg, oracle, gpu):
+    """One dense row among singletons, a permutation matrix, a single column, a single row: the shapes
+    that stress the carry chains, the row lists and the hot-column logic of every strategy."""
+    capi = pkg.capi
+    rng = np.random.default_rng(9)
+    n = 300_000
+    cases = {
+        "dense row": (n, n, np.concatenate([[0, n], n + np.arange(1, n, dtype=np.int64)]).astype(np.int32),
+                      np.concatenate([np.arange(n, dtype=np.int32), rng.integers(0, n, n - 1).astype(np.int32)]), 64),
+        "permutation": (n, n, np.arange(n + 1, dtype=np.int32), rng.permutation(n).astype(np.int32), 32),
+        "one column": (n, 1, (np.arange(n + 1, dtype=np.int64) * 4).astype(np.int32), np.zeros(4 * n, np.int32), 128),
+        "one row": (1, n, np.array([0, n], np.int32), np.arange(n, dtype=np.int32), 32),
+    }
+    strategies = [("auto", capi.PLAN_DEFAULT), ("seg", capi.PLAN_FORCE_SEGMENTS), ("seg32", capi.PLAN_FORCE_SEGMENTS
+                  | capi.plan_segment_shift(5)), ("routed", capi.PLAN_FORCE_ROUTED),
+                  ("cluster", capi.PLAN_CLUSTER | capi.PLAN_FORCE_SEGMENTS | capi.PLAN_NO_HUB_CACHE)]
+    for what, (rows, cols, rowptr, col, k) in cases.items():
+        val = rng.uniform(-1, 1, col.size).astype(np.float32)
+        g = pkg.graphs.CSR(rows, cols, rowptr, col, val)
+        B = rng.standard_normal((cols, k)).astype(np.float32)
+        hi = min(rows, 64)
+        C64, S64 = oracle.csr_spmm_f64_rows(g.rowptr, g.col, g.val, B, 0, hi)
+        for name, flags in strategies:
+            C, _ = _run(pkg, gpu, g, B, flags)
+            assert not np.isnan(C).any(), f"{what} {name}: C not fully written"
+            err, _ = oracle.max_norm_err(C[:hi], C64, S64)
+            assert err <= TOL, f"{what} {name}: normalised error {err:.3e}"

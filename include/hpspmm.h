@@ -71,7 +71,9 @@ typedef enum hpspmm_status {
 #define HPSPMM_PLAN_CLUSTER 4096u     /* square A: always look for clusters of rows that share columns and use the
                                          ordered strategy on the order found (default: only for large graphs
                                          without hot columns, and only if >= 15 % of the nonzeros then read B
-                                         from LDS) */
+                                         from LDS).  The clustering updates its labels asynchronously: two
+                                         plans of one matrix may order the rows differently and then differ
+                                         in the last bits of C; one plan always gives the same bits */
 #define HPSPMM_PLAN_NO_CLUSTER 8192u  /* never */
 
 /* strategy reported by hpspmm_plan_get_info */

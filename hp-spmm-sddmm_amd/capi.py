@@ -30,6 +30,7 @@ PLAN_FORCE_ROUTED = 64
 PLAN_NO_ROUTED = 128
 PLAN_CLUSTER = 4096
 PLAN_NO_CLUSTER = 8192
+PLAN_NO_ROW_TILES = 16384
 
 
 def plan_hub_log2(log2_rows):

@@ -1,0 +1,129 @@
+// gfx950 device code for the rows strategy over *row tiles*: the layout a plan
+// builds for a small matrix so that one SpMM is a single launch whose every
+// wavefront has the same, short chain of dependent memory round trips.
+//
+// A small SpMM (the 20k-vertex citation graph: 6 us) is bound by that chain, not
+// by bandwidth: a sub-wave that walks a CSR row goes rowptr -> col/val -> B ->
+// store, and a row longer than one staging step repeats col -> B once per step
+// while the rest of its wavefront idles.  Here the plan cuts every row into
+// slots of 8 nonzeros and packs 8 slots into a 64-entry tile, one tile per
+// wavefront:
+//
+//   tcol[tile][64]   column of every entry, -1 = padding
+//   tdesc[tile][8]   per slot: row (-1 = padding slot), index of its first value
+//
+// Both are indexed by the wavefront's own number, so columns arrive after one
+// round trip and the B rows and the values after the second.  A row of up to
+// 8 / 16 / 32 / 64 nonzeros takes 1 / 2 / 4 / 8 adjacent slots of one tile
+// (tiles hold rows of one size class only, so the reduction over a row's slots
+// is the same wavefront shuffle for the whole tile); a longer row owns
+// consecutive tiles that one wavefront works through.  Long rows come first in
+// the grid, since their chain is the longest.
+//
+// K > 32 is served in 32-column tiles of B and C by K/32 workgroups per group
+// of row tiles (workgroup b serves column tile b % (K/32), so an XCD only ever
+// touches one column tile of B).  A wavefront that serves two or four column
+// tiles itself, with 16 or 32 loads in flight per lane, is slower (20k-vertex
+// citation graph, K=128: 5.7 us with one, 6.4 with two, 8.2 with four).
+//
+// What this replaces in the reference: the row-per-warp kernels
+// topoCacheSPMMKernel / topoCacheCoarsenSPMMKernel (spmm/mm/spmm_kernel.cu:247-370).
+#pragma once
+
+#include "spmm_kernels.hpp"
+
+namespace hpspmm {
+
+constexpr int kSlot = 8;          // nonzeros per slot = lanes per sub-wave at a 32-column tile
+constexpr int kSlotsPerTile = 8;  // slots per tile = sub-waves per wavefront
+constexpr int kRowTile = kSlot * kSlotsPerTile;
+
+// acc += the slot's (up to 8) products.  `c` is this lane's entry of the tile, `v` its value.
+template <int K>
+__device__ __forceinline__ void gather_slot(float4& acc, int32_t c, float v, int tid, int base, int l, int k0,
+                                            int32_t* s_col, float* s_val, const float* __restrict__ B) {
+  s_col[tid] = c;
+  wave_lds_fence();
+  int32_t cc[kSlot];
+  float4 b[kSlot];
+#pragma unroll
+  for (int i = 0; i < kSlot; ++i) cc[i] = s_col[base + i];
+  // predicated loads, all in flight together; padding reads nothing, so a
+  // non-finite value in an unreferenced row of B cannot leak in
+#pragma unroll
+  for (int i = 0; i < kSlot; ++i) {
+    b[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (cc[i] >= 0) b[i] = load_b_tile<K>(B, cc[i], k0, l);
+  }
+  s_val[tid] = v;
+  wave_lds_fence();
+#pragma unroll
+  for (int i = 0; i < kSlot; ++i) fma4(acc, s_val[base + i], b[i]);
+  wave_lds_fence();
+}
+
+// Wavefront w < n_loop works through the tiles of long row w (ldesc[w] = first
+// tile, tile count); wavefront w >= n_loop owns tile loop_tiles + (w - n_loop).
+// Tiles [loop_tiles, end3) hold 64-nonzero rows (8 slots each), [end3, end2)
+// 4-slot rows, [end2, end1) 2-slot rows, the rest 1-slot rows.
+template <int K, int WPB>
+__global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves, int32_t n_loop, int32_t loop_tiles,
+                                                               int32_t end3, int32_t end2, int32_t end1,
+                                                               const int2* __restrict__ ldesc,
+                                                               const int32_t* __restrict__ tcol,
+                                                               const int2* __restrict__ tdesc,
+                                                               const float* __restrict__ val,
+                                                               const float* __restrict__ B, float* __restrict__ C) {
+  constexpr int T = K / 32;
+  __shared__ int32_t s_col[WPB * 64];
+  __shared__ float s_val[WPB * 64];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int l = lane & (kSlot - 1);
+  const int s = lane / kSlot;
+  const int base = tid - l;
+  const int k0 = (int)(blockIdx.x % T) * 32;
+  const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(blockIdx.x / T) * WPB + (tid >> 6));
+  if (w >= n_waves) return;
+
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  int lg = 3;
+  int32_t row;
+  if (w >= n_loop) {
+    const int32_t tile = loop_tiles + (w - n_loop);
+    lg = tile < end3 ? 3 : tile < end2 ? 2 : tile < end1 ? 1 : 0;
+    const int32_t c = tcol[(int64_t)tile * kRowTile + lane];
+    const int2 d = tdesc[(int64_t)tile * kSlotsPerTile + s];
+    const float v = c >= 0 ? val[d.y + l] : 0.f;
+    row = d.x;
+    gather_slot<K>(acc, c, v, tid, base, l, k0, s_col, s_val, B);
+  } else {
+    const int2 ld = ldesc[w];
+    int32_t c = tcol[(int64_t)ld.x * kRowTile + lane];
+    int2 d = tdesc[(int64_t)ld.x * kSlotsPerTile + s];
+    row = d.x;
+    for (int32_t t = 0; t < ld.y; ++t) {
+      const float v = c >= 0 ? val[d.y + l] : 0.f;
+      const int32_t c_now = c;
+      if (t + 1 < ld.y) {  // next tile's entries on their way while this one is gathered
+        c = tcol[(int64_t)(ld.x + t + 1) * kRowTile + lane];
+        d = tdesc[(int64_t)(ld.x + t + 1) * kSlotsPerTile + s];
+      }
+      gather_slot<K>(acc, c_now, v, tid, base, l, k0, s_col, s_val, B);
+    }
+  }
+  // the slots of a row are adjacent and aligned to their count: xor shuffles, in a fixed order
+#pragma unroll
+  for (int step = 0; step < 3; ++step) {
+    if (lg > step) {
+      acc.x += __shfl_xor(acc.x, kSlot << step);
+      acc.y += __shfl_xor(acc.y, kSlot << step);
+      acc.z += __shfl_xor(acc.z, kSlot << step);
+      acc.w += __shfl_xor(acc.w, kSlot << step);
+    }
+  }
+  if ((s & ((1 << lg) - 1)) == 0 && row >= 0) store_result(C + (uint64_t)(uint32_t)row * K + k0 + 4 * l, acc);
+}
+
+}  // namespace hpspmm

@@ -75,6 +75,7 @@ typedef enum hpspmm_status {
                                          plans of one matrix may order the rows differently and then differ
                                          in the last bits of C; one plan always gives the same bits */
 #define HPSPMM_PLAN_NO_CLUSTER 8192u  /* never */
+#define HPSPMM_PLAN_NO_ROW_TILES 16384u /* rows strategy: walk the caller's CSR arrays instead of building row tiles */
 
 /* strategy reported by hpspmm_plan_get_info */
 #define HPSPMM_STRATEGY_ROWS 1

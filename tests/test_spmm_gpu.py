@@ -48,6 +48,7 @@ def _check(oracle, g, B, C, what=""):
 
 def _strategies(capi):
     return [("auto", capi.PLAN_DEFAULT), ("rows", capi.PLAN_FORCE_ROWS),
+            ("rows_csr", capi.PLAN_FORCE_ROWS | capi.PLAN_NO_ROW_TILES),
             ("seg", capi.PLAN_FORCE_SEGMENTS),
             ("seg8_nohub", capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(3) | capi.PLAN_NO_HUB_CACHE),
             ("seg64_noremap", capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(6) | capi.PLAN_NO_XCD_REMAP),
@@ -595,7 +596,9 @@ def test_extreme_shapes(pkg, oracle, gpu):
         "one column": (n, 1, (np.arange(n + 1, dtype=np.int64) * 4).astype(np.int32), np.zeros(4 * n, np.int32), 128),
         "one row": (1, n, np.array([0, n], np.int32), np.arange(n, dtype=np.int32), 32),
     }
-    strategies = [("auto", capi.PLAN_DEFAULT), ("seg", capi.PLAN_FORCE_SEGMENTS), ("seg32", capi.PLAN_FORCE_SEGMENTS
+    strategies = [("auto", capi.PLAN_DEFAULT), ("rows", capi.PLAN_FORCE_ROWS),
+                  ("rows_csr", capi.PLAN_FORCE_ROWS | capi.PLAN_NO_ROW_TILES),
+                  ("seg", capi.PLAN_FORCE_SEGMENTS), ("seg32", capi.PLAN_FORCE_SEGMENTS
                   | capi.plan_segment_shift(5)), ("routed", capi.PLAN_FORCE_ROUTED),
                   ("cluster", capi.PLAN_CLUSTER | capi.PLAN_FORCE_SEGMENTS | capi.PLAN_NO_HUB_CACHE)]
     for what, (rows, cols, rowptr, col, k) in cases.items():
@@ -609,3 +612,39 @@ def test_extreme_shapes(pkg, oracle, gpu):
             assert not np.isnan(C).any(), f"{what} {name}: C not fully written"
             err, _ = oracle.max_norm_err(C[:hi], C64, S64)
             assert err <= TOL, f"{what} {name}: normalised error {err:.3e}"
+
+
+def test_row_tiles_layout_and_fallback(pkg, oracle, gpu):
+    """The rows strategy builds row tiles (every size class of row present: 1, 2, 4, 8 slots, several
+    tiles) unless padding would dominate (mostly empty rows): then it walks the CSR arrays.  Both agree
+    with the oracle; the tile layout shows in the plan's workspace."""
+    capi = pkg.capi
+    rng = np.random.default_rng(21)
+    # one row of every length 0..200, shuffled, twice over
+    lens = rng.permutation(np.concatenate([np.arange(201), np.arange(201)])).astype(np.int64)
+    rows, cols = lens.size, 5000
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = rng.integers(0, cols, int(lens.sum())).astype(np.int32)
+    val = rng.uniform(-1, 1, col.size).astype(np.float32)
+    g = pkg.graphs.CSR(rows, cols, rowptr, col, val)
+    for k in (32, 64, 128):
+        B = rng.standard_normal((cols, k)).astype(np.float32)
+        C, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+        assert info["strategy"] == capi.STRATEGY_ROWS
+        assert info["workspace_bytes"] >= 4 * col.size       # tcol alone is at least one int per nonzero
+        _check(oracle, g, B, C, f"all row lengths k={k} tiles")
+        C2, info2 = _run(pkg, gpu, g, B, capi.PLAN_NO_ROW_TILES)
+        assert info2["strategy"] == capi.STRATEGY_ROWS and info2["workspace_bytes"] < 4 * col.size
+        _check(oracle, g, B, C2, f"all row lengths k={k} csr")
+    # 400k rows, 2k nonzeros: 50k tiles of padding for 2k entries - not built
+    rows = 400_000
+    lens = np.zeros(rows, np.int64)
+    lens[rng.choice(rows, 1000, replace=False)] = 2
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = rng.integers(0, 777, 2000).astype(np.int32)
+    val = rng.uniform(-1, 1, 2000).astype(np.float32)
+    g = pkg.graphs.CSR(rows, 777, rowptr, col, val)
+    B = rng.standard_normal((777, 32)).astype(np.float32)
+    C, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+    assert info["strategy"] == capi.STRATEGY_ROWS and info["workspace_bytes"] < 100_000
+    _check(oracle, g, B, C, "mostly empty rows")

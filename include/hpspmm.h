@@ -51,7 +51,7 @@ typedef enum hpspmm_status {
 /* hpspmm_plan_create flags */
 #define HPSPMM_PLAN_DEFAULT 0u
 #define HPSPMM_PLAN_NO_VALIDATE 1u    /* skip the device-side CSR check */
-#define HPSPMM_PLAN_FORCE_ROWS 2u     /* always use the whole-row kernel */
+#define HPSPMM_PLAN_FORCE_ROWS 2u     /* always use the whole-row strategy */
 #define HPSPMM_PLAN_FORCE_SEGMENTS 4u /* always use the nnz-segment kernel + carry fix-up */
 #define HPSPMM_PLAN_NO_XCD_REMAP 8u   /* keep the hardware's round-robin workgroup->XCD order */
 #define HPSPMM_PLAN_HUB_CACHE 16u     /* segments strategy: always keep the most referenced rows of B in a compact
@@ -109,8 +109,10 @@ const char *hpspmm_last_error(void);
 /*
  * Analyse the sparsity structure of A for a given k and build the device-side
  * work assignment.  The plan picks a strategy (reported by
- * hpspmm_plan_get_info): whole rows for small matrices; fixed-length segments
- * of nonzeros with a carry buffer; the same inside column slices pinned to
+ * hpspmm_plan_get_info): whole rows for small matrices (the rows cut into
+ * 8-nonzero slots and packed, by length class, into one 64-entry tile per
+ * wavefront, so that a microsecond-scale SpMM is one launch with a two-step
+ * dependent chain); fixed-length segments of nonzeros with a carry buffer; the same inside column slices pinned to
  * one XCD each when a few columns take most of the nonzeros ("routed"); or
  * segments over a clustered row order with the reused rows of B held in LDS
  * when the matrix is a graph with communities ("ordered").

@@ -117,7 +117,7 @@ struct hpspmm_plan {
   int32_t* d_tcol = nullptr;  // [rt_tiles * 64] column of every tile entry, -1 = padding
   int2* d_tdesc = nullptr;    // [rt_tiles * 8] per slot: row (-1 = padding), index of its first value
   int2* d_ldesc = nullptr;    // [rt_loop] per long row: first tile, tile count
-  int32_t rt_tiles = 0, rt_waves = 0, rt_loop = 0, rt_loop_tiles = 0, rt_end3 = 0, rt_end2 = 0, rt_end1 = 0;
+  int32_t rt_tiles = 0, rt_waves = 0, rt_loop = 0, rt_wg = 0, rt_loop_tiles = 0, rt_end3 = 0, rt_end2 = 0, rt_end1 = 0;
   int64_t workspace_bytes = 0;
 };
 
@@ -169,7 +169,12 @@ int launch_rows(int64_t rows, int64_t cols, const int32_t* rp, const int32_t* ci
 // only serves matrices below 2^21 nonzeros.  Skipped (the kernel then walks the CSR arrays)
 // when padding would blow the layout up, which is what a matrix of mostly empty rows does.
 constexpr int64_t kRowTilePadFactor = 8;
-constexpr int64_t kRowTileMaxNnz = 1 << 23;  // beyond this (rows strategy forced on a large matrix) not built either
+constexpr int64_t kRowTileMaxNnz = (int64_t)1 << 28;
+// automatic use of the rows strategy beyond tiny matrices
+constexpr int64_t kRowsAutoMaxNnz = 1 << 24;
+constexpr int64_t kRowsAutoMaxWork = (int64_t)1 << 30;  // nnz * K
+constexpr int64_t kRowsAutoMaxRow = 1 << 16;
+constexpr int32_t kRowTileWorkgroupRows = 512;  // rows beyond this many nonzeros get a whole workgroup  // beyond this (rows strategy forced on a large matrix) not built either
 
 int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st) {
   using hpspmm::kSlot;
@@ -198,10 +203,14 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
   std::vector<int32_t> tcol((size_t)tiles * kTile, -1);
   std::vector<int2> tdesc((size_t)tiles * kSlotsPerTile, make_int2(-1, 0));
   std::vector<int2> ldesc((size_t)(count[4] > 0 ? count[4] : 1));
-  int64_t group[4] = {0, 0, 0, 0}, next_loop_tile = 0, n_loop = 0;
+  int64_t group[4] = {0, 0, 0, 0}, next_loop_tile = 0, n_loop = 0, n_wg = 0;
+  // two passes: the rows that get a whole workgroup first in ldesc (and in the tile order), then the rest
+  for (int pass = 0; pass < 2; ++pass)
   for (int64_t r = 0; r < rows; ++r) {
     const int32_t lb = rp[r], n = rp[r + 1] - lb;
     const int c = class_of(n);
+    if ((pass == 0) != (n > kRowTileWorkgroupRows)) continue;
+    if (pass == 0) ++n_wg;
     int64_t slot;  // first slot of the row
     int64_t slots;
     if (c == 4) {
@@ -238,6 +247,7 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
   HPSPMM_HIP(hipStreamSynchronize(st));  // the host vectors go out of scope
   p->rt_tiles = (int32_t)tiles;
   p->rt_loop = (int32_t)n_loop;
+  p->rt_wg = (int32_t)n_wg;
   p->rt_loop_tiles = (int32_t)loop_tiles;
   p->rt_end3 = (int32_t)first[2];
   p->rt_end2 = (int32_t)first[1];
@@ -254,12 +264,29 @@ int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, flo
                      p->d_tcol, p->d_tdesc, v, B, C);
   return HPSPMM_OK;
 }
+template <int K, int WPB>
+int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
+  const int64_t wave_items = (p->rt_loop - p->rt_wg) + (p->rt_tiles - p->rt_loop_tiles);
+  const int64_t blocks = (p->rt_wg + ceil_div(wave_items, WPB)) * (K / 32);
+  if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
+                     p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->rt_end3, p->rt_end2, p->rt_end1, p->d_ldesc,
+                     p->d_tcol, p->d_tdesc, v, B, C);
+  return HPSPMM_OK;
+}
+
 // One wavefront per workgroup while the grid stays small (20k-vertex citation graph, K=32:
-// 3.66 us against 3.75 us with four), four beyond that.
+// 3.66 us against 3.75 us with four), four beyond that.  A matrix with rows beyond
+// kRowTileWorkgroupRows nonzeros gets a workgroup of 8 or 16 wavefronts on each of those rows:
+// one wavefront needs about 0.6 us per 64 nonzeros, which a 16k-nonzero row turns into 150 us.
 constexpr int64_t kRowTileSmallGrid = 1 << 15;
 
 template <int K>
 int launch_row_tiles(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
+  if (p->rt_wg > 0) {
+    if (p->max_row_nnz > 8192) return launch_row_tiles_wg<K, 16>(p, v, B, C, st);
+    return launch_row_tiles_wg<K, 8>(p, v, B, C, st);
+  }
   if ((int64_t)p->rt_waves * (K / 32) <= kRowTileSmallGrid) return launch_row_tiles_w<K, 1>(p, v, B, C, st);
   return launch_row_tiles_w<K, hpspmm::kWavesPerBlock>(p, v, B, C, st);
 }
@@ -925,6 +952,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   p->empty_rows = stats[1];
   p->xcd_remap = !(flags & HPSPMM_PLAN_NO_XCD_REMAP);
 
+  bool rows_need_tiles = false;  // rows strategy chosen on the strength of the row tiles
   if (!fast_k(k)) {
     p->strategy = HPSPMM_STRATEGY_GENERIC_K;
   } else if (d_order && nnz > 0) {
@@ -939,12 +967,23 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   } else if (flags & (HPSPMM_PLAN_FORCE_SEGMENTS | HPSPMM_PLAN_FORCE_ROUTED)) {
     p->strategy = HPSPMM_STRATEGY_SEGMENTS;  // the routed layout is built on top of it below
   } else {
-    // Whole rows (one launch; long rows get a wavefront each) when the matrix is
-    // small enough that a second (fix-up) launch would be felt and no row is so
-    // long that a single wavefront would be the critical path.
-    const bool small = nnz < (1 << 21);
-    p->strategy = (nnz == 0 || (small && p->max_row_nnz <= 4096)) ? HPSPMM_STRATEGY_ROWS : HPSPMM_STRATEGY_SEGMENTS;
+    // Whole rows (one launch) while the matrix is small enough that the second and third launch of
+    // the other strategies are felt and L2 reuse across rows is not yet what decides: measured
+    // against segments / routed / ordered on scaled copies of the benchmark graphs, row tiles win up
+    // to about 2^23 nonzeros at K=128 and 2^25 at K=32 (R-MAT, 3.7 M nonzeros, K=32: 42 vs 198 us).
+    const bool tiny = nnz < (1 << 21) && p->max_row_nnz <= 4096;  // fine even over the CSR arrays
+    const bool mid = nnz < kRowsAutoMaxNnz && nnz * k < kRowsAutoMaxWork && p->max_row_nnz <= kRowsAutoMaxRow;
+    p->strategy = (nnz == 0 || tiny || mid) ? HPSPMM_STRATEGY_ROWS : HPSPMM_STRATEGY_SEGMENTS;
+    rows_need_tiles = !(nnz == 0 || tiny);
   }
+
+  if (p->strategy == HPSPMM_STRATEGY_ROWS && rows > 0 && nnz < kRowTileMaxNnz && !(flags & HPSPMM_PLAN_NO_ROW_TILES)) {
+    if (int rc = build_row_tiles(p, d_rowptr, d_col, st)) {
+      hpspmm_plan_destroy(p);
+      return rc;
+    }
+  }
+  if (p->strategy == HPSPMM_STRATEGY_ROWS && rows_need_tiles && !p->d_tcol) p->strategy = HPSPMM_STRATEGY_SEGMENTS;
 
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS) {
     int forced = (int)((flags >> 8) & 0xFu);
@@ -1000,12 +1039,6 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     if (rc == HPSPMM_OK) rc = build_ordered(p, d_rowptr, d_col, d_order, want_cluster ? 0.0 : kClusterMinServed, st);
     if (d_order) (void)hipFree(d_order);
     if (rc) {
-      hpspmm_plan_destroy(p);
-      return rc;
-    }
-  }
-  if (p->strategy == HPSPMM_STRATEGY_ROWS && rows > 0 && nnz < kRowTileMaxNnz && !(flags & HPSPMM_PLAN_NO_ROW_TILES)) {
-    if (int rc = build_row_tiles(p, d_rowptr, d_col, st)) {
       hpspmm_plan_destroy(p);
       return rc;
     }

@@ -62,6 +62,26 @@ __device__ __forceinline__ void gather_slot(float4& acc, int32_t c, float v, int
   wave_lds_fence();
 }
 
+// acc += the products of tiles [t0, t1) of one long row, worked through by one wavefront.
+template <int K>
+__device__ __forceinline__ void gather_tiles(float4& acc, int32_t t0, int32_t t1, int lane, int s, int l, int tid,
+                                             int base, int k0, int32_t* s_col, float* s_val,
+                                             const int32_t* __restrict__ tcol, const int2* __restrict__ tdesc,
+                                             const float* __restrict__ val, const float* __restrict__ B) {
+  if (t0 >= t1) return;
+  int32_t c = tcol[(int64_t)t0 * kRowTile + lane];
+  int2 d = tdesc[(int64_t)t0 * kSlotsPerTile + s];
+  for (int32_t t = t0; t < t1; ++t) {
+    const float v = c >= 0 ? val[d.y + l] : 0.f;
+    const int32_t c_now = c;
+    if (t + 1 < t1) {  // next tile's entries on their way while this one is gathered
+      c = tcol[(int64_t)(t + 1) * kRowTile + lane];
+      d = tdesc[(int64_t)(t + 1) * kSlotsPerTile + s];
+    }
+    gather_slot<K>(acc, c_now, v, tid, base, l, k0, s_col, s_val, B);
+  }
+}
+
 // Wavefront w < n_loop works through the tiles of long row w (ldesc[w] = first
 // tile, tile count); wavefront w >= n_loop owns tile loop_tiles + (w - n_loop).
 // Tiles [loop_tiles, end3) hold 64-nonzero rows (8 slots each), [end3, end2)
@@ -100,20 +120,98 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
     gather_slot<K>(acc, c, v, tid, base, l, k0, s_col, s_val, B);
   } else {
     const int2 ld = ldesc[w];
-    int32_t c = tcol[(int64_t)ld.x * kRowTile + lane];
-    int2 d = tdesc[(int64_t)ld.x * kSlotsPerTile + s];
-    row = d.x;
-    for (int32_t t = 0; t < ld.y; ++t) {
-      const float v = c >= 0 ? val[d.y + l] : 0.f;
-      const int32_t c_now = c;
-      if (t + 1 < ld.y) {  // next tile's entries on their way while this one is gathered
-        c = tcol[(int64_t)(ld.x + t + 1) * kRowTile + lane];
-        d = tdesc[(int64_t)(ld.x + t + 1) * kSlotsPerTile + s];
-      }
-      gather_slot<K>(acc, c_now, v, tid, base, l, k0, s_col, s_val, B);
-    }
+    row = tdesc[(int64_t)ld.x * kSlotsPerTile].x;
+    gather_tiles<K>(acc, ld.x, ld.x + ld.y, lane, s, l, tid, base, k0, s_col, s_val, tcol, tdesc, val, B);
   }
   // the slots of a row are adjacent and aligned to their count: xor shuffles, in a fixed order
+#pragma unroll
+  for (int step = 0; step < 3; ++step) {
+    if (lg > step) {
+      acc.x += __shfl_xor(acc.x, kSlot << step);
+      acc.y += __shfl_xor(acc.y, kSlot << step);
+      acc.z += __shfl_xor(acc.z, kSlot << step);
+      acc.w += __shfl_xor(acc.w, kSlot << step);
+    }
+  }
+  if ((s & ((1 << lg) - 1)) == 0 && row >= 0) store_result(C + (uint64_t)(uint32_t)row * K + k0 + 4 * l, acc);
+}
+
+// The same with a whole workgroup of WPB wavefronts on each of the n_wg longest rows (the first
+// n_wg entries of ldesc; workgroups [0, n_wg) of a column tile; the row's tiles dealt in contiguous
+// shares, the shares' sums added in wavefront order through LDS), for matrices whose longest rows
+// would otherwise be the critical path of the launch.  The wavefronts of the other workgroups take
+// one remaining long row or one ordinary tile each, as above.
+template <int K, int WPB>
+__global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_tiles, int32_t n_wg, int32_t n_loop,
+                                                                    int32_t loop_tiles, int32_t end3, int32_t end2,
+                                                                    int32_t end1, const int2* __restrict__ ldesc,
+                                                                    const int32_t* __restrict__ tcol,
+                                                                    const int2* __restrict__ tdesc,
+                                                                    const float* __restrict__ val,
+                                                                    const float* __restrict__ B,
+                                                                    float* __restrict__ C) {
+  constexpr int T = K / 32;
+  __shared__ int32_t s_col[WPB * 64];
+  __shared__ float s_val[WPB * 64];
+  __shared__ float4 s_part[WPB][kSlot];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l = lane & (kSlot - 1);
+  const int s = lane / kSlot;
+  const int base = tid - l;
+  const int k0 = (int)(blockIdx.x % T) * 32;
+  const int32_t blk = (int32_t)(blockIdx.x / T);
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+
+  if (blk < n_wg) {  // uniform over the workgroup: every wavefront reaches the barrier
+    const int2 ld = ldesc[blk];
+    const int32_t per = (ld.y + WPB - 1) / WPB;
+    const int32_t t0 = ld.x + wave * per;
+    const int32_t t1 = t0 + per < ld.x + ld.y ? t0 + per : ld.x + ld.y;
+    gather_tiles<K>(acc, t0, t1, lane, s, l, tid, base, k0, s_col, s_val, tcol, tdesc, val, B);
+#pragma unroll
+    for (int off = kSlot; off < 64; off <<= 1) {
+      acc.x += __shfl_xor(acc.x, off);
+      acc.y += __shfl_xor(acc.y, off);
+      acc.z += __shfl_xor(acc.z, off);
+      acc.w += __shfl_xor(acc.w, off);
+    }
+    if (lane < kSlot) s_part[wave][lane] = acc;
+    __syncthreads();
+    if (tid < kSlot) {
+      float4 sum = s_part[0][tid];
+      for (int j = 1; j < WPB; ++j) {
+        const float4 p = s_part[j][tid];
+        sum.x += p.x;
+        sum.y += p.y;
+        sum.z += p.z;
+        sum.w += p.w;
+      }
+      const int32_t row = tdesc[(int64_t)ld.x * kSlotsPerTile].x;
+      store_result(C + (uint64_t)(uint32_t)row * K + k0 + 4 * l, sum);
+    }
+    return;
+  }
+
+  const int32_t w = __builtin_amdgcn_readfirstlane(n_wg + (blk - n_wg) * WPB + wave);
+  int lg = 3;
+  int32_t row;
+  if (w < n_loop) {
+    const int2 ld = ldesc[w];
+    row = tdesc[(int64_t)ld.x * kSlotsPerTile].x;
+    gather_tiles<K>(acc, ld.x, ld.x + ld.y, lane, s, l, tid, base, k0, s_col, s_val, tcol, tdesc, val, B);
+  } else {
+    const int32_t tile = loop_tiles + (w - n_loop);
+    if (tile >= n_tiles) return;
+    lg = tile < end3 ? 3 : tile < end2 ? 2 : tile < end1 ? 1 : 0;
+    const int32_t c = tcol[(int64_t)tile * kRowTile + lane];
+    const int2 d = tdesc[(int64_t)tile * kSlotsPerTile + s];
+    const float v = c >= 0 ? val[d.y + l] : 0.f;
+    row = d.x;
+    gather_slot<K>(acc, c, v, tid, base, l, k0, s_col, s_val, B);
+  }
 #pragma unroll
   for (int step = 0; step < 3; ++step) {
     if (lg > step) {

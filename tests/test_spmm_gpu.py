@@ -507,7 +507,7 @@ def test_auto_strategy_leaves_short_rows_unrouted(pkg, oracle, gpu):
     import torch
     capi = pkg.capi
     rng = np.random.default_rng(77)
-    rows, cols, per_row, k = 120_000, 150_000, 40, 64
+    rows, cols, per_row, k = 450_000, 500_000, 40, 64             # 18 M nonzeros: beyond the rows strategy
     pop = rng.zipf(1.6, size=rows * per_row) % cols               # heavy-tailed column popularity
     col = np.sort(pop.reshape(rows, per_row), axis=1).astype(np.int32).ravel()
     rowptr = (np.arange(rows + 1, dtype=np.int64) * per_row).astype(np.int32)
@@ -520,6 +520,15 @@ def test_auto_strategy_leaves_short_rows_unrouted(pkg, oracle, gpu):
     C64, S64 = oracle.csr_spmm_f64_rows(g.rowptr, g.col, g.val, B, lo, hi)
     err, _ = oracle.max_norm_err(C[lo:hi], C64, S64)
     assert err <= TOL
+    # a quarter of it is within the rows strategy's range (row tiles), and without the tiles it is not
+    sub = pkg.graphs.CSR(rows // 4, cols, rowptr[:rows // 4 + 1], col[:rows // 4 * per_row],
+                         val[:rows // 4 * per_row])
+    Cs, info_s = _run(pkg, gpu, sub, B, capi.PLAN_DEFAULT)
+    assert info_s["strategy"] == capi.STRATEGY_ROWS
+    err, _ = oracle.max_norm_err(Cs[:4000], *oracle.csr_spmm_f64_rows(sub.rowptr, sub.col, sub.val, B, 0, 4000))
+    assert err <= TOL
+    _, info_s = _run(pkg, gpu, sub, B, capi.PLAN_NO_ROW_TILES)
+    assert info_s["strategy"] == capi.STRATEGY_SEGMENTS
     Cr, info_r = _run(pkg, gpu, g, B, capi.PLAN_FORCE_ROUTED)
     assert info_r["strategy"] == capi.STRATEGY_ROUTED
     err, _ = oracle.max_norm_err(Cr[lo:hi], C64, S64)
@@ -636,6 +645,23 @@ def test_row_tiles_layout_and_fallback(pkg, oracle, gpu):
         C2, info2 = _run(pkg, gpu, g, B, capi.PLAN_NO_ROW_TILES)
         assert info2["strategy"] == capi.STRATEGY_ROWS and info2["workspace_bytes"] < 4 * col.size
         _check(oracle, g, B, C2, f"all row lengths k={k} csr")
+    # rows beyond 512 nonzeros get a workgroup each (8 wavefronts; 16 when a row exceeds 8192),
+    # next to rows of 65..512 that one wavefront works through
+    for longest in (5000, 9000):
+        lens = rng.permutation(np.concatenate([np.arange(0, 520, 7), [513, 600, 1025, longest],
+                                               np.full(300, 3)])).astype(np.int64)
+        rows = lens.size
+        rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        col = rng.integers(0, cols, int(lens.sum())).astype(np.int32)
+        val = rng.uniform(-1, 1, col.size).astype(np.float32)
+        g = pkg.graphs.CSR(rows, cols, rowptr, col, val)
+        for k in (32, 128):
+            B = rng.standard_normal((cols, k)).astype(np.float32)
+            C, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+            assert info["strategy"] == capi.STRATEGY_ROWS and info["workspace_bytes"] >= 4 * col.size
+            _check(oracle, g, B, C, f"long rows up to {longest} k={k}")
+            again, _ = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+            assert np.array_equal(C, again), "workgroup-per-row reduction must be bit-reproducible"
     # 400k rows, 2k nonzeros: 50k tiles of padding for 2k entries - not built
     rows = 400_000
     lens = np.zeros(rows, np.int64)

@@ -111,7 +111,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--scale", type=float, default=1.0, help="shrink every graph (debugging only; <1 is not the benchmark)")
     ap.add_argument("--only", default="", help="comma list of config names to run (debugging only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")

@@ -308,6 +308,10 @@ int launch_rows_any(int64_t rows, int64_t cols, int64_t k, const int32_t* rp, co
   }
 }
 
+// Rows scanned by one wavefront of the fix-up kernel: 64, or one per sub-wave while that still
+// leaves the grid small.
+inline int fixup_rows_per_wave(int64_t rows, int k) { return rows <= (1 << 18) ? 64 / (k / 4) : 64; }
+
 template <int K>
 int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, const float* v,
                     const float* B, float* C, hipStream_t st) {
@@ -330,9 +334,10 @@ int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, 
                          aligned16(ci, v, p->d_nnz_row));
     }
   }
-  const int64_t fix_blocks = ceil_div(ceil_div(p->rows, 64), hpspmm::kWavesPerBlock);
+  const int rpw = fixup_rows_per_wave(p->rows, K);
+  const int64_t fix_blocks = ceil_div(ceil_div(p->rows, rpw), hpspmm::kWavesPerBlock);
   hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st, p->rows,
-                     rp, (const int32_t*)nullptr, p->d_carry, C, p->shift);
+                     rp, (const int32_t*)nullptr, p->d_carry, C, p->shift, rpw);
   return HPSPMM_OK;
 }
 
@@ -351,9 +356,10 @@ int launch_ordered(const hpspmm_plan* p, const int32_t* rp, const float* v, cons
     hipLaunchKernelGGL(hpspmm::spmm_ordered_kernel<K>, dim3((unsigned)grid), dim3(hpspmm::kBlock),
                        (size_t)p->ocap * K * sizeof(float), st, rp, p->d_ostart, p->d_ocol, p->d_osrc, p->d_orow, v,
                        p->d_wcols, p->ocap, B, C, p->d_carry, p->nnz, p->shift, nblocks, p->xcd_remap);
-  const int64_t fix_blocks = ceil_div(ceil_div(p->rows, 64), hpspmm::kWavesPerBlock);
+  const int rpw = fixup_rows_per_wave(p->rows, K);
+  const int64_t fix_blocks = ceil_div(ceil_div(p->rows, rpw), hpspmm::kWavesPerBlock);
   hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st, p->rows,
-                     rp, p->d_ostart, p->d_carry, C, p->shift);
+                     rp, p->d_ostart, p->d_carry, C, p->shift, rpw);
   return HPSPMM_OK;
 }
 

@@ -447,27 +447,31 @@ __global__ __launch_bounds__(kBlock) void spmm_segments_kernel(
   flush_to(continues);
 }
 
-// Fix-up after the segments kernel.  A wavefront scans 64 consecutive rows (one
-// rowptr pair per lane, coalesced) and classifies them by ballot; its sub-waves
-// then zero the empty rows and, for rows that cross a segment boundary, add the
-// carry slots in segment order.  All other rows were already stored.
+// Fix-up after the segments kernel.  A wavefront scans `rpw` consecutive rows
+// (one rowptr pair per lane, coalesced) and classifies them by ballot; its
+// sub-waves then zero the empty rows and, for rows that cross a segment
+// boundary, add the carry slots in segment order.  All other rows were already
+// stored.  rpw = 64 when rows are plentiful; rpw = 64 / (K/4), one row per
+// sub-wave, when they are few and long - 4,659 rows of 310 nonzeros on average
+// left 73 wavefronts adding up eight chains each, one after the other (56 us,
+// five times the segments kernel before it).
 // `start` (may be NULL): first position of every row when the nonzeros were
 // processed in an order of the plan's own; NULL = stored order (rowptr).
 template <int K>
 __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                             const int32_t* __restrict__ start,
                                                             const float* __restrict__ carry,
-                                                            float* __restrict__ C, int shift) {
+                                                            float* __restrict__ C, int shift, int rpw) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
   const int sub = lane / G;
-  const int64_t r0 = ((int64_t)blockIdx.x * kWavesPerBlock + (tid >> 6)) * 64;
+  const int64_t r0 = ((int64_t)blockIdx.x * kWavesPerBlock + (tid >> 6)) * rpw;
   if (r0 >= rows) return;
   const int64_t r = r0 + lane;
-  const bool valid = r < rows;
+  const bool valid = r < rows && lane < rpw;
   int32_t lb = valid ? rowptr[r] : 0;
   int32_t hb = valid ? rowptr[r + 1] : 0;
   if (start != nullptr && valid) {
@@ -503,7 +507,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
     for (; g <= gb; g += step) add(acc, *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * g) * K + 4 * l));
   };
 
-  for (int i = sub; i < 64; i += P) {
+  for (int i = sub; i < rpw; i += P) {
     // every lane takes part in the shuffles; only then do the sub-waves diverge
     const int32_t lb_i = __shfl(lb, i);
     const int32_t hb_i = __shfl(hb, i);

@@ -17,8 +17,9 @@
 // 8 / 16 / 32 / 64 nonzeros takes 1 / 2 / 4 / 8 adjacent slots of one tile
 // (tiles hold rows of one size class only, so the reduction over a row's slots
 // is the same wavefront shuffle for the whole tile); a longer row owns
-// consecutive tiles that one wavefront works through.  Long rows come first in
-// the grid, since their chain is the longest.
+// consecutive tiles that one wavefront works through - or, in the second
+// kernel below, a whole workgroup when the row has more than a few hundred
+// nonzeros.  Long rows come first in the grid, since their chain is the longest.
 //
 // K > 32 is served in 32-column tiles of B and C by K/32 workgroups per group
 // of row tiles (workgroup b serves column tile b % (K/32), so an XCD only ever

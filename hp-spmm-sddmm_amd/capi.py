@@ -182,7 +182,12 @@ class Plan:
             lib().hpspmm_plan_destroy(self._h)
             self._h = None
 
-    __del__ = destroy
+    def __del__(self):
+        # at interpreter exit the module's globals may already be gone; the process frees the plan
+        try:
+            self.destroy()
+        except Exception:
+            pass
 
 
 def _check_operands(rows, cols, nnz, k, rowptr, col, val, B, C):

@@ -165,16 +165,17 @@ int launch_rows(int64_t rows, int64_t cols, const int32_t* rp, const int32_t* ci
 
 // Row tiles (rows strategy): every row cut into slots of 8 nonzeros, 8 slots to a tile, a row's
 // slots adjacent in one tile (1 / 2 / 4 / 8 of them for up to 8 / 16 / 32 / 64 nonzeros, tiles
-// sorted by that class), longer rows over consecutive tiles.  Built on the host: the strategy
-// only serves matrices below 2^21 nonzeros.  Skipped (the kernel then walks the CSR arrays)
-// when padding would blow the layout up, which is what a matrix of mostly empty rows does.
+// sorted by that class), longer rows over consecutive tiles, those that get a whole workgroup
+// first.  Built on the host, about 3 ms per million nonzeros.  Skipped (the kernel then walks the
+// CSR arrays) when padding would blow the layout up, which is what a matrix of mostly empty rows
+// does, and beyond kRowTileMaxNnz (rows strategy forced on a very large matrix).
 constexpr int64_t kRowTilePadFactor = 8;
 constexpr int64_t kRowTileMaxNnz = (int64_t)1 << 28;
+constexpr int32_t kRowTileWorkgroupRows = 512;  // rows beyond this many nonzeros get a whole workgroup
 // automatic use of the rows strategy beyond tiny matrices
 constexpr int64_t kRowsAutoMaxNnz = 1 << 24;
 constexpr int64_t kRowsAutoMaxWork = (int64_t)1 << 30;  // nnz * K
 constexpr int64_t kRowsAutoMaxRow = 1 << 16;
-constexpr int32_t kRowTileWorkgroupRows = 512;  // rows beyond this many nonzeros get a whole workgroup  // beyond this (rows strategy forced on a large matrix) not built either
 
 int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st) {
   using hpspmm::kSlot;
@@ -264,6 +265,7 @@ int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, flo
                      p->d_tcol, p->d_tdesc, v, B, C);
   return HPSPMM_OK;
 }
+
 template <int K, int WPB>
 int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
   const int64_t wave_items = (p->rt_loop - p->rt_wg) + (p->rt_tiles - p->rt_loop_tiles);

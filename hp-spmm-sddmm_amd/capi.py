@@ -72,7 +72,7 @@ class PlanInfo(ctypes.Structure):
         ("strategy", ctypes.c_int32), ("segment_length", ctypes.c_int32),
         ("num_segments", _i64), ("max_row_nnz", _i64), ("empty_rows", _i64),
         ("workspace_bytes", _i64), ("launches_per_spmm", ctypes.c_int32), ("reserved", ctypes.c_int32),
-        ("hub_rows", _i64), ("lds_served_nnz", _i64),
+        ("hub_rows", _i64), ("lds_served_nnz", _i64), ("row_tiles", _i64),
     ]
 
     def as_dict(self):

@@ -1113,6 +1113,7 @@ int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
                                                                         : 1;
   out->hub_rows = plan->n_hub;
   out->lds_served_nnz = plan->oserved;
+  out->row_tiles = plan->d_tcol ? plan->rt_tiles : 0;
   return HPSPMM_OK;
 }
 

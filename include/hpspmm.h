@@ -98,6 +98,7 @@ typedef struct hpspmm_plan_info {
   int32_t reserved;
   int64_t hub_rows;        /* rows of B kept in the hub cache (0 = none) */
   int64_t lds_served_nnz;  /* ordered strategy: nonzeros whose row of B comes from a workgroup's LDS copy */
+  int64_t row_tiles;       /* rows strategy: 64-entry tiles of the plan's row-tile layout (0: the CSR arrays are walked) */
 } hpspmm_plan_info;
 
 /* Library version, major*10000 + minor*100 + patch. */

@@ -174,7 +174,9 @@ constexpr int64_t kRowTileMaxNnz = (int64_t)1 << 28;
 constexpr int32_t kRowTileWorkgroupRows = 512;  // rows beyond this many nonzeros get a whole workgroup
 // automatic use of the rows strategy beyond tiny matrices
 constexpr int64_t kRowsAutoMaxNnz = 1 << 24;
-constexpr int64_t kRowsAutoMaxWork = (int64_t)1 << 30;  // nnz * K
+constexpr int64_t kRowsAutoMaxWork = (int64_t)1 << 30;  // nnz * K, matrices of short rows
+constexpr double kRowsAutoLongMean = 128.0;             // mean nonzeros per non-empty row beyond which ...
+constexpr double kRowsAutoLongWork = 2.0e15;            // ... nnz^2 * K decides instead
 constexpr int64_t kRowsAutoMaxRow = 1 << 16;
 
 int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st) {
@@ -976,11 +978,16 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     p->strategy = HPSPMM_STRATEGY_SEGMENTS;  // the routed layout is built on top of it below
   } else {
     // Whole rows (one launch) while the matrix is small enough that the second and third launch of
-    // the other strategies are felt and L2 reuse across rows is not yet what decides: measured
-    // against segments / routed / ordered on scaled copies of the benchmark graphs, row tiles win up
-    // to about 2^23 nonzeros at K=128 and 2^25 at K=32 (R-MAT, 3.7 M nonzeros, K=32: 42 vs 198 us).
+    // the other strategies are felt and L2 reuse across rows is not yet what decides.  Measured
+    // against segments / routed / ordered on scaled copies of the benchmark graphs: with short rows
+    // (means of 30 and 50 nonzeros) row tiles win up to 12 M nonzeros at K=64 and draw at 31 M;
+    // with long rows (mean 400: every row a chain of tiles on one wavefront) they win at 4.3 M and
+    // lose at 9.6 M for every K, the crossing near nnz * sqrt(K) = 4.5e7.
     const bool tiny = nnz < (1 << 21) && p->max_row_nnz <= 4096;  // fine even over the CSR arrays
-    const bool mid = nnz < kRowsAutoMaxNnz && nnz * k < kRowsAutoMaxWork && p->max_row_nnz <= kRowsAutoMaxRow;
+    const double mean_row = (double)nnz / (double)std::max<int64_t>(1, rows - p->empty_rows);
+    const bool fits = mean_row > kRowsAutoLongMean ? (double)nnz * (double)nnz * (double)k < kRowsAutoLongWork
+                                                   : nnz * k < kRowsAutoMaxWork;
+    const bool mid = nnz < kRowsAutoMaxNnz && fits && p->max_row_nnz <= kRowsAutoMaxRow;
     p->strategy = (nnz == 0 || tiny || mid) ? HPSPMM_STRATEGY_ROWS : HPSPMM_STRATEGY_SEGMENTS;
     rows_need_tiles = !(nnz == 0 || tiny);
   }

@@ -110,14 +110,15 @@ const char *hpspmm_last_error(void);
 /*
  * Analyse the sparsity structure of A for a given k and build the device-side
  * work assignment.  The plan picks a strategy (reported by
- * hpspmm_plan_get_info): whole rows for matrices below 2^24 nonzeros with
- * nnz * k < 2^30 (the rows cut into 8-nonzero slots and packed, by length
- * class, into one 64-entry tile per wavefront, so that a microsecond-scale
- * SpMM is one launch with a two-step dependent chain); fixed-length segments
- * of nonzeros with a carry buffer; the same inside column slices pinned to
- * one XCD each when a few columns take most of the nonzeros ("routed"); or
- * segments over a clustered row order with the reused rows of B held in LDS
- * when the matrix is a graph with communities ("ordered").
+ * hpspmm_plan_get_info): whole rows for small and medium matrices (below 2^24
+ * nonzeros and nnz * k < 2^30, less when the rows are long; the rows cut into
+ * 8-nonzero slots and packed, by length class, into one 64-entry tile per
+ * wavefront, so that a microsecond-scale SpMM is one launch with a two-step
+ * dependent chain); fixed-length segments of nonzeros with a carry buffer;
+ * the same inside column slices pinned to one XCD each when a few columns
+ * take most of the nonzeros ("routed"); or segments over a clustered row
+ * order with the reused rows of B held in LDS when the matrix is a graph with
+ * communities ("ordered").
  * Replaces the host-side preprocessing the reference does before timing:
  * CSR->COO expansion (spmm/mm/spmm_common.cpp:185-235), the row re-ordering
  * (:237-296) and the choice of nnz_per_warp (spmm/mm/spmm_kernel.cu:749-751).

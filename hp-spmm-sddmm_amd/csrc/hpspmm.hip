@@ -174,7 +174,7 @@ constexpr int64_t kRowTileMaxNnz = (int64_t)1 << 28;
 constexpr int32_t kRowTileWorkgroupRows = 512;  // rows beyond this many nonzeros get a whole workgroup
 // automatic use of the rows strategy beyond tiny matrices
 constexpr int64_t kRowsAutoMaxNnz = 1 << 24;
-constexpr int64_t kRowsAutoMaxWork = (int64_t)1 << 30;  // nnz * K, matrices of short rows
+constexpr int64_t kRowsAutoMaxWork = (int64_t)3 << 28;  // nnz * K, matrices of short rows
 constexpr double kRowsAutoLongMean = 128.0;             // mean nonzeros per non-empty row beyond which ...
 constexpr double kRowsAutoLongWork = 2.0e15;            // ... nnz^2 * K decides instead
 constexpr int64_t kRowsAutoMaxRow = 1 << 16;
@@ -800,7 +800,9 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
 
 // Automatic clustering is tried for graphs of at least this size ...
 constexpr int64_t kClusterMinNnz = (int64_t)1 << 22;
-constexpr int64_t kClusterMinBBytes = (int64_t)64 << 20;
+constexpr int64_t kClusterMinBBytes = (int64_t)24 << 20;
+constexpr int32_t kClusterMaxSize = 4096;   // rows of a cluster that still counts as one a window can profit from
+constexpr double kClusterMinIntra = 0.15;   // share of the nonzeros inside such clusters for the order to be used
 constexpr int64_t kClusterMinMeanNnz = 8;
 // ... and its order is kept if this share of the nonzeros then reads B from LDS.
 constexpr double kClusterMinServed = 0.15;
@@ -811,9 +813,10 @@ constexpr double kClusterMinServed = 0.15;
 constexpr int kClusterMaxSweeps = 10;
 
 int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st,
-                 int32_t** d_order_out) {
+                 int32_t** d_order_out, double* intra_share_out) {
   const int64_t rows = p->rows;
   *d_order_out = nullptr;
+  *intra_share_out = 0.0;
   int32_t* d_label = nullptr;
   uint32_t* d_changed = nullptr;
   struct Guard {
@@ -845,6 +848,25 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
   HPSPMM_HIP(hipStreamSynchronize(st));
   std::vector<int32_t> first((size_t)rows + 1, 0);
   for (int64_t r = 0; r < rows; ++r) first[(size_t)label[(size_t)r] + 1]++;
+  {
+    // share of the nonzeros that stay inside a cluster small enough for a workgroup's window
+    int32_t* d_size = nullptr;
+    hipError_t e = hipMalloc(&d_size, (size_t)rows * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMemcpyAsync(d_size, first.data() + 1, (size_t)rows * sizeof(int32_t), hipMemcpyHostToDevice, st);
+    if (e == hipSuccess) e = hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st);
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL(hpspmm::cluster_intra_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
+                         dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_label, d_size, kClusterMaxSize,
+                         d_changed);
+      e = hipMemcpyAsync(counters.data(), d_changed, counters.size() * sizeof(uint32_t), hipMemcpyDeviceToHost, st);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (d_size) (void)hipFree(d_size);
+    if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "cluster scoring failed: %s", hipGetErrorString(e));
+    int64_t intra = 0;
+    for (uint32_t c : counters) intra += c;
+    *intra_share_out = p->nnz > 0 ? (double)intra / (double)p->nnz : 0.0;
+  }
   for (int64_t l = 0; l < rows; ++l) first[(size_t)l + 1] += first[(size_t)l];
   for (int64_t r = 0; r < rows; ++r) order[(size_t)first[(size_t)label[(size_t)r]]++] = (int32_t)r;
   int32_t* d_order = nullptr;
@@ -962,7 +984,11 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   p->empty_rows = stats[1];
   p->xcd_remap = !(flags & HPSPMM_PLAN_NO_XCD_REMAP);
 
+  // Automatic choice, in this order: tiny matrix -> rows; a matrix in the rows strategy's range
+  // (`rows_range`) -> ordered if it has communities, else rows; beyond that range -> routed if a
+  // few columns take most of the nonzeros, else ordered if it has communities, else segments.
   bool rows_need_tiles = false;  // rows strategy chosen on the strength of the row tiles
+  bool rows_range = false;       // provisional segments; rows unless the ordered strategy qualifies
   if (!fast_k(k)) {
     p->strategy = HPSPMM_STRATEGY_GENERIC_K;
   } else if (d_order && nnz > 0) {
@@ -979,17 +1005,24 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   } else {
     // Whole rows (one launch) while the matrix is small enough that the second and third launch of
     // the other strategies are felt and L2 reuse across rows is not yet what decides.  Measured
-    // against segments / routed / ordered on scaled copies of the benchmark graphs: with short rows
-    // (means of 30 and 50 nonzeros) row tiles win up to 12 M nonzeros at K=64 and draw at 31 M;
-    // with long rows (mean 400: every row a chain of tiles on one wavefront) they win at 4.3 M and
-    // lose at 9.6 M for every K, the crossing near nnz * sqrt(K) = 4.5e7.
+    // against segments and routed on scaled copies of the benchmark graphs: with short rows (means
+    // of 30 and 50 nonzeros) row tiles win up to nnz * K = 2^29.5 (R-MAT, 15 M nonzeros, K=32:
+    // 188 us against 258 us routed; 7.6 M nonzeros, K=128: 403 against 346 us); with long rows
+    // (mean 400: every row a chain of tiles on one wavefront) they win at 4.3 M nonzeros and lose
+    // at 9.6 M for every K, the crossing near nnz * sqrt(K) = 4.5e7.
     const bool tiny = nnz < (1 << 21) && p->max_row_nnz <= 4096;  // fine even over the CSR arrays
     const double mean_row = (double)nnz / (double)std::max<int64_t>(1, rows - p->empty_rows);
     const bool fits = mean_row > kRowsAutoLongMean ? (double)nnz * (double)nnz * (double)k < kRowsAutoLongWork
                                                    : nnz * k < kRowsAutoMaxWork;
-    const bool mid = nnz < kRowsAutoMaxNnz && fits && p->max_row_nnz <= kRowsAutoMaxRow;
-    p->strategy = (nnz == 0 || tiny || mid) ? HPSPMM_STRATEGY_ROWS : HPSPMM_STRATEGY_SEGMENTS;
-    rows_need_tiles = !(nnz == 0 || tiny);
+    const bool mid = nnz < kRowsAutoMaxNnz && fits && p->max_row_nnz <= kRowsAutoMaxRow &&
+                     !(flags & HPSPMM_PLAN_NO_ROW_TILES);
+    if (nnz == 0 || tiny || (mid && nnz < kClusterMinNnz)) {
+      p->strategy = HPSPMM_STRATEGY_ROWS;
+      rows_need_tiles = !(nnz == 0 || tiny);
+    } else {
+      p->strategy = HPSPMM_STRATEGY_SEGMENTS;
+      rows_range = mid;
+    }
   }
 
   if (p->strategy == HPSPMM_STRATEGY_ROWS && rows > 0 && nnz < kRowTileMaxNnz && !(flags & HPSPMM_PLAN_NO_ROW_TILES)) {
@@ -1026,7 +1059,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       }
     }
   }
-  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && !(flags & HPSPMM_PLAN_NO_ROUTED) && nnz > 0 &&
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && !(flags & HPSPMM_PLAN_NO_ROUTED) && nnz > 0 && !rows_range &&
       !(flags & HPSPMM_PLAN_FORCE_SEGMENTS && !(flags & HPSPMM_PLAN_FORCE_ROUTED))) {
     if (int rc = build_routed(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_ROUTED) != 0,
                               (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 16) & 0xFFu) : 0,
@@ -1036,24 +1069,45 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       return rc;
     }
   }
-  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && !(flags & HPSPMM_PLAN_NO_HUB_CACHE) && nnz > 0) {
-    if (int rc = build_hub_cache(p, d_col, (int)((flags >> 16) & 0xFFu), (flags & HPSPMM_PLAN_HUB_CACHE) != 0, st)) {
+  // Community structure: not routed, the matrix is a graph (square) and B does not fit the L2s -
+  // look for clusters of rows that share columns.  Tried before the hub cache: a graph can have
+  // both popular columns and communities (the co-purchase graph at a quarter of its size: the 64k
+  // most referenced columns take a quarter of the nonzeros there), and the ordered strategy is then
+  // the faster of the two (0.73 ms against 1.15 ms for segments with the hub cache).
+  const bool want_cluster = (flags & HPSPMM_PLAN_CLUSTER) != 0;
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && rows == cols && nnz > 0 && !(flags & HPSPMM_PLAN_NO_CLUSTER) &&
+      (want_cluster || (!(flags & HPSPMM_PLAN_FORCE_SEGMENTS) && nnz >= kClusterMinNnz &&
+                        cols * k * 4 >= kClusterMinBBytes && nnz >= rows * kClusterMinMeanNnz))) {
+    int32_t* d_order = nullptr;
+    double intra_share = 0.0;
+    int rc = cluster_rows(p, d_rowptr, d_col, st, &d_order, &intra_share);
+    if (rc == HPSPMM_OK && (want_cluster || intra_share >= kClusterMinIntra))
+      rc = build_ordered(p, d_rowptr, d_col, d_order, want_cluster ? 0.0 : kClusterMinServed, st);
+    if (d_order) (void)hipFree(d_order);
+    if (rc) {
       hpspmm_plan_destroy(p);
       return rc;
     }
   }
-  // Community structure: neither hot columns nor anything else to exploit so far, the matrix is a
-  // graph (square) and B does not fit the L2s - look for clusters of rows that share columns.
-  const bool want_cluster = (flags & HPSPMM_PLAN_CLUSTER) != 0;
-  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && p->n_hub == 0 && rows == cols && nnz > 0 &&
-      !(flags & HPSPMM_PLAN_NO_CLUSTER) &&
-      (want_cluster || (!(flags & HPSPMM_PLAN_FORCE_SEGMENTS) && nnz >= kClusterMinNnz &&
-                        cols * k * 4 >= kClusterMinBBytes && nnz >= rows * kClusterMinMeanNnz))) {
-    int32_t* d_order = nullptr;
-    int rc = cluster_rows(p, d_rowptr, d_col, st, &d_order);
-    if (rc == HPSPMM_OK) rc = build_ordered(p, d_rowptr, d_col, d_order, want_cluster ? 0.0 : kClusterMinServed, st);
-    if (d_order) (void)hipFree(d_order);
-    if (rc) {
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && rows_range) {
+    // no communities: whole rows after all, if the row tiles get built
+    if (int rc = build_row_tiles(p, d_rowptr, d_col, st)) {
+      hpspmm_plan_destroy(p);
+      return rc;
+    }
+    if (p->d_tcol) {
+      (void)hipFree(p->d_nnz_row);
+      (void)hipFree(p->d_carry);
+      p->d_nnz_row = nullptr;
+      p->d_carry = nullptr;
+      p->workspace_bytes -= (int64_t)((size_t)nnz * sizeof(int32_t) + (size_t)p->nseg * 2 * (size_t)k * sizeof(float));
+      p->nseg = 0;
+      p->shift = 0;
+      p->strategy = HPSPMM_STRATEGY_ROWS;
+    }
+  }
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && !(flags & HPSPMM_PLAN_NO_HUB_CACHE) && nnz > 0) {
+    if (int rc = build_hub_cache(p, d_col, (int)((flags >> 16) & 0xFFu), (flags & HPSPMM_PLAN_HUB_CACHE) != 0, st)) {
       hpspmm_plan_destroy(p);
       return rc;
     }

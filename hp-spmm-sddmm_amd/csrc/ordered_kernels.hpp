@@ -109,6 +109,33 @@ __global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, con
   }
 }
 
+// What the labels are worth: counts the nonzeros (r, c) with label[c] == label[r] in clusters of
+// at most max_size rows (size[l] = rows carrying label l) - the nonzeros whose row of B a
+// workgroup can expect to meet again within its window once the rows are ordered by label.  Hot
+// columns also produce reuse inside a window, but that is the routed strategy's and the hub
+// cache's business; a graph without communities ends up in one giant cluster or in singletons and
+// scores nothing here.  One wavefront per row; intra[] has kClusterCounters entries.
+__global__ __launch_bounds__(kBlock) void cluster_intra_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                               const int32_t* __restrict__ col,
+                                                               const int32_t* __restrict__ label,
+                                                               const int32_t* __restrict__ size, int32_t max_size,
+                                                               uint32_t* __restrict__ intra) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const int32_t mine = label[r];
+  if (size[mine] > max_size) return;
+  const int32_t lb = rowptr[r], hb = rowptr[r + 1];
+  uint32_t cnt = 0;
+  for (int32_t j = lb + lane; j < hb; j += 64) {
+    const int32_t c = col[j];
+    cnt += ((int64_t)c < rows && label[c] == mine) ? 1u : 0u;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off);
+  if (lane == 0 && cnt) atomicAdd(&intra[r & (kClusterCounters - 1)], cnt);
+}
+
 // label[r] = r.
 __global__ __launch_bounds__(kBlock) void cluster_init_kernel(int64_t rows, int32_t* __restrict__ label) {
   const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;

@@ -69,8 +69,9 @@ typedef enum hpspmm_status {
 /* bits 8..11: log2 of the segment length to force (0 = choose automatically) */
 #define HPSPMM_PLAN_SEGMENT_SHIFT(log2_len) (((uint32_t)(log2_len) & 0xFu) << 8)
 #define HPSPMM_PLAN_CLUSTER 4096u     /* square A: always look for clusters of rows that share columns and use the
-                                         ordered strategy on the order found (default: only for large graphs
-                                         without hot columns, and only if >= 15 % of the nonzeros then read B
+                                         ordered strategy on the order found (default: from 2^22 nonzeros and
+                                         24 MB of B up, when the graph is not routed, and only if >= 15 % of the
+                                         nonzeros stay inside clusters of <= 4096 rows and >= 15 % then read B
                                          from LDS).  The clustering updates its labels asynchronously: two
                                          plans of one matrix may order the rows differently and then differ
                                          in the last bits of C; one plan always gives the same bits */

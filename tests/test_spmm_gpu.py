@@ -674,3 +674,29 @@ def test_row_tiles_layout_and_fallback(pkg, oracle, gpu):
     C, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
     assert info["strategy"] == capi.STRATEGY_ROWS and info["row_tiles"] == 0
     _check(oracle, g, B, C, "mostly empty rows")
+
+
+def test_auto_choice_at_mid_size(pkg, oracle, gpu):
+    """Between the small and the large graphs: a community graph of 6 M nonzeros gets the ordered
+    strategy by itself (label propagation finds its clusters), an R-MAT of the same size - hot columns,
+    no communities - does not and stays with whole rows; both agree with the oracle."""
+    capi = pkg.capi
+    for name, scale, k, want in (("c3_copurchase", 0.05, 64, capi.STRATEGY_ORDERED),
+                                 ("c4_rmat", 0.0625, 32, capi.STRATEGY_ROWS)):
+        g = pkg.graphs.make_graph(name, scale)
+        B = pkg.graphs.make_dense(name, g.cols, k)
+        C, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+        assert info["strategy"] == want, (name, info)
+        if want == capi.STRATEGY_ROWS:
+            assert info["row_tiles"] > 0
+        else:
+            assert info["lds_served_nnz"] >= 0.15 * g.nnz
+        lo, hi = g.rows // 3, g.rows // 3 + 3000
+        C64, S64 = oracle.csr_spmm_f64_rows(g.rowptr, g.col, g.val, B, lo, hi)
+        err, _ = oracle.max_norm_err(C[lo:hi], C64, S64)
+        assert err <= TOL, f"{name}: normalised error {err:.3e}"
+        heavy = np.argsort(-np.diff(g.rowptr))[:4]
+        for r in heavy:
+            C64, S64 = oracle.csr_spmm_f64_rows(g.rowptr, g.col, g.val, B, int(r), int(r) + 1)
+            err, _ = oracle.max_norm_err(C[r:r + 1], C64, S64)
+            assert err <= TOL, f"{name}: heaviest rows: normalised error {err:.3e}"

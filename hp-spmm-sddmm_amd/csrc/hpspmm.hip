@@ -117,6 +117,8 @@ struct hpspmm_plan {
   int32_t* d_tcol = nullptr;  // [rt_tiles * 64] column of every tile entry, -1 = padding
   int2* d_tdesc = nullptr;    // [rt_tiles * 8] per slot: row (-1 = padding), index of its first value
   int2* d_ldesc = nullptr;    // [rt_loop] per long row: first tile, tile count
+  float* d_zrow = nullptr;    // 32 zeros: what a padding entry gathers instead of a row of B
+  int32_t* d_tdepth = nullptr;  // [rt_tiles] entries per slot that any slot of the tile uses (0..8)
   int32_t rt_tiles = 0, rt_waves = 0, rt_loop = 0, rt_wg = 0, rt_loop_tiles = 0, rt_end3 = 0, rt_end2 = 0, rt_end1 = 0;
   int64_t workspace_bytes = 0;
 };
@@ -191,11 +193,18 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
 
   auto class_of = [](int32_t n) { return n <= 8 ? 0 : n <= 16 ? 1 : n <= 32 ? 2 : n <= 64 ? 3 : 4; };
   int64_t count[5] = {0, 0, 0, 0, 0}, loop_tiles = 0;
+  int64_t by_len[kSlot + 1] = {0};  // one-slot rows by length, longest first: tiles of equal depth
   for (int64_t r = 0; r < rows; ++r) {
     const int32_t n = rp[r + 1] - rp[r];
     const int c = class_of(n);
     ++count[c];
+    if (c == 0) ++by_len[n];
     if (c == 4) loop_tiles += ceil_div(n, kTile);
+  }
+  int64_t next_of_len[kSlot + 1];
+  for (int64_t n = kSlot, at = 0; n >= 0; --n) {
+    next_of_len[n] = at;
+    at += by_len[n];
   }
   // tile ranges: long rows, then the classes from 8 slots a row down to 1
   const int64_t t3 = count[3], t2 = ceil_div(count[2], 2), t1 = ceil_div(count[1], 4), t0 = ceil_div(count[0], 8);
@@ -206,6 +215,8 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
   std::vector<int32_t> tcol((size_t)tiles * kTile, -1);
   std::vector<int2> tdesc((size_t)tiles * kSlotsPerTile, make_int2(-1, 0));
   std::vector<int2> ldesc((size_t)(count[4] > 0 ? count[4] : 1));
+  std::vector<int32_t> tdepth((size_t)tiles, kSlot);
+  for (int64_t t = first[0]; t < tiles; ++t) tdepth[(size_t)t] = 0;  // one-slot tiles: set by their rows below
   int64_t group[4] = {0, 0, 0, 0}, next_loop_tile = 0, n_loop = 0, n_wg = 0;
   // two passes: the rows that get a whole workgroup first in ldesc (and in the tile order), then the rest
   for (int pass = 0; pass < 2; ++pass)
@@ -224,7 +235,9 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
       next_loop_tile += nt;
     } else {
       slots = (int64_t)1 << c;
-      slot = first[c] * kSlotsPerTile + group[c]++ * slots;
+      const int64_t g = c == 0 ? next_of_len[n]++ : group[c]++;
+      slot = first[c] * kSlotsPerTile + g * slots;
+      if (c == 0) tdepth[(size_t)(slot / kSlotsPerTile)] = std::max(tdepth[(size_t)(slot / kSlotsPerTile)], n);
     }
     for (int64_t j = 0; j < slots; ++j) {
       tdesc[(size_t)(slot + j)] = make_int2((int)r, (int)(lb + j * kSlot));
@@ -236,17 +249,20 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
   }
 
   const size_t bytes_col = tcol.size() * sizeof(int32_t), bytes_desc = tdesc.size() * sizeof(int2),
-               bytes_loop = ldesc.size() * sizeof(int2);
+               bytes_loop = ldesc.size() * sizeof(int2), bytes_depth = tdepth.size() * sizeof(int32_t);
   if (hipMalloc(&p->d_tcol, bytes_col) != hipSuccess || hipMalloc(&p->d_tdesc, bytes_desc) != hipSuccess ||
-      hipMalloc(&p->d_ldesc, bytes_loop) != hipSuccess) {
+      hipMalloc(&p->d_ldesc, bytes_loop) != hipSuccess || hipMalloc(&p->d_zrow, 32 * sizeof(float)) != hipSuccess ||
+      hipMalloc(&p->d_tdepth, bytes_depth) != hipSuccess) {
     (void)hipGetLastError();
     return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the row tiles failed",
                 bytes_col + bytes_desc + bytes_loop);
   }
-  p->workspace_bytes += (int64_t)(bytes_col + bytes_desc + bytes_loop);
+  p->workspace_bytes += (int64_t)(bytes_col + bytes_desc + bytes_loop + bytes_depth + 32 * sizeof(float));
   HPSPMM_HIP(hipMemcpyAsync(p->d_tcol, tcol.data(), bytes_col, hipMemcpyHostToDevice, st));
   HPSPMM_HIP(hipMemcpyAsync(p->d_tdesc, tdesc.data(), bytes_desc, hipMemcpyHostToDevice, st));
   HPSPMM_HIP(hipMemcpyAsync(p->d_ldesc, ldesc.data(), bytes_loop, hipMemcpyHostToDevice, st));
+  HPSPMM_HIP(hipMemsetAsync(p->d_zrow, 0, 32 * sizeof(float), st));
+  HPSPMM_HIP(hipMemcpyAsync(p->d_tdepth, tdepth.data(), bytes_depth, hipMemcpyHostToDevice, st));
   HPSPMM_HIP(hipStreamSynchronize(st));  // the host vectors go out of scope
   p->rt_tiles = (int32_t)tiles;
   p->rt_loop = (int32_t)n_loop;
@@ -259,12 +275,18 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
   return HPSPMM_OK;
 }
 
+// The row-tile kernels read val[0] for padding entries (and discard it): a matrix without
+// nonzeros may come with val == NULL, so give them some readable address then.
+inline const float* readable_values(const hpspmm_plan* p, const float* v) {
+  return p->nnz > 0 ? v : reinterpret_cast<const float*>(p->d_tcol);
+}
+
 template <int K, int WPB>
 int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
   const int64_t blocks = ceil_div(p->rt_waves, WPB) * (K / 32);
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->rt_end3, p->rt_end2, p->rt_end1, p->d_ldesc,
-                     p->d_tcol, p->d_tdesc, v, B, C);
+                     p->d_tcol, p->d_tdesc, readable_values(p, v), B, C, p->d_zrow, p->d_tdepth);
   return HPSPMM_OK;
 }
 
@@ -275,7 +297,7 @@ int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, fl
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->rt_end3, p->rt_end2, p->rt_end1, p->d_ldesc,
-                     p->d_tcol, p->d_tdesc, v, B, C);
+                     p->d_tcol, p->d_tdesc, readable_values(p, v), B, C, p->d_zrow, p->d_tdepth);
   return HPSPMM_OK;
 }
 
@@ -1191,7 +1213,8 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
                   (void*)plan->d_vval, (void*)plan->d_vrow, (void*)plan->d_bhot_src, (void*)plan->d_partial,
                   (void*)plan->d_routed_rows, (void*)plan->d_cross_rows, (void*)plan->d_zero_rows,
                   (void*)plan->d_ostart, (void*)plan->d_ocol, (void*)plan->d_osrc, (void*)plan->d_orow,
-                  (void*)plan->d_wcols, (void*)plan->d_tcol, (void*)plan->d_tdesc, (void*)plan->d_ldesc})
+                  (void*)plan->d_wcols, (void*)plan->d_tcol, (void*)plan->d_tdesc, (void*)plan->d_ldesc,
+                  (void*)plan->d_zrow, (void*)plan->d_tdepth})
     if (q) (void)hipFree(q);
   delete plan;
   return HPSPMM_OK;

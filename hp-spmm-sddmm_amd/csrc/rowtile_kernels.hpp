@@ -39,28 +39,57 @@ constexpr int kSlot = 8;          // nonzeros per slot = lanes per sub-wave at a
 constexpr int kSlotsPerTile = 8;  // slots per tile = sub-waves per wavefront
 constexpr int kRowTile = kSlot * kSlotsPerTile;
 
-// acc += the slot's (up to 8) products.  `c` is this lane's entry of the tile, `v` its value.
+// acc += the first N products of the slot, after `c` (this lane's entry of the tile) has been
+// staged in s_col and the load of `v` (its value) issued.  `zrow` = 32 zeros in device memory.
+// Nothing in here is conditional: a padding entry among the first N gathers the zero row instead
+// of a row of B (so that a non-finite value in an unreferenced row of B cannot leak in).
+template <int K, int N>
+__device__ __forceinline__ void gather_n(float4& acc, int32_t c, float v, int tid, int base, int l, int k0,
+                                         const int32_t* s_col, float* s_val, const float* __restrict__ B,
+                                         const float* __restrict__ zrow) {
+  int32_t cc[N];
+  float4 b[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) cc[i] = s_col[base + i];
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const float* src = cc[i] >= 0 ? B + (uint64_t)(uint32_t)cc[i] * (uint64_t)K + (uint32_t)k0 : zrow;
+    b[i] = *reinterpret_cast<const float4*>(src + 4 * l);
+  }
+  s_val[tid] = c >= 0 ? v : 0.f;
+  wave_lds_fence();
+#pragma unroll
+  for (int i = 0; i < N; ++i) fma4(acc, s_val[base + i], b[i]);
+  wave_lds_fence();
+}
+
+// acc += the slot's products.  `vi` = index of this lane's value; `depth` (0..8, the same for the
+// whole wavefront) = entries per slot that any slot of the tile uses: the plan sorts the short rows
+// by length before it packs them, so a tile of 3-nonzero rows issues 3 gathers per lane, not 8.
+// The order matters in a kernel that is nothing but dependent round trips: the value is loaded
+// unconditionally (a padding entry reads val[0] and discards it) and the columns are staged before
+// anything branches on `depth`, so that columns, slot descriptors and depth arrive together (first
+// round trip) and values and rows of B together (second).  With `c >= 0 ? val[vi] : 0`, with
+// `if (c >= 0)` around the gathers, or with the branch on `depth` ahead of the staging, the
+// compiler moved one of the first loads behind a condition that waits for another - a third trip.
 template <int K>
-__device__ __forceinline__ void gather_slot(float4& acc, int32_t c, float v, int tid, int base, int l, int k0,
-                                            int32_t* s_col, float* s_val, const float* __restrict__ B) {
+__device__ __forceinline__ void gather_slot(float4& acc, int depth, int32_t c, int32_t vi, int tid, int base, int l,
+                                            int k0, int32_t* s_col, float* s_val, const float* __restrict__ val,
+                                            const float* __restrict__ B, const float* __restrict__ zrow) {
+  const float v = val[c >= 0 ? vi : 0];
   s_col[tid] = c;
   wave_lds_fence();
-  int32_t cc[kSlot];
-  float4 b[kSlot];
-#pragma unroll
-  for (int i = 0; i < kSlot; ++i) cc[i] = s_col[base + i];
-  // predicated loads, all in flight together; padding reads nothing, so a
-  // non-finite value in an unreferenced row of B cannot leak in
-#pragma unroll
-  for (int i = 0; i < kSlot; ++i) {
-    b[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (cc[i] >= 0) b[i] = load_b_tile<K>(B, cc[i], k0, l);
+  switch (depth) {
+    case 0: break;
+    case 1: gather_n<K, 1>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 2: gather_n<K, 2>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 3: gather_n<K, 3>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 4: gather_n<K, 4>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 5: gather_n<K, 5>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 6: gather_n<K, 6>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 7: gather_n<K, 7>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    default: gather_n<K, 8>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
   }
-  s_val[tid] = v;
-  wave_lds_fence();
-#pragma unroll
-  for (int i = 0; i < kSlot; ++i) fma4(acc, s_val[base + i], b[i]);
-  wave_lds_fence();
 }
 
 // acc += the products of tiles [t0, t1) of one long row, worked through by one wavefront.
@@ -68,18 +97,18 @@ template <int K>
 __device__ __forceinline__ void gather_tiles(float4& acc, int32_t t0, int32_t t1, int lane, int s, int l, int tid,
                                              int base, int k0, int32_t* s_col, float* s_val,
                                              const int32_t* __restrict__ tcol, const int2* __restrict__ tdesc,
-                                             const float* __restrict__ val, const float* __restrict__ B) {
+                                             const float* __restrict__ val, const float* __restrict__ B,
+                                             const float* __restrict__ zrow) {
   if (t0 >= t1) return;
   int32_t c = tcol[(int64_t)t0 * kRowTile + lane];
   int2 d = tdesc[(int64_t)t0 * kSlotsPerTile + s];
   for (int32_t t = t0; t < t1; ++t) {
-    const float v = c >= 0 ? val[d.y + l] : 0.f;
-    const int32_t c_now = c;
+    const int32_t c_now = c, vi_now = d.y + l;
     if (t + 1 < t1) {  // next tile's entries on their way while this one is gathered
       c = tcol[(int64_t)(t + 1) * kRowTile + lane];
       d = tdesc[(int64_t)(t + 1) * kSlotsPerTile + s];
     }
-    gather_slot<K>(acc, c_now, v, tid, base, l, k0, s_col, s_val, B);
+    gather_slot<K>(acc, kSlot, c_now, vi_now, tid, base, l, k0, s_col, s_val, val, B, zrow);
   }
 }
 
@@ -94,7 +123,8 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
                                                                const int32_t* __restrict__ tcol,
                                                                const int2* __restrict__ tdesc,
                                                                const float* __restrict__ val,
-                                                               const float* __restrict__ B, float* __restrict__ C) {
+                                                               const float* __restrict__ B, float* __restrict__ C,
+                                                               const float* __restrict__ zrow, const int32_t* __restrict__ tdepth) {
   constexpr int T = K / 32;
   __shared__ int32_t s_col[WPB * 64];
   __shared__ float s_val[WPB * 64];
@@ -116,13 +146,14 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
     lg = tile < end3 ? 3 : tile < end2 ? 2 : tile < end1 ? 1 : 0;
     const int32_t c = tcol[(int64_t)tile * kRowTile + lane];
     const int2 d = tdesc[(int64_t)tile * kSlotsPerTile + s];
-    const float v = c >= 0 ? val[d.y + l] : 0.f;
+    const int depth = __builtin_amdgcn_readfirstlane(tdepth[tile]);
+    __builtin_amdgcn_sched_barrier(0);  // the three loads above are issued before anything waits for one of them
     row = d.x;
-    gather_slot<K>(acc, c, v, tid, base, l, k0, s_col, s_val, B);
+    gather_slot<K>(acc, depth, c, d.y + l, tid, base, l, k0, s_col, s_val, val, B, zrow);
   } else {
     const int2 ld = ldesc[w];
     row = tdesc[(int64_t)ld.x * kSlotsPerTile].x;
-    gather_tiles<K>(acc, ld.x, ld.x + ld.y, lane, s, l, tid, base, k0, s_col, s_val, tcol, tdesc, val, B);
+    gather_tiles<K>(acc, ld.x, ld.x + ld.y, lane, s, l, tid, base, k0, s_col, s_val, tcol, tdesc, val, B, zrow);
   }
   // the slots of a row are adjacent and aligned to their count: xor shuffles, in a fixed order
 #pragma unroll
@@ -150,7 +181,8 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
                                                                     const int2* __restrict__ tdesc,
                                                                     const float* __restrict__ val,
                                                                     const float* __restrict__ B,
-                                                                    float* __restrict__ C) {
+                                                                    float* __restrict__ C,
+                                                                    const float* __restrict__ zrow, const int32_t* __restrict__ tdepth) {
   constexpr int T = K / 32;
   __shared__ int32_t s_col[WPB * 64];
   __shared__ float s_val[WPB * 64];
@@ -171,7 +203,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
     const int32_t per = (ld.y + WPB - 1) / WPB;
     const int32_t t0 = ld.x + wave * per;
     const int32_t t1 = t0 + per < ld.x + ld.y ? t0 + per : ld.x + ld.y;
-    gather_tiles<K>(acc, t0, t1, lane, s, l, tid, base, k0, s_col, s_val, tcol, tdesc, val, B);
+    gather_tiles<K>(acc, t0, t1, lane, s, l, tid, base, k0, s_col, s_val, tcol, tdesc, val, B, zrow);
 #pragma unroll
     for (int off = kSlot; off < 64; off <<= 1) {
       acc.x += __shfl_xor(acc.x, off);
@@ -202,16 +234,17 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
   if (w < n_loop) {
     const int2 ld = ldesc[w];
     row = tdesc[(int64_t)ld.x * kSlotsPerTile].x;
-    gather_tiles<K>(acc, ld.x, ld.x + ld.y, lane, s, l, tid, base, k0, s_col, s_val, tcol, tdesc, val, B);
+    gather_tiles<K>(acc, ld.x, ld.x + ld.y, lane, s, l, tid, base, k0, s_col, s_val, tcol, tdesc, val, B, zrow);
   } else {
     const int32_t tile = loop_tiles + (w - n_loop);
     if (tile >= n_tiles) return;
     lg = tile < end3 ? 3 : tile < end2 ? 2 : tile < end1 ? 1 : 0;
     const int32_t c = tcol[(int64_t)tile * kRowTile + lane];
     const int2 d = tdesc[(int64_t)tile * kSlotsPerTile + s];
-    const float v = c >= 0 ? val[d.y + l] : 0.f;
+    const int depth = __builtin_amdgcn_readfirstlane(tdepth[tile]);
+    __builtin_amdgcn_sched_barrier(0);  // the three loads above are issued before anything waits for one of them
     row = d.x;
-    gather_slot<K>(acc, c, v, tid, base, l, k0, s_col, s_val, B);
+    gather_slot<K>(acc, depth, c, d.y + l, tid, base, l, k0, s_col, s_val, val, B, zrow);
   }
 #pragma unroll
   for (int step = 0; step < 3; ++step) {

@@ -114,12 +114,10 @@ struct hpspmm_plan {
   int64_t n_long = 0;
   int32_t long_threshold = INT32_MAX;
   // rows strategy over row tiles
-  int32_t* d_tcol = nullptr;  // [rt_tiles * 64] column of every tile entry, -1 = padding
-  int2* d_tdesc = nullptr;    // [rt_tiles * 8] per slot: row (-1 = padding), index of its first value
+  int2* d_tent = nullptr;     // [rt_tiles * 64] per tile entry: column (-1 = padding), slot / tile data by lane
   int2* d_ldesc = nullptr;    // [rt_loop] per long row: first tile, tile count
   float* d_zrow = nullptr;    // 32 zeros: what a padding entry gathers instead of a row of B
-  int32_t* d_tdepth = nullptr;  // [rt_tiles] entries per slot that any slot of the tile uses (0..8)
-  int32_t rt_tiles = 0, rt_waves = 0, rt_loop = 0, rt_wg = 0, rt_loop_tiles = 0, rt_end3 = 0, rt_end2 = 0, rt_end1 = 0;
+  int32_t rt_tiles = 0, rt_waves = 0, rt_loop = 0, rt_wg = 0, rt_loop_tiles = 0;
   int64_t workspace_bytes = 0;
 };
 
@@ -212,8 +210,10 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
   const int64_t tiles = loop_tiles + t3 + t2 + t1 + t0;
   if (tiles * kTile > kRowTilePadFactor * nnz + (1 << 20) || tiles >= (1 << 24)) return HPSPMM_OK;  // not worth it
 
-  std::vector<int32_t> tcol((size_t)tiles * kTile, -1);
-  std::vector<int2> tdesc((size_t)tiles * kSlotsPerTile, make_int2(-1, 0));
+  // per entry {column, x}; x: lane 0 of a slot = row, lane 1 = index of the slot's first value,
+  // slot 0 lane 2 = depth of the tile, slot 0 lane 3 = log2(slots per row)
+  std::vector<int2> tent((size_t)tiles * kTile, make_int2(-1, 0));
+  for (int64_t q = 0; q < tiles * kSlotsPerTile; ++q) tent[(size_t)(q * kSlot)].y = -1;  // padding slot until a row takes it
   std::vector<int2> ldesc((size_t)(count[4] > 0 ? count[4] : 1));
   std::vector<int32_t> tdepth((size_t)tiles, kSlot);
   for (int64_t t = first[0]; t < tiles; ++t) tdepth[(size_t)t] = 0;  // one-slot tiles: set by their rows below
@@ -240,37 +240,35 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
       if (c == 0) tdepth[(size_t)(slot / kSlotsPerTile)] = std::max(tdepth[(size_t)(slot / kSlotsPerTile)], n);
     }
     for (int64_t j = 0; j < slots; ++j) {
-      tdesc[(size_t)(slot + j)] = make_int2((int)r, (int)(lb + j * kSlot));
+      int2* ent = &tent[(size_t)((slot + j) * kSlot)];
+      ent[0].y = (int)r;
+      ent[1].y = (int)(lb + j * kSlot);
       for (int e = 0; e < kSlot; ++e) {
         const int64_t at = j * kSlot + e;
-        if (at < n) tcol[(size_t)((slot + j) * kSlot + e)] = ci[(size_t)(lb + at)];
+        if (at < n) ent[e].x = ci[(size_t)(lb + at)];
       }
     }
   }
 
-  const size_t bytes_col = tcol.size() * sizeof(int32_t), bytes_desc = tdesc.size() * sizeof(int2),
-               bytes_loop = ldesc.size() * sizeof(int2), bytes_depth = tdepth.size() * sizeof(int32_t);
-  if (hipMalloc(&p->d_tcol, bytes_col) != hipSuccess || hipMalloc(&p->d_tdesc, bytes_desc) != hipSuccess ||
-      hipMalloc(&p->d_ldesc, bytes_loop) != hipSuccess || hipMalloc(&p->d_zrow, 32 * sizeof(float)) != hipSuccess ||
-      hipMalloc(&p->d_tdepth, bytes_depth) != hipSuccess) {
+  for (int64_t t = 0; t < tiles; ++t) {
+    tent[(size_t)(t * kTile + 2)].y = tdepth[(size_t)t];
+    tent[(size_t)(t * kTile + 3)].y = t < loop_tiles || t < first[2] ? 3 : t < first[1] ? 2 : t < first[0] ? 1 : 0;
+  }
+  const size_t bytes_ent = tent.size() * sizeof(int2), bytes_loop = ldesc.size() * sizeof(int2);
+  if (hipMalloc(&p->d_tent, bytes_ent) != hipSuccess || hipMalloc(&p->d_ldesc, bytes_loop) != hipSuccess || hipMalloc(&p->d_zrow, 32 * sizeof(float)) != hipSuccess) {
     (void)hipGetLastError();
     return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the row tiles failed",
-                bytes_col + bytes_desc + bytes_loop);
+                bytes_ent + bytes_loop);
   }
-  p->workspace_bytes += (int64_t)(bytes_col + bytes_desc + bytes_loop + bytes_depth + 32 * sizeof(float));
-  HPSPMM_HIP(hipMemcpyAsync(p->d_tcol, tcol.data(), bytes_col, hipMemcpyHostToDevice, st));
-  HPSPMM_HIP(hipMemcpyAsync(p->d_tdesc, tdesc.data(), bytes_desc, hipMemcpyHostToDevice, st));
+  p->workspace_bytes += (int64_t)(bytes_ent + bytes_loop + 32 * sizeof(float));
+  HPSPMM_HIP(hipMemcpyAsync(p->d_tent, tent.data(), bytes_ent, hipMemcpyHostToDevice, st));
   HPSPMM_HIP(hipMemcpyAsync(p->d_ldesc, ldesc.data(), bytes_loop, hipMemcpyHostToDevice, st));
   HPSPMM_HIP(hipMemsetAsync(p->d_zrow, 0, 32 * sizeof(float), st));
-  HPSPMM_HIP(hipMemcpyAsync(p->d_tdepth, tdepth.data(), bytes_depth, hipMemcpyHostToDevice, st));
   HPSPMM_HIP(hipStreamSynchronize(st));  // the host vectors go out of scope
   p->rt_tiles = (int32_t)tiles;
   p->rt_loop = (int32_t)n_loop;
   p->rt_wg = (int32_t)n_wg;
   p->rt_loop_tiles = (int32_t)loop_tiles;
-  p->rt_end3 = (int32_t)first[2];
-  p->rt_end2 = (int32_t)first[1];
-  p->rt_end1 = (int32_t)first[0];
   p->rt_waves = (int32_t)(n_loop + (tiles - loop_tiles));
   return HPSPMM_OK;
 }
@@ -278,15 +276,15 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
 // The row-tile kernels read val[0] for padding entries (and discard it): a matrix without
 // nonzeros may come with val == NULL, so give them some readable address then.
 inline const float* readable_values(const hpspmm_plan* p, const float* v) {
-  return p->nnz > 0 ? v : reinterpret_cast<const float*>(p->d_tcol);
+  return p->nnz > 0 ? v : reinterpret_cast<const float*>(p->d_tent);
 }
 
 template <int K, int WPB>
 int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
   const int64_t blocks = ceil_div(p->rt_waves, WPB) * (K / 32);
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
-                     p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->rt_end3, p->rt_end2, p->rt_end1, p->d_ldesc,
-                     p->d_tcol, p->d_tdesc, readable_values(p, v), B, C, p->d_zrow, p->d_tdepth);
+                     p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent, readable_values(p, v), B, C,
+                     p->d_zrow);
   return HPSPMM_OK;
 }
 
@@ -296,8 +294,8 @@ int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, fl
   const int64_t blocks = (p->rt_wg + ceil_div(wave_items, WPB)) * (K / 32);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
-                     p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->rt_end3, p->rt_end2, p->rt_end1, p->d_ldesc,
-                     p->d_tcol, p->d_tdesc, readable_values(p, v), B, C, p->d_zrow, p->d_tdepth);
+                     p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent,
+                     readable_values(p, v), B, C, p->d_zrow);
   return HPSPMM_OK;
 }
 
@@ -1053,7 +1051,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       return rc;
     }
   }
-  if (p->strategy == HPSPMM_STRATEGY_ROWS && rows_need_tiles && !p->d_tcol) p->strategy = HPSPMM_STRATEGY_SEGMENTS;
+  if (p->strategy == HPSPMM_STRATEGY_ROWS && rows_need_tiles && !p->d_tent) p->strategy = HPSPMM_STRATEGY_SEGMENTS;
 
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS) {
     int forced = (int)((flags >> 8) & 0xFu);
@@ -1117,7 +1115,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       hpspmm_plan_destroy(p);
       return rc;
     }
-    if (p->d_tcol) {
+    if (p->d_tent) {
       (void)hipFree(p->d_nnz_row);
       (void)hipFree(p->d_carry);
       p->d_nnz_row = nullptr;
@@ -1134,7 +1132,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       return rc;
     }
   }
-  if (p->strategy == HPSPMM_STRATEGY_ROWS && !p->d_tcol && p->max_row_nnz > kLongRowThreshold) {
+  if (p->strategy == HPSPMM_STRATEGY_ROWS && !p->d_tent && p->max_row_nnz > kLongRowThreshold) {
     // list of the rows that get a whole wavefront; d_meta[3] counts them
     p->long_threshold = kLongRowThreshold;
     const int64_t cap = nnz / (kLongRowThreshold + 1) + 1;  // cannot be more rows than that
@@ -1196,7 +1194,7 @@ int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
                                                                         : 1;
   out->hub_rows = plan->n_hub;
   out->lds_served_nnz = plan->oserved;
-  out->row_tiles = plan->d_tcol ? plan->rt_tiles : 0;
+  out->row_tiles = plan->d_tent ? plan->rt_tiles : 0;
   return HPSPMM_OK;
 }
 
@@ -1213,8 +1211,7 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
                   (void*)plan->d_vval, (void*)plan->d_vrow, (void*)plan->d_bhot_src, (void*)plan->d_partial,
                   (void*)plan->d_routed_rows, (void*)plan->d_cross_rows, (void*)plan->d_zero_rows,
                   (void*)plan->d_ostart, (void*)plan->d_ocol, (void*)plan->d_osrc, (void*)plan->d_orow,
-                  (void*)plan->d_wcols, (void*)plan->d_tcol, (void*)plan->d_tdesc, (void*)plan->d_ldesc,
-                  (void*)plan->d_zrow, (void*)plan->d_tdepth})
+                  (void*)plan->d_wcols, (void*)plan->d_tent, (void*)plan->d_ldesc, (void*)plan->d_zrow})
     if (q) (void)hipFree(q);
   delete plan;
   return HPSPMM_OK;
@@ -1268,7 +1265,7 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
       case 64: rc = launch_segments<64>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;
       default: rc = launch_segments<128>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;
     }
-  } else if (plan->d_tcol) {
+  } else if (plan->d_tent) {
     switch (plan->k) {
       case 32: rc = launch_row_tiles<32>(plan, d_val, d_B, d_C, st); break;
       case 64: rc = launch_row_tiles<64>(plan, d_val, d_B, d_C, st); break;

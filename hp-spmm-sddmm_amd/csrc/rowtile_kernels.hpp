@@ -1,25 +1,33 @@
 // gfx950 device code for the rows strategy over *row tiles*: the layout a plan
-// builds for a small matrix so that one SpMM is a single launch whose every
-// wavefront has the same, short chain of dependent memory round trips.
+// builds for a small or medium matrix so that one SpMM is a single launch whose
+// every wavefront has the same, short chain of dependent memory round trips.
 //
-// A small SpMM (the 20k-vertex citation graph: 6 us) is bound by that chain, not
-// by bandwidth: a sub-wave that walks a CSR row goes rowptr -> col/val -> B ->
-// store, and a row longer than one staging step repeats col -> B once per step
-// while the rest of its wavefront idles.  Here the plan cuts every row into
-// slots of 8 nonzeros and packs 8 slots into a 64-entry tile, one tile per
-// wavefront:
+// A small SpMM (the 20k-vertex citation graph: 6 us over the CSR arrays) is
+// bound by that chain, not by bandwidth: a sub-wave that walks a CSR row goes
+// rowptr -> col/val -> B -> store, and a row longer than one staging step
+// repeats col -> B once per step while the rest of its wavefront idles.  Here
+// the plan cuts every row into slots of 8 nonzeros and packs 8 slots into a
+// 64-entry tile, one tile per wavefront, one 8-byte record per entry:
 //
-//   tcol[tile][64]   column of every entry, -1 = padding
-//   tdesc[tile][8]   per slot: row (-1 = padding slot), index of its first value
+//   tent[tile][64] = { column (-1 = padding), x }
 //
-// Both are indexed by the wavefront's own number, so columns arrive after one
-// round trip and the B rows and the values after the second.  A row of up to
-// 8 / 16 / 32 / 64 nonzeros takes 1 / 2 / 4 / 8 adjacent slots of one tile
-// (tiles hold rows of one size class only, so the reduction over a row's slots
-// is the same wavefront shuffle for the whole tile); a longer row owns
-// consecutive tiles that one wavefront works through - or, in the second
-// kernel below, a whole workgroup when the row has more than a few hundred
-// nonzeros.  Long rows come first in the grid, since their chain is the longest.
+// where x carries, in the first lanes of a slot, what the slot needs besides
+// its columns: lane 0 the row (-1 = padding slot), lane 1 the index of the
+// slot's first value, and in slot 0 lane 2 the tile's depth (entries per slot
+// that any of its slots uses) and lane 3 log2 of the slots per row.  One load
+// per lane, indexed by the wavefront's own number, brings all of it (first
+// round trip); values and rows of B follow together (second).  Keeping it ONE
+// load is the point: with columns and slot descriptors in two arrays the
+// compiler issued the second load only after the first had arrived.
+//
+// A row of up to 8 / 16 / 32 / 64 nonzeros takes 1 / 2 / 4 / 8 adjacent slots
+// of one tile (tiles hold rows of one size class only, so the reduction over
+// a row's slots is the same wavefront shuffle for the whole tile; one-slot
+// rows are sorted by length first, so a tile of 3-nonzero rows issues 3
+// gathers per lane, not 8); a longer row owns consecutive tiles that one
+// wavefront works through - or, in the second kernel below, a whole workgroup
+// when the row has more than a few hundred nonzeros.  Long rows come first in
+// the grid, since their chain is the longest.
 //
 // K > 32 is served in 32-column tiles of B and C by K/32 workgroups per group
 // of row tiles (workgroup b serves column tile b % (K/32), so an XCD only ever
@@ -39,10 +47,12 @@ constexpr int kSlot = 8;          // nonzeros per slot = lanes per sub-wave at a
 constexpr int kSlotsPerTile = 8;  // slots per tile = sub-waves per wavefront
 constexpr int kRowTile = kSlot * kSlotsPerTile;
 
-// acc += the first N products of the slot, after `c` (this lane's entry of the tile) has been
-// staged in s_col and the load of `v` (its value) issued.  `zrow` = 32 zeros in device memory.
-// Nothing in here is conditional: a padding entry among the first N gathers the zero row instead
-// of a row of B (so that a non-finite value in an unreferenced row of B cannot leak in).
+// acc += the first N products of the slot whose columns are staged in s_col; `c` is this lane's
+// own column, `v` its value (load already issued), `zrow` = 32 zeros in device memory.  Nothing in
+// here is conditional: a padding entry among the first N gathers the zero row instead of a row of
+// B (so that a non-finite value in an unreferenced row of B cannot leak in).  With `if (c >= 0)`
+// around the gathers the compiler copied a loaded register inside the batch and waited for it
+// there - one more dependent round trip in a kernel that is nothing but round trips.
 template <int K, int N>
 __device__ __forceinline__ void gather_n(float4& acc, int32_t c, float v, int tid, int base, int l, int k0,
                                          const int32_t* s_col, float* s_val, const float* __restrict__ B,
@@ -63,99 +73,66 @@ __device__ __forceinline__ void gather_n(float4& acc, int32_t c, float v, int ti
   wave_lds_fence();
 }
 
-// acc += the slot's products.  `vi` = index of this lane's value; `depth` (0..8, the same for the
-// whole wavefront) = entries per slot that any slot of the tile uses: the plan sorts the short rows
-// by length before it packs them, so a tile of 3-nonzero rows issues 3 gathers per lane, not 8.
-// The order matters in a kernel that is nothing but dependent round trips: the value is loaded
-// unconditionally (a padding entry reads val[0] and discards it) and the columns are staged before
-// anything branches on `depth`, so that columns, slot descriptors and depth arrive together (first
-// round trip) and values and rows of B together (second).  With `c >= 0 ? val[vi] : 0`, with
-// `if (c >= 0)` around the gathers, or with the branch on `depth` ahead of the staging, the
-// compiler moved one of the first loads behind a condition that waits for another - a third trip.
+// What a wavefront knows about its tile once the records are staged.
+struct TileInfo {
+  int32_t row;  // of this lane's slot (-1: padding slot)
+  int depth;    // wavefront-uniform
+  int lg;       // wavefront-uniform
+};
+
+// Stages the tile's records (e = this lane's) in LDS, issues the load of this lane's value
+// (unconditionally: a padding entry reads val[0] and discards it) and gathers `depth` entries per
+// slot; depth < 0 = take the tile's own.
 template <int K>
-__device__ __forceinline__ void gather_slot(float4& acc, int depth, int32_t c, int32_t vi, int tid, int base, int l,
-                                            int k0, int32_t* s_col, float* s_val, const float* __restrict__ val,
-                                            const float* __restrict__ B, const float* __restrict__ zrow) {
-  const float v = val[c >= 0 ? vi : 0];
-  s_col[tid] = c;
+__device__ __forceinline__ TileInfo gather_tile(float4& acc, int2 e, int depth, int tid, int base, int l, int k0,
+                                                int32_t* s_col, int32_t* s_x, float* s_val,
+                                                const float* __restrict__ val, const float* __restrict__ B,
+                                                const float* __restrict__ zrow) {
+  s_col[tid] = e.x;
+  s_x[tid] = e.y;
   wave_lds_fence();
-  switch (depth) {
-    case 0: break;
-    case 1: gather_n<K, 1>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    case 2: gather_n<K, 2>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    case 3: gather_n<K, 3>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    case 4: gather_n<K, 4>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    case 5: gather_n<K, 5>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    case 6: gather_n<K, 6>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    case 7: gather_n<K, 7>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    default: gather_n<K, 8>(acc, c, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+  const int wbase = tid & ~63;
+  TileInfo info;
+  info.row = s_x[base];
+  info.depth = depth >= 0 ? depth : __builtin_amdgcn_readfirstlane(s_x[wbase + 2]);
+  info.lg = __builtin_amdgcn_readfirstlane(s_x[wbase + 3]);
+  const float v = val[e.x >= 0 ? s_x[base + 1] + l : 0];
+  switch (info.depth) {
+    case 0: wave_lds_fence(); break;
+    case 1: gather_n<K, 1>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 2: gather_n<K, 2>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 3: gather_n<K, 3>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 4: gather_n<K, 4>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 5: gather_n<K, 5>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 6: gather_n<K, 6>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 7: gather_n<K, 7>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    default: gather_n<K, 8>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
   }
+  return info;
 }
 
-// acc += the products of tiles [t0, t1) of one long row, worked through by one wavefront.
+// acc += the products of tiles [t0, t1) (t0 < t1) of one long row, worked through by one
+// wavefront; returns the row.
 template <int K>
-__device__ __forceinline__ void gather_tiles(float4& acc, int32_t t0, int32_t t1, int lane, int s, int l, int tid,
-                                             int base, int k0, int32_t* s_col, float* s_val,
-                                             const int32_t* __restrict__ tcol, const int2* __restrict__ tdesc,
-                                             const float* __restrict__ val, const float* __restrict__ B,
-                                             const float* __restrict__ zrow) {
-  if (t0 >= t1) return;
-  int32_t c = tcol[(int64_t)t0 * kRowTile + lane];
-  int2 d = tdesc[(int64_t)t0 * kSlotsPerTile + s];
+__device__ __forceinline__ int32_t gather_tiles(float4& acc, int32_t t0, int32_t t1, int lane, int l, int tid,
+                                                int base, int k0, int32_t* s_col, int32_t* s_x, float* s_val,
+                                                const int2* __restrict__ tent, const float* __restrict__ val,
+                                                const float* __restrict__ B, const float* __restrict__ zrow) {
+  int2 e = tent[(int64_t)t0 * kRowTile + lane];
+  int32_t row = -1;
   for (int32_t t = t0; t < t1; ++t) {
-    const int32_t c_now = c, vi_now = d.y + l;
-    if (t + 1 < t1) {  // next tile's entries on their way while this one is gathered
-      c = tcol[(int64_t)(t + 1) * kRowTile + lane];
-      d = tdesc[(int64_t)(t + 1) * kSlotsPerTile + s];
-    }
-    gather_slot<K>(acc, kSlot, c_now, vi_now, tid, base, l, k0, s_col, s_val, val, B, zrow);
+    const int2 e_now = e;
+    if (t + 1 < t1) e = tent[(int64_t)(t + 1) * kRowTile + lane];  // on its way while this tile is gathered
+    row = gather_tile<K>(acc, e_now, kSlot, tid, base, l, k0, s_col, s_x, s_val, val, B, zrow).row;
   }
+  return row;
 }
 
-// Wavefront w < n_loop works through the tiles of long row w (ldesc[w] = first
-// tile, tile count); wavefront w >= n_loop owns tile loop_tiles + (w - n_loop).
-// Tiles [loop_tiles, end3) hold 64-nonzero rows (8 slots each), [end3, end2)
-// 4-slot rows, [end2, end1) 2-slot rows, the rest 1-slot rows.
-template <int K, int WPB>
-__global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves, int32_t n_loop, int32_t loop_tiles,
-                                                               int32_t end3, int32_t end2, int32_t end1,
-                                                               const int2* __restrict__ ldesc,
-                                                               const int32_t* __restrict__ tcol,
-                                                               const int2* __restrict__ tdesc,
-                                                               const float* __restrict__ val,
-                                                               const float* __restrict__ B, float* __restrict__ C,
-                                                               const float* __restrict__ zrow, const int32_t* __restrict__ tdepth) {
-  constexpr int T = K / 32;
-  __shared__ int32_t s_col[WPB * 64];
-  __shared__ float s_val[WPB * 64];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int l = lane & (kSlot - 1);
-  const int s = lane / kSlot;
-  const int base = tid - l;
-  const int k0 = (int)(blockIdx.x % T) * 32;
-  const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(blockIdx.x / T) * WPB + (tid >> 6));
-  if (w >= n_waves) return;
-
-  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  int lg = 3;
-  int32_t row;
-  if (w >= n_loop) {
-    const int32_t tile = loop_tiles + (w - n_loop);
-    lg = tile < end3 ? 3 : tile < end2 ? 2 : tile < end1 ? 1 : 0;
-    const int32_t c = tcol[(int64_t)tile * kRowTile + lane];
-    const int2 d = tdesc[(int64_t)tile * kSlotsPerTile + s];
-    const int depth = __builtin_amdgcn_readfirstlane(tdepth[tile]);
-    __builtin_amdgcn_sched_barrier(0);  // the three loads above are issued before anything waits for one of them
-    row = d.x;
-    gather_slot<K>(acc, depth, c, d.y + l, tid, base, l, k0, s_col, s_val, val, B, zrow);
-  } else {
-    const int2 ld = ldesc[w];
-    row = tdesc[(int64_t)ld.x * kSlotsPerTile].x;
-    gather_tiles<K>(acc, ld.x, ld.x + ld.y, lane, s, l, tid, base, k0, s_col, s_val, tcol, tdesc, val, B, zrow);
-  }
-  // the slots of a row are adjacent and aligned to their count: xor shuffles, in a fixed order
+// Sum over the 2^lg adjacent slots of a row (xor shuffles, in a fixed order), then the row's
+// first slot stores.
+template <int K>
+__device__ __forceinline__ void reduce_and_store(float4 acc, int lg, int32_t row, int s, int l, int k0,
+                                                 float* __restrict__ C) {
 #pragma unroll
   for (int step = 0; step < 3; ++step) {
     if (lg > step) {
@@ -168,6 +145,43 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
   if ((s & ((1 << lg) - 1)) == 0 && row >= 0) store_result(C + (uint64_t)(uint32_t)row * K + k0 + 4 * l, acc);
 }
 
+// Wavefront w < n_loop works through the tiles of long row w (ldesc[w] = first
+// tile, tile count); wavefront w >= n_loop owns tile loop_tiles + (w - n_loop).
+template <int K, int WPB>
+__global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves, int32_t n_loop, int32_t loop_tiles,
+                                                               const int2* __restrict__ ldesc,
+                                                               const int2* __restrict__ tent,
+                                                               const float* __restrict__ val,
+                                                               const float* __restrict__ B, float* __restrict__ C,
+                                                               const float* __restrict__ zrow) {
+  constexpr int T = K / 32;
+  __shared__ int32_t s_col[WPB * 64];
+  __shared__ int32_t s_x[WPB * 64];
+  __shared__ float s_val[WPB * 64];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int l = lane & (kSlot - 1);
+  const int s = lane / kSlot;
+  const int base = tid - l;
+  const int k0 = (int)(blockIdx.x % T) * 32;
+  const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(blockIdx.x / T) * WPB + (tid >> 6));
+  if (w >= n_waves) return;
+
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (w >= n_loop) {
+    const int32_t tile = loop_tiles + (w - n_loop);
+    const int2 e = tent[(int64_t)tile * kRowTile + lane];
+    const TileInfo info = gather_tile<K>(acc, e, -1, tid, base, l, k0, s_col, s_x, s_val, val, B, zrow);
+    reduce_and_store<K>(acc, info.lg, info.row, s, l, k0, C);
+  } else {
+    const int2 ld = ldesc[w];
+    const int32_t row = gather_tiles<K>(acc, ld.x, ld.x + ld.y, lane, l, tid, base, k0, s_col, s_x, s_val, tent, val,
+                                        B, zrow);
+    reduce_and_store<K>(acc, 3, row, s, l, k0, C);
+  }
+}
+
 // The same with a whole workgroup of WPB wavefronts on each of the n_wg longest rows (the first
 // n_wg entries of ldesc; workgroups [0, n_wg) of a column tile; the row's tiles dealt in contiguous
 // shares, the shares' sums added in wavefront order through LDS), for matrices whose longest rows
@@ -175,16 +189,16 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
 // one remaining long row or one ordinary tile each, as above.
 template <int K, int WPB>
 __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_tiles, int32_t n_wg, int32_t n_loop,
-                                                                    int32_t loop_tiles, int32_t end3, int32_t end2,
-                                                                    int32_t end1, const int2* __restrict__ ldesc,
-                                                                    const int32_t* __restrict__ tcol,
-                                                                    const int2* __restrict__ tdesc,
+                                                                    int32_t loop_tiles,
+                                                                    const int2* __restrict__ ldesc,
+                                                                    const int2* __restrict__ tent,
                                                                     const float* __restrict__ val,
                                                                     const float* __restrict__ B,
                                                                     float* __restrict__ C,
-                                                                    const float* __restrict__ zrow, const int32_t* __restrict__ tdepth) {
+                                                                    const float* __restrict__ zrow) {
   constexpr int T = K / 32;
   __shared__ int32_t s_col[WPB * 64];
+  __shared__ int32_t s_x[WPB * 64];
   __shared__ float s_val[WPB * 64];
   __shared__ float4 s_part[WPB][kSlot];
 
@@ -203,7 +217,8 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
     const int32_t per = (ld.y + WPB - 1) / WPB;
     const int32_t t0 = ld.x + wave * per;
     const int32_t t1 = t0 + per < ld.x + ld.y ? t0 + per : ld.x + ld.y;
-    gather_tiles<K>(acc, t0, t1, lane, s, l, tid, base, k0, s_col, s_val, tcol, tdesc, val, B, zrow);
+    int32_t row = -1;  // wavefront 0 always has tiles, the later ones may not
+    if (t0 < t1) row = gather_tiles<K>(acc, t0, t1, lane, l, tid, base, k0, s_col, s_x, s_val, tent, val, B, zrow);
 #pragma unroll
     for (int off = kSlot; off < 64; off <<= 1) {
       acc.x += __shfl_xor(acc.x, off);
@@ -222,40 +237,24 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
         sum.z += p.z;
         sum.w += p.w;
       }
-      const int32_t row = tdesc[(int64_t)ld.x * kSlotsPerTile].x;
       store_result(C + (uint64_t)(uint32_t)row * K + k0 + 4 * l, sum);
     }
     return;
   }
 
   const int32_t w = __builtin_amdgcn_readfirstlane(n_wg + (blk - n_wg) * WPB + wave);
-  int lg = 3;
-  int32_t row;
   if (w < n_loop) {
     const int2 ld = ldesc[w];
-    row = tdesc[(int64_t)ld.x * kSlotsPerTile].x;
-    gather_tiles<K>(acc, ld.x, ld.x + ld.y, lane, s, l, tid, base, k0, s_col, s_val, tcol, tdesc, val, B, zrow);
+    const int32_t row = gather_tiles<K>(acc, ld.x, ld.x + ld.y, lane, l, tid, base, k0, s_col, s_x, s_val, tent, val,
+                                        B, zrow);
+    reduce_and_store<K>(acc, 3, row, s, l, k0, C);
   } else {
     const int32_t tile = loop_tiles + (w - n_loop);
     if (tile >= n_tiles) return;
-    lg = tile < end3 ? 3 : tile < end2 ? 2 : tile < end1 ? 1 : 0;
-    const int32_t c = tcol[(int64_t)tile * kRowTile + lane];
-    const int2 d = tdesc[(int64_t)tile * kSlotsPerTile + s];
-    const int depth = __builtin_amdgcn_readfirstlane(tdepth[tile]);
-    __builtin_amdgcn_sched_barrier(0);  // the three loads above are issued before anything waits for one of them
-    row = d.x;
-    gather_slot<K>(acc, depth, c, d.y + l, tid, base, l, k0, s_col, s_val, val, B, zrow);
+    const int2 e = tent[(int64_t)tile * kRowTile + lane];
+    const TileInfo info = gather_tile<K>(acc, e, -1, tid, base, l, k0, s_col, s_x, s_val, val, B, zrow);
+    reduce_and_store<K>(acc, info.lg, info.row, s, l, k0, C);
   }
-#pragma unroll
-  for (int step = 0; step < 3; ++step) {
-    if (lg > step) {
-      acc.x += __shfl_xor(acc.x, kSlot << step);
-      acc.y += __shfl_xor(acc.y, kSlot << step);
-      acc.z += __shfl_xor(acc.z, kSlot << step);
-      acc.w += __shfl_xor(acc.w, kSlot << step);
-    }
-  }
-  if ((s & ((1 << lg) - 1)) == 0 && row >= 0) store_result(C + (uint64_t)(uint32_t)row * K + k0 + 4 * l, acc);
 }
 
 }  // namespace hpspmm

@@ -492,7 +492,7 @@ constexpr int kRoutedLog2Cached = 16;
 // (8.6 -> 6.1 ms); not on the co-purchase graph, whose columns are too evenly
 // used (4.5 -> 5.5 ms)).
 constexpr int64_t kRoutedMinNnz = (int64_t)1 << 22;
-constexpr int64_t kRoutedMinBBytes = (int64_t)24 << 20;  // a B that one or two L2s hold needs no routing
+constexpr int64_t kRoutedMinBBytes = (int64_t)10 << 20;  // a B that one or two L2s hold needs no routing (social graph at 26 M nonzeros: B = 7 MB, routed 309 us against 246; B = 14 MB, 464 against 474)
 constexpr double kRoutedMinShare = 0.35;     // of the nonzeros in the 64k most referenced columns
 constexpr double kRoutedMinRowNnz = 32.0;    // mean nonzeros per non-empty row
 constexpr int32_t kRoutedRowThreshold = 128;  // rows shorter than this are not split over the classes

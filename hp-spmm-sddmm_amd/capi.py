@@ -31,6 +31,7 @@ PLAN_NO_ROUTED = 128
 PLAN_CLUSTER = 4096
 PLAN_NO_CLUSTER = 8192
 PLAN_NO_ROW_TILES = 16384
+PLAN_ROUTED_SORT_VALUES = 32768
 
 
 def plan_hub_log2(log2_rows):

@@ -90,7 +90,8 @@ struct hpspmm_plan {
   uint16_t* d_lslot = nullptr;    // [nnz] rank of every stored nonzero within its chunk sorted by class-major position
   int32_t* d_chunk_base = nullptr;  // [nchunks * ncls] first class-major position of the chunk's run in each class
   int32_t* d_chunk_pref = nullptr;  // [nchunks * ncls] nonzeros of the chunk in lower classes
-  float* d_vval = nullptr;        // [vtotal] the values in that order, rewritten by every SpMM
+  float* d_vval = nullptr;        // [vtotal] the values in that order, rewritten by every SpMM (not with d_vsrc)
+  int32_t* d_vsrc = nullptr;      // [vtotal] column-range slices: index of every position in the caller's arrays
   int32_t* d_vrow = nullptr;      // [vtotal] routed-row number (hub classes) or row (cold class)
   int32_t* d_bhot_src = nullptr;  // [n_bhot] source column of every compact-buffer row (-1 = unused)
   int32_t* d_routed_rows = nullptr;  // [n_routed] row of every routed-row number
@@ -504,10 +505,30 @@ constexpr double kRoutedMinRoutedShare = 0.3;  // of the nonzeros in rows of at 
 // 2.51 ms; R-MAT scale 22, K = 128 (268 MB a slice) 6.63 / 6.23 / 6.32 ms.
 constexpr int64_t kRoutedPhaseBytes = (int64_t)8 << 20;
 
+// True if the column indices of every row are in non-decreasing order (p->d_nnz_row = row of every
+// nonzero must be there).  Errors count as "no".
+bool columns_sorted(const hpspmm_plan* p, const int32_t* d_col, hipStream_t st) {
+  int32_t* d_flag = nullptr;
+  if (hipMalloc(&d_flag, sizeof(int32_t)) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  int32_t unsorted = 1;
+  hipError_t e = hipMemsetAsync(d_flag, 0, sizeof(int32_t), st);
+  if (e == hipSuccess) {
+    hipLaunchKernelGGL(hpspmm::columns_unsorted_kernel, dim3(grid_for(p->nnz, 1 << 16)), dim3(hpspmm::kBlock), 0, st,
+                       p->nnz, p->d_nnz_row, d_col, d_flag);
+    e = hipMemcpyAsync(&unsorted, d_flag, sizeof(int32_t), hipMemcpyDeviceToHost, st);
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  (void)hipFree(d_flag);
+  return e == hipSuccess && unsorted == 0;
+}
+
 // Builds the routed layout.  Returns HPSPMM_OK with p->strategy left at
 // SEGMENTS when the graph does not qualify (and `forced` is false).
 int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, int log2_hubs,
-                 int log2_row_threshold, int want_sub, hipStream_t st) {
+                 int log2_row_threshold, int want_sub, bool sort_values, hipStream_t st) {
   const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
   if (!forced && (nnz < kRoutedMinNnz || p->cols * k * 4 < kRoutedMinBBytes)) return HPSPMM_OK;
   // cached rows per class
@@ -540,7 +561,34 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   const int32_t min_row_nnz =
       std::max<int32_t>(1, forced && log2_row_threshold ? (1 << log2_row_threshold) : kRoutedRowThreshold);
 
+  // Column-range slices: the columns cut into 8 * nsub consecutive ranges of equal nonzero count
+  // instead of spread by rank and hash.  In a row with sorted columns the nonzeros of one class are
+  // then consecutive, so the kernel reads the values where the caller keeps them and the per-call
+  // re-ordering of the values (0.21 ms of the social graph's 1.2 ms at K = 32) goes away.  Only when
+  // the hot columns spread evenly over the ranges (random vertex labels do that; R-MAT's hot
+  // columns all have small indices and would land in one slice, whose L2 could not hold them) and
+  // with one phase: with two the runs are half as long, the value loads fetch 1.8 lines per run, and
+  // what the re-ordering pass saved is spent inside the main kernel (social graph, K = 128: 3.73 ms
+  // either way; R-MAT: 6.0 -> 6.85 ms).
+  std::vector<uint8_t> colrange;
+  if (!sort_values && nsub == 1 && nnz > 0 && p->d_nnz_row && columns_sorted(p, d_col, st)) {
+    const int groups = nhub;
+    const int64_t target = ceil_div(nnz, groups);
+    std::vector<uint8_t> range((size_t)p->cols);
+    std::vector<int64_t> hot((size_t)groups, 0);
+    int64_t before = 0;
+    for (int64_t c = 0; c < p->cols; ++c) {
+      range[(size_t)c] = (uint8_t)std::min<int64_t>(groups - 1, before / target);
+      before += count[(size_t)c];
+    }
+    for (int32_t c : ids) ++hot[range[(size_t)c]];
+    const int64_t most = *std::max_element(hot.begin(), hot.end());
+    if (most * 2 * groups <= 3 * (int64_t)ids.size() + 32 * groups) colrange.swap(range);
+  }
+  const bool inplace = !colrange.empty();
+
   // temporaries of the layout construction
+  uint8_t* d_colrange = nullptr;
   int32_t* d_colmap = nullptr;
   uint32_t* d_ridx = nullptr;     // [rows + 1] routed flag, then (scanned in place) routed-row number
   uint32_t* d_cnt = nullptr;      // [nhub * n_routed + 1] class-major counts, then their scan
@@ -549,14 +597,18 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   int32_t* d_counts = nullptr;    // [2] list lengths
   int32_t* d_vpos = nullptr;      // [nnz] position of every stored nonzero in the class-major order
   struct Guard {
-    void** q[7];
+    void** q[8];
     ~Guard() {
       for (void** x : q)
         if (*x) (void)hipFree(*x);
     }
   } guard{{(void**)&d_colmap, (void**)&d_ridx, (void**)&d_cnt, (void**)&d_coldcnt, (void**)&d_action,
-           (void**)&d_counts, (void**)&d_vpos}};
+           (void**)&d_counts, (void**)&d_vpos, (void**)&d_colrange}};
   HPSPMM_HIP(hipMalloc(&d_colmap, (size_t)std::max<int64_t>(1, p->cols) * sizeof(int32_t)));
+  if (inplace) {
+    HPSPMM_HIP(hipMalloc(&d_colrange, colrange.size()));
+    HPSPMM_HIP(hipMemcpyAsync(d_colrange, colrange.data(), colrange.size(), hipMemcpyHostToDevice, st));
+  }
   HPSPMM_HIP(hipMalloc(&d_ridx, (size_t)(rows + 1) * sizeof(uint32_t)));
   HPSPMM_HIP(hipMalloc(&d_coldcnt, (size_t)(rows + 1) * sizeof(uint32_t)));
   HPSPMM_HIP(hipMalloc(&d_action, (size_t)rows));
@@ -577,7 +629,8 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   HPSPMM_HIP(hipMalloc(&d_cnt, (size_t)ncnt * sizeof(uint32_t)));
   const unsigned row_grid = (unsigned)ceil_div(rows, hpspmm::kWavesPerBlock);
   hipLaunchKernelGGL(hpspmm::routed_count_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, n_routed,
-                     d_rowptr, d_col, d_colmap, d_ridx, (int32_t)h, nsub, min_row_nnz, d_cnt, d_coldcnt);
+                     d_rowptr, d_col, d_colmap, d_ridx, (int32_t)h, nsub, (const uint8_t*)d_colrange, min_row_nnz, d_cnt,
+                     d_coldcnt);
   if (int rc = exclusive_scan_u32(d_cnt, d_cnt, ncnt, st)) return rc;
   if (int rc = exclusive_scan_u32(d_coldcnt, d_coldcnt, rows + 1, st)) return rc;
 
@@ -639,14 +692,20 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   // the segments strategy's buffers are not needed any more
   if (p->d_nnz_row) { (void)hipFree(p->d_nnz_row); p->d_nnz_row = nullptr; }
   if (p->d_carry) { (void)hipFree(p->d_carry); p->d_carry = nullptr; }
-  const size_t total_bytes = rvptr_bytes + coldptr_bytes + 3 * v_bytes + lslot_bytes + 2 * chunk_bytes +
-                             partial_bytes + carry_bytes + bhot_bytes + (size_t)n_bhot * 4 + 2 * list_bytes +
-                             routed_rows_bytes;
-  if (hipMalloc(&p->d_rvptr, rvptr_bytes) != hipSuccess || hipMalloc(&p->d_coldptr, coldptr_bytes) != hipSuccess ||
-      hipMalloc(&p->d_vcol, v_bytes) != hipSuccess || hipMalloc(&p->d_vval, v_bytes) != hipSuccess ||
-      hipMalloc(&p->d_vrow, v_bytes) != hipSuccess || hipMalloc(&d_vpos, vpos_bytes) != hipSuccess ||
-      hipMalloc(&p->d_lslot, lslot_bytes) != hipSuccess || hipMalloc(&p->d_chunk_base, chunk_bytes) != hipSuccess ||
-      hipMalloc(&p->d_chunk_pref, chunk_bytes) != hipSuccess ||
+  const size_t total_bytes = rvptr_bytes + coldptr_bytes + 3 * v_bytes +
+                             (inplace ? 0 : lslot_bytes + 2 * chunk_bytes) + partial_bytes + carry_bytes +
+                             bhot_bytes + (size_t)n_bhot * 4 + 2 * list_bytes + routed_rows_bytes;
+  // (the order of these allocations is felt: with the values allocated after the rows instead of
+  // between columns and rows the social graph at K = 32 ran 3 % slower - where the three streams
+  // that a sub-wave reads in step lie relative to each other decides how they share the channels)
+  bool ok = hipMalloc(&p->d_rvptr, rvptr_bytes) == hipSuccess && hipMalloc(&p->d_coldptr, coldptr_bytes) == hipSuccess &&
+            hipMalloc(&p->d_vcol, v_bytes) == hipSuccess &&
+            hipMalloc(inplace ? (void**)&p->d_vsrc : (void**)&p->d_vval, v_bytes) == hipSuccess &&
+            hipMalloc(&p->d_vrow, v_bytes) == hipSuccess && hipMalloc(&d_vpos, vpos_bytes) == hipSuccess;
+  if (ok && !inplace)
+    ok = hipMalloc(&p->d_lslot, lslot_bytes) == hipSuccess && hipMalloc(&p->d_chunk_base, chunk_bytes) == hipSuccess &&
+         hipMalloc(&p->d_chunk_pref, chunk_bytes) == hipSuccess;
+  if (!ok ||
       hipMalloc(&p->d_partial, partial_bytes) != hipSuccess || hipMalloc(&p->d_carry, carry_bytes) != hipSuccess ||
       hipMalloc(&p->d_bhot, bhot_bytes) != hipSuccess ||
       hipMalloc(&p->d_bhot_src, (size_t)n_bhot * sizeof(int32_t)) != hipSuccess ||
@@ -660,7 +719,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
                             hipMemcpyHostToDevice, st));
   // unused compact-buffer rows and the padding between the classes are never used; keep them defined anyway
   HPSPMM_HIP(hipMemsetAsync(p->d_bhot, 0, bhot_bytes, st));
-  HPSPMM_HIP(hipMemsetAsync(p->d_vval, 0, v_bytes, st));
+  HPSPMM_HIP(hipMemsetAsync(inplace ? (void*)p->d_vsrc : (void*)p->d_vval, 0, v_bytes, st));
   HPSPMM_HIP(hipMemsetAsync(d_counts, 0, 2 * sizeof(int32_t), st));
   const int64_t nrv = (n_routed + 1) * nhub;
   hipLaunchKernelGGL(hpspmm::routed_vptr_kernel, dim3((unsigned)ceil_div(nrv, hpspmm::kBlock)), dim3(hpspmm::kBlock),
@@ -668,12 +727,13 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   hipLaunchKernelGGL(hpspmm::routed_coldptr_kernel, dim3((unsigned)ceil_div(rows + 1, hpspmm::kBlock)),
                      dim3(hpspmm::kBlock), 0, st, rows, lay.cls_begin[nhub], d_coldcnt, p->d_coldptr);
   hipLaunchKernelGGL(hpspmm::routed_fill_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col,
-                     d_colmap, d_ridx, (int32_t)h, nsub, min_row_nnz, p->d_rvptr, p->d_coldptr, p->d_vcol, d_vpos,
-                     p->d_vrow, p->d_routed_rows, d_action, p->shift);
+                     d_colmap, d_ridx, (int32_t)h, nsub, (const uint8_t*)d_colrange, min_row_nnz, p->d_rvptr,
+                     p->d_coldptr, p->d_vcol, d_vpos, p->d_vsrc, p->d_vrow, p->d_routed_rows, d_action, p->shift);
   // chunk tables of the value scatter
   if (nchunks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
-  hipLaunchKernelGGL(hpspmm::routed_chunk_kernel, dim3((unsigned)nchunks), dim3(hpspmm::kBlock), 0, st, lay, nnz, d_vpos,
-                     p->d_lslot, p->d_chunk_base, p->d_chunk_pref);
+  if (!inplace)
+    hipLaunchKernelGGL(hpspmm::routed_chunk_kernel, dim3((unsigned)nchunks), dim3(hpspmm::kBlock), 0, st, lay, nnz,
+                       d_vpos, p->d_lslot, p->d_chunk_base, p->d_chunk_pref);
   // compact lists of the short rows the final kernel has to visit
   const unsigned cgrid = (unsigned)ceil_div(rows, hpspmm::kBlock);
   hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(cgrid), dim3(hpspmm::kBlock), 0, st, rows, d_action,
@@ -696,7 +756,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
 template <int K>
 int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
   // values bound to the plan are already in class-major order: only the hub rows of B are refreshed
-  const int64_t permute_nnz = (p->bound_val && p->bound_val == v) ? 0 : p->nnz;
+  const int64_t permute_nnz = (p->d_vsrc || (p->bound_val && p->bound_val == v)) ? 0 : p->nnz;
   const int64_t gather_blocks = ceil_div(p->n_bhot * (K / 4), hpspmm::kBlock);
   const int64_t prep_blocks = gather_blocks + ceil_div(permute_nnz, hpspmm::kPermChunk);
   if (prep_blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
@@ -704,10 +764,16 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
     hipLaunchKernelGGL(hpspmm::routed_prepare_kernel<K>, dim3((unsigned)prep_blocks), dim3(hpspmm::kBlock), 0, st,
                        p->n_bhot, gather_blocks, p->d_bhot_src, B, p->d_bhot, p->nnz, p->lay.nhub + 1, v, p->d_lslot,
                        p->d_chunk_base, p->d_chunk_pref, p->d_vval);
-  if (p->routed_grid > 0)
-    hipLaunchKernelGGL(hpspmm::spmm_routed_kernel<K>, dim3((unsigned)p->routed_grid), dim3(hpspmm::kBlock), 0, st,
-                       p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval, p->d_vrow, B, p->d_bhot, p->d_partial,
-                       p->d_carry, C);
+  if (p->routed_grid > 0) {
+    if (p->d_vsrc)
+      hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, true>), dim3((unsigned)p->routed_grid), dim3(hpspmm::kBlock), 0,
+                         st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, v, p->d_vsrc, p->d_vrow, B, p->d_bhot,
+                         p->d_partial, p->d_carry, C);
+    else
+      hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false>), dim3((unsigned)p->routed_grid), dim3(hpspmm::kBlock),
+                         0, st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval, (const int32_t*)nullptr,
+                         p->d_vrow, B, p->d_bhot, p->d_partial, p->d_carry, C);
+  }
   const int64_t routed_blocks = row_blocks(p->lay.n_routed, K);
   const int64_t cross_blocks = row_blocks(p->n_cross, K);
   const int64_t fin_blocks = routed_blocks + cross_blocks + row_blocks(p->n_zero, K);
@@ -1084,7 +1150,8 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     if (int rc = build_routed(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_ROUTED) != 0,
                               (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 16) & 0xFFu) : 0,
                               (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 24) & 0x1Fu) : 0,
-                              (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 29) & 0x7u) : 0, st)) {
+                              (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 29) & 0x7u) : 0,
+                              (flags & HPSPMM_PLAN_ROUTED_SORT_VALUES) != 0, st)) {
       hpspmm_plan_destroy(p);
       return rc;
     }
@@ -1208,7 +1275,7 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
   if (plan->d_bhot) (void)hipFree(plan->d_bhot);
   for (void* q : {(void*)plan->d_rvptr, (void*)plan->d_coldptr, (void*)plan->d_vcol, (void*)plan->d_lslot,
                   (void*)plan->d_chunk_base, (void*)plan->d_chunk_pref,
-                  (void*)plan->d_vval, (void*)plan->d_vrow, (void*)plan->d_bhot_src, (void*)plan->d_partial,
+                  (void*)plan->d_vval, (void*)plan->d_vsrc, (void*)plan->d_vrow, (void*)plan->d_bhot_src, (void*)plan->d_partial,
                   (void*)plan->d_routed_rows, (void*)plan->d_cross_rows, (void*)plan->d_zero_rows,
                   (void*)plan->d_ostart, (void*)plan->d_ocol, (void*)plan->d_osrc, (void*)plan->d_orow,
                   (void*)plan->d_wcols, (void*)plan->d_tent, (void*)plan->d_ldesc, (void*)plan->d_zrow})
@@ -1221,7 +1288,7 @@ int hpspmm_plan_bind_values(hpspmm_plan* plan, const float* d_val, void* stream)
   if (!plan) return fail(HPSPMM_ERR_INVALID_ARG, "plan is NULL");
   plan->bound_val = nullptr;
   if (!d_val || plan->nnz == 0) return HPSPMM_OK;
-  if (plan->strategy == HPSPMM_STRATEGY_ROUTED) {
+  if (plan->strategy == HPSPMM_STRATEGY_ROUTED && !plan->d_vsrc) {
     hipStream_t st = (hipStream_t)stream;
     // the value half of routed_prepare_kernel alone (its template argument only shapes the other half)
     const int64_t blocks = ceil_div(plan->nnz, hpspmm::kPermChunk);

@@ -91,10 +91,29 @@ __device__ __forceinline__ int hub_class_of(int32_t c, int32_t mapped, int32_t h
   return sub * kSlices + slice;
 }
 
+// The same when the plan has cut the columns into 8 * nsub consecutive ranges of equal nonzero count
+// instead (colrange[c] = range of column c; slice = range / nsub, phase = range % nsub): in a row
+// with sorted columns the nonzeros of one class are then consecutive, so the values can be read
+// where the caller keeps them.  `single` = the row keeps everything in phase 0.
+__device__ __forceinline__ int range_class_of(int range, int nsub, bool single) {
+  const int slice = range / nsub;
+  return single ? slice : (range - slice * nsub) * kSlices + slice;
+}
+
 // A routed row shorter than this many times the routing threshold keeps all its nonzeros in phase 0
 // (one partial-result row per slice instead of one per slice and phase; 233k-vertex social graph,
 // K = 128: 3.77 -> 3.70 ms with 2, no further gain with 4, where R-MAT loses 0.1 ms).
 constexpr int kSinglePhaseFactor = 2;
+
+// *flag |= 1 if some row has a column index smaller than the one before it (row[] = row of every nonzero).
+__global__ __launch_bounds__(kBlock) void columns_unsorted_kernel(int64_t nnz, const int32_t* __restrict__ row,
+                                                                  const int32_t* __restrict__ col,
+                                                                  int32_t* __restrict__ flag) {
+  bool bad = false;
+  for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j + 1 < nnz; j += (int64_t)gridDim.x * kBlock)
+    bad |= row[j] == row[j + 1] && col[j] > col[j + 1];
+  if (__ballot(bad) != 0 && (threadIdx.x & 63) == 0) atomicOr(flag, 1);
+}
 
 // flag[r] = 1 if row r is routed (r < rows), flag[rows] = 0.
 __global__ __launch_bounds__(kBlock) void routed_flag_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
@@ -114,6 +133,7 @@ __global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t rows, int6
                                                               const int32_t* __restrict__ colmap,
                                                               const uint32_t* __restrict__ ridx,
                                                               int32_t hub_rows_per_slice, int nsub,
+                                                              const uint8_t* __restrict__ colrange,
                                                               int32_t min_row_nnz, uint32_t* __restrict__ cnt,
                                                               uint32_t* __restrict__ coldcnt) {
   const int lane = threadIdx.x & 63;
@@ -137,7 +157,9 @@ __global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t rows, int6
     int cls = -1;
     if (j < hb) {
       const int32_t c = col[j];
-      cls = hub_class_of(c, colmap[c], hub_rows_per_slice, hb - lb < kSinglePhaseFactor * min_row_nnz ? 1 : nsub);
+      const bool single = hb - lb < kSinglePhaseFactor * min_row_nnz;
+      cls = colrange ? range_class_of(colrange[c], nsub, single)
+                     : hub_class_of(c, colmap[c], hub_rows_per_slice, single ? 1 : nsub);
     }
     for (int x = 0; x < nhub; ++x) {
       const uint64_t m = __ballot(cls == x);
@@ -255,9 +277,11 @@ __global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const
                                                              const int32_t* __restrict__ colmap,
                                                              const uint32_t* __restrict__ ridx,
                                                              int32_t hub_rows_per_slice, int nsub,
+                                                             const uint8_t* __restrict__ colrange,
                                                              int32_t min_row_nnz, const int32_t* __restrict__ rvptr,
                                                              const int32_t* __restrict__ coldptr,
                                                              int32_t* __restrict__ vcol, int32_t* __restrict__ vpos,
+                                                             int32_t* __restrict__ vsrc /* or NULL */,
                                                              int32_t* __restrict__ vrow,
                                                              int32_t* __restrict__ routed_rows,
                                                              uint8_t* __restrict__ action, int shift) {
@@ -282,6 +306,7 @@ __global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const
       const int32_t pos = start + (j - lb);
       vcol[pos] = mapped >= 0 ? ~mapped : c;  // ~compact-buffer row if the column is cached
       vpos[j] = pos;
+      if (vsrc) vsrc[pos] = j;
       vrow[pos] = (int32_t)row;
     }
     return;
@@ -298,8 +323,10 @@ __global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const
     const bool valid = j < hb;
     const int32_t c = valid ? col[j] : 0;
     const int32_t mapped = valid ? colmap[c] : -1;
-    const int cls =
-        valid ? hub_class_of(c, mapped, hub_rows_per_slice, hb - lb < kSinglePhaseFactor * min_row_nnz ? 1 : nsub) : -1;
+    const bool single = hb - lb < kSinglePhaseFactor * min_row_nnz;
+    const int cls = !valid      ? -1
+                    : colrange ? range_class_of(colrange[c], nsub, single)
+                               : hub_class_of(c, mapped, hub_rows_per_slice, single ? 1 : nsub);
     for (int x = 0; x < nhub; ++x) {
       const uint64_t m = __ballot(cls == x);
       if (m == 0) continue;
@@ -308,6 +335,7 @@ __global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const
         const int32_t pos = start + (int32_t)__popcll(m & below);
         vcol[pos] = mapped >= 0 ? ~mapped : c;
         vpos[j] = pos;
+        if (vsrc) vsrc[pos] = j;
         vrow[pos] = r;
       }
       if (lane == x) cursor += (int32_t)__popcll(m);
@@ -449,11 +477,15 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
 // Each sub-wave owns one segment of its class; see the carry rule of the
 // segments kernel - in a hub class "stored to C" becomes "stored to the routed
 // row's partial-result slot of the class".
-template <int K>
+// kInPlace: vval is the caller's value array in its own order and vsrc[q] the index into it of
+// the class-major position q (column-range slices: consecutive positions of a run are consecutive
+// indices, so these loads stay coalesced).
+template <int K, bool kInPlace>
 __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, const int32_t* __restrict__ rvptr,
                                                              const int32_t* __restrict__ coldptr,
                                                              const int32_t* __restrict__ vcol,
                                                              const float* __restrict__ vval,
+                                                             const int32_t* __restrict__ vsrc,
                                                              const int32_t* __restrict__ vrow,
                                                              const float* __restrict__ B,
                                                              const float* __restrict__ Bhot,
@@ -515,7 +547,14 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
   auto fetch = [&](TileRegs<TL>& m, int64_t t) {
     const int64_t q = t + l * TL;
     load_run<TL>(m.c, vcol, q, e, true);
-    load_run<TL>(m.v, vval, q, e, true);
+    if constexpr (kInPlace) {
+      int32_t src[TL];
+      load_run<TL>(src, vsrc, q, e, true);  // 0 beyond e: a readable index, the value is never consumed
+#pragma unroll
+      for (int i = 0; i < TL; ++i) m.v[i] = vval[src[i]];
+    } else {
+      load_run<TL>(m.v, vval, q, e, true);
+    }
     load_run<TL>(m.r, vrow, q, e, true);
   };
   TileRegs<TL> m;

@@ -76,6 +76,9 @@ typedef enum hpspmm_status {
                                          plans of one matrix may order the rows differently and then differ
                                          in the last bits of C; one plan always gives the same bits */
 #define HPSPMM_PLAN_NO_CLUSTER 8192u  /* never */
+#define HPSPMM_PLAN_ROUTED_SORT_VALUES 32768u /* routed strategy: never cut the columns into consecutive ranges (which lets
+                                         the kernel read the values in place); always spread them by popularity rank and
+                                         hash and bring the values into the plan's order at the start of every SpMM */
 #define HPSPMM_PLAN_NO_ROW_TILES 16384u /* rows strategy: walk the caller's CSR arrays instead of building row tiles */
 
 /* strategy reported by hpspmm_plan_get_info */

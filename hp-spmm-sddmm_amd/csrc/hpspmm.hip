@@ -756,7 +756,9 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
 template <int K>
 int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
   // values bound to the plan are already in class-major order: only the hub rows of B are refreshed
-  const int64_t permute_nnz = (p->d_vsrc || (p->bound_val && p->bound_val == v)) ? 0 : p->nnz;
+  const bool bound = p->bound_val && p->bound_val == v;
+  const bool inplace = p->d_vsrc && !(bound && p->d_vval);
+  const int64_t permute_nnz = (p->d_vsrc || bound) ? 0 : p->nnz;
   const int64_t gather_blocks = ceil_div(p->n_bhot * (K / 4), hpspmm::kBlock);
   const int64_t prep_blocks = gather_blocks + ceil_div(permute_nnz, hpspmm::kPermChunk);
   if (prep_blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
@@ -765,7 +767,7 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
                        p->n_bhot, gather_blocks, p->d_bhot_src, B, p->d_bhot, p->nnz, p->lay.nhub + 1, v, p->d_lslot,
                        p->d_chunk_base, p->d_chunk_pref, p->d_vval);
   if (p->routed_grid > 0) {
-    if (p->d_vsrc)
+    if (inplace)
       hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, true>), dim3((unsigned)p->routed_grid), dim3(hpspmm::kBlock), 0,
                          st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, v, p->d_vsrc, p->d_vrow, B, p->d_bhot,
                          p->d_partial, p->d_carry, C);
@@ -1288,7 +1290,23 @@ int hpspmm_plan_bind_values(hpspmm_plan* plan, const float* d_val, void* stream)
   if (!plan) return fail(HPSPMM_ERR_INVALID_ARG, "plan is NULL");
   plan->bound_val = nullptr;
   if (!d_val || plan->nnz == 0) return HPSPMM_OK;
-  if (plan->strategy == HPSPMM_STRATEGY_ROUTED && !plan->d_vsrc) {
+  if (plan->strategy == HPSPMM_STRATEGY_ROUTED && plan->d_vsrc) {
+    // column-range slices: constant values are worth a copy in the plan's order after all (reading them
+    // in place costs the main kernel what a bound plan no longer pays in re-ordering)
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t vtotal = plan->lay.cls_end[plan->lay.nhub];
+    if (!plan->d_vval) {
+      if (hipMalloc(&plan->d_vval, (size_t)std::max<int64_t>(vtotal, 1) * sizeof(float)) != hipSuccess) {
+        (void)hipGetLastError();
+        plan->d_vval = nullptr;
+        return fail(HPSPMM_ERR_ALLOC, "device allocation for the bound values failed");
+      }
+      plan->workspace_bytes += vtotal * (int64_t)sizeof(float);
+    }
+    hipLaunchKernelGGL(hpspmm::routed_gather_values_kernel, dim3(grid_for(vtotal, 1 << 16)), dim3(hpspmm::kBlock), 0,
+                       st, vtotal, plan->d_vsrc, d_val, plan->d_vval);
+    HPSPMM_HIP(hipGetLastError());
+  } else if (plan->strategy == HPSPMM_STRATEGY_ROUTED) {
     hipStream_t st = (hipStream_t)stream;
     // the value half of routed_prepare_kernel alone (its template argument only shapes the other half)
     const int64_t blocks = ceil_div(plan->nnz, hpspmm::kPermChunk);

@@ -115,6 +115,14 @@ __global__ __launch_bounds__(kBlock) void columns_unsorted_kernel(int64_t nnz, c
   if (__ballot(bad) != 0 && (threadIdx.x & 63) == 0) atomicOr(flag, 1);
 }
 
+// dst[q] = val[src[q]]: the values in the plan's order, once, for a caller who has declared them constant.
+__global__ __launch_bounds__(kBlock) void routed_gather_values_kernel(int64_t n, const int32_t* __restrict__ src,
+                                                                      const float* __restrict__ val,
+                                                                      float* __restrict__ dst) {
+  for (int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x; q < n; q += (int64_t)gridDim.x * kBlock)
+    dst[q] = val[src[q]];
+}
+
 // flag[r] = 1 if row r is routed (r < rows), flag[rows] = 0.
 __global__ __launch_bounds__(kBlock) void routed_flag_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                              int32_t min_row_nnz, uint32_t* __restrict__ flag) {

@@ -56,6 +56,7 @@ def _strategies(capi):
             ("seg16_hub_all", capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(4) | capi.PLAN_HUB_CACHE
              | capi.plan_hub_log2(24)),
             ("routed", capi.PLAN_FORCE_ROUTED),
+            ("routed_sort_values", capi.PLAN_FORCE_ROUTED | capi.PLAN_ROUTED_SORT_VALUES),
             ("routed_tiny", capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(3) | capi.plan_segment_shift(3)
              | capi.plan_routed_row_log2(1)),
             ("routed_s16", capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(10) | capi.plan_segment_shift(4)

@@ -161,7 +161,10 @@ int hpspmm_plan_destroy(hpspmm_plan *plan);
  * that order once, here, instead of at the start of every SpMM; later
  * hpspmm_csr_spmm calls that pass this same d_val use the stored copy; a call
  * with any other pointer works as if nothing was bound and drops the binding.
- * d_val = NULL unbinds.
+ * d_val = NULL unbinds.  (Where a plan reads the values in place anyway - rows,
+ * ordered, routed with column-range slices - binding changes nothing or, in
+ * the last case, makes the plan keep a copy in its own order: device memory
+ * for nnz floats is allocated here, not in hpspmm_csr_spmm.)
  * This is where the reference's HP-SpMM does the same work: its preprocessing
  * emits the values in its own processing order before the timed loop
  * (spmm/mm/spmm_common.cpp:269-277, test/test_all.cpp:38-40).  A caller that

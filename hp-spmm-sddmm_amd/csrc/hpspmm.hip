@@ -571,7 +571,8 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   // what the re-ordering pass saved is spent inside the main kernel (social graph, K = 128: 3.73 ms
   // either way; R-MAT: 6.0 -> 6.85 ms).
   std::vector<uint8_t> colrange;
-  if (!sort_values && nsub == 1 && nnz > 0 && p->d_nnz_row && columns_sorted(p, d_col, st)) {
+  if (!sort_values && nsub == 1 && nnz > 0 && p->cols * k * 4 < ((int64_t)1 << 32) && p->d_nnz_row &&
+      columns_sorted(p, d_col, st)) {
     const int groups = nhub;
     const int64_t target = ceil_div(nnz, groups);
     std::vector<uint8_t> range((size_t)p->cols);
@@ -586,6 +587,14 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
     if (most * 2 * groups <= 3 * (int64_t)ids.size() + 32 * groups) colrange.swap(range);
   }
   const bool inplace = !colrange.empty();
+  // Evenly spread hot columns also mean that their rows of B do not crowd a few memory channels, which
+  // is what the compact buffer is for (R-MAT): without it (social graph, K = 32: 1.128 against
+  // 1.135 ms with it) the kernel's gather address is a 32-bit offset from B and the hot rows need
+  // no copying at the start of every SpMM.
+  if (inplace) {
+    std::fill(colmap.begin(), colmap.end(), -1);
+    std::fill(bhot_src.begin(), bhot_src.end(), -1);
+  }
 
   // temporaries of the layout construction
   uint8_t* d_colrange = nullptr;
@@ -746,8 +755,8 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   HPSPMM_HIP(hipGetLastError());
   p->n_cross = counts[0];
   p->n_zero = counts[1];
-  p->n_bhot = n_bhot;
-  p->n_hub = (int64_t)ids.size();
+  p->n_bhot = inplace ? 0 : n_bhot;
+  p->n_hub = inplace ? 0 : (int64_t)ids.size();
   p->nseg = nseg;
   p->strategy = HPSPMM_STRATEGY_ROUTED;
   return HPSPMM_OK;
@@ -768,13 +777,17 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
                        p->d_chunk_base, p->d_chunk_pref, p->d_vval);
   if (p->routed_grid > 0) {
     if (inplace)
-      hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, true>), dim3((unsigned)p->routed_grid), dim3(hpspmm::kBlock), 0,
-                         st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, v, p->d_vsrc, p->d_vrow, B, p->d_bhot,
-                         p->d_partial, p->d_carry, C);
-    else
-      hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false>), dim3((unsigned)p->routed_grid), dim3(hpspmm::kBlock),
-                         0, st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval, (const int32_t*)nullptr,
+      hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, true, false>), dim3((unsigned)p->routed_grid),
+                         dim3(hpspmm::kBlock), 0, st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, v, p->d_vsrc,
                          p->d_vrow, B, p->d_bhot, p->d_partial, p->d_carry, C);
+    else if (p->d_vsrc)  // column-range slices, values bound: the plan's own copy of them, still no compact buffer
+      hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false, false>), dim3((unsigned)p->routed_grid),
+                         dim3(hpspmm::kBlock), 0, st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval,
+                         (const int32_t*)nullptr, p->d_vrow, B, p->d_bhot, p->d_partial, p->d_carry, C);
+    else
+      hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false, true>), dim3((unsigned)p->routed_grid),
+                         dim3(hpspmm::kBlock), 0, st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval,
+                         (const int32_t*)nullptr, p->d_vrow, B, p->d_bhot, p->d_partial, p->d_carry, C);
   }
   const int64_t routed_blocks = row_blocks(p->lay.n_routed, K);
   const int64_t cross_blocks = row_blocks(p->n_cross, K);
@@ -1257,7 +1270,7 @@ int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
   out->max_row_nnz = plan->max_row_nnz;
   out->empty_rows = plan->empty_rows;
   out->workspace_bytes = plan->workspace_bytes;
-  out->launches_per_spmm = plan->strategy == HPSPMM_STRATEGY_ROUTED    ? 3
+  out->launches_per_spmm = plan->strategy == HPSPMM_STRATEGY_ROUTED    ? (plan->d_vsrc ? 2 : 3)
                            : plan->strategy == HPSPMM_STRATEGY_ORDERED ? 2
                            : plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? (plan->n_hub > 0 ? 3 : 2)
                                                                         : 1;

@@ -487,8 +487,10 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
 // row's partial-result slot of the class".
 // kInPlace: vval is the caller's value array in its own order and vsrc[q] the index into it of
 // the class-major position q (column-range slices: consecutive positions of a run are consecutive
-// indices, so these loads stay coalesced).
-template <int K, bool kInPlace>
+// indices, so these loads stay coalesced).  kHub: vcol may hold ~(compact-buffer row); without it
+// every entry is a plain column and the gather address is B plus a 32-bit byte offset (the plan
+// checks that B is below 4 GB), three instructions instead of eight.
+template <int K, bool kInPlace, bool kHub>
 __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, const int32_t* __restrict__ rvptr,
                                                              const int32_t* __restrict__ coldptr,
                                                              const int32_t* __restrict__ vcol,
@@ -549,7 +551,14 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
     store_result(dst + 4 * l, acc);
   };
   auto flush = [&]() { flush_to(false); };
-  auto loadb = [&](int32_t c) { return load_b_hub<K, true>(B, Bhot, c, l); };
+  auto loadb = [&](int32_t c) {
+    if constexpr (kHub) {
+      return load_b_hub<K, true>(B, Bhot, c, l);
+    } else {
+      const uint32_t off = (uint32_t)c * (uint32_t)(K * 4) + (uint32_t)(16 * l);
+      return *reinterpret_cast<const float4*>(reinterpret_cast<const char*>(B) + off);
+    }
+  };
 
   // the plan's arrays are allocated by the library, hence always aligned for the vector loads
   // In place the value of a position needs its index first: the indices are fetched two tiles ahead

@@ -106,11 +106,20 @@ def test_deterministic_and_strategies_agree(pkg, oracle, gpu):
     ref, _ = _run(pkg, gpu, g, B, pkg.capi.PLAN_FORCE_SEGMENTS)
     again, _ = _run(pkg, gpu, g, B, pkg.capi.PLAN_FORCE_SEGMENTS)
     assert np.array_equal(ref, again), "segments strategy must be bit-reproducible"
-    fl = pkg.capi.PLAN_FORCE_ROUTED | pkg.capi.plan_hub_log2(9) | pkg.capi.plan_routed_row_log2(2)
+    # hashed slices with the compact buffer of hot rows (the column-range slices keep none)
+    fl = (pkg.capi.PLAN_FORCE_ROUTED | pkg.capi.PLAN_ROUTED_SORT_VALUES | pkg.capi.plan_hub_log2(9)
+          | pkg.capi.plan_routed_row_log2(2))
     r1, info = _run(pkg, gpu, g, B, fl)
     r2, _ = _run(pkg, gpu, g, B, fl)
     assert info["strategy"] == pkg.capi.STRATEGY_ROUTED and info["hub_rows"] > 0
     assert np.array_equal(r1, r2), "routed strategy must be bit-reproducible"
+    # column-range slices where the plan finds them usable: values in place, no compact buffer, two launches
+    fl = pkg.capi.PLAN_FORCE_ROUTED | pkg.capi.plan_routed_row_log2(2)
+    q1, info = _run(pkg, gpu, g, B, fl)
+    q2, _ = _run(pkg, gpu, g, B, fl)
+    assert info["strategy"] == pkg.capi.STRATEGY_ROUTED
+    assert (info["launches_per_spmm"], info["hub_rows"] > 0) in ((2, False), (3, True))
+    assert np.array_equal(q1, q2), "routed strategy must be bit-reproducible"
     rows, _ = _run(pkg, gpu, g, B, pkg.capi.PLAN_FORCE_ROWS)
     # the whole-row kernel accumulates in stored order with FMA; rows that fit one
     # segment are accumulated identically by the segments kernel

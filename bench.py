@@ -9,9 +9,21 @@ HBM once, and every timed region starts with them resident.
 
     value        geometric mean of the per-workload GFLOPS
     ms_per_step  sum of the per-workload mean SpMM times
-    roofline     social graph, K=128 (the longest-running launch of a step):
-                 algorithmic bytes 4(M+1) + 8 nnz + 4 K nnz + 4 K M per SpMM
-                 divided by the mean SpMM time, against 8 TB/s
+    roofline     social graph, K=128, its dominant kernel (spmm_routed_kernel):
+                 frac         algorithmic bytes 4(M+1) + 8 nnz + 4 K nnz + 4 K M
+                              (the B gather counted once per nonzero) divided by
+                              that kernel's mean duration, against 8 TB/s.  L2 and
+                              LDS serve most of the gather, so this figure is not
+                              bounded by 1;
+                 traffic_frac bytes that kernel moves between the L2s and the
+                              fabric (rocprofv3 FETCH_SIZE / WRITE_SIZE, carried
+                              in MEASURED_TRAFFIC below and checked against
+                              profiles/ by tests/test_bench_constants.py) divided
+                              by the same duration, against 8 TB/s: <= 1;
+                 unique_frac  the bytes that must move at least once
+                              (A, every row of B once, C) over the same time.
+                 Every per_workload record carries the same three figures for
+                 the whole SpMM, the per-launch times and the roof that applies.
     cpu_baseline the FP32 CPU oracle on a bounded row sample of the same
                  social-graph workload, on this machine's host cores
 
@@ -44,12 +56,35 @@ WORKLOADS = [
 ]
 ROOFLINE_WORKLOAD = ("c2_social", 128)
 
-# L2<->fabric bytes per SpMM (all launches) of the roofline workload, from two rocprofv3 --pmc
-# runs (FETCH_SIZE, WRITE_SIZE, each scaled by what a 1 GiB copy kernel reads on the same
-# counter); summary in profiles/spmm_routed_kernel__c2_social.txt.  Counters cannot be read
-# from inside this process, so the figure is carried here and only reported for the exact
-# configuration it was measured on: (workload, K, strategy) at scale 1.
-MEASURED_TRAFFIC_BYTES = {("c2_social", 128, 4): 1.238e9 + 19.809e9 + 1.433e9}
+# L2<->fabric bytes per launch, by kernel, of the five large workloads: rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (two runs), each scaled by what a 1 GiB copy kernel reads on the same counter (x2 for
+# FETCH_SIZE, x1 for WRITE_SIZE).  Counters cannot be read from inside this process, so the figures
+# are carried here, in GB as the summaries under profiles/ print them; tests/test_bench_constants.py
+# fails when they differ from those files.  They are reported only for the configuration they were
+# measured on: same workload, K, strategy and number of launches, scale 1, default plan.
+MEASURED_TRAFFIC = {
+    ("c2_social", 32): {"strategy": 4, "launches": 2, "profile": "profiles/spmm_routed_kernel__c2_social.txt",
+                        "kernels": {"spmm_routed_kernel": 4.770, "spmm_routed_final_kernel": 0.268}},
+    ("c2_social", 64): {"strategy": 4, "launches": 2, "profile": "profiles/spmm_routed_kernel__c2_social.txt",
+                        "kernels": {"spmm_routed_kernel": 10.631, "spmm_routed_final_kernel": 0.529}},
+    ("c2_social", 128): {"strategy": 4, "launches": 3, "profile": "profiles/spmm_routed_kernel__c2_social.txt",
+                         "kernels": {"routed_prepare_kernel": 1.238, "spmm_routed_kernel": 19.813,
+                                     "spmm_routed_final_kernel": 1.433}},
+    ("c3_copurchase", 64): {"strategy": 5, "launches": 2, "profile": "profiles/spmm_ordered_kernel__c3_copurchase.txt",
+                            "kernels": {"spmm_ordered_kernel": 21.233, "spmm_fixup_kernel": 0.203}},
+    ("c4_rmat", 128): {"strategy": 4, "launches": 3, "profile": "profiles/spmm_routed_kernel__c4_rmat.txt",
+                       "kernels": {"routed_prepare_kernel": 1.378, "spmm_routed_kernel": 37.833,
+                                   "spmm_routed_final_kernel": 2.118}},
+}
+
+# What bounds each workload.
+ROOF = {
+    "c1_citation": "launch latency: one launch of ~2 dependent memory round trips; no bandwidth roof applies",
+    "c2_social": "L2 delivery: B fits no L2 whole but its hot rows do; the gather runs against the all-hit "
+                 "gather rate of the L2 -> CU path (l2_delivery_frac), traffic_frac is the secondary roof",
+    "c3_copurchase": "fabric: L2 misses move at the rate the L2 <-> fabric path sustains (traffic_frac)",
+    "c4_rmat": "fabric: L2 misses move at the rate the L2 <-> fabric path sustains (traffic_frac)",
+}
 
 
 def log(*a):
@@ -72,6 +107,21 @@ def ensure_built():
     if not all(os.path.exists(p) for p in needed):
         import __graft_entry__
         __graft_entry__.build()
+
+
+def l2_delivery_ceiling(capi, graphs, dev, stream, k, steps):
+    """GB/s of B-row bytes delivered to the CUs when every gather hits the L2: the segments kernel on
+    a matrix whose B (2048 rows) fits every L2, 32 M nonzeros.  Measured live, per K."""
+    import torch
+    g = graphs.uniform_rows(65536, 2048, 512, 99)
+    B = graphs.dense_normal(g.cols, k, 99)
+    d = [torch.from_numpy(a).to(dev) for a in (g.rowptr, g.col, g.val, B)]
+    C = torch.empty((g.rows, k), device=dev, dtype=torch.float32)
+    plan = capi.Plan(g.rows, g.cols, d[0], d[1], k,
+                     capi.PLAN_FORCE_SEGMENTS | capi.PLAN_NO_HUB_CACHE | capi.PLAN_NO_ROUTED | capi.PLAN_NO_CLUSTER)
+    ms = capi.csr_spmm_timed(plan, d[0], d[1], d[2], d[3], C, warmup=3, iters=max(5, min(steps, 30)), stream=stream)
+    plan.destroy()
+    return 4.0 * k * g.nnz / (ms * 1e-3) / 1e9
 
 
 def cpu_baseline(graphs, g, B, k, C_gpu_host_rows, budget_nnz):
@@ -121,6 +171,9 @@ def main():
     ap.add_argument("--no-values-bound", action="store_true",
                     help="skip the additional timing with hpspmm_plan_bind_values (keeps a profile of this "
                          "run to the launches of the figure of merit)")
+    ap.add_argument("--no-launch-breakdown", action="store_true",
+                    help="skip the per-launch timing and the all-hit gather probe (keeps a profile of this run "
+                         "to the launches of the figure of merit)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three 1 GiB device-to-device copies (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -207,34 +260,72 @@ def main():
                 plan.bind_values(None, stream)
             gflops = 2.0 * g.nnz * k / (ms * 1e-3) / 1e9
             abytes = algorithmic_bytes(g.rows, g.nnz, k)
+            ubytes = unique_bytes(g.rows, g.cols, g.nnz, k)
             gbs = abytes / (ms * 1e-3) / 1e9
+            # every launch of one SpMM on its own (events between the launches)
+            if args.no_launch_breakdown:
+                launches = [("all launches of one SpMM", ms)]
+            else:
+                launches = capi.csr_spmm_timed_launches(plan, d_rp, d_ci, d_v, d_B, d_C, warmup=2,
+                                                        iters=max(3, min(args.steps, 50)), stream=stream)
+            main_name, main_ms = max(launches, key=lambda kv: kv[1])
             rec = {
                 "workload": name, "k": k, "rows": g.rows, "nnz": g.nnz, "ms": ms, "wall_ms": wall_ms,
                 "gflops": gflops, "ms_values_bound": ms_bound,
                 "gflops_values_bound": 2.0 * g.nnz * k / (ms_bound * 1e-3) / 1e9, "algorithmic_gb": abytes / 1e9, "achieved_gbs": gbs,
                 "roofline_frac": gbs / HBM_PEAK_GBS,
-                "unique_bytes_gb": unique_bytes(g.rows, g.cols, g.nnz, k) / 1e9,
+                "unique_bytes_gb": ubytes / 1e9,
+                "unique_frac": ubytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                "launch_ms": {n_: t_ for n_, t_ in launches},
+                "roof": ROOF.get(name, ""),
                 "strategy": info["strategy"], "segment_length": info["segment_length"],
                 "launches_per_spmm": info["launches_per_spmm"], "plan_ms": plan_ms,
+                "plan_over_spmm": plan_ms / ms,
                 "plan_workspace_mb": info["workspace_bytes"] / 1e6,
+                "plan_workspace_over_csr": info["workspace_bytes"] / (4.0 * (g.rows + 1) + 8.0 * g.nnz),
                 "max_degree": st["max_degree"], "cv": st["cv"],
             }
+            mt = MEASURED_TRAFFIC.get((name, k))
+            if not (mt and args.scale == 1.0 and args.plan_flags == 0 and mt["strategy"] == info["strategy"]
+                    and mt["launches"] == info["launches_per_spmm"]):
+                mt = None
+            if mt:
+                total = sum(mt["kernels"].values()) * 1e9
+                rec["traffic_gb"] = total / 1e9
+                rec["traffic_frac"] = total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+                rec["traffic_over_unique"] = total / ubytes
+                rec["traffic_profile"] = mt["profile"]
+            if name == "c2_social" and not args.no_launch_breakdown:
+                ceil_gbs = l2_delivery_ceiling(capi, graphs, dev, stream, k, args.steps)
+                rec["l2_delivery_ceiling_gbs"] = ceil_gbs
+                rec["l2_delivery_frac"] = 4.0 * k * g.nnz / (main_ms * 1e-3) / 1e9 / ceil_gbs
             results.append(rec)
             log(f"[{name} K={k}] {ms:.4f} ms  {gflops:.1f} GFLOPS  {gbs:.0f} GB/s algorithmic "
                 f"({100 * gbs / HBM_PEAK_GBS:.1f}% of 8 TB/s)  strategy={info['strategy']} seg={info['segment_length']} "
                 f"plan={plan_ms:.1f} ms" + ("" if args.no_values_bound else f"  [values bound: {ms_bound:.4f} ms]"))
+            log("    launches: " + ", ".join(f"{n_} {t_ * 1e3:.1f} us" for n_, t_ in launches)
+                + (f";  traffic {rec['traffic_gb']:.2f} GB = {rec['traffic_frac']:.2f} of 8 TB/s, "
+                   f"{rec['traffic_over_unique']:.1f}x unique" if mt else "")
+                + (f";  L2 delivery {rec['l2_delivery_frac']:.2f} of {rec['l2_delivery_ceiling_gbs']:.0f} GB/s all-hit"
+                   if "l2_delivery_frac" in rec else ""))
             if (name, k) == ROOFLINE_WORKLOAD:
-                roofline = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                            "frac": gbs / HBM_PEAK_GBS,
-                            "traffic": MEASURED_TRAFFIC_BYTES.get((name, k, info["strategy"]))
-                            if args.scale == 1.0 and args.plan_flags == 0 else None,
-                            "kernel": {1: "spmm_rowtiles_kernel<128>",
-                                       2: "spmm_segments_kernel<128> + spmm_fixup_kernel<128>",
-                                       4: "routed_prepare_kernel<128> + spmm_routed_kernel<128> + "
-                                          "spmm_routed_final_kernel<128>"}.get(info["strategy"], "?")
-                                      + " (all launches of one SpMM)",
+                main_gbs = abytes / (main_ms * 1e-3) / 1e9
+                main_traffic = mt["kernels"].get(main_name) * 1e9 if mt and main_name in mt["kernels"] else None
+                roofline = {"bound": "hbm", "achieved": main_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": main_gbs / HBM_PEAK_GBS,
+                            "traffic": main_traffic,
+                            "traffic_frac": (main_traffic / (main_ms * 1e-3) / 1e9 / HBM_PEAK_GBS) if main_traffic else None,
+                            "unique_frac": ubytes / (main_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                            "kernel": f"{main_name}<{k}> (the dominant launch of one SpMM)",
                             "workload": f"{name} K={k}", "algorithmic_bytes_per_launch": abytes,
-                            "mean_launch_ms": ms}
+                            "mean_launch_ms": main_ms,
+                            "whole_spmm_ms": ms,
+                            "roof": ROOF.get(name, ""),
+                            "l2_delivery_frac": rec.get("l2_delivery_frac"),
+                            "note": "frac follows the byte model that counts the B gather once per nonzero; most of "
+                                    "that gather is served by L2 and LDS, so frac exceeds 1 and bounds nothing. "
+                                    "traffic_frac (measured L2<->fabric bytes of this kernel / its duration / 8 TB/s) "
+                                    "is the bounded figure; per_workload carries it for every large workload."}
                 if not args.no_cpu_baseline:
                     rows_chk = min(g.rows, 4096)
                     c_rows = d_C[:rows_chk].cpu().numpy()

@@ -32,10 +32,11 @@ PLAN_CLUSTER = 4096
 PLAN_NO_CLUSTER = 8192
 PLAN_NO_ROW_TILES = 16384
 PLAN_ROUTED_SORT_VALUES = 32768
+PLAN_ALLOW_MOVED_CSR = 1 << 21
 
 
 def plan_hub_log2(log2_rows):
-    return (int(log2_rows) & 0xFF) << 16
+    return (int(log2_rows) & 0x1F) << 16
 
 
 def plan_routed_row_log2(log2_nnz):
@@ -61,6 +62,7 @@ EXPORTS = (
     "hpspmm_version", "hpspmm_last_error", "hpspmm_plan_create", "hpspmm_plan_get_info",
     "hpspmm_plan_destroy", "hpspmm_csr_spmm", "hpspmm_csr_spmm_noplan", "hpspmm_coo_spmm_accumulate",
     "hpspmm_fill_f32", "hpspmm_csr_spmm_timed", "hpspmm_plan_bind_values", "hpspmm_plan_create_ordered",
+    "hpspmm_csr_spmm_timed_launches",
 )
 
 _i64 = ctypes.c_int64
@@ -112,6 +114,9 @@ def lib():
         L.hpspmm_fill_f32.argtypes = [_p, _i64, ctypes.c_float, _p]
         L.hpspmm_csr_spmm_timed.argtypes = [_p, _p, _p, _p, _p, _p, _p, ctypes.c_int, ctypes.c_int,
                                             ctypes.POINTER(ctypes.c_float)]
+        L.hpspmm_csr_spmm_timed_launches.argtypes = [_p, _p, _p, _p, _p, _p, _p, ctypes.c_int, ctypes.c_int,
+                                                     ctypes.c_int, ctypes.POINTER(ctypes.c_float),
+                                                     ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(ctypes.c_int)]
         _lib = L
     return _lib
 
@@ -251,3 +256,15 @@ def csr_spmm_timed(plan, rowptr, col, val, B, C, warmup=20, iters=200, stream=No
     check(lib().hpspmm_csr_spmm_timed(plan._h, _ptr(rowptr), _ptr(col), _ptr(val), _ptr(B), _ptr(C),
                                       _stream(stream), warmup, iters, ctypes.byref(ms)))
     return float(ms.value)
+
+
+def csr_spmm_timed_launches(plan, rowptr, col, val, B, C, warmup=5, iters=50, stream=None):
+    """[(kernel name, mean ms)] for every launch of one SpMM, in launch order (HIP events between the launches)."""
+    _check_operands(plan.rows, plan.cols, plan.nnz, plan.k, rowptr, col, val, B, C)
+    cap = 8
+    ms = (ctypes.c_float * cap)()
+    names = (ctypes.c_char_p * cap)()
+    n = ctypes.c_int(0)
+    check(lib().hpspmm_csr_spmm_timed_launches(plan._h, _ptr(rowptr), _ptr(col), _ptr(val), _ptr(B), _ptr(C),
+                                               _stream(stream), warmup, iters, cap, ms, names, ctypes.byref(n)))
+    return [(names[i].decode(), float(ms[i])) for i in range(n.value)]

@@ -8,7 +8,9 @@
 #include <climits>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -41,6 +43,22 @@ int fail(int code, const char* fmt, ...) {
   } while (0)
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Per-launch timing (hpspmm_csr_spmm_timed_launches): while a trace is active on the calling
+// thread, every kernel launch of an SpMM is followed by an event record on the launch stream.
+constexpr int kMaxTracedLaunches = 8;
+struct LaunchTrace {
+  hipEvent_t ev[kMaxTracedLaunches];
+  const char* name[kMaxTracedLaunches];
+  int n = 0;
+};
+thread_local LaunchTrace* g_trace = nullptr;
+inline void mark_launch(hipStream_t st, const char* name) {
+  LaunchTrace* t = g_trace;
+  if (!t || t->n >= kMaxTracedLaunches) return;
+  (void)hipEventRecord(t->ev[t->n], st);
+  t->name[t->n++] = name;
+}
 
 inline bool fast_k(int64_t k) { return k == 32 || k == 64 || k == 128; }
 
@@ -75,6 +93,10 @@ struct hpspmm_plan {
   int64_t nseg = 0;
   int64_t max_row_nnz = 0, empty_rows = 0;
   bool xcd_remap = true;
+  // the arrays the plan was built from: hpspmm_csr_spmm refuses others unless the caller opted out
+  const int32_t* src_rowptr = nullptr;
+  const int32_t* src_col = nullptr;
+  bool allow_moved = false;
   int32_t* d_nnz_row = nullptr;  // [nnz]
   float* d_carry = nullptr;      // [2 * nseg * k]
   // hub cache (segments strategy, optional): the n_hub most referenced rows of B
@@ -124,6 +146,47 @@ struct hpspmm_plan {
 
 namespace {
 
+// The routed strategy pins column slices to XCDs and xcd_remap deals row ranges to them; both rely on
+// workgroup b of a launch running on XCD b % 8.  That holds for the whole device (8 XCDs, 256 CUs);
+// a partitioned device (fewer XCDs behind one HIP device) or a future dispatcher would break it
+// silently, so it is measured once per device: 512 probe workgroups report the XCD they ran on.
+// 0 = not probed yet, 1 = workgroup b runs on XCD b % 8, 2 = it does not (the plan then keeps to the
+// strategies that do not depend on it).
+constexpr int kMaxDevices = 64;
+constexpr int kProbeBlocks = 512;
+std::mutex g_xcd_mutex;
+int g_xcd_state[kMaxDevices] = {0};
+
+bool xcd_dealing_holds(hipStream_t st) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return false;
+  }
+  if (const char* forced = std::getenv("HPSPMM_XCD_DEALING")) {  // diagnostics: skip the probe
+    if (forced[0] == '0' || forced[0] == '1') return forced[0] == '1';
+  }
+  std::lock_guard<std::mutex> lock(g_xcd_mutex);
+  if (g_xcd_state[dev]) return g_xcd_state[dev] == 1;
+  int32_t* d_ids = nullptr;
+  int32_t ids[kProbeBlocks];
+  bool ok = hipMalloc(&d_ids, sizeof ids) == hipSuccess;
+  if (ok) {
+    hipLaunchKernelGGL(hpspmm::xcc_probe_kernel, dim3(kProbeBlocks), dim3(64), 0, st, d_ids);
+    ok = hipMemcpyAsync(ids, d_ids, sizeof ids, hipMemcpyDeviceToHost, st) == hipSuccess &&
+         hipStreamSynchronize(st) == hipSuccess;
+  }
+  if (d_ids) (void)hipFree(d_ids);
+  if (!ok) {
+    (void)hipGetLastError();
+    return false;  // not cached: a transient failure should not decide for the life of the process
+  }
+  int match = 0;
+  for (int b = 0; b < kProbeBlocks; ++b) match += ids[b] == b % hpspmm::kXcds;
+  g_xcd_state[dev] = match == kProbeBlocks ? 1 : 2;
+  return g_xcd_state[dev] == 1;
+}
+
 // Launch geometry of the kernels that run one sub-wave per row.
 inline int64_t row_blocks(int64_t rows, int64_t k) {
   const int64_t per_wave = 64 / (k / 4);
@@ -150,6 +213,7 @@ int launch_rows_tiled(int64_t rows, const int32_t* rp, const int32_t* ci, const 
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   hipLaunchKernelGGL((hpspmm::spmm_rows_kernel<K, KT>), dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rows, rp,
                      ci, v, B, C, short_blocks, long_threshold, long_rows, n_long);
+  mark_launch(st, "spmm_rows_kernel");
   return HPSPMM_OK;
 }
 
@@ -195,6 +259,9 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
   int64_t by_len[kSlot + 1] = {0};  // one-slot rows by length, longest first: tiles of equal depth
   for (int64_t r = 0; r < rows; ++r) {
     const int32_t n = rp[r + 1] - rp[r];
+    // an unchecked rowptr (HPSPMM_PLAN_NO_VALIDATE) that is not monotone or runs past nnz: no tiles,
+    // the CSR kernel is left to the caller's arrays as they are
+    if (n < 0 || rp[r] < 0 || (int64_t)rp[r] + n > nnz) return HPSPMM_OK;
     const int c = class_of(n);
     ++count[c];
     if (c == 0) ++by_len[n];
@@ -286,6 +353,7 @@ int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, flo
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent, readable_values(p, v), B, C,
                      p->d_zrow);
+  mark_launch(st, "spmm_rowtiles_kernel");
   return HPSPMM_OK;
 }
 
@@ -297,6 +365,7 @@ int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, fl
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent,
                      readable_values(p, v), B, C, p->d_zrow);
+  mark_launch(st, "spmm_rowtiles_wg_kernel");
   return HPSPMM_OK;
 }
 
@@ -328,6 +397,7 @@ int launch_rows_any(int64_t rows, int64_t cols, int64_t k, const int32_t* rp, co
       const int64_t blocks = ceil_div(rows, hpspmm::kWavesPerBlock);
       hipLaunchKernelGGL(hpspmm::spmm_rows_generic_kernel, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st,
                          rows, k, rp, ci, v, B, C);
+      mark_launch(st, "spmm_rows_generic_kernel");
       return HPSPMM_OK;
     }
   }
@@ -349,6 +419,7 @@ int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, 
       const int64_t threads = p->n_hub * (K / 4);
       hipLaunchKernelGGL(hpspmm::gather_hub_rows_kernel<K>, dim3((unsigned)ceil_div(threads, hpspmm::kBlock)),
                          dim3(hpspmm::kBlock), 0, st, p->n_hub, p->d_hub_ids, B, p->d_bhot);
+      mark_launch(st, "gather_hub_rows_kernel");
       hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, false, true>), dim3((unsigned)grid), dim3(hpspmm::kBlock),
                          0, st, rp, p->d_hub_col, v, p->d_nnz_row, B, p->d_bhot, C, p->d_carry, p->nnz, p->shift,
                          p->nseg, nblocks, p->xcd_remap, aligned16(p->d_hub_col, v, p->d_nnz_row));
@@ -358,11 +429,13 @@ int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, 
                          p->d_carry, p->nnz, p->shift, p->nseg, nblocks, p->xcd_remap,
                          aligned16(ci, v, p->d_nnz_row));
     }
+    mark_launch(st, "spmm_segments_kernel");
   }
   const int rpw = fixup_rows_per_wave(p->rows, K);
   const int64_t fix_blocks = ceil_div(ceil_div(p->rows, rpw), hpspmm::kWavesPerBlock);
   hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st, p->rows,
                      rp, (const int32_t*)nullptr, p->d_carry, C, p->shift, rpw);
+  mark_launch(st, "spmm_fixup_kernel");
   return HPSPMM_OK;
 }
 
@@ -377,14 +450,17 @@ int launch_ordered(const hpspmm_plan* p, const int32_t* rp, const float* v, cons
   const int64_t nblocks = p->owindows;
   const int64_t grid = p->xcd_remap ? ceil_div(nblocks, hpspmm::kXcds) * hpspmm::kXcds : nblocks;
   if (grid > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
-  if (p->nnz > 0)
+  if (p->nnz > 0) {
     hipLaunchKernelGGL(hpspmm::spmm_ordered_kernel<K>, dim3((unsigned)grid), dim3(hpspmm::kBlock),
                        (size_t)p->ocap * K * sizeof(float), st, rp, p->d_ostart, p->d_ocol, p->d_osrc, p->d_orow, v,
                        p->d_wcols, p->ocap, B, C, p->d_carry, p->nnz, p->shift, nblocks, p->xcd_remap);
+    mark_launch(st, "spmm_ordered_kernel");
+  }
   const int rpw = fixup_rows_per_wave(p->rows, K);
   const int64_t fix_blocks = ceil_div(ceil_div(p->rows, rpw), hpspmm::kWavesPerBlock);
   hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st, p->rows,
                      rp, p->d_ostart, p->d_carry, C, p->shift, rpw);
+  mark_launch(st, "spmm_fixup_kernel");
   return HPSPMM_OK;
 }
 
@@ -771,10 +847,12 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
   const int64_t gather_blocks = ceil_div(p->n_bhot * (K / 4), hpspmm::kBlock);
   const int64_t prep_blocks = gather_blocks + ceil_div(permute_nnz, hpspmm::kPermChunk);
   if (prep_blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
-  if (prep_blocks > 0)
+  if (prep_blocks > 0) {
     hipLaunchKernelGGL(hpspmm::routed_prepare_kernel<K>, dim3((unsigned)prep_blocks), dim3(hpspmm::kBlock), 0, st,
                        p->n_bhot, gather_blocks, p->d_bhot_src, B, p->d_bhot, p->nnz, p->lay.nhub + 1, v, p->d_lslot,
                        p->d_chunk_base, p->d_chunk_pref, p->d_vval);
+    mark_launch(st, "routed_prepare_kernel");
+  }
   if (p->routed_grid > 0) {
     if (inplace)
       hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, true, false>), dim3((unsigned)p->routed_grid),
@@ -788,14 +866,17 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
       hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false, true>), dim3((unsigned)p->routed_grid),
                          dim3(hpspmm::kBlock), 0, st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval,
                          (const int32_t*)nullptr, p->d_vrow, B, p->d_bhot, p->d_partial, p->d_carry, C);
+    mark_launch(st, "spmm_routed_kernel");
   }
   const int64_t routed_blocks = row_blocks(p->lay.n_routed, K);
   const int64_t cross_blocks = row_blocks(p->n_cross, K);
   const int64_t fin_blocks = routed_blocks + cross_blocks + row_blocks(p->n_zero, K);
-  if (fin_blocks > 0)
+  if (fin_blocks > 0) {
     hipLaunchKernelGGL(hpspmm::spmm_routed_final_kernel<K>, dim3((unsigned)fin_blocks), dim3(hpspmm::kBlock), 0, st,
                        p->lay, p->d_rvptr, p->d_coldptr, p->d_routed_rows, routed_blocks, p->d_cross_rows, p->n_cross,
                        cross_blocks, p->d_zero_rows, p->n_zero, p->d_partial, p->d_carry, C);
+    mark_launch(st, "spmm_routed_final_kernel");
+  }
   return HPSPMM_OK;
 }
 
@@ -911,7 +992,7 @@ constexpr double kClusterMinServed = 0.15;
 // Finds a processing order for a square matrix by label propagation on its graph: rows of one
 // label next to each other, labels in increasing order, rows of a label in increasing order.
 // d_order_out receives a device array of `rows` entries (caller frees).
-constexpr int kClusterMaxSweeps = 10;
+constexpr int kClusterMaxSweeps = 16;
 
 int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st,
                  int32_t** d_order_out, double* intra_share_out) {
@@ -919,15 +1000,17 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
   *d_order_out = nullptr;
   *intra_share_out = 0.0;
   int32_t* d_label = nullptr;
+  int32_t* d_label_next = nullptr;
   uint32_t* d_changed = nullptr;
   struct Guard {
-    void** q[2];
+    void** q[3];
     ~Guard() {
       for (void** x : q)
         if (*x) (void)hipFree(*x);
     }
-  } guard{{(void**)&d_label, (void**)&d_changed}};
+  } guard{{(void**)&d_label, (void**)&d_label_next, (void**)&d_changed}};
   HPSPMM_HIP(hipMalloc(&d_label, (size_t)rows * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&d_label_next, (size_t)rows * sizeof(int32_t)));
   HPSPMM_HIP(hipMalloc(&d_changed, hpspmm::kClusterCounters * sizeof(uint32_t)));
   std::vector<uint32_t> counters((size_t)hpspmm::kClusterCounters);
   hipLaunchKernelGGL(hpspmm::cluster_init_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock),
@@ -935,7 +1018,9 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
   for (int sweep = 0; sweep < kClusterMaxSweeps; ++sweep) {
     HPSPMM_HIP(hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st));
     hipLaunchKernelGGL(hpspmm::cluster_sweep_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
-                       dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_label, (uint32_t)sweep, d_changed);
+                       dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_label, d_label_next, (uint32_t)sweep,
+                       d_changed);
+    std::swap(d_label, d_label_next);
     HPSPMM_HIP(hipMemcpyAsync(counters.data(), d_changed, counters.size() * sizeof(uint32_t), hipMemcpyDeviceToHost,
                               st));
     HPSPMM_HIP(hipStreamSynchronize(st));
@@ -1077,13 +1162,24 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
 
   hpspmm_plan* p = new (std::nothrow) hpspmm_plan;
   if (!p) return fail(HPSPMM_ERR_ALLOC, "out of host memory");
+  // every exit but the last - an error return or an exception - frees the plan and what it owns
+  struct PlanHolder {
+    hpspmm_plan* plan;
+    ~PlanHolder() { hpspmm_plan_destroy(plan); }
+  } holder{p};
   p->rows = rows;
   p->cols = cols;
   p->nnz = nnz;
   p->k = k;
   p->max_row_nnz = stats[0];
   p->empty_rows = stats[1];
-  p->xcd_remap = !(flags & HPSPMM_PLAN_NO_XCD_REMAP);
+  p->src_rowptr = d_rowptr;
+  p->src_col = d_col;
+  p->allow_moved = (flags & HPSPMM_PLAN_ALLOW_MOVED_CSR) != 0;
+  // strategies that place work on particular XCDs are used only where the dealing of workgroups to
+  // XCDs they assume has been observed on this device
+  const bool xcd_ok = xcd_dealing_holds(st);
+  p->xcd_remap = !(flags & HPSPMM_PLAN_NO_XCD_REMAP) && xcd_ok;
 
   // Automatic choice, in this order: tiny matrix -> rows; a matrix in the rows strategy's range
   // (`rows_range`) -> ordered if it has communities, else rows; beyond that range -> routed if a
@@ -1094,9 +1190,9 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     p->strategy = HPSPMM_STRATEGY_GENERIC_K;
   } else if (d_order && nnz > 0) {
     if (int rc = build_ordered(p, d_rowptr, d_col, d_order, 0.0, st)) {
-      hpspmm_plan_destroy(p);
       return rc;
     }
+    holder.plan = nullptr;
     *plan_out = p;
     return HPSPMM_OK;
   } else if (flags & HPSPMM_PLAN_FORCE_ROWS) {
@@ -1128,7 +1224,6 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
 
   if (p->strategy == HPSPMM_STRATEGY_ROWS && rows > 0 && nnz < kRowTileMaxNnz && !(flags & HPSPMM_PLAN_NO_ROW_TILES)) {
     if (int rc = build_row_tiles(p, d_rowptr, d_col, st)) {
-      hpspmm_plan_destroy(p);
       return rc;
     }
   }
@@ -1137,7 +1232,6 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS) {
     int forced = (int)((flags >> 8) & 0xFu);
     if (forced && (forced < 3 || forced > 15)) {
-      delete p;
       return fail(HPSPMM_ERR_INVALID_ARG, "forced segment shift %d outside [3, 15]", forced);
     }
     p->shift = forced ? forced : choose_shift(nnz, k, p->max_row_nnz);
@@ -1146,7 +1240,6 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     const size_t carry_bytes = (size_t)(p->nseg > 0 ? p->nseg : 1) * 2 * (size_t)k * sizeof(float);
     if (hipMalloc(&p->d_nnz_row, row_bytes) != hipSuccess || hipMalloc(&p->d_carry, carry_bytes) != hipSuccess) {
       (void)hipGetLastError();
-      hpspmm_plan_destroy(p);
       return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the plan failed", row_bytes + carry_bytes);
     }
     p->workspace_bytes = (int64_t)(row_bytes + carry_bytes);
@@ -1155,19 +1248,18 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
                          dim3(hpspmm::kBlock), 0, st, rows, nnz, d_rowptr, p->d_nnz_row);
       hipError_t e = hipStreamSynchronize(st);
       if (e != hipSuccess) {
-        hpspmm_plan_destroy(p);
         return fail(HPSPMM_ERR_HIP, "row expansion failed: %s", hipGetErrorString(e));
       }
     }
   }
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && !(flags & HPSPMM_PLAN_NO_ROUTED) && nnz > 0 && !rows_range &&
+      (xcd_ok || (flags & HPSPMM_PLAN_FORCE_ROUTED)) &&
       !(flags & HPSPMM_PLAN_FORCE_SEGMENTS && !(flags & HPSPMM_PLAN_FORCE_ROUTED))) {
     if (int rc = build_routed(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_ROUTED) != 0,
-                              (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 16) & 0xFFu) : 0,
+                              (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 16) & 0x1Fu) : 0,
                               (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 24) & 0x1Fu) : 0,
                               (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 29) & 0x7u) : 0,
                               (flags & HPSPMM_PLAN_ROUTED_SORT_VALUES) != 0, st)) {
-      hpspmm_plan_destroy(p);
       return rc;
     }
   }
@@ -1187,14 +1279,12 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       rc = build_ordered(p, d_rowptr, d_col, d_order, want_cluster ? 0.0 : kClusterMinServed, st);
     if (d_order) (void)hipFree(d_order);
     if (rc) {
-      hpspmm_plan_destroy(p);
       return rc;
     }
   }
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && rows_range) {
     // no communities: whole rows after all, if the row tiles get built
     if (int rc = build_row_tiles(p, d_rowptr, d_col, st)) {
-      hpspmm_plan_destroy(p);
       return rc;
     }
     if (p->d_tent) {
@@ -1209,8 +1299,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     }
   }
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && !(flags & HPSPMM_PLAN_NO_HUB_CACHE) && nnz > 0) {
-    if (int rc = build_hub_cache(p, d_col, (int)((flags >> 16) & 0xFFu), (flags & HPSPMM_PLAN_HUB_CACHE) != 0, st)) {
-      hpspmm_plan_destroy(p);
+    if (int rc = build_hub_cache(p, d_col, (int)((flags >> 16) & 0x1Fu), (flags & HPSPMM_PLAN_HUB_CACHE) != 0, st)) {
       return rc;
     }
   }
@@ -1220,7 +1309,6 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     const int64_t cap = nnz / (kLongRowThreshold + 1) + 1;  // cannot be more rows than that
     if (hipMalloc(&p->d_long_rows, (size_t)cap * sizeof(int32_t)) != hipSuccess) {
       (void)hipGetLastError();
-      hpspmm_plan_destroy(p);
       return fail(HPSPMM_ERR_ALLOC, "device allocation of the long-row list failed");
     }
     p->workspace_bytes += cap * (int64_t)sizeof(int32_t);
@@ -1230,29 +1318,48 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     hipError_t e = hipMemcpyAsync(&n_long, d_meta + 3, sizeof n_long, hipMemcpyDeviceToHost, st);
     if (e == hipSuccess) e = hipStreamSynchronize(st);
     if (e != hipSuccess || n_long < 0 || n_long > cap) {
-      hpspmm_plan_destroy(p);
       return fail(HPSPMM_ERR_HIP, "long-row collection failed: %s", hipGetErrorString(e));
     }
     p->n_long = n_long;
   }
+  holder.plan = nullptr;
   *plan_out = p;
   return HPSPMM_OK;
 }
 
+// No C++ exception crosses the C ABI: the host-side steps of plan construction allocate vectors
+// sized by the input, and a failed allocation there becomes HPSPMM_ERR_ALLOC; the plan under
+// construction and the temporaries of the step that threw are freed by their guards.
+static int plan_create_guarded(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr,
+                               const int32_t* d_col, int64_t k, uint32_t flags, const int32_t* d_order, void* stream,
+                               hpspmm_plan** plan_out) {
+  int rc;
+  try {
+    rc = plan_create_impl(rows, cols, nnz, d_rowptr, d_col, k, flags, d_order, stream, plan_out);
+  } catch (const std::bad_alloc&) {
+    if (plan_out) *plan_out = nullptr;
+    rc = fail(HPSPMM_ERR_ALLOC, "out of host memory while building the plan");
+  } catch (const std::exception& e) {
+    if (plan_out) *plan_out = nullptr;
+    rc = fail(HPSPMM_ERR_ALLOC, "plan construction failed: %s", e.what());
+  }
+  try {
+    g_rank_cache = RankCache{};  // a later plan may get the same address
+  } catch (...) {
+  }
+  return rc;
+}
+
 int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr, const int32_t* d_col,
                        int64_t k, uint32_t flags, void* stream, hpspmm_plan** plan_out) {
-  const int rc = plan_create_impl(rows, cols, nnz, d_rowptr, d_col, k, flags, nullptr, stream, plan_out);
-  g_rank_cache = RankCache{};  // a later plan may get the same address
-  return rc;
+  return plan_create_guarded(rows, cols, nnz, d_rowptr, d_col, k, flags, nullptr, stream, plan_out);
 }
 
 int hpspmm_plan_create_ordered(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr,
                                const int32_t* d_col, int64_t k, uint32_t flags, const int32_t* d_row_order,
                                void* stream, hpspmm_plan** plan_out) {
   if (rows > 0 && !d_row_order) return fail(HPSPMM_ERR_INVALID_ARG, "d_row_order is NULL");
-  const int rc = plan_create_impl(rows, cols, nnz, d_rowptr, d_col, k, flags, d_row_order, stream, plan_out);
-  g_rank_cache = RankCache{};
-  return rc;
+  return plan_create_guarded(rows, cols, nnz, d_rowptr, d_col, k, flags, d_row_order, stream, plan_out);
 }
 
 int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
@@ -1341,6 +1448,13 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
   if (!d_rowptr || !d_C) return fail(HPSPMM_ERR_INVALID_ARG, "d_rowptr or d_C is NULL");
   if (plan->nnz > 0 && (!d_col || !d_val || !d_B))
     return fail(HPSPMM_ERR_INVALID_ARG, "d_col, d_val or d_B is NULL with nnz > 0");
+  // The plan holds the structure of the arrays it was built from (some strategies run entirely
+  // from its own copy): other addresses most likely mean another matrix, whose product would
+  // silently be that of the old one.
+  if (!plan->allow_moved && (d_rowptr != plan->src_rowptr || (plan->nnz > 0 && d_col != plan->src_col)))
+    return fail(HPSPMM_ERR_INVALID_ARG,
+                "d_rowptr / d_col are not the arrays this plan was built from (build a new plan for another "
+                "structure, or create the plan with HPSPMM_PLAN_ALLOW_MOVED_CSR if the same structure has moved)");
   hipStream_t st = (hipStream_t)stream;
   int rc;
   // another value array overwrites the plan's copy of the bound one
@@ -1447,6 +1561,58 @@ int hpspmm_csr_spmm_timed(hpspmm_plan* plan, const int32_t* d_rowptr, const int3
   if (rc) return rc;
   if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "timing failed: %s", hipGetErrorString(e));
   *mean_ms_out = ms / (float)iters;
+  return HPSPMM_OK;
+}
+
+int hpspmm_csr_spmm_timed_launches(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d_col,
+                                   const float* d_val, const float* d_B, float* d_C, void* stream, int warmup,
+                                   int iters, int max_launches, float* mean_ms_out, const char** names_out,
+                                   int* n_launches_out) {
+  if (!mean_ms_out || !names_out || !n_launches_out || iters <= 0 || warmup < 0 || max_launches <= 0)
+    return fail(HPSPMM_ERR_INVALID_ARG, "bad timing arguments");
+  *n_launches_out = 0;
+  hipStream_t st = (hipStream_t)stream;
+  for (int i = 0; i < warmup; ++i)
+    if (int rc = hpspmm_csr_spmm(plan, d_rowptr, d_col, d_val, d_B, d_C, stream)) return rc;
+  LaunchTrace trace;
+  hipEvent_t begin;
+  HPSPMM_HIP(hipEventCreate(&begin));
+  int created = 0;
+  hipError_t e = hipSuccess;
+  for (; created < kMaxTracedLaunches && e == hipSuccess; ++created) e = hipEventCreate(&trace.ev[created]);
+  if (e != hipSuccess) {
+    for (int q = 0; q < created - 1; ++q) (void)hipEventDestroy(trace.ev[q]);
+    (void)hipEventDestroy(begin);
+    return fail(HPSPMM_ERR_HIP, "hipEventCreate: %s", hipGetErrorString(e));
+  }
+  double sum[kMaxTracedLaunches] = {0};
+  int rc = HPSPMM_OK, n = 0;
+  for (int i = 0; i < iters && rc == HPSPMM_OK && e == hipSuccess; ++i) {
+    trace.n = 0;
+    e = hipEventRecord(begin, st);
+    g_trace = &trace;
+    rc = hpspmm_csr_spmm(plan, d_rowptr, d_col, d_val, d_B, d_C, stream);
+    g_trace = nullptr;
+    if (rc != HPSPMM_OK || e != hipSuccess) break;
+    n = trace.n;
+    if (n == 0) break;
+    e = hipEventSynchronize(trace.ev[n - 1]);
+    for (int q = 0; q < n && e == hipSuccess; ++q) {
+      float ms = 0.f;
+      e = hipEventElapsedTime(&ms, q == 0 ? begin : trace.ev[q - 1], trace.ev[q]);
+      sum[q] += ms;
+    }
+  }
+  (void)hipEventDestroy(begin);
+  for (int q = 0; q < created; ++q) (void)hipEventDestroy(trace.ev[q]);
+  if (rc) return rc;
+  if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "timing failed: %s", hipGetErrorString(e));
+  const int out = n < max_launches ? n : max_launches;
+  for (int q = 0; q < out; ++q) {
+    mean_ms_out[q] = (float)(sum[q] / iters);
+    names_out[q] = trace.name[q];
+  }
+  *n_launches_out = out;
   return HPSPMM_OK;
 }
 

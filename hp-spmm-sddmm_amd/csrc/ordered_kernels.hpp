@@ -41,30 +41,38 @@ namespace hpspmm {
 // indices are its column indices; the matrix is taken as a graph, which is
 // meant for square, structurally symmetric A.  Ties are broken by a hash that
 // changes with the sweep, except that a row keeps its label when that is among
-// the most frequent.  Labels are updated in place (asynchronous propagation,
-// which does not oscillate the way the synchronous form does).  One wavefront
-// per row; the 64 sampled labels are sorted by a bitonic network of
-// wavefront shuffles.  The kClusterCounters entries of changed[] together
-// count the rows whose label changed.
+// the most frequent.  A sweep reads label_in and writes label_out (two buffers,
+// so the outcome does not depend on the order in which the wavefronts run: two
+// plans of one matrix get the same labels), and only a pseudo-random half of the
+// rows - another half in every sweep - may change: with every row updated at
+// once from the old labels, neighbours swap labels back and forth instead of
+// settling.  One wavefront per row; the 64 sampled labels are sorted by a bitonic
+// network of wavefront shuffles.  The kClusterCounters entries of changed[]
+// together count the rows whose label changed.
 constexpr int kClusterCounters = 1024;
 __global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                const int32_t* __restrict__ col,
-                                                               int32_t* __restrict__ label, uint32_t sweep,
+                                                               const int32_t* __restrict__ label_in,
+                                                               int32_t* __restrict__ label_out, uint32_t sweep,
                                                                uint32_t* __restrict__ changed) {
   const int lane = threadIdx.x & 63;
   const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   if (r >= rows) return;
+  const int32_t mine = label_in[r];
   const int32_t lb = rowptr[r];
   const int32_t n = rowptr[r + 1] - lb;
-  if (n == 0) return;
+  const uint32_t turn = (((uint32_t)r * 0x9E3779B1u) ^ ((sweep + 1u) * 0x85EBCA6Bu)) * 0xC2B2AE35u;
+  if (n == 0 || ((turn >> 31) & 1u)) {  // wavefront-uniform
+    if (lane == 0) label_out[r] = mine;
+    return;
+  }
   const int32_t stride = (n + 63) / 64;
   const bool valid = lane * stride < n;
   int32_t lab = INT32_MAX;  // sorts behind every label
   if (valid) {
     const int32_t c = col[lb + lane * stride];
-    if ((int64_t)c < rows) lab = label[c];
+    if ((int64_t)c < rows) lab = label_in[c];
   }
-  const int32_t mine = label[r];
   const int self_count = (int)__popcll(__ballot(lab == mine));
 #pragma unroll
   for (int size = 2; size <= 64; size <<= 1) {
@@ -83,29 +91,33 @@ __global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, con
   const bool head = real && (lane == 0 || lab != prev);
   const uint64_t heads = __ballot(head);
   const int n_real = (int)__popcll(__ballot(real));
-  if (n_real == 0) return;
-  unsigned long long key = 0;
-  if (head) {
-    const uint64_t later = lane < 63 ? (heads >> (lane + 1)) : 0ull;
-    const int next = later ? lane + 1 + (int)__ffsll((long long)later) - 1 : n_real;
-    const uint32_t h = ((uint32_t)lab * 0x9E3779B1u) ^ (sweep * 0x85EBCA6Bu) ^ ((uint32_t)r * 0xC2B2AE35u);
-    key = ((unsigned long long)(uint32_t)(next - lane) << 32) | (h >> 1);
-  }
-  unsigned long long best = key;
-  int32_t best_lab = lab;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    const unsigned long long o = __shfl_xor(best, off);
-    const int32_t ol = __shfl_xor(best_lab, off);
-    if (o > best) {
-      best = o;
-      best_lab = ol;
+  int32_t next_label = mine;
+  if (n_real != 0) {
+    unsigned long long key = 0;
+    if (head) {
+      const uint64_t later = lane < 63 ? (heads >> (lane + 1)) : 0ull;
+      const int next = later ? lane + 1 + (int)__ffsll((long long)later) - 1 : n_real;
+      const uint32_t h = ((uint32_t)lab * 0x9E3779B1u) ^ (sweep * 0x85EBCA6Bu) ^ ((uint32_t)r * 0xC2B2AE35u);
+      key = ((unsigned long long)(uint32_t)(next - lane) << 32) | (h >> 1);
     }
+    unsigned long long best = key;
+    int32_t best_lab = lab;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const unsigned long long o = __shfl_xor(best, off);
+      const int32_t ol = __shfl_xor(best_lab, off);
+      if (o > best || (o == best && ol < best_lab)) {
+        best = o;
+        best_lab = ol;
+      }
+    }
+    const int best_count = (int)(best >> 32);
+    if (self_count < best_count && best_lab != mine) next_label = best_lab;
   }
-  const int best_count = (int)(best >> 32);
-  if (lane == 0 && self_count < best_count && best_lab != mine) {
-    label[r] = best_lab;
-    atomicAdd(&changed[r & (kClusterCounters - 1)], 1u);  // spread: one counter would serialise the first sweep
+  if (lane == 0) {
+    label_out[r] = next_label;
+    if (next_label != mine)
+      atomicAdd(&changed[r & (kClusterCounters - 1)], 1u);  // spread: one counter would serialise the first sweep
   }
 }
 

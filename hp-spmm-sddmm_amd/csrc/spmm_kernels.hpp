@@ -675,6 +675,13 @@ __global__ __launch_bounds__(kBlock) void expand_rows_kernel(int64_t rows, int64
   nnz_row[j] = (int32_t)lo;
 }
 
+// out[b] = id of the XCD that workgroup b runs on (hardware register XCC_ID, bits 3:0): lets the
+// plan verify the dealing of workgroups to XCDs that the routed strategy and xcd_remap assume.
+__global__ __launch_bounds__(64) void xcc_probe_kernel(int32_t* __restrict__ out) {
+  const unsigned v = __builtin_amdgcn_s_getreg(((4 - 1) << 11) | (0 << 6) | 20);
+  if (threadIdx.x == 0) out[blockIdx.x] = (int32_t)(v & 0xFu);
+}
+
 __global__ __launch_bounds__(kBlock) void fill_f32_kernel(float* __restrict__ x, int64_t n, float v) {
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) x[i] = v;

@@ -11,6 +11,7 @@
 #include <string>
 #include <vector>
 
+#include "spmm/compare.h"
 #include "spmm/spmm_common.h"
 
 using namespace starml;
@@ -178,6 +179,23 @@ int main(int argc, char** argv) {
   }
   CHECK(eq && in_range);
   CHECK(throws([&] { Matrix bad({-1}, Device(kCPU), kFloat); }));
+
+  // result check: a NaN anywhere (not only in the last position) fails it, on either side
+  {
+    Matrix x = full({8}, Device(kCPU), kFloat, 1.0), y = full({8}, Device(kCPU), kFloat, 1.0);
+    int64_t at = -1;
+    CHECK(MaxAbsError(x, y, "", &at) == 0.f && at == -1);
+    y.mutable_data<float>()[6] = 1.05f;
+    CHECK(std::fabs(MaxAbsError(x, y, "", &at) - 0.05f) < 1e-6f && at == 6);
+    x.mutable_data<float>()[3] = NAN;  // followed by finite, smaller errors
+    CHECK(std::isinf(MaxAbsError(x, y, "", &at)) && at == 3);
+    CHECK(throws([&] { ExpectEqualDenseWithError(x, y); }));
+    x.mutable_data<float>()[3] = 1.0f;
+    y.mutable_data<float>()[0] = NAN;
+    CHECK(std::isinf(MaxAbsError(x, y, "", &at)) && at == 0);
+    Matrix z = full({8}, Device(kCPU), kFloat, 200.0), w = full({8}, Device(kCPU), kFloat, 1.0);
+    CHECK(MaxAbsError(z, w, "div", &at) == 0.f);  // "div": x / 200 launches against y
+  }
 
   if (g_failed) {
     std::cerr << g_failed << " check(s) failed\n";

@@ -20,7 +20,12 @@ float MaxAbsError(const Matrix& mat1, const Matrix& mat2, const std::string& kty
   int64_t pos = -1;
   for (int64_t i = 0; i < a.size(); ++i) {
     const float e = std::fabs((div == 1.0f ? x[i] : x[i] / div) - y[i]);
-    if (!(e <= worst)) {  // also catches NaN
+    if (e != e) {  // a NaN on either side is the worst possible error and ends the search
+      worst = INFINITY;
+      pos = i;
+      break;
+    }
+    if (e > worst) {
       worst = e;
       pos = i;
     }

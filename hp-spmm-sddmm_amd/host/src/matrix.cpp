@@ -6,6 +6,8 @@
 #include <cstdlib>
 #include <cstring>
 
+#include "hpspmm.h"
+
 extern "C" {
 void hpspmm_gen_dense_normal(uint64_t seed, int64_t count, float* out);
 void hpspmm_gen_dense_uniform(uint64_t seed, int64_t count, float lo, float hi, float* out);
@@ -80,7 +82,16 @@ Matrix empty(const Shape& shape, const Device& device, const DataType& data_type
 }
 
 Matrix full(const Shape& shape, const Device& device, const DataType& data_type, double init_val) {
-  // filled on the host, then moved: device fills of C go through fill_matrix
+  // FP32 on the device: allocated there and filled by a kernel, as the reference does
+  // (spmm/starml/operators/cuda/factories_kernel.cu:8-17) - nothing crosses PCIe
+  if (device.is_hip() && data_type.type() == kFloat) {
+    Matrix out(shape, device, data_type);
+    if (hpspmm_fill_f32(out.mutable_data<float>(), out.size(), (float)init_val, nullptr) != HPSPMM_OK)
+      throw Error(std::string("full: ") + hpspmm_last_error());
+    hip_check(hipStreamSynchronize(nullptr), "full");
+    return out;
+  }
+  // other types (index arrays, host matrices): filled on the host, then moved
   Matrix host(shape, Device(kCPU), data_type);
   const int64_t n = host.size();
   switch (data_type.type()) {

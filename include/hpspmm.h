@@ -58,23 +58,25 @@ typedef enum hpspmm_status {
                                          copy (default: only when they serve >= 25 % of the nonzeros) */
 #define HPSPMM_PLAN_NO_HUB_CACHE 32u  /* never build the hub cache */
 #define HPSPMM_PLAN_FORCE_ROUTED 64u  /* always use the routed strategy (hub columns pinned to one XCD each);
-                                         bits 16..23 then give log2 of the total number of hub rows (0 = auto) */
+                                         bits 16..20 then give log2 of the total number of hub rows (0 = auto) */
 #define HPSPMM_PLAN_NO_ROUTED 128u    /* never use the routed strategy */
 /* bits 24..28, with FORCE_ROUTED: log2 of the shortest row that is routed (0 = default, 128) */
 #define HPSPMM_PLAN_ROUTED_ROW_LOG2(log2_nnz) (((uint32_t)(log2_nnz) & 0x1Fu) << 24)
 /* bits 29..31, with FORCE_ROUTED: number of phases every XCD cuts its slice of the columns into, 1..7 (0 = auto) */
 #define HPSPMM_PLAN_ROUTED_PHASES(n) (((uint32_t)(n) & 0x7u) << 29)
-/* bits 16..23: log2 of the number of cached rows (0 = default, 2^16) */
-#define HPSPMM_PLAN_HUB_LOG2(log2_rows) (((uint32_t)(log2_rows) & 0xFFu) << 16)
+/* bits 16..20: log2 of the number of cached rows, 4..24 (0 = default, 2^16) */
+#define HPSPMM_PLAN_HUB_LOG2(log2_rows) (((uint32_t)(log2_rows) & 0x1Fu) << 16)
+#define HPSPMM_PLAN_ALLOW_MOVED_CSR (1u << 21) /* hpspmm_csr_spmm accepts d_rowptr / d_col at other addresses than
+                                         the plan was built from (the caller vouches that they hold the same
+                                         structure); default: other addresses are HPSPMM_ERR_INVALID_ARG */
 /* bits 8..11: log2 of the segment length to force (0 = choose automatically) */
 #define HPSPMM_PLAN_SEGMENT_SHIFT(log2_len) (((uint32_t)(log2_len) & 0xFu) << 8)
 #define HPSPMM_PLAN_CLUSTER 4096u     /* square A: always look for clusters of rows that share columns and use the
                                          ordered strategy on the order found (default: from 2^22 nonzeros and
                                          24 MB of B up, when the graph is not routed, and only if >= 15 % of the
                                          nonzeros stay inside clusters of <= 4096 rows and >= 15 % then read B
-                                         from LDS).  The clustering updates its labels asynchronously: two
-                                         plans of one matrix may order the rows differently and then differ
-                                         in the last bits of C; one plan always gives the same bits */
+                                         from LDS).  The clustering is deterministic: two plans of one matrix
+                                         order the rows alike and give the same bits of C */
 #define HPSPMM_PLAN_NO_CLUSTER 8192u  /* never */
 #define HPSPMM_PLAN_ROUTED_SORT_VALUES 32768u /* routed strategy: never cut the columns into consecutive ranges (which lets
                                          the kernel read the values in place); always spread them by popularity rank and
@@ -128,7 +130,15 @@ const char *hpspmm_last_error(void);
  * (:237-296) and the choice of nnz_per_warp (spmm/mm/spmm_kernel.cu:749-751).
  * Synchronises `stream`.
  * Values are not read: the plan stays valid when d_val or B change, and must
- * be rebuilt when rowptr / col change.
+ * be rebuilt when rowptr / col change - also when they are edited in place:
+ * most strategies run from the plan's own copy of the structure and would go
+ * on computing the old matrix.
+ * The strategies that place work on particular XCDs (routed; the row-range
+ * dealing of the others) are used only if a probe launch, once per device and
+ * process, has seen workgroup b run on XCD b % 8, which is how the whole
+ * (unpartitioned) device deals them; otherwise the plan keeps to segments,
+ * rows and ordered without that placement.  The environment variable
+ * HPSPMM_XCD_DEALING=0 / 1 overrides the probe (diagnostics).
  */
 int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
                        const int32_t *d_col, int64_t k, uint32_t flags, void *stream,
@@ -181,6 +191,10 @@ int hpspmm_plan_bind_values(hpspmm_plan *plan, const float *d_val, void *stream)
  * The result is deterministic (no atomics).  The call only launches kernels (no
  * allocation, no memset, no host synchronisation), so it may be captured in a
  * HIP graph; a replay reads d_val and d_B as they are then.
+ * d_rowptr and d_col must be the arrays the plan was built from: any other
+ * address is HPSPMM_ERR_INVALID_ARG (the reference's launchers take whatever
+ * they are given, spmm/mm/spmm_kernel.cu:389-426, and have no plan that could
+ * go stale), unless the plan was created with HPSPMM_PLAN_ALLOW_MOVED_CSR.
  */
 int hpspmm_csr_spmm(hpspmm_plan *plan, const int32_t *d_rowptr, const int32_t *d_col,
                     const float *d_val, const float *d_B, float *d_C, void *stream);
@@ -220,6 +234,20 @@ int hpspmm_fill_f32(float *d_x, int64_t n, float value, void *stream);
 int hpspmm_csr_spmm_timed(hpspmm_plan *plan, const int32_t *d_rowptr, const int32_t *d_col,
                           const float *d_val, const float *d_B, float *d_C, void *stream,
                           int warmup, int iters, float *mean_ms_out);
+
+/*
+ * The same protocol with one more event after every kernel launch of an SpMM:
+ * mean_ms_out[i] = mean duration of the i-th launch (i < *n_launches_out <=
+ * max_launches, at most 8), names_out[i] = its kernel's name (a string owned by
+ * the library).  For reporting which launch of a multi-launch strategy takes the
+ * time; the extra events keep launches from overlapping their neighbours'
+ * start-up, so the sum is slightly above hpspmm_csr_spmm_timed's mean.  The
+ * reference has no counterpart (its launchers are single kernels).
+ */
+int hpspmm_csr_spmm_timed_launches(hpspmm_plan *plan, const int32_t *d_rowptr, const int32_t *d_col,
+                                   const float *d_val, const float *d_B, float *d_C, void *stream,
+                                   int warmup, int iters, int max_launches, float *mean_ms_out,
+                                   const char **names_out, int *n_launches_out);
 
 #ifdef __cplusplus
 }

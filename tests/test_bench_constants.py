@@ -1,0 +1,65 @@
+"""bench.py carries measured L2<->fabric traffic per kernel as constants (hardware counters cannot
+be read from inside the benchmark process).  They must be the figures of the rocprofv3 summaries
+committed under profiles/: this test parses those files and fails on any drift."""
+import importlib.util
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _bench():
+    spec = importlib.util.spec_from_file_location("bench_module", os.path.join(ROOT, "bench.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def _traffic_table(path):
+    """{kernel name as printed: total_GB} from the counter table of a profile summary, and
+    {kernel name: avg_us} from its kernel_stats table."""
+    traffic, avg_us = {}, {}
+    for line in open(path):
+        m = re.match(r"^(hpspmm::\S.*?)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s*$", line)
+        if not m:
+            continue
+        # kernel_stats rows: calls avg min max pct (calls is an integer); counter rows: five decimals
+        cols = line.split()
+        if re.fullmatch(r"\d+", cols[-5]):
+            avg_us[m.group(1)] = float(cols[-4])
+        else:
+            traffic[m.group(1)] = float(cols[-1])
+    return traffic, avg_us
+
+
+def test_traffic_constants_match_the_profiles():
+    bench = _bench()
+    assert bench.MEASURED_TRAFFIC, "no measured traffic carried"
+    wanted = {("c2_social", 32), ("c2_social", 64), ("c2_social", 128), ("c3_copurchase", 64), ("c4_rmat", 128)}
+    assert set(bench.MEASURED_TRAFFIC) == wanted
+    for (workload, k), rec in bench.MEASURED_TRAFFIC.items():
+        path = os.path.join(ROOT, rec["profile"])
+        assert os.path.exists(path), f"{rec['profile']} is missing"
+        traffic, avg_us = _traffic_table(path)
+        assert traffic, f"no counter table found in {rec['profile']}"
+        assert len(rec["kernels"]) == rec["launches"]
+        for kernel, gb in rec["kernels"].items():
+            rows = [n for n in traffic if re.match(rf"hpspmm::{kernel}<{k}[,>]", n)]
+            assert len(rows) == 1, f"{workload} K={k}: {kernel} has {len(rows)} rows in {rec['profile']}"
+            assert abs(traffic[rows[0]] - gb) <= 5e-4, \
+                f"{workload} K={k} {kernel}: bench.py carries {gb} GB, {rec['profile']} says {traffic[rows[0]]} GB"
+            assert any(re.match(rf"hpspmm::{kernel}<{k}[,>]", n) for n in avg_us), \
+                f"{workload} K={k}: no duration for {kernel} in {rec['profile']}"
+
+
+def test_bounded_fractions_are_bounded():
+    """traffic_frac as bench.py defines it, recomputed from the profiles alone (traffic of all launches
+    of one SpMM / the sum of their mean durations / 8 TB/s), is a fraction: <= 1 for every workload."""
+    bench = _bench()
+    for (workload, k), rec in bench.MEASURED_TRAFFIC.items():
+        traffic, avg_us = _traffic_table(os.path.join(ROOT, rec["profile"]))
+        total_gb = sum(rec["kernels"].values())
+        total_us = sum(next(v for n, v in avg_us.items() if re.match(rf"hpspmm::{kernel}<{k}[,>]", n))
+                       for kernel in rec["kernels"])
+        frac = total_gb * 1e9 / (total_us * 1e-6) / (bench.HBM_PEAK_GBS * 1e9)
+        assert 0.05 < frac <= 1.0, (workload, k, frac)

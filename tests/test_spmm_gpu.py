@@ -306,6 +306,78 @@ def test_error_codes(pkg, gpu):
     plan.destroy()
 
 
+def test_other_csr_arrays_are_refused(pkg, oracle, gpu):
+    """A plan holds the structure it was built from; rowptr / col at other addresses are most likely
+    another matrix and are refused, whatever strategy the plan chose - unless the plan was created
+    with HPSPMM_PLAN_ALLOW_MOVED_CSR, in which case copies of the same structure give the same product."""
+    import torch
+    capi = pkg.capi
+    g = pkg.graphs.make_graph("c4_rmat", 0.004)
+    k = 64
+    B = pkg.graphs.make_dense("c4_rmat", g.cols, k)
+    rp, ci, v, Bd = _to_dev(gpu, g.rowptr, g.col, g.val, B)
+    rp2, ci2 = rp.clone(), ci.clone()
+    for name, flags in _strategies(capi):
+        plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
+        C = torch.full((g.rows, k), float("nan"), device=gpu)
+        for bad_rp, bad_ci in ((rp2, ci), (rp, ci2), (rp2, ci2)):
+            with pytest.raises(capi.HpSpmmError) as ei:
+                capi.csr_spmm(plan, bad_rp, bad_ci, v, Bd, C)
+            assert ei.value.code == capi.ERR_INVALID_ARG, name
+            assert "not the arrays this plan was built from" in str(ei.value)
+        torch.cuda.synchronize()
+        assert torch.isnan(C).all().item(), f"{name}: a refused call must not launch anything"
+        capi.csr_spmm(plan, rp, ci, v, Bd, C)  # the plan itself is still good
+        _check(oracle, g, B, C.cpu().numpy(), f"after refusals, {name}")
+        plan.destroy()
+        plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags | capi.PLAN_ALLOW_MOVED_CSR)
+        C.fill_(float("nan"))
+        capi.csr_spmm(plan, rp2, ci2, v, Bd, C)
+        _check(oracle, g, B, C.cpu().numpy(), f"moved arrays allowed, {name}")
+        plan.destroy()
+
+
+def test_two_plans_of_one_matrix_give_the_same_bits(pkg, oracle, gpu):
+    """Plan construction is deterministic, the clustering included: a second plan of the same matrix
+    orders the rows alike, so C agrees bit for bit between plans, not only between calls."""
+    capi = pkg.capi
+    for name, scale, k, flags in (("c3_copurchase", 0.05, 64, capi.PLAN_DEFAULT),
+                                  ("c3_copurchase", 0.02, 32, capi.PLAN_CLUSTER | capi.PLAN_FORCE_SEGMENTS),
+                                  ("c4_rmat", 0.008, 128, capi.PLAN_CLUSTER),
+                                  ("c2_social", 0.1, 128, capi.PLAN_DEFAULT)):
+        g = pkg.graphs.make_graph(name, scale)
+        B = pkg.graphs.make_dense(name, g.cols, k)
+        C1, i1 = _run(pkg, gpu, g, B, flags)
+        C2, i2 = _run(pkg, gpu, g, B, flags)
+        assert i1 == i2, (name, i1, i2)
+        assert np.array_equal(C1, C2), f"{name}: two plans, different bits"
+        if name == "c3_copurchase":
+            assert i1["strategy"] == capi.STRATEGY_ORDERED and i1["lds_served_nnz"] >= 0.3 * g.nnz, i1
+
+
+def test_xcd_placement_is_verified_at_plan_time(pkg, oracle, gpu):
+    """The routed strategy relies on workgroup b running on XCD b % 8.  The plan measures that once
+    per device; on the whole MI355X it holds and the social graph gets the routed strategy.  With the
+    probe overridden to 'does not hold' the plan keeps to a strategy without XCD placement and the
+    product is the same to rounding."""
+    import os
+    capi = pkg.capi
+    g = pkg.graphs.make_graph("c2_social", 0.1)
+    k = 128
+    B = pkg.graphs.make_dense("c2_social", g.cols, k)
+    assert "HPSPMM_XCD_DEALING" not in os.environ
+    C, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+    assert info["strategy"] == capi.STRATEGY_ROUTED, info
+    _check(oracle, g, B, C, "probe result")
+    os.environ["HPSPMM_XCD_DEALING"] = "0"
+    try:
+        C0, info0 = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+    finally:
+        del os.environ["HPSPMM_XCD_DEALING"]
+    assert info0["strategy"] in (capi.STRATEGY_SEGMENTS, capi.STRATEGY_ROWS), info0
+    _check(oracle, g, B, C0, "placement not available")
+
+
 def _sample_check(oracle, g, B, C_dev, ranges, what):
     """Oracle check on contiguous row ranges of a large result held on the GPU."""
     for lo, hi in ranges:
@@ -321,7 +393,7 @@ def _sample_check(oracle, g, B, C_dev, ranges, what):
                                     ("c2_social", 32)])
 def test_full_size_configs(pkg, oracle, gpu, name, k):
     """The benchmark configurations at full size, default plan (the strategy the benchmark times):
-    oracle on row samples, agreement between strategies, NaN-poisoned C fully overwritten."""
+    the oracle on every row, agreement between strategies, NaN-poisoned C fully overwritten."""
     import torch
     capi = pkg.capi
     g = pkg.graphs.make_graph(name)
@@ -351,11 +423,9 @@ def test_full_size_configs(pkg, oracle, gpu, name, k):
     diff = (out["auto"][0] - out["plain"][0]).abs()
     assert torch.all(diff <= TOL * S).item(), f"{name} K={k}: strategies disagree by {float((diff / S.clamp_min(1e-30)).max()):.3e}"
     del S, diff
-    # oracle on three row ranges, including the heaviest rows
-    deg = np.diff(g.rowptr)
-    top = int(np.argmax(deg))
-    lo = max(0, min(top - 50, g.rows - 200))
-    ranges = [(0, 300), (lo, lo + 200), (g.rows - 300, g.rows)]
+    # oracle over ALL rows, in slabs (the float64 result and its denominator of a slab at a time)
+    slab = max(1, (1 << 25) // k)
+    ranges = [(lo, min(lo + slab, g.rows)) for lo in range(0, g.rows, slab)]
     _sample_check(oracle, g, B, out["auto"][0], ranges, f"{name} K={k}")
 
 

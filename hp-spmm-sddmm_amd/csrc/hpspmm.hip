@@ -15,6 +15,7 @@
 #include <string>
 #include <vector>
 
+#include "anyk_kernels.hpp"
 #include "ordered_kernels.hpp"
 #include "routed_kernels.hpp"
 #include "rowtile_kernels.hpp"
@@ -61,6 +62,16 @@ inline void mark_launch(hipStream_t st, const char* name) {
 }
 
 inline bool fast_k(int64_t k) { return k == 32 || k == 64 || k == 128; }
+// Row lengths served by the run-time-K sub-wave kernels: multiples of 4 that are not a tuned size.
+inline bool anyk_k(int64_t k) { return !fast_k(k) && k % 4 == 0 && k <= (1 << 20); }
+// Lanes per sub-wave for such a K: the power of two that covers a column tile (at most 128 floats).
+inline int anyk_lanes(int64_t k) {
+  const int64_t g = (k < hpspmm::kAnyKTile ? k : hpspmm::kAnyKTile) / 4;
+  int gp = 2;
+  while (gp < g) gp <<= 1;
+  return gp;
+}
+inline int anyk_tiles(int64_t k) { return (int)((k + hpspmm::kAnyKTile - 1) / hpspmm::kAnyKTile); }
 
 inline bool aligned16(const void* a, const void* b, const void* c) {
   return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15u) == 0;
@@ -385,6 +396,60 @@ int launch_row_tiles(const hpspmm_plan* p, const float* v, const float* B, float
   return launch_row_tiles_w<K, hpspmm::kWavesPerBlock>(p, v, B, C, st);
 }
 
+template <int GP>
+int launch_rows_anyk_g(int64_t rows, int64_t k, const int32_t* rp, const int32_t* ci, const float* v, const float* B,
+                       float* C, int32_t long_threshold, const int32_t* long_rows, int64_t n_long, hipStream_t st) {
+  const int tiles = anyk_tiles(k);
+  const int64_t short_blocks = ceil_div(ceil_div(rows, 64 / GP), hpspmm::kWavesPerBlock);
+  const int64_t blocks = (short_blocks + ceil_div(n_long, hpspmm::kWavesPerBlock)) * tiles;
+  if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  hipLaunchKernelGGL(hpspmm::spmm_rows_anyk_kernel<GP>, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rows,
+                     (int)k, tiles, rp, ci, v, B, C, short_blocks, long_threshold, long_rows, n_long);
+  mark_launch(st, "spmm_rows_anyk_kernel");
+  return HPSPMM_OK;
+}
+
+int launch_rows_anyk(int64_t rows, int64_t k, const int32_t* rp, const int32_t* ci, const float* v, const float* B,
+                     float* C, int32_t long_threshold, const int32_t* long_rows, int64_t n_long, hipStream_t st) {
+  switch (anyk_lanes(k)) {
+    case 2: return launch_rows_anyk_g<2>(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+    case 4: return launch_rows_anyk_g<4>(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+    case 8: return launch_rows_anyk_g<8>(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+    case 16: return launch_rows_anyk_g<16>(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+    default: return launch_rows_anyk_g<32>(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+  }
+}
+
+template <int GP>
+int launch_segments_anyk_g(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, const float* v, const float* B,
+                           float* C, hipStream_t st) {
+  const int tiles = anyk_tiles(p->k);
+  const int64_t blocks = ceil_div(ceil_div(p->nseg, 64 / GP), hpspmm::kWavesPerBlock) * tiles;
+  if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  if (p->nnz > 0) {
+    hipLaunchKernelGGL(hpspmm::spmm_segments_anyk_kernel<GP>, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rp,
+                       ci, v, p->d_nnz_row, B, C, p->d_carry, p->nnz, p->shift, p->nseg, (int)p->k, tiles,
+                       aligned16(ci, v, p->d_nnz_row));
+    mark_launch(st, "spmm_segments_anyk_kernel");
+  }
+  const int64_t fix_blocks = ceil_div(ceil_div(p->rows, 64), hpspmm::kWavesPerBlock);
+  hipLaunchKernelGGL(hpspmm::spmm_fixup_anyk_kernel<GP>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st,
+                     p->rows, rp, (const float*)p->d_carry, C, p->shift, (int)p->k);
+  mark_launch(st, "spmm_fixup_anyk_kernel");
+  return HPSPMM_OK;
+}
+
+int launch_segments_anyk(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, const float* v, const float* B,
+                         float* C, hipStream_t st) {
+  switch (anyk_lanes(p->k)) {
+    case 2: return launch_segments_anyk_g<2>(p, rp, ci, v, B, C, st);
+    case 4: return launch_segments_anyk_g<4>(p, rp, ci, v, B, C, st);
+    case 8: return launch_segments_anyk_g<8>(p, rp, ci, v, B, C, st);
+    case 16: return launch_segments_anyk_g<16>(p, rp, ci, v, B, C, st);
+    default: return launch_segments_anyk_g<32>(p, rp, ci, v, B, C, st);
+  }
+}
+
 int launch_rows_any(int64_t rows, int64_t cols, int64_t k, const int32_t* rp, const int32_t* ci, const float* v,
                     const float* B, float* C, int32_t long_threshold, const int32_t* long_rows, int64_t n_long,
                     hipStream_t st) {
@@ -394,6 +459,7 @@ int launch_rows_any(int64_t rows, int64_t cols, int64_t k, const int32_t* rp, co
     case 64: return launch_rows<64>(rows, cols, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
     case 128: return launch_rows<128>(rows, cols, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
     default: {
+      if (anyk_k(k)) return launch_rows_anyk(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
       const int64_t blocks = ceil_div(rows, hpspmm::kWavesPerBlock);
       hipLaunchKernelGGL(hpspmm::spmm_rows_generic_kernel, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st,
                          rows, k, rp, ci, v, B, C);
@@ -486,7 +552,7 @@ int launch_coo(int64_t nnz, const int32_t* ri, const int32_t* ci, const float* v
 // segment, against S*(K+2) floats of gather) is small, short enough that there
 // are several waves of work per SIMD.
 int choose_shift(int64_t nnz, int64_t k, int64_t max_row_nnz) {
-  const int64_t subwaves = 64 / (k / 4);
+  const int64_t subwaves = fast_k(k) ? 64 / (k / 4) : 64 / anyk_lanes(k);
   const int64_t target_waves = 256 /*CUs*/ * 4 /*SIMDs*/ * 16;
   int shift = 5;
   while (shift < 9 && (nnz >> (shift + 1)) / subwaves >= target_waves) ++shift;
@@ -1186,8 +1252,16 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   // few columns take most of the nonzeros, else ordered if it has communities, else segments.
   bool rows_need_tiles = false;  // rows strategy chosen on the strength of the row tiles
   bool rows_range = false;       // provisional segments; rows unless the ordered strategy qualifies
-  if (!fast_k(k)) {
+  if (!fast_k(k) && !anyk_k(k)) {
     p->strategy = HPSPMM_STRATEGY_GENERIC_K;
+  } else if (!fast_k(k)) {
+    // a multiple of 4 that is not a tuned size: whole rows for small matrices (one launch), segments
+    // beyond (balanced over any degree distribution); the layouts built for the tuned sizes (row
+    // tiles, routed, ordered, hub cache) are not used
+    const bool small = nnz < (1 << 21) && p->max_row_nnz <= 4096;
+    p->strategy = (flags & HPSPMM_PLAN_FORCE_SEGMENTS)                   ? HPSPMM_STRATEGY_SEGMENTS
+                  : ((flags & HPSPMM_PLAN_FORCE_ROWS) || nnz == 0 || small) ? HPSPMM_STRATEGY_ROWS
+                                                                           : HPSPMM_STRATEGY_SEGMENTS;
   } else if (d_order && nnz > 0) {
     if (int rc = build_ordered(p, d_rowptr, d_col, d_order, 0.0, st)) {
       return rc;
@@ -1222,7 +1296,8 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     }
   }
 
-  if (p->strategy == HPSPMM_STRATEGY_ROWS && rows > 0 && nnz < kRowTileMaxNnz && !(flags & HPSPMM_PLAN_NO_ROW_TILES)) {
+  if (p->strategy == HPSPMM_STRATEGY_ROWS && fast_k(k) && rows > 0 && nnz < kRowTileMaxNnz &&
+      !(flags & HPSPMM_PLAN_NO_ROW_TILES)) {
     if (int rc = build_row_tiles(p, d_rowptr, d_col, st)) {
       return rc;
     }
@@ -1252,7 +1327,8 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       }
     }
   }
-  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && !(flags & HPSPMM_PLAN_NO_ROUTED) && nnz > 0 && !rows_range &&
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && !(flags & HPSPMM_PLAN_NO_ROUTED) && nnz > 0 &&
+      !rows_range &&
       (xcd_ok || (flags & HPSPMM_PLAN_FORCE_ROUTED)) &&
       !(flags & HPSPMM_PLAN_FORCE_SEGMENTS && !(flags & HPSPMM_PLAN_FORCE_ROUTED))) {
     if (int rc = build_routed(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_ROUTED) != 0,
@@ -1269,7 +1345,8 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   // most referenced columns take a quarter of the nonzeros there), and the ordered strategy is then
   // the faster of the two (0.73 ms against 1.15 ms for segments with the hub cache).
   const bool want_cluster = (flags & HPSPMM_PLAN_CLUSTER) != 0;
-  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && rows == cols && nnz > 0 && !(flags & HPSPMM_PLAN_NO_CLUSTER) &&
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && rows == cols && nnz > 0 &&
+      !(flags & HPSPMM_PLAN_NO_CLUSTER) &&
       (want_cluster || (!(flags & HPSPMM_PLAN_FORCE_SEGMENTS) && nnz >= kClusterMinNnz &&
                         cols * k * 4 >= kClusterMinBBytes && nnz >= rows * kClusterMinMeanNnz))) {
     int32_t* d_order = nullptr;
@@ -1298,7 +1375,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       p->strategy = HPSPMM_STRATEGY_ROWS;
     }
   }
-  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && !(flags & HPSPMM_PLAN_NO_HUB_CACHE) && nnz > 0) {
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && !(flags & HPSPMM_PLAN_NO_HUB_CACHE) && nnz > 0) {
     if (int rc = build_hub_cache(p, d_col, (int)((flags >> 16) & 0x1Fu), (flags & HPSPMM_PLAN_HUB_CACHE) != 0, st)) {
       return rc;
     }
@@ -1471,6 +1548,8 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
       case 64: rc = launch_routed<64>(plan, d_val, d_B, d_C, st); break;
       default: rc = launch_routed<128>(plan, d_val, d_B, d_C, st); break;
     }
+  } else if (plan->strategy == HPSPMM_STRATEGY_SEGMENTS && !fast_k(plan->k)) {
+    rc = launch_segments_anyk(plan, d_rowptr, d_col, d_val, d_B, d_C, st);
   } else if (plan->strategy == HPSPMM_STRATEGY_SEGMENTS) {
     switch (plan->k) {
       case 32: rc = launch_segments<32>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;

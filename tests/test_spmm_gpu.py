@@ -182,13 +182,52 @@ def test_linearity_and_column_tiles(pkg, oracle, gpu):
     assert np.array_equal(C32, C128[:, :32])
 
 
-@pytest.mark.parametrize("k", [1, 7, 20, 48, 96, 200, 256])
+@pytest.mark.parametrize("k", [1, 7, 30, 50, 130])
 def test_generic_k(pkg, oracle, gpu, k):
+    """Row lengths that are not a multiple of 4 (no 16-byte rows): the one-wavefront-per-row kernel."""
     g = pkg.graphs.make_graph("c4_rmat", 0.002)
     B = pkg.graphs.dense_normal(g.cols, k, 77)
     C, info = _run(pkg, gpu, g, B)
     assert info["strategy"] == pkg.capi.STRATEGY_GENERIC_K
     _check(oracle, g, B, C, f"generic k={k}")
+
+
+@pytest.mark.parametrize("k", [4, 8, 12, 16, 20, 24, 48, 96, 100, 160, 200, 256, 384])
+def test_multiple_of_four_k(pkg, oracle, gpu, k):
+    """Every multiple of 4 besides the tuned sizes goes through the planned sub-wave strategies
+    (the reference has a kernel of its own for K < 32, spmm_kernel.cu:372-387, 406-410): whole rows on a
+    small matrix - with hub rows on a wavefront each -, segments when forced or on a large one, and the
+    plan-less entry point; C poisoned with NaN beforehand, empty rows exact zeros."""
+    import torch
+    capi = pkg.capi
+    g = pkg.graphs.make_graph("c4_rmat", 0.004)  # hub rows of thousands of nonzeros, 40 % empty rows
+    B = pkg.graphs.dense_normal(g.cols, k, 78)
+    C, info = _run(pkg, gpu, g, B)
+    assert info["strategy"] == capi.STRATEGY_ROWS and info["launches_per_spmm"] == 1, info
+    _check(oracle, g, B, C, f"rows k={k}")
+    for shift in (0, 3, 7):
+        C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(shift))
+        assert info["strategy"] == capi.STRATEGY_SEGMENTS and info["launches_per_spmm"] == 2, info
+        assert shift == 0 or info["segment_length"] == 1 << shift
+        _check(oracle, g, B, C, f"segments k={k} shift={shift}")
+        again, _ = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(shift))
+        assert np.array_equal(C, again), "bit-reproducible"
+    rp, ci, v, Bd = _to_dev(gpu, g.rowptr, g.col, g.val, B)
+    Cn = torch.full((g.rows, k), float("nan"), device=gpu)
+    capi.csr_spmm_noplan(g.rows, g.cols, rp, ci, v, Bd, Cn)
+    _check(oracle, g, B, Cn.cpu().numpy(), f"noplan k={k}")
+
+
+@pytest.mark.parametrize("k", [16, 96])
+def test_multiple_of_four_k_large_graph(pkg, oracle, gpu, k):
+    """Beyond 2^21 nonzeros the plan picks segments for these K by itself."""
+    capi = pkg.capi
+    g = pkg.graphs.make_graph("c2_social", 0.05)
+    assert g.nnz > 1 << 21
+    B = pkg.graphs.dense_normal(g.cols, k, 79)
+    C, info = _run(pkg, gpu, g, B)
+    assert info["strategy"] == capi.STRATEGY_SEGMENTS, info
+    _check(oracle, g, B, C, f"auto segments k={k}")
 
 
 def test_edge_shapes(pkg, oracle, gpu):

@@ -62,7 +62,7 @@ EXPORTS = (
     "hpspmm_version", "hpspmm_last_error", "hpspmm_plan_create", "hpspmm_plan_get_info",
     "hpspmm_plan_destroy", "hpspmm_csr_spmm", "hpspmm_csr_spmm_noplan", "hpspmm_coo_spmm_accumulate",
     "hpspmm_fill_f32", "hpspmm_csr_spmm_timed", "hpspmm_plan_bind_values", "hpspmm_plan_create_ordered",
-    "hpspmm_csr_spmm_timed_launches",
+    "hpspmm_csr_spmm_static", "hpspmm_csr_spmm_timed_launches",
 )
 
 _i64 = ctypes.c_int64
@@ -110,6 +110,7 @@ def lib():
         L.hpspmm_plan_bind_values.argtypes = [_p, _p, _p]
         L.hpspmm_csr_spmm.argtypes = [_p, _p, _p, _p, _p, _p, _p]
         L.hpspmm_csr_spmm_noplan.argtypes = [_i64, _i64, _i64, _p, _p, _p, _p, _i64, _p, _p]
+        L.hpspmm_csr_spmm_static.argtypes = [_i64, _i64, _i64, _p, _p, _p, _p, _i64, _p, _p]
         L.hpspmm_coo_spmm_accumulate.argtypes = [_i64, _i64, _i64, _p, _p, _p, _p, _i64, _p, _p]
         L.hpspmm_fill_f32.argtypes = [_p, _i64, ctypes.c_float, _p]
         L.hpspmm_csr_spmm_timed.argtypes = [_p, _p, _p, _p, _p, _p, _p, ctypes.c_int, ctypes.c_int,
@@ -225,6 +226,15 @@ def csr_spmm_noplan(rows, cols, rowptr, col, val, B, C, stream=None):
     k = int(B.shape[1])
     _check_operands(rows, cols, int(col.numel()), k, rowptr, col, val, B, C)
     check(lib().hpspmm_csr_spmm_noplan(rows, cols, int(col.numel()), _ptr(rowptr), _ptr(col), _ptr(val),
+                                       _ptr(B), k, _ptr(C), _stream(stream)))
+    return C
+
+
+def csr_spmm_static(rows, cols, rowptr, col, val, B, C, stream=None):
+    """C = A @ B through hpspmm_csr_spmm_static (no plan, no allocation; k in {32,64,128}, nnz <= 2^22)."""
+    k = int(B.shape[1])
+    _check_operands(rows, cols, int(col.numel()), k, rowptr, col, val, B, C)
+    check(lib().hpspmm_csr_spmm_static(rows, cols, int(col.numel()), _ptr(rowptr), _ptr(col), _ptr(val),
                                        _ptr(B), k, _ptr(C), _stream(stream)))
     return C
 

@@ -1586,6 +1586,97 @@ int hpspmm_csr_spmm_noplan(int64_t rows, int64_t cols, int64_t nnz, const int32_
   return HPSPMM_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// hpspmm_csr_spmm_static: the segments strategy without a plan and without any allocation.  What a
+// plan would hold in its workspace lives in one file-scope device array: the row of every nonzero
+// (kStaticMaxNnz int32) followed by the carry slots (kStaticCarryFloats floats).  Every device the
+// library is loaded on holds its own copy of the array; its address there is looked up once per
+// device (hipGetSymbolAddress) and only that pointer is ever handed to kernels.
+// ---------------------------------------------------------------------------------------------
+}  // extern "C"
+
+namespace {
+constexpr int64_t kStaticMaxNnz = (int64_t)1 << 22;
+constexpr int64_t kStaticCarryFloats = (int64_t)1 << 22;
+constexpr size_t kStaticScratchBytes = (size_t)kStaticMaxNnz * sizeof(int32_t) + (size_t)kStaticCarryFloats * sizeof(float);
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+namespace {
+std::mutex g_static_mutex;
+void* g_static_ptr[kMaxDevices] = {nullptr};
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int static_scratch(void** out) {
+  int dev = 0;
+  HPSPMM_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(HPSPMM_ERR_INVALID_ARG, "device index %d not supported", dev);
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (!g_static_ptr[dev]) {
+    void* ptr = nullptr;
+    HPSPMM_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return fail(HPSPMM_ERR_HIP, "hipGetSymbolAddress returned a null address for the static workspace");
+    g_static_ptr[dev] = ptr;
+  }
+  *out = g_static_ptr[dev];
+  return HPSPMM_OK;
+}
+
+template <int K>
+int launch_static(int64_t rows, int64_t nnz, const int32_t* rp, const int32_t* ci, const float* v, const float* B,
+                  float* C, int32_t* nnz_row, float* carry, hipStream_t st) {
+  constexpr int P = 64 / (K / 4);
+  // segment length as a plan would choose it, then doubled until the carry slots fit the static array
+  int shift = 5;
+  const int64_t target_waves = 256 * 4 * 16;
+  while (shift < 9 && (nnz >> (shift + 1)) / P >= target_waves) ++shift;
+  while (2 * ceil_div(nnz, (int64_t)1 << shift) * K > kStaticCarryFloats) ++shift;
+  const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
+  if (nnz > 0) {
+    hipLaunchKernelGGL(hpspmm::expand_rows_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                       0, st, rows, nnz, rp, nnz_row);
+    const int64_t nblocks = ceil_div(ceil_div(nseg, P), hpspmm::kWavesPerBlock);
+    hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, false, false>), dim3((unsigned)nblocks), dim3(hpspmm::kBlock),
+                       0, st, rp, ci, v, (const int32_t*)nnz_row, B, (const float*)nullptr, C, carry, nnz, shift, nseg,
+                       nblocks, false, aligned16(ci, v, nnz_row));
+  }
+  const int rpw = fixup_rows_per_wave(rows, K);
+  const int64_t fix_blocks = ceil_div(ceil_div(rows, rpw), hpspmm::kWavesPerBlock);
+  hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st, rows, rp,
+                     (const int32_t*)nullptr, (const float*)carry, C, shift, rpw);
+  return HPSPMM_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int hpspmm_csr_spmm_static(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr, const int32_t* d_col,
+                           const float* d_val, const float* d_B, int64_t k, float* d_C, void* stream) {
+  if (int rc = check_dims(rows, cols, nnz, k)) return rc;
+  if (!fast_k(k)) return fail(HPSPMM_ERR_INVALID_ARG, "hpspmm_csr_spmm_static: k must be 32, 64 or 128, got %lld", (long long)k);
+  if (nnz > kStaticMaxNnz)
+    return fail(HPSPMM_ERR_INVALID_ARG,
+                "hpspmm_csr_spmm_static: nnz = %lld exceeds the static workspace (at most %lld nonzeros); use a plan",
+                (long long)nnz, (long long)kStaticMaxNnz);
+  if (rows == 0) return HPSPMM_OK;
+  if (!d_rowptr || !d_C) return fail(HPSPMM_ERR_INVALID_ARG, "d_rowptr or d_C is NULL");
+  if (nnz > 0 && (!d_col || !d_val || !d_B))
+    return fail(HPSPMM_ERR_INVALID_ARG, "d_col, d_val or d_B is NULL with nnz > 0");
+  void* base = nullptr;
+  if (int rc = static_scratch(&base)) return rc;
+  int32_t* nnz_row = static_cast<int32_t*>(base);
+  float* carry = reinterpret_cast<float*>(static_cast<unsigned char*>(base) + (size_t)kStaticMaxNnz * sizeof(int32_t));
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  switch (k) {
+    case 32: rc = launch_static<32>(rows, nnz, d_rowptr, d_col, d_val, d_B, d_C, nnz_row, carry, st); break;
+    case 64: rc = launch_static<64>(rows, nnz, d_rowptr, d_col, d_val, d_B, d_C, nnz_row, carry, st); break;
+    default: rc = launch_static<128>(rows, nnz, d_rowptr, d_col, d_val, d_B, d_C, nnz_row, carry, st); break;
+  }
+  if (rc) return rc;
+  HPSPMM_HIP(hipGetLastError());
+  return HPSPMM_OK;
+}
+
 int hpspmm_coo_spmm_accumulate(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_row,
                                const int32_t* d_col, const float* d_val, const float* d_B, int64_t k, float* d_C,
                                void* stream) {

@@ -209,6 +209,24 @@ int hpspmm_csr_spmm_noplan(int64_t rows, int64_t cols, int64_t nnz, const int32_
                            float *d_C, void *stream);
 
 /*
+ * C = A * B like hpspmm_csr_spmm under the segments strategy, for callers that
+ * cannot allocate device memory or keep a plan (code under HIP-graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): no hipMalloc, hipFree,
+ * memset or host synchronisation - three kernel launches on `stream`.  It has
+ * no counterpart in the reference.  The workspace a plan would own (row of
+ * every nonzero, carry slots of split rows) is a 32 MiB array inside the
+ * library's device image, one copy per GPU, kept until the process ends.
+ * Limits: k in {32, 64, 128} and nnz <= 2^22 (HPSPMM_ERR_INVALID_ARG beyond).
+ * Nothing in the array needs clearing between calls (every slot a call reads it
+ * has written before), but all calls on one GPU share it: calls that overlap in
+ * time on one GPU - two streams, two host threads - race.  The CSR arrays are
+ * not validated.
+ */
+int hpspmm_csr_spmm_static(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
+                           const int32_t *d_col, const float *d_val, const float *d_B, int64_t k,
+                           float *d_C, void *stream);
+
+/*
  * C += A * B for A in COO (row-index per nonzero), the contract of one launch
  * of LBSpMM (spmm/mm/spmm_kernel.cu:733-768: accumulates with atomics,
  * :463-476).  Entries of one row need not be contiguous, `nnz` may include

@@ -17,6 +17,7 @@
 
 #include "anyk_kernels.hpp"
 #include "ordered_kernels.hpp"
+#include "rank_kernels.hpp"
 #include "routed_kernels.hpp"
 #include "rowtile_kernels.hpp"
 #include "spmm_kernels.hpp"
@@ -563,53 +564,6 @@ int choose_shift(int64_t nnz, int64_t k, int64_t max_row_nnz) {
   return shift;
 }
 
-// Column popularity: count[c] = nonzeros in column c, and the `want` most
-// referenced columns in order of decreasing count (ties by lower index, so the
-// choice is reproducible); columns referenced fewer than twice are dropped.
-// The result of the last call is kept per thread and handed out again for the same plan and
-// `want`: the routed and the hub-cache decisions of one plan ask for the same ranking.
-struct RankCache {
-  const hpspmm_plan* plan = nullptr;
-  int64_t want = 0;
-  std::vector<int32_t> count, ids;
-};
-thread_local RankCache g_rank_cache;
-
-int rank_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t want, hipStream_t st,
-                 std::vector<int32_t>& count, std::vector<int32_t>& ids) {
-  if (g_rank_cache.plan == p && g_rank_cache.want == want) {
-    count = g_rank_cache.count;
-    ids = g_rank_cache.ids;
-    return HPSPMM_OK;
-  }
-  const int64_t asked = want;
-  int32_t* d_count = nullptr;
-  HPSPMM_HIP(hipMalloc(&d_count, (size_t)p->cols * sizeof(int32_t)));
-  struct Guard {
-    int32_t* q;
-    ~Guard() { (void)hipFree(q); }
-  } guard{d_count};
-  HPSPMM_HIP(hipMemsetAsync(d_count, 0, (size_t)p->cols * sizeof(int32_t), st));
-  hipLaunchKernelGGL(hpspmm::count_columns_kernel, dim3(grid_for(p->nnz, 1 << 16)), dim3(hpspmm::kBlock), 0, st,
-                     p->nnz, d_col, d_count);
-  count.resize((size_t)p->cols);
-  HPSPMM_HIP(hipMemcpyAsync(count.data(), d_count, count.size() * sizeof(int32_t), hipMemcpyDeviceToHost, st));
-  HPSPMM_HIP(hipStreamSynchronize(st));
-  want = std::min<int64_t>(want, p->cols);
-  ids.resize((size_t)p->cols);
-  for (int64_t i = 0; i < p->cols; ++i) ids[i] = (int32_t)i;
-  auto hotter = [&](int32_t a, int32_t b) { return count[a] != count[b] ? count[a] > count[b] : a < b; };
-  if (want < p->cols) std::nth_element(ids.begin(), ids.begin() + (want - 1), ids.end(), hotter);
-  ids.resize((size_t)want);
-  std::sort(ids.begin(), ids.end(), hotter);
-  while (!ids.empty() && count[ids.back()] < 2) ids.pop_back();
-  g_rank_cache.plan = p;
-  g_rank_cache.want = asked;
-  g_rank_cache.count = count;
-  g_rank_cache.ids = ids;
-  return HPSPMM_OK;
-}
-
 // Device exclusive scan of n uint32 values (three passes, tile sums in between); d_out may be d_in.
 int exclusive_scan_u32(const uint32_t* d_in, uint32_t* d_out, int64_t n, hipStream_t st) {
   const int64_t ntiles = ceil_div(n, hpspmm::kScanTile);
@@ -627,6 +581,183 @@ int exclusive_scan_u32(const uint32_t* d_in, uint32_t* d_out, int64_t n, hipStre
   return HPSPMM_OK;
 }
 
+// Column popularity, on the device: d_count[c] = nonzeros in column c, and d_ids = the `want` most
+// referenced columns in order of decreasing count (ties by lower index, so the choice is
+// reproducible); columns referenced fewer than twice are dropped.  One object per plan construction:
+// the routed and the hub-cache decisions share the histogram, and the ranking too when they ask for
+// the same `want`.
+struct ColumnRanking {
+  int32_t* d_count = nullptr;  // [cols]
+  int32_t* d_ids = nullptr;    // [n_ids]
+  int64_t want = 0, n_ids = 0, served = 0;  // served = nonzeros in the ranked columns
+  ~ColumnRanking() {
+    if (d_count) (void)hipFree(d_count);
+    if (d_ids) (void)hipFree(d_ids);
+  }
+};
+
+// Rank-by-counting sorts up to this many keys (m^2 compares: 0.5 ms at 2^16, 2 ms at 2^17).
+constexpr int64_t kRankMaxKeys = (int64_t)1 << 17;
+
+// Histogram of every `stride`-th column index into a fresh d_count_out (caller frees).
+int count_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t stride, hipStream_t st, int32_t** d_count_out) {
+  int32_t* d_count = nullptr;
+  HPSPMM_HIP(hipMalloc(&d_count, (size_t)std::max<int64_t>(1, p->cols) * sizeof(int32_t)));
+  hipError_t e = hipMemsetAsync(d_count, 0, (size_t)std::max<int64_t>(1, p->cols) * sizeof(int32_t), st);
+  if (e != hipSuccess) {
+    (void)hipFree(d_count);
+    return fail(HPSPMM_ERR_HIP, "hipMemsetAsync: %s", hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(hpspmm::count_columns_strided_kernel, dim3(grid_for(ceil_div(p->nnz, stride), 1 << 16)),
+                     dim3(hpspmm::kBlock), 0, st, p->nnz, stride, d_col, d_count);
+  *d_count_out = d_count;
+  return HPSPMM_OK;
+}
+
+// The `want` largest of the n counters at d_count (ties at the threshold by lower index, counters
+// below 2 never): *d_keys_out = their keys (~count << 32 | index) in index order (caller frees),
+// *m_out how many.
+int select_top_columns(const int32_t* d_count, int64_t n, int64_t want, hipStream_t st,
+                       unsigned long long** d_keys_out, int64_t* m_out) {
+  *d_keys_out = nullptr;
+  *m_out = 0;
+  want = std::min(want, n);
+  if (want <= 0 || n <= 0) return HPSPMM_OK;
+  uint32_t *d_hist = nullptr, *d_above = nullptr, *d_equal = nullptr;
+  struct Guard {
+    void** q[3];
+    ~Guard() {
+      for (void** x : q)
+        if (*x) (void)hipFree(*x);
+    }
+  } guard{{(void**)&d_hist, (void**)&d_above, (void**)&d_equal}};
+  HPSPMM_HIP(hipMalloc(&d_hist, 256 * sizeof(uint32_t)));
+  // radix select of the want-th largest counter, most significant byte first
+  uint32_t prefix = 0;
+  int64_t remaining = want;  // how many of the counters matching the prefix so far are wanted
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    uint32_t hist[256];
+    HPSPMM_HIP(hipMemsetAsync(d_hist, 0, sizeof hist, st));
+    hipLaunchKernelGGL(hpspmm::select_histogram_kernel, dim3(grid_for(n, 2048)), dim3(hpspmm::kBlock), 0, st, n,
+                       d_count, prefix, shift, d_hist);
+    HPSPMM_HIP(hipMemcpyAsync(hist, d_hist, sizeof hist, hipMemcpyDeviceToHost, st));
+    HPSPMM_HIP(hipStreamSynchronize(st));
+    int b = 255;
+    for (; b > 0 && remaining > (int64_t)hist[b]; --b) remaining -= hist[b];
+    prefix |= (uint32_t)b << shift;
+  }
+  // counters above max(threshold, 1), then as many at the threshold as are still wanted
+  const int32_t found = (int32_t)prefix;
+  const int32_t threshold = found < 2 ? 1 : found;
+  HPSPMM_HIP(hipMalloc(&d_above, (size_t)(n + 1) * sizeof(uint32_t)));
+  HPSPMM_HIP(hipMalloc(&d_equal, (size_t)(n + 1) * sizeof(uint32_t)));
+  hipLaunchKernelGGL(hpspmm::select_flags_kernel, dim3((unsigned)ceil_div(n + 1, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, n, d_count, threshold, d_above, d_equal);
+  if (int rc = exclusive_scan_u32(d_above, d_above, n + 1, st)) return rc;
+  if (int rc = exclusive_scan_u32(d_equal, d_equal, n + 1, st)) return rc;
+  uint32_t n_above = 0, n_equal = 0;
+  HPSPMM_HIP(hipMemcpyAsync(&n_above, d_above + n, sizeof n_above, hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipMemcpyAsync(&n_equal, d_equal + n, sizeof n_equal, hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  const int64_t ties = found < 2 ? 0 : std::min<int64_t>(n_equal, want - (int64_t)n_above);
+  const int64_t m = (int64_t)n_above + std::max<int64_t>(ties, 0);
+  if (m <= 0) return HPSPMM_OK;
+  unsigned long long* d_keys = nullptr;
+  HPSPMM_HIP(hipMalloc(&d_keys, (size_t)m * sizeof(unsigned long long)));
+  hipLaunchKernelGGL(hpspmm::select_compact_kernel, dim3((unsigned)ceil_div(n, hpspmm::kBlock)), dim3(hpspmm::kBlock), 0,
+                     st, n, d_count, threshold, d_above, d_equal, n_above, (uint32_t)std::max<int64_t>(ties, 0), d_keys);
+  hipError_t e = hipStreamSynchronize(st);  // the scans go out of scope
+  if (e != hipSuccess) {
+    (void)hipFree(d_keys);
+    return fail(HPSPMM_ERR_HIP, "column selection failed: %s", hipGetErrorString(e));
+  }
+  *d_keys_out = d_keys;
+  *m_out = m;
+  return HPSPMM_OK;
+}
+
+int rank_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t want, hipStream_t st, ColumnRanking& rk) {
+  if (rk.d_ids && rk.want == want) return HPSPMM_OK;
+  if (rk.d_ids) {
+    (void)hipFree(rk.d_ids);
+    rk.d_ids = nullptr;
+  }
+  rk.want = want;
+  rk.n_ids = 0;
+  rk.served = 0;
+  if (!rk.d_count)
+    if (int rc = count_columns(p, d_col, 1, st, &rk.d_count)) return rc;
+  unsigned long long* d_keys = nullptr;
+  int64_t m = 0;
+  if (int rc = select_top_columns(rk.d_count, p->cols, want, st, &d_keys, &m)) return rc;
+  struct Guard {
+    unsigned long long* q;
+    ~Guard() {
+      if (q) (void)hipFree(q);
+    }
+  } guard{d_keys};
+  HPSPMM_HIP(hipMalloc(&rk.d_ids, (size_t)std::max<int64_t>(1, m) * sizeof(int32_t)));
+  if (m == 0) return HPSPMM_OK;
+  unsigned long long served = 0;
+  if (m <= kRankMaxKeys) {
+    unsigned long long* d_served = nullptr;
+    HPSPMM_HIP(hipMalloc(&d_served, sizeof(unsigned long long)));
+    hipError_t e = hipMemsetAsync(d_served, 0, sizeof(unsigned long long), st);
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL(hpspmm::rank_sort_kernel, dim3((unsigned)ceil_div(m, hpspmm::kBlock)), dim3(hpspmm::kBlock), 0,
+                         st, (int32_t)m, d_keys, rk.d_ids, d_served);
+      e = hipMemcpyAsync(&served, d_served, sizeof served, hipMemcpyDeviceToHost, st);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    (void)hipFree(d_served);
+    if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "column ranking failed: %s", hipGetErrorString(e));
+  } else {
+    // more keys than the counting sort is meant for (a hub cache of millions of rows, asked for by
+    // flag): sorted on the host
+    std::vector<unsigned long long> keys((size_t)m);
+    HPSPMM_HIP(hipMemcpyAsync(keys.data(), d_keys, keys.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost, st));
+    HPSPMM_HIP(hipStreamSynchronize(st));
+    std::sort(keys.begin(), keys.end());
+    std::vector<int32_t> ids((size_t)m);
+    for (size_t i = 0; i < keys.size(); ++i) {
+      ids[i] = (int32_t)(uint32_t)keys[i];
+      served += (unsigned long long)(~(uint32_t)(keys[i] >> 32));
+    }
+    HPSPMM_HIP(hipMemcpyAsync(rk.d_ids, ids.data(), ids.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
+    HPSPMM_HIP(hipStreamSynchronize(st));
+  }
+  rk.n_ids = m;
+  rk.served = (int64_t)served;
+  return HPSPMM_OK;
+}
+
+// Share of the nonzeros that the `want` most referenced columns take, estimated from every 8th
+// nonzero (an overestimate when the columns are evenly used: the most referenced columns of a
+// sample are partly its noise).  Lets a graph without hot columns skip the full histogram.
+int estimate_hot_share(const hpspmm_plan* p, const int32_t* d_col, int64_t want, hipStream_t st, double* share_out) {
+  constexpr int64_t kStride = 8;
+  *share_out = 1.0;
+  if (p->nnz < (kStride << 16)) return HPSPMM_OK;  // too small to be worth a pass of its own
+  int32_t* d_count = nullptr;
+  if (int rc = count_columns(p, d_col, kStride, st, &d_count)) return rc;
+  unsigned long long* d_keys = nullptr;
+  int64_t m = 0;
+  int rc = select_top_columns(d_count, p->cols, want, st, &d_keys, &m);
+  (void)hipFree(d_count);
+  if (rc) return rc;
+  unsigned long long served = 0;
+  if (m > 0) {
+    std::vector<unsigned long long> keys((size_t)m);
+    hipError_t e = hipMemcpyAsync(keys.data(), d_keys, keys.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    (void)hipFree(d_keys);
+    if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "hot-share estimate failed: %s", hipGetErrorString(e));
+    for (unsigned long long k : keys) served += (unsigned long long)(~(uint32_t)(k >> 32));
+  }
+  *share_out = (double)served / (double)ceil_div(p->nnz, kStride);
+  return HPSPMM_OK;
+}
+
 // Rows of B kept in the compact buffer by the routed strategy (all slices together).
 constexpr int kRoutedLog2Cached = 16;
 // Automatic choice of the routed strategy (thresholds from measurements on the
@@ -637,6 +768,7 @@ constexpr int kRoutedLog2Cached = 16;
 constexpr int64_t kRoutedMinNnz = (int64_t)1 << 22;
 constexpr int64_t kRoutedMinBBytes = (int64_t)10 << 20;  // a B that one or two L2s hold needs no routing (social graph at 26 M nonzeros: B = 7 MB, routed 309 us against 246; B = 14 MB, 464 against 474)
 constexpr double kRoutedMinShare = 0.35;     // of the nonzeros in the 64k most referenced columns
+constexpr double kRoutedEstimateMargin = 0.7;  // the estimate from a sample must reach this part of it
 constexpr double kRoutedMinRowNnz = 32.0;    // mean nonzeros per non-empty row
 constexpr int32_t kRoutedRowThreshold = 128;  // rows shorter than this are not split over the classes
 constexpr double kRoutedMinRoutedShare = 0.3;  // of the nonzeros in rows of at least that length
@@ -670,34 +802,31 @@ bool columns_sorted(const hpspmm_plan* p, const int32_t* d_col, hipStream_t st) 
 // Builds the routed layout.  Returns HPSPMM_OK with p->strategy left at
 // SEGMENTS when the graph does not qualify (and `forced` is false).
 int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, int log2_hubs,
-                 int log2_row_threshold, int want_sub, bool sort_values, hipStream_t st) {
+                 int log2_row_threshold, int want_sub, bool sort_values, ColumnRanking& rk, hipStream_t st) {
   const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
   if (!forced && (nnz < kRoutedMinNnz || p->cols * k * 4 < kRoutedMinBBytes)) return HPSPMM_OK;
+  const int64_t nonempty = std::max<int64_t>(1, rows - p->empty_rows);
+  if (!forced && (double)nnz / (double)nonempty < kRoutedMinRowNnz) return HPSPMM_OK;
+  if (nnz > INT32_MAX - ((int64_t)1 << 24)) return HPSPMM_OK;  // virtual indices stay int32
   // cached rows per class
   const int64_t h =
       std::max<int64_t>(1, ((int64_t)1 << (log2_hubs ? log2_hubs : kRoutedLog2Cached)) / hpspmm::kSlices);
-  std::vector<int32_t> count, ids;
-  if (int rc = rank_columns(p, d_col, h * hpspmm::kSlices, st, count, ids)) return rc;
-  int64_t served = 0;
-  for (int32_t c : ids) served += count[c];
-  const int64_t nonempty = std::max<int64_t>(1, rows - p->empty_rows);
-  if (!forced && ((double)served < kRoutedMinShare * (double)nnz ||
-                  (double)nnz / (double)nonempty < kRoutedMinRowNnz))
-    return HPSPMM_OK;
-  if (nnz > INT32_MAX - ((int64_t)1 << 24)) return HPSPMM_OK;  // virtual indices stay int32
+  if (!forced) {
+    // a look at every 8th nonzero first: a graph whose columns are evenly used is told apart
+    // without the full histogram
+    double estimate = 1.0;
+    if (int rc = estimate_hot_share(p, d_col, h * hpspmm::kSlices, st, &estimate)) return rc;
+    if (estimate < kRoutedMinShare * kRoutedEstimateMargin) return HPSPMM_OK;
+  }
+  if (int rc = rank_columns(p, d_col, h * hpspmm::kSlices, st, rk)) return rc;
+  if (!forced && (double)rk.served < kRoutedMinShare * (double)nnz) return HPSPMM_OK;
+  const int32_t n_ids = (int32_t)rk.n_ids;
 
   const int64_t slice_bytes = p->cols * k * 4 / hpspmm::kSlices;
   int nsub = slice_bytes > kRoutedPhaseBytes ? 2 : 1;
   if (want_sub) nsub = std::min(want_sub, hpspmm::kMaxSub);
 
-  // popularity rank s -> slice s % 8, compact-buffer row (s % 8) * h + s / 8
   const int64_t n_bhot = h * hpspmm::kSlices;
-  std::vector<int32_t> colmap((size_t)p->cols, -1), bhot_src((size_t)n_bhot, -1);
-  for (size_t s2 = 0; s2 < ids.size(); ++s2) {
-    const int64_t slot = (int64_t)(s2 % hpspmm::kSlices) * h + (int64_t)(s2 / hpspmm::kSlices);
-    colmap[ids[s2]] = (int32_t)slot;
-    bhot_src[(size_t)slot] = ids[s2];
-  }
 
   const int nhub = hpspmm::kSlices * nsub;
   const int32_t min_row_nnz =
@@ -712,35 +841,10 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   // with one phase: with two the runs are half as long, the value loads fetch 1.8 lines per run, and
   // what the re-ordering pass saved is spent inside the main kernel (social graph, K = 128: 3.73 ms
   // either way; R-MAT: 6.0 -> 6.85 ms).
-  std::vector<uint8_t> colrange;
-  if (!sort_values && nsub == 1 && nnz > 0 && p->cols * k * 4 < ((int64_t)1 << 32) && p->d_nnz_row &&
-      columns_sorted(p, d_col, st)) {
-    const int groups = nhub;
-    const int64_t target = ceil_div(nnz, groups);
-    std::vector<uint8_t> range((size_t)p->cols);
-    std::vector<int64_t> hot((size_t)groups, 0);
-    int64_t before = 0;
-    for (int64_t c = 0; c < p->cols; ++c) {
-      range[(size_t)c] = (uint8_t)std::min<int64_t>(groups - 1, before / target);
-      before += count[(size_t)c];
-    }
-    for (int32_t c : ids) ++hot[range[(size_t)c]];
-    const int64_t most = *std::max_element(hot.begin(), hot.end());
-    if (most * 2 * groups <= 3 * (int64_t)ids.size() + 32 * groups) colrange.swap(range);
-  }
-  const bool inplace = !colrange.empty();
-  // Evenly spread hot columns also mean that their rows of B do not crowd a few memory channels, which
-  // is what the compact buffer is for (R-MAT): without it (social graph, K = 32: 1.128 against
-  // 1.135 ms with it) the kernel's gather address is a 32-bit offset from B and the hot rows need
-  // no copying at the start of every SpMM.
-  if (inplace) {
-    std::fill(colmap.begin(), colmap.end(), -1);
-    std::fill(bhot_src.begin(), bhot_src.end(), -1);
-  }
-
-  // temporaries of the layout construction
+  // temporaries of the layout construction (freed by the guard on every way out)
   uint8_t* d_colrange = nullptr;
   int32_t* d_colmap = nullptr;
+  int32_t* d_bhot_src_tmp = nullptr;  // [n_bhot], handed to the plan once the layout is accepted
   uint32_t* d_ridx = nullptr;     // [rows + 1] routed flag, then (scanned in place) routed-row number
   uint32_t* d_cnt = nullptr;      // [nhub * n_routed + 1] class-major counts, then their scan
   uint32_t* d_coldcnt = nullptr;  // [rows + 1] cold-class count per row, then its scan
@@ -748,23 +852,66 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   int32_t* d_counts = nullptr;    // [2] list lengths
   int32_t* d_vpos = nullptr;      // [nnz] position of every stored nonzero in the class-major order
   struct Guard {
-    void** q[8];
+    void** q[9];
     ~Guard() {
       for (void** x : q)
         if (*x) (void)hipFree(*x);
     }
   } guard{{(void**)&d_colmap, (void**)&d_ridx, (void**)&d_cnt, (void**)&d_coldcnt, (void**)&d_action,
-           (void**)&d_counts, (void**)&d_vpos, (void**)&d_colrange}};
-  HPSPMM_HIP(hipMalloc(&d_colmap, (size_t)std::max<int64_t>(1, p->cols) * sizeof(int32_t)));
-  if (inplace) {
-    HPSPMM_HIP(hipMalloc(&d_colrange, colrange.size()));
-    HPSPMM_HIP(hipMemcpyAsync(d_colrange, colrange.data(), colrange.size(), hipMemcpyHostToDevice, st));
+           (void**)&d_counts, (void**)&d_vpos, (void**)&d_colrange, (void**)&d_bhot_src_tmp}};
+
+  bool inplace = false;
+  if (!sort_values && nsub == 1 && nnz > 0 && p->cols * k * 4 < ((int64_t)1 << 32) && p->d_nnz_row &&
+      columns_sorted(p, d_col, st)) {
+    const int groups = nhub;
+    const int64_t target = ceil_div(nnz, groups);
+    uint32_t* d_before = nullptr;
+    uint32_t* d_hot = nullptr;
+    uint32_t hot[hpspmm::kMaxHub] = {0};
+    hipError_t e = hipMalloc(&d_before, (size_t)(p->cols + 1) * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMalloc(&d_hot, sizeof hot);
+    if (e == hipSuccess) e = hipMalloc(&d_colrange, (size_t)p->cols);
+    if (e == hipSuccess) e = hipMemsetAsync(d_hot, 0, sizeof hot, st);
+    int rc = HPSPMM_OK;
+    if (e == hipSuccess)  // the counts are non-negative: scanned as uint32 (one spare slot keeps the scan's tail in bounds)
+      rc = exclusive_scan_u32(reinterpret_cast<const uint32_t*>(rk.d_count), d_before, p->cols, st);
+    if (e == hipSuccess && rc == HPSPMM_OK) {
+      hipLaunchKernelGGL(hpspmm::column_range_kernel, dim3((unsigned)ceil_div(p->cols, hpspmm::kBlock)),
+                         dim3(hpspmm::kBlock), 0, st, p->cols, d_before, target, groups, d_colrange);
+      if (n_ids > 0)
+        hipLaunchKernelGGL(hpspmm::range_hot_count_kernel, dim3((unsigned)ceil_div(n_ids, hpspmm::kBlock)),
+                           dim3(hpspmm::kBlock), 0, st, n_ids, rk.d_ids, d_colrange, d_hot);
+      e = hipMemcpyAsync(hot, d_hot, sizeof hot, hipMemcpyDeviceToHost, st);
+      if (e == hipSuccess) e = hipStreamSynchronize(st);
+    }
+    if (d_before) (void)hipFree(d_before);
+    if (d_hot) (void)hipFree(d_hot);
+    if (rc) return rc;
+    if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "column ranges: %s", hipGetErrorString(e));
+    const int64_t most = *std::max_element(hot, hot + groups);
+    inplace = most * 2 * groups <= 3 * (int64_t)n_ids + 32 * groups;
+    if (!inplace) {
+      (void)hipFree(d_colrange);
+      d_colrange = nullptr;
+    }
   }
+  // Evenly spread hot columns also mean that their rows of B do not crowd a few memory channels, which
+  // is what the compact buffer is for (R-MAT): without it (social graph, K = 32: 1.128 against
+  // 1.135 ms with it) the kernel's gather address is a 32-bit offset from B and the hot rows need
+  // no copying at the start of every SpMM.
+
+  // popularity rank s -> slice s % 8, compact-buffer row (s % 8) * h + s / 8 (none with column ranges)
+  HPSPMM_HIP(hipMalloc(&d_colmap, (size_t)std::max<int64_t>(1, p->cols) * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&d_bhot_src_tmp, (size_t)n_bhot * sizeof(int32_t)));
+  HPSPMM_HIP(hipMemsetAsync(d_colmap, 0xFF, (size_t)std::max<int64_t>(1, p->cols) * sizeof(int32_t), st));
+  HPSPMM_HIP(hipMemsetAsync(d_bhot_src_tmp, 0xFF, (size_t)n_bhot * sizeof(int32_t), st));
+  if (!inplace && n_ids > 0)
+    hipLaunchKernelGGL(hpspmm::hot_slots_kernel, dim3((unsigned)ceil_div(n_ids, hpspmm::kBlock)), dim3(hpspmm::kBlock), 0,
+                       st, n_ids, rk.d_ids, hpspmm::kSlices, (int32_t)h, d_colmap, d_bhot_src_tmp);
   HPSPMM_HIP(hipMalloc(&d_ridx, (size_t)(rows + 1) * sizeof(uint32_t)));
   HPSPMM_HIP(hipMalloc(&d_coldcnt, (size_t)(rows + 1) * sizeof(uint32_t)));
   HPSPMM_HIP(hipMalloc(&d_action, (size_t)rows));
   HPSPMM_HIP(hipMalloc(&d_counts, 2 * sizeof(int32_t)));
-  HPSPMM_HIP(hipMemcpyAsync(d_colmap, colmap.data(), colmap.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
 
   // number the routed rows
   hipLaunchKernelGGL(hpspmm::routed_flag_kernel, dim3((unsigned)ceil_div(rows + 1, hpspmm::kBlock)),
@@ -859,15 +1006,14 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   if (!ok ||
       hipMalloc(&p->d_partial, partial_bytes) != hipSuccess || hipMalloc(&p->d_carry, carry_bytes) != hipSuccess ||
       hipMalloc(&p->d_bhot, bhot_bytes) != hipSuccess ||
-      hipMalloc(&p->d_bhot_src, (size_t)n_bhot * sizeof(int32_t)) != hipSuccess ||
       hipMalloc(&p->d_routed_rows, routed_rows_bytes) != hipSuccess ||
       hipMalloc(&p->d_cross_rows, list_bytes) != hipSuccess || hipMalloc(&p->d_zero_rows, list_bytes) != hipSuccess) {
     (void)hipGetLastError();
     return fail(HPSPMM_ERR_ALLOC, "device allocation for the routed plan failed (%zu bytes)", total_bytes);
   }
   p->workspace_bytes = (int64_t)total_bytes;
-  HPSPMM_HIP(hipMemcpyAsync(p->d_bhot_src, bhot_src.data(), bhot_src.size() * sizeof(int32_t),
-                            hipMemcpyHostToDevice, st));
+  p->d_bhot_src = d_bhot_src_tmp;  // the plan owns it from here on
+  d_bhot_src_tmp = nullptr;
   // unused compact-buffer rows and the padding between the classes are never used; keep them defined anyway
   HPSPMM_HIP(hipMemsetAsync(p->d_bhot, 0, bhot_bytes, st));
   HPSPMM_HIP(hipMemsetAsync(inplace ? (void*)p->d_vsrc : (void*)p->d_vval, 0, v_bytes, st));
@@ -898,7 +1044,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   p->n_cross = counts[0];
   p->n_zero = counts[1];
   p->n_bhot = inplace ? 0 : n_bhot;
-  p->n_hub = inplace ? 0 : (int64_t)ids.size();
+  p->n_hub = inplace ? 0 : (int64_t)n_ids;
   p->nseg = nseg;
   p->strategy = HPSPMM_STRATEGY_ROUTED;
   return HPSPMM_OK;
@@ -920,19 +1066,31 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
     mark_launch(st, "routed_prepare_kernel");
   }
   if (p->routed_grid > 0) {
-    if (inplace)
-      hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, true, false>), dim3((unsigned)p->routed_grid),
-                         dim3(hpspmm::kBlock), 0, st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, v, p->d_vsrc,
-                         p->d_vrow, B, p->d_bhot, p->d_partial, p->d_carry, C);
-    else if (p->d_vsrc)  // column-range slices, values bound: the plan's own copy of them, still no compact buffer
-      hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false, false>), dim3((unsigned)p->routed_grid),
-                         dim3(hpspmm::kBlock), 0, st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval,
-                         (const int32_t*)nullptr, p->d_vrow, B, p->d_bhot, p->d_partial, p->d_carry, C);
-    else
-      hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false, true>), dim3((unsigned)p->routed_grid),
-                         dim3(hpspmm::kBlock), 0, st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval,
-                         (const int32_t*)nullptr, p->d_vrow, B, p->d_bhot, p->d_partial, p->d_carry, C);
-    mark_launch(st, "spmm_routed_kernel");
+    // One launch; with HPSPMM_ROUTED_SPLIT_LAUNCH=1 (diagnostics: per-class times and counters) one per
+    // phase of the hub classes and one for the cold class, each from its first workgroup on.
+    const char* split_env = std::getenv("HPSPMM_ROUTED_SPLIT_LAUNCH");
+    const bool split = split_env && split_env[0] == '1';
+    const int parts = split ? p->lay.nsub + 1 : 1;
+    for (int part = 0; part < parts; ++part) {
+      const int64_t first = split ? p->lay.phase_begin[part] : 0;
+      const int64_t last = split ? (part < p->lay.nsub ? p->lay.phase_begin[part + 1] : p->routed_grid) : p->routed_grid;
+      if (last <= first) continue;
+      const dim3 grid((unsigned)(last - first));
+      if (inplace)
+        hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, true, false>), grid, dim3(hpspmm::kBlock), 0, st, p->lay,
+                           p->d_rvptr, p->d_coldptr, p->d_vcol, v, p->d_vsrc, p->d_vrow, B, p->d_bhot, p->d_partial,
+                           p->d_carry, C, first);
+      else if (p->d_vsrc)  // column-range slices, values bound: the plan's own copy of them, still no compact buffer
+        hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false, false>), grid, dim3(hpspmm::kBlock), 0, st, p->lay,
+                           p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval, (const int32_t*)nullptr, p->d_vrow, B,
+                           p->d_bhot, p->d_partial, p->d_carry, C, first);
+      else
+        hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false, true>), grid, dim3(hpspmm::kBlock), 0, st, p->lay,
+                           p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval, (const int32_t*)nullptr, p->d_vrow, B,
+                           p->d_bhot, p->d_partial, p->d_carry, C, first);
+      mark_launch(st, !split ? "spmm_routed_kernel" : part < p->lay.nsub ? "spmm_routed_kernel(hub phase)"
+                                                                          : "spmm_routed_kernel(cold class)");
+    }
   }
   const int64_t routed_blocks = row_blocks(p->lay.n_routed, K);
   const int64_t cross_blocks = row_blocks(p->n_cross, K);
@@ -1139,31 +1297,32 @@ constexpr double kHubMinShare = 0.25;
 // Picks the most referenced columns of A (by nonzero count; ties by lower index, so
 // the choice is reproducible), gives each a slot in a compact copy of B and
 // rewrites the column array accordingly.  log2_hubs = 0 picks the default size.
-int build_hub_cache(hpspmm_plan* p, const int32_t* d_col, int log2_hubs, bool forced, hipStream_t st) {
+int build_hub_cache(hpspmm_plan* p, const int32_t* d_col, int log2_hubs, bool forced, ColumnRanking& rk,
+                    hipStream_t st) {
   if (log2_hubs == 0) log2_hubs = 16;
   if (log2_hubs < 4 || log2_hubs > 24) return fail(HPSPMM_ERR_INVALID_ARG, "hub cache size 2^%d outside [2^4, 2^24]", log2_hubs);
-  std::vector<int32_t> count, ids;
-  if (int rc = rank_columns(p, d_col, (int64_t)1 << log2_hubs, st, count, ids)) return rc;
-  if (ids.empty()) return HPSPMM_OK;
   if (!forced) {
-    // worth the extra column array only when the cached rows serve a good part of the gathers
-    int64_t served = 0;
-    for (int32_t c : ids) served += count[c];
-    if ((double)served < kHubMinShare * (double)p->nnz) return HPSPMM_OK;
+    double estimate = 1.0;
+    if (int rc = estimate_hot_share(p, d_col, (int64_t)1 << log2_hubs, st, &estimate)) return rc;
+    if (estimate < kHubMinShare * kRoutedEstimateMargin) return HPSPMM_OK;
   }
-  std::vector<int32_t> colmap((size_t)p->cols, -1);
-  for (size_t s = 0; s < ids.size(); ++s) colmap[ids[s]] = (int32_t)s;
+  if (int rc = rank_columns(p, d_col, (int64_t)1 << log2_hubs, st, rk)) return rc;
+  if (rk.n_ids == 0) return HPSPMM_OK;
+  // worth the extra column array only when the cached rows serve a good part of the gathers
+  if (!forced && (double)rk.served < kHubMinShare * (double)p->nnz) return HPSPMM_OK;
 
-  const int64_t n_hub = (int64_t)ids.size();
+  const int64_t n_hub = rk.n_ids;
   HPSPMM_HIP(hipMalloc(&p->d_hub_ids, (size_t)n_hub * sizeof(int32_t)));
   HPSPMM_HIP(hipMalloc(&p->d_hub_col, (size_t)p->nnz * sizeof(int32_t)));
   HPSPMM_HIP(hipMalloc(&p->d_bhot, (size_t)n_hub * (size_t)p->k * sizeof(float)));
   p->workspace_bytes += n_hub * 4 + p->nnz * 4 + n_hub * p->k * 4;
-  HPSPMM_HIP(hipMemcpyAsync(p->d_hub_ids, ids.data(), (size_t)n_hub * sizeof(int32_t), hipMemcpyHostToDevice, st));
+  HPSPMM_HIP(hipMemcpyAsync(p->d_hub_ids, rk.d_ids, (size_t)n_hub * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
   int32_t* d_colmap = nullptr;
-  HPSPMM_HIP(hipMalloc(&d_colmap, colmap.size() * sizeof(int32_t)));
-  hipError_t e = hipMemcpyAsync(d_colmap, colmap.data(), colmap.size() * sizeof(int32_t), hipMemcpyHostToDevice, st);
+  HPSPMM_HIP(hipMalloc(&d_colmap, (size_t)p->cols * sizeof(int32_t)));
+  hipError_t e = hipMemsetAsync(d_colmap, 0xFF, (size_t)p->cols * sizeof(int32_t), st);
   if (e == hipSuccess) {
+    hipLaunchKernelGGL(hpspmm::hot_index_kernel, dim3((unsigned)ceil_div(n_hub, hpspmm::kBlock)), dim3(hpspmm::kBlock), 0,
+                       st, (int32_t)n_hub, rk.d_ids, d_colmap);
     hipLaunchKernelGGL(hpspmm::remap_columns_kernel, dim3(grid_for(p->nnz, 1 << 16)), dim3(hpspmm::kBlock), 0, st,
                        p->nnz, d_col, d_colmap, p->d_hub_col);
     e = hipStreamSynchronize(st);
@@ -1250,6 +1409,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   // Automatic choice, in this order: tiny matrix -> rows; a matrix in the rows strategy's range
   // (`rows_range`) -> ordered if it has communities, else rows; beyond that range -> routed if a
   // few columns take most of the nonzeros, else ordered if it has communities, else segments.
+  ColumnRanking ranking;         // column popularity, shared by the routed and the hub-cache decisions
   bool rows_need_tiles = false;  // rows strategy chosen on the strength of the row tiles
   bool rows_range = false;       // provisional segments; rows unless the ordered strategy qualifies
   if (!fast_k(k) && !anyk_k(k)) {
@@ -1335,7 +1495,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
                               (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 16) & 0x1Fu) : 0,
                               (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 24) & 0x1Fu) : 0,
                               (flags & HPSPMM_PLAN_FORCE_ROUTED) ? (int)((flags >> 29) & 0x7u) : 0,
-                              (flags & HPSPMM_PLAN_ROUTED_SORT_VALUES) != 0, st)) {
+                              (flags & HPSPMM_PLAN_ROUTED_SORT_VALUES) != 0, ranking, st)) {
       return rc;
     }
   }
@@ -1376,7 +1536,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     }
   }
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && !(flags & HPSPMM_PLAN_NO_HUB_CACHE) && nnz > 0) {
-    if (int rc = build_hub_cache(p, d_col, (int)((flags >> 16) & 0x1Fu), (flags & HPSPMM_PLAN_HUB_CACHE) != 0, st)) {
+    if (int rc = build_hub_cache(p, d_col, (int)((flags >> 16) & 0x1Fu), (flags & HPSPMM_PLAN_HUB_CACHE) != 0, ranking, st)) {
       return rc;
     }
   }
@@ -1419,10 +1579,6 @@ static int plan_create_guarded(int64_t rows, int64_t cols, int64_t nnz, const in
   } catch (const std::exception& e) {
     if (plan_out) *plan_out = nullptr;
     rc = fail(HPSPMM_ERR_ALLOC, "plan construction failed: %s", e.what());
-  }
-  try {
-    g_rank_cache = RankCache{};  // a later plan may get the same address
-  } catch (...) {
   }
   return rc;
 }

@@ -1,0 +1,137 @@
+// Plan-time device code: column popularity ranking.
+//
+// Several strategies want the `want` most referenced columns of A in order of decreasing nonzero
+// count (ties by lower index, so that the choice is reproducible).  Everything happens on the
+// device: a histogram of the column indices, a radix select of the want-th largest count (four
+// passes over the counters, 8 bits each), a stable compaction of the selected columns (flags, scan,
+// scatter: ties in index order) and a rank-by-counting sort of the at most 2^17 selected keys.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "spmm_kernels.hpp"
+
+namespace hpspmm {
+
+// count[col[j]] += 1 for every `stride`-th nonzero (count[] zeroed by the caller); stride 1 = all.
+__global__ __launch_bounds__(kBlock) void count_columns_strided_kernel(int64_t nnz, int64_t stride,
+                                                                       const int32_t* __restrict__ col,
+                                                                       int32_t* __restrict__ count) {
+  const int64_t n = (nnz + stride - 1) / stride;
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step) atomicAdd(&count[col[i * stride]], 1);
+}
+
+// hist[b] += number of counters whose bits above `shift + 8` equal those of `prefix` and whose byte
+// at `shift` is b (hist[256] zeroed by the caller).  With shift = 24 every counter takes part.
+__global__ __launch_bounds__(kBlock) void select_histogram_kernel(int64_t n, const int32_t* __restrict__ count,
+                                                                  uint32_t prefix, int shift,
+                                                                  uint32_t* __restrict__ hist) {
+  __shared__ uint32_t s_hist[256];
+  s_hist[threadIdx.x] = 0;
+  __syncthreads();
+  const uint32_t high_mask = shift >= 24 ? 0u : ~((1u << (shift + 8)) - 1u);
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step) {
+    const uint32_t v = (uint32_t)count[i];
+    if ((v & high_mask) == (prefix & high_mask)) atomicAdd(&s_hist[(v >> shift) & 255u], 1u);
+  }
+  __syncthreads();
+  if (s_hist[threadIdx.x]) atomicAdd(&hist[threadIdx.x], s_hist[threadIdx.x]);
+}
+
+// above[i] = count[i] > threshold, equal[i] = count[i] == threshold (i < n); both get a trailing 0 at n
+// so that their exclusive scans end in the totals.
+__global__ __launch_bounds__(kBlock) void select_flags_kernel(int64_t n, const int32_t* __restrict__ count,
+                                                              int32_t threshold, uint32_t* __restrict__ above,
+                                                              uint32_t* __restrict__ equal) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i > n) return;
+  const int32_t c = i < n ? count[i] : INT32_MIN;
+  above[i] = c > threshold ? 1u : 0u;
+  equal[i] = (i < n && c == threshold) ? 1u : 0u;
+}
+
+// The selected columns in index order: every column above the threshold, then the first `ties`
+// columns at the threshold.  key = (~count << 32) | index sorts by decreasing count, then index.
+__global__ __launch_bounds__(kBlock) void select_compact_kernel(int64_t n, const int32_t* __restrict__ count,
+                                                                int32_t threshold,
+                                                                const uint32_t* __restrict__ above_scan,
+                                                                const uint32_t* __restrict__ equal_scan,
+                                                                uint32_t n_above, uint32_t ties,
+                                                                unsigned long long* __restrict__ keys) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  const int32_t c = count[i];
+  int64_t slot = -1;
+  if (c > threshold) slot = above_scan[i];
+  else if (c == threshold && equal_scan[i] < ties) slot = (int64_t)n_above + equal_scan[i];
+  if (slot >= 0) keys[slot] = ((unsigned long long)(~(uint32_t)c) << 32) | (uint32_t)i;
+}
+
+// ids[rank of key i] = low word of key i, rank = number of smaller keys (keys are distinct).  One
+// thread per key, the keys passed through LDS in tiles; m <= 2^17 keeps the m^2 compares cheap.
+// *served += the counts of the ranked columns.
+__global__ __launch_bounds__(kBlock) void rank_sort_kernel(int32_t m, const unsigned long long* __restrict__ keys,
+                                                           int32_t* __restrict__ ids,
+                                                           unsigned long long* __restrict__ served) {
+  __shared__ unsigned long long s_keys[kBlock];
+  const int32_t i = (int32_t)blockIdx.x * kBlock + threadIdx.x;
+  const unsigned long long mine = i < m ? keys[i] : ~0ull;
+  int32_t rank = 0;
+  for (int32_t t0 = 0; t0 < m; t0 += kBlock) {
+    __syncthreads();
+    s_keys[threadIdx.x] = t0 + (int32_t)threadIdx.x < m ? keys[t0 + threadIdx.x] : ~0ull;
+    __syncthreads();
+    const int32_t cnt = m - t0 < kBlock ? m - t0 : kBlock;
+    for (int32_t q = 0; q < cnt; ++q) rank += s_keys[q] < mine ? 1 : 0;
+  }
+  unsigned long long c = 0;
+  if (i < m) {
+    ids[rank] = (int32_t)(uint32_t)mine;
+    c = (unsigned long long)(~(uint32_t)(mine >> 32));
+  }
+  for (int off = 32; off > 0; off >>= 1) c += __shfl_down(c, off);
+  if ((threadIdx.x & 63) == 0 && c) atomicAdd(served, c);
+}
+
+// Popularity rank s -> compact-buffer slot (s % slices) * per_slice + s / slices:
+// colmap[ids[s]] = slot, slot_src[slot] = ids[s] (both preset to -1 by the caller).
+__global__ __launch_bounds__(kBlock) void hot_slots_kernel(int32_t m, const int32_t* __restrict__ ids, int slices,
+                                                           int32_t per_slice, int32_t* __restrict__ colmap,
+                                                           int32_t* __restrict__ slot_src) {
+  const int32_t s = (int32_t)blockIdx.x * kBlock + threadIdx.x;
+  if (s >= m) return;
+  const int32_t slot = (s % slices) * per_slice + s / slices;
+  colmap[ids[s]] = slot;
+  slot_src[slot] = ids[s];
+}
+
+// colmap[ids[s]] = s.
+__global__ __launch_bounds__(kBlock) void hot_index_kernel(int32_t m, const int32_t* __restrict__ ids,
+                                                           int32_t* __restrict__ colmap) {
+  const int32_t s = (int32_t)blockIdx.x * kBlock + threadIdx.x;
+  if (s < m) colmap[ids[s]] = s;
+}
+
+// Column ranges of equal nonzero count: range[c] = min(groups - 1, (nonzeros in columns < c) / target),
+// from the exclusive scan of the column counts.
+__global__ __launch_bounds__(kBlock) void column_range_kernel(int64_t cols, const uint32_t* __restrict__ before,
+                                                              int64_t target, int groups,
+                                                              uint8_t* __restrict__ range) {
+  const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (c >= cols) return;
+  const int64_t r = (int64_t)before[c] / target;
+  range[c] = (uint8_t)(r < groups - 1 ? r : groups - 1);
+}
+
+// hot[range[ids[s]]] += 1 (hot[] zeroed by the caller; at most 56 ranges).
+__global__ __launch_bounds__(kBlock) void range_hot_count_kernel(int32_t m, const int32_t* __restrict__ ids,
+                                                                 const uint8_t* __restrict__ range,
+                                                                 uint32_t* __restrict__ hot) {
+  const int32_t s = (int32_t)blockIdx.x * kBlock + threadIdx.x;
+  if (s < m) atomicAdd(&hot[range[ids[s]]], 1u);
+}
+
+}  // namespace hpspmm

@@ -500,7 +500,8 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
                                                              const float* __restrict__ B,
                                                              const float* __restrict__ Bhot,
                                                              float* __restrict__ partial,
-                                                             float* __restrict__ carry, float* __restrict__ C) {
+                                                             float* __restrict__ carry, float* __restrict__ C,
+                                                             int64_t first_block) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
   constexpr int TL = kTile / G;
@@ -508,10 +509,13 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
   __shared__ __attribute__((aligned(16))) float s_val[kWavesPerBlock * P * kTileStride];
   __shared__ __attribute__((aligned(16))) int32_t s_row[kWavesPerBlock * P * kTileStride];
 
+  // first_block: 0 in an ordinary launch; a diagnostic launch of one part of the grid passes the
+  // number of its first workgroup (a multiple of 8, so that the workgroup -> XCD dealing is kept)
+  const int64_t bid = (int64_t)blockIdx.x + first_block;
   const int nhub = lay.nhub;
   int p = 0;
-  while (p < lay.nsub && (int64_t)blockIdx.x >= lay.phase_begin[p + 1]) ++p;
-  const int64_t rel = (int64_t)blockIdx.x - lay.phase_begin[p];
+  while (p < lay.nsub && bid >= lay.phase_begin[p + 1]) ++p;
+  const int64_t rel = bid - lay.phase_begin[p];
   const bool hub = p < lay.nsub;
   int x;
   int64_t i;

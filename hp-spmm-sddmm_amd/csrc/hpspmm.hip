@@ -608,8 +608,10 @@ int count_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t stride, hi
     (void)hipFree(d_count);
     return fail(HPSPMM_ERR_HIP, "hipMemsetAsync: %s", hipGetErrorString(e));
   }
-  hipLaunchKernelGGL(hpspmm::count_columns_strided_kernel, dim3(grid_for(ceil_div(p->nnz, stride), 1 << 16)),
-                     dim3(hpspmm::kBlock), 0, st, p->nnz, stride, d_col, d_count);
+  const int64_t chunks = ceil_div(ceil_div(p->nnz, stride), hpspmm::kCountChunk);
+  if (chunks > 0)
+    hipLaunchKernelGGL(hpspmm::count_columns_strided_kernel, dim3((unsigned)chunks), dim3(hpspmm::kBlock), 0, st,
+                       p->nnz, stride, d_col, d_count);
   *d_count_out = d_count;
   return HPSPMM_OK;
 }
@@ -851,14 +853,15 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   uint8_t* d_action = nullptr;    // [rows]
   int32_t* d_counts = nullptr;    // [2] list lengths
   int32_t* d_vpos = nullptr;      // [nnz] position of every stored nonzero in the class-major order
+  int32_t* d_rlist = nullptr;     // [n_routed] row of every routed-row number
   struct Guard {
-    void** q[9];
+    void** q[10];
     ~Guard() {
       for (void** x : q)
         if (*x) (void)hipFree(*x);
     }
   } guard{{(void**)&d_colmap, (void**)&d_ridx, (void**)&d_cnt, (void**)&d_coldcnt, (void**)&d_action,
-           (void**)&d_counts, (void**)&d_vpos, (void**)&d_colrange, (void**)&d_bhot_src_tmp}};
+           (void**)&d_counts, (void**)&d_vpos, (void**)&d_colrange, (void**)&d_bhot_src_tmp, (void**)&d_rlist}};
 
   bool inplace = false;
   if (!sort_values && nsub == 1 && nnz > 0 && p->cols * k * 4 < ((int64_t)1 << 32) && p->d_nnz_row &&
@@ -922,13 +925,18 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   HPSPMM_HIP(hipStreamSynchronize(st));
   const int64_t n_routed = n_routed_u;
 
-  // per-row class counts and their scans
+  // per-row class counts and their scans: a wavefront per routed row, a thread per short row
   const int64_t ncnt = (int64_t)nhub * n_routed + 1;
   HPSPMM_HIP(hipMalloc(&d_cnt, (size_t)ncnt * sizeof(uint32_t)));
-  const unsigned row_grid = (unsigned)ceil_div(rows, hpspmm::kWavesPerBlock);
-  hipLaunchKernelGGL(hpspmm::routed_count_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, n_routed,
-                     d_rowptr, d_col, d_colmap, d_ridx, (int32_t)h, nsub, (const uint8_t*)d_colrange, min_row_nnz, d_cnt,
-                     d_coldcnt);
+  HPSPMM_HIP(hipMalloc(&d_rlist, (size_t)std::max<int64_t>(n_routed, 1) * sizeof(int32_t)));
+  const unsigned thread_per_row_grid = (unsigned)ceil_div(rows + 1, hpspmm::kBlock);
+  const unsigned routed_grid = (unsigned)std::max<int64_t>(1, ceil_div(n_routed, hpspmm::kWavesPerBlock));
+  hipLaunchKernelGGL(hpspmm::routed_list_kernel, dim3(thread_per_row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr,
+                     min_row_nnz, d_ridx, d_rlist);
+  hipLaunchKernelGGL(hpspmm::routed_cold_count_kernel, dim3(thread_per_row_grid), dim3(hpspmm::kBlock), 0, st, rows,
+                     d_rowptr, min_row_nnz, d_coldcnt);
+  hipLaunchKernelGGL(hpspmm::routed_count_kernel, dim3(routed_grid), dim3(hpspmm::kBlock), 0, st, n_routed, d_rlist,
+                     d_rowptr, d_col, d_colmap, (int32_t)h, nsub, (const uint8_t*)d_colrange, min_row_nnz, d_cnt);
   if (int rc = exclusive_scan_u32(d_cnt, d_cnt, ncnt, st)) return rc;
   if (int rc = exclusive_scan_u32(d_coldcnt, d_coldcnt, rows + 1, st)) return rc;
 
@@ -987,8 +995,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   const size_t bhot_bytes = (size_t)n_bhot * (size_t)k * sizeof(float);
   const size_t list_bytes = (size_t)std::max<int64_t>(rows, 1) * sizeof(int32_t);
   const size_t routed_rows_bytes = (size_t)std::max<int64_t>(n_routed, 1) * sizeof(int32_t);
-  // the segments strategy's buffers are not needed any more
-  if (p->d_nnz_row) { (void)hipFree(p->d_nnz_row); p->d_nnz_row = nullptr; }
+  // the segments strategy's carry slots are not needed any more (the row of every nonzero is, for the fill)
   if (p->d_carry) { (void)hipFree(p->d_carry); p->d_carry = nullptr; }
   const size_t total_bytes = rvptr_bytes + coldptr_bytes + 3 * v_bytes +
                              (inplace ? 0 : lslot_bytes + 2 * chunk_bytes) + partial_bytes + carry_bytes +
@@ -1023,9 +1030,16 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
                      0, st, lay, d_cnt, p->d_rvptr);
   hipLaunchKernelGGL(hpspmm::routed_coldptr_kernel, dim3((unsigned)ceil_div(rows + 1, hpspmm::kBlock)),
                      dim3(hpspmm::kBlock), 0, st, rows, lay.cls_begin[nhub], d_coldcnt, p->d_coldptr);
-  hipLaunchKernelGGL(hpspmm::routed_fill_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col,
-                     d_colmap, d_ridx, (int32_t)h, nsub, (const uint8_t*)d_colrange, min_row_nnz, p->d_rvptr,
-                     p->d_coldptr, p->d_vcol, d_vpos, p->d_vsrc, p->d_vrow, p->d_routed_rows, d_action, p->shift);
+  HPSPMM_HIP(hipMemcpyAsync(p->d_routed_rows, d_rlist, (size_t)n_routed * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
+  hipLaunchKernelGGL(hpspmm::routed_fill_kernel, dim3(routed_grid), dim3(hpspmm::kBlock), 0, st, n_routed, d_rlist,
+                     d_rowptr, d_col, d_colmap, (int32_t)h, nsub, (const uint8_t*)d_colrange, min_row_nnz, p->d_rvptr,
+                     p->d_vcol, d_vpos, p->d_vsrc, p->d_vrow);
+  if (nnz > 0)
+    hipLaunchKernelGGL(hpspmm::routed_fill_cold_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)),
+                       dim3(hpspmm::kBlock), 0, st, nnz, p->d_nnz_row, d_rowptr, d_col, d_colmap, min_row_nnz,
+                       p->d_coldptr, p->d_vcol, d_vpos, p->d_vsrc, p->d_vrow);
+  hipLaunchKernelGGL(hpspmm::routed_action_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                     0, st, rows, d_rowptr, min_row_nnz, p->d_coldptr, p->shift, d_action);
   // chunk tables of the value scatter
   if (nchunks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   if (!inplace)
@@ -1043,6 +1057,8 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   HPSPMM_HIP(hipGetLastError());
   p->n_cross = counts[0];
   p->n_zero = counts[1];
+  (void)hipFree(p->d_nnz_row);  // the row of every nonzero was the segments strategy's; the class-major arrays replace it
+  p->d_nnz_row = nullptr;
   p->n_bhot = inplace ? 0 : n_bhot;
   p->n_hub = inplace ? 0 : (int64_t)n_ids;
   p->nseg = nseg;
@@ -1241,7 +1257,7 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
                      0, st, rows, d_label);
   for (int sweep = 0; sweep < kClusterMaxSweeps; ++sweep) {
     HPSPMM_HIP(hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st));
-    hipLaunchKernelGGL(hpspmm::cluster_sweep_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
+    hipLaunchKernelGGL(hpspmm::cluster_sweep_kernel, dim3((unsigned)ceil_div(ceil_div(rows, 2), hpspmm::kWavesPerBlock)),
                        dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_label, d_label_next, (uint32_t)sweep,
                        d_changed);
     std::swap(d_label, d_label_next);

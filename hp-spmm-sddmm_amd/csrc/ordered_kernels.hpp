@@ -43,12 +43,13 @@ namespace hpspmm {
 // changes with the sweep, except that a row keeps its label when that is among
 // the most frequent.  A sweep reads label_in and writes label_out (two buffers,
 // so the outcome does not depend on the order in which the wavefronts run: two
-// plans of one matrix get the same labels), and only a pseudo-random half of the
-// rows - another half in every sweep - may change: with every row updated at
-// once from the old labels, neighbours swap labels back and forth instead of
-// settling.  One wavefront per row; the 64 sampled labels are sorted by a bitonic
-// network of wavefront shuffles.  The kClusterCounters entries of changed[]
-// together count the rows whose label changed.
+// plans of one matrix get the same labels), and only half of the rows may
+// change - of every pair of rows (2w, 2w + 1) the one a hash of w and the sweep
+// picks: with every row updated at once from the old labels, neighbours swap
+// labels back and forth instead of settling.  One wavefront per pair (it copies
+// the label of the row that sits the sweep out); the 64 sampled labels are
+// sorted by a bitonic network of wavefront shuffles.  The kClusterCounters
+// entries of changed[] together count the rows whose label changed.
 constexpr int kClusterCounters = 1024;
 __global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                const int32_t* __restrict__ col,
@@ -56,13 +57,16 @@ __global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, con
                                                                int32_t* __restrict__ label_out, uint32_t sweep,
                                                                uint32_t* __restrict__ changed) {
   const int lane = threadIdx.x & 63;
-  const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-  if (r >= rows) return;
+  const int64_t w = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (2 * w >= rows) return;
+  const uint32_t turn = (((uint32_t)w * 0x9E3779B1u) ^ ((sweep + 1u) * 0x85EBCA6Bu)) * 0xC2B2AE35u;
+  const int64_t r = 2 * w + (int64_t)((turn >> 31) & 1u) < rows ? 2 * w + (int64_t)((turn >> 31) & 1u) : 2 * w;
+  const int64_t idle = r ^ 1;  // the other row of the pair keeps its label in this sweep
+  if (lane == 1 && idle < rows) label_out[idle] = label_in[idle];
   const int32_t mine = label_in[r];
   const int32_t lb = rowptr[r];
   const int32_t n = rowptr[r + 1] - lb;
-  const uint32_t turn = (((uint32_t)r * 0x9E3779B1u) ^ ((sweep + 1u) * 0x85EBCA6Bu)) * 0xC2B2AE35u;
-  if (n == 0 || ((turn >> 31) & 1u)) {  // wavefront-uniform
+  if (n == 0) {  // wavefront-uniform
     if (lane == 0) label_out[r] = mine;
     return;
   }
@@ -213,89 +217,99 @@ __global__ __launch_bounds__(kBlock) void ordered_fill_kernel(int64_t rows, cons
 // frequent of them (ties: an occurrence count is either kept whole or dropped
 // whole), in increasing column order -> wcols[w * cap + slot] (-1 = unused
 // slot); the nonzeros of those columns get ocol = ~slot.  One workgroup per
-// window: bitonic sort of the window's columns in LDS, run lengths, a
-// threshold on the run length, compaction.  served[0] += rewritten nonzeros.
+// window.  Most columns of a window occur once, so two bitmaps first tell which
+// hash values were seen twice; only those nonzeros are counted exactly, in an LDS
+// hash table (as many slots as a window has nonzeros: it cannot overflow);
+// then a histogram of the counts, a threshold, the compaction of the selected
+// columns and a bitonic sort of those few.  Every step depends only on the set
+// of the window's columns, not on the order the threads run in: the same plan
+// every time.  served[0] += rewritten nonzeros.
 constexpr int kOrderedMaxWindow = 8192;
-constexpr int kOrderedHistMax = 65;  // run lengths are told apart up to this one
+constexpr int kOrderedHistMax = 65;       // occurrence counts are told apart up to this one
+constexpr int kOrderedBitmapWords = 1024;  // 32768 bits per bitmap
+constexpr int kOrderedMaxCap = 512;        // LDS slots a window can ask for, at most
 
 __global__ __launch_bounds__(kBlock) void ordered_hot_kernel(int64_t nnz, int window, int cap,
                                                              int32_t* __restrict__ ocol,
                                                              int32_t* __restrict__ wcols,
                                                              unsigned long long* __restrict__ served) {
-  __shared__ int32_t s_key[kOrderedMaxWindow];   // the window's columns, sorted (INT32_MAX pads)
-  __shared__ int32_t s_sel[kOrderedMaxWindow / 2];  // selected columns (each occurs >= 2 times)
+  __shared__ uint32_t s_once[kOrderedBitmapWords];
+  __shared__ uint32_t s_twice[kOrderedBitmapWords];
+  __shared__ int32_t s_key[kOrderedMaxWindow];        // hash table: column, -1 = free
+  __shared__ uint32_t s_cnt[kOrderedMaxWindow / 2];   // two 16-bit occurrence counts per word
+  __shared__ int32_t s_sel[kOrderedMaxCap];           // selected columns
+  __shared__ int32_t s_hist[kOrderedHistMax + 1];     // s_hist[t] = columns that occur >= t times, t in [2, kOrderedHistMax]
   __shared__ int32_t s_count;
-  __shared__ int32_t s_scan[kBlock];
-  __shared__ int32_t s_hist[kOrderedHistMax + 1];  // s_hist[t] = runs of length >= t, t in [2, kOrderedHistMax]
   const int tid = threadIdx.x;
   const int64_t w = blockIdx.x;
   const int64_t p0 = w * window;
   const int n = nnz - p0 < window ? (int)(nnz - p0) : window;
-  int npow = 1;
-  while (npow < n) npow <<= 1;
-  for (int i = tid; i < npow; i += kBlock) s_key[i] = i < n ? ocol[p0 + i] : INT32_MAX;
+  for (int i = tid; i < kOrderedBitmapWords; i += kBlock) {
+    s_once[i] = 0;
+    s_twice[i] = 0;
+  }
+  for (int i = tid; i < kOrderedMaxWindow; i += kBlock) s_key[i] = -1;
+  for (int i = tid; i < kOrderedMaxWindow / 2; i += kBlock) s_cnt[i] = 0;
   for (int i = tid; i <= kOrderedHistMax; i += kBlock) s_hist[i] = 0;
+  for (int i = tid; i < kOrderedMaxCap; i += kBlock) s_sel[i] = INT32_MAX;
   if (tid == 0) s_count = 0;
   __syncthreads();
-  for (int size = 2; size <= npow; size <<= 1) {
+  auto bit_of = [](int32_t c) { return ((uint32_t)c * 0x9E3779B1u) >> 17; };  // 15 bits
+  for (int i = tid; i < n; i += kBlock) {
+    const uint32_t h = bit_of(ocol[p0 + i]);
+    const uint32_t m = 1u << (h & 31);
+    if (atomicOr(&s_once[h >> 5], m) & m) atomicOr(&s_twice[h >> 5], m);
+  }
+  __syncthreads();
+  // exact counts of the columns whose hash value was seen twice
+  for (int i = tid; i < n; i += kBlock) {
+    const int32_t c = ocol[p0 + i];
+    const uint32_t h = bit_of(c);
+    if (!((s_twice[h >> 5] >> (h & 31)) & 1u)) continue;
+    uint32_t slot = ((uint32_t)c * 0x85EBCA6Bu) >> 19;  // 13 bits
+    for (;;) {
+      const int32_t seen = atomicCAS(&s_key[slot], -1, c);
+      if (seen == -1 || seen == c) break;
+      slot = (slot + 1) & (kOrderedMaxWindow - 1);
+    }
+    atomicAdd(&s_cnt[slot >> 1], 1u << (16 * (slot & 1)));
+  }
+  __syncthreads();
+  auto count_of = [&](int slot) { return (int)((s_cnt[slot >> 1] >> (16 * (slot & 1))) & 0xFFFFu); };
+  for (int i = tid; i < kOrderedMaxWindow; i += kBlock) {
+    const int len = s_key[i] >= 0 ? count_of(i) : 0;
+    if (len >= 2) atomicAdd(&s_hist[len < kOrderedHistMax ? len : kOrderedHistMax], 1);
+  }
+  __syncthreads();
+  if (tid == 0)  // s_hist[t] = columns with exactly t occurrences  ->  with at least t
+    for (int t = kOrderedHistMax - 1; t >= 2; --t) s_hist[t] += s_hist[t + 1];
+  __syncthreads();
+  const int limit = cap < kOrderedMaxCap ? cap : kOrderedMaxCap;
+  int threshold = 2;
+  while (threshold < kOrderedHistMax && s_hist[threshold] > limit) ++threshold;
+  const bool fits = s_hist[threshold] <= limit;  // always, as long as cap >= window / kOrderedHistMax
+  if (fits) {
+    for (int i = tid; i < kOrderedMaxWindow; i += kBlock)
+      if (s_key[i] >= 0 && count_of(i) >= threshold) s_sel[atomicAdd(&s_count, 1)] = s_key[i];
+  }
+  __syncthreads();
+  const int m = s_count;
+  // the selected columns in increasing order (unused entries hold INT32_MAX and sort behind them)
+  for (int size = 2; size <= kOrderedMaxCap; size <<= 1) {
     for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      for (int i = tid; i < npow / 2; i += kBlock) {
+      for (int i = tid; i < kOrderedMaxCap / 2; i += kBlock) {
         const int lo = ((i / stride) * stride * 2) + (i % stride);
         const int hi = lo + stride;
         const bool up = ((lo & size) == 0);
-        const int32_t a = s_key[lo], b = s_key[hi];
+        const int32_t a = s_sel[lo], b = s_sel[hi];
         if ((a > b) == up) {
-          s_key[lo] = b;
-          s_key[hi] = a;
+          s_sel[lo] = b;
+          s_sel[hi] = a;
         }
       }
       __syncthreads();
     }
   }
-  // run heads: position i starts a run if it differs from its predecessor
-  auto run_length = [&](int i) {
-    int len = 1;
-    while (i + len < n && s_key[i + len] == s_key[i]) ++len;
-    return len;
-  };
-  // every thread owns a contiguous stretch of the sorted window
-  const int per = (npow + kBlock - 1) / kBlock;
-  const int i_begin = tid * per < n ? tid * per : n;
-  const int i_end = i_begin + per < n ? i_begin + per : n;
-  for (int i = i_begin; i < i_end; ++i) {
-    if (i > 0 && s_key[i] == s_key[i - 1]) continue;
-    const int len = run_length(i);
-    if (len >= 2) atomicAdd(&s_hist[len < kOrderedHistMax ? len : kOrderedHistMax], 1);
-  }
-  __syncthreads();
-  if (tid == 0)  // s_hist[t] = runs of exactly t  ->  runs of at least t
-    for (int t = kOrderedHistMax - 1; t >= 2; --t) s_hist[t] += s_hist[t + 1];
-  __syncthreads();
-  int threshold = 2;
-  while (threshold < kOrderedHistMax && s_hist[threshold] > cap) ++threshold;
-  const bool fits = s_hist[threshold] <= cap;  // always, as long as cap >= window / kOrderedHistMax
-  // selection in column order: count per stretch, exclusive scan over the threads, write
-  int mine_sel = 0;
-  for (int i = i_begin; i < i_end && fits; ++i) {
-    if (i > 0 && s_key[i] == s_key[i - 1]) continue;
-    if (run_length(i) >= threshold) ++mine_sel;
-  }
-  s_scan[tid] = mine_sel;
-  __syncthreads();
-  for (int off = 1; off < kBlock; off <<= 1) {
-    const int add = tid >= off ? s_scan[tid - off] : 0;
-    __syncthreads();
-    s_scan[tid] += add;
-    __syncthreads();
-  }
-  int at = s_scan[tid] - mine_sel;
-  for (int i = i_begin; i < i_end && fits; ++i) {
-    if (i > 0 && s_key[i] == s_key[i - 1]) continue;
-    if (run_length(i) >= threshold) s_sel[at++] = s_key[i];
-  }
-  if (tid == kBlock - 1) s_count = s_scan[tid];
-  __syncthreads();
-  const int m = s_count;
   for (int i = tid; i < cap; i += kBlock) wcols[w * cap + i] = i < m ? s_sel[i] : -1;
   unsigned long long mine = 0;
   for (int i = tid; i < n; i += kBlock) {

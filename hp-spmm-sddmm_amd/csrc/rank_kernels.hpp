@@ -15,12 +15,47 @@
 namespace hpspmm {
 
 // count[col[j]] += 1 for every `stride`-th nonzero (count[] zeroed by the caller); stride 1 = all.
+// A column of a power-law graph receives up to 10^5 of these increments, and atomics on one address
+// are served one after the other (the 163k increments of R-MAT's hottest column alone took 12 ms).
+// So every workgroup first counts its stretch of kCountChunk sampled nonzeros in an LDS table
+// (open addressing by a hash of the column, a handful of probes; a nonzero that finds no slot goes
+// to memory directly) and then adds each table entry to memory once: the increments of a hot column
+// reach memory once per workgroup instead of once per nonzero.
+constexpr int kCountChunk = 1 << 15;
+constexpr int kCountSlots = 1 << 12;
+constexpr int kCountProbes = 4;
+
 __global__ __launch_bounds__(kBlock) void count_columns_strided_kernel(int64_t nnz, int64_t stride,
                                                                        const int32_t* __restrict__ col,
                                                                        int32_t* __restrict__ count) {
+  __shared__ int32_t s_key[kCountSlots];
+  __shared__ int32_t s_cnt[kCountSlots];
+  for (int i = threadIdx.x; i < kCountSlots; i += kBlock) {
+    s_key[i] = -1;
+    s_cnt[i] = 0;
+  }
+  __syncthreads();
   const int64_t n = (nnz + stride - 1) / stride;
-  const int64_t step = (int64_t)gridDim.x * kBlock;
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step) atomicAdd(&count[col[i * stride]], 1);
+  const int64_t i0 = (int64_t)blockIdx.x * kCountChunk;
+  const int64_t i1 = i0 + kCountChunk < n ? i0 + kCountChunk : n;
+  for (int64_t i = i0 + threadIdx.x; i < i1; i += kBlock) {
+    const int32_t c = col[i * stride];
+    uint32_t slot = ((uint32_t)c * 0x9E3779B1u) >> 20;  // 12 bits
+    bool placed = false;
+#pragma unroll
+    for (int probe = 0; probe < kCountProbes && !placed; ++probe) {
+      const int32_t seen = atomicCAS(&s_key[slot], -1, c);
+      if (seen == -1 || seen == c) {
+        atomicAdd(&s_cnt[slot], 1);
+        placed = true;
+      }
+      slot = (slot + 1) & (kCountSlots - 1);
+    }
+    if (!placed) atomicAdd(&count[c], 1);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < kCountSlots; i += kBlock)
+    if (s_cnt[i]) atomicAdd(&count[s_key[i]], s_cnt[i]);
 }
 
 // hist[b] += number of counters whose bits above `shift + 8` equal those of `prefix` and whose byte
@@ -126,12 +161,18 @@ __global__ __launch_bounds__(kBlock) void column_range_kernel(int64_t cols, cons
   range[c] = (uint8_t)(r < groups - 1 ? r : groups - 1);
 }
 
-// hot[range[ids[s]]] += 1 (hot[] zeroed by the caller; at most 56 ranges).
+// hot[range[ids[s]]] += 1 (hot[] zeroed by the caller; at most 64 ranges), through a workgroup's LDS
+// histogram: a few dozen counters would otherwise take every increment one after the other.
 __global__ __launch_bounds__(kBlock) void range_hot_count_kernel(int32_t m, const int32_t* __restrict__ ids,
                                                                  const uint8_t* __restrict__ range,
                                                                  uint32_t* __restrict__ hot) {
+  __shared__ uint32_t s_hot[64];
+  if (threadIdx.x < 64) s_hot[threadIdx.x] = 0;
+  __syncthreads();
   const int32_t s = (int32_t)blockIdx.x * kBlock + threadIdx.x;
-  if (s < m) atomicAdd(&hot[range[ids[s]]], 1u);
+  if (s < m) atomicAdd(&s_hot[range[ids[s]] & 63], 1u);
+  __syncthreads();
+  if (threadIdx.x < 64 && s_hot[threadIdx.x]) atomicAdd(&hot[threadIdx.x], s_hot[threadIdx.x]);
 }
 
 }  // namespace hpspmm

@@ -131,41 +131,54 @@ __global__ __launch_bounds__(kBlock) void routed_flag_kernel(int64_t rows, const
   flag[r] = r < rows && rowptr[r + 1] - rowptr[r] >= min_row_nnz ? 1u : 0u;
 }
 
-// One wavefront per row.  Routed row (number ridx[r]): cnt[x * n_routed +
-// ridx[r]] = its nonzeros in hub class x, coldcnt[r] = 0.  Short row:
-// coldcnt[r] = its nonzeros.  coldcnt[rows] = 0 and cnt[nhub * n_routed] = 0
-// (the scans' total slots) are written by the first wavefront.
-__global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t rows, int64_t n_routed,
+// routed_rows[ridx[r]] = r for every routed row (ridx = exclusive scan of the routed flags).
+__global__ __launch_bounds__(kBlock) void routed_list_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                             int32_t min_row_nnz, const uint32_t* __restrict__ ridx,
+                                                             int32_t* __restrict__ routed_rows) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r < rows && rowptr[r + 1] - rowptr[r] >= min_row_nnz) routed_rows[ridx[r]] = (int32_t)r;
+}
+
+// coldcnt[r] = nonzeros of row r if it is a short row, else 0 (r < rows); coldcnt[rows] = 0 (the
+// scan's total slot).  One thread per row: most rows of a large skewed matrix are short or empty.
+__global__ __launch_bounds__(kBlock) void routed_cold_count_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                                   int32_t min_row_nnz,
+                                                                   uint32_t* __restrict__ coldcnt) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r > rows) return;
+  uint32_t n = 0;
+  if (r < rows) {
+    const int32_t len = rowptr[r + 1] - rowptr[r];
+    if (len < min_row_nnz) n = (uint32_t)len;
+  }
+  coldcnt[r] = n;
+}
+
+// One wavefront per routed row (number i, row routed_rows[i]): cnt[x * n_routed + i] = its nonzeros
+// in hub class x.  cnt[nhub * n_routed] = 0 (the scan's total slot) is written by the first wavefront.
+__global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t n_routed,
+                                                              const int32_t* __restrict__ routed_rows,
                                                               const int32_t* __restrict__ rowptr,
                                                               const int32_t* __restrict__ col,
                                                               const int32_t* __restrict__ colmap,
-                                                              const uint32_t* __restrict__ ridx,
                                                               int32_t hub_rows_per_slice, int nsub,
                                                               const uint8_t* __restrict__ colrange,
-                                                              int32_t min_row_nnz, uint32_t* __restrict__ cnt,
-                                                              uint32_t* __restrict__ coldcnt) {
+                                                              int32_t min_row_nnz, uint32_t* __restrict__ cnt) {
   const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-  if (row >= rows) return;
+  const int64_t i = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   const int nhub = kSlices * nsub;
-  if (row == 0 && lane == 0) {
-    coldcnt[rows] = 0;
-    cnt[(int64_t)nhub * n_routed] = 0;
-  }
+  if (i == 0 && lane == 0) cnt[(int64_t)nhub * n_routed] = 0;
+  if (i >= n_routed) return;
+  const int64_t row = routed_rows[i];
   const int32_t lb = rowptr[row];
   const int32_t hb = rowptr[row + 1];
-  if (hb - lb < min_row_nnz) {
-    if (lane == 0) coldcnt[row] = (uint32_t)(hb - lb);
-    return;
-  }
-  if (lane == 0) coldcnt[row] = 0;
+  const bool single = hb - lb < kSinglePhaseFactor * min_row_nnz;
   uint32_t mine = 0;  // lane x < nhub accumulates the count of class x
   for (int32_t j0 = lb; j0 < hb; j0 += 64) {
     const int32_t j = j0 + lane;
     int cls = -1;
     if (j < hb) {
       const int32_t c = col[j];
-      const bool single = hb - lb < kSinglePhaseFactor * min_row_nnz;
       cls = colrange ? range_class_of(colrange[c], nsub, single)
                      : hub_class_of(c, colmap[c], hub_rows_per_slice, single ? 1 : nsub);
     }
@@ -174,7 +187,7 @@ __global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t rows, int6
       if (lane == x) mine += (uint32_t)__popcll(m);
     }
   }
-  if (lane < nhub) cnt[(int64_t)lane * n_routed + ridx[row]] = mine;
+  if (lane < nhub) cnt[(int64_t)lane * n_routed + i] = mine;
 }
 
 // Three-pass exclusive scan of uint32 (n up to 2^32, total < 2^32).
@@ -278,52 +291,28 @@ __global__ __launch_bounds__(kBlock) void routed_coldptr_kernel(int64_t rows, in
   coldptr[r] = (int32_t)(cold_begin + (int64_t)scanned[r]);
 }
 
-// Scatter the nonzeros into class-major order, keeping the stored order inside
-// every run.  One wavefront per row; positions in the hub classes from ballots.
-__global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+// Scatter the nonzeros of the routed rows into class-major order, keeping the stored order inside
+// every run.  One wavefront per routed row; positions in the hub classes from ballots.
+__global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t n_routed,
+                                                             const int32_t* __restrict__ routed_rows,
+                                                             const int32_t* __restrict__ rowptr,
                                                              const int32_t* __restrict__ col,
                                                              const int32_t* __restrict__ colmap,
-                                                             const uint32_t* __restrict__ ridx,
                                                              int32_t hub_rows_per_slice, int nsub,
                                                              const uint8_t* __restrict__ colrange,
                                                              int32_t min_row_nnz, const int32_t* __restrict__ rvptr,
-                                                             const int32_t* __restrict__ coldptr,
                                                              int32_t* __restrict__ vcol, int32_t* __restrict__ vpos,
                                                              int32_t* __restrict__ vsrc /* or NULL */,
-                                                             int32_t* __restrict__ vrow,
-                                                             int32_t* __restrict__ routed_rows,
-                                                             uint8_t* __restrict__ action, int shift) {
+                                                             int32_t* __restrict__ vrow) {
   const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-  if (row >= rows) return;
+  const int64_t i = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (i >= n_routed) return;
   const int nhub = kSlices * nsub;
+  const int64_t row = routed_rows[i];
   const int32_t lb = rowptr[row];
   const int32_t hb = rowptr[row + 1];
-  if (hb - lb < min_row_nnz) {
-    // everything goes to the cold class, in stored order
-    const int32_t start = coldptr[row];
-    if (lane == 0) {
-      uint8_t a = kActionNone;
-      if (hb == lb) a = kActionZero;
-      else if (((int64_t)start >> shift) != ((int64_t)(start + (hb - lb) - 1) >> shift)) a = kActionCross;
-      action[row] = a;
-    }
-    for (int32_t j = lb + lane; j < hb; j += 64) {
-      const int32_t c = col[j];
-      const int32_t mapped = colmap[c];
-      const int32_t pos = start + (j - lb);
-      vcol[pos] = mapped >= 0 ? ~mapped : c;  // ~compact-buffer row if the column is cached
-      vpos[j] = pos;
-      if (vsrc) vsrc[pos] = j;
-      vrow[pos] = (int32_t)row;
-    }
-    return;
-  }
-  const int32_t r = (int32_t)ridx[row];
-  if (lane == 0) {
-    action[row] = kActionNone;
-    routed_rows[r] = (int32_t)row;
-  }
+  const int32_t r = (int32_t)i;
+  const bool single = hb - lb < kSinglePhaseFactor * min_row_nnz;
   int32_t cursor = lane < nhub ? rvptr[(int64_t)r * nhub + lane] : 0;  // lane x: next slot of class x
   const uint64_t below = (1ull << lane) - 1ull;
   for (int32_t j0 = lb; j0 < hb; j0 += 64) {
@@ -331,7 +320,6 @@ __global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const
     const bool valid = j < hb;
     const int32_t c = valid ? col[j] : 0;
     const int32_t mapped = valid ? colmap[c] : -1;
-    const bool single = hb - lb < kSinglePhaseFactor * min_row_nnz;
     const int cls = !valid      ? -1
                     : colrange ? range_class_of(colrange[c], nsub, single)
                                : hub_class_of(c, mapped, hub_rows_per_slice, single ? 1 : nsub);
@@ -349,6 +337,51 @@ __global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t rows, const
       if (lane == x) cursor += (int32_t)__popcll(m);
     }
   }
+}
+
+// The nonzeros of the short rows go to the cold class in stored order.  One thread per nonzero
+// (nnz_row[j] = its row): a wavefront per row would idle on the millions of rows of a few nonzeros.
+__global__ __launch_bounds__(kBlock) void routed_fill_cold_kernel(int64_t nnz, const int32_t* __restrict__ nnz_row,
+                                                                  const int32_t* __restrict__ rowptr,
+                                                                  const int32_t* __restrict__ col,
+                                                                  const int32_t* __restrict__ colmap,
+                                                                  int32_t min_row_nnz,
+                                                                  const int32_t* __restrict__ coldptr,
+                                                                  int32_t* __restrict__ vcol,
+                                                                  int32_t* __restrict__ vpos,
+                                                                  int32_t* __restrict__ vsrc /* or NULL */,
+                                                                  int32_t* __restrict__ vrow) {
+  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (j >= nnz) return;
+  const int32_t row = nnz_row[j];
+  const int32_t lb = rowptr[row];
+  if (rowptr[row + 1] - lb >= min_row_nnz) return;
+  const int32_t c = col[j];
+  const int32_t mapped = colmap[c];
+  const int32_t pos = coldptr[row] + ((int32_t)j - lb);
+  vcol[pos] = mapped >= 0 ? ~mapped : c;  // ~compact-buffer row if the column is cached
+  vpos[j] = pos;
+  if (vsrc) vsrc[pos] = (int32_t)j;
+  vrow[pos] = row;
+}
+
+// What the final kernel has to do with every row: nothing (stored by the main kernel, or routed),
+// write zeros (no nonzeros), or add carry slots (a short row whose run crosses a segment boundary).
+__global__ __launch_bounds__(kBlock) void routed_action_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                               int32_t min_row_nnz,
+                                                               const int32_t* __restrict__ coldptr, int shift,
+                                                               uint8_t* __restrict__ action) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r >= rows) return;
+  const int32_t len = rowptr[r + 1] - rowptr[r];
+  uint8_t a = kActionNone;
+  if (len == 0) {
+    a = kActionZero;
+  } else if (len < min_row_nnz) {
+    const int64_t start = coldptr[r];
+    if ((start >> shift) != ((start + len - 1) >> shift)) a = kActionCross;
+  }
+  action[r] = a;
 }
 
 // Chunk tables for the value scatter.  The stored nonzeros are cut into chunks

@@ -627,13 +627,6 @@ __global__ __launch_bounds__(kBlock) void collect_long_rows_kernel(int64_t rows,
   if (is_long) list[base + __popcll(mask & ((1ull << lane) - 1ull))] = (int32_t)i;
 }
 
-// count[c] = number of nonzeros in column c (count[] zeroed by the caller).
-__global__ __launch_bounds__(kBlock) void count_columns_kernel(int64_t nnz, const int32_t* __restrict__ col,
-                                                               int32_t* __restrict__ count) {
-  const int64_t stride = (int64_t)gridDim.x * kBlock;
-  for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < nnz; j += stride) atomicAdd(&count[col[j]], 1);
-}
-
 // out[j] = ~slot if column col[j] is cached in slot colmap[col[j]] >= 0, else col[j].
 __global__ __launch_bounds__(kBlock) void remap_columns_kernel(int64_t nnz, const int32_t* __restrict__ col,
                                                                const int32_t* __restrict__ colmap,

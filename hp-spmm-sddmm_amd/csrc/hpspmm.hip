@@ -587,9 +587,11 @@ int exclusive_scan_u32(const uint32_t* d_in, uint32_t* d_out, int64_t n, hipStre
 // the routed and the hub-cache decisions share the histogram, and the ranking too when they ask for
 // the same `want`.
 struct ColumnRanking {
-  int32_t* d_count = nullptr;  // [cols]
+  int32_t* d_count = nullptr;  // [cols] occurrences among the sampled nonzeros
   int32_t* d_ids = nullptr;    // [n_ids]
-  int64_t want = 0, n_ids = 0, served = 0;  // served = nonzeros in the ranked columns
+  int64_t stride = 1;          // every stride-th nonzero was counted
+  int64_t sampled = 0;         // how many that is
+  int64_t want = 0, n_ids = 0, served = 0;  // served = nonzeros in the ranked columns (sample count x stride)
   ~ColumnRanking() {
     if (d_count) (void)hipFree(d_count);
     if (d_ids) (void)hipFree(d_ids);
@@ -687,8 +689,15 @@ int rank_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t want, hipSt
   rk.want = want;
   rk.n_ids = 0;
   rk.served = 0;
-  if (!rk.d_count)
-    if (int rc = count_columns(p, d_col, 1, st, &rk.d_count)) return rc;
+  if (!rk.d_count) {
+    // A large matrix is ranked from a sample of its nonzeros: which columns are hot, and roughly how
+    // hot, shows in every 4th nonzero as well as in all of them, and the histogram is the most
+    // expensive step of the plan (random read-modify-writes: 12 ms for the 128 M nonzeros of R-MAT
+    // scale 22).  Strided, hence the same sample every time.
+    rk.stride = p->nnz >= ((int64_t)1 << 25) ? 4 : p->nnz >= ((int64_t)1 << 23) ? 2 : 1;
+    rk.sampled = ceil_div(p->nnz, rk.stride);
+    if (int rc = count_columns(p, d_col, rk.stride, st, &rk.d_count)) return rc;
+  }
   unsigned long long* d_keys = nullptr;
   int64_t m = 0;
   if (int rc = select_top_columns(rk.d_count, p->cols, want, st, &d_keys, &m)) return rc;
@@ -729,34 +738,7 @@ int rank_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t want, hipSt
     HPSPMM_HIP(hipStreamSynchronize(st));
   }
   rk.n_ids = m;
-  rk.served = (int64_t)served;
-  return HPSPMM_OK;
-}
-
-// Share of the nonzeros that the `want` most referenced columns take, estimated from every 8th
-// nonzero (an overestimate when the columns are evenly used: the most referenced columns of a
-// sample are partly its noise).  Lets a graph without hot columns skip the full histogram.
-int estimate_hot_share(const hpspmm_plan* p, const int32_t* d_col, int64_t want, hipStream_t st, double* share_out) {
-  constexpr int64_t kStride = 8;
-  *share_out = 1.0;
-  if (p->nnz < (kStride << 16)) return HPSPMM_OK;  // too small to be worth a pass of its own
-  int32_t* d_count = nullptr;
-  if (int rc = count_columns(p, d_col, kStride, st, &d_count)) return rc;
-  unsigned long long* d_keys = nullptr;
-  int64_t m = 0;
-  int rc = select_top_columns(d_count, p->cols, want, st, &d_keys, &m);
-  (void)hipFree(d_count);
-  if (rc) return rc;
-  unsigned long long served = 0;
-  if (m > 0) {
-    std::vector<unsigned long long> keys((size_t)m);
-    hipError_t e = hipMemcpyAsync(keys.data(), d_keys, keys.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost, st);
-    if (e == hipSuccess) e = hipStreamSynchronize(st);
-    (void)hipFree(d_keys);
-    if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "hot-share estimate failed: %s", hipGetErrorString(e));
-    for (unsigned long long k : keys) served += (unsigned long long)(~(uint32_t)(k >> 32));
-  }
-  *share_out = (double)served / (double)ceil_div(p->nnz, kStride);
+  rk.served = (int64_t)served * rk.stride;
   return HPSPMM_OK;
 }
 
@@ -770,7 +752,6 @@ constexpr int kRoutedLog2Cached = 16;
 constexpr int64_t kRoutedMinNnz = (int64_t)1 << 22;
 constexpr int64_t kRoutedMinBBytes = (int64_t)10 << 20;  // a B that one or two L2s hold needs no routing (social graph at 26 M nonzeros: B = 7 MB, routed 309 us against 246; B = 14 MB, 464 against 474)
 constexpr double kRoutedMinShare = 0.35;     // of the nonzeros in the 64k most referenced columns
-constexpr double kRoutedEstimateMargin = 0.7;  // the estimate from a sample must reach this part of it
 constexpr double kRoutedMinRowNnz = 32.0;    // mean nonzeros per non-empty row
 constexpr int32_t kRoutedRowThreshold = 128;  // rows shorter than this are not split over the classes
 constexpr double kRoutedMinRoutedShare = 0.3;  // of the nonzeros in rows of at least that length
@@ -813,13 +794,6 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   // cached rows per class
   const int64_t h =
       std::max<int64_t>(1, ((int64_t)1 << (log2_hubs ? log2_hubs : kRoutedLog2Cached)) / hpspmm::kSlices);
-  if (!forced) {
-    // a look at every 8th nonzero first: a graph whose columns are evenly used is told apart
-    // without the full histogram
-    double estimate = 1.0;
-    if (int rc = estimate_hot_share(p, d_col, h * hpspmm::kSlices, st, &estimate)) return rc;
-    if (estimate < kRoutedMinShare * kRoutedEstimateMargin) return HPSPMM_OK;
-  }
   if (int rc = rank_columns(p, d_col, h * hpspmm::kSlices, st, rk)) return rc;
   if (!forced && (double)rk.served < kRoutedMinShare * (double)nnz) return HPSPMM_OK;
   const int32_t n_ids = (int32_t)rk.n_ids;
@@ -854,20 +828,23 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   int32_t* d_counts = nullptr;    // [2] list lengths
   int32_t* d_vpos = nullptr;      // [nnz] position of every stored nonzero in the class-major order
   int32_t* d_rlist = nullptr;     // [n_routed] row of every routed-row number
+  uint32_t* d_chunk_base = nullptr;  // [n_routed + 1] chunks per routed row, then (scanned) its first chunk
+  int32_t* d_chunk_row = nullptr;    // [n_chunks] routed-row number of every chunk
   struct Guard {
-    void** q[10];
+    void** q[12];
     ~Guard() {
       for (void** x : q)
         if (*x) (void)hipFree(*x);
     }
   } guard{{(void**)&d_colmap, (void**)&d_ridx, (void**)&d_cnt, (void**)&d_coldcnt, (void**)&d_action,
-           (void**)&d_counts, (void**)&d_vpos, (void**)&d_colrange, (void**)&d_bhot_src_tmp, (void**)&d_rlist}};
+           (void**)&d_counts, (void**)&d_vpos, (void**)&d_colrange, (void**)&d_bhot_src_tmp, (void**)&d_rlist,
+           (void**)&d_chunk_base, (void**)&d_chunk_row}};
 
   bool inplace = false;
   if (!sort_values && nsub == 1 && nnz > 0 && p->cols * k * 4 < ((int64_t)1 << 32) && p->d_nnz_row &&
       columns_sorted(p, d_col, st)) {
     const int groups = nhub;
-    const int64_t target = ceil_div(nnz, groups);
+    const int64_t target = ceil_div(rk.sampled, groups);  // the column counts are those of the sample
     uint32_t* d_before = nullptr;
     uint32_t* d_hot = nullptr;
     uint32_t hot[hpspmm::kMaxHub] = {0};
@@ -925,25 +902,38 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   HPSPMM_HIP(hipStreamSynchronize(st));
   const int64_t n_routed = n_routed_u;
 
-  // per-row class counts and their scans: a wavefront per routed row, a thread per short row
-  const int64_t ncnt = (int64_t)nhub * n_routed + 1;
-  HPSPMM_HIP(hipMalloc(&d_cnt, (size_t)ncnt * sizeof(uint32_t)));
+  // class counts and their scans: a wavefront per chunk of a routed row, a thread per short row
   HPSPMM_HIP(hipMalloc(&d_rlist, (size_t)std::max<int64_t>(n_routed, 1) * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&d_chunk_base, (size_t)(n_routed + 1) * sizeof(uint32_t)));
   const unsigned thread_per_row_grid = (unsigned)ceil_div(rows + 1, hpspmm::kBlock);
-  const unsigned routed_grid = (unsigned)std::max<int64_t>(1, ceil_div(n_routed, hpspmm::kWavesPerBlock));
+  const unsigned thread_per_routed_grid = (unsigned)ceil_div(n_routed + 1, hpspmm::kBlock);
   hipLaunchKernelGGL(hpspmm::routed_list_kernel, dim3(thread_per_row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr,
                      min_row_nnz, d_ridx, d_rlist);
   hipLaunchKernelGGL(hpspmm::routed_cold_count_kernel, dim3(thread_per_row_grid), dim3(hpspmm::kBlock), 0, st, rows,
                      d_rowptr, min_row_nnz, d_coldcnt);
-  hipLaunchKernelGGL(hpspmm::routed_count_kernel, dim3(routed_grid), dim3(hpspmm::kBlock), 0, st, n_routed, d_rlist,
-                     d_rowptr, d_col, d_colmap, (int32_t)h, nsub, (const uint8_t*)d_colrange, min_row_nnz, d_cnt);
+  hipLaunchKernelGGL(hpspmm::routed_row_chunks_kernel, dim3(thread_per_routed_grid), dim3(hpspmm::kBlock), 0, st,
+                     n_routed, d_rlist, d_rowptr, d_chunk_base);
+  if (int rc = exclusive_scan_u32(d_chunk_base, d_chunk_base, n_routed + 1, st)) return rc;
+  uint32_t n_chunks_u = 0;
+  HPSPMM_HIP(hipMemcpyAsync(&n_chunks_u, d_chunk_base + n_routed, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  const int64_t n_chunks = n_chunks_u;
+  HPSPMM_HIP(hipMalloc(&d_chunk_row, (size_t)std::max<int64_t>(n_chunks, 1) * sizeof(int32_t)));
+  const int64_t ncnt = (int64_t)nhub * n_chunks + 1;
+  HPSPMM_HIP(hipMalloc(&d_cnt, (size_t)ncnt * sizeof(uint32_t)));
+  const unsigned chunk_grid = (unsigned)std::max<int64_t>(1, ceil_div(n_chunks, hpspmm::kWavesPerBlock));
+  hipLaunchKernelGGL(hpspmm::routed_chunk_rows_kernel, dim3(thread_per_routed_grid), dim3(hpspmm::kBlock), 0, st,
+                     n_routed, d_chunk_base, d_chunk_row);
+  hipLaunchKernelGGL(hpspmm::routed_count_kernel, dim3(chunk_grid), dim3(hpspmm::kBlock), 0, st, n_chunks, d_chunk_row,
+                     d_chunk_base, d_rlist, d_rowptr, d_col, d_colmap, (int32_t)h, nsub, (const uint8_t*)d_colrange,
+                     min_row_nnz, d_cnt);
   if (int rc = exclusive_scan_u32(d_cnt, d_cnt, ncnt, st)) return rc;
   if (int rc = exclusive_scan_u32(d_coldcnt, d_coldcnt, rows + 1, st)) return rc;
 
   // class sizes = differences of the scan at the class origins
   uint32_t origin[hpspmm::kMaxHub + 1];
   for (int x = 0; x <= nhub; ++x)
-    HPSPMM_HIP(hipMemcpyAsync(&origin[x], d_cnt + (int64_t)x * n_routed, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    HPSPMM_HIP(hipMemcpyAsync(&origin[x], d_cnt + (int64_t)x * n_chunks, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
   uint32_t cold_total = 0;
   HPSPMM_HIP(hipMemcpyAsync(&cold_total, d_coldcnt + rows, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
   HPSPMM_HIP(hipStreamSynchronize(st));
@@ -1027,13 +1017,13 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   HPSPMM_HIP(hipMemsetAsync(d_counts, 0, 2 * sizeof(int32_t), st));
   const int64_t nrv = (n_routed + 1) * nhub;
   hipLaunchKernelGGL(hpspmm::routed_vptr_kernel, dim3((unsigned)ceil_div(nrv, hpspmm::kBlock)), dim3(hpspmm::kBlock),
-                     0, st, lay, d_cnt, p->d_rvptr);
+                     0, st, lay, n_chunks, d_chunk_base, d_cnt, p->d_rvptr);
   hipLaunchKernelGGL(hpspmm::routed_coldptr_kernel, dim3((unsigned)ceil_div(rows + 1, hpspmm::kBlock)),
                      dim3(hpspmm::kBlock), 0, st, rows, lay.cls_begin[nhub], d_coldcnt, p->d_coldptr);
   HPSPMM_HIP(hipMemcpyAsync(p->d_routed_rows, d_rlist, (size_t)n_routed * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
-  hipLaunchKernelGGL(hpspmm::routed_fill_kernel, dim3(routed_grid), dim3(hpspmm::kBlock), 0, st, n_routed, d_rlist,
-                     d_rowptr, d_col, d_colmap, (int32_t)h, nsub, (const uint8_t*)d_colrange, min_row_nnz, p->d_rvptr,
-                     p->d_vcol, d_vpos, p->d_vsrc, p->d_vrow);
+  hipLaunchKernelGGL(hpspmm::routed_fill_kernel, dim3(chunk_grid), dim3(hpspmm::kBlock), 0, st, lay, n_chunks,
+                     d_chunk_row, d_chunk_base, d_cnt, d_rlist, d_rowptr, d_col, d_colmap, (int32_t)h,
+                     (const uint8_t*)d_colrange, min_row_nnz, p->d_vcol, d_vpos, p->d_vsrc, p->d_vrow);
   if (nnz > 0)
     hipLaunchKernelGGL(hpspmm::routed_fill_cold_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)),
                        dim3(hpspmm::kBlock), 0, st, nnz, p->d_nnz_row, d_rowptr, d_col, d_colmap, min_row_nnz,
@@ -1234,6 +1224,46 @@ constexpr double kClusterMinServed = 0.15;
 // d_order_out receives a device array of `rows` entries (caller frees).
 constexpr int kClusterMaxSweeps = 16;
 
+// *d_order_out = the row numbers sorted by label[row], rows of one label in increasing order (a new
+// device array of `rows` entries, caller frees).  Stable radix sort, 8 bits a pass, over as many
+// bits as the largest possible label (rows - 1) has.
+int sort_rows_by_label(int64_t rows, const int32_t* d_label, hipStream_t st, int32_t** d_order_out) {
+  *d_order_out = nullptr;
+  const int64_t n_tiles = ceil_div(rows, hpspmm::kSortTile);
+  uint32_t *d_keys[2] = {nullptr, nullptr}, *d_hist = nullptr;
+  int32_t* d_vals[2] = {nullptr, nullptr};
+  struct Guard {
+    void** q[5];
+    ~Guard() {
+      for (void** x : q)
+        if (*x) (void)hipFree(*x);
+    }
+  } guard{{(void**)&d_keys[0], (void**)&d_keys[1], (void**)&d_vals[0], (void**)&d_vals[1], (void**)&d_hist}};
+  for (int i = 0; i < 2; ++i) {
+    HPSPMM_HIP(hipMalloc(&d_keys[i], (size_t)rows * sizeof(uint32_t)));
+    HPSPMM_HIP(hipMalloc(&d_vals[i], (size_t)rows * sizeof(int32_t)));
+  }
+  HPSPMM_HIP(hipMalloc(&d_hist, (size_t)(256 * n_tiles + 1) * sizeof(uint32_t)));
+  hipLaunchKernelGGL(hpspmm::label_pairs_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock), 0,
+                     st, rows, d_label, d_keys[0], d_vals[0]);
+  int bits = 1;
+  while (bits < 32 && ((int64_t)1 << bits) < rows) ++bits;
+  int cur = 0;
+  for (int shift = 0; shift < bits; shift += 8) {
+    hipLaunchKernelGGL(hpspmm::sort_count_kernel, dim3((unsigned)n_tiles), dim3(hpspmm::kBlock), 0, st, rows,
+                       d_keys[cur], shift, n_tiles, d_hist);
+    if (int rc = exclusive_scan_u32(d_hist, d_hist, 256 * n_tiles, st)) return rc;
+    hipLaunchKernelGGL(hpspmm::sort_scatter_kernel, dim3((unsigned)n_tiles), dim3(hpspmm::kBlock), 0, st, rows,
+                       d_keys[cur], d_vals[cur], shift, n_tiles, d_hist, d_keys[cur ^ 1], d_vals[cur ^ 1]);
+    cur ^= 1;
+  }
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  HPSPMM_HIP(hipGetLastError());
+  *d_order_out = d_vals[cur];
+  d_vals[cur] = nullptr;  // handed to the caller
+  return HPSPMM_OK;
+}
+
 int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st,
                  int32_t** d_order_out, double* intra_share_out) {
   const int64_t rows = p->rows;
@@ -1268,19 +1298,15 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
     for (uint32_t c : counters) changed += c;
     if (changed * 200 < rows) break;
   }
-  // counting sort by label on the host: stable, hence the same order on every run
-  std::vector<int32_t> label((size_t)rows), order((size_t)rows);
-  HPSPMM_HIP(hipMemcpyAsync(label.data(), d_label, label.size() * sizeof(int32_t), hipMemcpyDeviceToHost, st));
-  HPSPMM_HIP(hipStreamSynchronize(st));
-  std::vector<int32_t> first((size_t)rows + 1, 0);
-  for (int64_t r = 0; r < rows; ++r) first[(size_t)label[(size_t)r] + 1]++;
+  // share of the nonzeros that stay inside a cluster small enough for a workgroup's window
   {
-    // share of the nonzeros that stay inside a cluster small enough for a workgroup's window
     int32_t* d_size = nullptr;
     hipError_t e = hipMalloc(&d_size, (size_t)rows * sizeof(int32_t));
-    if (e == hipSuccess) e = hipMemcpyAsync(d_size, first.data() + 1, (size_t)rows * sizeof(int32_t), hipMemcpyHostToDevice, st);
+    if (e == hipSuccess) e = hipMemsetAsync(d_size, 0, (size_t)rows * sizeof(int32_t), st);
     if (e == hipSuccess) e = hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st);
     if (e == hipSuccess) {
+      hipLaunchKernelGGL(hpspmm::label_sizes_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                         0, st, rows, d_label, d_size);
       hipLaunchKernelGGL(hpspmm::cluster_intra_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
                          dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_label, d_size, kClusterMaxSize,
                          d_changed);
@@ -1293,16 +1319,10 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
     for (uint32_t c : counters) intra += c;
     *intra_share_out = p->nnz > 0 ? (double)intra / (double)p->nnz : 0.0;
   }
-  for (int64_t l = 0; l < rows; ++l) first[(size_t)l + 1] += first[(size_t)l];
-  for (int64_t r = 0; r < rows; ++r) order[(size_t)first[(size_t)label[(size_t)r]]++] = (int32_t)r;
+  // rows ordered by label, the rows of a label in increasing order: a stable sort, hence the same
+  // order on every run
   int32_t* d_order = nullptr;
-  HPSPMM_HIP(hipMalloc(&d_order, (size_t)rows * sizeof(int32_t)));
-  hipError_t e = hipMemcpyAsync(d_order, order.data(), order.size() * sizeof(int32_t), hipMemcpyHostToDevice, st);
-  if (e == hipSuccess) e = hipStreamSynchronize(st);
-  if (e != hipSuccess) {
-    (void)hipFree(d_order);
-    return fail(HPSPMM_ERR_HIP, "upload of the row order failed: %s", hipGetErrorString(e));
-  }
+  if (int rc = sort_rows_by_label(rows, d_label, st, &d_order)) return rc;
   *d_order_out = d_order;
   return HPSPMM_OK;
 }
@@ -1317,11 +1337,6 @@ int build_hub_cache(hpspmm_plan* p, const int32_t* d_col, int log2_hubs, bool fo
                     hipStream_t st) {
   if (log2_hubs == 0) log2_hubs = 16;
   if (log2_hubs < 4 || log2_hubs > 24) return fail(HPSPMM_ERR_INVALID_ARG, "hub cache size 2^%d outside [2^4, 2^24]", log2_hubs);
-  if (!forced) {
-    double estimate = 1.0;
-    if (int rc = estimate_hot_share(p, d_col, (int64_t)1 << log2_hubs, st, &estimate)) return rc;
-    if (estimate < kHubMinShare * kRoutedEstimateMargin) return HPSPMM_OK;
-  }
   if (int rc = rank_columns(p, d_col, (int64_t)1 << log2_hubs, st, rk)) return rc;
   if (rk.n_ids == 0) return HPSPMM_OK;
   // worth the extra column array only when the cached rows serve a good part of the gathers

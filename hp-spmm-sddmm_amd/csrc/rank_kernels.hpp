@@ -175,4 +175,89 @@ __global__ __launch_bounds__(kBlock) void range_hot_count_kernel(int32_t m, cons
   if (threadIdx.x < 64 && s_hot[threadIdx.x]) atomicAdd(&hot[threadIdx.x], s_hot[threadIdx.x]);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Stable radix sort of (key, value) pairs by 8-bit digits, least significant first: three kernels a
+// pass (digit counts per tile, their scan - the caller's -, scatter).  Used to order the rows by
+// cluster label with the rows of one label in increasing order.
+// ---------------------------------------------------------------------------------------------
+constexpr int kSortItems = 8;                     // elements per thread
+constexpr int kSortTile = kBlock * kSortItems;    // elements per workgroup
+
+// hist[d * n_tiles + tile] = elements of the tile whose digit is d.
+__global__ __launch_bounds__(kBlock) void sort_count_kernel(int64_t n, const uint32_t* __restrict__ keys, int shift,
+                                                            int64_t n_tiles, uint32_t* __restrict__ hist) {
+  __shared__ uint32_t s_hist[256];
+  s_hist[threadIdx.x] = 0;
+  __syncthreads();
+  const int64_t base = (int64_t)blockIdx.x * kSortTile;
+  for (int q = 0; q < kSortItems; ++q) {
+    const int64_t i = base + q * kBlock + threadIdx.x;
+    if (i < n) atomicAdd(&s_hist[(keys[i] >> shift) & 255u], 1u);
+  }
+  __syncthreads();
+  hist[(int64_t)threadIdx.x * n_tiles + blockIdx.x] = s_hist[threadIdx.x];
+}
+
+// Scatter of one pass: element i of the tile goes to offsets[d * n_tiles + tile] + (number of
+// elements of the tile before i with the same digit d).  That number is found round by round (256
+// consecutive elements a round), wavefront by wavefront within a round (running counts per digit in
+// LDS) and by ballots within a wavefront - in index order throughout, which is what keeps the sort stable.
+__global__ __launch_bounds__(kBlock) void sort_scatter_kernel(int64_t n, const uint32_t* __restrict__ keys_in,
+                                                              const int32_t* __restrict__ vals_in, int shift,
+                                                              int64_t n_tiles, const uint32_t* __restrict__ offsets,
+                                                              uint32_t* __restrict__ keys_out,
+                                                              int32_t* __restrict__ vals_out) {
+  __shared__ uint32_t s_run[256];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  s_run[threadIdx.x] = offsets[(int64_t)threadIdx.x * n_tiles + blockIdx.x];
+  __syncthreads();
+  const int64_t base = (int64_t)blockIdx.x * kSortTile;
+  const uint64_t below = (1ull << lane) - 1ull;
+  for (int q = 0; q < kSortItems; ++q) {
+    const int64_t i = base + q * kBlock + threadIdx.x;
+    const bool valid = i < n;
+    const uint32_t key = valid ? keys_in[i] : 0u;
+    const int32_t val = valid ? vals_in[i] : 0;
+    const uint32_t d = (key >> shift) & 255u;
+    // lanes of this wavefront that hold a valid element with the same digit
+    uint64_t same = __ballot(valid);
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const uint64_t set = __ballot((d >> b) & 1u);
+      same &= ((d >> b) & 1u) ? set : ~set;
+    }
+    const uint32_t before = (uint32_t)__popcll(same & below);
+    uint32_t dest = 0;
+    for (int w = 0; w < kWavesPerBlock; ++w) {
+      if (wave == w && valid) {
+        dest = s_run[d] + before;
+      }
+      __syncthreads();
+      if (wave == w && valid && before == 0) s_run[d] += (uint32_t)__popcll(same);
+      __syncthreads();
+    }
+    if (valid) {
+      keys_out[dest] = key;
+      vals_out[dest] = val;
+    }
+  }
+}
+
+// keys[r] = label[r], vals[r] = r.
+__global__ __launch_bounds__(kBlock) void label_pairs_kernel(int64_t rows, const int32_t* __restrict__ label,
+                                                             uint32_t* __restrict__ keys, int32_t* __restrict__ vals) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r >= rows) return;
+  keys[r] = (uint32_t)label[r];
+  vals[r] = (int32_t)r;
+}
+
+// size[label[r]] += 1 (size[] zeroed by the caller).
+__global__ __launch_bounds__(kBlock) void label_sizes_kernel(int64_t rows, const int32_t* __restrict__ label,
+                                                             int32_t* __restrict__ size) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r < rows) atomicAdd(&size[label[r]], 1);
+}
+
 }  // namespace hpspmm

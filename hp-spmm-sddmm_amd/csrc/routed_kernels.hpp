@@ -154,9 +154,57 @@ __global__ __launch_bounds__(kBlock) void routed_cold_count_kernel(int64_t rows,
   coldcnt[r] = n;
 }
 
-// One wavefront per routed row (number i, row routed_rows[i]): cnt[x * n_routed + i] = its nonzeros
-// in hub class x.  cnt[nhub * n_routed] = 0 (the scan's total slot) is written by the first wavefront.
-__global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t n_routed,
+// The routed rows are counted and laid out in chunks of kRoutedChunk consecutive nonzeros, one
+// wavefront each: a hub row of 10^5 nonzeros on a single wavefront was the critical path of the
+// whole plan.  nch[i] = chunks of routed row i (nch[n_routed] = 0: the scan's total slot).
+constexpr int kRoutedChunk = 4096;
+
+__global__ __launch_bounds__(kBlock) void routed_row_chunks_kernel(int64_t n_routed,
+                                                                   const int32_t* __restrict__ routed_rows,
+                                                                   const int32_t* __restrict__ rowptr,
+                                                                   uint32_t* __restrict__ nch) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i > n_routed) return;
+  uint32_t n = 0;
+  if (i < n_routed) {
+    const int32_t row = routed_rows[i];
+    n = (uint32_t)((rowptr[row + 1] - rowptr[row] + kRoutedChunk - 1) / kRoutedChunk);
+  }
+  nch[i] = n;
+}
+
+// chunk_row[c] = routed-row number of chunk c (chunk_base = exclusive scan of nch).
+__global__ __launch_bounds__(kBlock) void routed_chunk_rows_kernel(int64_t n_routed,
+                                                                   const uint32_t* __restrict__ chunk_base,
+                                                                   int32_t* __restrict__ chunk_row) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n_routed) return;
+  for (uint32_t c = chunk_base[i]; c < chunk_base[i + 1]; ++c) chunk_row[c] = (int32_t)i;
+}
+
+// Bounds of chunk c: nonzeros [lb, hb) of routed row number i; `single` = the row keeps everything in phase 0.
+struct RoutedChunk {
+  int32_t i, lb, hb;
+  bool single;
+};
+__device__ __forceinline__ RoutedChunk routed_chunk(int64_t c, const int32_t* __restrict__ chunk_row,
+                                                    const uint32_t* __restrict__ chunk_base,
+                                                    const int32_t* __restrict__ routed_rows,
+                                                    const int32_t* __restrict__ rowptr, int32_t min_row_nnz) {
+  RoutedChunk k;
+  k.i = chunk_row[c];
+  const int32_t row = routed_rows[k.i];
+  const int32_t row_lb = rowptr[row], row_hb = rowptr[row + 1];
+  k.lb = row_lb + (int32_t)(c - chunk_base[k.i]) * kRoutedChunk;
+  k.hb = k.lb + kRoutedChunk < row_hb ? k.lb + kRoutedChunk : row_hb;
+  k.single = row_hb - row_lb < kSinglePhaseFactor * min_row_nnz;
+  return k;
+}
+
+// One wavefront per chunk: cnt[x * n_chunks + c] = its nonzeros in hub class x.
+// cnt[nhub * n_chunks] = 0 (the scan's total slot) is written by the first wavefront.
+__global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t n_chunks, const int32_t* __restrict__ chunk_row,
+                                                              const uint32_t* __restrict__ chunk_base,
                                                               const int32_t* __restrict__ routed_rows,
                                                               const int32_t* __restrict__ rowptr,
                                                               const int32_t* __restrict__ col,
@@ -165,29 +213,26 @@ __global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t n_routed,
                                                               const uint8_t* __restrict__ colrange,
                                                               int32_t min_row_nnz, uint32_t* __restrict__ cnt) {
   const int lane = threadIdx.x & 63;
-  const int64_t i = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t c = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   const int nhub = kSlices * nsub;
-  if (i == 0 && lane == 0) cnt[(int64_t)nhub * n_routed] = 0;
-  if (i >= n_routed) return;
-  const int64_t row = routed_rows[i];
-  const int32_t lb = rowptr[row];
-  const int32_t hb = rowptr[row + 1];
-  const bool single = hb - lb < kSinglePhaseFactor * min_row_nnz;
+  if (c == 0 && lane == 0) cnt[(int64_t)nhub * n_chunks] = 0;
+  if (c >= n_chunks) return;
+  const RoutedChunk ch = routed_chunk(c, chunk_row, chunk_base, routed_rows, rowptr, min_row_nnz);
   uint32_t mine = 0;  // lane x < nhub accumulates the count of class x
-  for (int32_t j0 = lb; j0 < hb; j0 += 64) {
+  for (int32_t j0 = ch.lb; j0 < ch.hb; j0 += 64) {
     const int32_t j = j0 + lane;
     int cls = -1;
-    if (j < hb) {
-      const int32_t c = col[j];
-      cls = colrange ? range_class_of(colrange[c], nsub, single)
-                     : hub_class_of(c, colmap[c], hub_rows_per_slice, single ? 1 : nsub);
+    if (j < ch.hb) {
+      const int32_t cc = col[j];
+      cls = colrange ? range_class_of(colrange[cc], nsub, ch.single)
+                     : hub_class_of(cc, colmap[cc], hub_rows_per_slice, ch.single ? 1 : nsub);
     }
     for (int x = 0; x < nhub; ++x) {
       const uint64_t m = __ballot(cls == x);
       if (lane == x) mine += (uint32_t)__popcll(m);
     }
   }
-  if (lane < nhub) cnt[(int64_t)lane * n_routed + i] = mine;
+  if (lane < nhub) cnt[(int64_t)lane * n_chunks + c] = mine;
 }
 
 // Three-pass exclusive scan of uint32 (n up to 2^32, total < 2^32).
@@ -268,17 +313,17 @@ __global__ __launch_bounds__(kBlock) void scan_apply_kernel(int64_t n, const uin
 
 // rvptr[r * nhub + x] = virtual index of the first class-x nonzero of routed
 // row number r (r = n_routed: one past the class), from the exclusive scan of
-// the class-major counts and the padded class origins.  The end of the (r, x)
-// run is rvptr[(r + 1) * nhub + x].
-__global__ __launch_bounds__(kBlock) void routed_vptr_kernel(RoutedLayout lay, const uint32_t* __restrict__ scanned,
+// the class-major chunk counts (scanned[x * n_chunks + c]) and the padded class
+// origins.  The end of the (r, x) run is rvptr[(r + 1) * nhub + x].
+__global__ __launch_bounds__(kBlock) void routed_vptr_kernel(RoutedLayout lay, int64_t n_chunks,
+                                                             const uint32_t* __restrict__ chunk_base,
+                                                             const uint32_t* __restrict__ scanned,
                                                              int32_t* __restrict__ rvptr) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= (lay.n_routed + 1) * lay.nhub) return;
   const int64_t r = i / lay.nhub;
   const int x = (int)(i - r * lay.nhub);
-  const int64_t first = scanned[(int64_t)x * lay.n_routed];
-  const int64_t local = r < lay.n_routed ? (int64_t)scanned[(int64_t)x * lay.n_routed + r] - first
-                                         : lay.cls_end[x] - lay.cls_begin[x];
+  const int64_t local = (int64_t)scanned[(int64_t)x * n_chunks + chunk_base[r]] - (int64_t)scanned[(int64_t)x * n_chunks];
   rvptr[i] = (int32_t)(lay.cls_begin[x] + local);
 }
 
@@ -292,47 +337,51 @@ __global__ __launch_bounds__(kBlock) void routed_coldptr_kernel(int64_t rows, in
 }
 
 // Scatter the nonzeros of the routed rows into class-major order, keeping the stored order inside
-// every run.  One wavefront per routed row; positions in the hub classes from ballots.
-__global__ __launch_bounds__(kBlock) void routed_fill_kernel(int64_t n_routed,
+// every run.  One wavefront per chunk (its first slot in class x follows from the scan of the chunk
+// counts); positions within the chunk from ballots.
+__global__ __launch_bounds__(kBlock) void routed_fill_kernel(RoutedLayout lay, int64_t n_chunks,
+                                                             const int32_t* __restrict__ chunk_row,
+                                                             const uint32_t* __restrict__ chunk_base,
+                                                             const uint32_t* __restrict__ scanned,
                                                              const int32_t* __restrict__ routed_rows,
                                                              const int32_t* __restrict__ rowptr,
                                                              const int32_t* __restrict__ col,
                                                              const int32_t* __restrict__ colmap,
-                                                             int32_t hub_rows_per_slice, int nsub,
+                                                             int32_t hub_rows_per_slice,
                                                              const uint8_t* __restrict__ colrange,
-                                                             int32_t min_row_nnz, const int32_t* __restrict__ rvptr,
+                                                             int32_t min_row_nnz,
                                                              int32_t* __restrict__ vcol, int32_t* __restrict__ vpos,
                                                              int32_t* __restrict__ vsrc /* or NULL */,
                                                              int32_t* __restrict__ vrow) {
   const int lane = threadIdx.x & 63;
-  const int64_t i = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-  if (i >= n_routed) return;
-  const int nhub = kSlices * nsub;
-  const int64_t row = routed_rows[i];
-  const int32_t lb = rowptr[row];
-  const int32_t hb = rowptr[row + 1];
-  const int32_t r = (int32_t)i;
-  const bool single = hb - lb < kSinglePhaseFactor * min_row_nnz;
-  int32_t cursor = lane < nhub ? rvptr[(int64_t)r * nhub + lane] : 0;  // lane x: next slot of class x
+  const int64_t c = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  if (c >= n_chunks) return;
+  const int nsub = lay.nsub;
+  const int nhub = lay.nhub;
+  const RoutedChunk ch = routed_chunk(c, chunk_row, chunk_base, routed_rows, rowptr, min_row_nnz);
+  int32_t cursor = 0;  // lane x: next slot of class x
+  if (lane < nhub)
+    cursor = (int32_t)(lay.cls_begin[lane] + (int64_t)scanned[(int64_t)lane * n_chunks + c] -
+                       (int64_t)scanned[(int64_t)lane * n_chunks]);
   const uint64_t below = (1ull << lane) - 1ull;
-  for (int32_t j0 = lb; j0 < hb; j0 += 64) {
+  for (int32_t j0 = ch.lb; j0 < ch.hb; j0 += 64) {
     const int32_t j = j0 + lane;
-    const bool valid = j < hb;
-    const int32_t c = valid ? col[j] : 0;
-    const int32_t mapped = valid ? colmap[c] : -1;
+    const bool valid = j < ch.hb;
+    const int32_t cc = valid ? col[j] : 0;
+    const int32_t mapped = valid ? colmap[cc] : -1;
     const int cls = !valid      ? -1
-                    : colrange ? range_class_of(colrange[c], nsub, single)
-                               : hub_class_of(c, mapped, hub_rows_per_slice, single ? 1 : nsub);
+                    : colrange ? range_class_of(colrange[cc], nsub, ch.single)
+                               : hub_class_of(cc, mapped, hub_rows_per_slice, ch.single ? 1 : nsub);
     for (int x = 0; x < nhub; ++x) {
       const uint64_t m = __ballot(cls == x);
       if (m == 0) continue;
       const int32_t start = __shfl(cursor, x);
       if (cls == x) {
         const int32_t pos = start + (int32_t)__popcll(m & below);
-        vcol[pos] = mapped >= 0 ? ~mapped : c;
+        vcol[pos] = mapped >= 0 ? ~mapped : cc;
         vpos[j] = pos;
         if (vsrc) vsrc[pos] = j;
-        vrow[pos] = r;
+        vrow[pos] = ch.i;
       }
       if (lane == x) cursor += (int32_t)__popcll(m);
     }

@@ -161,8 +161,10 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_anyk_kernel(int64_t rows, in
 }
 
 // The segments kernel (see spmm_segments_kernel for the carry rule) with the row length at run time.
-// Workgroup b serves column tile b % tiles of segment group b / tiles.
-template <int GP>
+// Workgroup b serves column tile b % tiles of segment group b / tiles.  kAtomic = the COO
+// "accumulate" form: nnz_row is the caller's row array (any order), no carry slots, every flush an
+// FP32 atomic add into C.
+template <int GP, bool kAtomic>
 __global__ __launch_bounds__(kBlock) void spmm_segments_anyk_kernel(
     const int32_t* __restrict__ rowptr, const int32_t* __restrict__ col, const float* __restrict__ val,
     const int32_t* __restrict__ nnz_row, const float* __restrict__ B, float* __restrict__ C,
@@ -189,14 +191,25 @@ __global__ __launch_bounds__(kBlock) void spmm_segments_anyk_kernel(
   const int64_t off = ct.k0 + 4 * l;
 
   int32_t cur = nnz_row[s];
-  bool head_pending = (int64_t)rowptr[cur] < s;
+  bool head_pending = false;
+  if constexpr (!kAtomic) head_pending = (int64_t)rowptr[cur] < s;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 
   auto flush_to = [&](bool is_tail) {
-    float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
-                              : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : C + (uint64_t)(uint32_t)cur * K);
-    head_pending = false;
-    if (ct.active) store_result(dst + off, acc);
+    if constexpr (kAtomic) {
+      if (ct.active) {
+        float* dst = C + (uint64_t)(uint32_t)cur * K + off;
+        unsafeAtomicAdd(dst + 0, acc.x);
+        unsafeAtomicAdd(dst + 1, acc.y);
+        unsafeAtomicAdd(dst + 2, acc.z);
+        unsafeAtomicAdd(dst + 3, acc.w);
+      }
+    } else {
+      float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
+                                : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : C + (uint64_t)(uint32_t)cur * K);
+      head_pending = false;
+      if (ct.active) store_result(dst + off, acc);
+    }
   };
   auto flush = [&]() { flush_to(false); };
   auto loadb = [&](int32_t c) {
@@ -220,7 +233,9 @@ __global__ __launch_bounds__(kBlock) void spmm_segments_anyk_kernel(
     consume_tile(cnt, sbase, s_col, s_val, s_row, cur, acc, loadb, flush);
     wave_lds_fence();
   }
-  flush_to((int64_t)rowptr[cur + 1] > e);
+  bool continues = false;
+  if constexpr (!kAtomic) continues = (int64_t)rowptr[cur + 1] > e;
+  flush_to(continues);
 }
 
 // Fix-up after the segments kernel (see spmm_fixup_kernel): one row per lane is classified, the

@@ -428,7 +428,7 @@ int launch_segments_anyk_g(const hpspmm_plan* p, const int32_t* rp, const int32_
   const int64_t blocks = ceil_div(ceil_div(p->nseg, 64 / GP), hpspmm::kWavesPerBlock) * tiles;
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   if (p->nnz > 0) {
-    hipLaunchKernelGGL(hpspmm::spmm_segments_anyk_kernel<GP>, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rp,
+    hipLaunchKernelGGL((hpspmm::spmm_segments_anyk_kernel<GP, false>), dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rp,
                        ci, v, p->d_nnz_row, B, C, p->d_carry, p->nnz, p->shift, p->nseg, (int)p->k, tiles,
                        aligned16(ci, v, p->d_nnz_row));
     mark_launch(st, "spmm_segments_anyk_kernel");
@@ -448,6 +448,33 @@ int launch_segments_anyk(const hpspmm_plan* p, const int32_t* rp, const int32_t*
     case 8: return launch_segments_anyk_g<8>(p, rp, ci, v, B, C, st);
     case 16: return launch_segments_anyk_g<16>(p, rp, ci, v, B, C, st);
     default: return launch_segments_anyk_g<32>(p, rp, ci, v, B, C, st);
+  }
+}
+
+template <int GP>
+int launch_coo_anyk_g(int64_t nnz, int64_t k, const int32_t* ri, const int32_t* ci, const float* v, const float* B,
+                      float* C, hipStream_t st) {
+  constexpr int P = 64 / GP;
+  const int tiles = anyk_tiles(k);
+  int shift = 6;  // as launch_coo: 64 nonzeros per sub-wave, fewer while that leaves SIMDs idle
+  while (shift > 4 && (nnz >> shift) / P < 4096) --shift;
+  const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
+  const int64_t blocks = ceil_div(ceil_div(nseg, P), hpspmm::kWavesPerBlock) * tiles;
+  if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  hipLaunchKernelGGL((hpspmm::spmm_segments_anyk_kernel<GP, true>), dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st,
+                     (const int32_t*)nullptr, ci, v, ri, B, C, (float*)nullptr, nnz, shift, nseg, (int)k, tiles,
+                     aligned16(ci, v, ri));
+  return HPSPMM_OK;
+}
+
+int launch_coo_anyk(int64_t nnz, int64_t k, const int32_t* ri, const int32_t* ci, const float* v, const float* B,
+                    float* C, hipStream_t st) {
+  switch (anyk_lanes(k)) {
+    case 2: return launch_coo_anyk_g<2>(nnz, k, ri, ci, v, B, C, st);
+    case 4: return launch_coo_anyk_g<4>(nnz, k, ri, ci, v, B, C, st);
+    case 8: return launch_coo_anyk_g<8>(nnz, k, ri, ci, v, B, C, st);
+    case 16: return launch_coo_anyk_g<16>(nnz, k, ri, ci, v, B, C, st);
+    default: return launch_coo_anyk_g<32>(nnz, k, ri, ci, v, B, C, st);
   }
 }
 
@@ -1878,8 +1905,11 @@ int hpspmm_coo_spmm_accumulate(int64_t rows, int64_t cols, int64_t nnz, const in
     case 64: rc = launch_coo<64>(nnz, d_row, d_col, d_val, d_B, d_C, st); break;
     case 128: rc = launch_coo<128>(nnz, d_row, d_col, d_val, d_B, d_C, st); break;
     default:
-      hipLaunchKernelGGL(hpspmm::spmm_coo_generic_kernel, dim3(grid_for(nnz * k, 1 << 16)), dim3(hpspmm::kBlock), 0,
-                         st, nnz, k, d_row, d_col, d_val, d_B, d_C);
+      if (anyk_k(k))  // a multiple of 4: segments reduced in registers, one atomic per flush
+        rc = launch_coo_anyk(nnz, k, d_row, d_col, d_val, d_B, d_C, st);
+      else
+        hipLaunchKernelGGL(hpspmm::spmm_coo_generic_kernel, dim3(grid_for(nnz * k, 1 << 16)), dim3(hpspmm::kBlock), 0,
+                           st, nnz, k, d_row, d_col, d_val, d_B, d_C);
   }
   if (rc) return rc;
   HPSPMM_HIP(hipGetLastError());

@@ -288,7 +288,7 @@ def test_fill(pkg, gpu):
     assert torch.all(x == -2.5).item()
 
 
-@pytest.mark.parametrize("k", [32, 64, 128, 24])
+@pytest.mark.parametrize("k", [32, 64, 128, 24, 16, 96, 200, 7])
 def test_coo_accumulate(pkg, oracle, gpu, k):
     """The LBSpMM contract: C += A B, padded zero entries, rows in permuted order."""
     import torch

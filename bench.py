@@ -124,6 +124,28 @@ def l2_delivery_ceiling(capi, graphs, dev, stream, k, steps):
     return 4.0 * k * g.nnz / (ms * 1e-3) / 1e9
 
 
+def fabric_probe(capi, graphs, dev, stream, steps):
+    """Gather rate against the size of B: the segments kernel (no hub cache, no routing) on matrices of
+    512 uniformly random nonzeros per row, K = 128, with B from 1 MB (every gather an L2 hit) over sizes
+    that fit the 256 MB Infinity Cache to 2 GB.  Prints one line per size: what a gather that misses the
+    L2 can be served at, and whether the Infinity Cache changes that."""
+    import torch
+    k = 128
+    for cols in (2048, 32768, 131072, 262144, 393216, 524288, 1048576, 4194304):
+        g = graphs.uniform_rows(65536, cols, 512, 98)
+        B = graphs.dense_normal(g.cols, k, 98)
+        d = [torch.from_numpy(a).to(dev) for a in (g.rowptr, g.col, g.val, B)]
+        C = torch.empty((g.rows, k), device=dev, dtype=torch.float32)
+        plan = capi.Plan(g.rows, g.cols, d[0], d[1], k,
+                         capi.PLAN_FORCE_SEGMENTS | capi.PLAN_NO_HUB_CACHE | capi.PLAN_NO_ROUTED | capi.PLAN_NO_CLUSTER)
+        ms = capi.csr_spmm_timed(plan, d[0], d[1], d[2], d[3], C, warmup=3, iters=max(5, min(steps, 30)), stream=stream)
+        plan.destroy()
+        log(f"[fabric probe] B = {cols * k * 4 / 2**20:7.0f} MiB ({cols} rows of 512 B): {ms:.3f} ms, "
+            f"{4.0 * k * g.nnz / (ms * 1e-3) / 1e12:.2f} TB/s of gathered rows ({g.nnz} gathers)")
+        del d, C, B, g
+        torch.cuda.empty_cache()
+
+
 def cpu_baseline(graphs, g, B, k, C_gpu_host_rows, budget_nnz):
     """Time the CPU oracle (FP32, OpenMP, all host threads) on the first rows of the
     workload holding about budget_nnz nonzeros; also use it to check those GPU rows."""
@@ -174,6 +196,8 @@ def main():
     ap.add_argument("--no-launch-breakdown", action="store_true",
                     help="skip the per-launch timing and the all-hit gather probe (keeps a profile of this run "
                          "to the launches of the figure of merit)")
+    ap.add_argument("--fabric-probe", action="store_true",
+                    help="instead of the benchmark: the gather rate of the segments kernel against the size of B")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three 1 GiB device-to-device copies (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -195,6 +219,10 @@ def main():
     capi.lib()
     dev = torch.device("cuda:0")
     stream = torch.cuda.current_stream()
+
+    if args.fabric_probe:
+        fabric_probe(capi, graphs, dev, stream, args.steps)
+        return 0
 
     if args.calibrate_copy:
         src = torch.empty(1 << 28, device=dev, dtype=torch.float32).normal_()

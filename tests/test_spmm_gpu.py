@@ -376,6 +376,27 @@ def test_other_csr_arrays_are_refused(pkg, oracle, gpu):
         plan.destroy()
 
 
+def test_hot_set_beyond_the_device_ranking(pkg, oracle, gpu):
+    """A hot set of 2^18 columns is more than the plan's counting-rank sort takes (2^17 keys): the
+    selected columns are then sorted on the host.  Forced routed strategy with that hot set and 4
+    phases on an R-MAT of 524k columns; checked on row ranges that include the heaviest rows."""
+    capi = pkg.capi
+    g = pkg.graphs.make_graph("c4_rmat", 0.125)
+    assert g.cols > 1 << 18
+    k = 32
+    B = pkg.graphs.make_dense("c4_rmat", g.cols, k)
+    flags = capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(18) | capi.plan_routed_phases(4) | capi.PLAN_ROUTED_SORT_VALUES
+    C, info = _run(pkg, gpu, g, B, flags)
+    assert info["strategy"] == capi.STRATEGY_ROUTED and info["hub_rows"] > 1 << 17, info
+    again, info2 = _run(pkg, gpu, g, B, flags)
+    assert info == info2 and np.array_equal(C, again)
+    top = int(np.argmax(np.diff(g.rowptr)))
+    for lo, hi in ((0, 2000), (max(0, top - 10), min(g.rows, top + 10)), (g.rows - 2000, g.rows)):
+        C64, S64 = oracle.csr_spmm_f64_rows(g.rowptr, g.col, g.val, B, lo, hi)
+        err, pos = oracle.max_norm_err(C[lo:hi], C64, S64)
+        assert err <= TOL, (lo, hi, err, pos)
+
+
 def test_two_plans_of_one_matrix_give_the_same_bits(pkg, oracle, gpu):
     """Plan construction is deterministic, the clustering included: a second plan of the same matrix
     orders the rows alike, so C agrees bit for bit between plans, not only between calls."""

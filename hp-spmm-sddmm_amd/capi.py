@@ -33,6 +33,8 @@ PLAN_NO_CLUSTER = 8192
 PLAN_NO_ROW_TILES = 16384
 PLAN_ROUTED_SORT_VALUES = 32768
 PLAN_ALLOW_MOVED_CSR = 1 << 21
+PLAN_FORCE_SWEEP = 1 << 22
+PLAN_NO_SWEEP = 1 << 23
 
 
 def plan_hub_log2(log2_rows):
@@ -56,6 +58,7 @@ STRATEGY_SEGMENTS = 2
 STRATEGY_GENERIC_K = 3
 STRATEGY_ROUTED = 4
 STRATEGY_ORDERED = 5
+STRATEGY_SWEEP = 6
 
 # every symbol include/hpspmm.h declares
 EXPORTS = (

@@ -21,6 +21,7 @@
 #include "routed_kernels.hpp"
 #include "rowtile_kernels.hpp"
 #include "spmm_kernels.hpp"
+#include "sweep_kernels.hpp"
 
 namespace {
 
@@ -153,6 +154,19 @@ struct hpspmm_plan {
   int2* d_ldesc = nullptr;    // [rt_loop] per long row: first tile, tile count
   float* d_zrow = nullptr;    // 32 zeros: what a padding entry gathers instead of a row of B
   int32_t rt_tiles = 0, rt_waves = 0, rt_loop = 0, rt_wg = 0, rt_loop_tiles = 0;
+  // sweep strategy (its stream arrays are d_vcol = entry words, d_vsrc, d_vval when values are bound;
+  // partial-result rows of split rows in d_partial; rows without nonzeros in d_zero_rows)
+  hpspmm::SweepLayout sw{};
+  uint32_t* d_sw_base = nullptr;       // [n_waves + 1] first stream position of every wavefront
+  uint32_t* d_sw_len = nullptr;        // [n_waves] length of each of its sub-wave streams
+  int32_t* d_sw_ends = nullptr;        // [n_waves * n_windows] end of every window's chunk in those streams
+  int32_t* d_sw_slot_row = nullptr;    // [n_waves * slots] where every accumulator slot is stored
+  uint32_t* d_sw_part_base = nullptr;  // [rows + 1] first partial-result row of every split row
+  int32_t* d_sw_split_rows = nullptr;  // rows cut into several pieces
+  float* d_sw_zrow = nullptr;          // 128 zeros: what a padding entry gathers
+  int64_t n_split = 0, sw_total = 0;
+  int32_t sw_limit = 0;                // nonzeros per piece, at most
+  int32_t sw_bands = 0;
   int64_t workspace_bytes = 0;
 };
 
@@ -1391,6 +1405,315 @@ int build_hub_cache(hpspmm_plan* p, const int32_t* d_col, int log2_hubs, bool fo
   return HPSPMM_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Sweep strategy: plan construction and launch.
+// ---------------------------------------------------------------------------------------------
+
+// Frees what it holds when it goes out of scope (temporaries of a plan-construction step).
+struct DeviceTemps {
+  std::vector<void*> held;
+  ~DeviceTemps() {
+    for (void* q : held)
+      if (q) (void)hipFree(q);
+  }
+  template <class T>
+  int alloc(T** out, size_t count) {
+    *out = nullptr;
+    void* q = nullptr;
+    if (hipMalloc(&q, std::max<size_t>(count, 1) * sizeof(T)) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the plan failed", count * sizeof(T));
+    }
+    held.push_back(q);
+    *out = (T*)q;
+    return HPSPMM_OK;
+  }
+};
+
+// Stable LSD radix sort of n (key, value) pairs over the low `bits` bits of the keys.  d_keys[0] /
+// d_vals[0] hold the input, [1] are buffers of the same size, d_hist has 256 * tiles + 1 counters;
+// returns in *result which of the two value buffers holds the sorted values.
+int radix_sort_pairs(int64_t n, uint32_t* d_keys[2], int32_t* d_vals[2], uint32_t* d_hist, int bits, hipStream_t st,
+                     int* result) {
+  const int64_t n_tiles = ceil_div(n, hpspmm::kSortTile);
+  int cur = 0;
+  for (int shift = 0; shift < bits; shift += 8) {
+    hipLaunchKernelGGL(hpspmm::sort_count_kernel, dim3((unsigned)n_tiles), dim3(hpspmm::kBlock), 0, st, n, d_keys[cur],
+                       shift, n_tiles, d_hist);
+    if (int rc = exclusive_scan_u32(d_hist, d_hist, 256 * n_tiles, st)) return rc;
+    hipLaunchKernelGGL(hpspmm::sort_scatter_kernel, dim3((unsigned)n_tiles), dim3(hpspmm::kBlock), 0, st, n,
+                       d_keys[cur], d_vals[cur], shift, n_tiles, d_hist, d_keys[cur ^ 1], d_vals[cur ^ 1]);
+    cur ^= 1;
+  }
+  *result = cur;
+  return HPSPMM_OK;
+}
+
+int env_int(const char* name, int fallback) {
+  const char* v = std::getenv(name);
+  return v && *v ? std::atoi(v) : fallback;
+}
+
+constexpr int kSweepMaxBands = 64;
+constexpr int32_t kSweepMaxWindows = 8192;
+constexpr int32_t kSweepMaxLimit = 32768;  // piece lengths are sorted as 16-bit keys
+constexpr int kSweepWindowLog2 = 20;       // bytes of B per window
+constexpr int kSweepLead = 4;
+constexpr int kSweepSpinLimit = 400;
+
+// Lets the sweep kernels have their LDS; *out = workgroups of them that one CU holds (1 is what the
+// layout is made for).
+template <int K>
+int sweep_prepare_kernels(int* out) {
+  const size_t lds = hpspmm::sweep_lds_bytes<K>();
+  HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_sweep_kernel<K, true>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_sweep_kernel<K, false>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  HPSPMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(out, hpspmm::spmm_sweep_kernel<K, true>,
+                                                          hpspmm::sweep_waves<K>() * 64, lds));
+  return HPSPMM_OK;
+}
+
+// Builds the sweep layout on top of a segments plan (p->d_nnz_row must be there).  Returns HPSPMM_OK
+// with p->strategy left at SEGMENTS when the matrix does not qualify.  Diagnostics: the environment
+// variables HPSPMM_SWEEP_WINDOW_LOG2 (bytes of B per window), HPSPMM_SWEEP_LEAD, HPSPMM_SWEEP_SPIN,
+// HPSPMM_SWEEP_LIMIT (nonzeros per piece) and HPSPMM_SWEEP_PRIORITIES override the defaults.
+int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, hipStream_t st) {
+  const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
+  if (nnz <= 0 || !p->d_nnz_row) return HPSPMM_OK;
+  // gather offsets are 32-bit, stream entries keep the column in 24 bits
+  if (p->cols * k * 4 >= ((int64_t)1 << 32) || p->cols > ((int64_t)1 << hpspmm::kSweepColBits)) {
+    if (forced) return fail(HPSPMM_ERR_INVALID_ARG, "the sweep strategy takes at most 2^24 columns and 4 GB of B");
+    return HPSPMM_OK;
+  }
+  const int P = (int)(64 / (k / 4));
+  const int WS = P * hpspmm::kSweepSlots;
+  const int wpb = k == 32 ? hpspmm::sweep_waves<32>() : k == 64 ? hpspmm::sweep_waves<64>() : hpspmm::sweep_waves<128>();
+
+  // one workgroup fills a CU, and a band fills the device exactly: every CU then runs the same
+  // load (a CU with less runs its wavefronts faster, and they leave the others behind)
+  int per_cu = 0;
+  if (int rc = k == 32 ? sweep_prepare_kernels<32>(&per_cu) : k == 64 ? sweep_prepare_kernels<64>(&per_cu)
+                                                                     : sweep_prepare_kernels<128>(&per_cu))
+    return rc;
+  if (per_cu < 1) return HPSPMM_OK;
+  int dev = 0;
+  hipDeviceProp_t prop;
+  HPSPMM_HIP(hipGetDevice(&dev));
+  HPSPMM_HIP(hipGetDeviceProperties(&prop, dev));
+  const int64_t band_blocks = prop.multiProcessorCount;
+  const int64_t band_waves = band_blocks * wpb;
+
+  // piece limit: a good half of what a sub-wave gets in all, so that the slots of a wavefront even out
+  const int64_t nonempty = std::max<int64_t>(1, rows - p->empty_rows);
+  const int64_t bands_guess = ceil_div(nonempty + nonempty / 8, band_waves * WS);
+  int64_t limit64 = nnz / (bands_guess * band_waves * P) * 6 / 10;
+  limit64 = std::max<int64_t>(64, std::min<int64_t>(limit64, kSweepMaxLimit));
+  const int32_t limit = std::max(1, std::min<int>(env_int("HPSPMM_SWEEP_LIMIT", (int)limit64), kSweepMaxLimit));
+
+  const int wlog2 = env_int("HPSPMM_SWEEP_WINDOW_LOG2", kSweepWindowLog2);
+  int wshift = 0;  // log2 of the columns per window
+  while (wshift < 30 && (((int64_t)1 << (wshift + 1)) * k * 4) <= ((int64_t)1 << wlog2)) ++wshift;
+  const int64_t n_windows = ceil_div(p->cols, (int64_t)1 << wshift);
+  if (n_windows > kSweepMaxWindows) return HPSPMM_OK;
+  if (!columns_sorted(p, d_col, st)) {
+    if (forced) return fail(HPSPMM_ERR_INVALID_ARG, "the sweep strategy needs sorted column indices within every row");
+    return HPSPMM_OK;
+  }
+
+  DeviceTemps tmp;
+  // pieces per row, their scans
+  uint32_t *d_pbase = nullptr, *d_part = nullptr;
+  if (int rc = tmp.alloc(&d_pbase, (size_t)rows + 1)) return rc;
+  if (hipMalloc(&p->d_sw_part_base, (size_t)(rows + 1) * sizeof(uint32_t)) != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(HPSPMM_ERR_ALLOC, "device allocation for the plan failed");
+  }
+  d_part = p->d_sw_part_base;
+  hipLaunchKernelGGL(hpspmm::sweep_row_pieces_kernel, dim3((unsigned)ceil_div(rows + 1, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, limit, d_pbase, d_part);
+  if (int rc = exclusive_scan_u32(d_pbase, d_pbase, rows + 1, st)) return rc;
+  if (int rc = exclusive_scan_u32(d_part, d_part, rows + 1, st)) return rc;
+  uint32_t n_pieces = 0, n_parts = 0;
+  HPSPMM_HIP(hipMemcpyAsync(&n_pieces, d_pbase + rows, sizeof n_pieces, hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipMemcpyAsync(&n_parts, d_part + rows, sizeof n_parts, hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  if (n_pieces == 0) return HPSPMM_OK;
+
+  const int64_t n_bands = ceil_div((int64_t)n_pieces, band_waves * WS);
+  // every band re-reads B once on every XCD: worth it while that stays well below the gather volume,
+  // and while a piece still finds a few nonzeros in a window
+  if (!forced && (n_bands * hpspmm::kXcds * p->cols > nnz / 4 || (int64_t)n_pieces * n_windows > nnz / 2))
+    return HPSPMM_OK;
+  if (n_bands > kSweepMaxBands) {
+    if (forced) return fail(HPSPMM_ERR_INVALID_ARG, "the sweep strategy would need %lld bands", (long long)n_bands);
+    return HPSPMM_OK;
+  }
+  const int64_t n_waves = n_bands * band_waves;
+  const int64_t n_slots = n_waves * WS;
+
+  // pieces by decreasing length, dealt to the wavefronts
+  const int64_t n_tiles = ceil_div((int64_t)n_pieces, hpspmm::kSortTile);
+  uint32_t* d_keys[2] = {nullptr, nullptr};
+  int32_t* d_vals[2] = {nullptr, nullptr};
+  uint32_t* d_hist = nullptr;
+  int32_t *d_piece_row = nullptr, *d_slot_of = nullptr, *d_piece_of = nullptr;
+  for (int i = 0; i < 2; ++i) {
+    if (int rc = tmp.alloc(&d_keys[i], n_pieces)) return rc;
+    if (int rc = tmp.alloc(&d_vals[i], n_pieces)) return rc;
+  }
+  if (int rc = tmp.alloc(&d_hist, (size_t)(256 * n_tiles + 1))) return rc;
+  if (int rc = tmp.alloc(&d_piece_row, n_pieces)) return rc;
+  if (int rc = tmp.alloc(&d_slot_of, n_pieces)) return rc;
+  if (int rc = tmp.alloc(&d_piece_of, (size_t)n_slots)) return rc;
+  hipLaunchKernelGGL(hpspmm::sweep_piece_keys_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, limit, d_pbase, d_keys[0], d_vals[0], d_piece_row);
+  int sorted = 0;
+  if (int rc = radix_sort_pairs(n_pieces, d_keys, d_vals, d_hist, 16, st, &sorted)) return rc;
+  HPSPMM_HIP(hipMemsetAsync(d_piece_of, 0xFF, (size_t)n_slots * sizeof(int32_t), st));
+  hipLaunchKernelGGL(hpspmm::sweep_assign_kernel, dim3((unsigned)ceil_div((int64_t)n_pieces, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, (int64_t)n_pieces, d_vals[sorted], (int32_t)n_bands, (int32_t)band_waves,
+                     (int32_t)WS, d_slot_of, d_piece_of);
+
+  // where every row enters every window
+  int32_t *d_wstart = nullptr, *d_run_at = nullptr;
+  uint32_t* d_stream_len = nullptr;
+  if (int rc = tmp.alloc(&d_wstart, (size_t)rows * (size_t)(n_windows + 1))) return rc;
+  if (int rc = tmp.alloc(&d_run_at, (size_t)n_slots * (size_t)n_windows)) return rc;
+  if (int rc = tmp.alloc(&d_stream_len, (size_t)n_waves + 1)) return rc;
+  hipLaunchKernelGGL(hpspmm::sweep_row_windows_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, nnz, p->d_nnz_row, d_rowptr, d_col, wshift, (int32_t)n_windows, d_wstart);
+
+  // chunk lengths, stream lengths, stream origins
+  if (hipMalloc(&p->d_sw_base, (size_t)(n_waves + 1) * sizeof(uint32_t)) != hipSuccess ||
+      hipMalloc(&p->d_sw_len, (size_t)n_waves * sizeof(uint32_t)) != hipSuccess ||
+      hipMalloc(&p->d_sw_ends, (size_t)n_waves * (size_t)n_windows * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&p->d_sw_slot_row, (size_t)n_slots * sizeof(int32_t)) != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(HPSPMM_ERR_ALLOC, "device allocation for the plan failed");
+  }
+  const dim3 wave_grid((unsigned)n_waves);
+  switch (P) {
+    case 8:
+      hipLaunchKernelGGL(hpspmm::sweep_chunks_kernel<8>, wave_grid, dim3(hpspmm::kBlock), 0, st, (int32_t)n_windows, limit,
+                         d_piece_of, d_piece_row, d_pbase, d_rowptr, d_wstart, d_run_at, p->d_sw_ends, p->d_sw_len);
+      break;
+    case 4:
+      hipLaunchKernelGGL(hpspmm::sweep_chunks_kernel<4>, wave_grid, dim3(hpspmm::kBlock), 0, st, (int32_t)n_windows, limit,
+                         d_piece_of, d_piece_row, d_pbase, d_rowptr, d_wstart, d_run_at, p->d_sw_ends, p->d_sw_len);
+      break;
+    default:
+      hipLaunchKernelGGL(hpspmm::sweep_chunks_kernel<2>, wave_grid, dim3(hpspmm::kBlock), 0, st, (int32_t)n_windows, limit,
+                         d_piece_of, d_piece_row, d_pbase, d_rowptr, d_wstart, d_run_at, p->d_sw_ends, p->d_sw_len);
+      break;
+  }
+  hipLaunchKernelGGL(hpspmm::sweep_stream_lengths_kernel, dim3((unsigned)ceil_div(n_waves + 1, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, n_waves, P, p->d_sw_len, d_stream_len);
+  // the total must stay an int32 position: checked on the 64-bit sum of the lengths before the 32-bit scan
+  {
+    std::vector<uint32_t> lens((size_t)n_waves);
+    HPSPMM_HIP(hipMemcpyAsync(lens.data(), p->d_sw_len, (size_t)n_waves * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    HPSPMM_HIP(hipStreamSynchronize(st));
+    int64_t total = 0;
+    for (uint32_t v : lens) total += (int64_t)v * P;
+    if (total >= INT32_MAX - 64) {
+      if (forced) return fail(HPSPMM_ERR_INVALID_ARG, "sweep streams of %lld entries exceed the int32 range", (long long)total);
+      return HPSPMM_OK;
+    }
+    p->sw_total = total;
+  }
+  if (int rc = exclusive_scan_u32(d_stream_len, p->d_sw_base, n_waves + 1, st)) return rc;
+
+  // the streams
+  const int64_t total = p->sw_total;
+  if (hipMalloc(&p->d_vcol, (size_t)std::max<int64_t>(total, 1) * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&p->d_vsrc, (size_t)std::max<int64_t>(total, 1) * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&p->d_partial, (size_t)std::max<int64_t>(n_parts, 1) * (size_t)k * sizeof(float)) != hipSuccess ||
+      hipMalloc(&p->d_sw_split_rows, (size_t)std::max<int64_t>(n_parts / 2, 1) * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&p->d_zero_rows, (size_t)std::max<int64_t>(p->empty_rows, 1) * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&p->d_sw_zrow, 128 * sizeof(float)) != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(HPSPMM_ERR_ALLOC, "device allocation for the plan failed");
+  }
+  hipLaunchKernelGGL(hpspmm::sweep_clear_stream_kernel, dim3(grid_for(total, 1 << 16)), dim3(hpspmm::kBlock), 0, st, total,
+                     p->d_vcol, p->d_vsrc);
+  hipLaunchKernelGGL(hpspmm::sweep_fill_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)), dim3(hpspmm::kBlock), 0, st,
+                     nnz, (int32_t)n_windows, wshift, limit, (int32_t)WS, p->d_nnz_row, d_rowptr, d_col, d_pbase, d_slot_of,
+                     d_wstart, d_run_at, p->d_sw_ends, p->d_sw_base, p->d_sw_len, p->d_vcol, p->d_vsrc);
+  hipLaunchKernelGGL(hpspmm::sweep_slot_rows_kernel, dim3((unsigned)ceil_div(n_slots, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                     0, st, n_slots, d_piece_of, d_piece_row, d_pbase, d_part, d_rowptr, limit, p->d_sw_slot_row);
+
+  // rows cut into pieces, rows without nonzeros
+  int32_t* d_counts = nullptr;
+  if (int rc = tmp.alloc(&d_counts, 2)) return rc;
+  HPSPMM_HIP(hipMemsetAsync(d_counts, 0, 2 * sizeof(int32_t), st));
+  HPSPMM_HIP(hipMemsetAsync(p->d_sw_zrow, 0, 128 * sizeof(float), st));
+  const dim3 row_grid((unsigned)ceil_div(rows, hpspmm::kBlock));
+  hipLaunchKernelGGL(hpspmm::sweep_collect_rows_kernel, row_grid, dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, limit, 1,
+                     p->d_sw_split_rows, d_counts);
+  hipLaunchKernelGGL(hpspmm::sweep_collect_rows_kernel, row_grid, dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, limit, 0,
+                     p->d_zero_rows, d_counts + 1);
+  int32_t counts[2] = {0, 0};
+  HPSPMM_HIP(hipMemcpyAsync(counts, d_counts, sizeof counts, hipMemcpyDeviceToHost, st));
+  hipError_t e = hipStreamSynchronize(st);
+  if (e == hipSuccess) e = hipGetLastError();
+  if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "sweep layout failed: %s", hipGetErrorString(e));
+  if (counts[0] < 0 || counts[0] > (int32_t)(n_parts / 2) || counts[1] != p->empty_rows)
+    return fail(HPSPMM_ERR_HIP, "sweep layout: inconsistent row lists");
+  p->n_split = counts[0];
+  p->n_zero = counts[1];
+  p->sw_limit = limit;
+  p->sw_bands = (int32_t)n_bands;
+  p->sw.n_waves = n_waves;
+  p->sw.n_windows = (int32_t)n_windows;
+  p->sw.lead = std::max(1, env_int("HPSPMM_SWEEP_LEAD", kSweepLead));
+  p->sw.spin_limit = std::max(0, env_int("HPSPMM_SWEEP_SPIN", kSweepSpinLimit));
+  p->sw.priorities = env_int("HPSPMM_SWEEP_PRIORITIES", 1);
+  if (std::getenv("HPSPMM_SWEEP_DEBUG"))
+    fprintf(stderr, "sweep plan: bands=%lld waves=%lld windows=%lld limit=%d pieces=%u split_rows=%d nnz=%lld stream=%lld (%.3f)\n",
+            (long long)n_bands, (long long)n_waves, (long long)n_windows, limit, n_pieces, counts[0], (long long)nnz,
+            (long long)total, (double)total / (double)nnz);
+  // the segments plan underneath is no longer needed
+  (void)hipFree(p->d_nnz_row);
+  (void)hipFree(p->d_carry);
+  p->d_nnz_row = nullptr;
+  p->d_carry = nullptr;
+  p->workspace_bytes = 2 * total * 4 + (int64_t)std::max<int64_t>(n_parts, 1) * k * 4 + (n_waves + 1) * 4 + n_waves * 4 +
+                       n_waves * n_windows * 4 + n_slots * 4 + (rows + 1) * 4 + std::max<int64_t>(n_parts / 2, 1) * 4 +
+                       std::max<int64_t>(p->empty_rows, 1) * 4 + 512;
+  p->nseg = 0;
+  p->shift = 0;
+  p->strategy = HPSPMM_STRATEGY_SWEEP;
+  return HPSPMM_OK;
+}
+
+template <int K>
+int launch_sweep(const hpspmm_plan* p, const int32_t* rp, const float* v, const float* B, float* C, hipStream_t st) {
+  const bool bound = p->bound_val && p->bound_val == v && p->d_vval;
+  constexpr int wpb = hpspmm::sweep_waves<K>();
+  const dim3 grid((unsigned)(p->sw.n_waves / wpb));
+  const size_t lds = hpspmm::sweep_lds_bytes<K>();
+  if (bound)
+    hipLaunchKernelGGL((hpspmm::spmm_sweep_kernel<K, false>), grid, dim3(wpb * 64), lds, st, p->sw, p->d_sw_base,
+                       p->d_sw_len, p->d_sw_ends, p->d_vcol, p->d_vval, (const int32_t*)nullptr, p->d_sw_slot_row, B,
+                       p->d_sw_zrow, p->d_partial, C);
+  else
+    hipLaunchKernelGGL((hpspmm::spmm_sweep_kernel<K, true>), grid, dim3(wpb * 64), lds, st, p->sw, p->d_sw_base,
+                       p->d_sw_len, p->d_sw_ends, p->d_vcol, v, p->d_vsrc, p->d_sw_slot_row, B, p->d_sw_zrow,
+                       p->d_partial, C);
+  mark_launch(st, "spmm_sweep_kernel");
+  const int64_t split_blocks = row_blocks(p->n_split, K);
+  const int64_t fin_blocks = split_blocks + row_blocks(p->n_zero, K);
+  if (fin_blocks > 0) {
+    hipLaunchKernelGGL(hpspmm::spmm_sweep_final_kernel<K>, dim3((unsigned)fin_blocks), dim3(hpspmm::kBlock), 0, st, rp,
+                       p->sw_limit, p->d_sw_split_rows, p->n_split, split_blocks, p->d_sw_part_base, p->d_zero_rows,
+                       p->n_zero, p->d_partial, C);
+    mark_launch(st, "spmm_sweep_final_kernel");
+  }
+  return HPSPMM_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1489,8 +1812,8 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     return HPSPMM_OK;
   } else if (flags & HPSPMM_PLAN_FORCE_ROWS) {
     p->strategy = HPSPMM_STRATEGY_ROWS;
-  } else if (flags & (HPSPMM_PLAN_FORCE_SEGMENTS | HPSPMM_PLAN_FORCE_ROUTED)) {
-    p->strategy = HPSPMM_STRATEGY_SEGMENTS;  // the routed layout is built on top of it below
+  } else if (flags & (HPSPMM_PLAN_FORCE_SEGMENTS | HPSPMM_PLAN_FORCE_ROUTED | HPSPMM_PLAN_FORCE_SWEEP)) {
+    p->strategy = HPSPMM_STRATEGY_SEGMENTS;  // the routed and sweep layouts are built on top of it below
   } else {
     // Whole rows (one launch) while the matrix is small enough that the second and third launch of
     // the other strategies are felt and L2 reuse across rows is not yet what decides.  Measured
@@ -1544,6 +1867,9 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
         return fail(HPSPMM_ERR_HIP, "row expansion failed: %s", hipGetErrorString(e));
       }
     }
+  }
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && (flags & HPSPMM_PLAN_FORCE_SWEEP) && nnz > 0) {
+    if (int rc = build_sweep(p, d_rowptr, d_col, true, st)) return rc;
   }
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && !(flags & HPSPMM_PLAN_NO_ROUTED) && nnz > 0 &&
       !rows_range &&
@@ -1670,6 +1996,7 @@ int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
   out->workspace_bytes = plan->workspace_bytes;
   out->launches_per_spmm = plan->strategy == HPSPMM_STRATEGY_ROUTED    ? (plan->d_vsrc ? 2 : 3)
                            : plan->strategy == HPSPMM_STRATEGY_ORDERED ? 2
+                           : plan->strategy == HPSPMM_STRATEGY_SWEEP   ? 2
                            : plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? (plan->n_hub > 0 ? 3 : 2)
                                                                         : 1;
   out->hub_rows = plan->n_hub;
@@ -1691,7 +2018,9 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
                   (void*)plan->d_vval, (void*)plan->d_vsrc, (void*)plan->d_vrow, (void*)plan->d_bhot_src, (void*)plan->d_partial,
                   (void*)plan->d_routed_rows, (void*)plan->d_cross_rows, (void*)plan->d_zero_rows,
                   (void*)plan->d_ostart, (void*)plan->d_ocol, (void*)plan->d_osrc, (void*)plan->d_orow,
-                  (void*)plan->d_wcols, (void*)plan->d_tent, (void*)plan->d_ldesc, (void*)plan->d_zrow})
+                  (void*)plan->d_wcols, (void*)plan->d_tent, (void*)plan->d_ldesc, (void*)plan->d_zrow,
+                  (void*)plan->d_sw_base, (void*)plan->d_sw_len, (void*)plan->d_sw_ends, (void*)plan->d_sw_slot_row,
+                  (void*)plan->d_sw_part_base, (void*)plan->d_sw_split_rows, (void*)plan->d_sw_zrow})
     if (q) (void)hipFree(q);
   delete plan;
   return HPSPMM_OK;
@@ -1701,7 +2030,20 @@ int hpspmm_plan_bind_values(hpspmm_plan* plan, const float* d_val, void* stream)
   if (!plan) return fail(HPSPMM_ERR_INVALID_ARG, "plan is NULL");
   plan->bound_val = nullptr;
   if (!d_val || plan->nnz == 0) return HPSPMM_OK;
-  if (plan->strategy == HPSPMM_STRATEGY_ROUTED && plan->d_vsrc) {
+  if (plan->strategy == HPSPMM_STRATEGY_SWEEP) {
+    hipStream_t st = (hipStream_t)stream;
+    if (!plan->d_vval) {
+      if (hipMalloc(&plan->d_vval, (size_t)std::max<int64_t>(plan->sw_total, 1) * sizeof(float)) != hipSuccess) {
+        (void)hipGetLastError();
+        plan->d_vval = nullptr;
+        return fail(HPSPMM_ERR_ALLOC, "device allocation for the bound values failed");
+      }
+      plan->workspace_bytes += plan->sw_total * (int64_t)sizeof(float);
+    }
+    hipLaunchKernelGGL(hpspmm::sweep_gather_values_kernel, dim3(grid_for(plan->sw_total, 1 << 16)), dim3(hpspmm::kBlock),
+                       0, st, plan->sw_total, plan->d_vcol, plan->d_vsrc, d_val, plan->d_vval);
+    HPSPMM_HIP(hipGetLastError());
+  } else if (plan->strategy == HPSPMM_STRATEGY_ROUTED && plan->d_vsrc) {
     // column-range slices: constant values are worth a copy in the plan's order after all (reading them
     // in place costs the main kernel what a bound plan no longer pays in re-ordering)
     hipStream_t st = (hipStream_t)stream;
@@ -1755,6 +2097,12 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
       case 32: rc = launch_ordered<32>(plan, d_rowptr, d_val, d_B, d_C, st); break;
       case 64: rc = launch_ordered<64>(plan, d_rowptr, d_val, d_B, d_C, st); break;
       default: rc = launch_ordered<128>(plan, d_rowptr, d_val, d_B, d_C, st); break;
+    }
+  } else if (plan->strategy == HPSPMM_STRATEGY_SWEEP) {
+    switch (plan->k) {
+      case 32: rc = launch_sweep<32>(plan, d_rowptr, d_val, d_B, d_C, st); break;
+      case 64: rc = launch_sweep<64>(plan, d_rowptr, d_val, d_B, d_C, st); break;
+      default: rc = launch_sweep<128>(plan, d_rowptr, d_val, d_B, d_C, st); break;
     }
   } else if (plan->strategy == HPSPMM_STRATEGY_ROUTED) {
     switch (plan->k) {

@@ -82,6 +82,9 @@ typedef enum hpspmm_status {
                                          the kernel read the values in place); always spread them by popularity rank and
                                          hash and bring the values into the plan's order at the start of every SpMM */
 #define HPSPMM_PLAN_NO_ROW_TILES 16384u /* rows strategy: walk the caller's CSR arrays instead of building row tiles */
+#define HPSPMM_PLAN_FORCE_SWEEP (1u << 22) /* always use the sweep strategy (all wavefronts walk the columns of B window
+                                         by window, row accumulators in LDS); needs sorted columns within every row */
+#define HPSPMM_PLAN_NO_SWEEP (1u << 23)    /* never use the sweep strategy */
 
 /* strategy reported by hpspmm_plan_get_info */
 #define HPSPMM_STRATEGY_ROWS 1
@@ -89,6 +92,7 @@ typedef enum hpspmm_status {
 #define HPSPMM_STRATEGY_GENERIC_K 3
 #define HPSPMM_STRATEGY_ROUTED 4
 #define HPSPMM_STRATEGY_ORDERED 5
+#define HPSPMM_STRATEGY_SWEEP 6
 
 typedef struct hpspmm_plan hpspmm_plan;
 

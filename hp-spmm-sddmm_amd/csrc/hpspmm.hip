@@ -1457,9 +1457,15 @@ int env_int(const char* name, int fallback) {
 constexpr int kSweepMaxBands = 64;
 constexpr int32_t kSweepMaxWindows = 8192;
 constexpr int32_t kSweepMaxLimit = 32768;  // piece lengths are sorted as 16-bit keys
-constexpr int kSweepWindowLog2 = 20;       // bytes of B per window
-constexpr int kSweepLead = 4;
+constexpr int kSweepWindowLog2 = 19;       // bytes of B per window
 constexpr int kSweepSpinLimit = 400;
+// Windows a wavefront may be ahead of the slowest of its CU.  Social graph, 233k vertices, ms at
+// K = 32 / 64 / 128: windows of 512 KB with lead 2: 1.09 / 1.68 / 3.17, lead 3: 1.11 / 1.70 / 2.86;
+// 1 MB with lead 2: 1.09 / 1.70 / 2.92, lead 4: 1.12 / 1.71 / 3.07; 256 KB with lead 4: 1.09 / 1.67 / 3.15.
+inline int sweep_lead(int64_t k) { return k >= 128 ? 3 : 2; }
+// Automatic choice: B beyond what the L2s hold between them without help, enough work to fill the device.
+constexpr int64_t kSweepMinNnz = (int64_t)1 << 22;
+constexpr int64_t kSweepMinBBytes = (int64_t)8 << 20;
 
 // Lets the sweep kernels have their LDS; *out = workgroups of them that one CU holds (1 is what the
 // layout is made for).
@@ -1475,6 +1481,15 @@ int sweep_prepare_kernels(int* out) {
   return HPSPMM_OK;
 }
 
+// Gives back what an abandoned attempt at the sweep layout has allocated in the plan so far.
+void drop_sweep_buffers(hpspmm_plan* p) {
+  for (void** q : {(void**)&p->d_sw_part_base, (void**)&p->d_sw_base, (void**)&p->d_sw_len, (void**)&p->d_sw_ends,
+                   (void**)&p->d_sw_slot_row}) {
+    if (*q) (void)hipFree(*q);
+    *q = nullptr;
+  }
+}
+
 // Builds the sweep layout on top of a segments plan (p->d_nnz_row must be there).  Returns HPSPMM_OK
 // with p->strategy left at SEGMENTS when the matrix does not qualify.  Diagnostics: the environment
 // variables HPSPMM_SWEEP_WINDOW_LOG2 (bytes of B per window), HPSPMM_SWEEP_LEAD, HPSPMM_SWEEP_SPIN,
@@ -1483,10 +1498,8 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
   if (nnz <= 0 || !p->d_nnz_row) return HPSPMM_OK;
   // gather offsets are 32-bit, stream entries keep the column in 24 bits
-  if (p->cols * k * 4 >= ((int64_t)1 << 32) || p->cols > ((int64_t)1 << hpspmm::kSweepColBits)) {
-    if (forced) return fail(HPSPMM_ERR_INVALID_ARG, "the sweep strategy takes at most 2^24 columns and 4 GB of B");
-    return HPSPMM_OK;
-  }
+  if (p->cols * k * 4 >= ((int64_t)1 << 32) || p->cols > ((int64_t)1 << hpspmm::kSweepColBits)) return HPSPMM_OK;
+  if (!forced && (nnz < kSweepMinNnz || p->cols * k * 4 < kSweepMinBBytes)) return HPSPMM_OK;
   const int P = (int)(64 / (k / 4));
   const int WS = P * hpspmm::kSweepSlots;
   const int wpb = k == 32 ? hpspmm::sweep_waves<32>() : k == 64 ? hpspmm::sweep_waves<64>() : hpspmm::sweep_waves<128>();
@@ -1517,10 +1530,7 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   while (wshift < 30 && (((int64_t)1 << (wshift + 1)) * k * 4) <= ((int64_t)1 << wlog2)) ++wshift;
   const int64_t n_windows = ceil_div(p->cols, (int64_t)1 << wshift);
   if (n_windows > kSweepMaxWindows) return HPSPMM_OK;
-  if (!columns_sorted(p, d_col, st)) {
-    if (forced) return fail(HPSPMM_ERR_INVALID_ARG, "the sweep strategy needs sorted column indices within every row");
-    return HPSPMM_OK;
-  }
+  if (!columns_sorted(p, d_col, st)) return HPSPMM_OK;  // a row must meet the windows in stored order
 
   DeviceTemps tmp;
   // pieces per row, their scans
@@ -1539,15 +1549,17 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   HPSPMM_HIP(hipMemcpyAsync(&n_pieces, d_pbase + rows, sizeof n_pieces, hipMemcpyDeviceToHost, st));
   HPSPMM_HIP(hipMemcpyAsync(&n_parts, d_part + rows, sizeof n_parts, hipMemcpyDeviceToHost, st));
   HPSPMM_HIP(hipStreamSynchronize(st));
-  if (n_pieces == 0) return HPSPMM_OK;
+  if (n_pieces == 0) {
+    drop_sweep_buffers(p);
+    return HPSPMM_OK;
+  }
 
   const int64_t n_bands = ceil_div((int64_t)n_pieces, band_waves * WS);
   // every band re-reads B once on every XCD: worth it while that stays well below the gather volume,
   // and while a piece still finds a few nonzeros in a window
-  if (!forced && (n_bands * hpspmm::kXcds * p->cols > nnz / 4 || (int64_t)n_pieces * n_windows > nnz / 2))
-    return HPSPMM_OK;
-  if (n_bands > kSweepMaxBands) {
-    if (forced) return fail(HPSPMM_ERR_INVALID_ARG, "the sweep strategy would need %lld bands", (long long)n_bands);
+  if (n_bands > kSweepMaxBands ||
+      (!forced && (n_bands * hpspmm::kXcds * p->cols > nnz / 4 || (int64_t)n_pieces * n_windows > nnz))) {
+    drop_sweep_buffers(p);
     return HPSPMM_OK;
   }
   const int64_t n_waves = n_bands * band_waves;
@@ -1618,7 +1630,7 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
     int64_t total = 0;
     for (uint32_t v : lens) total += (int64_t)v * P;
     if (total >= INT32_MAX - 64) {
-      if (forced) return fail(HPSPMM_ERR_INVALID_ARG, "sweep streams of %lld entries exceed the int32 range", (long long)total);
+      drop_sweep_buffers(p);
       return HPSPMM_OK;
     }
     p->sw_total = total;
@@ -1667,7 +1679,7 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   p->sw_bands = (int32_t)n_bands;
   p->sw.n_waves = n_waves;
   p->sw.n_windows = (int32_t)n_windows;
-  p->sw.lead = std::max(1, env_int("HPSPMM_SWEEP_LEAD", kSweepLead));
+  p->sw.lead = std::max(1, env_int("HPSPMM_SWEEP_LEAD", sweep_lead(k)));
   p->sw.spin_limit = std::max(0, env_int("HPSPMM_SWEEP_SPIN", kSweepSpinLimit));
   p->sw.priorities = env_int("HPSPMM_SWEEP_PRIORITIES", 1);
   if (std::getenv("HPSPMM_SWEEP_DEBUG"))
@@ -1868,8 +1880,15 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       }
     }
   }
-  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && (flags & HPSPMM_PLAN_FORCE_SWEEP) && nnz > 0) {
-    if (int rc = build_sweep(p, d_rowptr, d_col, true, st)) return rc;
+  // Long rows over a B that is small against the gather volume: every wavefront walks B window by
+  // window (tried first: where it qualifies it beats the routed strategy - social graph, 233k
+  // vertices, K = 32 / 64 / 128: 1.09 / 1.68 / 2.86 ms against 1.11 / 1.92 / 3.72).  When the matrix
+  // does not qualify, or cannot be laid out that way (unsorted columns, more than 2^24 columns),
+  // the plan stays what it was.
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && nnz > 0 && !(flags & HPSPMM_PLAN_NO_SWEEP) &&
+      ((flags & HPSPMM_PLAN_FORCE_SWEEP) ||
+       (!rows_range && !(flags & (HPSPMM_PLAN_FORCE_SEGMENTS | HPSPMM_PLAN_FORCE_ROUTED | HPSPMM_PLAN_CLUSTER))))) {
+    if (int rc = build_sweep(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_SWEEP) != 0, st)) return rc;
   }
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && !(flags & HPSPMM_PLAN_NO_ROUTED) && nnz > 0 &&
       !rows_range &&

@@ -65,7 +65,8 @@ def _strategies(capi):
             ("cluster_seg", capi.PLAN_CLUSTER | capi.PLAN_FORCE_SEGMENTS | capi.PLAN_NO_HUB_CACHE),
             ("routed_3phases", capi.PLAN_FORCE_ROUTED | capi.plan_routed_phases(3) | capi.plan_routed_row_log2(4)),
             ("routed_7phases_tiny", capi.PLAN_FORCE_ROUTED | capi.plan_routed_phases(7) | capi.plan_hub_log2(5)
-             | capi.plan_segment_shift(3) | capi.plan_routed_row_log2(1))]
+             | capi.plan_segment_shift(3) | capi.plan_routed_row_log2(1)),
+            ("sweep", capi.PLAN_FORCE_SWEEP)]
 
 
 @pytest.mark.parametrize("k", [32, 64, 128])
@@ -426,12 +427,12 @@ def test_xcd_placement_is_verified_at_plan_time(pkg, oracle, gpu):
     k = 128
     B = pkg.graphs.make_dense("c2_social", g.cols, k)
     assert "HPSPMM_XCD_DEALING" not in os.environ
-    C, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+    C, info = _run(pkg, gpu, g, B, capi.PLAN_NO_SWEEP)  # (the sweep strategy, which this graph gets by default, places nothing)
     assert info["strategy"] == capi.STRATEGY_ROUTED, info
     _check(oracle, g, B, C, "probe result")
     os.environ["HPSPMM_XCD_DEALING"] = "0"
     try:
-        C0, info0 = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+        C0, info0 = _run(pkg, gpu, g, B, capi.PLAN_NO_SWEEP)
     finally:
         del os.environ["HPSPMM_XCD_DEALING"]
     assert info0["strategy"] in (capi.STRATEGY_SEGMENTS, capi.STRATEGY_ROWS), info0
@@ -470,9 +471,9 @@ def test_full_size_configs(pkg, oracle, gpu, name, k):
         plan.destroy()
         assert not torch.isnan(C).any().item(), f"{name} K={k} {tag}: C not fully written"
         out[tag] = (C, info)
-    expect = {("c2_social", 128): capi.STRATEGY_ROUTED, ("c2_social", 64): capi.STRATEGY_ROUTED,
+    expect = {("c2_social", 128): capi.STRATEGY_SWEEP, ("c2_social", 64): capi.STRATEGY_SWEEP,
               ("c4_rmat", 128): capi.STRATEGY_ROUTED, ("c3_copurchase", 64): capi.STRATEGY_ORDERED,
-              ("c2_social", 32): capi.STRATEGY_ROUTED}[(name, k)]
+              ("c2_social", 32): capi.STRATEGY_SWEEP}[(name, k)]
     assert out["auto"][1]["strategy"] == expect
     # the two strategies sum in different orders: they agree to rounding, scaled by |A| |B|
     plan = capi.Plan(g.rows, g.cols, rp, ci, k, capi.PLAN_FORCE_SEGMENTS | capi.PLAN_NO_HUB_CACHE | capi.PLAN_NO_ROUTED)
@@ -840,3 +841,80 @@ def test_auto_choice_at_mid_size(pkg, oracle, gpu):
             C64, S64 = oracle.csr_spmm_f64_rows(g.rowptr, g.col, g.val, B, int(r), int(r) + 1)
             err, _ = oracle.max_norm_err(C[r:r + 1], C64, S64)
             assert err <= TOL, f"{name}: heaviest rows: normalised error {err:.3e}"
+
+
+def test_sweep_strategy(pkg, oracle, gpu):
+    """The sweep strategy (row accumulators in LDS, all wavefronts walking B window by window): chosen
+    by itself for a graph of long rows whose B is beyond the L2s, two launches, bit-reproducible across
+    calls and across plans, same bits with bound values; PLAN_NO_SWEEP gives the routed strategy back."""
+    import torch
+    capi = pkg.capi
+    g = pkg.graphs.make_graph("c2_social", 0.1)
+    for k in (32, 64, 128):
+        B = pkg.graphs.make_dense("c2_social", g.cols, k)
+        C1, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SWEEP)
+        assert info["strategy"] == capi.STRATEGY_SWEEP and info["launches_per_spmm"] == 2, info
+        _check(oracle, g, B, C1, f"sweep k={k}")
+        C2, info2 = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SWEEP)
+        assert info2 == info and np.array_equal(C1, C2), "two sweep plans, different bits"
+        rp, ci, v, Bd = _to_dev(gpu, g.rowptr, g.col, g.val, B)
+        plan = capi.Plan(g.rows, g.cols, rp, ci, k, capi.PLAN_FORCE_SWEEP)
+        C = torch.full((g.rows, k), float("nan"), device=gpu)
+        plan.bind_values(v)
+        capi.csr_spmm(plan, rp, ci, v, Bd, C)
+        torch.cuda.synchronize()
+        assert np.array_equal(C.cpu().numpy(), C1), "bound values, different bits"
+        plan.destroy()
+    # automatic choice: 12 MB of B and 9.6 M nonzeros in rows of 400 qualify, 3 MB of B (K = 32) do not
+    B = pkg.graphs.make_dense("c2_social", g.cols, 128)
+    _, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+    assert info["strategy"] == capi.STRATEGY_SWEEP, info
+    _, info = _run(pkg, gpu, g, B, capi.PLAN_NO_SWEEP)
+    assert info["strategy"] == capi.STRATEGY_ROUTED, info
+    B = pkg.graphs.make_dense("c2_social", g.cols, 32)
+    _, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+    assert info["strategy"] != capi.STRATEGY_SWEEP, info
+
+
+def test_sweep_layout_corners(pkg, oracle, gpu):
+    """Forced sweep plans whose layout is all corners: windows of a few columns, pieces of 64 nonzeros
+    (most rows split, several bands), a lead of one window; a matrix with empty rows and a row of
+    every column; unsorted columns (the plan then keeps to segments)."""
+    import os
+    capi = pkg.capi
+    rng = np.random.default_rng(11)
+    cases = []
+    g = pkg.graphs.make_graph("c2_social", 0.05)
+    cases.append(("social", g))
+    # empty rows, one-nonzero rows, one dense row, a last column that only the dense row uses
+    rows, cols = 3000, 5000
+    deg = rng.integers(0, 60, rows)
+    deg[rng.random(rows) < 0.3] = 0
+    deg[7] = cols
+    deg[11] = 1
+    rowptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.choice(cols - 1 if d < cols else cols, int(d), replace=False)) for d in deg]).astype(np.int32)
+    val = rng.uniform(-1, 1, col.size).astype(np.float32)
+    cases.append(("ragged", pkg.graphs.CSR(rows, cols, rowptr, col, val)))
+    for env in ({}, {"HPSPMM_SWEEP_WINDOW_LOG2": "12", "HPSPMM_SWEEP_LIMIT": "64", "HPSPMM_SWEEP_LEAD": "1"},
+                {"HPSPMM_SWEEP_WINDOW_LOG2": "30", "HPSPMM_SWEEP_LIMIT": "1", "HPSPMM_SWEEP_SPIN": "0"}):
+        os.environ.update(env)
+        try:
+            for name, g in cases:
+                if env.get("HPSPMM_SWEEP_LIMIT") == "1" and name == "social":
+                    continue  # one piece per nonzero: only for the small matrix
+                for k in (32, 64, 128):
+                    B = pkg.graphs.dense_normal(g.cols, k, 5)
+                    C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SWEEP)
+                    assert info["strategy"] == capi.STRATEGY_SWEEP, (name, env, info)
+                    _check(oracle, g, B, C, f"sweep corners {name} k={k} {env}")
+        finally:
+            for key in env:
+                del os.environ[key]
+    # columns out of order within the rows: no sweep layout, the forced flag falls back to segments
+    rowptr, col, val = _random_csr(rng, 500, 700, 20, 1.5, 0.1, sorted_unique=False)
+    g = pkg.graphs.CSR(500, 700, rowptr, col, val)
+    B = pkg.graphs.dense_normal(700, 64, 6)
+    C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SWEEP)
+    assert info["strategy"] == capi.STRATEGY_SEGMENTS, info
+    _check(oracle, g, B, C, "sweep forced on unsorted columns")

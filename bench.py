@@ -9,7 +9,7 @@ HBM once, and every timed region starts with them resident.
 
     value        geometric mean of the per-workload GFLOPS
     ms_per_step  sum of the per-workload mean SpMM times
-    roofline     social graph, K=128, its dominant kernel (spmm_routed_kernel):
+    roofline     social graph, K=128, its dominant kernel (spmm_sweep_kernel):
                  frac         algorithmic bytes 4(M+1) + 8 nnz + 4 K nnz + 4 K M
                               (the B gather counted once per nonzero) divided by
                               that kernel's mean duration, against 8 TB/s.  L2 and
@@ -63,13 +63,12 @@ ROOFLINE_WORKLOAD = ("c2_social", 128)
 # fails when they differ from those files.  They are reported only for the configuration they were
 # measured on: same workload, K, strategy and number of launches, scale 1, default plan.
 MEASURED_TRAFFIC = {
-    ("c2_social", 32): {"strategy": 4, "launches": 2, "profile": "profiles/spmm_routed_kernel__c2_social.txt",
-                        "kernels": {"spmm_routed_kernel": 4.771, "spmm_routed_final_kernel": 0.268}},
-    ("c2_social", 64): {"strategy": 4, "launches": 2, "profile": "profiles/spmm_routed_kernel__c2_social.txt",
-                        "kernels": {"spmm_routed_kernel": 10.632, "spmm_routed_final_kernel": 0.529}},
-    ("c2_social", 128): {"strategy": 4, "launches": 3, "profile": "profiles/spmm_routed_kernel__c2_social.txt",
-                         "kernels": {"routed_prepare_kernel": 1.238, "spmm_routed_kernel": 19.815,
-                                     "spmm_routed_final_kernel": 1.433}},
+    ("c2_social", 32): {"strategy": 6, "launches": 2, "profile": "profiles/spmm_sweep_kernel__c2_social.txt",
+                        "kernels": {"spmm_sweep_kernel": 4.584, "spmm_sweep_final_kernel": 0.012}},
+    ("c2_social", 64): {"strategy": 6, "launches": 2, "profile": "profiles/spmm_sweep_kernel__c2_social.txt",
+                        "kernels": {"spmm_sweep_kernel": 4.672, "spmm_sweep_final_kernel": 0.010}},
+    ("c2_social", 128): {"strategy": 6, "launches": 2, "profile": "profiles/spmm_sweep_kernel__c2_social.txt",
+                         "kernels": {"spmm_sweep_kernel": 6.700, "spmm_sweep_final_kernel": 0.019}},
     ("c3_copurchase", 64): {"strategy": 5, "launches": 2, "profile": "profiles/spmm_ordered_kernel__c3_copurchase.txt",
                             "kernels": {"spmm_ordered_kernel": 21.274, "spmm_fixup_kernel": 0.203}},
     ("c4_rmat", 128): {"strategy": 4, "launches": 3, "profile": "profiles/spmm_routed_kernel__c4_rmat.txt",
@@ -80,8 +79,9 @@ MEASURED_TRAFFIC = {
 # What bounds each workload.
 ROOF = {
     "c1_citation": "launch latency: one launch of ~2 dependent memory round trips; no bandwidth roof applies",
-    "c2_social": "L2 delivery: B fits no L2 whole but its hot rows do; the gather runs against the all-hit "
-                 "gather rate of the L2 -> CU path (l2_delivery_frac), traffic_frac is the secondary roof",
+    "c2_social": "L2 delivery: all wavefronts walk B window by window, so every L2 holds the stretch in use; the "
+                 "gather runs against the all-hit gather rate of the L2 -> CU path (l2_delivery_frac), "
+                 "traffic_frac is the secondary roof",
     "c3_copurchase": "fabric: L2 misses move at the rate the L2 <-> fabric path sustains (traffic_frac)",
     "c4_rmat": "fabric: L2 misses move at the rate the L2 <-> fabric path sustains (traffic_frac)",
 }

@@ -1465,7 +1465,7 @@ constexpr int kSweepSpinLimit = 400;
 inline int sweep_lead(int64_t k) { return k >= 128 ? 3 : 2; }
 // Automatic choice: B beyond what the L2s hold between them without help, enough work to fill the device.
 constexpr int64_t kSweepMinNnz = (int64_t)1 << 22;
-constexpr int64_t kSweepMinBBytes = (int64_t)8 << 20;
+constexpr int64_t kSweepMinBBytes = (int64_t)5 << 20;  // social graph: 6 MB of B, sweep 103 / 127 us against 123 / 141; 3 MB: 90 / 65 against 87 / 63
 
 // Lets the sweep kernels have their LDS; *out = workgroups of them that one CU holds (1 is what the
 // layout is made for).
@@ -1556,9 +1556,10 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
 
   const int64_t n_bands = ceil_div((int64_t)n_pieces, band_waves * WS);
   // every band re-reads B once on every XCD: worth it while that stays well below the gather volume,
-  // and while a piece still finds a few nonzeros in a window
+  // and while a piece still finds one or two nonzeros in a window (the co-purchase graph at 6 M
+  // nonzeros has 0.85 on average and takes 251 us against 134 with the ordered strategy)
   if (n_bands > kSweepMaxBands ||
-      (!forced && (n_bands * hpspmm::kXcds * p->cols > nnz / 4 || (int64_t)n_pieces * n_windows > nnz))) {
+      (!forced && (n_bands * hpspmm::kXcds * p->cols > nnz / 4 || (int64_t)n_pieces * n_windows * 3 > nnz * 2))) {
     drop_sweep_buffers(p);
     return HPSPMM_OK;
   }

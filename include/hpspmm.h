@@ -82,8 +82,11 @@ typedef enum hpspmm_status {
                                          the kernel read the values in place); always spread them by popularity rank and
                                          hash and bring the values into the plan's order at the start of every SpMM */
 #define HPSPMM_PLAN_NO_ROW_TILES 16384u /* rows strategy: walk the caller's CSR arrays instead of building row tiles */
-#define HPSPMM_PLAN_FORCE_SWEEP (1u << 22) /* always use the sweep strategy (all wavefronts walk the columns of B window
-                                         by window, row accumulators in LDS); needs sorted columns within every row */
+#define HPSPMM_PLAN_FORCE_SWEEP (1u << 22) /* use the sweep strategy (all wavefronts walk the columns of B window by
+                                         window, the row accumulators stay in LDS) whatever the size of the matrix
+                                         (default: from 2^22 nonzeros and 8 MB of B up, when the rows are long
+                                         against the size of B).  It needs sorted columns within every row, at most
+                                         2^24 columns and less than 4 GB of B; otherwise the plan keeps to segments */
 #define HPSPMM_PLAN_NO_SWEEP (1u << 23)    /* never use the sweep strategy */
 
 /* strategy reported by hpspmm_plan_get_info */
@@ -125,10 +128,14 @@ const char *hpspmm_last_error(void);
  * 8-nonzero slots and packed, by length class, into one 64-entry tile per
  * wavefront, so that a microsecond-scale SpMM is one launch with a two-step
  * dependent chain); fixed-length segments of nonzeros with a carry buffer;
- * the same inside column slices pinned to one XCD each when a few columns
- * take most of the nonzeros ("routed"); or segments over a clustered row
- * order with the reused rows of B held in LDS when the matrix is a graph with
- * communities ("ordered").
+ * for a large matrix of long rows whose B is small against the gather volume,
+ * one workgroup per CU that keeps the accumulators of its rows in LDS while
+ * all wavefronts walk the columns of B window by window at the same pace, so
+ * that every L2 holds the stretch of B in use ("sweep"); segments inside
+ * column slices pinned to one XCD each when a few columns take most of the
+ * nonzeros ("routed"); or segments over a clustered row order with the reused
+ * rows of B held in LDS when the matrix is a graph with communities
+ * ("ordered").
  * Replaces the host-side preprocessing the reference does before timing:
  * CSR->COO expansion (spmm/mm/spmm_common.cpp:185-235), the row re-ordering
  * (:237-296) and the choice of nnz_per_warp (spmm/mm/spmm_kernel.cu:749-751).

@@ -605,7 +605,24 @@ int choose_shift(int64_t nnz, int64_t k, int64_t max_row_nnz) {
   return shift;
 }
 
-// Device exclusive scan of n uint32 values (three passes, tile sums in between); d_out may be d_in.
+// Words of scratch the scan below needs for n values.
+inline int64_t scan_scratch_words(int64_t n) { return ceil_div(n, hpspmm::kScanTile) + 1; }
+
+// Device exclusive scan of n uint32 values (three passes, tile sums in between) with the caller's
+// scratch (scan_scratch_words(n) words): launches only, no allocation, no synchronisation.  d_out may be d_in.
+int exclusive_scan_u32(const uint32_t* d_in, uint32_t* d_out, int64_t n, hipStream_t st, uint32_t* d_tiles) {
+  const int64_t ntiles = ceil_div(n, hpspmm::kScanTile);
+  if (ntiles > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "scan too large");
+  if (ntiles <= 0) return HPSPMM_OK;
+  hipLaunchKernelGGL(hpspmm::scan_tile_sums_kernel, dim3((unsigned)ntiles), dim3(hpspmm::kBlock), 0, st, n, d_in,
+                     d_tiles);
+  hipLaunchKernelGGL(hpspmm::scan_tile_offsets_kernel, dim3(1), dim3(hpspmm::kBlock), 0, st, ntiles, d_tiles);
+  hipLaunchKernelGGL(hpspmm::scan_apply_kernel, dim3((unsigned)ntiles), dim3(hpspmm::kBlock), 0, st, n, d_in, d_tiles,
+                     d_out);
+  return HPSPMM_OK;
+}
+
+// The same with scratch of its own; synchronises the stream.
 int exclusive_scan_u32(const uint32_t* d_in, uint32_t* d_out, int64_t n, hipStream_t st) {
   const int64_t ntiles = ceil_div(n, hpspmm::kScanTile);
   if (ntiles > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "scan too large");
@@ -1428,19 +1445,37 @@ struct DeviceTemps {
     *out = (T*)q;
     return HPSPMM_OK;
   }
+  // One allocation cut into pieces (an allocation costs 50-200 us, a plan step has a dozen temporaries):
+  // room(count) for every piece first, then reserve(), then take() in the same order.
+  size_t arena_bytes = 0, arena_used = 0;
+  char* arena = nullptr;
+  template <class T>
+  void room(size_t count) { arena_bytes += (std::max<size_t>(count, 1) * sizeof(T) + 255) & ~(size_t)255; }
+  int reserve() {
+    if (int rc = alloc(&arena, arena_bytes)) return rc;
+    arena_used = 0;
+    return HPSPMM_OK;
+  }
+  template <class T>
+  T* take(size_t count) {
+    T* out = reinterpret_cast<T*>(arena + arena_used);
+    arena_used += (std::max<size_t>(count, 1) * sizeof(T) + 255) & ~(size_t)255;
+    return out;
+  }
 };
 
 // Stable LSD radix sort of n (key, value) pairs over the low `bits` bits of the keys.  d_keys[0] /
-// d_vals[0] hold the input, [1] are buffers of the same size, d_hist has 256 * tiles + 1 counters;
-// returns in *result which of the two value buffers holds the sorted values.
-int radix_sort_pairs(int64_t n, uint32_t* d_keys[2], int32_t* d_vals[2], uint32_t* d_hist, int bits, hipStream_t st,
-                     int* result) {
+// d_vals[0] hold the input, [1] are buffers of the same size, d_hist has 256 * tiles + 1 counters,
+// d_scan_scratch scan_scratch_words(256 * tiles) words; returns in *result which of the two value
+// buffers holds the sorted values.  Launches only.
+int radix_sort_pairs(int64_t n, uint32_t* d_keys[2], int32_t* d_vals[2], uint32_t* d_hist, uint32_t* d_scan_scratch,
+                     int bits, hipStream_t st, int* result) {
   const int64_t n_tiles = ceil_div(n, hpspmm::kSortTile);
   int cur = 0;
   for (int shift = 0; shift < bits; shift += 8) {
     hipLaunchKernelGGL(hpspmm::sort_count_kernel, dim3((unsigned)n_tiles), dim3(hpspmm::kBlock), 0, st, n, d_keys[cur],
                        shift, n_tiles, d_hist);
-    if (int rc = exclusive_scan_u32(d_hist, d_hist, 256 * n_tiles, st)) return rc;
+    if (int rc = exclusive_scan_u32(d_hist, d_hist, 256 * n_tiles, st, d_scan_scratch)) return rc;
     hipLaunchKernelGGL(hpspmm::sort_scatter_kernel, dim3((unsigned)n_tiles), dim3(hpspmm::kBlock), 0, st, n,
                        d_keys[cur], d_vals[cur], shift, n_tiles, d_hist, d_keys[cur ^ 1], d_vals[cur ^ 1]);
     cur ^= 1;
@@ -1534,8 +1569,9 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
 
   DeviceTemps tmp;
   // pieces per row, their scans
-  uint32_t *d_pbase = nullptr, *d_part = nullptr;
-  if (int rc = tmp.alloc(&d_pbase, (size_t)rows + 1)) return rc;
+  uint32_t *d_pbase = nullptr, *d_part = nullptr, *d_scan0 = nullptr;
+  if (int rc = tmp.alloc(&d_pbase, (size_t)rows + 1 + (size_t)scan_scratch_words(rows + 1))) return rc;
+  d_scan0 = d_pbase + rows + 1;
   if (hipMalloc(&p->d_sw_part_base, (size_t)(rows + 1) * sizeof(uint32_t)) != hipSuccess) {
     (void)hipGetLastError();
     return fail(HPSPMM_ERR_ALLOC, "device allocation for the plan failed");
@@ -1543,8 +1579,8 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   d_part = p->d_sw_part_base;
   hipLaunchKernelGGL(hpspmm::sweep_row_pieces_kernel, dim3((unsigned)ceil_div(rows + 1, hpspmm::kBlock)),
                      dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, limit, d_pbase, d_part);
-  if (int rc = exclusive_scan_u32(d_pbase, d_pbase, rows + 1, st)) return rc;
-  if (int rc = exclusive_scan_u32(d_part, d_part, rows + 1, st)) return rc;
+  if (int rc = exclusive_scan_u32(d_pbase, d_pbase, rows + 1, st, d_scan0)) return rc;
+  if (int rc = exclusive_scan_u32(d_part, d_part, rows + 1, st, d_scan0)) return rc;
   uint32_t n_pieces = 0, n_parts = 0;
   HPSPMM_HIP(hipMemcpyAsync(&n_pieces, d_pbase + rows, sizeof n_pieces, hipMemcpyDeviceToHost, st));
   HPSPMM_HIP(hipMemcpyAsync(&n_parts, d_part + rows, sizeof n_parts, hipMemcpyDeviceToHost, st));
@@ -1566,35 +1602,50 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   const int64_t n_waves = n_bands * band_waves;
   const int64_t n_slots = n_waves * WS;
 
-  // pieces by decreasing length, dealt to the wavefronts
+  // the other temporaries, one allocation
   const int64_t n_tiles = ceil_div((int64_t)n_pieces, hpspmm::kSortTile);
-  uint32_t* d_keys[2] = {nullptr, nullptr};
-  int32_t* d_vals[2] = {nullptr, nullptr};
-  uint32_t* d_hist = nullptr;
-  int32_t *d_piece_row = nullptr, *d_slot_of = nullptr, *d_piece_of = nullptr;
+  const size_t scan_words = (size_t)std::max(scan_scratch_words(256 * n_tiles), scan_scratch_words(n_waves + 1));
   for (int i = 0; i < 2; ++i) {
-    if (int rc = tmp.alloc(&d_keys[i], n_pieces)) return rc;
-    if (int rc = tmp.alloc(&d_vals[i], n_pieces)) return rc;
+    tmp.room<uint32_t>(n_pieces);
+    tmp.room<int32_t>(n_pieces);
   }
-  if (int rc = tmp.alloc(&d_hist, (size_t)(256 * n_tiles + 1))) return rc;
-  if (int rc = tmp.alloc(&d_piece_row, n_pieces)) return rc;
-  if (int rc = tmp.alloc(&d_slot_of, n_pieces)) return rc;
-  if (int rc = tmp.alloc(&d_piece_of, (size_t)n_slots)) return rc;
+  tmp.room<uint32_t>((size_t)(256 * n_tiles + 1));
+  tmp.room<uint32_t>(scan_words);
+  tmp.room<int32_t>(n_pieces);
+  tmp.room<int32_t>(n_pieces);
+  tmp.room<int32_t>((size_t)n_slots);
+  tmp.room<int32_t>((size_t)rows * (size_t)(n_windows + 1));
+  tmp.room<int32_t>((size_t)n_slots * (size_t)n_windows);
+  tmp.room<uint32_t>((size_t)n_waves + 1);
+  tmp.room<int32_t>(2);
+  if (int rc = tmp.reserve()) return rc;
+  uint32_t* d_keys[2];
+  int32_t* d_vals[2];
+  for (int i = 0; i < 2; ++i) {
+    d_keys[i] = tmp.take<uint32_t>(n_pieces);
+    d_vals[i] = tmp.take<int32_t>(n_pieces);
+  }
+  uint32_t* d_hist = tmp.take<uint32_t>((size_t)(256 * n_tiles + 1));
+  uint32_t* d_scan = tmp.take<uint32_t>(scan_words);
+  int32_t* d_piece_row = tmp.take<int32_t>(n_pieces);
+  int32_t* d_slot_of = tmp.take<int32_t>(n_pieces);
+  int32_t* d_piece_of = tmp.take<int32_t>((size_t)n_slots);
+  int32_t* d_wstart = tmp.take<int32_t>((size_t)rows * (size_t)(n_windows + 1));
+  int32_t* d_run_at = tmp.take<int32_t>((size_t)n_slots * (size_t)n_windows);
+  uint32_t* d_stream_len = tmp.take<uint32_t>((size_t)n_waves + 1);
+  int32_t* d_counts = tmp.take<int32_t>(2);
+
+  // pieces by decreasing length, dealt to the wavefronts
   hipLaunchKernelGGL(hpspmm::sweep_piece_keys_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)),
                      dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, limit, d_pbase, d_keys[0], d_vals[0], d_piece_row);
   int sorted = 0;
-  if (int rc = radix_sort_pairs(n_pieces, d_keys, d_vals, d_hist, 16, st, &sorted)) return rc;
+  if (int rc = radix_sort_pairs(n_pieces, d_keys, d_vals, d_hist, d_scan, 16, st, &sorted)) return rc;
   HPSPMM_HIP(hipMemsetAsync(d_piece_of, 0xFF, (size_t)n_slots * sizeof(int32_t), st));
   hipLaunchKernelGGL(hpspmm::sweep_assign_kernel, dim3((unsigned)ceil_div((int64_t)n_pieces, hpspmm::kBlock)),
                      dim3(hpspmm::kBlock), 0, st, (int64_t)n_pieces, d_vals[sorted], (int32_t)n_bands, (int32_t)band_waves,
                      (int32_t)WS, d_slot_of, d_piece_of);
 
   // where every row enters every window
-  int32_t *d_wstart = nullptr, *d_run_at = nullptr;
-  uint32_t* d_stream_len = nullptr;
-  if (int rc = tmp.alloc(&d_wstart, (size_t)rows * (size_t)(n_windows + 1))) return rc;
-  if (int rc = tmp.alloc(&d_run_at, (size_t)n_slots * (size_t)n_windows)) return rc;
-  if (int rc = tmp.alloc(&d_stream_len, (size_t)n_waves + 1)) return rc;
   hipLaunchKernelGGL(hpspmm::sweep_row_windows_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)),
                      dim3(hpspmm::kBlock), 0, st, nnz, p->d_nnz_row, d_rowptr, d_col, wshift, (int32_t)n_windows, d_wstart);
 
@@ -1636,7 +1687,7 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
     }
     p->sw_total = total;
   }
-  if (int rc = exclusive_scan_u32(d_stream_len, p->d_sw_base, n_waves + 1, st)) return rc;
+  if (int rc = exclusive_scan_u32(d_stream_len, p->d_sw_base, n_waves + 1, st, d_scan)) return rc;
 
   // the streams
   const int64_t total = p->sw_total;
@@ -1658,8 +1709,6 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
                      0, st, n_slots, d_piece_of, d_piece_row, d_pbase, d_part, d_rowptr, limit, p->d_sw_slot_row);
 
   // rows cut into pieces, rows without nonzeros
-  int32_t* d_counts = nullptr;
-  if (int rc = tmp.alloc(&d_counts, 2)) return rc;
   HPSPMM_HIP(hipMemsetAsync(d_counts, 0, 2 * sizeof(int32_t), st));
   HPSPMM_HIP(hipMemsetAsync(p->d_sw_zrow, 0, 128 * sizeof(float), st));
   const dim3 row_grid((unsigned)ceil_div(rows, hpspmm::kBlock));

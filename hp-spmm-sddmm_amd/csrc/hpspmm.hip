@@ -1703,7 +1703,8 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   hipLaunchKernelGGL(hpspmm::sweep_clear_stream_kernel, dim3(grid_for(total, 1 << 16)), dim3(hpspmm::kBlock), 0, st, total,
                      p->d_vcol, p->d_vsrc);
   hipLaunchKernelGGL(hpspmm::sweep_fill_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)), dim3(hpspmm::kBlock), 0, st,
-                     nnz, (int32_t)n_windows, wshift, limit, (int32_t)WS, p->d_nnz_row, d_rowptr, d_col, d_pbase, d_slot_of,
+                     nnz, (int32_t)n_windows, wshift, limit, (int32_t)WS, (int32_t)(k / 4), p->d_nnz_row, d_rowptr, d_col,
+                     d_pbase, d_slot_of,
                      d_wstart, d_run_at, p->d_sw_ends, p->d_sw_base, p->d_sw_len, p->d_vcol, p->d_vsrc);
   hipLaunchKernelGGL(hpspmm::sweep_slot_rows_kernel, dim3((unsigned)ceil_div(n_slots, hpspmm::kBlock)), dim3(hpspmm::kBlock),
                      0, st, n_slots, d_piece_of, d_piece_row, d_pbase, d_part, d_rowptr, limit, p->d_sw_slot_row);
@@ -2110,7 +2111,7 @@ int hpspmm_plan_bind_values(hpspmm_plan* plan, const float* d_val, void* stream)
       plan->workspace_bytes += plan->sw_total * (int64_t)sizeof(float);
     }
     hipLaunchKernelGGL(hpspmm::sweep_gather_values_kernel, dim3(grid_for(plan->sw_total, 1 << 16)), dim3(hpspmm::kBlock),
-                       0, st, plan->sw_total, plan->d_vcol, plan->d_vsrc, d_val, plan->d_vval);
+                       0, st, plan->sw_total, plan->d_vsrc, d_val, plan->d_vval);
     HPSPMM_HIP(hipGetLastError());
   } else if (plan->strategy == HPSPMM_STRATEGY_ROUTED && plan->d_vsrc) {
     // column-range slices: constant values are worth a copy in the plan's order after all (reading them

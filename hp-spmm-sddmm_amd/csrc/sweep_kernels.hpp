@@ -155,7 +155,7 @@ __device__ __forceinline__ int32_t sweep_count_below(int32_t n, int32_t m, int32
 // run_at[slot * n_windows + p] = sub-wave << 28 | position of the run within that sub-wave's chunk.
 // The chunk of the wavefront is the longest of its sub-waves: chunk_end[wave * n_windows + p] = end
 // of that chunk in the sub-wave streams (inclusive prefix sum over the windows); wave_len[wave] =
-// length of every sub-wave stream of the wavefront, rounded up to a multiple of 8.
+// length of every sub-wave stream of the wavefront, rounded up to whole tiles of 32 entries.
 template <int P>
 __global__ __launch_bounds__(kBlock) void sweep_chunks_kernel(int32_t n_windows, int32_t limit,
                                                               const int32_t* __restrict__ piece_of,
@@ -220,7 +220,7 @@ __global__ __launch_bounds__(kBlock) void sweep_chunks_kernel(int32_t n_windows,
     if (p < n_windows) chunk_end[wave * n_windows + p] = (int32_t)(carry + before + longest);
     carry += total;
   }
-  if (threadIdx.x == 0) wave_len[wave] = (carry + 7u) & ~7u;
+  if (threadIdx.x == 0) wave_len[wave] = (carry + (uint32_t)(kTile - 1)) & ~(uint32_t)(kTile - 1);
 }
 
 // stream_len[w] = P * wave_len[w] (entries of the wavefront in the stream arrays); [n_waves] = 0.
@@ -244,7 +244,8 @@ __global__ __launch_bounds__(kBlock) void sweep_clear_stream_kernel(int64_t n, i
 // Every nonzero goes to its place: wave_base + sub-wave * wave_len + start of the window's chunk +
 // position of its run in the chunk + rank in the run.
 __global__ __launch_bounds__(kBlock) void sweep_fill_kernel(int64_t nnz, int32_t n_windows, int wshift, int32_t limit,
-                                                            int32_t slots, const int32_t* __restrict__ nnz_row,
+                                                            int32_t slots, int32_t lanes,
+                                                            const int32_t* __restrict__ nnz_row,
                                                             const int32_t* __restrict__ rowptr,
                                                             const int32_t* __restrict__ col,
                                                             const uint32_t* __restrict__ pbase,
@@ -275,7 +276,12 @@ __global__ __launch_bounds__(kBlock) void sweep_fill_kernel(int64_t nnz, int32_t
   const int64_t chunk = p > 0 ? chunk_end[wave * n_windows + p - 1] : 0;
   const int64_t pos = (int64_t)wave_base[wave] + (int64_t)(at >> 28) * wave_len[wave] + chunk + (at & 0x0FFFFFFFu) + rank;
   vent[pos] = c | ((slot % slots) << kSweepColBits) | (last ? kSweepFlush : 0);
-  vsrc[pos] = (int32_t)j;
+  // The value indices of a tile of 32 entries are stored lane-major: lane l of the sub-wave (of
+  // `lanes` lanes) fetches 32 / lanes of them with one load, and they belong to the entries l, l +
+  // lanes, ... of the tile, so that one gather instruction of the values covers neighbouring entries
+  // (mostly one line of the value array per piece instead of one per lane).
+  const int32_t u = (int32_t)(pos % kTile);  // the streams start at multiples of 32
+  vsrc[pos - u + (u % lanes) * (kTile / lanes) + u / lanes] = (int32_t)j;
 }
 
 // slot_row[slot] = what the slot's result is: row r >= 0 (a whole row, stored to C), ~i (partial
@@ -319,14 +325,13 @@ __global__ __launch_bounds__(kBlock) void sweep_collect_rows_kernel(int64_t rows
   if (hit) list[base + __popcll(mask & ((1ull << lane) - 1ull))] = (int32_t)i;
 }
 
-// dst[q] = value of stream position q (0 for padding): the values in stream order, once, for a
-// caller who has declared them constant.
-__global__ __launch_bounds__(kBlock) void sweep_gather_values_kernel(int64_t n, const int32_t* __restrict__ vent,
-                                                                     const int32_t* __restrict__ vsrc,
+// dst[q] = val[vsrc[q]]: the values in the order of the index stream (padding reads index 0; the
+// kernel ignores what it finds there), once, for a caller who has declared them constant.
+__global__ __launch_bounds__(kBlock) void sweep_gather_values_kernel(int64_t n, const int32_t* __restrict__ vsrc,
                                                                      const float* __restrict__ val,
                                                                      float* __restrict__ dst) {
   for (int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x; q < n; q += (int64_t)gridDim.x * kBlock)
-    dst[q] = (vent[q] & kSweepPad) ? 0.f : val[vsrc[q]];
+    dst[q] = val[vsrc[q]];
 }
 
 // ---- SpMM kernels ----------------------------------------------------------
@@ -403,10 +408,7 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
     load_run<TL>(ent, vent, pos, e, true);
     if constexpr (kInPlace) {
 #pragma unroll
-      for (int i = 0; i < TL; ++i) {
-        const float v = vval[src[i]];
-        val[i] = (ent[i] & kSweepPad) ? 0.f : v;  // whatever value sits at index 0 must not meet the zeros as inf * 0
-      }
+      for (int i = 0; i < TL; ++i) val[i] = vval[src[i]];  // of the tile's entries l, l + G, ...
     } else {
       load_run<TL>(val, vval, pos, e, true);
     }
@@ -415,14 +417,14 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
     const int at = sbase + l * TL;
     if constexpr (TL == 4) {
       *reinterpret_cast<int4*>(s_ent + at) = make_int4(ent[0], ent[1], ent[2], ent[3]);
-      *reinterpret_cast<float4*>(s_val + at) = make_float4(val[0], val[1], val[2], val[3]);
     } else if constexpr (TL == 2) {
       *reinterpret_cast<int2*>(s_ent + at) = make_int2(ent[0], ent[1]);
-      *reinterpret_cast<float2*>(s_val + at) = make_float2(val[0], val[1]);
     } else {
       s_ent[at] = ent[0];
-      s_val[at] = val[0];
     }
+    // the values arrive lane-major (see sweep_fill_kernel) and are staged in processing order
+#pragma unroll
+    for (int i = 0; i < TL; ++i) s_val[sbase + i * G + l] = val[i];
   };
 
   // window bookkeeping, uniform over the wavefront: `window` = the one the next tile starts in
@@ -483,7 +485,8 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
       for (int i = 0; i < kBatch; ++i) b[i] = loadb(w[i]);
 #pragma unroll
       for (int i = 0; i < kBatch; ++i) {
-        fma4(acc, v[i], b[i]);
+        // padding: whatever value sits at index 0 must not meet the zeros as inf * 0
+        fma4(acc, (w[i] & kSweepPad) ? 0.f : v[i], b[i]);
         if (w[i] < 0) {
           float4* a = reinterpret_cast<float4*>(acc_wave + ((w[i] >> kSweepColBits) & (WS - 1)) * K + 4 * l);
           float4 sum = *a;

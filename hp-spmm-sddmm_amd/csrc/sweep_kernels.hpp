@@ -232,12 +232,12 @@ __global__ __launch_bounds__(kBlock) void sweep_stream_lengths_kernel(int64_t n_
   stream_len[w] = w < n_waves ? wave_len[w] * (uint32_t)P : 0u;
 }
 
-// Padding everywhere: the padding flag, value index 0.
+// Padding everywhere: the padding flag, value index -1 (= the value 0).
 __global__ __launch_bounds__(kBlock) void sweep_clear_stream_kernel(int64_t n, int32_t* __restrict__ vent,
                                                                     int32_t* __restrict__ vsrc) {
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
     vent[i] = kSweepPad;
-    vsrc[i] = 0;
+    vsrc[i] = -1;
   }
 }
 
@@ -325,13 +325,13 @@ __global__ __launch_bounds__(kBlock) void sweep_collect_rows_kernel(int64_t rows
   if (hit) list[base + __popcll(mask & ((1ull << lane) - 1ull))] = (int32_t)i;
 }
 
-// dst[q] = val[vsrc[q]]: the values in the order of the index stream (padding reads index 0; the
-// kernel ignores what it finds there), once, for a caller who has declared them constant.
+// dst[q] = val[vsrc[q]], 0 for padding: the values in the order of the index stream, once, for a
+// caller who has declared them constant.
 __global__ __launch_bounds__(kBlock) void sweep_gather_values_kernel(int64_t n, const int32_t* __restrict__ vsrc,
                                                                      const float* __restrict__ val,
                                                                      float* __restrict__ dst) {
   for (int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x; q < n; q += (int64_t)gridDim.x * kBlock)
-    dst[q] = val[vsrc[q]];
+    dst[q] = vsrc[q] < 0 ? 0.f : val[vsrc[q]];
 }
 
 // ---- SpMM kernels ----------------------------------------------------------
@@ -401,14 +401,18 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
   int32_t src[TL], ent[TL];
   float val[TL];
   auto fetch_src = [&](int64_t t) {
-    if constexpr (kInPlace) load_run<TL>(src, vsrc, t + l * TL, e, true);  // 0 beyond e: a readable index
+    if constexpr (kInPlace) load_run<TL>(src, vsrc, t + l * TL, e, true);
   };
   auto fetch = [&](int64_t t) {
     const int64_t pos = t + l * TL;
     load_run<TL>(ent, vent, pos, e, true);
     if constexpr (kInPlace) {
 #pragma unroll
-      for (int i = 0; i < TL; ++i) val[i] = vval[src[i]];  // of the tile's entries l, l + G, ...
+      for (int i = 0; i < TL; ++i) {  // of the tile's entries l, l + G, ...
+        // padding (index -1) is the value 0: whatever else it read must not meet the zeros it gathers as inf * 0
+        const float v = vval[src[i] < 0 ? 0 : src[i]];
+        val[i] = src[i] < 0 ? 0.f : v;
+      }
     } else {
       load_run<TL>(val, vval, pos, e, true);
     }
@@ -485,8 +489,7 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
       for (int i = 0; i < kBatch; ++i) b[i] = loadb(w[i]);
 #pragma unroll
       for (int i = 0; i < kBatch; ++i) {
-        // padding: whatever value sits at index 0 must not meet the zeros as inf * 0
-        fma4(acc, (w[i] & kSweepPad) ? 0.f : v[i], b[i]);
+        fma4(acc, v[i], b[i]);
         if (w[i] < 0) {
           float4* a = reinterpret_cast<float4*>(acc_wave + ((w[i] >> kSweepColBits) & (WS - 1)) * K + 4 * l);
           float4 sum = *a;

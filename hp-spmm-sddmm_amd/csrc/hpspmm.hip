@@ -1499,6 +1499,7 @@ constexpr int kSweepSpinLimit = 400;
 // 1 MB with lead 2: 1.09 / 1.70 / 2.92, lead 4: 1.12 / 1.71 / 3.07; 256 KB with lead 4: 1.09 / 1.67 / 3.15.
 inline int sweep_lead(int64_t k) { return k >= 128 ? 3 : 2; }
 // Automatic choice: B beyond what the L2s hold between them without help, enough work to fill the device.
+constexpr double kSweepMinSpan = 0.5;  // mean distance from a row's first to its last column, as a share of the columns
 constexpr int64_t kSweepMinNnz = (int64_t)1 << 22;
 constexpr int64_t kSweepMinBBytes = (int64_t)5 << 20;  // social graph: 6 MB of B, sweep 103 / 127 us against 123 / 141; 3 MB: 90 / 65 against 87 / 63
 
@@ -1566,6 +1567,22 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   const int64_t n_windows = ceil_div(p->cols, (int64_t)1 << wshift);
   if (n_windows > kSweepMaxWindows) return HPSPMM_OK;
   if (!columns_sorted(p, d_col, st)) return HPSPMM_OK;  // a row must meet the windows in stored order
+  if (!forced) {
+    // rows that reach across most of the columns (a banded matrix is better off with whole rows or segments)
+    unsigned long long* d_span = nullptr;
+    unsigned long long span = 0;
+    HPSPMM_HIP(hipMalloc(&d_span, sizeof span));
+    hipError_t e = hipMemsetAsync(d_span, 0, sizeof span, st);
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL(hpspmm::sweep_row_span_kernel, dim3(grid_for(rows, 4096)), dim3(hpspmm::kBlock), 0, st, rows,
+                         d_rowptr, d_col, d_span);
+      e = hipMemcpyAsync(&span, d_span, sizeof span, hipMemcpyDeviceToHost, st);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    (void)hipFree(d_span);
+    if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "row span: %s", hipGetErrorString(e));
+    if ((double)span < kSweepMinSpan * (double)p->cols * (double)std::max<int64_t>(1, rows - p->empty_rows)) return HPSPMM_OK;
+  }
 
   DeviceTemps tmp;
   // pieces per row, their scans

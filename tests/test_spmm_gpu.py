@@ -918,3 +918,26 @@ def test_sweep_layout_corners(pkg, oracle, gpu):
     C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SWEEP)
     assert info["strategy"] == capi.STRATEGY_SEGMENTS, info
     _check(oracle, g, B, C, "sweep forced on unsorted columns")
+
+
+def test_sweep_is_not_chosen_for_a_banded_matrix(pkg, oracle, gpu):
+    """Long rows over a large B, but every row inside a narrow band of columns: the walk over B would
+    leave each wavefront busy in a few windows of its own, so the plan keeps to another strategy (and
+    the forced sweep still gives the right product)."""
+    capi = pkg.capi
+    rng = np.random.default_rng(5)
+    rows = cols = 40000
+    per_row, half_band = 128, 600
+    centre = np.arange(rows)
+    lo = np.clip(centre - half_band, 0, cols - 2 * half_band)
+    col = np.sort(lo[:, None] + np.argsort(rng.random((rows, 2 * half_band)), axis=1)[:, :per_row], axis=1)
+    rowptr = (np.arange(rows + 1) * per_row).astype(np.int32)
+    g = pkg.graphs.CSR(rows, cols, rowptr, col.reshape(-1).astype(np.int32),
+                       rng.uniform(-1, 1, rows * per_row).astype(np.float32))
+    B = pkg.graphs.dense_normal(cols, 64, 8)
+    C, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+    assert info["strategy"] != capi.STRATEGY_SWEEP, info
+    _check(oracle, g, B, C, "banded, default plan")
+    C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SWEEP)
+    assert info["strategy"] == capi.STRATEGY_SWEEP, info
+    _check(oracle, g, B, C, "banded, forced sweep")

@@ -64,11 +64,11 @@ ROOFLINE_WORKLOAD = ("c2_social", 128)
 # measured on: same workload, K, strategy and number of launches, scale 1, default plan.
 MEASURED_TRAFFIC = {
     ("c2_social", 32): {"strategy": 6, "launches": 2, "profile": "profiles/spmm_sweep_kernel__c2_social.txt",
-                        "kernels": {"spmm_sweep_kernel": 4.584, "spmm_sweep_final_kernel": 0.012}},
+                        "kernels": {"spmm_sweep_kernel": 3.922, "spmm_sweep_final_kernel": 0.012}},
     ("c2_social", 64): {"strategy": 6, "launches": 2, "profile": "profiles/spmm_sweep_kernel__c2_social.txt",
-                        "kernels": {"spmm_sweep_kernel": 4.672, "spmm_sweep_final_kernel": 0.010}},
+                        "kernels": {"spmm_sweep_kernel": 4.034, "spmm_sweep_final_kernel": 0.010}},
     ("c2_social", 128): {"strategy": 6, "launches": 2, "profile": "profiles/spmm_sweep_kernel__c2_social.txt",
-                         "kernels": {"spmm_sweep_kernel": 6.700, "spmm_sweep_final_kernel": 0.019}},
+                         "kernels": {"spmm_sweep_kernel": 6.376, "spmm_sweep_final_kernel": 0.019}},
     ("c3_copurchase", 64): {"strategy": 5, "launches": 2, "profile": "profiles/spmm_ordered_kernel__c3_copurchase.txt",
                             "kernels": {"spmm_ordered_kernel": 21.274, "spmm_fixup_kernel": 0.203}},
     ("c4_rmat", 128): {"strategy": 4, "launches": 3, "profile": "profiles/spmm_routed_kernel__c4_rmat.txt",

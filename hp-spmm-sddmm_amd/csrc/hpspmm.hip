@@ -639,6 +639,64 @@ int exclusive_scan_u32(const uint32_t* d_in, uint32_t* d_out, int64_t n, hipStre
   return HPSPMM_OK;
 }
 
+// Frees what it holds when it goes out of scope (temporaries of a plan-construction step).
+struct DeviceTemps {
+  std::vector<void*> held;
+  ~DeviceTemps() {
+    for (void* q : held)
+      if (q) (void)hipFree(q);
+  }
+  template <class T>
+  int alloc(T** out, size_t count) {
+    *out = nullptr;
+    void* q = nullptr;
+    if (hipMalloc(&q, std::max<size_t>(count, 1) * sizeof(T)) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the plan failed", count * sizeof(T));
+    }
+    held.push_back(q);
+    *out = (T*)q;
+    return HPSPMM_OK;
+  }
+  // One allocation cut into pieces (an allocation costs 50-200 us, a plan step has a dozen temporaries):
+  // room(count) for every piece first, then reserve(), then take() in the same order.
+  size_t arena_bytes = 0, arena_used = 0;
+  char* arena = nullptr;
+  template <class T>
+  void room(size_t count) { arena_bytes += (std::max<size_t>(count, 1) * sizeof(T) + 255) & ~(size_t)255; }
+  int reserve() {
+    if (int rc = alloc(&arena, arena_bytes)) return rc;
+    arena_used = 0;
+    return HPSPMM_OK;
+  }
+  template <class T>
+  T* take(size_t count) {
+    T* out = reinterpret_cast<T*>(arena + arena_used);
+    arena_used += (std::max<size_t>(count, 1) * sizeof(T) + 255) & ~(size_t)255;
+    return out;
+  }
+};
+
+// Stable LSD radix sort of n (key, value) pairs over the low `bits` bits of the keys.  d_keys[0] /
+// d_vals[0] hold the input, [1] are buffers of the same size, d_hist has 256 * tiles + 1 counters,
+// d_scan_scratch scan_scratch_words(256 * tiles) words; returns in *result which of the two value
+// buffers holds the sorted values.  Launches only.
+int radix_sort_pairs(int64_t n, uint32_t* d_keys[2], int32_t* d_vals[2], uint32_t* d_hist, uint32_t* d_scan_scratch,
+                     int bits, hipStream_t st, int* result) {
+  const int64_t n_tiles = ceil_div(n, hpspmm::kSortTile);
+  int cur = 0;
+  for (int shift = 0; shift < bits; shift += 8) {
+    hipLaunchKernelGGL(hpspmm::sort_count_kernel, dim3((unsigned)n_tiles), dim3(hpspmm::kBlock), 0, st, n, d_keys[cur],
+                       shift, n_tiles, d_hist);
+    if (int rc = exclusive_scan_u32(d_hist, d_hist, 256 * n_tiles, st, d_scan_scratch)) return rc;
+    hipLaunchKernelGGL(hpspmm::sort_scatter_kernel, dim3((unsigned)n_tiles), dim3(hpspmm::kBlock), 0, st, n,
+                       d_keys[cur], d_vals[cur], shift, n_tiles, d_hist, d_keys[cur ^ 1], d_vals[cur ^ 1]);
+    cur ^= 1;
+  }
+  *result = cur;
+  return HPSPMM_OK;
+}
+
 // Column popularity, on the device: d_count[c] = nonzeros in column c, and d_ids = the `want` most
 // referenced columns in order of decreasing count (ties by lower index, so the choice is
 // reproducible); columns referenced fewer than twice are dropped.  One object per plan construction:
@@ -656,8 +714,6 @@ struct ColumnRanking {
   }
 };
 
-// Rank-by-counting sorts up to this many keys (m^2 compares: 0.5 ms at 2^16, 2 ms at 2^17).
-constexpr int64_t kRankMaxKeys = (int64_t)1 << 17;
 
 // Histogram of every `stride`-th column index into a fresh d_count_out (caller frees).
 int count_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t stride, hipStream_t st, int32_t** d_count_out) {
@@ -768,32 +824,38 @@ int rank_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t want, hipSt
   HPSPMM_HIP(hipMalloc(&rk.d_ids, (size_t)std::max<int64_t>(1, m) * sizeof(int32_t)));
   if (m == 0) return HPSPMM_OK;
   unsigned long long served = 0;
-  if (m <= kRankMaxKeys) {
-    unsigned long long* d_served = nullptr;
-    HPSPMM_HIP(hipMalloc(&d_served, sizeof(unsigned long long)));
-    hipError_t e = hipMemsetAsync(d_served, 0, sizeof(unsigned long long), st);
-    if (e == hipSuccess) {
-      hipLaunchKernelGGL(hpspmm::rank_sort_kernel, dim3((unsigned)ceil_div(m, hpspmm::kBlock)), dim3(hpspmm::kBlock), 0,
-                         st, (int32_t)m, d_keys, rk.d_ids, d_served);
-      e = hipMemcpyAsync(&served, d_served, sizeof served, hipMemcpyDeviceToHost, st);
+  {
+    // The keys arrive in column order within "above the threshold" and then "at the threshold": a
+    // stable sort by inverted count alone leaves ties in column order, as a sort of the whole keys would.
+    DeviceTemps tmp;
+    const int64_t n_tiles = ceil_div(m, hpspmm::kSortTile);
+    for (int i = 0; i < 2; ++i) {
+      tmp.room<uint32_t>((size_t)m);
+      tmp.room<int32_t>((size_t)m);
     }
-    if (e == hipSuccess) e = hipStreamSynchronize(st);
-    (void)hipFree(d_served);
+    tmp.room<uint32_t>((size_t)(256 * n_tiles + 1));
+    tmp.room<uint32_t>((size_t)scan_scratch_words(256 * n_tiles));
+    tmp.room<unsigned long long>(1);
+    if (int rc = tmp.reserve()) return rc;
+    uint32_t* d_sort_keys[2];
+    int32_t* d_sort_ids[2];
+    for (int i = 0; i < 2; ++i) {
+      d_sort_keys[i] = tmp.take<uint32_t>((size_t)m);
+      d_sort_ids[i] = tmp.take<int32_t>((size_t)m);
+    }
+    uint32_t* d_hist = tmp.take<uint32_t>((size_t)(256 * n_tiles + 1));
+    uint32_t* d_scan = tmp.take<uint32_t>((size_t)scan_scratch_words(256 * n_tiles));
+    unsigned long long* d_served = tmp.take<unsigned long long>(1);
+    HPSPMM_HIP(hipMemsetAsync(d_served, 0, sizeof(unsigned long long), st));
+    hipLaunchKernelGGL(hpspmm::rank_split_kernel, dim3((unsigned)ceil_div(m, hpspmm::kBlock)), dim3(hpspmm::kBlock), 0, st,
+                       (int32_t)m, d_keys, d_sort_keys[0], d_sort_ids[0], d_served);
+    int sorted = 0;
+    if (int rc = radix_sort_pairs(m, d_sort_keys, d_sort_ids, d_hist, d_scan, 32, st, &sorted)) return rc;
+    HPSPMM_HIP(hipMemcpyAsync(rk.d_ids, d_sort_ids[sorted], (size_t)m * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
+    HPSPMM_HIP(hipMemcpyAsync(&served, d_served, sizeof served, hipMemcpyDeviceToHost, st));
+    hipError_t e = hipStreamSynchronize(st);
+    if (e == hipSuccess) e = hipGetLastError();
     if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "column ranking failed: %s", hipGetErrorString(e));
-  } else {
-    // more keys than the counting sort is meant for (a hub cache of millions of rows, asked for by
-    // flag): sorted on the host
-    std::vector<unsigned long long> keys((size_t)m);
-    HPSPMM_HIP(hipMemcpyAsync(keys.data(), d_keys, keys.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost, st));
-    HPSPMM_HIP(hipStreamSynchronize(st));
-    std::sort(keys.begin(), keys.end());
-    std::vector<int32_t> ids((size_t)m);
-    for (size_t i = 0; i < keys.size(); ++i) {
-      ids[i] = (int32_t)(uint32_t)keys[i];
-      served += (unsigned long long)(~(uint32_t)(keys[i] >> 32));
-    }
-    HPSPMM_HIP(hipMemcpyAsync(rk.d_ids, ids.data(), ids.size() * sizeof(int32_t), hipMemcpyHostToDevice, st));
-    HPSPMM_HIP(hipStreamSynchronize(st));
   }
   rk.n_ids = m;
   rk.served = (int64_t)served * rk.stride;
@@ -1277,6 +1339,12 @@ constexpr int64_t kClusterMinMeanNnz = 8;
 // ... and its order is kept if this share of the nonzeros then reads B from LDS.
 constexpr double kClusterMinServed = 0.15;
 
+// Integer from the environment (diagnostic overrides of the plan's defaults).
+int env_int(const char* name, int fallback) {
+  const char* v = std::getenv(name);
+  return v && *v ? std::atoi(v) : fallback;
+}
+
 // Finds a processing order for a square matrix by label propagation on its graph: rows of one
 // label next to each other, labels in increasing order, rows of a label in increasing order.
 // d_order_out receives a device array of `rows` entries (caller frees).
@@ -1343,9 +1411,12 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
   std::vector<uint32_t> counters((size_t)hpspmm::kClusterCounters);
   hipLaunchKernelGGL(hpspmm::cluster_init_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock),
                      0, st, rows, d_label);
-  for (int sweep = 0; sweep < kClusterMaxSweeps; ++sweep) {
+  const int max_sweeps = std::max(1, env_int("HPSPMM_CLUSTER_SWEEPS", kClusterMaxSweeps));  // diagnostics
+  const bool debug = std::getenv("HPSPMM_CLUSTER_DEBUG") != nullptr;
+  for (int sweep = 0; sweep < max_sweeps; ++sweep) {
     HPSPMM_HIP(hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st));
-    hipLaunchKernelGGL(hpspmm::cluster_sweep_kernel, dim3((unsigned)ceil_div(ceil_div(rows, 2), hpspmm::kWavesPerBlock)),
+    hipLaunchKernelGGL(hpspmm::cluster_sweep_kernel,
+                       dim3((unsigned)ceil_div(ceil_div(rows, 2), hpspmm::kWavesPerBlock * hpspmm::kClusterRowsPerWave)),
                        dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_label, d_label_next, (uint32_t)sweep,
                        d_changed);
     std::swap(d_label, d_label_next);
@@ -1354,6 +1425,7 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
     HPSPMM_HIP(hipStreamSynchronize(st));
     int64_t changed = 0;
     for (uint32_t c : counters) changed += c;
+    if (debug) fprintf(stderr, "cluster sweep %d: %lld of %lld rows changed their label\n", sweep, (long long)changed, (long long)rows);
     if (changed * 200 < rows) break;
   }
   // share of the nonzeros that stay inside a cluster small enough for a workgroup's window
@@ -1376,6 +1448,7 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
     int64_t intra = 0;
     for (uint32_t c : counters) intra += c;
     *intra_share_out = p->nnz > 0 ? (double)intra / (double)p->nnz : 0.0;
+    if (debug) fprintf(stderr, "cluster: %.4f of the nonzeros inside clusters of at most %d rows\n", *intra_share_out, kClusterMaxSize);
   }
   // rows ordered by label, the rows of a label in increasing order: a stable sort, hence the same
   // order on every run
@@ -1425,69 +1498,6 @@ int build_hub_cache(hpspmm_plan* p, const int32_t* d_col, int log2_hubs, bool fo
 // ---------------------------------------------------------------------------------------------
 // Sweep strategy: plan construction and launch.
 // ---------------------------------------------------------------------------------------------
-
-// Frees what it holds when it goes out of scope (temporaries of a plan-construction step).
-struct DeviceTemps {
-  std::vector<void*> held;
-  ~DeviceTemps() {
-    for (void* q : held)
-      if (q) (void)hipFree(q);
-  }
-  template <class T>
-  int alloc(T** out, size_t count) {
-    *out = nullptr;
-    void* q = nullptr;
-    if (hipMalloc(&q, std::max<size_t>(count, 1) * sizeof(T)) != hipSuccess) {
-      (void)hipGetLastError();
-      return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the plan failed", count * sizeof(T));
-    }
-    held.push_back(q);
-    *out = (T*)q;
-    return HPSPMM_OK;
-  }
-  // One allocation cut into pieces (an allocation costs 50-200 us, a plan step has a dozen temporaries):
-  // room(count) for every piece first, then reserve(), then take() in the same order.
-  size_t arena_bytes = 0, arena_used = 0;
-  char* arena = nullptr;
-  template <class T>
-  void room(size_t count) { arena_bytes += (std::max<size_t>(count, 1) * sizeof(T) + 255) & ~(size_t)255; }
-  int reserve() {
-    if (int rc = alloc(&arena, arena_bytes)) return rc;
-    arena_used = 0;
-    return HPSPMM_OK;
-  }
-  template <class T>
-  T* take(size_t count) {
-    T* out = reinterpret_cast<T*>(arena + arena_used);
-    arena_used += (std::max<size_t>(count, 1) * sizeof(T) + 255) & ~(size_t)255;
-    return out;
-  }
-};
-
-// Stable LSD radix sort of n (key, value) pairs over the low `bits` bits of the keys.  d_keys[0] /
-// d_vals[0] hold the input, [1] are buffers of the same size, d_hist has 256 * tiles + 1 counters,
-// d_scan_scratch scan_scratch_words(256 * tiles) words; returns in *result which of the two value
-// buffers holds the sorted values.  Launches only.
-int radix_sort_pairs(int64_t n, uint32_t* d_keys[2], int32_t* d_vals[2], uint32_t* d_hist, uint32_t* d_scan_scratch,
-                     int bits, hipStream_t st, int* result) {
-  const int64_t n_tiles = ceil_div(n, hpspmm::kSortTile);
-  int cur = 0;
-  for (int shift = 0; shift < bits; shift += 8) {
-    hipLaunchKernelGGL(hpspmm::sort_count_kernel, dim3((unsigned)n_tiles), dim3(hpspmm::kBlock), 0, st, n, d_keys[cur],
-                       shift, n_tiles, d_hist);
-    if (int rc = exclusive_scan_u32(d_hist, d_hist, 256 * n_tiles, st, d_scan_scratch)) return rc;
-    hipLaunchKernelGGL(hpspmm::sort_scatter_kernel, dim3((unsigned)n_tiles), dim3(hpspmm::kBlock), 0, st, n,
-                       d_keys[cur], d_vals[cur], shift, n_tiles, d_hist, d_keys[cur ^ 1], d_vals[cur ^ 1]);
-    cur ^= 1;
-  }
-  *result = cur;
-  return HPSPMM_OK;
-}
-
-int env_int(const char* name, int fallback) {
-  const char* v = std::getenv(name);
-  return v && *v ? std::atoi(v) : fallback;
-}
 
 constexpr int kSweepMaxBands = 64;
 constexpr int32_t kSweepMaxWindows = 8192;
@@ -1629,7 +1639,6 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   tmp.room<uint32_t>((size_t)(256 * n_tiles + 1));
   tmp.room<uint32_t>(scan_words);
   tmp.room<int32_t>(n_pieces);
-  tmp.room<int32_t>(n_pieces);
   tmp.room<int32_t>((size_t)n_slots);
   tmp.room<int32_t>((size_t)rows * (size_t)(n_windows + 1));
   tmp.room<int32_t>((size_t)n_slots * (size_t)n_windows);
@@ -1645,7 +1654,6 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   uint32_t* d_hist = tmp.take<uint32_t>((size_t)(256 * n_tiles + 1));
   uint32_t* d_scan = tmp.take<uint32_t>(scan_words);
   int32_t* d_piece_row = tmp.take<int32_t>(n_pieces);
-  int32_t* d_slot_of = tmp.take<int32_t>(n_pieces);
   int32_t* d_piece_of = tmp.take<int32_t>((size_t)n_slots);
   int32_t* d_wstart = tmp.take<int32_t>((size_t)rows * (size_t)(n_windows + 1));
   int32_t* d_run_at = tmp.take<int32_t>((size_t)n_slots * (size_t)n_windows);
@@ -1660,7 +1668,7 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   HPSPMM_HIP(hipMemsetAsync(d_piece_of, 0xFF, (size_t)n_slots * sizeof(int32_t), st));
   hipLaunchKernelGGL(hpspmm::sweep_assign_kernel, dim3((unsigned)ceil_div((int64_t)n_pieces, hpspmm::kBlock)),
                      dim3(hpspmm::kBlock), 0, st, (int64_t)n_pieces, d_vals[sorted], (int32_t)n_bands, (int32_t)band_waves,
-                     (int32_t)WS, d_slot_of, d_piece_of);
+                     (int32_t)WS, d_piece_of);
 
   // where every row enters every window
   hipLaunchKernelGGL(hpspmm::sweep_row_windows_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)),
@@ -1697,8 +1705,13 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
     HPSPMM_HIP(hipMemcpyAsync(lens.data(), p->d_sw_len, (size_t)n_waves * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
     HPSPMM_HIP(hipStreamSynchronize(st));
     int64_t total = 0;
-    for (uint32_t v : lens) total += (int64_t)v * P;
-    if (total >= INT32_MAX - 64) {
+    uint32_t longest = 0;
+    for (uint32_t v : lens) {
+      total += (int64_t)v * P;
+      longest = std::max(longest, v);
+    }
+    // (positions within a window's chunk are kept in 28 bits while the streams are laid out)
+    if (total >= INT32_MAX - 64 || longest >= (1u << 28)) {
       drop_sweep_buffers(p);
       return HPSPMM_OK;
     }
@@ -1719,10 +1732,9 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   }
   hipLaunchKernelGGL(hpspmm::sweep_clear_stream_kernel, dim3(grid_for(total, 1 << 16)), dim3(hpspmm::kBlock), 0, st, total,
                      p->d_vcol, p->d_vsrc);
-  hipLaunchKernelGGL(hpspmm::sweep_fill_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)), dim3(hpspmm::kBlock), 0, st,
-                     nnz, (int32_t)n_windows, wshift, limit, (int32_t)WS, (int32_t)(k / 4), p->d_nnz_row, d_rowptr, d_col,
-                     d_pbase, d_slot_of,
-                     d_wstart, d_run_at, p->d_sw_ends, p->d_sw_base, p->d_sw_len, p->d_vcol, p->d_vsrc);
+  hipLaunchKernelGGL(hpspmm::sweep_fill_kernel, wave_grid, dim3(hpspmm::kBlock), 0, st, (int32_t)n_windows, wshift, limit,
+                     (int32_t)WS, (int32_t)(k / 4), d_piece_of, d_piece_row, d_pbase, d_rowptr, d_col, d_wstart, d_run_at,
+                     p->d_sw_ends, p->d_sw_base, p->d_sw_len, p->d_vcol, p->d_vsrc);
   hipLaunchKernelGGL(hpspmm::sweep_slot_rows_kernel, dim3((unsigned)ceil_div(n_slots, hpspmm::kBlock)), dim3(hpspmm::kBlock),
                      0, st, n_slots, d_piece_of, d_piece_row, d_pbase, d_part, d_rowptr, limit, p->d_sw_slot_row);
 
@@ -1940,7 +1952,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     }
     p->workspace_bytes = (int64_t)(row_bytes + carry_bytes);
     if (nnz > 0) {
-      hipLaunchKernelGGL(hpspmm::expand_rows_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)),
+      hipLaunchKernelGGL(hpspmm::expand_rows_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kExpandPerBlock)),
                          dim3(hpspmm::kBlock), 0, st, rows, nnz, d_rowptr, p->d_nnz_row);
       hipError_t e = hipStreamSynchronize(st);
       if (e != hipSuccess) {
@@ -2281,7 +2293,7 @@ int launch_static(int64_t rows, int64_t nnz, const int32_t* rp, const int32_t* c
   while (2 * ceil_div(nnz, (int64_t)1 << shift) * K > kStaticCarryFloats) ++shift;
   const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
   if (nnz > 0) {
-    hipLaunchKernelGGL(hpspmm::expand_rows_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+    hipLaunchKernelGGL(hpspmm::expand_rows_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kExpandPerBlock)), dim3(hpspmm::kBlock),
                        0, st, rows, nnz, rp, nnz_row);
     const int64_t nblocks = ceil_div(ceil_div(nseg, P), hpspmm::kWavesPerBlock);
     hipLaunchKernelGGL((hpspmm::spmm_segments_kernel<K, false, false>), dim3((unsigned)nblocks), dim3(hpspmm::kBlock),

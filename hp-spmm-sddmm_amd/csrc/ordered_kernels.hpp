@@ -46,37 +46,16 @@ namespace hpspmm {
 // plans of one matrix get the same labels), and only half of the rows may
 // change - of every pair of rows (2w, 2w + 1) the one a hash of w and the sweep
 // picks: with every row updated at once from the old labels, neighbours swap
-// labels back and forth instead of settling.  One wavefront per pair (it copies
+// labels back and forth instead of settling.  A wavefront per pair in turn (it copies
 // the label of the row that sits the sweep out); the 64 sampled labels are
 // sorted by a bitonic network of wavefront shuffles.  The kClusterCounters
 // entries of changed[] together count the rows whose label changed.
 constexpr int kClusterCounters = 1024;
-__global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
-                                                               const int32_t* __restrict__ col,
-                                                               const int32_t* __restrict__ label_in,
-                                                               int32_t* __restrict__ label_out, uint32_t sweep,
-                                                               uint32_t* __restrict__ changed) {
-  const int lane = threadIdx.x & 63;
-  const int64_t w = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-  if (2 * w >= rows) return;
-  const uint32_t turn = (((uint32_t)w * 0x9E3779B1u) ^ ((sweep + 1u) * 0x85EBCA6Bu)) * 0xC2B2AE35u;
-  const int64_t r = 2 * w + (int64_t)((turn >> 31) & 1u) < rows ? 2 * w + (int64_t)((turn >> 31) & 1u) : 2 * w;
-  const int64_t idle = r ^ 1;  // the other row of the pair keeps its label in this sweep
-  if (lane == 1 && idle < rows) label_out[idle] = label_in[idle];
-  const int32_t mine = label_in[r];
-  const int32_t lb = rowptr[r];
-  const int32_t n = rowptr[r + 1] - lb;
-  if (n == 0) {  // wavefront-uniform
-    if (lane == 0) label_out[r] = mine;
-    return;
-  }
-  const int32_t stride = (n + 63) / 64;
-  const bool valid = lane * stride < n;
-  int32_t lab = INT32_MAX;  // sorts behind every label
-  if (valid) {
-    const int32_t c = col[lb + lane * stride];
-    if ((int64_t)c < rows) lab = label_in[c];
-  }
+constexpr int kClusterRowsPerWave = 4;  // pairs a wavefront takes, their loads in flight together
+
+// The label that row r takes: lab = the sampled neighbour labels of the wavefront's lanes
+// (INT32_MAX where a lane has none), mine = the row's own.  Same value in every lane.
+__device__ __forceinline__ int32_t cluster_vote(int32_t lab, int32_t mine, int64_t r, uint32_t sweep, int lane) {
   const int self_count = (int)__popcll(__ballot(lab == mine));
 #pragma unroll
   for (int size = 2; size <= 64; size <<= 1) {
@@ -118,10 +97,57 @@ __global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, con
     const int best_count = (int)(best >> 32);
     if (self_count < best_count && best_lab != mine) next_label = best_lab;
   }
-  if (lane == 0) {
-    label_out[r] = next_label;
-    if (next_label != mine)
-      atomicAdd(&changed[r & (kClusterCounters - 1)], 1u);  // spread: one counter would serialise the first sweep
+  return next_label;
+}
+
+// A sweep is a chain of three dependent round trips per row (row pointer, columns, labels) and
+// little else, so a wavefront takes kClusterRowsPerWave pairs and issues each stage for all of
+// them before it needs any of the answers.
+__global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                               const int32_t* __restrict__ col,
+                                                               const int32_t* __restrict__ label_in,
+                                                               int32_t* __restrict__ label_out, uint32_t sweep,
+                                                               uint32_t* __restrict__ changed) {
+  constexpr int R = kClusterRowsPerWave;
+  const int lane = threadIdx.x & 63;
+  const int64_t w0 = ((int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)) * R;
+  if (2 * w0 >= rows) return;
+  int64_t r[R];
+  bool live[R];
+  int32_t mine[R], lb[R], n[R], c[R], lab[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int64_t w = w0 + i;
+    live[i] = 2 * w < rows;
+    r[i] = 0;
+    if (!live[i]) continue;  // wavefront-uniform
+    const uint32_t turn = (((uint32_t)w * 0x9E3779B1u) ^ ((sweep + 1u) * 0x85EBCA6Bu)) * 0xC2B2AE35u;
+    r[i] = 2 * w + (int64_t)((turn >> 31) & 1u) < rows ? 2 * w + (int64_t)((turn >> 31) & 1u) : 2 * w;
+    const int64_t idle = r[i] ^ 1;  // the other row of the pair keeps its label in this sweep
+    if (lane == 1 && idle < rows) label_out[idle] = label_in[idle];
+  }
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    mine[i] = live[i] ? label_in[r[i]] : 0;
+    lb[i] = live[i] ? rowptr[r[i]] : 0;
+    n[i] = live[i] ? rowptr[r[i] + 1] - lb[i] : 0;
+  }
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int32_t stride = (n[i] + 63) / 64;
+    c[i] = lane * stride < n[i] ? col[lb[i] + lane * stride] : -1;
+  }
+#pragma unroll
+  for (int i = 0; i < R; ++i) lab[i] = (c[i] >= 0 && (int64_t)c[i] < rows) ? label_in[c[i]] : INT32_MAX;  // sorts behind every label
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    if (!live[i]) continue;
+    const int32_t next_label = cluster_vote(lab[i], mine[i], r[i], sweep, lane);
+    if (lane == 0) {
+      label_out[r[i]] = next_label;
+      if (next_label != mine[i])
+        atomicAdd(&changed[r[i] & (kClusterCounters - 1)], 1u);  // spread: one counter would serialise the first sweep
+    }
   }
 }
 

@@ -105,26 +105,17 @@ __global__ __launch_bounds__(kBlock) void select_compact_kernel(int64_t n, const
   if (slot >= 0) keys[slot] = ((unsigned long long)(~(uint32_t)c) << 32) | (uint32_t)i;
 }
 
-// ids[rank of key i] = low word of key i, rank = number of smaller keys (keys are distinct).  One
-// thread per key, the keys passed through LDS in tiles; m <= 2^17 keeps the m^2 compares cheap.
-// *served += the counts of the ranked columns.
-__global__ __launch_bounds__(kBlock) void rank_sort_kernel(int32_t m, const unsigned long long* __restrict__ keys,
-                                                           int32_t* __restrict__ ids,
-                                                           unsigned long long* __restrict__ served) {
-  __shared__ unsigned long long s_keys[kBlock];
+// The selected keys taken apart for the radix sort: sort_key[i] = high word (the inverted count:
+// ascending = most referenced first), id[i] = low word (the column).  *served += the counts.
+__global__ __launch_bounds__(kBlock) void rank_split_kernel(int32_t m, const unsigned long long* __restrict__ keys,
+                                                            uint32_t* __restrict__ sort_key, int32_t* __restrict__ id,
+                                                            unsigned long long* __restrict__ served) {
   const int32_t i = (int32_t)blockIdx.x * kBlock + threadIdx.x;
-  const unsigned long long mine = i < m ? keys[i] : ~0ull;
-  int32_t rank = 0;
-  for (int32_t t0 = 0; t0 < m; t0 += kBlock) {
-    __syncthreads();
-    s_keys[threadIdx.x] = t0 + (int32_t)threadIdx.x < m ? keys[t0 + threadIdx.x] : ~0ull;
-    __syncthreads();
-    const int32_t cnt = m - t0 < kBlock ? m - t0 : kBlock;
-    for (int32_t q = 0; q < cnt; ++q) rank += s_keys[q] < mine ? 1 : 0;
-  }
   unsigned long long c = 0;
   if (i < m) {
-    ids[rank] = (int32_t)(uint32_t)mine;
+    const unsigned long long mine = keys[i];
+    sort_key[i] = (uint32_t)(mine >> 32);
+    id[i] = (int32_t)(uint32_t)mine;
     c = (unsigned long long)(~(uint32_t)(mine >> 32));
   }
   for (int off = 32; off > 0; off >>= 1) c += __shfl_down(c, off);

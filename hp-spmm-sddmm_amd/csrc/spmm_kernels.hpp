@@ -652,20 +652,31 @@ __global__ __launch_bounds__(kBlock) void gather_hub_rows_kernel(int64_t n_hub, 
   *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) = load_b<K>(B, hub_ids[s], l);
 }
 
-// nnz_row[j] = the row r with rowptr[r] <= j < rowptr[r+1] (CSR -> COO row
-// expansion, the device-side form of spmm/mm/spmm_common.cpp:210-216).
-__global__ __launch_bounds__(kBlock) void expand_rows_kernel(int64_t rows, int64_t nnz,
-                                                             const int32_t* __restrict__ rowptr,
-                                                             int32_t* __restrict__ nnz_row) {
-  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (j >= nnz) return;
-  // largest r in [0, rows) with rowptr[r] <= j
-  int64_t lo = 0, hi = rows;  // invariant: rowptr[lo] <= j, answer in [lo, hi)
+// Largest r in [lo, hi) with rowptr[r] <= j (rowptr[lo] <= j must hold): the row of nonzero j.
+__device__ __forceinline__ int64_t row_of_nonzero(const int32_t* __restrict__ rowptr, int64_t lo, int64_t hi, int64_t j) {
   while (hi - lo > 1) {
     const int64_t mid = (lo + hi) >> 1;
     if ((int64_t)rowptr[mid] <= j) lo = mid; else hi = mid;
   }
-  nnz_row[j] = (int32_t)lo;
+  return lo;
+}
+
+// nnz_row[j] = the row r with rowptr[r] <= j < rowptr[r+1] (CSR -> COO row
+// expansion, the device-side form of spmm/mm/spmm_common.cpp:210-216).  A workgroup takes
+// kExpandPerBlock consecutive nonzeros: two threads bisect all of rowptr for its first and last
+// one, the others only between those two rows (a handful of steps instead of log2(rows)).
+constexpr int kExpandPerBlock = 4 * kBlock;
+__global__ __launch_bounds__(kBlock) void expand_rows_kernel(int64_t rows, int64_t nnz,
+                                                             const int32_t* __restrict__ rowptr,
+                                                             int32_t* __restrict__ nnz_row) {
+  __shared__ int64_t s_ends[2];
+  const int64_t first = (int64_t)blockIdx.x * kExpandPerBlock;
+  const int64_t last = first + kExpandPerBlock - 1 < nnz ? first + kExpandPerBlock - 1 : nnz - 1;
+  if (threadIdx.x == 0) s_ends[0] = row_of_nonzero(rowptr, 0, rows, first);
+  if (threadIdx.x == 64) s_ends[1] = row_of_nonzero(rowptr, 0, rows, last);
+  __syncthreads();
+  const int64_t lo = s_ends[0], hi = s_ends[1] + 1;
+  for (int64_t j = first + threadIdx.x; j <= last; j += kBlock) nnz_row[j] = (int32_t)row_of_nonzero(rowptr, lo, hi, j);
 }
 
 // out[b] = id of the XCD that workgroup b runs on (hardware register XCC_ID, bits 3:0): lets the

@@ -3,7 +3,7 @@
 // For a matrix with long rows whose B is larger than the L2s but small against the gather volume
 // (nnz * K * 4 bytes), the gather can be made L2-resident by construction instead of by popularity:
 // all wavefronts walk the columns of B in the same order and at about the same pace, window after
-// window of about a megabyte, so that at any moment the whole chip reads one short stretch of B
+// window of half a megabyte of B, so that at any moment the whole chip reads one short stretch of B
 // that every L2 holds.  What makes that possible without writing partial results to memory is that
 // the accumulators of a row stay on the chip for the whole walk:
 //
@@ -124,10 +124,9 @@ __global__ __launch_bounds__(kBlock) void sweep_piece_keys_kernel(int64_t rows, 
 
 // The i-th longest piece goes to band i % n_bands; within the band, pieces are dealt to the band's
 // wavefronts in rounds, alternately forwards and backwards; round j fills slot j of every wavefront.
-// slot_of[piece] = wavefront * slots + round, piece_of[that] = piece (preset to -1).
+// piece_of[wavefront * slots + round] = piece (preset to -1).
 __global__ __launch_bounds__(kBlock) void sweep_assign_kernel(int64_t n_pieces, const int32_t* __restrict__ order,
                                                               int32_t n_bands, int32_t band_waves, int32_t slots,
-                                                              int32_t* __restrict__ slot_of,
                                                               int32_t* __restrict__ piece_of) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= n_pieces) return;
@@ -137,9 +136,7 @@ __global__ __launch_bounds__(kBlock) void sweep_assign_kernel(int64_t n_pieces, 
   const int32_t pos = (int32_t)(within % band_waves);
   const int32_t bin = (round & 1) ? band_waves - 1 - pos : pos;
   const int32_t slot = (band * band_waves + bin) * slots + round;
-  const int32_t piece = order[i];
-  slot_of[piece] = slot;
-  piece_of[slot] = piece;
+  piece_of[slot] = order[i];
 }
 
 // wstart[r * (n_windows + 1) + p] = index of the first nonzero of row r whose column lies in window
@@ -205,28 +202,49 @@ __global__ __launch_bounds__(kBlock) void sweep_chunks_kernel(int32_t n_windows,
     const int32_t p = p0 + threadIdx.x;
     uint32_t longest = 0;
     if (p < n_windows) {
-      int32_t len[WS];
+      // key = length << 8 | (255 - slot): sorted downwards, the runs come longest first, ties lower slot first
+      int32_t key[WS];
+#pragma unroll
       for (int slot = 0; slot < WS; ++slot) {
         const int32_t row = s_row[slot];
-        len[slot] = 0;
-        if (row < 0) continue;
-        const int32_t* w = wstart + (int64_t)row * (n_windows + 1) + p;
-        const int32_t a = w[0] - s_lb[slot], b = w[1] - s_lb[slot];
-        len[slot] = sweep_count_below(b, s_m[slot], s_k[slot]) - sweep_count_below(a, s_m[slot], s_k[slot]);
+        int32_t len = 0;
+        if (row >= 0) {
+          const int32_t* w = wstart + (int64_t)row * (n_windows + 1) + p;
+          const int32_t a = w[0] - s_lb[slot], b = w[1] - s_lb[slot];
+          len = sweep_count_below(b, s_m[slot], s_k[slot]) - sweep_count_below(a, s_m[slot], s_k[slot]);
+        }
+        key[slot] = len > 0 ? (len << 8 | (255 - slot)) : 0;
+      }
+      // bitonic network over the registers (every index a compile-time constant)
+#pragma unroll
+      for (int span = 2; span <= WS; span <<= 1) {
+#pragma unroll
+        for (int step = span >> 1; step > 0; step >>= 1) {
+#pragma unroll
+          for (int i = 0; i < WS; ++i) {
+            const int l = i ^ step;
+            if (l > i) {
+              const int32_t x = key[i], y = key[l];
+              const int32_t hi = x > y ? x : y, lo = x > y ? y : x;
+              const bool down = (i & span) == 0;
+              key[i] = down ? hi : lo;
+              key[l] = down ? lo : hi;
+            }
+          }
+        }
       }
       uint32_t load[P];
       for (int q = 0; q < P; ++q) load[q] = 0;
-      for (int round = 0; round < WS; ++round) {
-        int best = 0;
-        for (int slot = 1; slot < WS; ++slot)
-          if (len[slot] > len[best]) best = slot;
-        if (len[best] <= 0) break;
-        int q = 0;
-        for (int i = 1; i < P; ++i)
-          if (load[i] < load[q]) q = i;
-        run_at[(wave * WS + best) * n_windows + p] = (int32_t)((uint32_t)q << 28 | load[q]);
-        load[q] += (uint32_t)len[best];
-        len[best] = 0;
+#pragma unroll
+      for (int i = 0; i < WS; ++i) {
+        if (key[i] != 0) {
+          const int32_t len = key[i] >> 8, slot = 255 - (key[i] & 255);
+          int q = 0;
+          for (int t = 1; t < P; ++t)
+            if (load[t] < load[q]) q = t;
+          run_at[(wave * WS + slot) * n_windows + p] = (int32_t)((uint32_t)q << 28 | load[q]);
+          load[q] += (uint32_t)len;
+        }
       }
       for (int q = 0; q < P; ++q) longest = load[q] > longest ? load[q] : longest;
     }
@@ -257,46 +275,85 @@ __global__ __launch_bounds__(kBlock) void sweep_clear_stream_kernel(int64_t n, i
 }
 
 // Every nonzero goes to its place: wave_base + sub-wave * wave_len + start of the window's chunk +
-// position of its run in the chunk + rank in the run.
-__global__ __launch_bounds__(kBlock) void sweep_fill_kernel(int64_t nnz, int32_t n_windows, int wshift, int32_t limit,
-                                                            int32_t slots, int32_t lanes,
-                                                            const int32_t* __restrict__ nnz_row,
+// position of its run in the chunk + rank in the run.  One workgroup per wavefront of the layout,
+// its threads over the nonzeros of the wavefront's pieces one after the other: reads of a piece are
+// consecutive, the entries of a run are written by neighbouring lanes, and what a workgroup writes
+// is one wavefront's streams and nothing else, so the L2 sees every line of them completed within a
+// short time (one thread per nonzero of the matrix, in matrix order, wrote a few bytes here and a
+// few there all over the streams: 2-3 ms instead of well under one on 115 M nonzeros).
+__global__ __launch_bounds__(kBlock) void sweep_fill_kernel(int32_t n_windows, int wshift, int32_t limit, int32_t slots,
+                                                            int32_t lanes, const int32_t* __restrict__ piece_of,
+                                                            const int32_t* __restrict__ piece_row,
+                                                            const uint32_t* __restrict__ pbase,
                                                             const int32_t* __restrict__ rowptr,
                                                             const int32_t* __restrict__ col,
-                                                            const uint32_t* __restrict__ pbase,
-                                                            const int32_t* __restrict__ slot_of,
                                                             const int32_t* __restrict__ wstart,
                                                             const int32_t* __restrict__ run_at,
                                                             const int32_t* __restrict__ chunk_end,
                                                             const uint32_t* __restrict__ wave_base,
                                                             const uint32_t* __restrict__ wave_len,
                                                             int32_t* __restrict__ vent, int32_t* __restrict__ vsrc) {
-  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (j >= nnz) return;
-  const int32_t r = nnz_row[j];
-  const int32_t lb = rowptr[r];
-  const int32_t m = (rowptr[r + 1] - lb + limit - 1) / limit;
-  const int32_t x = (int32_t)j - lb;
-  const int32_t k = x % m;
-  const int32_t slot = slot_of[pbase[r] + k];  // wavefront * slots + slot of the wavefront
-  const int64_t wave = slot / slots;
-  const int32_t c = col[j];
-  const int32_t p = c >> wshift;
-  const int32_t* w = wstart + (int64_t)r * (n_windows + 1) + p;
-  const int32_t a = w[0] - lb, b = w[1] - lb;
-  const int32_t first = sweep_count_below(a, m, k);
-  const int32_t rank = sweep_count_below(x, m, k) - first;
-  const bool last = sweep_count_below(b, m, k) - first == rank + 1;
-  const uint32_t at = (uint32_t)run_at[(int64_t)slot * n_windows + p];
-  const int64_t chunk = p > 0 ? chunk_end[wave * n_windows + p - 1] : 0;
-  const int64_t pos = (int64_t)wave_base[wave] + (int64_t)(at >> 28) * wave_len[wave] + chunk + (at & 0x0FFFFFFFu) + rank;
-  vent[pos] = c | ((slot % slots) << kSweepColBits) | (last ? kSweepFlush : 0);
-  // The value indices of a tile of 32 entries are stored lane-major: lane l of the sub-wave (of
-  // `lanes` lanes) fetches 32 / lanes of them with one load, and they belong to the entries l, l +
-  // lanes, ... of the tile, so that one gather instruction of the values covers neighbouring entries
-  // (mostly one line of the value array per piece instead of one per lane).
-  const int32_t u = (int32_t)(pos % kTile);  // the streams start at multiples of 32
-  vsrc[pos - u + (u % lanes) * (kTile / lanes) + u / lanes] = (int32_t)j;
+  constexpr int kMaxSlots = 64;  // 8 slots for each of at most 8 sub-waves
+  __shared__ int32_t s_row[kMaxSlots], s_lb[kMaxSlots], s_m[kMaxSlots], s_k[kMaxSlots], s_size[kMaxSlots];
+  __shared__ int32_t s_begin[kMaxSlots + 1];  // entries of the slots before this one
+  const int64_t wave = blockIdx.x;
+  if ((int)threadIdx.x < kMaxSlots) {
+    int32_t row = -1, lb = 0, m = 1, k = 0, size = 0;
+    if ((int)threadIdx.x < slots) {
+      const int32_t piece = piece_of[wave * slots + threadIdx.x];
+      if (piece >= 0) {
+        row = piece_row[piece];
+        lb = rowptr[row];
+        const int32_t len = rowptr[row + 1] - lb;
+        m = (len + limit - 1) / limit;
+        k = piece - (int32_t)pbase[row];
+        size = sweep_count_below(len, m, k);
+      }
+    }
+    s_row[threadIdx.x] = row;
+    s_lb[threadIdx.x] = lb;
+    s_m[threadIdx.x] = m;
+    s_k[threadIdx.x] = k;
+    s_size[threadIdx.x] = size;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t sum = 0;
+    for (int i = 0; i < kMaxSlots; ++i) {
+      s_begin[i] = sum;
+      sum += s_size[i];
+    }
+    s_begin[kMaxSlots] = sum;
+  }
+  __syncthreads();
+  const int64_t base = wave_base[wave];
+  const int64_t wlen = wave_len[wave];
+  const int32_t* ends = chunk_end + wave * n_windows;
+  const int32_t total = s_begin[kMaxSlots];
+  const int32_t per_lane = kTile / lanes;
+  for (int32_t e = threadIdx.x; e < total; e += kBlock) {
+    int slot = 0;  // the last slot with s_begin[slot] <= e (empty slots repeat a value: the last of them has the entries)
+#pragma unroll
+    for (int step = kMaxSlots / 2; step > 0; step >>= 1)
+      if (s_begin[slot + step] <= e) slot += step;
+    const int32_t row = s_row[slot], lb = s_lb[slot], m = s_m[slot], k = s_k[slot];
+    const int32_t x = e - s_begin[slot];  // the piece's x-th nonzero
+    const int32_t j = lb + k + x * m;     // a piece takes every m-th nonzero of its row
+    const int32_t c = col[j];
+    const int32_t p = c >> wshift;
+    const int32_t* w = wstart + (int64_t)row * (n_windows + 1) + p;
+    const int32_t first = sweep_count_below(w[0] - lb, m, k);
+    const bool last = sweep_count_below(w[1] - lb, m, k) == x + 1;
+    const uint32_t at = (uint32_t)run_at[(wave * slots + slot) * n_windows + p];
+    const int64_t pos = base + (int64_t)(at >> 28) * wlen + (p > 0 ? ends[p - 1] : 0) + (at & 0x0FFFFFFFu) + (x - first);
+    vent[pos] = c | (slot << kSweepColBits) | (last ? kSweepFlush : 0);
+    // The value indices of a tile of 32 entries are stored lane-major: lane l of the sub-wave (of
+    // `lanes` lanes) fetches 32 / lanes of them with one load, and they belong to the entries l, l +
+    // lanes, ... of the tile, so that one gather instruction of the values covers neighbouring entries
+    // (mostly one line of the value array per piece instead of one per lane).
+    const int32_t u = (int32_t)(pos % kTile);  // the streams start at multiples of 32
+    vsrc[pos - u + (u % lanes) * per_lane + u / lanes] = j;
+  }
 }
 
 // slot_row[slot] = what the slot's result is: row r >= 0 (a whole row, stored to C), ~i (partial

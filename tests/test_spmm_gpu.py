@@ -377,10 +377,10 @@ def test_other_csr_arrays_are_refused(pkg, oracle, gpu):
         plan.destroy()
 
 
-def test_hot_set_beyond_the_device_ranking(pkg, oracle, gpu):
-    """A hot set of 2^18 columns is more than the plan's counting-rank sort takes (2^17 keys): the
-    selected columns are then sorted on the host.  Forced routed strategy with that hot set and 4
-    phases on an R-MAT of 524k columns; checked on row ranges that include the heaviest rows."""
+def test_large_hot_set(pkg, oracle, gpu):
+    """A hot set of 2^18 columns, four times the plan's own choice (the selected columns are ranked by
+    a radix sort of several tiles).  Forced routed strategy with that hot set and 4 phases on an
+    R-MAT of 524k columns; checked on row ranges that include the heaviest rows."""
     capi = pkg.capi
     g = pkg.graphs.make_graph("c4_rmat", 0.125)
     assert g.cols > 1 << 18

@@ -77,12 +77,12 @@ class PlanInfo(ctypes.Structure):
         ("rows", _i64), ("cols", _i64), ("nnz", _i64), ("k", _i64),
         ("strategy", ctypes.c_int32), ("segment_length", ctypes.c_int32),
         ("num_segments", _i64), ("max_row_nnz", _i64), ("empty_rows", _i64),
-        ("workspace_bytes", _i64), ("launches_per_spmm", ctypes.c_int32), ("reserved", ctypes.c_int32),
+        ("workspace_bytes", _i64), ("launches_per_spmm", ctypes.c_int32), ("column_tiles", ctypes.c_int32),
         ("hub_rows", _i64), ("lds_served_nnz", _i64), ("row_tiles", _i64),
     ]
 
     def as_dict(self):
-        return {name: getattr(self, name) for name, _ in self._fields_ if name != "reserved"}
+        return {name: getattr(self, name) for name, _ in self._fields_}
 
 
 class HpSpmmError(RuntimeError):

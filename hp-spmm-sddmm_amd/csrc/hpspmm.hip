@@ -64,6 +64,11 @@ inline void mark_launch(hipStream_t st, const char* name) {
 }
 
 inline bool fast_k(int64_t k) { return k == 32 || k == 64 || k == 128; }
+// Width of the column tiles by which a tuned layout can serve row length k (0: none, or k is tuned itself).
+inline int64_t tile_width(int64_t k) {
+  if (fast_k(k) || k <= 0) return 0;
+  return k % 128 == 0 ? 128 : k % 64 == 0 ? 64 : k % 32 == 0 ? 32 : 0;
+}
 // Row lengths served by the run-time-K sub-wave kernels: multiples of 4 that are not a tuned size.
 inline bool anyk_k(int64_t k) { return !fast_k(k) && k % 4 == 0 && k <= (1 << 20); }
 // Lanes per sub-wave for such a K: the power of two that covers a column tile (at most 128 floats).
@@ -101,6 +106,11 @@ int grid_for(int64_t items, int64_t cap = 1 << 20) {
 
 struct hpspmm_plan {
   int64_t rows = 0, cols = 0, nnz = 0, k = 0;
+  // A row length that is a multiple of a tuned one (256 = 2 x 128, 96 = 3 x 32) can be served by a
+  // layout built for the tuned length, one column tile after the other: k is then the tile width,
+  // k_full the row length of B and C, tiles = k_full / k.  Otherwise k_full = k, tiles = 1.
+  int64_t k_full = 0;
+  int tiles = 1;
   int strategy = 0;
   int shift = 0;  // log2(segment length)
   int64_t nseg = 0;
@@ -542,7 +552,7 @@ int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, 
   const int rpw = fixup_rows_per_wave(p->rows, K);
   const int64_t fix_blocks = ceil_div(ceil_div(p->rows, rpw), hpspmm::kWavesPerBlock);
   hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st, p->rows,
-                     rp, (const int32_t*)nullptr, p->d_carry, C, p->shift, rpw);
+                     rp, (const int32_t*)nullptr, p->d_carry, C, p->shift, rpw, (uint32_t)K);
   mark_launch(st, "spmm_fixup_kernel");
   return HPSPMM_OK;
 }
@@ -552,22 +562,23 @@ int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, 
 // 32 KB for the rows of B, 2.92 ms with 45 KB, 3.39 ms with 46 KB, where only two fit).
 constexpr int kOrderedBlockLdsBytes = 52992;
 
-template <int K>
+// kLd: B and C are K columns of wider arrays whose rows are `ld` floats apart (one column tile).
+template <int K, bool kLd = false>
 int launch_ordered(const hpspmm_plan* p, const int32_t* rp, const float* v, const float* B, float* C,
-                   hipStream_t st) {
+                   hipStream_t st, uint32_t ld = K) {
   const int64_t nblocks = p->owindows;
   const int64_t grid = p->xcd_remap ? ceil_div(nblocks, hpspmm::kXcds) * hpspmm::kXcds : nblocks;
   if (grid > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   if (p->nnz > 0) {
-    hipLaunchKernelGGL(hpspmm::spmm_ordered_kernel<K>, dim3((unsigned)grid), dim3(hpspmm::kBlock),
+    hipLaunchKernelGGL((hpspmm::spmm_ordered_kernel<K, kLd>), dim3((unsigned)grid), dim3(hpspmm::kBlock),
                        (size_t)p->ocap * K * sizeof(float), st, rp, p->d_ostart, p->d_ocol, p->d_osrc, p->d_orow, v,
-                       p->d_wcols, p->ocap, B, C, p->d_carry, p->nnz, p->shift, nblocks, p->xcd_remap);
+                       p->d_wcols, p->ocap, B, C, p->d_carry, p->nnz, p->shift, nblocks, p->xcd_remap, ld);
     mark_launch(st, "spmm_ordered_kernel");
   }
   const int rpw = fixup_rows_per_wave(p->rows, K);
   const int64_t fix_blocks = ceil_div(ceil_div(p->rows, rpw), hpspmm::kWavesPerBlock);
-  hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st, p->rows,
-                     rp, p->d_ostart, p->d_carry, C, p->shift, rpw);
+  hipLaunchKernelGGL((hpspmm::spmm_fixup_kernel<K, kLd>), dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st,
+                     p->rows, rp, p->d_ostart, p->d_carry, C, p->shift, rpw, ld);
   mark_launch(st, "spmm_fixup_kernel");
   return HPSPMM_OK;
 }
@@ -961,7 +972,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
            (void**)&d_chunk_base, (void**)&d_chunk_row}};
 
   bool inplace = false;
-  if (!sort_values && nsub == 1 && nnz > 0 && p->cols * k * 4 < ((int64_t)1 << 32) && p->d_nnz_row &&
+  if (!sort_values && nsub == 1 && nnz > 0 && p->cols * p->k_full * 4 < ((int64_t)1 << 32) && p->d_nnz_row &&
       columns_sorted(p, d_col, st)) {
     const int groups = nhub;
     const int64_t target = ceil_div(rk.sampled, groups);  // the column counts are those of the sample
@@ -1176,19 +1187,22 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   return HPSPMM_OK;
 }
 
-template <int K>
-int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
+// kLd: B and C are K columns of wider arrays whose rows are `ld` floats apart (one column tile);
+// values_ready: an earlier tile of the same product has already brought the values into the plan's order.
+template <int K, bool kLd = false>
+int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st, uint32_t ld = K,
+                  bool values_ready = false) {
   // values bound to the plan are already in class-major order: only the hub rows of B are refreshed
   const bool bound = p->bound_val && p->bound_val == v;
   const bool inplace = p->d_vsrc && !(bound && p->d_vval);
-  const int64_t permute_nnz = (p->d_vsrc || bound) ? 0 : p->nnz;
+  const int64_t permute_nnz = (p->d_vsrc || bound || values_ready) ? 0 : p->nnz;
   const int64_t gather_blocks = ceil_div(p->n_bhot * (K / 4), hpspmm::kBlock);
   const int64_t prep_blocks = gather_blocks + ceil_div(permute_nnz, hpspmm::kPermChunk);
   if (prep_blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   if (prep_blocks > 0) {
-    hipLaunchKernelGGL(hpspmm::routed_prepare_kernel<K>, dim3((unsigned)prep_blocks), dim3(hpspmm::kBlock), 0, st,
+    hipLaunchKernelGGL((hpspmm::routed_prepare_kernel<K, kLd>), dim3((unsigned)prep_blocks), dim3(hpspmm::kBlock), 0, st,
                        p->n_bhot, gather_blocks, p->d_bhot_src, B, p->d_bhot, p->nnz, p->lay.nhub + 1, v, p->d_lslot,
-                       p->d_chunk_base, p->d_chunk_pref, p->d_vval);
+                       p->d_chunk_base, p->d_chunk_pref, p->d_vval, ld);
     mark_launch(st, "routed_prepare_kernel");
   }
   if (p->routed_grid > 0) {
@@ -1203,17 +1217,17 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
       if (last <= first) continue;
       const dim3 grid((unsigned)(last - first));
       if (inplace)
-        hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, true, false>), grid, dim3(hpspmm::kBlock), 0, st, p->lay,
+        hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, true, false, kLd>), grid, dim3(hpspmm::kBlock), 0, st, p->lay,
                            p->d_rvptr, p->d_coldptr, p->d_vcol, v, p->d_vsrc, p->d_vrow, B, p->d_bhot, p->d_partial,
-                           p->d_carry, C, first);
+                           p->d_carry, C, first, ld);
       else if (p->d_vsrc)  // column-range slices, values bound: the plan's own copy of them, still no compact buffer
-        hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false, false>), grid, dim3(hpspmm::kBlock), 0, st, p->lay,
+        hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false, false, kLd>), grid, dim3(hpspmm::kBlock), 0, st, p->lay,
                            p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval, (const int32_t*)nullptr, p->d_vrow, B,
-                           p->d_bhot, p->d_partial, p->d_carry, C, first);
+                           p->d_bhot, p->d_partial, p->d_carry, C, first, ld);
       else
-        hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false, true>), grid, dim3(hpspmm::kBlock), 0, st, p->lay,
+        hipLaunchKernelGGL((hpspmm::spmm_routed_kernel<K, false, true, kLd>), grid, dim3(hpspmm::kBlock), 0, st, p->lay,
                            p->d_rvptr, p->d_coldptr, p->d_vcol, p->d_vval, (const int32_t*)nullptr, p->d_vrow, B,
-                           p->d_bhot, p->d_partial, p->d_carry, C, first);
+                           p->d_bhot, p->d_partial, p->d_carry, C, first, ld);
       mark_launch(st, !split ? "spmm_routed_kernel" : part < p->lay.nsub ? "spmm_routed_kernel(hub phase)"
                                                                           : "spmm_routed_kernel(cold class)");
     }
@@ -1222,9 +1236,9 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
   const int64_t cross_blocks = row_blocks(p->n_cross, K);
   const int64_t fin_blocks = routed_blocks + cross_blocks + row_blocks(p->n_zero, K);
   if (fin_blocks > 0) {
-    hipLaunchKernelGGL(hpspmm::spmm_routed_final_kernel<K>, dim3((unsigned)fin_blocks), dim3(hpspmm::kBlock), 0, st,
+    hipLaunchKernelGGL((hpspmm::spmm_routed_final_kernel<K, kLd>), dim3((unsigned)fin_blocks), dim3(hpspmm::kBlock), 0, st,
                        p->lay, p->d_rvptr, p->d_coldptr, p->d_routed_rows, routed_blocks, p->d_cross_rows, p->n_cross,
-                       cross_blocks, p->d_zero_rows, p->n_zero, p->d_partial, p->d_carry, C);
+                       cross_blocks, p->d_zero_rows, p->n_zero, p->d_partial, p->d_carry, C, ld);
     mark_launch(st, "spmm_routed_final_kernel");
   }
   return HPSPMM_OK;
@@ -1522,6 +1536,10 @@ int sweep_prepare_kernels(int* out) {
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_sweep_kernel<K, false>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_sweep_kernel<K, true, true>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_sweep_kernel<K, false, true>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   HPSPMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(out, hpspmm::spmm_sweep_kernel<K, true>,
                                                           hpspmm::sweep_waves<K>() * 64, lds));
   return HPSPMM_OK;
@@ -1544,7 +1562,7 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
   if (nnz <= 0 || !p->d_nnz_row) return HPSPMM_OK;
   // gather offsets are 32-bit, stream entries keep the column in 24 bits
-  if (p->cols * k * 4 >= ((int64_t)1 << 32) || p->cols > ((int64_t)1 << hpspmm::kSweepColBits)) return HPSPMM_OK;
+  if (p->cols * p->k_full * 4 >= ((int64_t)1 << 32) || p->cols > ((int64_t)1 << hpspmm::kSweepColBits)) return HPSPMM_OK;
   if (!forced && (nnz < kSweepMinNnz || p->cols * k * 4 < kSweepMinBBytes)) return HPSPMM_OK;
   const int P = (int)(64 / (k / 4));
   const int WS = P * hpspmm::kSweepSlots;
@@ -1780,27 +1798,29 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   return HPSPMM_OK;
 }
 
-template <int K>
-int launch_sweep(const hpspmm_plan* p, const int32_t* rp, const float* v, const float* B, float* C, hipStream_t st) {
+// kLd: B and C are K columns of wider arrays whose rows are `ld` floats apart (one column tile).
+template <int K, bool kLd = false>
+int launch_sweep(const hpspmm_plan* p, const int32_t* rp, const float* v, const float* B, float* C, hipStream_t st,
+                 uint32_t ld = K) {
   const bool bound = p->bound_val && p->bound_val == v && p->d_vval;
   constexpr int wpb = hpspmm::sweep_waves<K>();
   const dim3 grid((unsigned)(p->sw.n_waves / wpb));
   const size_t lds = hpspmm::sweep_lds_bytes<K>();
   if (bound)
-    hipLaunchKernelGGL((hpspmm::spmm_sweep_kernel<K, false>), grid, dim3(wpb * 64), lds, st, p->sw, p->d_sw_base,
+    hipLaunchKernelGGL((hpspmm::spmm_sweep_kernel<K, false, kLd>), grid, dim3(wpb * 64), lds, st, p->sw, p->d_sw_base,
                        p->d_sw_len, p->d_sw_ends, p->d_vcol, p->d_vval, (const int32_t*)nullptr, p->d_sw_slot_row, B,
-                       p->d_sw_zrow, p->d_partial, C);
+                       p->d_sw_zrow, p->d_partial, C, ld);
   else
-    hipLaunchKernelGGL((hpspmm::spmm_sweep_kernel<K, true>), grid, dim3(wpb * 64), lds, st, p->sw, p->d_sw_base,
+    hipLaunchKernelGGL((hpspmm::spmm_sweep_kernel<K, true, kLd>), grid, dim3(wpb * 64), lds, st, p->sw, p->d_sw_base,
                        p->d_sw_len, p->d_sw_ends, p->d_vcol, v, p->d_vsrc, p->d_sw_slot_row, B, p->d_sw_zrow,
-                       p->d_partial, C);
+                       p->d_partial, C, ld);
   mark_launch(st, "spmm_sweep_kernel");
   const int64_t split_blocks = row_blocks(p->n_split, K);
   const int64_t fin_blocks = split_blocks + row_blocks(p->n_zero, K);
   if (fin_blocks > 0) {
-    hipLaunchKernelGGL(hpspmm::spmm_sweep_final_kernel<K>, dim3((unsigned)fin_blocks), dim3(hpspmm::kBlock), 0, st, rp,
-                       p->sw_limit, p->d_sw_split_rows, p->n_split, split_blocks, p->d_sw_part_base, p->d_zero_rows,
-                       p->n_zero, p->d_partial, C);
+    hipLaunchKernelGGL((hpspmm::spmm_sweep_final_kernel<K, kLd>), dim3((unsigned)fin_blocks), dim3(hpspmm::kBlock), 0, st,
+                       rp, p->sw_limit, p->d_sw_split_rows, p->n_split, split_blocks, p->d_sw_part_base, p->d_zero_rows,
+                       p->n_zero, p->d_partial, C, ld);
     mark_launch(st, "spmm_sweep_final_kernel");
   }
   return HPSPMM_OK;
@@ -1814,15 +1834,40 @@ int hpspmm_version(void) { return 100; }
 
 const char* hpspmm_last_error(void) { return g_last_error.c_str(); }
 
+// Column tiles are tried for matrices of at least this many nonzeros (below, whole rows or plain
+// segments at the full row length are as good), or when the caller forces one of the layouts.
+constexpr int64_t kTiledMinNnz = (int64_t)1 << 22;
+
+// k_full = 0: the plan is for row length k.  Otherwise: a plan of tile width k for B and C of row
+// length k_full (see hpspmm_plan::k_full).
 static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_rowptr, const int32_t* d_col,
                             int64_t k, uint32_t flags, const int32_t* d_order, void* stream,
-                            hpspmm_plan** plan_out) {
+                            hpspmm_plan** plan_out, int64_t k_full = 0) {
   if (!plan_out) return fail(HPSPMM_ERR_INVALID_ARG, "plan_out is NULL");
   *plan_out = nullptr;
   if (int rc = check_dims(rows, cols, nnz, k)) return rc;
   if (!d_rowptr) return fail(HPSPMM_ERR_INVALID_ARG, "d_rowptr is NULL");
   if (nnz > 0 && !d_col) return fail(HPSPMM_ERR_INVALID_ARG, "d_col is NULL with nnz > 0");
   hipStream_t st = (hipStream_t)stream;
+
+  // A multiple of a tuned row length: the layouts built for the tuned length (sweep, routed,
+  // ordered) serve it tile by tile, if the matrix gets one of them; if not, the plan is built for
+  // the full length as for any other multiple of 4.
+  // (HPSPMM_NO_COLUMN_TILES in the environment switches this off, for comparisons)
+  if (k_full == 0 && tile_width(k) > 0 && nnz > 0 && !std::getenv("HPSPMM_NO_COLUMN_TILES") &&
+      (nnz >= kTiledMinNnz || d_order ||
+       (flags & (HPSPMM_PLAN_FORCE_ROUTED | HPSPMM_PLAN_FORCE_SWEEP | HPSPMM_PLAN_CLUSTER)))) {
+    hpspmm_plan* tiled = nullptr;
+    const int rc = plan_create_impl(rows, cols, nnz, d_rowptr, d_col, tile_width(k), flags, d_order, stream, &tiled, k);
+    if (rc == HPSPMM_OK && tiled &&
+        (tiled->strategy == HPSPMM_STRATEGY_SWEEP || tiled->strategy == HPSPMM_STRATEGY_ROUTED ||
+         tiled->strategy == HPSPMM_STRATEGY_ORDERED)) {
+      *plan_out = tiled;
+      return HPSPMM_OK;
+    }
+    if (tiled) hpspmm_plan_destroy(tiled);
+    if (rc == HPSPMM_ERR_BAD_CSR || rc == HPSPMM_ERR_NO_DEVICE) return rc;
+  }
 
   int ndev = 0;
   if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
@@ -1869,6 +1914,8 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   p->cols = cols;
   p->nnz = nnz;
   p->k = k;
+  p->k_full = k_full ? k_full : k;
+  p->tiles = (int)(p->k_full / k);
   p->max_row_nnz = stats[0];
   p->empty_rows = stats[1];
   p->src_rowptr = d_rowptr;
@@ -2084,7 +2131,7 @@ int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
   out->rows = plan->rows;
   out->cols = plan->cols;
   out->nnz = plan->nnz;
-  out->k = plan->k;
+  out->k = plan->k_full;
   out->strategy = plan->strategy;
   const bool segmented = plan->strategy == HPSPMM_STRATEGY_SEGMENTS || plan->strategy == HPSPMM_STRATEGY_ROUTED ||
                          plan->strategy == HPSPMM_STRATEGY_ORDERED;
@@ -2098,6 +2145,8 @@ int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
                            : plan->strategy == HPSPMM_STRATEGY_SWEEP   ? 2
                            : plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? (plan->n_hub > 0 ? 3 : 2)
                                                                         : 1;
+  out->launches_per_spmm *= plan->tiles;  // one pass per column tile
+  out->column_tiles = plan->tiles;
   out->hub_rows = plan->n_hub;
   out->lds_served_nnz = plan->oserved;
   out->row_tiles = plan->d_tent ? plan->rt_tiles : 0;
@@ -2166,7 +2215,7 @@ int hpspmm_plan_bind_values(hpspmm_plan* plan, const float* d_val, void* stream)
     hipLaunchKernelGGL(hpspmm::routed_prepare_kernel<32>, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st,
                        (int64_t)0, (int64_t)0, (const int32_t*)nullptr, (const float*)nullptr, (float*)nullptr,
                        plan->nnz, plan->lay.nhub + 1, d_val, plan->d_lslot, plan->d_chunk_base, plan->d_chunk_pref,
-                       plan->d_vval);
+                       plan->d_vval, 32u);
     HPSPMM_HIP(hipGetLastError());
   }
   plan->bound_val = d_val;
@@ -2191,7 +2240,37 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
   int rc;
   // another value array overwrites the plan's copy of the bound one
   if (plan->bound_val && plan->bound_val != d_val) plan->bound_val = nullptr;
-  if (plan->strategy == HPSPMM_STRATEGY_ORDERED) {
+  if (plan->tiles > 1) {
+    // one column tile after the other through the layout built for the tile width; the operands of
+    // tile t are columns [t * k, (t + 1) * k) of B and C, whose rows are k_full floats apart
+    const uint32_t ld = (uint32_t)plan->k_full;
+    rc = HPSPMM_OK;
+    for (int t = 0; t < plan->tiles && rc == HPSPMM_OK; ++t) {
+      const float* Bt = d_B + (int64_t)t * plan->k;
+      float* Ct = d_C + (int64_t)t * plan->k;
+      if (plan->strategy == HPSPMM_STRATEGY_ORDERED) {
+        switch (plan->k) {
+          case 32: rc = launch_ordered<32, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+          case 64: rc = launch_ordered<64, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+          default: rc = launch_ordered<128, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+        }
+      } else if (plan->strategy == HPSPMM_STRATEGY_SWEEP) {
+        switch (plan->k) {
+          case 32: rc = launch_sweep<32, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+          case 64: rc = launch_sweep<64, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+          default: rc = launch_sweep<128, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+        }
+      } else if (plan->strategy == HPSPMM_STRATEGY_ROUTED) {
+        switch (plan->k) {
+          case 32: rc = launch_routed<32, true>(plan, d_val, Bt, Ct, st, ld, t > 0); break;
+          case 64: rc = launch_routed<64, true>(plan, d_val, Bt, Ct, st, ld, t > 0); break;
+          default: rc = launch_routed<128, true>(plan, d_val, Bt, Ct, st, ld, t > 0); break;
+        }
+      } else {
+        rc = fail(HPSPMM_ERR_INVALID_ARG, "plan of column tiles without a tiled strategy");
+      }
+    }
+  } else if (plan->strategy == HPSPMM_STRATEGY_ORDERED) {
     switch (plan->k) {
       case 32: rc = launch_ordered<32>(plan, d_rowptr, d_val, d_B, d_C, st); break;
       case 64: rc = launch_ordered<64>(plan, d_rowptr, d_val, d_B, d_C, st); break;
@@ -2303,7 +2382,7 @@ int launch_static(int64_t rows, int64_t nnz, const int32_t* rp, const int32_t* c
   const int rpw = fixup_rows_per_wave(rows, K);
   const int64_t fix_blocks = ceil_div(ceil_div(rows, rpw), hpspmm::kWavesPerBlock);
   hipLaunchKernelGGL(hpspmm::spmm_fixup_kernel<K>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st, rows, rp,
-                     (const int32_t*)nullptr, (const float*)carry, C, shift, rpw);
+                     (const int32_t*)nullptr, (const float*)carry, C, shift, rpw, (uint32_t)K);
   return HPSPMM_OK;
 }
 }  // namespace

@@ -400,15 +400,16 @@ __global__ __launch_bounds__(kBlock) void ordered_partition_kernel(int64_t rows,
 
 // One workgroup per window = kWavesPerBlock * P segments of 2^shift nonzeros.
 // Dynamic LDS: cap * K floats, the window's slotted rows of B.
-template <int K>
+template <int K, bool kLd = false>
 __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
     const int32_t* __restrict__ rowptr, const int32_t* __restrict__ start, const int32_t* __restrict__ ocol,
     const int32_t* __restrict__ osrc, const int32_t* __restrict__ orow, const float* __restrict__ val,
     const int32_t* __restrict__ wcols, int cap, const float* __restrict__ B, float* __restrict__ C,
-    float* __restrict__ carry, int64_t nnz, int shift, int64_t nblocks, bool remap) {
+    float* __restrict__ carry, int64_t nnz, int shift, int64_t nblocks, bool remap, uint32_t ld_arg) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
   constexpr int TL = kTile / G;
+  const uint32_t ld = row_length<K, kLd>(ld_arg);  // floats between the rows of B and of C
   __shared__ __attribute__((aligned(16))) int32_t s_col[kWavesPerBlock * P * kTileStride];
   __shared__ __attribute__((aligned(16))) float s_val[kWavesPerBlock * P * kTileStride];
   __shared__ __attribute__((aligned(16))) int32_t s_row[kWavesPerBlock * P * kTileStride];
@@ -424,7 +425,7 @@ __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
   for (int i = tid; i < cap * G; i += kBlock) {
     const int slot = i / G;
     const int32_t c = wcols[blk * cap + slot];
-    if (c >= 0) *reinterpret_cast<float4*>(s_b + slot * K + 4 * (i % G)) = load_b<K>(B, c, i % G);
+    if (c >= 0) *reinterpret_cast<float4*>(s_b + slot * K + 4 * (i % G)) = load_b_ld(B, c, i % G, ld);
   }
   __syncthreads();
 
@@ -440,7 +441,7 @@ __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
 
   auto flush_to = [&](bool is_tail) {
     float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
-                              : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : C + (uint64_t)(uint32_t)cur * K);
+                              : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : C + (uint64_t)(uint32_t)cur * ld);
     head_pending = false;
     store_result(dst + 4 * l, acc);
   };
@@ -449,7 +450,7 @@ __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
   // per gather would make every load of a batch wait for the one before it.
   const float* lds_b = s_b;
   auto loadb = [&](int32_t c) {
-    const float* row = c < 0 ? lds_b + (uint32_t)(~c) * (uint32_t)K : B + (uint64_t)(uint32_t)c * (uint64_t)K;
+    const float* row = c < 0 ? lds_b + (uint32_t)(~c) * (uint32_t)K : B + (uint64_t)(uint32_t)c * (uint64_t)ld;
     return *reinterpret_cast<const float4*>(row + 4 * l);
   };
 

@@ -501,7 +501,7 @@ __global__ __launch_bounds__(kBlock) void routed_chunk_kernel(RoutedLayout lay, 
 // single values costs one L2 transaction for every two or three of them; so
 // the chunk is sorted by destination in LDS (lslot) and written out run by
 // run in full lines (233k-vertex social graph: 0.28 ms for the plain scatter).
-template <int K>
+template <int K, bool kLd = false>
 __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, int64_t gather_blocks,
                                                                 const int32_t* __restrict__ src,
                                                                 const float* __restrict__ B,
@@ -510,7 +510,7 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
                                                                 const uint16_t* __restrict__ lslot,
                                                                 const int32_t* __restrict__ chunk_base,
                                                                 const int32_t* __restrict__ chunk_pref,
-                                                                float* __restrict__ vval) {
+                                                                float* __restrict__ vval, uint32_t ld_arg) {
   constexpr int G = K / 4;
   __shared__ float s_buf[kPermChunk];
   __shared__ int32_t s_base[kMaxClasses];
@@ -522,7 +522,7 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
     if (s >= n_bhot) return;
     const int32_t c = src[s];
     if (c < 0) return;
-    *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) = load_b<K>(B, c, l);
+    *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) = load_b_ld(B, c, l, row_length<K, kLd>(ld_arg));
     return;
   }
   const int64_t chunk = (int64_t)blockIdx.x - gather_blocks;
@@ -572,7 +572,7 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
 // indices, so these loads stay coalesced).  kHub: vcol may hold ~(compact-buffer row); without it
 // every entry is a plain column and the gather address is B plus a 32-bit byte offset (the plan
 // checks that B is below 4 GB), three instructions instead of eight.
-template <int K, bool kInPlace, bool kHub>
+template <int K, bool kInPlace, bool kHub, bool kLd = false>
 __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, const int32_t* __restrict__ rvptr,
                                                              const int32_t* __restrict__ coldptr,
                                                              const int32_t* __restrict__ vcol,
@@ -583,9 +583,10 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
                                                              const float* __restrict__ Bhot,
                                                              float* __restrict__ partial,
                                                              float* __restrict__ carry, float* __restrict__ C,
-                                                             int64_t first_block) {
+                                                             int64_t first_block, uint32_t ld_arg) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
+  const uint32_t ld = row_length<K, kLd>(ld_arg);  // floats between the rows of B and of C
   constexpr int TL = kTile / G;
   __shared__ __attribute__((aligned(16))) int32_t s_col[kWavesPerBlock * P * kTileStride];
   __shared__ __attribute__((aligned(16))) float s_val[kWavesPerBlock * P * kTileStride];
@@ -624,7 +625,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
   const int32_t* vp = hub ? rvptr + x : coldptr;
   const int64_t vstride = hub ? nhub : 1;
   float* out = hub ? partial + (uint64_t)x * K : C;
-  const uint64_t ostride = hub ? (uint64_t)nhub * K : (uint64_t)K;
+  const uint64_t ostride = hub ? (uint64_t)nhub * K : (uint64_t)ld;
 
   int32_t cur = vrow[s];
   bool head_pending = (int64_t)vp[(int64_t)cur * vstride] < s;
@@ -639,9 +640,9 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
   auto flush = [&]() { flush_to(false); };
   auto loadb = [&](int32_t c) {
     if constexpr (kHub) {
-      return load_b_hub<K, true>(B, Bhot, c, l);
+      return load_b_hub_ld<K, true>(B, Bhot, c, l, ld);
     } else {
-      const uint32_t off = (uint32_t)c * (uint32_t)(K * 4) + (uint32_t)(16 * l);
+      const uint32_t off = (uint32_t)c * (ld * 4u) + (uint32_t)(16 * l);
       return *reinterpret_cast<const float4*>(reinterpret_cast<const char*>(B) + off);
     }
   };
@@ -716,14 +717,15 @@ __global__ __launch_bounds__(kBlock) void routed_collect_rows_kernel(int64_t row
 // cold-class run crossed a segment boundary, from the carry slots alone.
 // The rest: rows without nonzeros, which get zeros.
 // Rows in none of the lists were stored by the main kernel.
-template <int K>
+template <int K, bool kLd = false>
 __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
     RoutedLayout lay, const int32_t* __restrict__ rvptr, const int32_t* __restrict__ coldptr,
     const int32_t* __restrict__ routed_rows, int64_t routed_blocks, const int32_t* __restrict__ cross_rows,
     int64_t n_cross, int64_t cross_blocks, const int32_t* __restrict__ zero_rows, int64_t n_zero,
-    const float* __restrict__ partial, const float* __restrict__ carry, float* __restrict__ C) {
+    const float* __restrict__ partial, const float* __restrict__ carry, float* __restrict__ C, uint32_t ld_arg) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
+  const uint32_t ld = row_length<K, kLd>(ld_arg);  // floats between the rows of C
   constexpr int kGroup = kSlices;  // classes whose loads are in flight together; divides nhub
   __shared__ int32_t s_bounds[kWavesPerBlock * P][2 * kMaxHub + 1];  // odd stride: sub-waves on different banks
   const int tid = threadIdx.x;
@@ -758,7 +760,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
   if ((int64_t)blockIdx.x >= routed_blocks + cross_blocks) {
     const int64_t idx = ((int64_t)blockIdx.x - routed_blocks - cross_blocks) * (kWavesPerBlock * P) + sub;
     if (idx >= n_zero) return;
-    *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * K + 4 * l) = acc;
+    *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * ld + 4 * l) = acc;
     return;
   }
   if ((int64_t)blockIdx.x >= routed_blocks) {
@@ -769,7 +771,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
     const int64_t gb = (coldptr[row + 1] - 1) >> shift;
     add(*reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * ga + 1) * K));
     add_heads(ga + 1, gb);
-    *reinterpret_cast<float4*>(C + (uint64_t)row * K + 4 * l) = acc;
+    *reinterpret_cast<float4*>(C + (uint64_t)row * ld + 4 * l) = acc;
     return;
   }
   const int64_t idx = (int64_t)blockIdx.x * (kWavesPerBlock * P) + sub;
@@ -828,7 +830,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
       if (gb > ga + 1) add_heads(ga + 2, gb);
     }
   }
-  *reinterpret_cast<float4*>(C + (uint64_t)row * K + 4 * l) = acc;
+  *reinterpret_cast<float4*>(C + (uint64_t)row * ld + 4 * l) = acc;
 }
 
 }  // namespace hpspmm

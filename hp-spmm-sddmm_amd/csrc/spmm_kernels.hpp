@@ -71,6 +71,17 @@ __device__ __forceinline__ float4 load_b(const float* __restrict__ B, int32_t c,
   return *reinterpret_cast<const float4*>(B + (uint64_t)(uint32_t)c * (uint64_t)K + (uint32_t)(4 * l));
 }
 
+// The same with the row length of B given at run time: the operands of a tuned kernel may be K
+// columns of a wider B and C (one column tile of a product whose row length is a multiple of K).
+// kLd = false compiles to the fixed form.
+template <int K, bool kLd>
+__device__ __forceinline__ uint32_t row_length(uint32_t ld_arg) {
+  return kLd ? ld_arg : (uint32_t)K;
+}
+__device__ __forceinline__ float4 load_b_ld(const float* __restrict__ B, int32_t c, int l, uint32_t ld) {
+  return *reinterpret_cast<const float4*>(B + (uint64_t)(uint32_t)c * (uint64_t)ld + (uint32_t)(4 * l));
+}
+
 // Fragment l of a KT-wide column tile starting at column k0 of row c (leading dimension K).
 template <int K>
 __device__ __forceinline__ float4 load_b_tile(const float* __restrict__ B, int32_t c, int k0, int l) {
@@ -90,6 +101,20 @@ __device__ __forceinline__ float4 load_b_hub(const float* __restrict__ B, const 
     return *reinterpret_cast<const float4*>(base + (uint64_t)idx * (uint64_t)K + (uint32_t)(4 * l));
   } else {
     return load_b<K>(B, c, l);
+  }
+}
+
+// The same with rows of B that are ld floats apart (the compact buffer's rows stay K apart).
+template <int K, bool kHub>
+__device__ __forceinline__ float4 load_b_hub_ld(const float* __restrict__ B, const float* __restrict__ Bhot, int32_t c,
+                                                int l, uint32_t ld) {
+  if constexpr (kHub) {
+    const bool hot = c < 0;
+    const float* base = hot ? Bhot : B;
+    const uint32_t idx = hot ? (uint32_t)~c : (uint32_t)c;
+    return *reinterpret_cast<const float4*>(base + (uint64_t)idx * (uint64_t)(hot ? (uint32_t)K : ld) + (uint32_t)(4 * l));
+  } else {
+    return load_b_ld(B, c, l, ld);
   }
 }
 
@@ -457,13 +482,15 @@ __global__ __launch_bounds__(kBlock) void spmm_segments_kernel(
 // five times the segments kernel before it).
 // `start` (may be NULL): first position of every row when the nonzeros were
 // processed in an order of the plan's own; NULL = stored order (rowptr).
-template <int K>
+template <int K, bool kLd = false>
 __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                             const int32_t* __restrict__ start,
                                                             const float* __restrict__ carry,
-                                                            float* __restrict__ C, int shift, int rpw) {
+                                                            float* __restrict__ C, int shift, int rpw,
+                                                            uint32_t ld_arg) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
+  const uint32_t ld = row_length<K, kLd>(ld_arg);  // floats between the rows of C
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
@@ -511,7 +538,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
     // every lane takes part in the shuffles; only then do the sub-waves diverge
     const int32_t lb_i = __shfl(lb, i);
     const int32_t hb_i = __shfl(hb, i);
-    float4* out = reinterpret_cast<float4*>(C + (uint64_t)(r0 + i) * K + 4 * l);
+    float4* out = reinterpret_cast<float4*>(C + (uint64_t)(r0 + i) * ld + 4 * l);
     if ((m_empty >> i) & 1ull) {
       *out = make_float4(0.f, 0.f, 0.f, 0.f);
     } else if ((m_split >> i) & 1ull) {
@@ -544,7 +571,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
       t.w = __shfl(part.w, s * G + l);
       add(acc, t);
     }
-    if (sub == 0) *reinterpret_cast<float4*>(C + (uint64_t)(r0 + i) * K + 4 * l) = acc;
+    if (sub == 0) *reinterpret_cast<float4*>(C + (uint64_t)(r0 + i) * ld + 4 * l) = acc;
   }
 }
 

@@ -412,15 +412,16 @@ __global__ __launch_bounds__(kBlock) void sweep_gather_values_kernel(int64_t n, 
 // entries each, side by side.  kInPlace: vval is the caller's value array and vsrc[q] the index into
 // it of stream position q (fetched two tiles ahead, so that the value loads of the next tile never
 // wait for their indices); otherwise vval holds the values in stream order.
-template <int K, bool kInPlace>
+template <int K, bool kInPlace, bool kLd = false>
 __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
     SweepLayout lay, const uint32_t* __restrict__ wave_base, const uint32_t* __restrict__ wave_len,
     const int32_t* __restrict__ chunk_end, const int32_t* __restrict__ vent, const float* __restrict__ vval,
     const int32_t* __restrict__ vsrc, const int32_t* __restrict__ slot_row, const float* __restrict__ B,
-    const float* __restrict__ zrow, float* __restrict__ partial, float* __restrict__ C) {
+    const float* __restrict__ zrow, float* __restrict__ partial, float* __restrict__ C, uint32_t ld_arg) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
   constexpr int TL = kTile / G;
+  const uint32_t ld = row_length<K, kLd>(ld_arg);  // floats between the rows of B and of C
   constexpr int WS = P * kSweepSlots;  // accumulator slots of a wavefront: WS * K floats = 8 KB
   constexpr int WPB = sweep_waves<K>();
   extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
@@ -464,7 +465,7 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   // the plan checks that B is below 4 GB: a 32-bit byte offset
   auto loadb = [&](int32_t w) {
-    const uint32_t off = (uint32_t)(w & kSweepColMask) * (uint32_t)(K * 4) + (uint32_t)(16 * l);
+    const uint32_t off = (uint32_t)(w & kSweepColMask) * (ld * 4u) + (uint32_t)(16 * l);
     const char* base =
         (w & kSweepPad) ? reinterpret_cast<const char*>(zrow) + 16 * l : reinterpret_cast<const char*>(B) + off;
     return *reinterpret_cast<const float4*>(base);
@@ -587,20 +588,21 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
     const int32_t dest = slot_row[wave * WS + slot];
     if (dest == kSweepUnused) continue;
     const float4 sum = *reinterpret_cast<const float4*>(acc_wave + slot * K + 4 * l);
-    float* out = dest >= 0 ? C + (uint64_t)(uint32_t)dest * K : partial + (uint64_t)(uint32_t)~dest * K;
+    float* out = dest >= 0 ? C + (uint64_t)(uint32_t)dest * ld : partial + (uint64_t)(uint32_t)~dest * K;
     store_result(out + 4 * l, sum);
   }
 }
 
 // Final pass.  Workgroups [0, split_blocks): one sub-wave per split row adds the row's partial
 // results in piece order and writes C.  The others: rows without nonzeros get zeros.
-template <int K>
+template <int K, bool kLd = false>
 __global__ __launch_bounds__(kBlock) void spmm_sweep_final_kernel(
     const int32_t* __restrict__ rowptr, int32_t limit, const int32_t* __restrict__ split_rows, int64_t n_split,
     int64_t split_blocks, const uint32_t* __restrict__ part_base, const int32_t* __restrict__ zero_rows,
-    int64_t n_zero, const float* __restrict__ partial, float* __restrict__ C) {
+    int64_t n_zero, const float* __restrict__ partial, float* __restrict__ C, uint32_t ld_arg) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
+  const uint32_t ld = row_length<K, kLd>(ld_arg);  // floats between the rows of C
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
@@ -608,7 +610,7 @@ __global__ __launch_bounds__(kBlock) void spmm_sweep_final_kernel(
   if ((int64_t)blockIdx.x >= split_blocks) {
     const int64_t idx = ((int64_t)blockIdx.x - split_blocks) * (kWavesPerBlock * P) + sub;
     if (idx >= n_zero) return;
-    *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * K + 4 * l) = make_float4(0.f, 0.f, 0.f, 0.f);
+    *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * ld + 4 * l) = make_float4(0.f, 0.f, 0.f, 0.f);
     return;
   }
   const int64_t idx = (int64_t)blockIdx.x * (kWavesPerBlock * P) + sub;
@@ -637,7 +639,7 @@ __global__ __launch_bounds__(kBlock) void spmm_sweep_final_kernel(
     acc.z += t.z;
     acc.w += t.w;
   }
-  *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)row * K + 4 * l) = acc;
+  *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)row * ld + 4 * l) = acc;
 }
 
 }  // namespace hpspmm

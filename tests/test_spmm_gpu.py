@@ -941,3 +941,56 @@ def test_sweep_is_not_chosen_for_a_banded_matrix(pkg, oracle, gpu):
     C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SWEEP)
     assert info["strategy"] == capi.STRATEGY_SWEEP, info
     _check(oracle, g, B, C, "banded, forced sweep")
+
+
+@pytest.mark.parametrize("k,tile", [(96, 32), (160, 32), (192, 64), (256, 128), (384, 128)])
+def test_column_tiles(pkg, oracle, gpu, k, tile):
+    """A row length that is a multiple of a tuned one goes through the tuned layouts (sweep, routed,
+    ordered) one column tile after the other: the plan reports that strategy, the full row length and
+    one set of launches per tile; the product meets the oracle's bar; tile t of C has the bits of the
+    product with columns [t * tile, (t + 1) * tile) of B alone (same layout, same order of additions);
+    bound values give the same bits.  Without a tuned layout the plan is the one for any multiple of 4."""
+    import torch
+    capi = pkg.capi
+    cases = [("c2_social", 0.02, "sweep", capi.PLAN_FORCE_SWEEP, capi.STRATEGY_SWEEP),
+             ("c4_rmat", 0.004, "routed", capi.PLAN_FORCE_ROUTED | capi.plan_routed_row_log2(2), capi.STRATEGY_ROUTED),
+             ("c4_rmat", 0.004, "routed_hub", capi.PLAN_FORCE_ROUTED | capi.PLAN_ROUTED_SORT_VALUES | capi.plan_hub_log2(9)
+              | capi.plan_routed_row_log2(2) | capi.plan_routed_phases(3), capi.STRATEGY_ROUTED),
+             ("c3_copurchase", 0.01, "cluster", capi.PLAN_CLUSTER | capi.PLAN_FORCE_SEGMENTS | capi.PLAN_NO_HUB_CACHE,
+              capi.STRATEGY_ORDERED)]
+    for name, scale, label, flags, strategy in cases:
+        g = pkg.graphs.make_graph(name, scale)
+        B = pkg.graphs.make_dense(name, g.cols, k)
+        C, info = _run(pkg, gpu, g, B, flags)
+        what = f"{name} k={k} {label}"
+        assert info["strategy"] == strategy and info["k"] == k and info["column_tiles"] == k // tile, (what, info)
+        _check(oracle, g, B, C, what)
+        for t in sorted({0, k // tile - 1}):
+            Bt = np.ascontiguousarray(B[:, t * tile:(t + 1) * tile])
+            Ct, info_t = _run(pkg, gpu, g, Bt, flags)
+            assert info_t["strategy"] == strategy and info_t["launches_per_spmm"] * (k // tile) == info["launches_per_spmm"]
+            assert np.array_equal(C[:, t * tile:(t + 1) * tile], Ct), f"{what}: tile {t} differs from the product of that tile alone"
+        rp, ci, v, Bd = _to_dev(gpu, g.rowptr, g.col, g.val, B)
+        plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
+        Cb = torch.full((g.rows, k), float("nan"), device=gpu)
+        plan.bind_values(v)
+        capi.csr_spmm(plan, rp, ci, v, Bd, Cb)
+        torch.cuda.synchronize()
+        assert np.array_equal(Cb.cpu().numpy(), C), f"{what}: bound values, different bits"
+        plan.destroy()
+    # a caller's row order
+    g = pkg.graphs.make_graph("c3_copurchase", 0.01)
+    B = pkg.graphs.make_dense("c3_copurchase", g.cols, k)
+    rp, ci, v, Bd = _to_dev(gpu, g.rowptr, g.col, g.val, B)
+    order = np.random.default_rng(5).permutation(g.rows).astype(np.int32)
+    od, = _to_dev(gpu, order)
+    plan = capi.Plan(g.rows, g.cols, rp, ci, k, 0, row_order=od)
+    assert plan.info["strategy"] == capi.STRATEGY_ORDERED and plan.info["k"] == k
+    Co = torch.full((g.rows, k), float("nan"), device=gpu)
+    capi.csr_spmm(plan, rp, ci, v, Bd, Co)
+    torch.cuda.synchronize()
+    _check(oracle, g, B, Co.cpu().numpy(), f"row order k={k}")
+    plan.destroy()
+    # small and unforced: no tiles, the plan for any multiple of 4
+    _, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+    assert info["strategy"] in (capi.STRATEGY_ROWS, capi.STRATEGY_SEGMENTS) and info["k"] == k and info["column_tiles"] == 1, info

@@ -275,10 +275,18 @@ def main():
             B = graphs.make_dense(name, g.cols, k)
             d_B = torch.from_numpy(B).to(dev)
             d_C = torch.empty((g.rows, k), device=dev, dtype=torch.float32)
-            t0 = time.perf_counter()
-            plan = capi.Plan(g.rows, g.cols, d_rp, d_ci, k, args.plan_flags)
-            torch.cuda.synchronize()
-            plan_ms = (time.perf_counter() - t0) * 1e3
+            # plan construction, timed twice: the first one of a kind in a process also pays for loading the
+            # kernels it uses (plan_first_ms); plan_ms is what every further plan costs
+            plan_times = []
+            for attempt in range(2):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                plan = capi.Plan(g.rows, g.cols, d_rp, d_ci, k, args.plan_flags)
+                torch.cuda.synchronize()
+                plan_times.append((time.perf_counter() - t0) * 1e3)
+                if attempt == 0:
+                    plan.destroy()
+            plan_first_ms, plan_ms = plan_times
             info = plan.info
             def timed(warmup, steps):
                 # hpspmm_csr_spmm_timed: `warmup` launches, then `steps` launches issued back to back
@@ -322,7 +330,7 @@ def main():
                 "launch_ms": {n_: t_ for n_, t_ in launches},
                 "roof": ROOF.get(name, ""),
                 "strategy": info["strategy"], "segment_length": info["segment_length"],
-                "launches_per_spmm": info["launches_per_spmm"], "plan_ms": plan_ms,
+                "launches_per_spmm": info["launches_per_spmm"], "plan_ms": plan_ms, "plan_first_ms": plan_first_ms,
                 "plan_over_spmm": plan_ms / ms,
                 "plan_workspace_mb": info["workspace_bytes"] / 1e6,
                 "plan_workspace_over_csr": info["workspace_bytes"] / (4.0 * (g.rows + 1) + 8.0 * g.nnz),

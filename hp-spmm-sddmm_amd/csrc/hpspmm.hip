@@ -819,7 +819,7 @@ int rank_columns(const hpspmm_plan* p, const int32_t* d_col, int64_t want, hipSt
     // hot, shows in every 4th nonzero as well as in all of them, and the histogram is the most
     // expensive step of the plan (random read-modify-writes: 12 ms for the 128 M nonzeros of R-MAT
     // scale 22).  Strided, hence the same sample every time.
-    rk.stride = p->nnz >= ((int64_t)1 << 25) ? 4 : p->nnz >= ((int64_t)1 << 23) ? 2 : 1;
+    rk.stride = p->nnz >= ((int64_t)1 << 26) ? 8 : p->nnz >= ((int64_t)1 << 25) ? 4 : p->nnz >= ((int64_t)1 << 23) ? 2 : 1;
     rk.sampled = ceil_div(p->nnz, rk.stride);
     if (int rc = count_columns(p, d_col, rk.stride, st, &rk.d_count)) return rc;
   }
@@ -1430,7 +1430,7 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
   for (int sweep = 0; sweep < max_sweeps; ++sweep) {
     HPSPMM_HIP(hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st));
     hipLaunchKernelGGL(hpspmm::cluster_sweep_kernel,
-                       dim3((unsigned)ceil_div(ceil_div(rows, 2), hpspmm::kWavesPerBlock * hpspmm::kClusterRowsPerWave)),
+                       dim3((unsigned)ceil_div(ceil_div(rows, 2), hpspmm::kWavesPerBlock * 2 * hpspmm::kClusterRowsPerHalf)),
                        dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_label, d_label_next, (uint32_t)sweep,
                        d_changed);
     std::swap(d_label, d_label_next);
@@ -1442,7 +1442,9 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
     if (debug) fprintf(stderr, "cluster sweep %d: %lld of %lld rows changed their label\n", sweep, (long long)changed, (long long)rows);
     if (changed * 200 < rows) break;
   }
-  // share of the nonzeros that stay inside a cluster small enough for a workgroup's window
+  // share of the nonzeros that stay inside a cluster small enough for a workgroup's window, from
+  // every 4th row when there are a million of them (a threshold decision: 1.4 -> 0.4 ms at 2.4 M rows)
+  const int64_t score_stride = rows >= ((int64_t)1 << 20) ? 4 : 1;
   {
     int32_t* d_size = nullptr;
     hipError_t e = hipMalloc(&d_size, (size_t)rows * sizeof(int32_t));
@@ -1451,9 +1453,10 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
     if (e == hipSuccess) {
       hipLaunchKernelGGL(hpspmm::label_sizes_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock),
                          0, st, rows, d_label, d_size);
-      hipLaunchKernelGGL(hpspmm::cluster_intra_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
-                         dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_label, d_size, kClusterMaxSize,
-                         d_changed);
+      hipLaunchKernelGGL(hpspmm::cluster_intra_kernel,
+                         dim3((unsigned)ceil_div(ceil_div(rows, score_stride), hpspmm::kWavesPerBlock)),
+                         dim3(hpspmm::kBlock), 0, st, rows, score_stride, d_rowptr, d_col, d_label, d_size,
+                         kClusterMaxSize, d_changed);
       e = hipMemcpyAsync(counters.data(), d_changed, counters.size() * sizeof(uint32_t), hipMemcpyDeviceToHost, st);
     }
     if (e == hipSuccess) e = hipStreamSynchronize(st);
@@ -1461,6 +1464,7 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
     if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "cluster scoring failed: %s", hipGetErrorString(e));
     int64_t intra = 0;
     for (uint32_t c : counters) intra += c;
+    intra *= score_stride;
     *intra_share_out = p->nnz > 0 ? (double)intra / (double)p->nnz : 0.0;
     if (debug) fprintf(stderr, "cluster: %.4f of the nonzeros inside clusters of at most %d rows\n", *intra_share_out, kClusterMaxSize);
   }
@@ -1594,6 +1598,10 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   while (wshift < 30 && (((int64_t)1 << (wshift + 1)) * k * 4) <= ((int64_t)1 << wlog2)) ++wshift;
   const int64_t n_windows = ceil_div(p->cols, (int64_t)1 << wshift);
   if (n_windows > kSweepMaxWindows) return HPSPMM_OK;
+  // every non-empty row is at least one piece: what the two criteria below come to at the very least
+  // (rules the layout out for a matrix of many short rows before any kernel has run)
+  if (!forced && (ceil_div(nonempty, band_waves * WS) * hpspmm::kXcds * p->cols > nnz / 4 || nonempty * n_windows * 3 > nnz * 2))
+    return HPSPMM_OK;
   if (!columns_sorted(p, d_col, st)) return HPSPMM_OK;  // a row must meet the windows in stored order
   if (!forced) {
     // rows that reach across most of the columns (a banded matrix is better off with whole rows or segments)

@@ -613,11 +613,16 @@ def test_hip_graph_capture_and_replay(pkg, oracle, gpu):
     import torch
     capi = pkg.capi
     g = pkg.graphs.make_graph("c4_rmat", 0.004)
-    k = 64
-    B = pkg.graphs.make_dense("c4_rmat", g.cols, k)
-    rp, ci, v, Bd = _to_dev(gpu, g.rowptr, g.col, g.val, B)
-    for name, flags in _strategies(capi):
+    # every strategy at a tuned row length, then the tiled forms (3 tiles of 64 columns) of the three layouts that have one
+    tiled = [(n, f) for n, f in _strategies(capi) if n in ("sweep", "routed", "routed_sort_values", "cluster_seg")]
+    operands = {}
+    for name, flags, k in [(n, f, 64) for n, f in _strategies(capi)] + [(n + "_tiled", f, 192) for n, f in tiled]:
+        if k not in operands:
+            operands[k] = _to_dev(gpu, g.rowptr, g.col, g.val, pkg.graphs.make_dense("c4_rmat", g.cols, k))
+        rp, ci, v, Bd = operands[k]
         plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
+        if name.endswith("_tiled"):
+            assert plan.info["column_tiles"] == 3, (name, plan.info)
         C = torch.full((g.rows, k), float("nan"), device=gpu)
         eager = torch.empty_like(C)
         capi.csr_spmm(plan, rp, ci, v, Bd, eager)

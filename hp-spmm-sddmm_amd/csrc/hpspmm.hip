@@ -267,12 +267,13 @@ int launch_rows(int64_t rows, int64_t cols, const int32_t* rp, const int32_t* ci
 // Row tiles (rows strategy): every row cut into slots of 8 nonzeros, 8 slots to a tile, a row's
 // slots adjacent in one tile (1 / 2 / 4 / 8 of them for up to 8 / 16 / 32 / 64 nonzeros, tiles
 // sorted by that class), longer rows over consecutive tiles, those that get a whole workgroup
-// first.  Built on the host, about 3 ms per million nonzeros.  Skipped (the kernel then walks the
+// first.  Built on the device (0.2 ms at 100k nonzeros, 1 ms at 10 M; on the host it took about
+// 3 ms per million nonzeros, after copying the column indices over).  Skipped (the kernel then walks the
 // CSR arrays) when padding would blow the layout up, which is what a matrix of mostly empty rows
 // does, and beyond kRowTileMaxNnz (rows strategy forced on a very large matrix).
 constexpr int64_t kRowTilePadFactor = 8;
 constexpr int64_t kRowTileMaxNnz = (int64_t)1 << 28;
-constexpr int32_t kRowTileWorkgroupRows = 512;  // rows beyond this many nonzeros get a whole workgroup
+using hpspmm::kRowTileWorkgroupRows;  // rows beyond this many nonzeros get a whole workgroup
 // automatic use of the rows strategy beyond tiny matrices
 constexpr int64_t kRowsAutoMaxNnz = 1 << 24;
 constexpr int64_t kRowsAutoMaxWork = (int64_t)3 << 28;  // nnz * K, matrices of short rows
@@ -280,102 +281,7 @@ constexpr double kRowsAutoLongMean = 128.0;             // mean nonzeros per non
 constexpr double kRowsAutoLongWork = 2.0e15;            // ... nnz^2 * K decides instead
 constexpr int64_t kRowsAutoMaxRow = 1 << 16;
 
-int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st) {
-  using hpspmm::kSlot;
-  using hpspmm::kSlotsPerTile;
-  constexpr int kTile = hpspmm::kRowTile;
-  const int64_t rows = p->rows, nnz = p->nnz;
-  std::vector<int32_t> rp((size_t)rows + 1), ci((size_t)(nnz > 0 ? nnz : 1));
-  HPSPMM_HIP(hipMemcpyAsync(rp.data(), d_rowptr, rp.size() * sizeof(int32_t), hipMemcpyDeviceToHost, st));
-  if (nnz > 0) HPSPMM_HIP(hipMemcpyAsync(ci.data(), d_col, (size_t)nnz * sizeof(int32_t), hipMemcpyDeviceToHost, st));
-  HPSPMM_HIP(hipStreamSynchronize(st));
-
-  auto class_of = [](int32_t n) { return n <= 8 ? 0 : n <= 16 ? 1 : n <= 32 ? 2 : n <= 64 ? 3 : 4; };
-  int64_t count[5] = {0, 0, 0, 0, 0}, loop_tiles = 0;
-  int64_t by_len[kSlot + 1] = {0};  // one-slot rows by length, longest first: tiles of equal depth
-  for (int64_t r = 0; r < rows; ++r) {
-    const int32_t n = rp[r + 1] - rp[r];
-    // an unchecked rowptr (HPSPMM_PLAN_NO_VALIDATE) that is not monotone or runs past nnz: no tiles,
-    // the CSR kernel is left to the caller's arrays as they are
-    if (n < 0 || rp[r] < 0 || (int64_t)rp[r] + n > nnz) return HPSPMM_OK;
-    const int c = class_of(n);
-    ++count[c];
-    if (c == 0) ++by_len[n];
-    if (c == 4) loop_tiles += ceil_div(n, kTile);
-  }
-  int64_t next_of_len[kSlot + 1];
-  for (int64_t n = kSlot, at = 0; n >= 0; --n) {
-    next_of_len[n] = at;
-    at += by_len[n];
-  }
-  // tile ranges: long rows, then the classes from 8 slots a row down to 1
-  const int64_t t3 = count[3], t2 = ceil_div(count[2], 2), t1 = ceil_div(count[1], 4), t0 = ceil_div(count[0], 8);
-  const int64_t first[4] = {loop_tiles + t3 + t2 + t1, loop_tiles + t3 + t2, loop_tiles + t3, loop_tiles};
-  const int64_t tiles = loop_tiles + t3 + t2 + t1 + t0;
-  if (tiles * kTile > kRowTilePadFactor * nnz + (1 << 20) || tiles >= (1 << 24)) return HPSPMM_OK;  // not worth it
-
-  // per entry {column, x}; x: lane 0 of a slot = row, lane 1 = index of the slot's first value,
-  // slot 0 lane 2 = depth of the tile, slot 0 lane 3 = log2(slots per row)
-  std::vector<int2> tent((size_t)tiles * kTile, make_int2(-1, 0));
-  for (int64_t q = 0; q < tiles * kSlotsPerTile; ++q) tent[(size_t)(q * kSlot)].y = -1;  // padding slot until a row takes it
-  std::vector<int2> ldesc((size_t)(count[4] > 0 ? count[4] : 1));
-  std::vector<int32_t> tdepth((size_t)tiles, kSlot);
-  for (int64_t t = first[0]; t < tiles; ++t) tdepth[(size_t)t] = 0;  // one-slot tiles: set by their rows below
-  int64_t group[4] = {0, 0, 0, 0}, next_loop_tile = 0, n_loop = 0, n_wg = 0;
-  // two passes: the rows that get a whole workgroup first in ldesc (and in the tile order), then the rest
-  for (int pass = 0; pass < 2; ++pass)
-  for (int64_t r = 0; r < rows; ++r) {
-    const int32_t lb = rp[r], n = rp[r + 1] - lb;
-    const int c = class_of(n);
-    if ((pass == 0) != (n > kRowTileWorkgroupRows)) continue;
-    if (pass == 0) ++n_wg;
-    int64_t slot;  // first slot of the row
-    int64_t slots;
-    if (c == 4) {
-      const int64_t nt = ceil_div(n, kTile);
-      ldesc[(size_t)n_loop++] = make_int2((int)next_loop_tile, (int)nt);
-      slot = next_loop_tile * kSlotsPerTile;
-      slots = nt * kSlotsPerTile;
-      next_loop_tile += nt;
-    } else {
-      slots = (int64_t)1 << c;
-      const int64_t g = c == 0 ? next_of_len[n]++ : group[c]++;
-      slot = first[c] * kSlotsPerTile + g * slots;
-      if (c == 0) tdepth[(size_t)(slot / kSlotsPerTile)] = std::max(tdepth[(size_t)(slot / kSlotsPerTile)], n);
-    }
-    for (int64_t j = 0; j < slots; ++j) {
-      int2* ent = &tent[(size_t)((slot + j) * kSlot)];
-      ent[0].y = (int)r;
-      ent[1].y = (int)(lb + j * kSlot);
-      for (int e = 0; e < kSlot; ++e) {
-        const int64_t at = j * kSlot + e;
-        if (at < n) ent[e].x = ci[(size_t)(lb + at)];
-      }
-    }
-  }
-
-  for (int64_t t = 0; t < tiles; ++t) {
-    tent[(size_t)(t * kTile + 2)].y = tdepth[(size_t)t];
-    tent[(size_t)(t * kTile + 3)].y = t < loop_tiles || t < first[2] ? 3 : t < first[1] ? 2 : t < first[0] ? 1 : 0;
-  }
-  const size_t bytes_ent = tent.size() * sizeof(int2), bytes_loop = ldesc.size() * sizeof(int2);
-  if (hipMalloc(&p->d_tent, bytes_ent) != hipSuccess || hipMalloc(&p->d_ldesc, bytes_loop) != hipSuccess || hipMalloc(&p->d_zrow, 32 * sizeof(float)) != hipSuccess) {
-    (void)hipGetLastError();
-    return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the row tiles failed",
-                bytes_ent + bytes_loop);
-  }
-  p->workspace_bytes += (int64_t)(bytes_ent + bytes_loop + 32 * sizeof(float));
-  HPSPMM_HIP(hipMemcpyAsync(p->d_tent, tent.data(), bytes_ent, hipMemcpyHostToDevice, st));
-  HPSPMM_HIP(hipMemcpyAsync(p->d_ldesc, ldesc.data(), bytes_loop, hipMemcpyHostToDevice, st));
-  HPSPMM_HIP(hipMemsetAsync(p->d_zrow, 0, 32 * sizeof(float), st));
-  HPSPMM_HIP(hipStreamSynchronize(st));  // the host vectors go out of scope
-  p->rt_tiles = (int32_t)tiles;
-  p->rt_loop = (int32_t)n_loop;
-  p->rt_wg = (int32_t)n_wg;
-  p->rt_loop_tiles = (int32_t)loop_tiles;
-  p->rt_waves = (int32_t)(n_loop + (tiles - loop_tiles));
-  return HPSPMM_OK;
-}
+int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st);
 
 // The row-tile kernels read val[0] for padding entries (and discard it): a matrix without
 // nonzeros may come with val == NULL, so give them some readable address then.
@@ -705,6 +611,106 @@ int radix_sort_pairs(int64_t n, uint32_t* d_keys[2], int32_t* d_vals[2], uint32_
     cur ^= 1;
   }
   *result = cur;
+  return HPSPMM_OK;
+}
+
+// The rows sorted by group (one radix pass over the group numbers, stable: rows of a group stay in
+// row order), the tile ranges from the group sizes, then one thread per record of the layout.
+int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st) {
+  using hpspmm::kSlotsPerTile;
+  constexpr int kTile = hpspmm::kRowTile;
+  constexpr int kGroups = hpspmm::kRowTileGroups;
+  const int64_t rows = p->rows, nnz = p->nnz;
+  if (rows <= 0) return HPSPMM_OK;
+
+  DeviceTemps tmp;
+  const int64_t n_tiles = ceil_div(rows, hpspmm::kSortTile);
+  const size_t scan_words = (size_t)std::max(scan_scratch_words(256 * n_tiles), scan_scratch_words(rows + 1));
+  for (int i = 0; i < 2; ++i) {
+    tmp.room<uint32_t>((size_t)rows);
+    tmp.room<int32_t>((size_t)rows);
+  }
+  tmp.room<uint32_t>((size_t)(256 * n_tiles + 1));
+  tmp.room<uint32_t>(scan_words);
+  tmp.room<uint32_t>(kGroups + 2);
+  tmp.room<uint32_t>((size_t)rows + 1);
+  if (int rc = tmp.reserve()) return rc;
+  uint32_t* d_keys[2];
+  int32_t* d_ids[2];
+  for (int i = 0; i < 2; ++i) {
+    d_keys[i] = tmp.take<uint32_t>((size_t)rows);
+    d_ids[i] = tmp.take<int32_t>((size_t)rows);
+  }
+  uint32_t* d_hist = tmp.take<uint32_t>((size_t)(256 * n_tiles + 1));
+  uint32_t* d_scan = tmp.take<uint32_t>(scan_words);
+  uint32_t* d_count = tmp.take<uint32_t>(kGroups + 2);
+  uint32_t* d_long = tmp.take<uint32_t>((size_t)rows + 1);  // tiles of the rows with tiles of their own, then their scan
+
+  HPSPMM_HIP(hipMemsetAsync(d_count, 0, (kGroups + 2) * sizeof(uint32_t), st));
+  hipLaunchKernelGGL(hpspmm::rowtile_classify_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                     0, st, rows, nnz, d_rowptr, d_keys[0], d_ids[0], d_count);
+  int sorted = 0;
+  if (int rc = radix_sort_pairs(rows, d_keys, d_ids, d_hist, d_scan, 8, st, &sorted)) return rc;
+  const int32_t* d_order = d_ids[sorted];
+  uint32_t cnt[kGroups + 2];
+  HPSPMM_HIP(hipMemcpyAsync(cnt, d_count, sizeof cnt, hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  // an unchecked rowptr (HPSPMM_PLAN_NO_VALIDATE) that is not monotone or runs past nnz: no tiles,
+  // the CSR kernel is left to the caller's arrays as they are
+  if (cnt[kGroups + 1] != 0) return HPSPMM_OK;
+
+  hpspmm::RowTileLayout lay{};
+  lay.count[4] = (int64_t)cnt[0] + cnt[1];
+  lay.count[3] = cnt[2];
+  lay.count[2] = cnt[3];
+  lay.count[1] = cnt[4];
+  lay.count[0] = 0;
+  for (int g = 5; g < kGroups; ++g) lay.count[0] += cnt[g];
+  lay.loop_tiles = cnt[kGroups];
+  lay.start[4] = 0;
+  lay.start[3] = lay.count[4];
+  lay.start[2] = lay.start[3] + lay.count[3];
+  lay.start[1] = lay.start[2] + lay.count[2];
+  lay.start[0] = lay.start[1] + lay.count[1];
+  // tile ranges: long rows, then the classes from 8 slots a row down to 1
+  const int64_t t3 = lay.count[3], t2 = ceil_div(lay.count[2], 2), t1 = ceil_div(lay.count[1], 4),
+                t0 = ceil_div(lay.count[0], 8);
+  lay.first[3] = lay.loop_tiles;
+  lay.first[2] = lay.loop_tiles + t3;
+  lay.first[1] = lay.loop_tiles + t3 + t2;
+  lay.first[0] = lay.loop_tiles + t3 + t2 + t1;
+  lay.tiles = lay.loop_tiles + t3 + t2 + t1 + t0;
+  const int64_t tiles = lay.tiles;
+  if (tiles * kTile > kRowTilePadFactor * nnz + (1 << 20) || tiles >= (1 << 24)) return HPSPMM_OK;  // not worth it
+
+  const int64_t n_loop = lay.count[4];
+  const size_t bytes_ent = (size_t)tiles * kTile * sizeof(int2);
+  const size_t bytes_loop = (size_t)std::max<int64_t>(n_loop, 1) * sizeof(int2);
+  if (hipMalloc(&p->d_tent, bytes_ent) != hipSuccess || hipMalloc(&p->d_ldesc, bytes_loop) != hipSuccess ||
+      hipMalloc(&p->d_zrow, 32 * sizeof(float)) != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the row tiles failed", bytes_ent + bytes_loop);
+  }
+  p->workspace_bytes += (int64_t)(bytes_ent + bytes_loop + 32 * sizeof(float));
+  if (n_loop > 0) {
+    hipLaunchKernelGGL(hpspmm::rowtile_long_tiles_kernel, dim3((unsigned)ceil_div(n_loop + 1, hpspmm::kBlock)),
+                       dim3(hpspmm::kBlock), 0, st, n_loop, d_order, d_rowptr, d_long);
+    if (int rc = exclusive_scan_u32(d_long, d_long, n_loop + 1, st, d_scan)) return rc;
+    hipLaunchKernelGGL(hpspmm::rowtile_ldesc_kernel, dim3((unsigned)ceil_div(n_loop, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                       0, st, n_loop, d_long, p->d_ldesc);
+  }
+  if (tiles > 0)
+    hipLaunchKernelGGL(hpspmm::rowtile_fill_kernel, dim3((unsigned)ceil_div(tiles * kTile, hpspmm::kBlock)),
+                       dim3(hpspmm::kBlock), 0, st, lay, d_order, p->d_ldesc, d_rowptr, d_col, p->d_tent);
+  HPSPMM_HIP(hipMemsetAsync(p->d_zrow, 0, 32 * sizeof(float), st));
+  hipError_t e = hipStreamSynchronize(st);  // the temporaries go out of scope
+  if (e == hipSuccess) e = hipGetLastError();
+  if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "row tiles: %s", hipGetErrorString(e));
+  p->rt_tiles = (int32_t)tiles;
+  p->rt_loop = (int32_t)n_loop;
+  p->rt_wg = (int32_t)cnt[0];
+  p->rt_loop_tiles = (int32_t)lay.loop_tiles;
+  p->rt_waves = (int32_t)(n_loop + (tiles - lay.loop_tiles));
   return HPSPMM_OK;
 }
 

@@ -47,6 +47,130 @@ constexpr int kSlot = 8;          // nonzeros per slot = lanes per sub-wave at a
 constexpr int kSlotsPerTile = 8;  // slots per tile = sub-waves per wavefront
 constexpr int kRowTile = kSlot * kSlotsPerTile;
 
+// ---- plan-time kernels: the row-tile layout is built on the device -----------------------------
+
+constexpr int32_t kRowTileWorkgroupRows = 512;  // rows beyond this many nonzeros get a whole workgroup
+constexpr int kRowTileGroups = 14;              // sort groups, in the order of the tiles (see rowtile_group)
+
+// Size class of a row: 0..3 = 1 / 2 / 4 / 8 slots of one tile, 4 = tiles of its own.
+__device__ __host__ __forceinline__ int rowtile_class(int32_t n) { return n <= 8 ? 0 : n <= 16 ? 1 : n <= 32 ? 2 : n <= 64 ? 3 : 4; }
+
+// Position of a row's group in the tile order: rows that get a workgroup, the other rows with tiles
+// of their own, then 8 / 4 / 2 slots a row, then the one-slot rows from 8 nonzeros down to none.
+__device__ __forceinline__ int rowtile_group(int32_t n) {
+  const int c = rowtile_class(n);
+  return c == 4 ? (n > kRowTileWorkgroupRows ? 0 : 1) : c == 3 ? 2 : c == 2 ? 3 : c == 1 ? 4 : 5 + (kSlot - n);
+}
+
+// key[r] = group of row r, id[r] = r; count[g] += rows of group g; count[kRowTileGroups] += tiles
+// of the rows with tiles of their own; count[kRowTileGroups + 1] != 0 if rowptr is not a row
+// pointer array of a matrix with nnz nonzeros (unchecked input: the layout is then not built).
+__global__ __launch_bounds__(kBlock) void rowtile_classify_kernel(int64_t rows, int64_t nnz,
+                                                                  const int32_t* __restrict__ rowptr,
+                                                                  uint32_t* __restrict__ key, int32_t* __restrict__ id,
+                                                                  uint32_t* __restrict__ count) {
+  __shared__ uint32_t s_count[kRowTileGroups + 2];
+  if (threadIdx.x < kRowTileGroups + 2) s_count[threadIdx.x] = 0;
+  __syncthreads();
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r < rows) {
+    const int32_t lb = rowptr[r];
+    const int64_t n = (int64_t)rowptr[r + 1] - lb;
+    if (n < 0 || lb < 0 || (int64_t)lb + n > nnz) {
+      atomicAdd(&s_count[kRowTileGroups + 1], 1u);
+      key[r] = 0;
+    } else {
+      const int g = rowtile_group((int32_t)n);
+      key[r] = (uint32_t)g;
+      atomicAdd(&s_count[g], 1u);
+      if (g < 2) atomicAdd(&s_count[kRowTileGroups], (uint32_t)((n + kRowTile - 1) / kRowTile));
+    }
+    id[r] = (int32_t)r;
+  }
+  __syncthreads();
+  if (threadIdx.x < kRowTileGroups + 2 && s_count[threadIdx.x]) atomicAdd(&count[threadIdx.x], s_count[threadIdx.x]);
+}
+
+// tiles[i] = tiles of the i-th row with tiles of its own (order[] = rows sorted by group), [n] = 0.
+__global__ __launch_bounds__(kBlock) void rowtile_long_tiles_kernel(int64_t n, const int32_t* __restrict__ order,
+                                                                    const int32_t* __restrict__ rowptr,
+                                                                    uint32_t* __restrict__ tiles) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i > n) return;
+  uint32_t t = 0;
+  if (i < n) {
+    const int32_t r = order[i];
+    t = (uint32_t)((rowptr[r + 1] - rowptr[r] + kRowTile - 1) / kRowTile);
+  }
+  tiles[i] = t;
+}
+
+// ldesc[i] = {first tile, tiles} of the i-th such row, from the scan of tiles[].
+__global__ __launch_bounds__(kBlock) void rowtile_ldesc_kernel(int64_t n, const uint32_t* __restrict__ first,
+                                                               int2* __restrict__ ldesc) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) ldesc[i] = make_int2((int)first[i], (int)(first[i + 1] - first[i]));
+}
+
+struct RowTileLayout {
+  int64_t tiles, loop_tiles;
+  int64_t first[4];  // first tile of size class 0..3
+  int64_t start[5];  // first position in order[] of size class 0..4
+  int64_t count[5];  // rows of size class 0..4
+};
+
+// Every record of the layout, one thread each: record e of slot q belongs to slot j of some row, or
+// to no row (padding).  Lane 0 of a slot carries the row, lane 1 the index of the slot's first value,
+// lanes 2 and 3 of a tile's first slot the tile's depth and log2 of the slots per row.
+__global__ __launch_bounds__(kBlock) void rowtile_fill_kernel(RowTileLayout lay, const int32_t* __restrict__ order,
+                                                              const int2* __restrict__ ldesc,
+                                                              const int32_t* __restrict__ rowptr,
+                                                              const int32_t* __restrict__ col, int2* __restrict__ tent) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= lay.tiles * kRowTile) return;
+  const int e = (int)(i % kSlot);
+  const int64_t q = i / kSlot;  // slot
+  const int64_t t = q / kSlotsPerTile;
+  int32_t row = -1;
+  int64_t j = 0;  // the row's slot number
+  int lg = 3, depth = kSlot;
+  if (t < lay.loop_tiles) {
+    // the row whose tiles include t: the last one that starts at or before t
+    int64_t lo = 0, hi = lay.count[4];
+    while (hi - lo > 1) {
+      const int64_t mid = (lo + hi) >> 1;
+      if ((int64_t)ldesc[mid].x <= t) lo = mid; else hi = mid;
+    }
+    row = order[lay.start[4] + lo];
+    j = q - (int64_t)ldesc[lo].x * kSlotsPerTile;
+  } else {
+    const int c = t >= lay.first[0] ? 0 : t >= lay.first[1] ? 1 : t >= lay.first[2] ? 2 : 3;
+    lg = c;
+    const int64_t rel = q - lay.first[c] * kSlotsPerTile;
+    const int64_t g = rel >> c;
+    if (g < lay.count[c]) {
+      row = order[lay.start[c] + g];
+      j = rel & (((int64_t)1 << c) - 1);
+    }
+    if (c == 0) {  // one-slot rows are sorted by length, longest first: the tile's first row has its depth
+      const int32_t r0 = order[lay.start[0] + (t - lay.first[0]) * kSlotsPerTile];
+      depth = rowptr[r0 + 1] - rowptr[r0];
+    }
+  }
+  int2 rec = make_int2(-1, e == 0 ? -1 : 0);
+  if (row >= 0) {
+    const int32_t lb = rowptr[row], n = rowptr[row + 1] - lb;
+    const int64_t at = j * kSlot + e;
+    rec.x = at < n ? col[lb + at] : -1;
+    rec.y = e == 0 ? row : e == 1 ? (int32_t)(lb + j * kSlot) : 0;
+  }
+  if (q % kSlotsPerTile == 0) {
+    if (e == 2) rec.y = depth;
+    if (e == 3) rec.y = lg;
+  }
+  tent[i] = rec;
+}
+
 // acc += the first N products of the slot whose columns are staged in s_col; `c` is this lane's
 // own column, `v` its value (load already issued), `zrow` = 32 zeros in device memory.  Nothing in
 // here is conditional: a padding entry among the first N gathers the zero row instead of a row of

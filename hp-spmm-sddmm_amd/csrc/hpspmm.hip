@@ -267,7 +267,7 @@ int launch_rows(int64_t rows, int64_t cols, const int32_t* rp, const int32_t* ci
 // Row tiles (rows strategy): every row cut into slots of 8 nonzeros, 8 slots to a tile, a row's
 // slots adjacent in one tile (1 / 2 / 4 / 8 of them for up to 8 / 16 / 32 / 64 nonzeros, tiles
 // sorted by that class), longer rows over consecutive tiles, those that get a whole workgroup
-// first.  Built on the device (0.2 ms at 100k nonzeros, 1 ms at 10 M; on the host it took about
+// first.  Built on the device (0.2 ms at 100k nonzeros, 0.5 ms at 12 M; on the host it took about
 // 3 ms per million nonzeros, after copying the column indices over).  Skipped (the kernel then walks the
 // CSR arrays) when padding would blow the layout up, which is what a matrix of mostly empty rows
 // does, and beyond kRowTileMaxNnz (rows strategy forced on a very large matrix).

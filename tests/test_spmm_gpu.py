@@ -532,6 +532,34 @@ def test_random_matrices_all_strategies(pkg, oracle, gpu, seed):
         assert not C[np.diff(rowptr) == 0].any()
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_matrices_column_tiles(pkg, oracle, gpu, seed):
+    """The same at row lengths that are multiples of a tuned one: the forced sweep, routed and ordered
+    plans run in column tiles, the others through the kernels for any multiple of 4."""
+    import scipy.sparse as sp
+    rng = np.random.default_rng(2000 + seed)
+    rows = int(rng.integers(1, 3000))
+    cols = int(rng.integers(1, 3000))
+    k = int(rng.choice([96, 160, 192, 256, 384]))
+    rowptr, col, val = _random_csr(rng, rows, cols, mean_deg=float(rng.uniform(0.5, 40)),
+                                   skew=float(rng.uniform(0.8, 3.0)), empty_frac=float(rng.uniform(0, 0.6)),
+                                   sorted_unique=(seed % 3 != 2))
+    g = pkg.graphs.CSR(rows, cols, rowptr, col, val)
+    B = rng.standard_normal((cols, k)).astype(np.float32)
+    A = sp.csr_matrix((val.astype(np.float64), col.copy(), rowptr.copy()), shape=(rows, cols))
+    Aabs = sp.csr_matrix((np.abs(val).astype(np.float64), col.copy(), rowptr.copy()), shape=(rows, cols))
+    want = A @ B.astype(np.float64)
+    S = Aabs @ np.abs(B).astype(np.float64)
+    tiled = 0
+    for name, flags in _strategies(pkg.capi):
+        C, info = _run(pkg, gpu, g, B, flags)
+        tiled += info["column_tiles"] > 1
+        bad = np.abs(C - want) > TOL * S
+        assert not bad.any(), f"seed {seed} rows={rows} cols={cols} k={k} {name}: {int(bad.sum())} elements off"
+        assert not C[np.diff(rowptr) == 0].any()
+    assert tiled >= 4 or col.size == 0, f"seed {seed}: only {tiled} plans ran in column tiles"
+
+
 def test_non_finite_values_stay_in_their_rows(pkg, oracle, gpu):
     """An inf / NaN in B reaches exactly the rows that reference that row of B (no 0 * inf leaks
     from padding or predication)."""

@@ -899,9 +899,28 @@ constexpr double kRoutedMinRoutedShare = 0.3;  // of the nonzeros in rows of at 
 // 2.51 ms; R-MAT scale 22, K = 128 (268 MB a slice) 6.63 / 6.23 / 6.32 ms.
 constexpr int64_t kRoutedPhaseBytes = (int64_t)8 << 20;
 
-// True if the column indices of every row are in non-decreasing order (p->d_nnz_row = row of every
-// nonzero must be there).  Errors count as "no".
-bool columns_sorted(const hpspmm_plan* p, const int32_t* d_col, hipStream_t st) {
+// p->d_nnz_row = the row of every nonzero, built the first time a step of the construction needs it
+// (the segments kernels, the sortedness check, the routed and sweep layouts do; a plan that ends up
+// with the ordered strategy or with row tiles never does).
+int ensure_row_expansion(hpspmm_plan* p, const int32_t* d_rowptr, hipStream_t st) {
+  if (p->d_nnz_row) return HPSPMM_OK;
+  const size_t row_bytes = (size_t)std::max<int64_t>(p->nnz, 1) * sizeof(int32_t);
+  if (hipMalloc(&p->d_nnz_row, row_bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    p->d_nnz_row = nullptr;
+    return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the plan failed", row_bytes);
+  }
+  p->workspace_bytes += (int64_t)row_bytes;
+  if (p->nnz > 0)
+    hipLaunchKernelGGL(hpspmm::expand_rows_kernel, dim3((unsigned)ceil_div(p->nnz, hpspmm::kExpandPerBlock)),
+                       dim3(hpspmm::kBlock), 0, st, p->rows, p->nnz, d_rowptr, p->d_nnz_row);
+  HPSPMM_HIP(hipGetLastError());
+  return HPSPMM_OK;
+}
+
+// True if the column indices of every row are in non-decreasing order.  Errors count as "no".
+bool columns_sorted(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st) {
+  if (ensure_row_expansion(p, d_rowptr, st) != HPSPMM_OK) return false;
   int32_t* d_flag = nullptr;
   if (hipMalloc(&d_flag, sizeof(int32_t)) != hipSuccess) {
     (void)hipGetLastError();
@@ -978,8 +997,8 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
            (void**)&d_chunk_base, (void**)&d_chunk_row}};
 
   bool inplace = false;
-  if (!sort_values && nsub == 1 && nnz > 0 && p->cols * p->k_full * 4 < ((int64_t)1 << 32) && p->d_nnz_row &&
-      columns_sorted(p, d_col, st)) {
+  if (!sort_values && nsub == 1 && nnz > 0 && p->cols * p->k_full * 4 < ((int64_t)1 << 32) &&
+      columns_sorted(p, d_rowptr, d_col, st)) {
     const int groups = nhub;
     const int64_t target = ceil_div(rk.sampled, groups);  // the column counts are those of the sample
     uint32_t* d_before = nullptr;
@@ -1124,6 +1143,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   const size_t routed_rows_bytes = (size_t)std::max<int64_t>(n_routed, 1) * sizeof(int32_t);
   // the segments strategy's carry slots are not needed any more (the row of every nonzero is, for the fill)
   if (p->d_carry) { (void)hipFree(p->d_carry); p->d_carry = nullptr; }
+  if (int rc = ensure_row_expansion(p, d_rowptr, st)) return rc;
   const size_t total_bytes = rvptr_bytes + coldptr_bytes + 3 * v_bytes +
                              (inplace ? 0 : lslot_bytes + 2 * chunk_bytes) + partial_bytes + carry_bytes +
                              bhot_bytes + (size_t)n_bhot * 4 + 2 * list_bytes + routed_rows_bytes;
@@ -1184,7 +1204,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   HPSPMM_HIP(hipGetLastError());
   p->n_cross = counts[0];
   p->n_zero = counts[1];
-  (void)hipFree(p->d_nnz_row);  // the row of every nonzero was the segments strategy's; the class-major arrays replace it
+  (void)hipFree(p->d_nnz_row);  // the row of every nonzero served the fill; the class-major arrays replace it
   p->d_nnz_row = nullptr;
   p->n_bhot = inplace ? 0 : n_bhot;
   p->n_hub = inplace ? 0 : (int64_t)n_ids;
@@ -1564,13 +1584,13 @@ void drop_sweep_buffers(hpspmm_plan* p) {
   }
 }
 
-// Builds the sweep layout on top of a segments plan (p->d_nnz_row must be there).  Returns HPSPMM_OK
+// Builds the sweep layout on top of a segments plan.  Returns HPSPMM_OK
 // with p->strategy left at SEGMENTS when the matrix does not qualify.  Diagnostics: the environment
 // variables HPSPMM_SWEEP_WINDOW_LOG2 (bytes of B per window), HPSPMM_SWEEP_LEAD, HPSPMM_SWEEP_SPIN,
 // HPSPMM_SWEEP_LIMIT (nonzeros per piece) and HPSPMM_SWEEP_PRIORITIES override the defaults.
 int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, hipStream_t st) {
   const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
-  if (nnz <= 0 || !p->d_nnz_row) return HPSPMM_OK;
+  if (nnz <= 0) return HPSPMM_OK;
   // gather offsets are 32-bit, stream entries keep the column in 24 bits
   if (p->cols * p->k_full * 4 >= ((int64_t)1 << 32) || p->cols > ((int64_t)1 << hpspmm::kSweepColBits)) return HPSPMM_OK;
   if (!forced && (nnz < kSweepMinNnz || p->cols * k * 4 < kSweepMinBBytes)) return HPSPMM_OK;
@@ -1608,7 +1628,7 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   // (rules the layout out for a matrix of many short rows before any kernel has run)
   if (!forced && (ceil_div(nonempty, band_waves * WS) * hpspmm::kXcds * p->cols > nnz / 4 || nonempty * n_windows * 3 > nnz * 2))
     return HPSPMM_OK;
-  if (!columns_sorted(p, d_col, st)) return HPSPMM_OK;  // a row must meet the windows in stored order
+  if (!columns_sorted(p, d_rowptr, d_col, st)) return HPSPMM_OK;  // a row must meet the windows in stored order
   if (!forced) {
     // rows that reach across most of the columns (a banded matrix is better off with whole rows or segments)
     unsigned long long* d_span = nullptr;
@@ -1799,8 +1819,8 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
             (long long)n_bands, (long long)n_waves, (long long)n_windows, limit, n_pieces, counts[0], (long long)nnz,
             (long long)total, (double)total / (double)nnz);
   // the segments plan underneath is no longer needed
-  (void)hipFree(p->d_nnz_row);
-  (void)hipFree(p->d_carry);
+  if (p->d_nnz_row) (void)hipFree(p->d_nnz_row);
+  if (p->d_carry) (void)hipFree(p->d_carry);
   p->d_nnz_row = nullptr;
   p->d_carry = nullptr;
   p->workspace_bytes = 2 * total * 4 + (int64_t)std::max<int64_t>(n_parts, 1) * k * 4 + (n_waves + 1) * 4 + n_waves * 4 +
@@ -2005,21 +2025,8 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     }
     p->shift = forced ? forced : choose_shift(nnz, k, p->max_row_nnz);
     p->nseg = ceil_div(nnz, (int64_t)1 << p->shift);
-    const size_t row_bytes = (size_t)(nnz > 0 ? nnz : 1) * sizeof(int32_t);
-    const size_t carry_bytes = (size_t)(p->nseg > 0 ? p->nseg : 1) * 2 * (size_t)k * sizeof(float);
-    if (hipMalloc(&p->d_nnz_row, row_bytes) != hipSuccess || hipMalloc(&p->d_carry, carry_bytes) != hipSuccess) {
-      (void)hipGetLastError();
-      return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the plan failed", row_bytes + carry_bytes);
-    }
-    p->workspace_bytes = (int64_t)(row_bytes + carry_bytes);
-    if (nnz > 0) {
-      hipLaunchKernelGGL(hpspmm::expand_rows_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kExpandPerBlock)),
-                         dim3(hpspmm::kBlock), 0, st, rows, nnz, d_rowptr, p->d_nnz_row);
-      hipError_t e = hipStreamSynchronize(st);
-      if (e != hipSuccess) {
-        return fail(HPSPMM_ERR_HIP, "row expansion failed: %s", hipGetErrorString(e));
-      }
-    }
+    // what the segments kernels need (the row of every nonzero, the carry slots) is allocated at the
+    // end, if the plan is still a segments plan then: the layouts tried below mostly replace both
   }
   // Long rows over a B that is small against the gather volume: every wavefront walks B window by
   // window (tried first: where it qualifies it beats the routed strategy - social graph, 233k
@@ -2069,11 +2076,11 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       return rc;
     }
     if (p->d_tent) {
-      (void)hipFree(p->d_nnz_row);
-      (void)hipFree(p->d_carry);
-      p->d_nnz_row = nullptr;
-      p->d_carry = nullptr;
-      p->workspace_bytes -= (int64_t)((size_t)nnz * sizeof(int32_t) + (size_t)p->nseg * 2 * (size_t)k * sizeof(float));
+      if (p->d_nnz_row) {  // a layout tried above has asked for it
+        (void)hipFree(p->d_nnz_row);
+        p->d_nnz_row = nullptr;
+        p->workspace_bytes -= (int64_t)((size_t)std::max<int64_t>(nnz, 1) * sizeof(int32_t));
+      }
       p->nseg = 0;
       p->shift = 0;
       p->strategy = HPSPMM_STRATEGY_ROWS;
@@ -2102,6 +2109,20 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       return fail(HPSPMM_ERR_HIP, "long-row collection failed: %s", hipGetErrorString(e));
     }
     p->n_long = n_long;
+  }
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS) {
+    if (int rc = ensure_row_expansion(p, d_rowptr, st)) return rc;
+    const size_t carry_bytes = (size_t)std::max<int64_t>(p->nseg, 1) * 2 * (size_t)k * sizeof(float);
+    if (!p->d_carry) {
+      if (hipMalloc(&p->d_carry, carry_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        p->d_carry = nullptr;
+        return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the plan failed", carry_bytes);
+      }
+      p->workspace_bytes += (int64_t)carry_bytes;
+    }
+    const hipError_t e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "row expansion failed: %s", hipGetErrorString(e));
   }
   holder.plan = nullptr;
   *plan_out = p;

@@ -69,11 +69,12 @@ inline int64_t tile_width(int64_t k) {
   if (fast_k(k) || k <= 0) return 0;
   return k % 128 == 0 ? 128 : k % 64 == 0 ? 64 : k % 32 == 0 ? 32 : 0;
 }
-// Row lengths served by the run-time-K sub-wave kernels: multiples of 4 that are not a tuned size.
-inline bool anyk_k(int64_t k) { return !fast_k(k) && k % 4 == 0 && k <= (1 << 20); }
+// Every row length that is not a tuned size goes to the run-time-K sub-wave kernels.
+// Not a multiple of 4: rows of B and C start at any multiple of 4 bytes, the last lane of a row owns 1 to 3 columns.
+inline bool odd_k(int64_t k) { return k % 4 != 0; }
 // Lanes per sub-wave for such a K: the power of two that covers a column tile (at most 128 floats).
 inline int anyk_lanes(int64_t k) {
-  const int64_t g = (k < hpspmm::kAnyKTile ? k : hpspmm::kAnyKTile) / 4;
+  const int64_t g = ((k < hpspmm::kAnyKTile ? k : hpspmm::kAnyKTile) + 3) / 4;
   int gp = 2;
   while (gp < g) gp <<= 1;
   return gp;
@@ -327,14 +328,14 @@ int launch_row_tiles(const hpspmm_plan* p, const float* v, const float* B, float
   return launch_row_tiles_w<K, hpspmm::kWavesPerBlock>(p, v, B, C, st);
 }
 
-template <int GP>
+template <int GP, bool kOdd>
 int launch_rows_anyk_g(int64_t rows, int64_t k, const int32_t* rp, const int32_t* ci, const float* v, const float* B,
                        float* C, int32_t long_threshold, const int32_t* long_rows, int64_t n_long, hipStream_t st) {
   const int tiles = anyk_tiles(k);
   const int64_t short_blocks = ceil_div(ceil_div(rows, 64 / GP), hpspmm::kWavesPerBlock);
   const int64_t blocks = (short_blocks + ceil_div(n_long, hpspmm::kWavesPerBlock)) * tiles;
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
-  hipLaunchKernelGGL(hpspmm::spmm_rows_anyk_kernel<GP>, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rows,
+  hipLaunchKernelGGL((hpspmm::spmm_rows_anyk_kernel<GP, kOdd>), dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rows,
                      (int)k, tiles, rp, ci, v, B, C, short_blocks, long_threshold, long_rows, n_long);
   mark_launch(st, "spmm_rows_anyk_kernel");
   return HPSPMM_OK;
@@ -342,29 +343,33 @@ int launch_rows_anyk_g(int64_t rows, int64_t k, const int32_t* rp, const int32_t
 
 int launch_rows_anyk(int64_t rows, int64_t k, const int32_t* rp, const int32_t* ci, const float* v, const float* B,
                      float* C, int32_t long_threshold, const int32_t* long_rows, int64_t n_long, hipStream_t st) {
+#define HPSPMM_ROWS_ANYK(GP)                                                                                        \
+  return odd_k(k) ? launch_rows_anyk_g<GP, true>(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st)   \
+                  : launch_rows_anyk_g<GP, false>(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st)
   switch (anyk_lanes(k)) {
-    case 2: return launch_rows_anyk_g<2>(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
-    case 4: return launch_rows_anyk_g<4>(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
-    case 8: return launch_rows_anyk_g<8>(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
-    case 16: return launch_rows_anyk_g<16>(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
-    default: return launch_rows_anyk_g<32>(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
+    case 2: HPSPMM_ROWS_ANYK(2);
+    case 4: HPSPMM_ROWS_ANYK(4);
+    case 8: HPSPMM_ROWS_ANYK(8);
+    case 16: HPSPMM_ROWS_ANYK(16);
+    default: HPSPMM_ROWS_ANYK(32);
   }
+#undef HPSPMM_ROWS_ANYK
 }
 
-template <int GP>
+template <int GP, bool kOdd>
 int launch_segments_anyk_g(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, const float* v, const float* B,
                            float* C, hipStream_t st) {
   const int tiles = anyk_tiles(p->k);
   const int64_t blocks = ceil_div(ceil_div(p->nseg, 64 / GP), hpspmm::kWavesPerBlock) * tiles;
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   if (p->nnz > 0) {
-    hipLaunchKernelGGL((hpspmm::spmm_segments_anyk_kernel<GP, false>), dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rp,
+    hipLaunchKernelGGL((hpspmm::spmm_segments_anyk_kernel<GP, false, kOdd>), dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st, rp,
                        ci, v, p->d_nnz_row, B, C, p->d_carry, p->nnz, p->shift, p->nseg, (int)p->k, tiles,
                        aligned16(ci, v, p->d_nnz_row));
     mark_launch(st, "spmm_segments_anyk_kernel");
   }
   const int64_t fix_blocks = ceil_div(ceil_div(p->rows, 64), hpspmm::kWavesPerBlock);
-  hipLaunchKernelGGL(hpspmm::spmm_fixup_anyk_kernel<GP>, dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st,
+  hipLaunchKernelGGL((hpspmm::spmm_fixup_anyk_kernel<GP, kOdd>), dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st,
                      p->rows, rp, (const float*)p->d_carry, C, p->shift, (int)p->k);
   mark_launch(st, "spmm_fixup_anyk_kernel");
   return HPSPMM_OK;
@@ -372,16 +377,20 @@ int launch_segments_anyk_g(const hpspmm_plan* p, const int32_t* rp, const int32_
 
 int launch_segments_anyk(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, const float* v, const float* B,
                          float* C, hipStream_t st) {
+#define HPSPMM_SEGMENTS_ANYK(GP)                                                       \
+  return odd_k(p->k) ? launch_segments_anyk_g<GP, true>(p, rp, ci, v, B, C, st)        \
+                     : launch_segments_anyk_g<GP, false>(p, rp, ci, v, B, C, st)
   switch (anyk_lanes(p->k)) {
-    case 2: return launch_segments_anyk_g<2>(p, rp, ci, v, B, C, st);
-    case 4: return launch_segments_anyk_g<4>(p, rp, ci, v, B, C, st);
-    case 8: return launch_segments_anyk_g<8>(p, rp, ci, v, B, C, st);
-    case 16: return launch_segments_anyk_g<16>(p, rp, ci, v, B, C, st);
-    default: return launch_segments_anyk_g<32>(p, rp, ci, v, B, C, st);
+    case 2: HPSPMM_SEGMENTS_ANYK(2);
+    case 4: HPSPMM_SEGMENTS_ANYK(4);
+    case 8: HPSPMM_SEGMENTS_ANYK(8);
+    case 16: HPSPMM_SEGMENTS_ANYK(16);
+    default: HPSPMM_SEGMENTS_ANYK(32);
   }
+#undef HPSPMM_SEGMENTS_ANYK
 }
 
-template <int GP>
+template <int GP, bool kOdd>
 int launch_coo_anyk_g(int64_t nnz, int64_t k, const int32_t* ri, const int32_t* ci, const float* v, const float* B,
                       float* C, hipStream_t st) {
   constexpr int P = 64 / GP;
@@ -391,7 +400,7 @@ int launch_coo_anyk_g(int64_t nnz, int64_t k, const int32_t* ri, const int32_t* 
   const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
   const int64_t blocks = ceil_div(ceil_div(nseg, P), hpspmm::kWavesPerBlock) * tiles;
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
-  hipLaunchKernelGGL((hpspmm::spmm_segments_anyk_kernel<GP, true>), dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st,
+  hipLaunchKernelGGL((hpspmm::spmm_segments_anyk_kernel<GP, true, kOdd>), dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st,
                      (const int32_t*)nullptr, ci, v, ri, B, C, (float*)nullptr, nnz, shift, nseg, (int)k, tiles,
                      aligned16(ci, v, ri));
   return HPSPMM_OK;
@@ -399,13 +408,17 @@ int launch_coo_anyk_g(int64_t nnz, int64_t k, const int32_t* ri, const int32_t* 
 
 int launch_coo_anyk(int64_t nnz, int64_t k, const int32_t* ri, const int32_t* ci, const float* v, const float* B,
                     float* C, hipStream_t st) {
+#define HPSPMM_COO_ANYK(GP)                                                        \
+  return odd_k(k) ? launch_coo_anyk_g<GP, true>(nnz, k, ri, ci, v, B, C, st)       \
+                  : launch_coo_anyk_g<GP, false>(nnz, k, ri, ci, v, B, C, st)
   switch (anyk_lanes(k)) {
-    case 2: return launch_coo_anyk_g<2>(nnz, k, ri, ci, v, B, C, st);
-    case 4: return launch_coo_anyk_g<4>(nnz, k, ri, ci, v, B, C, st);
-    case 8: return launch_coo_anyk_g<8>(nnz, k, ri, ci, v, B, C, st);
-    case 16: return launch_coo_anyk_g<16>(nnz, k, ri, ci, v, B, C, st);
-    default: return launch_coo_anyk_g<32>(nnz, k, ri, ci, v, B, C, st);
+    case 2: HPSPMM_COO_ANYK(2);
+    case 4: HPSPMM_COO_ANYK(4);
+    case 8: HPSPMM_COO_ANYK(8);
+    case 16: HPSPMM_COO_ANYK(16);
+    default: HPSPMM_COO_ANYK(32);
   }
+#undef HPSPMM_COO_ANYK
 }
 
 int launch_rows_any(int64_t rows, int64_t cols, int64_t k, const int32_t* rp, const int32_t* ci, const float* v,
@@ -416,14 +429,7 @@ int launch_rows_any(int64_t rows, int64_t cols, int64_t k, const int32_t* rp, co
     case 32: return launch_rows<32>(rows, cols, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
     case 64: return launch_rows<64>(rows, cols, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
     case 128: return launch_rows<128>(rows, cols, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
-    default: {
-      if (anyk_k(k)) return launch_rows_anyk(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
-      const int64_t blocks = ceil_div(rows, hpspmm::kWavesPerBlock);
-      hipLaunchKernelGGL(hpspmm::spmm_rows_generic_kernel, dim3((unsigned)blocks), dim3(hpspmm::kBlock), 0, st,
-                         rows, k, rp, ci, v, B, C);
-      mark_launch(st, "spmm_rows_generic_kernel");
-      return HPSPMM_OK;
-    }
+    default: return launch_rows_anyk(rows, k, rp, ci, v, B, C, long_threshold, long_rows, n_long, st);
   }
 }
 
@@ -1966,12 +1972,11 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   ColumnRanking ranking;         // column popularity, shared by the routed and the hub-cache decisions
   bool rows_need_tiles = false;  // rows strategy chosen on the strength of the row tiles
   bool rows_range = false;       // provisional segments; rows unless the ordered strategy qualifies
-  if (!fast_k(k) && !anyk_k(k)) {
-    p->strategy = HPSPMM_STRATEGY_GENERIC_K;
-  } else if (!fast_k(k)) {
-    // a multiple of 4 that is not a tuned size: whole rows for small matrices (one launch), segments
-    // beyond (balanced over any degree distribution); the layouts built for the tuned sizes (row
-    // tiles, routed, ordered, hub cache) are not used
+  if (!fast_k(k)) {
+    // not a tuned size (nor, at this point, a multiple of one on a matrix that gets a tiled layout):
+    // whole rows for small matrices (one launch), segments beyond (balanced over any degree
+    // distribution); the layouts built for the tuned sizes (row tiles, routed, ordered, hub cache)
+    // are not used
     const bool small = nnz < (1 << 21) && p->max_row_nnz <= 4096;
     p->strategy = (flags & HPSPMM_PLAN_FORCE_SEGMENTS)                   ? HPSPMM_STRATEGY_SEGMENTS
                   : ((flags & HPSPMM_PLAN_FORCE_ROWS) || nnz == 0 || small) ? HPSPMM_STRATEGY_ROWS
@@ -2112,7 +2117,8 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   }
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS) {
     if (int rc = ensure_row_expansion(p, d_rowptr, st)) return rc;
-    const size_t carry_bytes = (size_t)std::max<int64_t>(p->nseg, 1) * 2 * (size_t)k * sizeof(float);
+    // (a carry slot holds a row of K rounded up to 4 floats, so that slots stay 16-byte aligned for any K)
+    const size_t carry_bytes = (size_t)std::max<int64_t>(p->nseg, 1) * 2 * (size_t)((k + 3) & ~(int64_t)3) * sizeof(float);
     if (!p->d_carry) {
       if (hipMalloc(&p->d_carry, carry_bytes) != hipSuccess) {
         (void)hipGetLastError();
@@ -2465,12 +2471,7 @@ int hpspmm_coo_spmm_accumulate(int64_t rows, int64_t cols, int64_t nnz, const in
     case 32: rc = launch_coo<32>(nnz, d_row, d_col, d_val, d_B, d_C, st); break;
     case 64: rc = launch_coo<64>(nnz, d_row, d_col, d_val, d_B, d_C, st); break;
     case 128: rc = launch_coo<128>(nnz, d_row, d_col, d_val, d_B, d_C, st); break;
-    default:
-      if (anyk_k(k))  // a multiple of 4: segments reduced in registers, one atomic per flush
-        rc = launch_coo_anyk(nnz, k, d_row, d_col, d_val, d_B, d_C, st);
-      else
-        hipLaunchKernelGGL(hpspmm::spmm_coo_generic_kernel, dim3(grid_for(nnz * k, 1 << 16)), dim3(hpspmm::kBlock), 0,
-                           st, nnz, k, d_row, d_col, d_val, d_B, d_C);
+    default: rc = launch_coo_anyk(nnz, k, d_row, d_col, d_val, d_B, d_C, st);  // segments reduced in registers, one atomic per flush
   }
   if (rc) return rc;
   HPSPMM_HIP(hipGetLastError());

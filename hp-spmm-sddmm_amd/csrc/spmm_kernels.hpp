@@ -265,26 +265,6 @@ __global__ __launch_bounds__(kBlock) void spmm_rows_kernel(int64_t rows, const i
   }
 }
 
-// Any K: one wavefront per row, lanes stride over columns.
-__global__ __launch_bounds__(kBlock) void spmm_rows_generic_kernel(int64_t rows, int64_t K,
-                                                                   const int32_t* __restrict__ rowptr,
-                                                                   const int32_t* __restrict__ col,
-                                                                   const float* __restrict__ val,
-                                                                   const float* __restrict__ B,
-                                                                   float* __restrict__ C) {
-  const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-  if (row >= rows) return;
-  const int32_t lb = rowptr[row];
-  const int32_t hb = rowptr[row + 1];
-  for (int64_t k0 = lane; k0 < K; k0 += 64) {
-    float acc = 0.f;
-    for (int32_t j = lb; j < hb; ++j)
-      acc = __builtin_fmaf(val[j], B[(uint64_t)(uint32_t)col[j] * (uint64_t)K + (uint64_t)k0], acc);
-    C[(uint64_t)row * (uint64_t)K + (uint64_t)k0] = acc;
-  }
-}
-
 // ---------------------------------------------------------------------------
 // Tile engine of the segment-type kernels.
 //
@@ -572,22 +552,6 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
       add(acc, t);
     }
     if (sub == 0) *reinterpret_cast<float4*>(C + (uint64_t)(r0 + i) * ld + 4 * l) = acc;
-  }
-}
-
-// COO accumulate for any K: one thread per (entry, column).
-__global__ __launch_bounds__(kBlock) void spmm_coo_generic_kernel(int64_t nnz, int64_t K,
-                                                                  const int32_t* __restrict__ row,
-                                                                  const int32_t* __restrict__ col,
-                                                                  const float* __restrict__ val,
-                                                                  const float* __restrict__ B,
-                                                                  float* __restrict__ C) {
-  const int64_t total = nnz * K;
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
-    const int64_t j = i / K;
-    const int64_t k0 = i - j * K;
-    unsafeAtomicAdd(C + (uint64_t)(uint32_t)row[j] * (uint64_t)K + (uint64_t)k0,
-                    val[j] * B[(uint64_t)(uint32_t)col[j] * (uint64_t)K + (uint64_t)k0]);
   }
 }
 

@@ -92,7 +92,7 @@ typedef enum hpspmm_status {
 /* strategy reported by hpspmm_plan_get_info */
 #define HPSPMM_STRATEGY_ROWS 1
 #define HPSPMM_STRATEGY_SEGMENTS 2
-#define HPSPMM_STRATEGY_GENERIC_K 3
+#define HPSPMM_STRATEGY_GENERIC_K 3 /* no longer reported: every k runs whole rows or segments on sub-waves */
 #define HPSPMM_STRATEGY_ROUTED 4
 #define HPSPMM_STRATEGY_ORDERED 5
 #define HPSPMM_STRATEGY_SWEEP 6
@@ -142,8 +142,10 @@ const char *hpspmm_last_error(void);
  * reference tiles the columns the same way, spmm/mm/spmm_kernel.cu:412-420:
  * grid.y = ceil(k / 64)), when the matrix gets one of those layouts (at least
  * 2^22 nonzeros, or a forcing flag); launches_per_spmm counts every tile's.
- * Any other multiple of 4 runs whole rows or segments with sub-waves of k / 4
- * lanes rounded up to a power of two, other k one wavefront per row.
+ * Any other k runs whole rows or segments with sub-waves of ceil(k / 4) lanes
+ * rounded up to a power of two; when k is not a multiple of 4 (41 classes, 47,
+ * 173 ...) the rows of B and C are read and written at their 4-byte alignment
+ * and the lane that owns a row's last columns touches only those that exist.
  * Replaces the host-side preprocessing the reference does before timing:
  * CSR->COO expansion (spmm/mm/spmm_common.cpp:185-235), the row re-ordering
  * (:237-296) and the choice of nnz_per_warp (spmm/mm/spmm_kernel.cu:749-751).

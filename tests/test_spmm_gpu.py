@@ -183,14 +183,45 @@ def test_linearity_and_column_tiles(pkg, oracle, gpu):
     assert np.array_equal(C32, C128[:, :32])
 
 
-@pytest.mark.parametrize("k", [1, 7, 30, 50, 130])
-def test_generic_k(pkg, oracle, gpu, k):
-    """Row lengths that are not a multiple of 4 (no 16-byte rows): the one-wavefront-per-row kernel."""
-    g = pkg.graphs.make_graph("c4_rmat", 0.002)
+@pytest.mark.parametrize("k", [1, 2, 3, 5, 7, 30, 41, 47, 50, 127, 129, 130, 173, 259])
+def test_k_not_a_multiple_of_four(pkg, oracle, gpu, k):
+    """Row lengths that are not a multiple of 4 (rows of B and C start at any multiple of 4 bytes; the
+    number of classes of a node classifier is such a K): the same planned sub-wave strategies as for
+    the multiples of 4, the lane that owns the last columns of a row reading and writing only those
+    that exist.  Whole rows, forced segments (three lengths), the plan-less entry point; C poisoned
+    with NaN beforehand and laid out with guard rows, which must stay untouched."""
+    import torch
+    capi = pkg.capi
+    g = pkg.graphs.make_graph("c4_rmat", 0.004)
     B = pkg.graphs.dense_normal(g.cols, k, 77)
     C, info = _run(pkg, gpu, g, B)
-    assert info["strategy"] == pkg.capi.STRATEGY_GENERIC_K
-    _check(oracle, g, B, C, f"generic k={k}")
+    assert info["strategy"] == capi.STRATEGY_ROWS and info["launches_per_spmm"] == 1, info
+    _check(oracle, g, B, C, f"rows k={k}")
+    for shift in (0, 3, 7):
+        C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(shift))
+        assert info["strategy"] == capi.STRATEGY_SEGMENTS and info["launches_per_spmm"] == 2, info
+        _check(oracle, g, B, C, f"segments k={k} shift={shift}")
+        again, _ = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(shift))
+        assert np.array_equal(C, again), "bit-reproducible"
+    # B and C inside larger allocations: nothing may be read past the last row of B (NaN there would
+    # show) nor written past the last row of C
+    rp, ci, v = _to_dev(gpu, g.rowptr, g.col, g.val)
+    pad = 64
+    Bbig = torch.full((g.cols * k + pad,), float("nan"), device=gpu)
+    Bbig[:g.cols * k] = torch.from_numpy(B).to(gpu).reshape(-1)
+    Cbig = torch.full((g.rows * k + pad,), 12345.0, device=gpu)
+    Bd, Cd = Bbig[:g.cols * k].view(g.cols, k), Cbig[:g.rows * k].view(g.rows, k)
+    for flags in (capi.PLAN_DEFAULT, capi.PLAN_FORCE_SEGMENTS):
+        Cd.fill_(float("nan"))
+        plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
+        capi.csr_spmm(plan, rp, ci, v, Bd, Cd)
+        torch.cuda.synchronize()
+        plan.destroy()
+        _check(oracle, g, B, Cd.cpu().numpy(), f"guarded k={k} flags={flags}")
+        assert bool((Cbig[g.rows * k:] == 12345.0).all()), f"k={k}: wrote past the last row of C"
+    Cn = torch.full((g.rows, k), float("nan"), device=gpu)
+    capi.csr_spmm_noplan(g.rows, g.cols, rp, ci, v, Bd, Cn)
+    _check(oracle, g, B, Cn.cpu().numpy(), f"noplan k={k}")
 
 
 @pytest.mark.parametrize("k", [4, 8, 12, 16, 20, 24, 48, 96, 100, 160, 200, 256, 384])
@@ -219,7 +250,7 @@ def test_multiple_of_four_k(pkg, oracle, gpu, k):
     _check(oracle, g, B, Cn.cpu().numpy(), f"noplan k={k}")
 
 
-@pytest.mark.parametrize("k", [16, 96])
+@pytest.mark.parametrize("k", [16, 41, 96])
 def test_multiple_of_four_k_large_graph(pkg, oracle, gpu, k):
     """Beyond 2^21 nonzeros the plan picks segments for these K by itself."""
     capi = pkg.capi
@@ -289,7 +320,7 @@ def test_fill(pkg, gpu):
     assert torch.all(x == -2.5).item()
 
 
-@pytest.mark.parametrize("k", [32, 64, 128, 24, 16, 96, 200, 7])
+@pytest.mark.parametrize("k", [32, 64, 128, 24, 16, 96, 200, 7, 41, 173])
 def test_coo_accumulate(pkg, oracle, gpu, k):
     """The LBSpMM contract: C += A B, padded zero entries, rows in permuted order."""
     import torch

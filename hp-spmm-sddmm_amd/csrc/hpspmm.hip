@@ -64,10 +64,19 @@ inline void mark_launch(hipStream_t st, const char* name) {
 }
 
 inline bool fast_k(int64_t k) { return k == 32 || k == 64 || k == 128; }
-// Width of the column tiles by which a tuned layout can serve row length k (0: none, or k is tuned itself).
+// Width of the column tiles by which a tuned layout can serve row length k (0: none, or k is tuned
+// itself): any multiple of 4 from 16 up - the last tile may be narrower than the layout's width, the
+// lanes beyond it idle.  The width that costs least, a tile of 32 / 64 / 128 columns weighed as the
+// tuned sizes relate on the benchmark graphs (1 : 1.56 : 2.75): 40 -> one tile of 64, 96 -> one of
+// 128, 160 -> 64 + 64 + 32 of 64, 200 -> 128 + 72 of 128, 256 -> two of 128.
 inline int64_t tile_width(int64_t k) {
-  if (fast_k(k) || k <= 0) return 0;
-  return k % 128 == 0 ? 128 : k % 64 == 0 ? 64 : k % 32 == 0 ? 32 : 0;
+  if (fast_k(k) || k < 16 || k % 4 != 0) return 0;
+  const int64_t width[3] = {128, 64, 32};
+  const double cost[3] = {2.75, 1.56, 1.0};
+  int best = 0;
+  for (int i = 1; i < 3; ++i)
+    if ((double)((k + width[i] - 1) / width[i]) * cost[i] < (double)((k + width[best] - 1) / width[best]) * cost[best]) best = i;
+  return width[best];
 }
 // Every row length that is not a tuned size goes to the run-time-K sub-wave kernels.
 // Not a multiple of 4: rows of B and C start at any multiple of 4 bytes, the last lane of a row owns 1 to 3 columns.
@@ -107,9 +116,10 @@ int grid_for(int64_t items, int64_t cap = 1 << 20) {
 
 struct hpspmm_plan {
   int64_t rows = 0, cols = 0, nnz = 0, k = 0;
-  // A row length that is a multiple of a tuned one (256 = 2 x 128, 96 = 3 x 32) can be served by a
-  // layout built for the tuned length, one column tile after the other: k is then the tile width,
-  // k_full the row length of B and C, tiles = k_full / k.  Otherwise k_full = k, tiles = 1.
+  // A row length that is a multiple of 4 but not a tuned one (256 = 2 x 128, 40 = one tile of 64 with
+  // 10 of its 16 lanes) can be served by a layout built for a tuned length, one column tile after
+  // the other: k is then the tile width, k_full the row length of B and C, tiles = ceil(k_full / k).
+  // Otherwise k_full = k, tiles = 1.
   int64_t k_full = 0;
   int tiles = 1;
   int strategy = 0;
@@ -1890,9 +1900,9 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   if (nnz > 0 && !d_col) return fail(HPSPMM_ERR_INVALID_ARG, "d_col is NULL with nnz > 0");
   hipStream_t st = (hipStream_t)stream;
 
-  // A multiple of a tuned row length: the layouts built for the tuned length (sweep, routed,
-  // ordered) serve it tile by tile, if the matrix gets one of them; if not, the plan is built for
-  // the full length as for any other multiple of 4.
+  // A multiple of 4 that is not a tuned row length: the layouts built for a tuned length (sweep,
+  // routed, ordered) serve it tile by tile, if the matrix gets one of them; if not, the plan is
+  // built for the full length as for any other row length.
   // (HPSPMM_NO_COLUMN_TILES in the environment switches this off, for comparisons)
   if (k_full == 0 && tile_width(k) > 0 && nnz > 0 && !std::getenv("HPSPMM_NO_COLUMN_TILES") &&
       (nnz >= kTiledMinNnz || d_order ||
@@ -1955,7 +1965,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   p->nnz = nnz;
   p->k = k;
   p->k_full = k_full ? k_full : k;
-  p->tiles = (int)(p->k_full / k);
+  p->tiles = (int)ceil_div(p->k_full, k);
   p->max_row_nnz = stats[0];
   p->empty_rows = stats[1];
   p->src_rowptr = d_rowptr;
@@ -2281,14 +2291,16 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
   int rc;
   // another value array overwrites the plan's copy of the bound one
   if (plan->bound_val && plan->bound_val != d_val) plan->bound_val = nullptr;
-  if (plan->tiles > 1) {
+  if (plan->k_full != plan->k) {
     // one column tile after the other through the layout built for the tile width; the operands of
     // tile t are columns [t * k, (t + 1) * k) of B and C, whose rows are k_full floats apart
-    const uint32_t ld = (uint32_t)plan->k_full;
     rc = HPSPMM_OK;
     for (int t = 0; t < plan->tiles && rc == HPSPMM_OK; ++t) {
       const float* Bt = d_B + (int64_t)t * plan->k;
       float* Ct = d_C + (int64_t)t * plan->k;
+      // the row length, and above it the columns of the tile that exist when the last one is narrower
+      const int64_t left = plan->k_full - (int64_t)t * plan->k;
+      const uint32_t ld = (uint32_t)plan->k_full | (left < plan->k ? (uint32_t)left << 24 : 0u);
       if (plan->strategy == HPSPMM_STRATEGY_ORDERED) {
         switch (plan->k) {
           case 32: rc = launch_ordered<32, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;

@@ -432,7 +432,8 @@ __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
   for (int i = tid; i < cap * G; i += kBlock) {
     const int slot = i / G;
     const int32_t c = wcols[blk * cap + slot];
-    if (c >= 0) *reinterpret_cast<float4*>(s_b + slot * K + 4 * (i % G)) = load_b_ld(B, c, i % G, ld);
+    if (c >= 0 && lane_in_tile<K, kLd>(ld_arg, i % G))
+      *reinterpret_cast<float4*>(s_b + slot * K + 4 * (i % G)) = load_b_ld(B, c, i % G, ld);
   }
   __syncthreads();
 
@@ -442,6 +443,7 @@ __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
   const int64_t e = (s + ((int64_t)1 << shift)) < nnz ? (s + ((int64_t)1 << shift)) : nnz;
   const int sbase = ((tid >> 6) * P + lane / G) * kTileStride;
 
+  const bool in_tile = lane_in_tile<K, kLd>(ld_arg, l);
   int32_t cur = orow[s];
   bool head_pending = (int64_t)start[cur] < s;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -450,13 +452,16 @@ __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
     float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
                               : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : C + (uint64_t)(uint32_t)cur * ld);
     head_pending = false;
-    store_result(dst + 4 * l, acc);
+    if (in_tile) store_result(dst + 4 * l, acc);  // (a lane beyond the tile holds zeros: nothing of it is ever read)
   };
   auto flush = [&]() { flush_to(false); };
   // One flat load per gather, its address selected between the LDS copy and memory: a branch
   // per gather would make every load of a batch wait for the one before it.
   const float* lds_b = s_b;
   auto loadb = [&](int32_t c) {
+    if constexpr (kLd) {
+      if (!in_tile) return make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     const float* row = c < 0 ? lds_b + (uint32_t)(~c) * (uint32_t)K : B + (uint64_t)(uint32_t)c * (uint64_t)ld;
     return *reinterpret_cast<const float4*>(row + 4 * l);
   };

@@ -522,7 +522,8 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
     if (s >= n_bhot) return;
     const int32_t c = src[s];
     if (c < 0) return;
-    *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) = load_b_ld(B, c, l, row_length<K, kLd>(ld_arg));
+    *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) =
+        lane_in_tile<K, kLd>(ld_arg, l) ? load_b_ld(B, c, l, row_length<K, kLd>(ld_arg)) : make_float4(0.f, 0.f, 0.f, 0.f);
     return;
   }
   const int64_t chunk = (int64_t)blockIdx.x - gather_blocks;
@@ -614,6 +615,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
+  const bool in_tile = lane_in_tile<K, kLd>(ld_arg, l);
   const int shift = lay.shift;
   const int64_t g = (lay.cls_begin[x] >> shift) + (i * kWavesPerBlock + (tid >> 6)) * P + lane / G;
   const int64_t s = g << shift;
@@ -635,10 +637,13 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
     float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
                               : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : out + (uint64_t)(uint32_t)cur * ostride);
     head_pending = false;
-    store_result(dst + 4 * l, acc);
+    if (in_tile) store_result(dst + 4 * l, acc);  // (a lane beyond the tile holds zeros: nothing of it is ever read)
   };
   auto flush = [&]() { flush_to(false); };
   auto loadb = [&](int32_t c) {
+    if constexpr (kLd) {
+      if (!in_tile) return make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     if constexpr (kHub) {
       return load_b_hub_ld<K, true>(B, Bhot, c, l, ld);
     } else {
@@ -731,6 +736,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
+  const bool in_tile = lane_in_tile<K, kLd>(ld_arg, l);
   const int shift = lay.shift;
   const int nhub = lay.nhub;
   const float* cbase = carry + 4 * l;
@@ -760,7 +766,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
   if ((int64_t)blockIdx.x >= routed_blocks + cross_blocks) {
     const int64_t idx = ((int64_t)blockIdx.x - routed_blocks - cross_blocks) * (kWavesPerBlock * P) + sub;
     if (idx >= n_zero) return;
-    *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * ld + 4 * l) = acc;
+    if (in_tile) *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * ld + 4 * l) = acc;
     return;
   }
   if ((int64_t)blockIdx.x >= routed_blocks) {
@@ -771,7 +777,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
     const int64_t gb = (coldptr[row + 1] - 1) >> shift;
     add(*reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * ga + 1) * K));
     add_heads(ga + 1, gb);
-    *reinterpret_cast<float4*>(C + (uint64_t)row * ld + 4 * l) = acc;
+    if (in_tile) *reinterpret_cast<float4*>(C + (uint64_t)row * ld + 4 * l) = acc;
     return;
   }
   const int64_t idx = (int64_t)blockIdx.x * (kWavesPerBlock * P) + sub;
@@ -830,7 +836,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
       if (gb > ga + 1) add_heads(ga + 2, gb);
     }
   }
-  *reinterpret_cast<float4*>(C + (uint64_t)row * ld + 4 * l) = acc;
+  if (in_tile) *reinterpret_cast<float4*>(C + (uint64_t)row * ld + 4 * l) = acc;
 }
 
 }  // namespace hpspmm

@@ -74,9 +74,18 @@ __device__ __forceinline__ float4 load_b(const float* __restrict__ B, int32_t c,
 // The same with the row length of B given at run time: the operands of a tuned kernel may be K
 // columns of a wider B and C (one column tile of a product whose row length is a multiple of K).
 // kLd = false compiles to the fixed form.
+// ld_arg carries two things: the row length in its low 24 bits and, in the bits above, how many of
+// the tile's K columns exist (0 = all of them): the last tile of a row length that is not a
+// multiple of K is narrower, and the lanes whose columns lie beyond it must neither read B nor write C.
 template <int K, bool kLd>
 __device__ __forceinline__ uint32_t row_length(uint32_t ld_arg) {
-  return kLd ? ld_arg : (uint32_t)K;
+  return kLd ? (ld_arg & 0xFFFFFFu) : (uint32_t)K;
+}
+template <int K, bool kLd>
+__device__ __forceinline__ bool lane_in_tile(uint32_t ld_arg, int l) {
+  if constexpr (!kLd) return true;
+  const uint32_t cols = ld_arg >> 24;
+  return cols == 0 || (uint32_t)(4 * l) < cols;
 }
 __device__ __forceinline__ float4 load_b_ld(const float* __restrict__ B, int32_t c, int l, uint32_t ld) {
   return *reinterpret_cast<const float4*>(B + (uint64_t)(uint32_t)c * (uint64_t)ld + (uint32_t)(4 * l));
@@ -474,6 +483,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
+  const bool in_tile = lane_in_tile<K, kLd>(ld_arg, l);
   const int sub = lane / G;
   const int64_t r0 = ((int64_t)blockIdx.x * kWavesPerBlock + (tid >> 6)) * rpw;
   if (r0 >= rows) return;
@@ -520,13 +530,13 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
     const int32_t hb_i = __shfl(hb, i);
     float4* out = reinterpret_cast<float4*>(C + (uint64_t)(r0 + i) * ld + 4 * l);
     if ((m_empty >> i) & 1ull) {
-      *out = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (in_tile) *out = make_float4(0.f, 0.f, 0.f, 0.f);
     } else if ((m_split >> i) & 1ull) {
       const int64_t ga = (int64_t)lb_i >> shift;
       const int64_t gb = (int64_t)(hb_i - 1) >> shift;
       float4 acc = *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * ga + 1) * K + 4 * l);
       add_heads(acc, ga + 1, gb, 1);
-      *out = acc;
+      if (in_tile) *out = acc;
     }
   }
   // Long chains, one row at a time, all P sub-waves together: sub-wave s adds the heads ga+1+s,
@@ -551,7 +561,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
       t.w = __shfl(part.w, s * G + l);
       add(acc, t);
     }
-    if (sub == 0) *reinterpret_cast<float4*>(C + (uint64_t)(r0 + i) * ld + 4 * l) = acc;
+    if (sub == 0 && in_tile) *reinterpret_cast<float4*>(C + (uint64_t)(r0 + i) * ld + 4 * l) = acc;
   }
 }
 

@@ -464,7 +464,11 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
 
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   // the plan checks that B is below 4 GB: a 32-bit byte offset
+  const bool in_tile = lane_in_tile<K, kLd>(ld_arg, l);
   auto loadb = [&](int32_t w) {
+    if constexpr (kLd) {
+      if (!in_tile) return make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     const uint32_t off = (uint32_t)(w & kSweepColMask) * (ld * 4u) + (uint32_t)(16 * l);
     const char* base =
         (w & kSweepPad) ? reinterpret_cast<const char*>(zrow) + 16 * l : reinterpret_cast<const char*>(B) + off;
@@ -589,7 +593,7 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
     if (dest == kSweepUnused) continue;
     const float4 sum = *reinterpret_cast<const float4*>(acc_wave + slot * K + 4 * l);
     float* out = dest >= 0 ? C + (uint64_t)(uint32_t)dest * ld : partial + (uint64_t)(uint32_t)~dest * K;
-    store_result(out + 4 * l, sum);
+    if (in_tile) store_result(out + 4 * l, sum);  // (a lane beyond the tile holds zeros: nothing of it is ever read)
   }
 }
 
@@ -610,7 +614,8 @@ __global__ __launch_bounds__(kBlock) void spmm_sweep_final_kernel(
   if ((int64_t)blockIdx.x >= split_blocks) {
     const int64_t idx = ((int64_t)blockIdx.x - split_blocks) * (kWavesPerBlock * P) + sub;
     if (idx >= n_zero) return;
-    *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * ld + 4 * l) = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (lane_in_tile<K, kLd>(ld_arg, l))
+      *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * ld + 4 * l) = make_float4(0.f, 0.f, 0.f, 0.f);
     return;
   }
   const int64_t idx = (int64_t)blockIdx.x * (kWavesPerBlock * P) + sub;
@@ -639,7 +644,7 @@ __global__ __launch_bounds__(kBlock) void spmm_sweep_final_kernel(
     acc.z += t.z;
     acc.w += t.w;
   }
-  *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)row * ld + 4 * l) = acc;
+  if (lane_in_tile<K, kLd>(ld_arg, l)) *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)row * ld + 4 * l) = acc;
 }
 
 }  // namespace hpspmm

@@ -108,7 +108,7 @@ typedef struct hpspmm_plan_info {
   int64_t empty_rows;
   int64_t workspace_bytes; /* device memory owned by the plan */
   int32_t launches_per_spmm;
-  int32_t column_tiles;    /* 1, or the number of column tiles a multiple of a tuned row length is served in */
+  int32_t column_tiles;    /* column tiles a row length other than 32 / 64 / 128 is served in by a tuned layout (else 1) */
   int64_t hub_rows;        /* rows of B kept in the hub cache (0 = none) */
   int64_t lds_served_nnz;  /* ordered strategy: nonzeros whose row of B comes from a workgroup's LDS copy */
   int64_t row_tiles;       /* rows strategy: 64-entry tiles of the plan's row-tile layout (0: the CSR arrays are walked) */
@@ -136,16 +136,19 @@ const char *hpspmm_last_error(void);
  * nonzeros ("routed"); or segments over a clustered row order with the reused
  * rows of B held in LDS when the matrix is a graph with communities
  * ("ordered").
- * k = 32, 64 and 128 are the tuned row lengths.  A multiple of one of them
- * (96, 160, 192, 256, 384, 512 ...) is served by the sweep, routed and ordered
- * layouts one column tile of 128, 64 or 32 columns after the other (the
- * reference tiles the columns the same way, spmm/mm/spmm_kernel.cu:412-420:
- * grid.y = ceil(k / 64)), when the matrix gets one of those layouts (at least
- * 2^22 nonzeros, or a forcing flag); launches_per_spmm counts every tile's.
- * Any other k runs whole rows or segments with sub-waves of ceil(k / 4) lanes
- * rounded up to a power of two; when k is not a multiple of 4 (41 classes, 47,
- * 173 ...) the rows of B and C are read and written at their 4-byte alignment
- * and the lane that owns a row's last columns touches only those that exist.
+ * k = 32, 64 and 128 are the tuned row lengths.  Any other multiple of 4 from
+ * 16 up (16, 40, 96, 160, 256, 512 ...) is served by the sweep, routed and
+ * ordered layouts one column tile of 128, 64 or 32 columns after the other
+ * (the reference tiles the columns the same way, spmm/mm/spmm_kernel.cu:
+ * 412-420: grid.y = ceil(k / 64)); a last tile narrower than the layout leaves
+ * its surplus lanes idle.  That is done when the matrix gets one of those
+ * layouts (at least 2^22 nonzeros, or a forcing flag); launches_per_spmm
+ * counts every tile's, column_tiles the tiles.
+ * Otherwise, and for every other k, whole rows or segments run with sub-waves
+ * of ceil(k / 4) lanes rounded up to a power of two; when k is not a multiple
+ * of 4 (41 classes, 47, 173 ...) the rows of B and C are read and written at
+ * their 4-byte alignment and the lane that owns a row's last columns touches
+ * only those that exist.
  * Replaces the host-side preprocessing the reference does before timing:
  * CSR->COO expansion (spmm/mm/spmm_common.cpp:185-235), the row re-ordering
  * (:237-296) and the choice of nnz_per_warp (spmm/mm/spmm_kernel.cu:749-751).
@@ -174,8 +177,8 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d
  * result is that of hpspmm_plan_create up to summation order.  The role of the
  * row permutation that the reference reads from a .cugraph_reorder file for
  * HP-SpMM (spmm/mm/spmm_common.cpp:237-296: nonzeros emitted in that row
- * order, row indices kept).  k must be a multiple of 32 for the order to be
- * used.
+ * order, row indices kept).  k must be a multiple of 4, and at least 16, for
+ * the order to be used.
  */
 int hpspmm_plan_create_ordered(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
                                const int32_t *d_col, int64_t k, uint32_t flags,

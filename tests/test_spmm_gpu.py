@@ -252,13 +252,15 @@ def test_multiple_of_four_k(pkg, oracle, gpu, k):
 
 @pytest.mark.parametrize("k", [16, 41, 96])
 def test_multiple_of_four_k_large_graph(pkg, oracle, gpu, k):
-    """Beyond 2^21 nonzeros the plan picks segments for these K by itself."""
+    """Beyond 2^21 nonzeros the plan picks segments for these K by itself - or, for a multiple of 4 on
+    a matrix of 2^22 nonzeros and more, one of the tuned layouts in column tiles."""
     capi = pkg.capi
     g = pkg.graphs.make_graph("c2_social", 0.05)
     assert g.nnz > 1 << 21
     B = pkg.graphs.dense_normal(g.cols, k, 79)
     C, info = _run(pkg, gpu, g, B)
-    assert info["strategy"] == capi.STRATEGY_SEGMENTS, info
+    tiled = (capi.STRATEGY_SWEEP, capi.STRATEGY_ROUTED, capi.STRATEGY_ORDERED)
+    assert info["strategy"] == capi.STRATEGY_SEGMENTS or (k % 4 == 0 and info["strategy"] in tiled), info
     _check(oracle, g, B, C, f"auto segments k={k}")
 
 
@@ -563,7 +565,7 @@ def test_random_matrices_all_strategies(pkg, oracle, gpu, seed):
         assert not C[np.diff(rowptr) == 0].any()
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(10))
 def test_random_matrices_column_tiles(pkg, oracle, gpu, seed):
     """The same at row lengths that are multiples of a tuned one: the forced sweep, routed and ordered
     plans run in column tiles, the others through the kernels for any multiple of 4."""
@@ -571,7 +573,7 @@ def test_random_matrices_column_tiles(pkg, oracle, gpu, seed):
     rng = np.random.default_rng(2000 + seed)
     rows = int(rng.integers(1, 3000))
     cols = int(rng.integers(1, 3000))
-    k = int(rng.choice([96, 160, 192, 256, 384]))
+    k = int(rng.choice([16, 20, 40, 96, 100, 160, 200, 256, 384]))
     rowptr, col, val = _random_csr(rng, rows, cols, mean_deg=float(rng.uniform(0.5, 40)),
                                    skew=float(rng.uniform(0.8, 3.0)), empty_frac=float(rng.uniform(0, 0.6)),
                                    sorted_unique=(seed % 3 != 2))
@@ -584,7 +586,7 @@ def test_random_matrices_column_tiles(pkg, oracle, gpu, seed):
     tiled = 0
     for name, flags in _strategies(pkg.capi):
         C, info = _run(pkg, gpu, g, B, flags)
-        tiled += info["column_tiles"] > 1
+        tiled += info["strategy"] in (pkg.capi.STRATEGY_SWEEP, pkg.capi.STRATEGY_ROUTED, pkg.capi.STRATEGY_ORDERED)
         bad = np.abs(C - want) > TOL * S
         assert not bad.any(), f"seed {seed} rows={rows} cols={cols} k={k} {name}: {int(bad.sum())} elements off"
         assert not C[np.diff(rowptr) == 0].any()
@@ -1007,13 +1009,16 @@ def test_sweep_is_not_chosen_for_a_banded_matrix(pkg, oracle, gpu):
     _check(oracle, g, B, C, "banded, forced sweep")
 
 
-@pytest.mark.parametrize("k,tile", [(96, 32), (160, 32), (192, 64), (256, 128), (384, 128)])
-def test_column_tiles(pkg, oracle, gpu, k, tile):
-    """A row length that is a multiple of a tuned one goes through the tuned layouts (sweep, routed,
-    ordered) one column tile after the other: the plan reports that strategy, the full row length and
-    one set of launches per tile; the product meets the oracle's bar; tile t of C has the bits of the
-    product with columns [t * tile, (t + 1) * tile) of B alone (same layout, same order of additions);
-    bound values give the same bits.  Without a tuned layout the plan is the one for any multiple of 4."""
+@pytest.mark.parametrize("k,tile,ntiles", [(16, 32, 1), (40, 64, 1), (96, 128, 1), (160, 64, 3), (192, 64, 3),
+                                           (200, 128, 2), (256, 128, 2), (384, 128, 3)])
+def test_column_tiles(pkg, oracle, gpu, k, tile, ntiles):
+    """A row length that is a multiple of 4 but not a tuned one goes through the tuned layouts (sweep,
+    routed, ordered) one column tile after the other, the last tile narrower than the layout when the
+    width does not divide the row length (its surplus lanes idle): the plan reports that strategy,
+    the full row length and one set of launches per tile; the product meets the oracle's bar; a full
+    tile t of C has the bits of the product with columns [t * tile, (t + 1) * tile) of B alone (same
+    layout, same order of additions); bound values give the same bits.  Without a tuned layout the
+    plan is the one for any row length."""
     import torch
     capi = pkg.capi
     cases = [("c2_social", 0.02, "sweep", capi.PLAN_FORCE_SWEEP, capi.STRATEGY_SWEEP),
@@ -1027,12 +1032,12 @@ def test_column_tiles(pkg, oracle, gpu, k, tile):
         B = pkg.graphs.make_dense(name, g.cols, k)
         C, info = _run(pkg, gpu, g, B, flags)
         what = f"{name} k={k} {label}"
-        assert info["strategy"] == strategy and info["k"] == k and info["column_tiles"] == k // tile, (what, info)
+        assert info["strategy"] == strategy and info["k"] == k and info["column_tiles"] == ntiles, (what, info)
         _check(oracle, g, B, C, what)
-        for t in sorted({0, k // tile - 1}):
+        for t in sorted({0, k // tile - 1} - {-1}):  # full tiles only
             Bt = np.ascontiguousarray(B[:, t * tile:(t + 1) * tile])
             Ct, info_t = _run(pkg, gpu, g, Bt, flags)
-            assert info_t["strategy"] == strategy and info_t["launches_per_spmm"] * (k // tile) == info["launches_per_spmm"]
+            assert info_t["strategy"] == strategy and info_t["launches_per_spmm"] * ntiles == info["launches_per_spmm"]
             assert np.array_equal(C[:, t * tile:(t + 1) * tile], Ct), f"{what}: tile {t} differs from the product of that tile alone"
         rp, ci, v, Bd = _to_dev(gpu, g.rowptr, g.col, g.val, B)
         plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)

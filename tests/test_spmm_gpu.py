@@ -573,7 +573,7 @@ def test_random_matrices_column_tiles(pkg, oracle, gpu, seed):
     rng = np.random.default_rng(2000 + seed)
     rows = int(rng.integers(1, 3000))
     cols = int(rng.integers(1, 3000))
-    k = int(rng.choice([16, 20, 40, 96, 100, 160, 200, 256, 384]))
+    k = int(rng.choice([16, 20, 40, 41, 47, 96, 100, 160, 173, 200, 256, 259, 384]))
     rowptr, col, val = _random_csr(rng, rows, cols, mean_deg=float(rng.uniform(0.5, 40)),
                                    skew=float(rng.uniform(0.8, 3.0)), empty_frac=float(rng.uniform(0, 0.6)),
                                    sorted_unique=(seed % 3 != 2))
@@ -590,7 +590,7 @@ def test_random_matrices_column_tiles(pkg, oracle, gpu, seed):
         bad = np.abs(C - want) > TOL * S
         assert not bad.any(), f"seed {seed} rows={rows} cols={cols} k={k} {name}: {int(bad.sum())} elements off"
         assert not C[np.diff(rowptr) == 0].any()
-    assert tiled >= 4 or col.size == 0, f"seed {seed}: only {tiled} plans ran in column tiles"
+    assert tiled >= 4 or col.size == 0 or k % 4 != 0, f"seed {seed}: only {tiled} plans ran in column tiles"
 
 
 def test_non_finite_values_stay_in_their_rows(pkg, oracle, gpu):
@@ -1014,7 +1014,8 @@ def test_sweep_is_not_chosen_for_a_banded_matrix(pkg, oracle, gpu):
 def test_column_tiles(pkg, oracle, gpu, k, tile, ntiles):
     """A row length that is a multiple of 4 but not a tuned one goes through the tuned layouts (sweep,
     routed, ordered) one column tile after the other, the last tile narrower than the layout when the
-    width does not divide the row length (its surplus lanes idle): the plan reports that strategy,
+    width does not divide the row length (its surplus lanes idle; B and C sit inside larger
+    allocations here, NaN behind B, a sentinel behind C): the plan reports that strategy,
     the full row length and one set of launches per tile; the product meets the oracle's bar; a full
     tile t of C has the bits of the product with columns [t * tile, (t + 1) * tile) of B alone (same
     layout, same order of additions); bound values give the same bits.  Without a tuned layout the
@@ -1039,13 +1040,19 @@ def test_column_tiles(pkg, oracle, gpu, k, tile, ntiles):
             Ct, info_t = _run(pkg, gpu, g, Bt, flags)
             assert info_t["strategy"] == strategy and info_t["launches_per_spmm"] * ntiles == info["launches_per_spmm"]
             assert np.array_equal(C[:, t * tile:(t + 1) * tile], Ct), f"{what}: tile {t} differs from the product of that tile alone"
-        rp, ci, v, Bd = _to_dev(gpu, g.rowptr, g.col, g.val, B)
+        rp, ci, v = _to_dev(gpu, g.rowptr, g.col, g.val)
+        pad = 64
+        Bbig = torch.full((g.cols * k + pad,), float("nan"), device=gpu)
+        Bbig[:g.cols * k] = torch.from_numpy(B).to(gpu).reshape(-1)
+        Cbig = torch.full((g.rows * k + pad,), 12345.0, device=gpu)
+        Bd, Cb = Bbig[:g.cols * k].view(g.cols, k), Cbig[:g.rows * k].view(g.rows, k)
+        Cb.fill_(float("nan"))
         plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
-        Cb = torch.full((g.rows, k), float("nan"), device=gpu)
         plan.bind_values(v)
         capi.csr_spmm(plan, rp, ci, v, Bd, Cb)
         torch.cuda.synchronize()
         assert np.array_equal(Cb.cpu().numpy(), C), f"{what}: bound values, different bits"
+        assert bool((Cbig[g.rows * k:] == 12345.0).all()), f"{what}: wrote past the last row of C"
         plan.destroy()
     # a caller's row order
     g = pkg.graphs.make_graph("c3_copurchase", 0.01)

@@ -458,12 +458,12 @@ __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
   // One flat load per gather, its address selected between the LDS copy and memory: a branch
   // per gather would make every load of a batch wait for the one before it.
   const float* lds_b = s_b;
+  // a lane beyond the tile gathers what lane 0 gathers (a valid address, no branch in the loop); its
+  // sums are never stored
+  const int lg = in_tile ? l : 0;
   auto loadb = [&](int32_t c) {
-    if constexpr (kLd) {
-      if (!in_tile) return make_float4(0.f, 0.f, 0.f, 0.f);
-    }
     const float* row = c < 0 ? lds_b + (uint32_t)(~c) * (uint32_t)K : B + (uint64_t)(uint32_t)c * (uint64_t)ld;
-    return *reinterpret_cast<const float4*>(row + 4 * l);
+    return *reinterpret_cast<const float4*>(row + 4 * lg);
   };
 
   // Two-deep prefetch: the original indices of tile t+2 and, through the indices

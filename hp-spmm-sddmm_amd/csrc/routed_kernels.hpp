@@ -640,14 +640,14 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
     if (in_tile) store_result(dst + 4 * l, acc);  // (a lane beyond the tile holds zeros: nothing of it is ever read)
   };
   auto flush = [&]() { flush_to(false); };
+  // a lane beyond the tile gathers what lane 0 gathers (a valid address, no branch in the loop); its
+  // sums are never stored
+  const int lg = in_tile ? l : 0;
   auto loadb = [&](int32_t c) {
-    if constexpr (kLd) {
-      if (!in_tile) return make_float4(0.f, 0.f, 0.f, 0.f);
-    }
     if constexpr (kHub) {
-      return load_b_hub_ld<K, true>(B, Bhot, c, l, ld);
+      return load_b_hub_ld<K, true>(B, Bhot, c, lg, ld);
     } else {
-      const uint32_t off = (uint32_t)c * (ld * 4u) + (uint32_t)(16 * l);
+      const uint32_t off = (uint32_t)c * (ld * 4u) + (uint32_t)(16 * lg);
       return *reinterpret_cast<const float4*>(reinterpret_cast<const char*>(B) + off);
     }
   };

@@ -465,13 +465,13 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   // the plan checks that B is below 4 GB: a 32-bit byte offset
   const bool in_tile = lane_in_tile<K, kLd>(ld_arg, l);
+  // a lane beyond the tile gathers what lane 0 gathers (a valid address, no branch in the loop); its
+  // sums are never stored to C
+  const int lg = in_tile ? l : 0;
   auto loadb = [&](int32_t w) {
-    if constexpr (kLd) {
-      if (!in_tile) return make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-    const uint32_t off = (uint32_t)(w & kSweepColMask) * (ld * 4u) + (uint32_t)(16 * l);
+    const uint32_t off = (uint32_t)(w & kSweepColMask) * (ld * 4u) + (uint32_t)(16 * lg);
     const char* base =
-        (w & kSweepPad) ? reinterpret_cast<const char*>(zrow) + 16 * l : reinterpret_cast<const char*>(B) + off;
+        (w & kSweepPad) ? reinterpret_cast<const char*>(zrow) + 16 * lg : reinterpret_cast<const char*>(B) + off;
     return *reinterpret_cast<const float4*>(base);
   };
 

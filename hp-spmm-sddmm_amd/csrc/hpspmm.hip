@@ -122,6 +122,11 @@ struct hpspmm_plan {
   // Otherwise k_full = k, tiles = 1.
   int64_t k_full = 0;
   int tiles = 1;
+  // The caller's row length when it is not a multiple of 4 and a tuned layout serves it all the same:
+  // k_full is then that length rounded up to 4, B is read through a copy with rows padded to k_full
+  // (d_bpad, refreshed at the start of every SpMM), C is written in place.  Otherwise k_user = k_full.
+  int64_t k_user = 0;
+  float* d_bpad = nullptr;
   int strategy = 0;
   int shift = 0;  // log2(segment length)
   int64_t nseg = 0;
@@ -1900,18 +1905,35 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   if (nnz > 0 && !d_col) return fail(HPSPMM_ERR_INVALID_ARG, "d_col is NULL with nnz > 0");
   hipStream_t st = (hipStream_t)stream;
 
-  // A multiple of 4 that is not a tuned row length: the layouts built for a tuned length (sweep,
-  // routed, ordered) serve it tile by tile, if the matrix gets one of them; if not, the plan is
-  // built for the full length as for any other row length.
+  // Not a tuned row length: the layouts built for a tuned length (sweep, routed, ordered) serve it
+  // tile by tile, if the matrix gets one of them; if not, the plan is built for the full length as
+  // for any other row length.  A row length that is not a multiple of 4 (from 16 up) is rounded up
+  // to one for that: 16-byte gathers at 4-byte alignment cost about twice, so B is read through a
+  // padded copy made at the start of every SpMM (0.02 ms for 233k rows of 41 floats; C is written
+  // in place, its stores are few).
   // (HPSPMM_NO_COLUMN_TILES in the environment switches this off, for comparisons)
-  if (k_full == 0 && tile_width(k) > 0 && nnz > 0 && !std::getenv("HPSPMM_NO_COLUMN_TILES") &&
+  const int64_t kp = (k + 3) & ~(int64_t)3;
+  const int64_t kw = fast_k(kp) ? kp : tile_width(kp);
+  if (k_full == 0 && !fast_k(k) && kw > 0 && (k % 4 == 0 || k >= 16) && nnz > 0 &&
+      !std::getenv("HPSPMM_NO_COLUMN_TILES") &&
       (nnz >= kTiledMinNnz || d_order ||
        (flags & (HPSPMM_PLAN_FORCE_ROUTED | HPSPMM_PLAN_FORCE_SWEEP | HPSPMM_PLAN_CLUSTER)))) {
     hpspmm_plan* tiled = nullptr;
-    const int rc = plan_create_impl(rows, cols, nnz, d_rowptr, d_col, tile_width(k), flags, d_order, stream, &tiled, k);
+    int rc = plan_create_impl(rows, cols, nnz, d_rowptr, d_col, kw, flags, d_order, stream, &tiled, kp);
     if (rc == HPSPMM_OK && tiled &&
         (tiled->strategy == HPSPMM_STRATEGY_SWEEP || tiled->strategy == HPSPMM_STRATEGY_ROUTED ||
          tiled->strategy == HPSPMM_STRATEGY_ORDERED)) {
+      if (kp != k) {
+        const size_t pad_bytes = (size_t)std::max<int64_t>(cols, 1) * (size_t)kp * sizeof(float);
+        if (hipMalloc(&tiled->d_bpad, pad_bytes) != hipSuccess) {
+          (void)hipGetLastError();
+          tiled->d_bpad = nullptr;
+          hpspmm_plan_destroy(tiled);
+          return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the padded copy of B failed", pad_bytes);
+        }
+        tiled->workspace_bytes += (int64_t)pad_bytes;
+        tiled->k_user = k;
+      }
       *plan_out = tiled;
       return HPSPMM_OK;
     }
@@ -1966,6 +1988,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   p->k = k;
   p->k_full = k_full ? k_full : k;
   p->tiles = (int)ceil_div(p->k_full, k);
+  p->k_user = p->k_full;
   p->max_row_nnz = stats[0];
   p->empty_rows = stats[1];
   p->src_rowptr = d_rowptr;
@@ -2182,7 +2205,7 @@ int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
   out->rows = plan->rows;
   out->cols = plan->cols;
   out->nnz = plan->nnz;
-  out->k = plan->k_full;
+  out->k = plan->k_user;
   out->strategy = plan->strategy;
   const bool segmented = plan->strategy == HPSPMM_STRATEGY_SEGMENTS || plan->strategy == HPSPMM_STRATEGY_ROUTED ||
                          plan->strategy == HPSPMM_STRATEGY_ORDERED;
@@ -2197,6 +2220,7 @@ int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* out) {
                            : plan->strategy == HPSPMM_STRATEGY_SEGMENTS ? (plan->n_hub > 0 ? 3 : 2)
                                                                         : 1;
   out->launches_per_spmm *= plan->tiles;  // one pass per column tile
+  if (plan->d_bpad) out->launches_per_spmm += 1;  // the padded copy of B
   out->column_tiles = plan->tiles;
   out->hub_rows = plan->n_hub;
   out->lds_served_nnz = plan->oserved;
@@ -2212,6 +2236,7 @@ int hpspmm_plan_destroy(hpspmm_plan* plan) {
   if (plan->d_hub_ids) (void)hipFree(plan->d_hub_ids);
   if (plan->d_hub_col) (void)hipFree(plan->d_hub_col);
   if (plan->d_bhot) (void)hipFree(plan->d_bhot);
+  if (plan->d_bpad) (void)hipFree(plan->d_bpad);
   for (void* q : {(void*)plan->d_rvptr, (void*)plan->d_coldptr, (void*)plan->d_vcol, (void*)plan->d_lslot,
                   (void*)plan->d_chunk_base, (void*)plan->d_chunk_pref,
                   (void*)plan->d_vval, (void*)plan->d_vsrc, (void*)plan->d_vrow, (void*)plan->d_bhot_src, (void*)plan->d_partial,
@@ -2291,16 +2316,27 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
   int rc;
   // another value array overwrites the plan's copy of the bound one
   if (plan->bound_val && plan->bound_val != d_val) plan->bound_val = nullptr;
-  if (plan->k_full != plan->k) {
+  if (plan->k_full != plan->k || plan->k_user != plan->k_full) {
     // one column tile after the other through the layout built for the tile width; the operands of
-    // tile t are columns [t * k, (t + 1) * k) of B and C, whose rows are k_full floats apart
+    // tile t are columns [t * k, (t + 1) * k) of B and C.  The rows of B are k_full floats apart -
+    // the caller's B, or its padded copy when the caller's row length is not a multiple of 4 -,
+    // those of C k_user floats.
     rc = HPSPMM_OK;
+    const float* Bsrc = d_B;
+    if (plan->k_user != plan->k_full) {
+      hipLaunchKernelGGL(hpspmm::pad_rows_kernel, dim3(grid_for(plan->cols * plan->k_full, 1 << 16)), dim3(hpspmm::kBlock),
+                         0, st, plan->cols, plan->k_user, plan->k_full, d_B, plan->d_bpad);
+      mark_launch(st, "pad_rows_kernel");
+      Bsrc = plan->d_bpad;
+    }
+    const uint32_t shorter = (uint32_t)(plan->k_full - plan->k_user);  // 0 ... 3
     for (int t = 0; t < plan->tiles && rc == HPSPMM_OK; ++t) {
-      const float* Bt = d_B + (int64_t)t * plan->k;
+      const float* Bt = Bsrc + (int64_t)t * plan->k;
       float* Ct = d_C + (int64_t)t * plan->k;
-      // the row length, and above it the columns of the tile that exist when the last one is narrower
-      const int64_t left = plan->k_full - (int64_t)t * plan->k;
-      const uint32_t ld = (uint32_t)plan->k_full | (left < plan->k ? (uint32_t)left << 24 : 0u);
+      // the row length of B; how much shorter C's rows are; the columns of the tile that exist when
+      // the last one is narrower than the layout
+      const int64_t left = plan->k_user - (int64_t)t * plan->k;
+      const uint32_t ld = (uint32_t)plan->k_full | shorter << 22 | (left < plan->k ? (uint32_t)left << 24 : 0u);
       if (plan->strategy == HPSPMM_STRATEGY_ORDERED) {
         switch (plan->k) {
           case 32: rc = launch_ordered<32, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;

@@ -432,7 +432,7 @@ __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
   for (int i = tid; i < cap * G; i += kBlock) {
     const int slot = i / G;
     const int32_t c = wcols[blk * cap + slot];
-    if (c >= 0 && lane_in_tile<K, kLd>(ld_arg, i % G))
+    if (c >= 0 && lane_columns<K, kLd>(ld_arg, i % G) > 0)
       *reinterpret_cast<float4*>(s_b + slot * K + 4 * (i % G)) = load_b_ld(B, c, i % G, ld);
   }
   __syncthreads();
@@ -443,16 +443,23 @@ __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
   const int64_t e = (s + ((int64_t)1 << shift)) < nnz ? (s + ((int64_t)1 << shift)) : nnz;
   const int sbase = ((tid >> 6) * P + lane / G) * kTileStride;
 
-  const bool in_tile = lane_in_tile<K, kLd>(ld_arg, l);
+  const int nv = lane_columns<K, kLd>(ld_arg, l);
+  const bool in_tile = nv > 0;
+  const bool c_aligned = c_rows_aligned<kLd>(ld_arg);
+  const uint32_t ldc = c_row_length<K, kLd>(ld_arg);
   int32_t cur = orow[s];
   bool head_pending = (int64_t)start[cur] < s;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 
   auto flush_to = [&](bool is_tail) {
+    const bool to_c = !head_pending && !is_tail;  // a row of C; else a carry slot (aligned, K floats)
     float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
-                              : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : C + (uint64_t)(uint32_t)cur * ld);
+                              : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : C + (uint64_t)(uint32_t)cur * ldc);
     head_pending = false;
-    if (in_tile) store_result(dst + 4 * l, acc);  // (a lane beyond the tile holds zeros: nothing of it is ever read)
+    if (in_tile) {  // (what a lane beyond the tile holds is never read)
+      if (to_c) store_c_row<kLd, true>(dst + 4 * l, acc, nv, c_aligned);
+      else store_result(dst + 4 * l, acc);
+    }
   };
   auto flush = [&]() { flush_to(false); };
   // One flat load per gather, its address selected between the LDS copy and memory: a branch

@@ -523,7 +523,7 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
     const int32_t c = src[s];
     if (c < 0) return;
     *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) =
-        lane_in_tile<K, kLd>(ld_arg, l) ? load_b_ld(B, c, l, row_length<K, kLd>(ld_arg)) : make_float4(0.f, 0.f, 0.f, 0.f);
+        lane_columns<K, kLd>(ld_arg, l) > 0 ? load_b_ld(B, c, l, row_length<K, kLd>(ld_arg)) : make_float4(0.f, 0.f, 0.f, 0.f);
     return;
   }
   const int64_t chunk = (int64_t)blockIdx.x - gather_blocks;
@@ -615,7 +615,9 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
-  const bool in_tile = lane_in_tile<K, kLd>(ld_arg, l);
+  const int nv = lane_columns<K, kLd>(ld_arg, l);
+  const bool in_tile = nv > 0;
+  const bool c_aligned = c_rows_aligned<kLd>(ld_arg);
   const int shift = lay.shift;
   const int64_t g = (lay.cls_begin[x] >> shift) + (i * kWavesPerBlock + (tid >> 6)) * P + lane / G;
   const int64_t s = g << shift;
@@ -627,17 +629,21 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
   const int32_t* vp = hub ? rvptr + x : coldptr;
   const int64_t vstride = hub ? nhub : 1;
   float* out = hub ? partial + (uint64_t)x * K : C;
-  const uint64_t ostride = hub ? (uint64_t)nhub * K : (uint64_t)ld;
+  const uint64_t ostride = hub ? (uint64_t)nhub * K : (uint64_t)c_row_length<K, kLd>(ld_arg);
 
   int32_t cur = vrow[s];
   bool head_pending = (int64_t)vp[(int64_t)cur * vstride] < s;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 
   auto flush_to = [&](bool is_tail) {
+    const bool to_c = !hub && !head_pending && !is_tail;  // a row of C; else a carry slot or a partial row (aligned, K floats)
     float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
                               : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : out + (uint64_t)(uint32_t)cur * ostride);
     head_pending = false;
-    if (in_tile) store_result(dst + 4 * l, acc);  // (a lane beyond the tile holds zeros: nothing of it is ever read)
+    if (in_tile) {  // (what a lane beyond the tile holds is never read)
+      if (to_c) store_c_row<kLd, true>(dst + 4 * l, acc, nv, c_aligned);
+      else store_result(dst + 4 * l, acc);
+    }
   };
   auto flush = [&]() { flush_to(false); };
   // a lane beyond the tile gathers what lane 0 gathers (a valid address, no branch in the loop); its
@@ -730,13 +736,15 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
     const float* __restrict__ partial, const float* __restrict__ carry, float* __restrict__ C, uint32_t ld_arg) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
-  const uint32_t ld = row_length<K, kLd>(ld_arg);  // floats between the rows of C
+  const uint32_t ld = c_row_length<K, kLd>(ld_arg);  // floats between the rows of C
+  const bool c_aligned = c_rows_aligned<kLd>(ld_arg);
   constexpr int kGroup = kSlices;  // classes whose loads are in flight together; divides nhub
   __shared__ int32_t s_bounds[kWavesPerBlock * P][2 * kMaxHub + 1];  // odd stride: sub-waves on different banks
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
-  const bool in_tile = lane_in_tile<K, kLd>(ld_arg, l);
+  const int nv = lane_columns<K, kLd>(ld_arg, l);
+  const bool in_tile = nv > 0;
   const int shift = lay.shift;
   const int nhub = lay.nhub;
   const float* cbase = carry + 4 * l;
@@ -766,7 +774,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
   if ((int64_t)blockIdx.x >= routed_blocks + cross_blocks) {
     const int64_t idx = ((int64_t)blockIdx.x - routed_blocks - cross_blocks) * (kWavesPerBlock * P) + sub;
     if (idx >= n_zero) return;
-    if (in_tile) *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * ld + 4 * l) = acc;
+    if (in_tile) store_c_row<kLd, false>(C + (uint64_t)(uint32_t)zero_rows[idx] * ld + 4 * l, acc, nv, c_aligned);
     return;
   }
   if ((int64_t)blockIdx.x >= routed_blocks) {
@@ -777,7 +785,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
     const int64_t gb = (coldptr[row + 1] - 1) >> shift;
     add(*reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * ga + 1) * K));
     add_heads(ga + 1, gb);
-    if (in_tile) *reinterpret_cast<float4*>(C + (uint64_t)row * ld + 4 * l) = acc;
+    if (in_tile) store_c_row<kLd, false>(C + (uint64_t)row * ld + 4 * l, acc, nv, c_aligned);
     return;
   }
   const int64_t idx = (int64_t)blockIdx.x * (kWavesPerBlock * P) + sub;
@@ -836,7 +844,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
       if (gb > ga + 1) add_heads(ga + 2, gb);
     }
   }
-  if (in_tile) *reinterpret_cast<float4*>(C + (uint64_t)row * ld + 4 * l) = acc;
+  if (in_tile) store_c_row<kLd, false>(C + (uint64_t)row * ld + 4 * l, acc, nv, c_aligned);
 }
 
 }  // namespace hpspmm

@@ -74,18 +74,46 @@ __device__ __forceinline__ float4 load_b(const float* __restrict__ B, int32_t c,
 // The same with the row length of B given at run time: the operands of a tuned kernel may be K
 // columns of a wider B and C (one column tile of a product whose row length is a multiple of K).
 // kLd = false compiles to the fixed form.
-// ld_arg carries two things: the row length in its low 24 bits and, in the bits above, how many of
-// the tile's K columns exist (0 = all of them): the last tile of a row length that is not a
-// multiple of K is narrower, and the lanes whose columns lie beyond it must neither read B nor write C.
+// ld_arg carries three things: in bits 0-21 the row length of B (a multiple of 4); in bits 22-23 by
+// how much the rows of C are shorter (0 ... 3: the caller's row length need not be a multiple of 4
+// - B is then a copy padded to one, C is the caller's own); in bits 24-31 how many of the tile's K
+// columns exist (0 = all of them): the last tile of a row length that is not a multiple of K is
+// narrower, and the lanes whose columns lie beyond it must not write C.
 template <int K, bool kLd>
 __device__ __forceinline__ uint32_t row_length(uint32_t ld_arg) {
-  return kLd ? (ld_arg & 0xFFFFFFu) : (uint32_t)K;
+  return kLd ? (ld_arg & 0x3FFFFFu) : (uint32_t)K;
 }
 template <int K, bool kLd>
-__device__ __forceinline__ bool lane_in_tile(uint32_t ld_arg, int l) {
-  if constexpr (!kLd) return true;
-  const uint32_t cols = ld_arg >> 24;
-  return cols == 0 || (uint32_t)(4 * l) < cols;
+__device__ __forceinline__ uint32_t c_row_length(uint32_t ld_arg) {
+  return kLd ? (ld_arg & 0x3FFFFFu) - ((ld_arg >> 22) & 3u) : (uint32_t)K;
+}
+// C's rows start at multiples of 16 bytes (when C itself does).
+template <bool kLd>
+__device__ __forceinline__ bool c_rows_aligned(uint32_t ld_arg) {
+  return !kLd || ((ld_arg >> 22) & 3u) == 0;
+}
+// How many of lane l's four columns exist in the tile (0 ... 4).
+template <int K, bool kLd>
+__device__ __forceinline__ int lane_columns(uint32_t ld_arg, int l) {
+  if constexpr (!kLd) return 4;
+  const int cols = (int)(ld_arg >> 24);
+  if (cols == 0) return 4;
+  const int left = cols - 4 * l;
+  return left < 0 ? 0 : left > 4 ? 4 : left;
+}
+// A lane's nv (1 ... 4) columns into a row of C: in the form the fixed kernels use when the rows are
+// aligned and the lane owns all four, else float by float.
+template <bool kLd, bool kStream>
+__device__ __forceinline__ void store_c_row(float* __restrict__ p, const float4& v, int nv, bool aligned) {
+  if (!kLd || (aligned && nv == 4)) {
+    if constexpr (kStream) store_result(p, v);
+    else *reinterpret_cast<float4*>(p) = v;
+  } else {
+    p[0] = v.x;
+    if (nv > 1) p[1] = v.y;
+    if (nv > 2) p[2] = v.z;
+    if (nv > 3) p[3] = v.w;
+  }
 }
 __device__ __forceinline__ float4 load_b_ld(const float* __restrict__ B, int32_t c, int l, uint32_t ld) {
   return *reinterpret_cast<const float4*>(B + (uint64_t)(uint32_t)c * (uint64_t)ld + (uint32_t)(4 * l));
@@ -479,11 +507,13 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
                                                             uint32_t ld_arg) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
-  const uint32_t ld = row_length<K, kLd>(ld_arg);  // floats between the rows of C
+  const uint32_t ld = c_row_length<K, kLd>(ld_arg);  // floats between the rows of C
+  const bool c_aligned = c_rows_aligned<kLd>(ld_arg);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
-  const bool in_tile = lane_in_tile<K, kLd>(ld_arg, l);
+  const int nv = lane_columns<K, kLd>(ld_arg, l);
+  const bool in_tile = nv > 0;
   const int sub = lane / G;
   const int64_t r0 = ((int64_t)blockIdx.x * kWavesPerBlock + (tid >> 6)) * rpw;
   if (r0 >= rows) return;
@@ -528,15 +558,15 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
     // every lane takes part in the shuffles; only then do the sub-waves diverge
     const int32_t lb_i = __shfl(lb, i);
     const int32_t hb_i = __shfl(hb, i);
-    float4* out = reinterpret_cast<float4*>(C + (uint64_t)(r0 + i) * ld + 4 * l);
+    float* out = C + (uint64_t)(r0 + i) * ld + 4 * l;
     if ((m_empty >> i) & 1ull) {
-      if (in_tile) *out = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (in_tile) store_c_row<kLd, false>(out, make_float4(0.f, 0.f, 0.f, 0.f), nv, c_aligned);
     } else if ((m_split >> i) & 1ull) {
       const int64_t ga = (int64_t)lb_i >> shift;
       const int64_t gb = (int64_t)(hb_i - 1) >> shift;
       float4 acc = *reinterpret_cast<const float4*>(carry + (uint64_t)(2 * ga + 1) * K + 4 * l);
       add_heads(acc, ga + 1, gb, 1);
-      if (in_tile) *out = acc;
+      if (in_tile) store_c_row<kLd, false>(out, acc, nv, c_aligned);
     }
   }
   // Long chains, one row at a time, all P sub-waves together: sub-wave s adds the heads ga+1+s,
@@ -561,7 +591,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
       t.w = __shfl(part.w, s * G + l);
       add(acc, t);
     }
-    if (sub == 0 && in_tile) *reinterpret_cast<float4*>(C + (uint64_t)(r0 + i) * ld + 4 * l) = acc;
+    if (sub == 0 && in_tile) store_c_row<kLd, false>(C + (uint64_t)(r0 + i) * ld + 4 * l, acc, nv, c_aligned);
   }
 }
 
@@ -685,6 +715,16 @@ __global__ __launch_bounds__(kBlock) void expand_rows_kernel(int64_t rows, int64
 __global__ __launch_bounds__(64) void xcc_probe_kernel(int32_t* __restrict__ out) {
   const unsigned v = __builtin_amdgcn_s_getreg(((4 - 1) << 11) | (0 << 6) | 20);
   if (threadIdx.x == 0) out[blockIdx.x] = (int32_t)(v & 0xFu);
+}
+
+// dst[r, 0:kp) = src[r, 0:k) followed by zeros: B with its rows padded to a multiple of 4 floats.
+__global__ __launch_bounds__(kBlock) void pad_rows_kernel(int64_t rows, int64_t k, int64_t kp,
+                                                          const float* __restrict__ src, float* __restrict__ dst) {
+  const int64_t total = rows * kp;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t r = i / kp, j = i - r * kp;
+    dst[i] = j < k ? src[r * k + j] : 0.f;
+  }
 }
 
 __global__ __launch_bounds__(kBlock) void fill_f32_kernel(float* __restrict__ x, int64_t n, float v) {

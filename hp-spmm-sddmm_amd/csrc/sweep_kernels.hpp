@@ -464,7 +464,8 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
 
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   // the plan checks that B is below 4 GB: a 32-bit byte offset
-  const bool in_tile = lane_in_tile<K, kLd>(ld_arg, l);
+  const int nv = lane_columns<K, kLd>(ld_arg, l);
+  const bool in_tile = nv > 0;
   // a lane beyond the tile gathers what lane 0 gathers (a valid address, no branch in the loop); its
   // sums are never stored to C
   const int lg = in_tile ? l : 0;
@@ -592,8 +593,12 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
     const int32_t dest = slot_row[wave * WS + slot];
     if (dest == kSweepUnused) continue;
     const float4 sum = *reinterpret_cast<const float4*>(acc_wave + slot * K + 4 * l);
-    float* out = dest >= 0 ? C + (uint64_t)(uint32_t)dest * ld : partial + (uint64_t)(uint32_t)~dest * K;
-    if (in_tile) store_result(out + 4 * l, sum);  // (a lane beyond the tile holds zeros: nothing of it is ever read)
+    float* out = dest >= 0 ? C + (uint64_t)(uint32_t)dest * c_row_length<K, kLd>(ld_arg)
+                           : partial + (uint64_t)(uint32_t)~dest * K;
+    if (in_tile) {  // (what a lane beyond the tile holds is never read)
+      if (dest >= 0) store_c_row<kLd, true>(out + 4 * l, sum, nv, c_rows_aligned<kLd>(ld_arg));
+      else store_result(out + 4 * l, sum);
+    }
   }
 }
 
@@ -606,7 +611,8 @@ __global__ __launch_bounds__(kBlock) void spmm_sweep_final_kernel(
     int64_t n_zero, const float* __restrict__ partial, float* __restrict__ C, uint32_t ld_arg) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
-  const uint32_t ld = row_length<K, kLd>(ld_arg);  // floats between the rows of C
+  const uint32_t ld = c_row_length<K, kLd>(ld_arg);  // floats between the rows of C
+  const bool c_aligned = c_rows_aligned<kLd>(ld_arg);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int l = lane % G;
@@ -614,8 +620,9 @@ __global__ __launch_bounds__(kBlock) void spmm_sweep_final_kernel(
   if ((int64_t)blockIdx.x >= split_blocks) {
     const int64_t idx = ((int64_t)blockIdx.x - split_blocks) * (kWavesPerBlock * P) + sub;
     if (idx >= n_zero) return;
-    if (lane_in_tile<K, kLd>(ld_arg, l))
-      *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)zero_rows[idx] * ld + 4 * l) = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int nvz = lane_columns<K, kLd>(ld_arg, l);
+    if (nvz > 0)
+      store_c_row<kLd, false>(C + (uint64_t)(uint32_t)zero_rows[idx] * ld + 4 * l, make_float4(0.f, 0.f, 0.f, 0.f), nvz, c_aligned);
     return;
   }
   const int64_t idx = (int64_t)blockIdx.x * (kWavesPerBlock * P) + sub;
@@ -644,7 +651,8 @@ __global__ __launch_bounds__(kBlock) void spmm_sweep_final_kernel(
     acc.z += t.z;
     acc.w += t.w;
   }
-  if (lane_in_tile<K, kLd>(ld_arg, l)) *reinterpret_cast<float4*>(C + (uint64_t)(uint32_t)row * ld + 4 * l) = acc;
+  const int nv = lane_columns<K, kLd>(ld_arg, l);
+  if (nv > 0) store_c_row<kLd, false>(C + (uint64_t)(uint32_t)row * ld + 4 * l, acc, nv, c_aligned);
 }
 
 }  // namespace hpspmm

@@ -136,19 +136,20 @@ const char *hpspmm_last_error(void);
  * nonzeros ("routed"); or segments over a clustered row order with the reused
  * rows of B held in LDS when the matrix is a graph with communities
  * ("ordered").
- * k = 32, 64 and 128 are the tuned row lengths.  Any other multiple of 4 from
- * 16 up (16, 40, 96, 160, 256, 512 ...) is served by the sweep, routed and
- * ordered layouts one column tile of 128, 64 or 32 columns after the other
- * (the reference tiles the columns the same way, spmm/mm/spmm_kernel.cu:
- * 412-420: grid.y = ceil(k / 64)); a last tile narrower than the layout leaves
- * its surplus lanes idle.  That is done when the matrix gets one of those
- * layouts (at least 2^22 nonzeros, or a forcing flag); launches_per_spmm
- * counts every tile's, column_tiles the tiles.
- * Otherwise, and for every other k, whole rows or segments run with sub-waves
- * of ceil(k / 4) lanes rounded up to a power of two; when k is not a multiple
- * of 4 (41 classes, 47, 173 ...) the rows of B and C are read and written at
- * their 4-byte alignment and the lane that owns a row's last columns touches
- * only those that exist.
+ * k = 32, 64 and 128 are the tuned row lengths.  Any other k from 16 up is
+ * served by the sweep, routed and ordered layouts one column tile of 128, 64
+ * or 32 columns after the other (the reference tiles the columns the same way,
+ * spmm/mm/spmm_kernel.cu:412-420: grid.y = ceil(k / 64)); a last tile narrower
+ * than the layout leaves its surplus lanes idle.  When k is not a multiple of
+ * 4 (41 classes, 47, 173 ...) the plan then keeps a copy of B with rows padded
+ * to one - refreshed by one more launch at the start of every SpMM, part of
+ * workspace_bytes - because 16-byte gathers from rows at 4-byte alignment cost
+ * about twice; C is written in place.  All that is done when the matrix gets
+ * one of those layouts (at least 2^22 nonzeros, or a forcing flag);
+ * launches_per_spmm counts every tile's launches, column_tiles the tiles.
+ * Otherwise, and for k < 16, whole rows or segments run with sub-waves of
+ * ceil(k / 4) lanes rounded up to a power of two, rows of B and C read and
+ * written at whatever alignment they have.
  * Replaces the host-side preprocessing the reference does before timing:
  * CSR->COO expansion (spmm/mm/spmm_common.cpp:185-235), the row re-ordering
  * (:237-296) and the choice of nnz_per_warp (spmm/mm/spmm_kernel.cu:749-751).
@@ -177,8 +178,7 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d
  * result is that of hpspmm_plan_create up to summation order.  The role of the
  * row permutation that the reference reads from a .cugraph_reorder file for
  * HP-SpMM (spmm/mm/spmm_common.cpp:237-296: nonzeros emitted in that row
- * order, row indices kept).  k must be a multiple of 4, and at least 16, for
- * the order to be used.
+ * order, row indices kept).  k must be at least 16 for the order to be used.
  */
 int hpspmm_plan_create_ordered(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
                                const int32_t *d_col, int64_t k, uint32_t flags,

@@ -490,7 +490,7 @@ int launch_segments(const hpspmm_plan* p, const int32_t* rp, const int32_t* ci, 
 constexpr int kOrderedBlockLdsBytes = 52992;
 
 // kLd: B and C are K columns of wider arrays whose rows are `ld` floats apart (one column tile).
-template <int K, bool kLd = false>
+template <int K, int kLd = 0>
 int launch_ordered(const hpspmm_plan* p, const int32_t* rp, const float* v, const float* B, float* C,
                    hipStream_t st, uint32_t ld = K) {
   const int64_t nblocks = p->owindows;
@@ -1236,7 +1236,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
 
 // kLd: B and C are K columns of wider arrays whose rows are `ld` floats apart (one column tile);
 // values_ready: an earlier tile of the same product has already brought the values into the plan's order.
-template <int K, bool kLd = false>
+template <int K, int kLd = 0>
 int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st, uint32_t ld = K,
                   bool values_ready = false) {
   // values bound to the plan are already in class-major order: only the hub rows of B are refreshed
@@ -1587,9 +1587,13 @@ int sweep_prepare_kernels(int* out) {
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_sweep_kernel<K, false>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_sweep_kernel<K, true, true>),
+  HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_sweep_kernel<K, true, 1>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_sweep_kernel<K, false, true>),
+  HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_sweep_kernel<K, false, 1>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_sweep_kernel<K, true, 2>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_sweep_kernel<K, false, 2>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   HPSPMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(out, hpspmm::spmm_sweep_kernel<K, true>,
                                                           hpspmm::sweep_waves<K>() * 64, lds));
@@ -1854,7 +1858,7 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
 }
 
 // kLd: B and C are K columns of wider arrays whose rows are `ld` floats apart (one column tile).
-template <int K, bool kLd = false>
+template <int K, int kLd = 0>
 int launch_sweep(const hpspmm_plan* p, const int32_t* rp, const float* v, const float* B, float* C, hipStream_t st,
                  uint32_t ld = K) {
   const bool bound = p->bound_val && p->bound_val == v && p->d_vval;
@@ -2337,26 +2341,49 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
       // the last one is narrower than the layout
       const int64_t left = plan->k_user - (int64_t)t * plan->k;
       const uint32_t ld = (uint32_t)plan->k_full | shorter << 22 | (left < plan->k ? (uint32_t)left << 24 : 0u);
-      if (plan->strategy == HPSPMM_STRATEGY_ORDERED) {
-        switch (plan->k) {
-          case 32: rc = launch_ordered<32, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
-          case 64: rc = launch_ordered<64, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
-          default: rc = launch_ordered<128, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
-        }
-      } else if (plan->strategy == HPSPMM_STRATEGY_SWEEP) {
-        switch (plan->k) {
-          case 32: rc = launch_sweep<32, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
-          case 64: rc = launch_sweep<64, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
-          default: rc = launch_sweep<128, true>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
-        }
-      } else if (plan->strategy == HPSPMM_STRATEGY_ROUTED) {
-        switch (plan->k) {
-          case 32: rc = launch_routed<32, true>(plan, d_val, Bt, Ct, st, ld, t > 0); break;
-          case 64: rc = launch_routed<64, true>(plan, d_val, Bt, Ct, st, ld, t > 0); break;
-          default: rc = launch_routed<128, true>(plan, d_val, Bt, Ct, st, ld, t > 0); break;
-        }
-      } else {
+      if (plan->strategy != HPSPMM_STRATEGY_ORDERED && plan->strategy != HPSPMM_STRATEGY_SWEEP &&
+          plan->strategy != HPSPMM_STRATEGY_ROUTED) {
         rc = fail(HPSPMM_ERR_INVALID_ARG, "plan of column tiles without a tiled strategy");
+      } else if (shorter == 0) {
+        if (plan->strategy == HPSPMM_STRATEGY_ORDERED) {
+          switch (plan->k) {
+            case 32: rc = launch_ordered<32, 1>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+            case 64: rc = launch_ordered<64, 1>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+            default: rc = launch_ordered<128, 1>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+          }
+        } else if (plan->strategy == HPSPMM_STRATEGY_SWEEP) {
+          switch (plan->k) {
+            case 32: rc = launch_sweep<32, 1>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+            case 64: rc = launch_sweep<64, 1>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+            default: rc = launch_sweep<128, 1>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+          }
+        } else {
+          switch (plan->k) {
+            case 32: rc = launch_routed<32, 1>(plan, d_val, Bt, Ct, st, ld, t > 0); break;
+            case 64: rc = launch_routed<64, 1>(plan, d_val, Bt, Ct, st, ld, t > 0); break;
+            default: rc = launch_routed<128, 1>(plan, d_val, Bt, Ct, st, ld, t > 0); break;
+          }
+        }
+      } else {  // rows of C shorter than those of B, at any 4-byte alignment
+        if (plan->strategy == HPSPMM_STRATEGY_ORDERED) {
+          switch (plan->k) {
+            case 32: rc = launch_ordered<32, 2>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+            case 64: rc = launch_ordered<64, 2>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+            default: rc = launch_ordered<128, 2>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+          }
+        } else if (plan->strategy == HPSPMM_STRATEGY_SWEEP) {
+          switch (plan->k) {
+            case 32: rc = launch_sweep<32, 2>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+            case 64: rc = launch_sweep<64, 2>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+            default: rc = launch_sweep<128, 2>(plan, d_rowptr, d_val, Bt, Ct, st, ld); break;
+          }
+        } else {
+          switch (plan->k) {
+            case 32: rc = launch_routed<32, 2>(plan, d_val, Bt, Ct, st, ld, t > 0); break;
+            case 64: rc = launch_routed<64, 2>(plan, d_val, Bt, Ct, st, ld, t > 0); break;
+            default: rc = launch_routed<128, 2>(plan, d_val, Bt, Ct, st, ld, t > 0); break;
+          }
+        }
       }
     }
   } else if (plan->strategy == HPSPMM_STRATEGY_ORDERED) {

@@ -407,7 +407,7 @@ __global__ __launch_bounds__(kBlock) void ordered_partition_kernel(int64_t rows,
 
 // One workgroup per window = kWavesPerBlock * P segments of 2^shift nonzeros.
 // Dynamic LDS: cap * K floats, the window's slotted rows of B.
-template <int K, bool kLd = false>
+template <int K, int kLd = 0>
 __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
     const int32_t* __restrict__ rowptr, const int32_t* __restrict__ start, const int32_t* __restrict__ ocol,
     const int32_t* __restrict__ osrc, const int32_t* __restrict__ orow, const float* __restrict__ val,

@@ -501,7 +501,7 @@ __global__ __launch_bounds__(kBlock) void routed_chunk_kernel(RoutedLayout lay, 
 // single values costs one L2 transaction for every two or three of them; so
 // the chunk is sorted by destination in LDS (lslot) and written out run by
 // run in full lines (233k-vertex social graph: 0.28 ms for the plain scatter).
-template <int K, bool kLd = false>
+template <int K, int kLd = 0>
 __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, int64_t gather_blocks,
                                                                 const int32_t* __restrict__ src,
                                                                 const float* __restrict__ B,
@@ -573,7 +573,7 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
 // indices, so these loads stay coalesced).  kHub: vcol may hold ~(compact-buffer row); without it
 // every entry is a plain column and the gather address is B plus a 32-bit byte offset (the plan
 // checks that B is below 4 GB), three instructions instead of eight.
-template <int K, bool kInPlace, bool kHub, bool kLd = false>
+template <int K, bool kInPlace, bool kHub, int kLd = 0>
 __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, const int32_t* __restrict__ rvptr,
                                                              const int32_t* __restrict__ coldptr,
                                                              const int32_t* __restrict__ vcol,
@@ -728,7 +728,7 @@ __global__ __launch_bounds__(kBlock) void routed_collect_rows_kernel(int64_t row
 // cold-class run crossed a segment boundary, from the carry slots alone.
 // The rest: rows without nonzeros, which get zeros.
 // Rows in none of the lists were stored by the main kernel.
-template <int K, bool kLd = false>
+template <int K, int kLd = 0>
 __global__ __launch_bounds__(kBlock) void spmm_routed_final_kernel(
     RoutedLayout lay, const int32_t* __restrict__ rvptr, const int32_t* __restrict__ coldptr,
     const int32_t* __restrict__ routed_rows, int64_t routed_blocks, const int32_t* __restrict__ cross_rows,

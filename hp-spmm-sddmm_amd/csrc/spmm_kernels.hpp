@@ -72,30 +72,32 @@ __device__ __forceinline__ float4 load_b(const float* __restrict__ B, int32_t c,
 }
 
 // The same with the row length of B given at run time: the operands of a tuned kernel may be K
-// columns of a wider B and C (one column tile of a product whose row length is a multiple of K).
-// kLd = false compiles to the fixed form.
+// columns of a wider B and C (one column tile of a product whose row length is not K).  kLd = 0
+// compiles to the fixed form; 1 = row lengths at run time, multiples of 4; 2 = the rows of C may be
+// up to three floats shorter than those of B and start at any multiple of 4 bytes (B is then a
+// padded copy of the caller's), and a lane may own fewer than four columns of C.
 // ld_arg carries three things: in bits 0-21 the row length of B (a multiple of 4); in bits 22-23 by
 // how much the rows of C are shorter (0 ... 3: the caller's row length need not be a multiple of 4
 // - B is then a copy padded to one, C is the caller's own); in bits 24-31 how many of the tile's K
 // columns exist (0 = all of them): the last tile of a row length that is not a multiple of K is
 // narrower, and the lanes whose columns lie beyond it must not write C.
-template <int K, bool kLd>
+template <int K, int kLd>
 __device__ __forceinline__ uint32_t row_length(uint32_t ld_arg) {
   return kLd ? (ld_arg & 0x3FFFFFu) : (uint32_t)K;
 }
-template <int K, bool kLd>
+template <int K, int kLd>
 __device__ __forceinline__ uint32_t c_row_length(uint32_t ld_arg) {
-  return kLd ? (ld_arg & 0x3FFFFFu) - ((ld_arg >> 22) & 3u) : (uint32_t)K;
+  return kLd == 2 ? (ld_arg & 0x3FFFFFu) - ((ld_arg >> 22) & 3u) : row_length<K, kLd>(ld_arg);
 }
 // C's rows start at multiples of 16 bytes (when C itself does).
-template <bool kLd>
+template <int kLd>
 __device__ __forceinline__ bool c_rows_aligned(uint32_t ld_arg) {
-  return !kLd || ((ld_arg >> 22) & 3u) == 0;
+  return kLd < 2 || ((ld_arg >> 22) & 3u) == 0;
 }
 // How many of lane l's four columns exist in the tile (0 ... 4).
-template <int K, bool kLd>
+template <int K, int kLd>
 __device__ __forceinline__ int lane_columns(uint32_t ld_arg, int l) {
-  if constexpr (!kLd) return 4;
+  if constexpr (kLd == 0) return 4;
   const int cols = (int)(ld_arg >> 24);
   if (cols == 0) return 4;
   const int left = cols - 4 * l;
@@ -103,9 +105,9 @@ __device__ __forceinline__ int lane_columns(uint32_t ld_arg, int l) {
 }
 // A lane's nv (1 ... 4) columns into a row of C: in the form the fixed kernels use when the rows are
 // aligned and the lane owns all four, else float by float.
-template <bool kLd, bool kStream>
+template <int kLd, bool kStream>
 __device__ __forceinline__ void store_c_row(float* __restrict__ p, const float4& v, int nv, bool aligned) {
-  if (!kLd || (aligned && nv == 4)) {
+  if (kLd < 2 || (aligned && nv == 4)) {  // (kLd < 2: nv is 4 wherever this is called)
     if constexpr (kStream) store_result(p, v);
     else *reinterpret_cast<float4*>(p) = v;
   } else {
@@ -499,7 +501,7 @@ __global__ __launch_bounds__(kBlock) void spmm_segments_kernel(
 // five times the segments kernel before it).
 // `start` (may be NULL): first position of every row when the nonzeros were
 // processed in an order of the plan's own; NULL = stored order (rowptr).
-template <int K, bool kLd = false>
+template <int K, int kLd = 0>
 __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                             const int32_t* __restrict__ start,
                                                             const float* __restrict__ carry,

@@ -412,7 +412,7 @@ __global__ __launch_bounds__(kBlock) void sweep_gather_values_kernel(int64_t n, 
 // entries each, side by side.  kInPlace: vval is the caller's value array and vsrc[q] the index into
 // it of stream position q (fetched two tiles ahead, so that the value loads of the next tile never
 // wait for their indices); otherwise vval holds the values in stream order.
-template <int K, bool kInPlace, bool kLd = false>
+template <int K, bool kInPlace, int kLd = 0>
 __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
     SweepLayout lay, const uint32_t* __restrict__ wave_base, const uint32_t* __restrict__ wave_len,
     const int32_t* __restrict__ chunk_end, const int32_t* __restrict__ vent, const float* __restrict__ vval,
@@ -604,7 +604,7 @@ __global__ __launch_bounds__(sweep_waves<K>() * 64) void spmm_sweep_kernel(
 
 // Final pass.  Workgroups [0, split_blocks): one sub-wave per split row adds the row's partial
 // results in piece order and writes C.  The others: rows without nonzeros get zeros.
-template <int K, bool kLd = false>
+template <int K, int kLd = 0>
 __global__ __launch_bounds__(kBlock) void spmm_sweep_final_kernel(
     const int32_t* __restrict__ rowptr, int32_t limit, const int32_t* __restrict__ split_rows, int64_t n_split,
     int64_t split_blocks, const uint32_t* __restrict__ part_base, const int32_t* __restrict__ zero_rows,

@@ -674,10 +674,11 @@ def test_hip_graph_capture_and_replay(pkg, oracle, gpu):
     import torch
     capi = pkg.capi
     g = pkg.graphs.make_graph("c4_rmat", 0.004)
-    # every strategy at a tuned row length, then the tiled forms (3 tiles of 64 columns) of the three layouts that have one
+    # every strategy at a tuned row length, then the tiled forms of the three layouts that have one, at a row
+    # length that is not a multiple of 4 (3 tiles of 64 columns behind a padded copy of B)
     tiled = [(n, f) for n, f in _strategies(capi) if n in ("sweep", "routed", "routed_sort_values", "cluster_seg")]
     operands = {}
-    for name, flags, k in [(n, f, 64) for n, f in _strategies(capi)] + [(n + "_tiled", f, 192) for n, f in tiled]:
+    for name, flags, k in [(n, f, 64) for n, f in _strategies(capi)] + [(n + "_tiled", f, 173) for n, f in tiled]:
         if k not in operands:
             operands[k] = _to_dev(gpu, g.rowptr, g.col, g.val, pkg.graphs.make_dense("c4_rmat", g.cols, k))
         rp, ci, v, Bd = operands[k]

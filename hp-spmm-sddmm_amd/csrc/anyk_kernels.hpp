@@ -48,11 +48,6 @@ __device__ __forceinline__ ColumnTile column_tile(int tile, int K, int l) {
   return t;
 }
 
-// Four floats at a 4-byte aligned address.
-struct __attribute__((packed, aligned(4))) Float4Unaligned {
-  float x, y, z, w;
-};
-
 // The first nv (1 ... 4) of the four floats at p, zeros for the rest; kOdd = false: all four, p 16-byte aligned.
 template <bool kOdd>
 __device__ __forceinline__ float4 load_columns(const float* __restrict__ p, int nv) {

@@ -82,6 +82,15 @@ inline int64_t tile_width(int64_t k) {
 // Not a multiple of 4: rows of B and C start at any multiple of 4 bytes, the last lane of a row owns 1 to 3 columns.
 inline bool odd_k(int64_t k) { return k % 4 != 0; }
 // Lanes per sub-wave for such a K: the power of two that covers a column tile (at most 128 floats).
+// Row tiles (32-column tiles of B and C) serve every row length from 4 up
+// (HPSPMM_ROW_TILES_MIN_K in the environment raises that, for comparisons).
+inline bool row_tiles_serve(int64_t k) {
+  if (fast_k(k)) return true;
+  if (k < 4 || k >= ((int64_t)1 << 22)) return false;
+  const char* e = std::getenv("HPSPMM_ROW_TILES_MIN_K");
+  return k >= (e ? (int64_t)std::atoll(e) : (int64_t)4);
+}
+
 inline int anyk_lanes(int64_t k) {
   const int64_t g = ((k < hpspmm::kAnyKTile ? k : hpspmm::kAnyKTile) + 3) / 4;
   int gp = 2;
@@ -178,8 +187,13 @@ struct hpspmm_plan {
   // rows strategy over row tiles
   int2* d_tent = nullptr;     // [rt_tiles * 64] per tile entry: column (-1 = padding), slot / tile data by lane
   int2* d_ldesc = nullptr;    // [rt_loop] per long row: first tile, tile count
-  float* d_zrow = nullptr;    // 32 zeros: what a padding entry gathers instead of a row of B
+  float* d_zrow = nullptr;    // 4 + 32 zeros: what a padding entry gathers instead of a row of B (from d_zrow + 4)
   int32_t rt_tiles = 0, rt_waves = 0, rt_loop = 0, rt_wg = 0, rt_loop_tiles = 0;
+  // Row tiles at a row length outside the tuned set: rt_mode = the kernels' kLd (1: k a multiple of
+  // 4, B as it lies; 2: B through d_bpad, its rows padded to rt_ldb floats; 3: any k, B as it lies,
+  // gathered at 4-byte alignment), 0 = a tuned row length.
+  int rt_mode = 0;
+  uint32_t rt_ldb = 0;
   // sweep strategy (its stream arrays are d_vcol = entry words, d_vsrc, d_vval when values are bound;
   // partial-result rows of split rows in d_partial; rows without nonzeros in d_zero_rows)
   hpspmm::SweepLayout sw{};
@@ -296,6 +310,8 @@ constexpr int64_t kRowsAutoMaxWork = (int64_t)3 << 28;  // nnz * K, matrices of 
 constexpr double kRowsAutoLongMean = 128.0;             // mean nonzeros per non-empty row beyond which ...
 constexpr double kRowsAutoLongWork = 2.0e15;            // ... nnz^2 * K decides instead
 constexpr int64_t kRowsAutoMaxRow = 1 << 16;
+constexpr double kRowsAutoFewPerRowWork = 3.0e7;         // nnz * K, rows of <= 8 nonzeros, K not a multiple of 32
+constexpr int64_t kRowTilePadMinNnz = 1 << 19;  // row tiles: matrices from here up read a B of odd row length through a padded copy
 
 int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st);
 
@@ -305,24 +321,33 @@ inline const float* readable_values(const hpspmm_plan* p, const float* v) {
   return p->nnz > 0 ? v : reinterpret_cast<const float*>(p->d_tent);
 }
 
-template <int K, int WPB>
-int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
-  const int64_t blocks = ceil_div(p->rt_waves, WPB) * (K / 32);
-  hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
+// Row tiles at a row length outside the tuned set (K = 0 in the templates below): ldb, ldc = floats
+// between the rows of B and of C (= the columns there are); column tiles of 32.
+inline int64_t row_tile_column_tiles(int k_template, uint32_t ldc) {
+  return k_template ? k_template / 32 : (int64_t)((ldc + 31u) / 32u);
+}
+
+template <int K, int WPB, int kLd>
+int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st, uint32_t ldb,
+                       uint32_t ldc) {
+  const int64_t blocks = ceil_div(p->rt_waves, WPB) * row_tile_column_tiles(K, ldc);
+  if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB, kLd>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent, readable_values(p, v), B, C,
-                     p->d_zrow);
+                     p->d_zrow + 4, ldb, ldc);
   mark_launch(st, "spmm_rowtiles_kernel");
   return HPSPMM_OK;
 }
 
-template <int K, int WPB>
-int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
+template <int K, int WPB, int kLd>
+int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st, uint32_t ldb,
+                        uint32_t ldc) {
   const int64_t wave_items = (p->rt_loop - p->rt_wg) + (p->rt_tiles - p->rt_loop_tiles);
-  const int64_t blocks = (p->rt_wg + ceil_div(wave_items, WPB)) * (K / 32);
+  const int64_t blocks = (p->rt_wg + ceil_div(wave_items, WPB)) * row_tile_column_tiles(K, ldc);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
-  hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
+  hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB, kLd>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent,
-                     readable_values(p, v), B, C, p->d_zrow);
+                     readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc);
   mark_launch(st, "spmm_rowtiles_wg_kernel");
   return HPSPMM_OK;
 }
@@ -333,14 +358,16 @@ int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, fl
 // one wavefront needs about 0.6 us per 64 nonzeros, which a 16k-nonzero row turns into 150 us.
 constexpr int64_t kRowTileSmallGrid = 1 << 15;
 
-template <int K>
-int launch_row_tiles(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st) {
+template <int K, int kLd = 0>
+int launch_row_tiles(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st,
+                     uint32_t ldb = K, uint32_t ldc = K) {
   if (p->rt_wg > 0) {
-    if (p->max_row_nnz > 8192) return launch_row_tiles_wg<K, 16>(p, v, B, C, st);
-    return launch_row_tiles_wg<K, 8>(p, v, B, C, st);
+    if (p->max_row_nnz > 8192) return launch_row_tiles_wg<K, 16, kLd>(p, v, B, C, st, ldb, ldc);
+    return launch_row_tiles_wg<K, 8, kLd>(p, v, B, C, st, ldb, ldc);
   }
-  if ((int64_t)p->rt_waves * (K / 32) <= kRowTileSmallGrid) return launch_row_tiles_w<K, 1>(p, v, B, C, st);
-  return launch_row_tiles_w<K, hpspmm::kWavesPerBlock>(p, v, B, C, st);
+  if ((int64_t)p->rt_waves * row_tile_column_tiles(K, ldc) <= kRowTileSmallGrid)
+    return launch_row_tiles_w<K, 1, kLd>(p, v, B, C, st, ldb, ldc);
+  return launch_row_tiles_w<K, hpspmm::kWavesPerBlock, kLd>(p, v, B, C, st, ldb, ldc);
 }
 
 template <int GP, bool kOdd>
@@ -708,11 +735,11 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
   const size_t bytes_ent = (size_t)tiles * kTile * sizeof(int2);
   const size_t bytes_loop = (size_t)std::max<int64_t>(n_loop, 1) * sizeof(int2);
   if (hipMalloc(&p->d_tent, bytes_ent) != hipSuccess || hipMalloc(&p->d_ldesc, bytes_loop) != hipSuccess ||
-      hipMalloc(&p->d_zrow, 32 * sizeof(float)) != hipSuccess) {
+      hipMalloc(&p->d_zrow, 36 * sizeof(float)) != hipSuccess) {
     (void)hipGetLastError();
     return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the row tiles failed", bytes_ent + bytes_loop);
   }
-  p->workspace_bytes += (int64_t)(bytes_ent + bytes_loop + 32 * sizeof(float));
+  p->workspace_bytes += (int64_t)(bytes_ent + bytes_loop + 36 * sizeof(float));
   if (n_loop > 0) {
     hipLaunchKernelGGL(hpspmm::rowtile_long_tiles_kernel, dim3((unsigned)ceil_div(n_loop + 1, hpspmm::kBlock)),
                        dim3(hpspmm::kBlock), 0, st, n_loop, d_order, d_rowptr, d_long);
@@ -723,7 +750,7 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
   if (tiles > 0)
     hipLaunchKernelGGL(hpspmm::rowtile_fill_kernel, dim3((unsigned)ceil_div(tiles * kTile, hpspmm::kBlock)),
                        dim3(hpspmm::kBlock), 0, st, lay, d_order, p->d_ldesc, d_rowptr, d_col, p->d_tent);
-  HPSPMM_HIP(hipMemsetAsync(p->d_zrow, 0, 32 * sizeof(float), st));
+  HPSPMM_HIP(hipMemsetAsync(p->d_zrow, 0, 36 * sizeof(float), st));
   hipError_t e = hipStreamSynchronize(st);  // the temporaries go out of scope
   if (e == hipSuccess) e = hipGetLastError();
   if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "row tiles: %s", hipGetErrorString(e));
@@ -2009,16 +2036,15 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   ColumnRanking ranking;         // column popularity, shared by the routed and the hub-cache decisions
   bool rows_need_tiles = false;  // rows strategy chosen on the strength of the row tiles
   bool rows_range = false;       // provisional segments; rows unless the ordered strategy qualifies
-  if (!fast_k(k)) {
-    // not a tuned size (nor, at this point, a multiple of one on a matrix that gets a tiled layout):
-    // whole rows for small matrices (one launch), segments beyond (balanced over any degree
-    // distribution); the layouts built for the tuned sizes (row tiles, routed, ordered, hub cache)
-    // are not used
+  bool want_row_tiles = true;    // rows strategy: over row tiles if they can be built
+  if (!row_tiles_serve(k)) {
+    // a row length that not even the row tiles serve: whole rows over the CSR arrays for small
+    // matrices (one launch), segments beyond (balanced over any degree distribution)
     const bool small = nnz < (1 << 21) && p->max_row_nnz <= 4096;
     p->strategy = (flags & HPSPMM_PLAN_FORCE_SEGMENTS)                   ? HPSPMM_STRATEGY_SEGMENTS
                   : ((flags & HPSPMM_PLAN_FORCE_ROWS) || nnz == 0 || small) ? HPSPMM_STRATEGY_ROWS
                                                                            : HPSPMM_STRATEGY_SEGMENTS;
-  } else if (d_order && nnz > 0) {
+  } else if (d_order && nnz > 0 && fast_k(k)) {
     if (int rc = build_ordered(p, d_rowptr, d_col, d_order, 0.0, st)) {
       return rc;
     }
@@ -2041,18 +2067,32 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     const double mean_row = (double)nnz / (double)std::max<int64_t>(1, rows - p->empty_rows);
     const bool fits = mean_row > kRowsAutoLongMean ? (double)nnz * (double)nnz * (double)k < kRowsAutoLongWork
                                                    : nnz * k < kRowsAutoMaxWork;
-    const bool mid = nnz < kRowsAutoMaxNnz && fits && p->max_row_nnz <= kRowsAutoMaxRow &&
-                     !(flags & HPSPMM_PLAN_NO_ROW_TILES);
+    // (A row length outside the tuned set, on a matrix that has not got one of the tiled layouts:
+    // the alternative to row tiles is the run-time-K segments kernel, which they beat at every size
+    // measured - R-MAT graph, 7.6 M nonzeros, K = 48: 206 against 817 us; 0.9 M, K = 96: 25 against 521.)
+    // The exception are matrices of few nonzeros per row whose B is far beyond the L2s: what decides
+    // there is the traffic, and at a row length that is not a multiple of 32 floats the 128-byte
+    // gathers of neighbouring column tiles - made by different workgroups - both fetch the line they
+    // share (citation graph at 16 times its size, 1.6 M nonzeros, K = 100: 246 us against 142 for
+    // the rows kernel over the CSR arrays, whose sub-waves read whole rows of B; K = 256: 334
+    // against 337), while a padded copy of B costs more than it saves.
+    const bool few_per_row = mean_row <= 8.0;
+    const bool any_k_range = !few_per_row       ? nnz < kRowTileMaxNnz
+                             : k % 32 == 0      ? nnz < kRowsAutoMaxNnz && fits
+                                                : k <= 32 || (double)nnz * (double)k < kRowsAutoFewPerRowWork;
+    const bool in_range = fast_k(k) ? nnz < kRowsAutoMaxNnz && fits : any_k_range;
+    const bool mid = in_range && p->max_row_nnz <= kRowsAutoMaxRow && !(flags & HPSPMM_PLAN_NO_ROW_TILES);
     if (nnz == 0 || tiny || (mid && nnz < kClusterMinNnz)) {
       p->strategy = HPSPMM_STRATEGY_ROWS;
       rows_need_tiles = !(nnz == 0 || tiny);
+      want_row_tiles = mid;
     } else {
       p->strategy = HPSPMM_STRATEGY_SEGMENTS;
       rows_range = mid;
     }
   }
 
-  if (p->strategy == HPSPMM_STRATEGY_ROWS && fast_k(k) && rows > 0 && nnz < kRowTileMaxNnz &&
+  if (p->strategy == HPSPMM_STRATEGY_ROWS && want_row_tiles && row_tiles_serve(k) && rows > 0 && nnz < kRowTileMaxNnz &&
       !(flags & HPSPMM_PLAN_NO_ROW_TILES)) {
     if (int rc = build_row_tiles(p, d_rowptr, d_col, st)) {
       return rc;
@@ -2112,7 +2152,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       return rc;
     }
   }
-  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && rows_range) {
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && rows_range && row_tiles_serve(k)) {
     // no communities: whole rows after all, if the row tiles get built
     if (int rc = build_row_tiles(p, d_rowptr, d_col, st)) {
       return rc;
@@ -2126,6 +2166,30 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
       p->nseg = 0;
       p->shift = 0;
       p->strategy = HPSPMM_STRATEGY_ROWS;
+    }
+  }
+  if (p->d_tent && !fast_k(k)) {
+    // Row tiles at a row length of its own.  The gathers are fastest when every 32-column tile of a
+    // row of B is one aligned 128-byte line (R-MAT graph, 3.7 M nonzeros: K = 96 131 us, K = 100
+    // 204 us as it lies), so from 32 columns up a B whose rows are not a multiple of 32 floats is
+    // read through a copy with padded rows, refreshed at the start of every SpMM - unless the matrix
+    // is so small that the one more launch costs more than that (HPSPMM_ROW_TILES_PAD = 0 / 1 in
+    // the environment: never / whenever the length is not a multiple of 32, for comparisons).
+    // Below 32 columns the rows stay as they lie; a length that is not a multiple of 4 is then
+    // gathered with 16-byte loads at 4-byte alignment.
+    const char* pad_env = std::getenv("HPSPMM_ROW_TILES_PAD");
+    const bool pad = k % 32 != 0 && (pad_env ? std::atoi(pad_env) != 0
+                                             : (k > 32 && nnz >= kRowTilePadMinNnz && (k % 4 != 0 || nnz >= 40 * cols)));
+    p->rt_ldb = (uint32_t)(pad ? (k + 31) & ~(int64_t)31 : k);
+    p->rt_mode = pad ? 2 : k % 4 ? 3 : 1;
+    if (pad) {
+      const size_t pad_bytes = (size_t)std::max<int64_t>(cols, 1) * (size_t)p->rt_ldb * sizeof(float);
+      if (hipMalloc(&p->d_bpad, pad_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        p->d_bpad = nullptr;
+        return fail(HPSPMM_ERR_ALLOC, "device allocation of %zu bytes for the padded copy of B failed", pad_bytes);
+      }
+      p->workspace_bytes += (int64_t)pad_bytes;
     }
   }
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && !(flags & HPSPMM_PLAN_NO_HUB_CACHE) && nnz > 0) {
@@ -2411,6 +2475,18 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
       case 32: rc = launch_segments<32>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;
       case 64: rc = launch_segments<64>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;
       default: rc = launch_segments<128>(plan, d_rowptr, d_col, d_val, d_B, d_C, st); break;
+    }
+  } else if (plan->d_tent && plan->rt_mode) {
+    const uint32_t ldb = plan->rt_ldb, ldc = (uint32_t)plan->k;
+    if (plan->rt_mode == 2) {
+      hipLaunchKernelGGL(hpspmm::pad_rows_kernel, dim3(grid_for(plan->cols * (int64_t)ldb, 1 << 16)),
+                         dim3(hpspmm::kBlock), 0, st, plan->cols, plan->k, (int64_t)ldb, d_B, plan->d_bpad);
+      mark_launch(st, "pad_rows_kernel");
+      rc = launch_row_tiles<0, 2>(plan, d_val, plan->d_bpad, d_C, st, ldb, ldc);
+    } else if (plan->rt_mode == 3) {
+      rc = launch_row_tiles<0, 3>(plan, d_val, d_B, d_C, st, ldb, ldc);
+    } else {
+      rc = launch_row_tiles<0, 1>(plan, d_val, d_B, d_C, st, ldb, ldc);
     }
   } else if (plan->d_tent) {
     switch (plan->k) {

@@ -35,6 +35,10 @@
 // tiles itself, with 16 or 32 loads in flight per lane, is slower (20k-vertex
 // citation graph, K=128: 5.7 us with one, 6.4 with two, 8.2 with four).
 //
+// Row lengths other than 32 / 64 / 128 run the same kernels with the lengths
+// as arguments (see TileColumns): ceil(K / 32) column tiles, the last one
+// narrower, B as it lies or as a copy with padded rows.
+//
 // What this replaces in the reference: the row-per-warp kernels
 // topoCacheSPMMKernel / topoCacheCoarsenSPMMKernel (spmm/mm/spmm_kernel.cu:247-370).
 #pragma once
@@ -171,14 +175,75 @@ __global__ __launch_bounds__(kBlock) void rowtile_fill_kernel(RowTileLayout lay,
   tent[i] = rec;
 }
 
+// Where a lane's four columns lie in a launch over 32-column tiles.  K > 0: rows of B and C of K
+// floats, K a multiple of 32, everything a constant.  K == 0: the row lengths come with the launch
+// (ldb floats between the rows of B, ldc between those of C = the columns there are), the last
+// column tile may be narrower than 32, and the lanes beyond it gather what lane 0 gathers (no
+// branch around the loads) and store nothing.
+//   kLd = 1: ldb = ldc, a multiple of 4: every lane that stores owns four aligned floats.
+//   kLd = 2: ldb >= ldc, ldb a multiple of 4 (B is a copy with padded rows); C's rows of any length.
+//   kLd = 3: ldb = ldc, any number from 4 up; B is gathered with 16-byte loads at 4-byte alignment,
+//            and the lane that owns the last nv < 4 columns of a row gathers the row's last four
+//            floats instead (so that it reads nothing beyond the row) and finds its columns in
+//            the last nv components of its sums.
+struct TileColumns {
+  uint32_t ldb;  // floats between the rows of B
+  uint32_t ldc;  // ... of C
+  int k0;        // first column of the tile
+  int lb;        // this lane's offset into the tile when it gathers (kLd = 3: may be as low as -3)
+  int nv;        // how many of this lane's four columns exist in C (0 ... 4)
+  bool aligned;  // C's rows start at multiples of 16 bytes
+};
+template <int K, int kLd>
+__device__ __forceinline__ TileColumns tile_columns(uint32_t ldb, uint32_t ldc, int tile, int l) {
+  TileColumns tc;
+  tc.k0 = tile * 32;
+  if constexpr (kLd == 0) {
+    tc.ldb = tc.ldc = (uint32_t)K;
+    tc.lb = 4 * l;
+    tc.nv = 4;
+    tc.aligned = true;
+  } else {
+    tc.ldb = ldb;
+    tc.ldc = ldc;
+    tc.aligned = kLd == 1 || (kLd == 2 && ldc % 4 == 0);
+    const int left = (int)ldc - (tc.k0 + 4 * l);
+    tc.nv = left < 0 ? 0 : left > 4 ? 4 : left;
+    if constexpr (kLd == 3) tc.lb = left >= 4 ? 4 * l : (int)ldb - 4 - tc.k0;  // (also a lane beyond the row: in bounds)
+    else tc.lb = left > 0 ? 4 * l : 0;
+  }
+  return tc;
+}
+// Column tiles of a launch.
+template <int K, int kLd>
+__device__ __forceinline__ int column_tiles(uint32_t ldc) {
+  return kLd ? (int)((ldc + 31u) / 32u) : K / 32;
+}
+// A lane's part of a row of C.
+template <int kLd>
+__device__ __forceinline__ void store_tile_row(float* __restrict__ C, int32_t row, int l, const TileColumns& tc,
+                                               const float4& v) {
+  float* p = C + (uint64_t)(uint32_t)row * tc.ldc + tc.k0 + 4 * l;
+  if constexpr (kLd == 0) {
+    store_result(p, v);
+  } else if constexpr (kLd == 3) {
+    // the lane of a row's last nv < 4 columns has gathered the row's last four floats
+    const float4 r = tc.nv == 3 ? make_float4(v.y, v.z, v.w, 0.f) : tc.nv == 2 ? make_float4(v.z, v.w, 0.f, 0.f)
+                   : tc.nv == 1 ? make_float4(v.w, 0.f, 0.f, 0.f) : v;
+    if (tc.nv > 0) store_c_row<2, true>(p, r, tc.nv, false);
+  } else if (tc.nv > 0) {
+    store_c_row<kLd, true>(p, v, tc.nv, tc.aligned);
+  }
+}
+
 // acc += the first N products of the slot whose columns are staged in s_col; `c` is this lane's
-// own column, `v` its value (load already issued), `zrow` = 32 zeros in device memory.  Nothing in
+// own column, `v` its value (load already issued), `zrow` = 32 zeros in device memory, 4 more in front of them.  Nothing in
 // here is conditional: a padding entry among the first N gathers the zero row instead of a row of
 // B (so that a non-finite value in an unreferenced row of B cannot leak in).  With `if (c >= 0)`
 // around the gathers the compiler copied a loaded register inside the batch and waited for it
 // there - one more dependent round trip in a kernel that is nothing but round trips.
-template <int K, int N>
-__device__ __forceinline__ void gather_n(float4& acc, int32_t c, float v, int tid, int base, int l, int k0,
+template <int N, bool kUnaligned>
+__device__ __forceinline__ void gather_n(float4& acc, int32_t c, float v, int tid, int base, const TileColumns& tc,
                                          const int32_t* s_col, float* s_val, const float* __restrict__ B,
                                          const float* __restrict__ zrow) {
   int32_t cc[N];
@@ -187,8 +252,13 @@ __device__ __forceinline__ void gather_n(float4& acc, int32_t c, float v, int ti
   for (int i = 0; i < N; ++i) cc[i] = s_col[base + i];
 #pragma unroll
   for (int i = 0; i < N; ++i) {
-    const float* src = cc[i] >= 0 ? B + (uint64_t)(uint32_t)cc[i] * (uint64_t)K + (uint32_t)k0 : zrow;
-    b[i] = *reinterpret_cast<const float4*>(src + 4 * l);
+    const float* src = cc[i] >= 0 ? B + (uint64_t)(uint32_t)cc[i] * (uint64_t)tc.ldb + (uint32_t)tc.k0 : zrow;
+    if constexpr (kUnaligned) {
+      const Float4Unaligned u = *reinterpret_cast<const Float4Unaligned*>(src + tc.lb);
+      b[i] = make_float4(u.x, u.y, u.z, u.w);
+    } else {
+      b[i] = *reinterpret_cast<const float4*>(src + tc.lb);
+    }
   }
   s_val[tid] = c >= 0 ? v : 0.f;
   wave_lds_fence();
@@ -207,9 +277,9 @@ struct TileInfo {
 // Stages the tile's records (e = this lane's) in LDS, issues the load of this lane's value
 // (unconditionally: a padding entry reads val[0] and discards it) and gathers `depth` entries per
 // slot; depth < 0 = take the tile's own.
-template <int K>
-__device__ __forceinline__ TileInfo gather_tile(float4& acc, int2 e, int depth, int tid, int base, int l, int k0,
-                                                int32_t* s_col, int32_t* s_x, float* s_val,
+template <bool kUnaligned>
+__device__ __forceinline__ TileInfo gather_tile(float4& acc, int2 e, int depth, int tid, int base, int l,
+                                                const TileColumns& tc, int32_t* s_col, int32_t* s_x, float* s_val,
                                                 const float* __restrict__ val, const float* __restrict__ B,
                                                 const float* __restrict__ zrow) {
   s_col[tid] = e.x;
@@ -223,23 +293,24 @@ __device__ __forceinline__ TileInfo gather_tile(float4& acc, int2 e, int depth, 
   const float v = val[e.x >= 0 ? s_x[base + 1] + l : 0];
   switch (info.depth) {
     case 0: wave_lds_fence(); break;
-    case 1: gather_n<K, 1>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    case 2: gather_n<K, 2>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    case 3: gather_n<K, 3>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    case 4: gather_n<K, 4>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    case 5: gather_n<K, 5>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    case 6: gather_n<K, 6>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    case 7: gather_n<K, 7>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
-    default: gather_n<K, 8>(acc, e.x, v, tid, base, l, k0, s_col, s_val, B, zrow); break;
+    case 1: gather_n<1, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 2: gather_n<2, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 3: gather_n<3, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 4: gather_n<4, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 5: gather_n<5, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 6: gather_n<6, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 7: gather_n<7, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    default: gather_n<8, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
   }
   return info;
 }
 
 // acc += the products of tiles [t0, t1) (t0 < t1) of one long row, worked through by one
 // wavefront; returns the row.
-template <int K>
+template <bool kUnaligned>
 __device__ __forceinline__ int32_t gather_tiles(float4& acc, int32_t t0, int32_t t1, int lane, int l, int tid,
-                                                int base, int k0, int32_t* s_col, int32_t* s_x, float* s_val,
+                                                int base, const TileColumns& tc, int32_t* s_col, int32_t* s_x,
+                                                float* s_val,
                                                 const int2* __restrict__ tent, const float* __restrict__ val,
                                                 const float* __restrict__ B, const float* __restrict__ zrow) {
   int2 e = tent[(int64_t)t0 * kRowTile + lane];
@@ -247,15 +318,15 @@ __device__ __forceinline__ int32_t gather_tiles(float4& acc, int32_t t0, int32_t
   for (int32_t t = t0; t < t1; ++t) {
     const int2 e_now = e;
     if (t + 1 < t1) e = tent[(int64_t)(t + 1) * kRowTile + lane];  // on its way while this tile is gathered
-    row = gather_tile<K>(acc, e_now, kSlot, tid, base, l, k0, s_col, s_x, s_val, val, B, zrow).row;
+    row = gather_tile<kUnaligned>(acc, e_now, kSlot, tid, base, l, tc, s_col, s_x, s_val, val, B, zrow).row;
   }
   return row;
 }
 
 // Sum over the 2^lg adjacent slots of a row (xor shuffles, in a fixed order), then the row's
 // first slot stores.
-template <int K>
-__device__ __forceinline__ void reduce_and_store(float4 acc, int lg, int32_t row, int s, int l, int k0,
+template <int kLd>
+__device__ __forceinline__ void reduce_and_store(float4 acc, int lg, int32_t row, int s, int l, const TileColumns& tc,
                                                  float* __restrict__ C) {
 #pragma unroll
   for (int step = 0; step < 3; ++step) {
@@ -266,19 +337,20 @@ __device__ __forceinline__ void reduce_and_store(float4 acc, int lg, int32_t row
       acc.w += __shfl_xor(acc.w, kSlot << step);
     }
   }
-  if ((s & ((1 << lg) - 1)) == 0 && row >= 0) store_result(C + (uint64_t)(uint32_t)row * K + k0 + 4 * l, acc);
+  if ((s & ((1 << lg) - 1)) == 0 && row >= 0) store_tile_row<kLd>(C, row, l, tc, acc);
 }
 
 // Wavefront w < n_loop works through the tiles of long row w (ldesc[w] = first
 // tile, tile count); wavefront w >= n_loop owns tile loop_tiles + (w - n_loop).
-template <int K, int WPB>
+template <int K, int WPB, int kLd = 0>
 __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves, int32_t n_loop, int32_t loop_tiles,
                                                                const int2* __restrict__ ldesc,
                                                                const int2* __restrict__ tent,
                                                                const float* __restrict__ val,
                                                                const float* __restrict__ B, float* __restrict__ C,
-                                                               const float* __restrict__ zrow) {
-  constexpr int T = K / 32;
+                                                               const float* __restrict__ zrow, uint32_t ldb,
+                                                               uint32_t ldc) {
+  const int T = column_tiles<K, kLd>(ldc);
   __shared__ int32_t s_col[WPB * 64];
   __shared__ int32_t s_x[WPB * 64];
   __shared__ float s_val[WPB * 64];
@@ -288,7 +360,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
   const int l = lane & (kSlot - 1);
   const int s = lane / kSlot;
   const int base = tid - l;
-  const int k0 = (int)(blockIdx.x % T) * 32;
+  const TileColumns tc = tile_columns<K, kLd>(ldb, ldc, (int)(blockIdx.x % T), l);
   const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(blockIdx.x / T) * WPB + (tid >> 6));
   if (w >= n_waves) return;
 
@@ -296,13 +368,13 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
   if (w >= n_loop) {
     const int32_t tile = loop_tiles + (w - n_loop);
     const int2 e = tent[(int64_t)tile * kRowTile + lane];
-    const TileInfo info = gather_tile<K>(acc, e, -1, tid, base, l, k0, s_col, s_x, s_val, val, B, zrow);
-    reduce_and_store<K>(acc, info.lg, info.row, s, l, k0, C);
+    const TileInfo info = gather_tile<kLd == 3>(acc, e, -1, tid, base, l, tc, s_col, s_x, s_val, val, B, zrow);
+    reduce_and_store<kLd>(acc, info.lg, info.row, s, l, tc, C);
   } else {
     const int2 ld = ldesc[w];
-    const int32_t row = gather_tiles<K>(acc, ld.x, ld.x + ld.y, lane, l, tid, base, k0, s_col, s_x, s_val, tent, val,
+    const int32_t row = gather_tiles<kLd == 3>(acc, ld.x, ld.x + ld.y, lane, l, tid, base, tc, s_col, s_x, s_val, tent, val,
                                         B, zrow);
-    reduce_and_store<K>(acc, 3, row, s, l, k0, C);
+    reduce_and_store<kLd>(acc, 3, row, s, l, tc, C);
   }
 }
 
@@ -311,7 +383,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
 // shares, the shares' sums added in wavefront order through LDS), for matrices whose longest rows
 // would otherwise be the critical path of the launch.  The wavefronts of the other workgroups take
 // one remaining long row or one ordinary tile each, as above.
-template <int K, int WPB>
+template <int K, int WPB, int kLd = 0>
 __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_tiles, int32_t n_wg, int32_t n_loop,
                                                                     int32_t loop_tiles,
                                                                     const int2* __restrict__ ldesc,
@@ -319,8 +391,9 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
                                                                     const float* __restrict__ val,
                                                                     const float* __restrict__ B,
                                                                     float* __restrict__ C,
-                                                                    const float* __restrict__ zrow) {
-  constexpr int T = K / 32;
+                                                                    const float* __restrict__ zrow,
+                                                                    uint32_t ldb, uint32_t ldc) {
+  const int T = column_tiles<K, kLd>(ldc);
   __shared__ int32_t s_col[WPB * 64];
   __shared__ int32_t s_x[WPB * 64];
   __shared__ float s_val[WPB * 64];
@@ -332,7 +405,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
   const int l = lane & (kSlot - 1);
   const int s = lane / kSlot;
   const int base = tid - l;
-  const int k0 = (int)(blockIdx.x % T) * 32;
+  const TileColumns tc = tile_columns<K, kLd>(ldb, ldc, (int)(blockIdx.x % T), l);
   const int32_t blk = (int32_t)(blockIdx.x / T);
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 
@@ -342,7 +415,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
     const int32_t t0 = ld.x + wave * per;
     const int32_t t1 = t0 + per < ld.x + ld.y ? t0 + per : ld.x + ld.y;
     int32_t row = -1;  // wavefront 0 always has tiles, the later ones may not
-    if (t0 < t1) row = gather_tiles<K>(acc, t0, t1, lane, l, tid, base, k0, s_col, s_x, s_val, tent, val, B, zrow);
+    if (t0 < t1) row = gather_tiles<kLd == 3>(acc, t0, t1, lane, l, tid, base, tc, s_col, s_x, s_val, tent, val, B, zrow);
 #pragma unroll
     for (int off = kSlot; off < 64; off <<= 1) {
       acc.x += __shfl_xor(acc.x, off);
@@ -361,7 +434,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
         sum.z += p.z;
         sum.w += p.w;
       }
-      store_result(C + (uint64_t)(uint32_t)row * K + k0 + 4 * l, sum);
+      store_tile_row<kLd>(C, row, l, tc, sum);
     }
     return;
   }
@@ -369,15 +442,15 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
   const int32_t w = __builtin_amdgcn_readfirstlane(n_wg + (blk - n_wg) * WPB + wave);
   if (w < n_loop) {
     const int2 ld = ldesc[w];
-    const int32_t row = gather_tiles<K>(acc, ld.x, ld.x + ld.y, lane, l, tid, base, k0, s_col, s_x, s_val, tent, val,
+    const int32_t row = gather_tiles<kLd == 3>(acc, ld.x, ld.x + ld.y, lane, l, tid, base, tc, s_col, s_x, s_val, tent, val,
                                         B, zrow);
-    reduce_and_store<K>(acc, 3, row, s, l, k0, C);
+    reduce_and_store<kLd>(acc, 3, row, s, l, tc, C);
   } else {
     const int32_t tile = loop_tiles + (w - n_loop);
     if (tile >= n_tiles) return;
     const int2 e = tent[(int64_t)tile * kRowTile + lane];
-    const TileInfo info = gather_tile<K>(acc, e, -1, tid, base, l, k0, s_col, s_x, s_val, val, B, zrow);
-    reduce_and_store<K>(acc, info.lg, info.row, s, l, k0, C);
+    const TileInfo info = gather_tile<kLd == 3>(acc, e, -1, tid, base, l, tc, s_col, s_x, s_val, val, B, zrow);
+    reduce_and_store<kLd>(acc, info.lg, info.row, s, l, tc, C);
   }
 }
 

@@ -117,6 +117,11 @@ __device__ __forceinline__ void store_c_row(float* __restrict__ p, const float4&
     if (nv > 3) p[3] = v.w;
   }
 }
+// Four floats at a 4-byte aligned address.
+struct __attribute__((packed, aligned(4))) Float4Unaligned {
+  float x, y, z, w;
+};
+
 __device__ __forceinline__ float4 load_b_ld(const float* __restrict__ B, int32_t c, int l, uint32_t ld) {
   return *reinterpret_cast<const float4*>(B + (uint64_t)(uint32_t)c * (uint64_t)ld + (uint32_t)(4 * l));
 }

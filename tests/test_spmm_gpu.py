@@ -186,17 +186,22 @@ def test_linearity_and_column_tiles(pkg, oracle, gpu):
 @pytest.mark.parametrize("k", [1, 2, 3, 5, 7, 30, 41, 47, 50, 127, 129, 130, 173, 259])
 def test_k_not_a_multiple_of_four(pkg, oracle, gpu, k):
     """Row lengths that are not a multiple of 4 (rows of B and C start at any multiple of 4 bytes; the
-    number of classes of a node classifier is such a K): the same planned sub-wave strategies as for
-    the multiples of 4, the lane that owns the last columns of a row reading and writing only those
-    that exist.  Whole rows, forced segments (three lengths), the plan-less entry point; C poisoned
-    with NaN beforehand and laid out with guard rows, which must stay untouched."""
+    number of classes of a node classifier is such a K): whole rows over row tiles (K >= 4: 16-byte
+    gathers at 4-byte alignment) and over the CSR arrays, forced segments (three lengths) and the
+    plan-less entry point with the run-time-K sub-wave kernels, the lane that owns the last columns
+    of a row reading and writing only those that exist.  C poisoned with NaN beforehand and laid out
+    with guard rows, which must stay untouched."""
     import torch
     capi = pkg.capi
     g = pkg.graphs.make_graph("c4_rmat", 0.004)
     B = pkg.graphs.dense_normal(g.cols, k, 77)
     C, info = _run(pkg, gpu, g, B)
     assert info["strategy"] == capi.STRATEGY_ROWS and info["launches_per_spmm"] == 1, info
+    assert (info["row_tiles"] > 0) == (k >= 4), info
     _check(oracle, g, B, C, f"rows k={k}")
+    C, info = _run(pkg, gpu, g, B, capi.PLAN_NO_ROW_TILES)
+    assert info["strategy"] == capi.STRATEGY_ROWS and info["row_tiles"] == 0, info
+    _check(oracle, g, B, C, f"rows over the CSR arrays k={k}")
     for shift in (0, 3, 7):
         C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(shift))
         assert info["strategy"] == capi.STRATEGY_SEGMENTS and info["launches_per_spmm"] == 2, info
@@ -211,7 +216,7 @@ def test_k_not_a_multiple_of_four(pkg, oracle, gpu, k):
     Bbig[:g.cols * k] = torch.from_numpy(B).to(gpu).reshape(-1)
     Cbig = torch.full((g.rows * k + pad,), 12345.0, device=gpu)
     Bd, Cd = Bbig[:g.cols * k].view(g.cols, k), Cbig[:g.rows * k].view(g.rows, k)
-    for flags in (capi.PLAN_DEFAULT, capi.PLAN_FORCE_SEGMENTS):
+    for flags in (capi.PLAN_DEFAULT, capi.PLAN_NO_ROW_TILES, capi.PLAN_FORCE_SEGMENTS):
         Cd.fill_(float("nan"))
         plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
         capi.csr_spmm(plan, rp, ci, v, Bd, Cd)
@@ -226,17 +231,21 @@ def test_k_not_a_multiple_of_four(pkg, oracle, gpu, k):
 
 @pytest.mark.parametrize("k", [4, 8, 12, 16, 20, 24, 48, 96, 100, 160, 200, 256, 384])
 def test_multiple_of_four_k(pkg, oracle, gpu, k):
-    """Every multiple of 4 besides the tuned sizes goes through the planned sub-wave strategies
-    (the reference has a kernel of its own for K < 32, spmm_kernel.cu:372-387, 406-410): whole rows on a
-    small matrix - with hub rows on a wavefront each -, segments when forced or on a large one, and the
-    plan-less entry point; C poisoned with NaN beforehand, empty rows exact zeros."""
+    """Every multiple of 4 besides the tuned sizes (the reference has a kernel of its own for K < 32,
+    spmm_kernel.cu:372-387, 406-410): whole rows on a small matrix - over row tiles in 32-column tiles,
+    the last one narrower, or over the CSR arrays with hub rows on a wavefront each -, the run-time-K
+    segments kernels when forced, and the plan-less entry point; C poisoned with NaN beforehand, empty
+    rows exact zeros."""
     import torch
     capi = pkg.capi
     g = pkg.graphs.make_graph("c4_rmat", 0.004)  # hub rows of thousands of nonzeros, 40 % empty rows
     B = pkg.graphs.dense_normal(g.cols, k, 78)
     C, info = _run(pkg, gpu, g, B)
-    assert info["strategy"] == capi.STRATEGY_ROWS and info["launches_per_spmm"] == 1, info
+    assert info["strategy"] == capi.STRATEGY_ROWS and info["launches_per_spmm"] == 1 and info["row_tiles"] > 0, info
     _check(oracle, g, B, C, f"rows k={k}")
+    C, info = _run(pkg, gpu, g, B, capi.PLAN_NO_ROW_TILES)
+    assert info["strategy"] == capi.STRATEGY_ROWS and info["row_tiles"] == 0, info
+    _check(oracle, g, B, C, f"rows over the CSR arrays k={k}")
     for shift in (0, 3, 7):
         C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SEGMENTS | capi.plan_segment_shift(shift))
         assert info["strategy"] == capi.STRATEGY_SEGMENTS and info["launches_per_spmm"] == 2, info
@@ -252,16 +261,17 @@ def test_multiple_of_four_k(pkg, oracle, gpu, k):
 
 @pytest.mark.parametrize("k", [16, 41, 96])
 def test_multiple_of_four_k_large_graph(pkg, oracle, gpu, k):
-    """Beyond 2^21 nonzeros the plan picks segments for these K by itself - or, from K = 16 on a
-    matrix of 2^22 nonzeros and more, one of the tuned layouts in column tiles."""
+    """Beyond 2^21 nonzeros the plan picks whole rows over row tiles for these K by itself - or, from
+    K = 16 on a matrix of 2^22 nonzeros and more, one of the tuned layouts in column tiles."""
     capi = pkg.capi
     g = pkg.graphs.make_graph("c2_social", 0.05)
     assert g.nnz > 1 << 21
     B = pkg.graphs.dense_normal(g.cols, k, 79)
     C, info = _run(pkg, gpu, g, B)
     tiled = (capi.STRATEGY_SWEEP, capi.STRATEGY_ROUTED, capi.STRATEGY_ORDERED)
-    assert info["strategy"] == capi.STRATEGY_SEGMENTS or (k >= 16 and info["strategy"] in tiled), info
-    _check(oracle, g, B, C, f"auto segments k={k}")
+    assert (info["strategy"] == capi.STRATEGY_ROWS and info["row_tiles"] > 0) or \
+        (k >= 16 and info["strategy"] in tiled), info
+    _check(oracle, g, B, C, f"auto k={k}")
 
 
 def test_edge_shapes(pkg, oracle, gpu):
@@ -322,6 +332,18 @@ def test_fill(pkg, gpu):
     assert torch.all(x == -2.5).item()
 
 
+def _check_accumulated(got, C0, C64, S64, calls, what):
+    """C0 + calls * (A B) within calls * TOL * (sum |a||b| + |C0|); a failure names the worst element."""
+    err = np.abs(got.astype(np.float64) - (C0 + calls * C64))
+    bound = calls * TOL * (S64 + np.abs(C0))
+    bad = ~(err <= bound)  # (also catches NaN)
+    if bad.any():
+        i, j = np.unravel_index(np.argmax(np.where(bad, err - bound, -np.inf)), err.shape)
+        raise AssertionError(f"{what}: {int(bad.sum())} elements out of tolerance in {len(np.unique(np.nonzero(bad)[0]))} "
+                             f"rows; worst at ({i}, {j}): got {got[i, j]!r}, expected {C0[i, j] + calls * C64[i, j]!r}, "
+                             f"C0 {C0[i, j]!r}, bound {bound[i, j]:.3e}")
+
+
 @pytest.mark.parametrize("k", [32, 64, 128, 24, 16, 96, 200, 7, 41, 173])
 def test_coo_accumulate(pkg, oracle, gpu, k):
     """The LBSpMM contract: C += A B, padded zero entries, rows in permuted order."""
@@ -343,13 +365,13 @@ def test_coo_accumulate(pkg, oracle, gpu, k):
     torch.cuda.synchronize()
     C64, S64 = oracle.csr_spmm_f64(g.rowptr, g.col, g.val, B)
     got = C.cpu().numpy()
-    assert np.all(np.abs(got.astype(np.float64) - (C0 + C64)) <= TOL * (S64 + np.abs(C0)))
+    _check_accumulated(got, C0, C64, S64, 1, f"k={k}, first call")
     # twice more: accumulates (the reference runs it 200 times and divides)
     pkg.capi.coo_spmm_accumulate(g.rows, g.cols, r_, c_, v_, Bd, C)
     pkg.capi.coo_spmm_accumulate(g.rows, g.cols, r_, c_, v_, Bd, C)
     torch.cuda.synchronize()
     got = C.cpu().numpy()
-    assert np.all(np.abs(got.astype(np.float64) - (C0 + 3 * C64)) <= 3 * TOL * (S64 + np.abs(C0)))
+    _check_accumulated(got, C0, C64, S64, 3, f"k={k}, three calls")
 
 
 def test_error_codes(pkg, gpu):
@@ -882,6 +904,63 @@ def test_row_tiles_layout_and_fallback(pkg, oracle, gpu):
     C, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
     assert info["strategy"] == capi.STRATEGY_ROWS and info["row_tiles"] == 0
     _check(oracle, g, B, C, "mostly empty rows")
+
+
+@pytest.mark.parametrize("k", [4, 5, 7, 20, 31, 33, 36, 41, 63, 65, 100, 130, 172, 259])
+def test_row_tiles_at_any_row_length(pkg, oracle, gpu, monkeypatch, k):
+    """Row tiles at a row length outside the tuned set: 32-column tiles, the last one narrower; B as it
+    lies (K a multiple of 4: aligned gathers; else 16-byte gathers at 4-byte alignment, the lane of a
+    row's last columns reading the row's last four floats) or through the plan's copy with rows padded
+    to a multiple of 32 floats (one more launch).  Every size class of row, rows that get a whole
+    workgroup, empty rows; B and C inside larger allocations whose surroundings hold NaN (B) and a
+    marker (C): nothing beyond them may be read into the result or written.  Both forms give the same
+    bits (the same gathers in the same order), and two runs of one form do."""
+    import torch
+    capi = pkg.capi
+    rng = np.random.default_rng(100 + k)
+    cols = 3000
+    lens = rng.permutation(np.concatenate([np.arange(0, 140), np.arange(0, 520, 11), [513, 700, 1500, 9000],
+                                           np.zeros(40, np.int64)])).astype(np.int64)
+    rows = lens.size
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = rng.integers(0, cols, int(lens.sum())).astype(np.int32)
+    col[-3:] = cols - 1  # the last row of B is gathered: a read past its end would reach the NaN behind it
+    val = rng.uniform(-1, 1, col.size).astype(np.float32)
+    g = pkg.graphs.CSR(rows, cols, rowptr, col, val)
+    B = rng.standard_normal((cols, k)).astype(np.float32)
+    rp, ci, v = _to_dev(gpu, g.rowptr, g.col, g.val)
+    guard = 64
+    Bbig = torch.full((guard + cols * k + guard,), float("nan"), device=gpu)
+    Bbig[guard:guard + cols * k] = torch.from_numpy(B).to(gpu).reshape(-1)
+    Cbig = torch.full((guard + rows * k + guard,), 12345.0, device=gpu)
+    Bd, Cd = Bbig[guard:guard + cols * k].view(cols, k), Cbig[guard:guard + rows * k].view(rows, k)
+    results = {}
+    for form, env in (("as it lies", "0"), ("padded copy", "1")):
+        monkeypatch.setenv("HPSPMM_ROW_TILES_PAD", env)
+        plan = capi.Plan(rows, cols, rp, ci, k, capi.PLAN_DEFAULT)
+        info = plan.info
+        padded = env == "1" and k % 32 != 0
+        assert info["strategy"] == capi.STRATEGY_ROWS and info["row_tiles"] * 64 >= col.size, info
+        assert info["launches_per_spmm"] == (2 if padded else 1) and info["k"] == k, info
+        for attempt in range(2):
+            Cd.fill_(float("nan"))
+            capi.csr_spmm(plan, rp, ci, v, Bd, Cd)
+            torch.cuda.synchronize()
+            C = Cd.cpu().numpy().copy()
+            _check(oracle, g, B, C, f"k={k} {form}")
+            assert bool((Cbig[:guard] == 12345.0).all()) and bool((Cbig[guard + rows * k:] == 12345.0).all()), \
+                f"k={k} {form}: wrote outside C"
+            assert np.array_equal(results.setdefault(form, C), C), "bit-reproducible"
+        plan.destroy()
+    assert np.array_equal(results["as it lies"], results["padded copy"])
+    # no row beyond 512 nonzeros: one wavefront per row tile, in workgroups of one (small grid) or four
+    monkeypatch.delenv("HPSPMM_ROW_TILES_PAD")
+    for scale in (0.25, 4.0):
+        g = pkg.graphs.make_graph("c1_citation", scale)
+        B = pkg.graphs.dense_normal(g.cols, k, 5)
+        C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_ROWS)
+        assert info["strategy"] == capi.STRATEGY_ROWS and info["row_tiles"] > 0, info
+        _check(oracle, g, B, C, f"k={k} citation graph x {scale}")
 
 
 def test_auto_choice_at_mid_size(pkg, oracle, gpu):

@@ -82,13 +82,13 @@ inline int64_t tile_width(int64_t k) {
 // Not a multiple of 4: rows of B and C start at any multiple of 4 bytes, the last lane of a row owns 1 to 3 columns.
 inline bool odd_k(int64_t k) { return k % 4 != 0; }
 // Lanes per sub-wave for such a K: the power of two that covers a column tile (at most 128 floats).
-// Row tiles (32-column tiles of B and C) serve every row length from 4 up
-// (HPSPMM_ROW_TILES_MIN_K in the environment raises that, for comparisons).
+// Row tiles (32-column tiles of B and C) serve every row length
+// (HPSPMM_ROW_TILES_MIN_K in the environment: only from there up, for comparisons).
 inline bool row_tiles_serve(int64_t k) {
   if (fast_k(k)) return true;
-  if (k < 4 || k >= ((int64_t)1 << 22)) return false;
+  if (k >= ((int64_t)1 << 22)) return false;
   const char* e = std::getenv("HPSPMM_ROW_TILES_MIN_K");
-  return k >= (e ? (int64_t)std::atoll(e) : (int64_t)4);
+  return k >= (e ? (int64_t)std::atoll(e) : (int64_t)1);
 }
 
 inline int anyk_lanes(int64_t k) {
@@ -2077,9 +2077,11 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     // the rows kernel over the CSR arrays, whose sub-waves read whole rows of B; K = 256: 334
     // against 337), while a padded copy of B costs more than it saves.
     const bool few_per_row = mean_row <= 8.0;
-    const bool any_k_range = !few_per_row       ? nnz < kRowTileMaxNnz
-                             : k % 32 == 0      ? nnz < kRowsAutoMaxNnz && fits
-                                                : k <= 32 || (double)nnz * (double)k < kRowsAutoFewPerRowWork;
+    // (K < 4, which row tiles read through a padded copy of B: 1.6 M nonzeros, K = 1: 30 against 18 us.)
+    const bool any_k_range = !few_per_row  ? nnz < kRowTileMaxNnz
+                             : k % 32 == 0 ? nnz < kRowsAutoMaxNnz && fits
+                             : k < 4       ? nnz < kRowTilePadMinNnz
+                                           : k <= 32 || (double)nnz * (double)k < kRowsAutoFewPerRowWork;
     const bool in_range = fast_k(k) ? nnz < kRowsAutoMaxNnz && fits : any_k_range;
     const bool mid = in_range && p->max_row_nnz <= kRowsAutoMaxRow && !(flags & HPSPMM_PLAN_NO_ROW_TILES);
     if (nnz == 0 || tiny || (mid && nnz < kClusterMinNnz)) {
@@ -2176,11 +2178,13 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     // is so small that the one more launch costs more than that (HPSPMM_ROW_TILES_PAD = 0 / 1 in
     // the environment: never / whenever the length is not a multiple of 32, for comparisons).
     // Below 32 columns the rows stay as they lie; a length that is not a multiple of 4 is then
-    // gathered with 16-byte loads at 4-byte alignment.
+    // gathered with 16-byte loads at 4-byte alignment - except below 4 columns, where a row is
+    // shorter than one such load: the copy then has rows of 4 floats.
     const char* pad_env = std::getenv("HPSPMM_ROW_TILES_PAD");
-    const bool pad = k % 32 != 0 && (pad_env ? std::atoi(pad_env) != 0
-                                             : (k > 32 && nnz >= kRowTilePadMinNnz && (k % 4 != 0 || nnz >= 40 * cols)));
-    p->rt_ldb = (uint32_t)(pad ? (k + 31) & ~(int64_t)31 : k);
+    const bool pad = k < 4 || (k % 32 != 0 && (pad_env ? std::atoi(pad_env) != 0
+                                                       : (k > 32 && nnz >= kRowTilePadMinNnz &&
+                                                          (k % 4 != 0 || nnz >= 40 * cols))));
+    p->rt_ldb = (uint32_t)(k < 4 ? 4 : pad ? (k + 31) & ~(int64_t)31 : k);
     p->rt_mode = pad ? 2 : k % 4 ? 3 : 1;
     if (pad) {
       const size_t pad_bytes = (size_t)std::max<int64_t>(cols, 1) * (size_t)p->rt_ldb * sizeof(float);

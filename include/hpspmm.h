@@ -147,14 +147,15 @@ const char *hpspmm_last_error(void);
  * about twice; C is written in place.  All that is done when the matrix gets
  * one of those layouts (at least 2^22 nonzeros, or a forcing flag);
  * launches_per_spmm counts every tile's launches, column_tiles the tiles.
- * Otherwise a k from 4 up runs whole rows over the plan's row tiles in
- * ceil(k / 32) column tiles within one launch (column_tiles stays 1), B as it
- * lies - 16-byte gathers at 4-byte alignment when k is not a multiple of 4 -
- * or, on matrices of 2^19 nonzeros and more where that pays (k > 32 and not a
- * multiple of 4, or not a multiple of 32 with 40 nonzeros a row), through
- * such a copy with rows padded to a multiple of 32 floats.  What remains -
- * k < 4, rows beyond 2^16 nonzeros, very short rows at a k that is not a
- * multiple of 32 on a large matrix - runs whole rows or segments with
+ * Otherwise whole rows run over the plan's row tiles in ceil(k / 32) column
+ * tiles within one launch (column_tiles stays 1), B as it lies - 16-byte
+ * gathers at 4-byte alignment when k is not a multiple of 4 - or, on matrices
+ * of 2^19 nonzeros and more where that pays (k > 32 and not a multiple of 4,
+ * or not a multiple of 32 with 40 nonzeros a row), through such a copy with
+ * rows padded to a multiple of 32 floats; k < 4 always through a copy with
+ * rows of 4 floats.  What remains - rows beyond 2^16 nonzeros, very short
+ * rows at a k that is not a multiple of 32 on a large matrix - runs whole rows
+ * or segments with
  * sub-waves of ceil(k / 4) lanes rounded up to a power of two, rows of B and C
  * read and written at whatever alignment they have.
  * Replaces the host-side preprocessing the reference does before timing:

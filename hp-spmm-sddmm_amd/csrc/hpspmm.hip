@@ -310,7 +310,7 @@ constexpr int64_t kRowsAutoMaxWork = (int64_t)3 << 28;  // nnz * K, matrices of 
 constexpr double kRowsAutoLongMean = 128.0;             // mean nonzeros per non-empty row beyond which ...
 constexpr double kRowsAutoLongWork = 2.0e15;            // ... nnz^2 * K decides instead
 constexpr int64_t kRowsAutoMaxRow = 1 << 16;
-constexpr double kRowsAutoFewPerRowWork = 3.0e7;         // nnz * K, rows of <= 8 nonzeros, K not a multiple of 32
+constexpr int64_t kRowsAutoFewPerRowNnz = 1 << 22;      // rows of <= 8 nonzeros, K > 32 and not a multiple of 32
 constexpr int64_t kRowTilePadMinNnz = 1 << 19;  // row tiles: matrices from here up read a B of odd row length through a padded copy
 
 int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st);
@@ -327,14 +327,25 @@ inline int64_t row_tile_column_tiles(int k_template, uint32_t ldc) {
   return k_template ? k_template / 32 : (int64_t)((ldc + 31u) / 32u);
 }
 
+// The column tiles of a group of row tiles on one XCD: where the rows of B are not whole 128-byte
+// lines, so that neighbouring tiles share lines (citation graph x 16, 1.6 M nonzeros, K = 100: 245 us
+// with the tiles dealt round robin, 148 so; R-MAT 3.7 M nonzeros, K = 172: 392 -> 291).
+// HPSPMM_ROW_TILES_XCD = 0 in the environment: round robin, for comparisons.
+inline bool row_tiles_same_xcd(int kLd, uint32_t ldb) {
+  const char* e = std::getenv("HPSPMM_ROW_TILES_XCD");
+  return kLd != 0 && ldb % 32 != 0 && (e ? std::atoi(e) != 0 : true);
+}
+
 template <int K, int WPB, int kLd>
 int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st, uint32_t ldb,
                        uint32_t ldc) {
-  const int64_t blocks = ceil_div(p->rt_waves, WPB) * row_tile_column_tiles(K, ldc);
+  const bool same_xcd = row_tiles_same_xcd(kLd, ldb);
+  const int64_t groups = ceil_div(p->rt_waves, WPB);
+  const int64_t blocks = (same_xcd ? ceil_div(groups, 8) * 8 : groups) * row_tile_column_tiles(K, ldc);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB, kLd>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent, readable_values(p, v), B, C,
-                     p->d_zrow + 4, ldb, ldc);
+                     p->d_zrow + 4, ldb, ldc, same_xcd);
   mark_launch(st, "spmm_rowtiles_kernel");
   return HPSPMM_OK;
 }
@@ -343,11 +354,13 @@ template <int K, int WPB, int kLd>
 int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st, uint32_t ldb,
                         uint32_t ldc) {
   const int64_t wave_items = (p->rt_loop - p->rt_wg) + (p->rt_tiles - p->rt_loop_tiles);
-  const int64_t blocks = (p->rt_wg + ceil_div(wave_items, WPB)) * row_tile_column_tiles(K, ldc);
+  const bool same_xcd = row_tiles_same_xcd(kLd, ldb);
+  const int64_t groups = p->rt_wg + ceil_div(wave_items, WPB);
+  const int64_t blocks = (same_xcd ? ceil_div(groups, 8) * 8 : groups) * row_tile_column_tiles(K, ldc);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB, kLd>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent,
-                     readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc);
+                     readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc, same_xcd);
   mark_launch(st, "spmm_rowtiles_wg_kernel");
   return HPSPMM_OK;
 }
@@ -2070,18 +2083,18 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     // (A row length outside the tuned set, on a matrix that has not got one of the tiled layouts:
     // the alternative to row tiles is the run-time-K segments kernel, which they beat at every size
     // measured - R-MAT graph, 7.6 M nonzeros, K = 48: 206 against 817 us; 0.9 M, K = 96: 25 against 521.)
-    // The exception are matrices of few nonzeros per row whose B is far beyond the L2s: what decides
-    // there is the traffic, and at a row length that is not a multiple of 32 floats the 128-byte
-    // gathers of neighbouring column tiles - made by different workgroups - both fetch the line they
-    // share (citation graph at 16 times its size, 1.6 M nonzeros, K = 100: 246 us against 142 for
-    // the rows kernel over the CSR arrays, whose sub-waves read whole rows of B; K = 256: 334
-    // against 337), while a padded copy of B costs more than it saves.
+    // The exception are large matrices of few nonzeros per row, whose B is far beyond the L2s: what
+    // decides there is the traffic, every 128-byte gather of a row of B that is not a whole number
+    // of lines touches two, and the segments kernel, whose sub-waves read whole rows of B, is ahead
+    // (citation graph at 64 times its size, 6.5 M nonzeros, K = 100: 774 us against 542; K = 41: 496
+    // against 370; at 16 times, 1.6 M: 148 against 142 for the rows kernel over the CSR arrays,
+    // K = 172: 231 against 273), while a padded copy of B costs more than it saves.
     const bool few_per_row = mean_row <= 8.0;
     // (K < 4, which row tiles read through a padded copy of B: 1.6 M nonzeros, K = 1: 30 against 18 us.)
     const bool any_k_range = !few_per_row  ? nnz < kRowTileMaxNnz
                              : k % 32 == 0 ? nnz < kRowsAutoMaxNnz && fits
                              : k < 4       ? nnz < kRowTilePadMinNnz
-                                           : k <= 32 || (double)nnz * (double)k < kRowsAutoFewPerRowWork;
+                                           : k <= 32 || nnz < kRowsAutoFewPerRowNnz;
     const bool in_range = fast_k(k) ? nnz < kRowsAutoMaxNnz && fits : any_k_range;
     const bool mid = in_range && p->max_row_nnz <= kRowsAutoMaxRow && !(flags & HPSPMM_PLAN_NO_ROW_TILES);
     if (nnz == 0 || tiny || (mid && nnz < kClusterMinNnz)) {
@@ -2173,17 +2186,20 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
   if (p->d_tent && !fast_k(k)) {
     // Row tiles at a row length of its own.  The gathers are fastest when every 32-column tile of a
     // row of B is one aligned 128-byte line (R-MAT graph, 3.7 M nonzeros: K = 96 131 us, K = 100
-    // 204 us as it lies), so from 32 columns up a B whose rows are not a multiple of 32 floats is
-    // read through a copy with padded rows, refreshed at the start of every SpMM - unless the matrix
-    // is so small that the one more launch costs more than that (HPSPMM_ROW_TILES_PAD = 0 / 1 in
-    // the environment: never / whenever the length is not a multiple of 32, for comparisons).
-    // Below 32 columns the rows stay as they lie; a length that is not a multiple of 4 is then
-    // gathered with 16-byte loads at 4-byte alignment - except below 4 columns, where a row is
-    // shorter than one such load: the copy then has rows of 4 floats.
+    // 186 us as it lies).  A B whose rows do not even start at multiples of 32 bytes is therefore
+    // read through a copy with rows padded to a multiple of 32 floats, refreshed at the start of
+    // every SpMM, where that copy is cheap against the gathers - 40 nonzeros for every row of B,
+    // 2^20 in all (co-purchase graph, 2.5 M nonzeros, K = 100: 140 -> 118 us, K = 41: 77 -> 66;
+    // but K = 200: 267 -> 319, K = 48: 58 -> 64; R-MAT, 28 nonzeros a row, K = 172: 291 -> 342;
+    // co-purchase graph at 0.6 M nonzeros, K = 41: 16.5 -> 20.2).  HPSPMM_ROW_TILES_PAD = 0 / 1 in
+    // the environment: never / whenever the length is not a multiple of 32, for comparisons.
+    // Otherwise the rows stay as they lie; a length that is not a multiple of 4 is then gathered
+    // with 16-byte loads at 4-byte alignment - except below 4 columns, where a row is shorter than
+    // one such load: the copy then has rows of 4 floats.
     const char* pad_env = std::getenv("HPSPMM_ROW_TILES_PAD");
     const bool pad = k < 4 || (k % 32 != 0 && (pad_env ? std::atoi(pad_env) != 0
-                                                       : (k > 32 && nnz >= kRowTilePadMinNnz &&
-                                                          (k % 4 != 0 || nnz >= 40 * cols))));
+                                                       : (k > 32 && k % 8 != 0 && nnz >= 2 * kRowTilePadMinNnz &&
+                                                          nnz >= 40 * cols)));
     p->rt_ldb = (uint32_t)(k < 4 ? 4 : pad ? (k + 31) & ~(int64_t)31 : k);
     p->rt_mode = pad ? 2 : k % 4 ? 3 : 1;
     if (pad) {

@@ -219,6 +219,22 @@ template <int K, int kLd>
 __device__ __forceinline__ int column_tiles(uint32_t ldc) {
   return kLd ? (int)((ldc + 31u) / 32u) : K / 32;
 }
+// Which column tile and which group of row tiles workgroup b serves.  The tuned row lengths deal the
+// column tiles round robin (b % T: with T = 1, 2, 4 column tiles an XCD only ever touches one of
+// them).  same_xcd: the T tiles of a group go to workgroups b, b + 8, b + 16 ... - one XCD, one after
+// the other - for rows of B that are not a whole number of 128-byte lines: the line that two
+// neighbouring tiles share is then fetched into one L2 once instead of into two.
+template <int kLd>
+__device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, int& tile, int32_t& group) {
+  if (kLd != 0 && same_xcd) {
+    const uint32_t per = 8u * (uint32_t)T, r = b % per;
+    tile = (int)(r / 8u);
+    group = (int32_t)((b / per) * 8u + r % 8u);
+  } else {
+    tile = (int)(b % (uint32_t)T);
+    group = (int32_t)(b / (uint32_t)T);
+  }
+}
 // A lane's part of a row of C.
 template <int kLd>
 __device__ __forceinline__ void store_tile_row(float* __restrict__ C, int32_t row, int l, const TileColumns& tc,
@@ -349,7 +365,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
                                                                const float* __restrict__ val,
                                                                const float* __restrict__ B, float* __restrict__ C,
                                                                const float* __restrict__ zrow, uint32_t ldb,
-                                                               uint32_t ldc) {
+                                                               uint32_t ldc, bool same_xcd) {
   const int T = column_tiles<K, kLd>(ldc);
   __shared__ int32_t s_col[WPB * 64];
   __shared__ int32_t s_x[WPB * 64];
@@ -360,8 +376,11 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
   const int l = lane & (kSlot - 1);
   const int s = lane / kSlot;
   const int base = tid - l;
-  const TileColumns tc = tile_columns<K, kLd>(ldb, ldc, (int)(blockIdx.x % T), l);
-  const int32_t w = __builtin_amdgcn_readfirstlane((int32_t)(blockIdx.x / T) * WPB + (tid >> 6));
+  int ctile;
+  int32_t group;
+  tile_of_workgroup<kLd>(blockIdx.x, T, same_xcd, ctile, group);
+  const TileColumns tc = tile_columns<K, kLd>(ldb, ldc, ctile, l);
+  const int32_t w = __builtin_amdgcn_readfirstlane(group * WPB + (tid >> 6));
   if (w >= n_waves) return;
 
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -392,7 +411,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
                                                                     const float* __restrict__ B,
                                                                     float* __restrict__ C,
                                                                     const float* __restrict__ zrow,
-                                                                    uint32_t ldb, uint32_t ldc) {
+                                                                    uint32_t ldb, uint32_t ldc, bool same_xcd) {
   const int T = column_tiles<K, kLd>(ldc);
   __shared__ int32_t s_col[WPB * 64];
   __shared__ int32_t s_x[WPB * 64];
@@ -405,8 +424,10 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
   const int l = lane & (kSlot - 1);
   const int s = lane / kSlot;
   const int base = tid - l;
-  const TileColumns tc = tile_columns<K, kLd>(ldb, ldc, (int)(blockIdx.x % T), l);
-  const int32_t blk = (int32_t)(blockIdx.x / T);
+  int ctile;
+  int32_t blk;
+  tile_of_workgroup<kLd>(blockIdx.x, T, same_xcd, ctile, blk);
+  const TileColumns tc = tile_columns<K, kLd>(ldb, ldc, ctile, l);
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 
   if (blk < n_wg) {  // uniform over the workgroup: every wavefront reaches the barrier

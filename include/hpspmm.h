@@ -149,11 +149,10 @@ const char *hpspmm_last_error(void);
  * launches_per_spmm counts every tile's launches, column_tiles the tiles.
  * Otherwise whole rows run over the plan's row tiles in ceil(k / 32) column
  * tiles within one launch (column_tiles stays 1), B as it lies - 16-byte
- * gathers at 4-byte alignment when k is not a multiple of 4 - or, on matrices
- * of 2^19 nonzeros and more where that pays (k > 32 and not a multiple of 4,
- * or not a multiple of 32 with 40 nonzeros a row), through such a copy with
- * rows padded to a multiple of 32 floats; k < 4 always through a copy with
- * rows of 4 floats.  What remains - rows beyond 2^16 nonzeros, very short
+ * gathers at 4-byte alignment when k is not a multiple of 4 - or, where that
+ * pays (k > 32 and not a multiple of 8, 2^20 nonzeros and more, 40 for every
+ * row of B), through such a copy with rows padded to a multiple of 32 floats;
+ * k < 4 always through a copy with rows of 4 floats.  What remains - rows beyond 2^16 nonzeros, very short
  * rows at a k that is not a multiple of 32 on a large matrix - runs whole rows
  * or segments with
  * sub-waves of ceil(k / 4) lanes rounded up to a power of two, rows of B and C

@@ -701,13 +701,18 @@ def test_hip_graph_capture_and_replay(pkg, oracle, gpu):
     # length that is not a multiple of 4 (3 tiles of 64 columns behind a padded copy of B)
     tiled = [(n, f) for n, f in _strategies(capi) if n in ("sweep", "routed", "routed_sort_values", "cluster_seg")]
     operands = {}
-    for name, flags, k in [(n, f, 64) for n, f in _strategies(capi)] + [(n + "_tiled", f, 173) for n, f in tiled]:
+    # and row tiles at row lengths of their own: B as it lies (aligned, at 4-byte alignment), B through the padded copy
+    other = [("row_tiles_k100", capi.PLAN_DEFAULT, 100), ("row_tiles_k41", capi.PLAN_DEFAULT, 41),
+             ("row_tiles_k3", capi.PLAN_DEFAULT, 3)]
+    for name, flags, k in [(n, f, 64) for n, f in _strategies(capi)] + [(n + "_tiled", f, 173) for n, f in tiled] + other:
         if k not in operands:
             operands[k] = _to_dev(gpu, g.rowptr, g.col, g.val, pkg.graphs.make_dense("c4_rmat", g.cols, k))
         rp, ci, v, Bd = operands[k]
         plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
         if name.endswith("_tiled"):
             assert plan.info["column_tiles"] == 3, (name, plan.info)
+        if name.startswith("row_tiles"):
+            assert plan.info["row_tiles"] > 0 and plan.info["launches_per_spmm"] == (2 if k == 3 else 1), (name, plan.info)
         C = torch.full((g.rows, k), float("nan"), device=gpu)
         eager = torch.empty_like(C)
         capi.csr_spmm(plan, rp, ci, v, Bd, eager)

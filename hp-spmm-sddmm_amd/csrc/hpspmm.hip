@@ -450,8 +450,8 @@ int launch_coo_anyk_g(int64_t nnz, int64_t k, const int32_t* ri, const int32_t* 
                       float* C, hipStream_t st) {
   constexpr int P = 64 / GP;
   const int tiles = anyk_tiles(k);
-  int shift = 6;  // as launch_coo: 64 nonzeros per sub-wave, fewer while that leaves SIMDs idle
-  while (shift > 4 && (nnz >> shift) / P < 4096) --shift;
+  int shift = 4;  // as launch_coo: 16 nonzeros per sub-wave, doubled while that leaves 4096 wavefronts, up to 512
+  while (shift < 9 && (nnz >> (shift + 1)) / P >= 4096) ++shift;
   const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
   const int64_t blocks = ceil_div(ceil_div(nseg, P), hpspmm::kWavesPerBlock) * tiles;
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
@@ -554,11 +554,12 @@ template <int K>
 int launch_coo(int64_t nnz, const int32_t* ri, const int32_t* ci, const float* v, const float* B, float* C,
                hipStream_t st) {
   constexpr int P = 64 / (K / 4);
-  // 64 nonzeros per sub-wave: short enough to balance, long enough that the
-  // one flush per segment end is amortised; shorter segments when that would
-  // leave most of the 1024 SIMDs without a wavefront
-  int shift = 6;
-  while (shift > 4 && (nnz >> shift) / P < 4096) --shift;
+  // 16 nonzeros per sub-wave, and twice that as long as this leaves 4096 wavefronts, up to 512: the
+  // one flush per segment end is the better amortised the longer the segment, and every SIMD still
+  // has several wavefronts (social graph, K = 32: 2.16 ms at 64 nonzeros, 1.44 ms at 512; K = 128:
+  // 8.33 -> 7.06; R-MAT K = 128: 14.3 -> 13.3; the 20k-vertex citation graph stays at 16)
+  int shift = 4;
+  while (shift < 9 && (nnz >> (shift + 1)) / P >= 4096) ++shift;
   const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
   const int64_t nblocks = ceil_div(ceil_div(nseg, P), hpspmm::kWavesPerBlock);
   if (nblocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");

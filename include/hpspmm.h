@@ -227,6 +227,9 @@ int hpspmm_plan_bind_values(hpspmm_plan *plan, const float *d_val, void *stream)
  * address is HPSPMM_ERR_INVALID_ARG (the reference's launchers take whatever
  * they are given, spmm/mm/spmm_kernel.cu:389-426, and have no plan that could
  * go stale), unless the plan was created with HPSPMM_PLAN_ALLOW_MOVED_CSR.
+ * All arrays may start at any multiple of 4 bytes; the kernels are tuned for
+ * d_B and d_C at multiples of 16 bytes (what hipMalloc returns), other
+ * addresses give the same result more slowly.
  */
 int hpspmm_csr_spmm(hpspmm_plan *plan, const int32_t *d_rowptr, const int32_t *d_col,
                     const float *d_val, const float *d_B, float *d_C, void *stream);

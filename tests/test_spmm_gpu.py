@@ -656,6 +656,13 @@ def test_unaligned_arrays_and_new_values_per_call(pkg, oracle, gpu):
             _check(oracle, g, B, C.cpu().numpy(), f"unaligned k={k} {name}")
             capi.csr_spmm(plan, rp, ci, v2, Bd, C)
             _check(oracle, g2, B, C.cpu().numpy(), f"unaligned, new values k={k} {name}")
+            # B and C one float into their buffers as well: the 16-byte accesses of the kernels are then
+            # misaligned, which the hardware serves (more slowly); the result must not change
+            Bu = torch.cat([torch.zeros(1, device=gpu), Bd.reshape(-1)])[1:].view(g.cols, k)
+            Cu = torch.full((g.rows * k + 1,), float("nan"), device=gpu)[1:].view(g.rows, k)
+            assert Bu.data_ptr() % 16 == 4 and Cu.data_ptr() % 16 == 4
+            capi.csr_spmm(plan, rp, ci, v2, Bu, Cu)
+            assert torch.equal(Cu, C), f"B and C at 4-byte alignment k={k} {name}"
             plan.destroy()
 
 

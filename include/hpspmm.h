@@ -238,6 +238,10 @@ int hpspmm_csr_spmm(hpspmm_plan *plan, const int32_t *d_rowptr, const int32_t *d
  * C = A * B without a plan: whole-row kernel, no preprocessing, no device
  * allocation.  Same contract as GESpMM's single launch
  * (spmm/mm/spmm_kernel.cu:406-421), for callers that cannot keep a plan.
+ * As there, a row is served by one group of lanes however long it is, so the
+ * longest row bounds the launch: on a matrix with hub rows a plan is several
+ * times faster (R-MAT, 4.2 M rows, K = 128: 35 ms against 6 ms; 131 k rows:
+ * 1.2 ms against 0.17 ms), on one without them 1.5 to 3 times.
  */
 int hpspmm_csr_spmm_noplan(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
                            const int32_t *d_col, const float *d_val, const float *d_B, int64_t k,

@@ -310,6 +310,7 @@ constexpr int64_t kRowsAutoMaxWork = (int64_t)3 << 28;  // nnz * K, matrices of 
 constexpr double kRowsAutoLongMean = 128.0;             // mean nonzeros per non-empty row beyond which ...
 constexpr double kRowsAutoLongWork = 2.0e15;            // ... nnz^2 * K decides instead
 constexpr int64_t kRowsAutoMaxRow = 1 << 16;
+constexpr int64_t kRowsAutoAnyKNnz = 1 << 25;            // K outside the tuned set, rows of even lengths: row tiles up to here
 constexpr int64_t kRowsAutoFewPerRowNnz = 1 << 22;      // rows of <= 8 nonzeros, K > 32 and not a multiple of 32
 constexpr int64_t kRowTilePadMinNnz = 1 << 19;  // row tiles: matrices from here up read a B of odd row length through a padded copy
 
@@ -2092,12 +2093,20 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     // K = 172: 231 against 273), while a padded copy of B costs more than it saves.
     const bool few_per_row = mean_row <= 8.0;
     // (K < 4, which row tiles read through a padded copy of B: 1.6 M nonzeros, K = 1: 30 against 18 us.)
-    const bool any_k_range = !few_per_row  ? nnz < kRowTileMaxNnz
+    // On the largest matrices the segments kernel is level or ahead as well, unless the row lengths
+    // are very uneven (social graph, 115 M nonzeros, K = 8: 0.97 ms against 1.40 for row tiles, K = 1:
+    // 0.68 against 1.33; at 26 M nonzeros 0.38 against 0.30, 0.31 against 0.30; R-MAT at 31 M,
+    // K = 1: 1.05 against 0.38).
+    const bool uneven = (double)p->max_row_nnz >= 64.0 * mean_row;
+    const bool any_k_range = !few_per_row  ? nnz < kRowTileMaxNnz && (uneven || nnz < (k < 4 ? kRowsAutoAnyKNnz / 4 : kRowsAutoAnyKNnz))
                              : k % 32 == 0 ? nnz < kRowsAutoMaxNnz && fits
                              : k < 4       ? nnz < kRowTilePadMinNnz
                                            : k <= 32 || nnz < kRowsAutoFewPerRowNnz;
     const bool in_range = fast_k(k) ? nnz < kRowsAutoMaxNnz && fits : any_k_range;
-    const bool mid = in_range && p->max_row_nnz <= kRowsAutoMaxRow && !(flags & HPSPMM_PLAN_NO_ROW_TILES);
+    // (a row gets at most one workgroup of 16 wavefronts; at K outside the tuned set that still beats
+    // the segments kernel with a row of 163k nonzeros - R-MAT, 128 M nonzeros, K = 8: 1.81 against 2.27 ms)
+    const int64_t longest_ok = fast_k(k) || k < 4 ? kRowsAutoMaxRow : 4 * kRowsAutoMaxRow;
+    const bool mid = in_range && p->max_row_nnz <= longest_ok && !(flags & HPSPMM_PLAN_NO_ROW_TILES);
     if (nnz == 0 || tiny || (mid && nnz < kClusterMinNnz)) {
       p->strategy = HPSPMM_STRATEGY_ROWS;
       rows_need_tiles = !(nnz == 0 || tiny);

@@ -152,11 +152,12 @@ const char *hpspmm_last_error(void);
  * gathers at 4-byte alignment when k is not a multiple of 4 - or, where that
  * pays (k > 32 and not a multiple of 8, 2^20 nonzeros and more, 40 for every
  * row of B), through such a copy with rows padded to a multiple of 32 floats;
- * k < 4 always through a copy with rows of 4 floats.  What remains - rows beyond 2^16 nonzeros, very short
- * rows at a k that is not a multiple of 32 on a large matrix - runs whole rows
- * or segments with
- * sub-waves of ceil(k / 4) lanes rounded up to a power of two, rows of B and C
- * read and written at whatever alignment they have.
+ * k < 4 always through a copy with rows of 4 floats.  What remains -
+ * matrices of 2^25 nonzeros and more whose rows are of even lengths, rows
+ * beyond 2^18 nonzeros, very short rows at a k that is not a multiple of 32
+ * on a large matrix - runs whole rows or segments with sub-waves of
+ * ceil(k / 4) lanes rounded up to a power of two, rows of B and C read and
+ * written at whatever alignment they have.
  * Replaces the host-side preprocessing the reference does before timing:
  * CSR->COO expansion (spmm/mm/spmm_common.cpp:185-235), the row re-ordering
  * (:237-296) and the choice of nnz_per_warp (spmm/mm/spmm_kernel.cu:749-751).

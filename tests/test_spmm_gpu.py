@@ -589,14 +589,16 @@ def test_random_matrices_all_strategies(pkg, oracle, gpu, seed):
 
 
 @pytest.mark.parametrize("seed", range(10))
-def test_random_matrices_column_tiles(pkg, oracle, gpu, seed):
-    """The same at row lengths that are multiples of a tuned one: the forced sweep, routed and ordered
-    plans run in column tiles, the others through the kernels for any multiple of 4."""
+def test_random_matrices_column_tiles(pkg, oracle, gpu, monkeypatch, seed):
+    """The same at row lengths outside the tuned set: from 16 columns up the forced sweep, routed and
+    ordered plans run in column tiles; whole rows run over row tiles - B as it lies, then through the
+    padded copy -, the others through the run-time-K kernels."""
     import scipy.sparse as sp
     rng = np.random.default_rng(2000 + seed)
     rows = int(rng.integers(1, 3000))
     cols = int(rng.integers(1, 3000))
-    k = int(rng.choice([16, 17, 20, 30, 40, 41, 47, 96, 100, 127, 160, 173, 200, 256, 259, 384]))
+    k = int(rng.choice([16, 17, 20, 30, 40, 41, 47, 96, 100, 127, 160, 173, 200, 256, 259, 384] if seed % 2 == 0 else
+                       [1, 2, 3, 5, 6, 7, 9, 13, 33, 34, 35, 37, 66, 97, 131]))
     rowptr, col, val = _random_csr(rng, rows, cols, mean_deg=float(rng.uniform(0.5, 40)),
                                    skew=float(rng.uniform(0.8, 3.0)), empty_frac=float(rng.uniform(0, 0.6)),
                                    sorted_unique=(seed % 3 != 2))
@@ -613,7 +615,14 @@ def test_random_matrices_column_tiles(pkg, oracle, gpu, seed):
         bad = np.abs(C - want) > TOL * S
         assert not bad.any(), f"seed {seed} rows={rows} cols={cols} k={k} {name}: {int(bad.sum())} elements off"
         assert not C[np.diff(rowptr) == 0].any()
-    assert tiled >= 4 or col.size == 0, f"seed {seed}: only {tiled} plans ran in column tiles"
+    assert tiled >= 4 or col.size == 0 or k < 16, f"seed {seed}: only {tiled} plans ran in column tiles"
+    monkeypatch.setenv("HPSPMM_ROW_TILES_PAD", "1")
+    C, info = _run(pkg, gpu, g, B, pkg.capi.PLAN_FORCE_ROWS)
+    assert info["row_tiles"] > 0 or col.size == 0 or rows > 40 * col.size, info
+    assert info["launches_per_spmm"] == (2 if info["row_tiles"] > 0 and k % 32 != 0 else 1), info
+    bad = np.abs(C - want) > TOL * S
+    assert not bad.any(), f"seed {seed} rows={rows} cols={cols} k={k} rows over the padded copy: {int(bad.sum())} elements off"
+    assert not C[np.diff(rowptr) == 0].any()
 
 
 def test_non_finite_values_stay_in_their_rows(pkg, oracle, gpu):

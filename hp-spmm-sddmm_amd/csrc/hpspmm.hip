@@ -2509,9 +2509,11 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
   } else if (plan->d_tent && plan->rt_mode) {
     const uint32_t ldb = plan->rt_ldb, ldc = (uint32_t)plan->k;
     if (plan->rt_mode == 2) {
-      hipLaunchKernelGGL(hpspmm::pad_rows_kernel, dim3(grid_for(plan->cols * (int64_t)ldb, 1 << 16)),
-                         dim3(hpspmm::kBlock), 0, st, plan->cols, plan->k, (int64_t)ldb, d_B, plan->d_bpad);
-      mark_launch(st, "pad_rows_kernel");
+      if (plan->nnz > 0) {  // (without nonzeros B is never read, and may be NULL)
+        hipLaunchKernelGGL(hpspmm::pad_rows_kernel, dim3(grid_for(plan->cols * (int64_t)ldb, 1 << 16)),
+                           dim3(hpspmm::kBlock), 0, st, plan->cols, plan->k, (int64_t)ldb, d_B, plan->d_bpad);
+        mark_launch(st, "pad_rows_kernel");
+      }
       rc = launch_row_tiles<0, 2>(plan, d_val, plan->d_bpad, d_C, st, ldb, ldc);
     } else if (plan->rt_mode == 3) {
       rc = launch_row_tiles<0, 3>(plan, d_val, d_B, d_C, st, ldb, ldc);

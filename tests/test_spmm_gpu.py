@@ -284,6 +284,19 @@ def test_edge_shapes(pkg, oracle, gpu):
     for _, flags in _strategies(capi):
         C, _ = _run(pkg, gpu, g, B, flags)
         assert C.shape == (100, 32) and not C.any()
+    # the same through the C ABI with NULL for everything a matrix without nonzeros never reads (col, val,
+    # B), at row lengths of every kind: tuned, a multiple of 4, not one, below 4 (B through a padded copy)
+    import ctypes
+    L = capi.lib()
+    rp = torch.zeros(101, dtype=torch.int32, device=gpu)
+    for k in (32, 100, 41, 5, 3, 1):
+        handle = ctypes.c_void_p()
+        capi.check(L.hpspmm_plan_create(100, 50, 0, rp.data_ptr(), None, k, capi.PLAN_DEFAULT, None, ctypes.byref(handle)))
+        C = torch.full((100, k), float("nan"), device=gpu)
+        capi.check(L.hpspmm_csr_spmm(handle, rp.data_ptr(), None, None, None, C.data_ptr(), None))
+        torch.cuda.synchronize()
+        assert not C.cpu().numpy().any(), f"empty matrix, k={k}"
+        L.hpspmm_plan_destroy(handle)
     # a single row, a single nonzero
     g = graphs.CSR(1, 3, np.array([0, 1], dtype=np.int32), np.array([2], dtype=np.int32), np.array([2.5], dtype=np.float32))
     B = graphs.dense_normal(3, 128, 2)

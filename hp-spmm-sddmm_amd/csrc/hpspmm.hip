@@ -342,7 +342,7 @@ int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, flo
                        uint32_t ldc) {
   const bool same_xcd = row_tiles_same_xcd(kLd, ldb);
   const int64_t groups = ceil_div(p->rt_waves, WPB);
-  const int64_t blocks = (same_xcd ? ceil_div(groups, 8) * 8 : groups) * row_tile_column_tiles(K, ldc);
+  const int64_t blocks = (same_xcd ? ceil_div(groups, hpspmm::kXcds) * hpspmm::kXcds : groups) * row_tile_column_tiles(K, ldc);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB, kLd>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent, readable_values(p, v), B, C,
@@ -357,7 +357,7 @@ int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, fl
   const int64_t wave_items = (p->rt_loop - p->rt_wg) + (p->rt_tiles - p->rt_loop_tiles);
   const bool same_xcd = row_tiles_same_xcd(kLd, ldb);
   const int64_t groups = p->rt_wg + ceil_div(wave_items, WPB);
-  const int64_t blocks = (same_xcd ? ceil_div(groups, 8) * 8 : groups) * row_tile_column_tiles(K, ldc);
+  const int64_t blocks = (same_xcd ? ceil_div(groups, hpspmm::kXcds) * hpspmm::kXcds : groups) * row_tile_column_tiles(K, ldc);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB, kLd>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent,

@@ -227,9 +227,9 @@ __device__ __forceinline__ int column_tiles(uint32_t ldc) {
 template <int kLd>
 __device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, int& tile, int32_t& group) {
   if (kLd != 0 && same_xcd) {
-    const uint32_t per = 8u * (uint32_t)T, r = b % per;
-    tile = (int)(r / 8u);
-    group = (int32_t)((b / per) * 8u + r % 8u);
+    const uint32_t per = (uint32_t)kXcds * (uint32_t)T, r = b % per;
+    tile = (int)(r / (uint32_t)kXcds);
+    group = (int32_t)((b / per) * (uint32_t)kXcds + r % (uint32_t)kXcds);
   } else {
     tile = (int)(b % (uint32_t)T);
     group = (int32_t)(b / (uint32_t)T);

@@ -337,21 +337,21 @@ inline bool row_tiles_same_xcd(int kLd, uint32_t ldb) {
   return kLd != 0 && ldb % 32 != 0 && (e ? std::atoi(e) != 0 : true);
 }
 
-template <int K, int WPB, int kLd>
+template <int K, int WPB, int kLd, int kSub>
 int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st, uint32_t ldb,
                        uint32_t ldc) {
   const bool same_xcd = row_tiles_same_xcd(kLd, ldb);
   const int64_t groups = ceil_div(p->rt_waves, WPB);
   const int64_t blocks = (same_xcd ? ceil_div(groups, hpspmm::kXcds) * hpspmm::kXcds : groups) * row_tile_column_tiles(K, ldc);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
-  hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB, kLd>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
+  hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB, kLd, kSub>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent, readable_values(p, v), B, C,
                      p->d_zrow + 4, ldb, ldc, same_xcd);
   mark_launch(st, "spmm_rowtiles_kernel");
   return HPSPMM_OK;
 }
 
-template <int K, int WPB, int kLd>
+template <int K, int WPB, int kLd, int kSub>
 int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st, uint32_t ldb,
                         uint32_t ldc) {
   const int64_t wave_items = (p->rt_loop - p->rt_wg) + (p->rt_tiles - p->rt_loop_tiles);
@@ -359,7 +359,7 @@ int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, fl
   const int64_t groups = p->rt_wg + ceil_div(wave_items, WPB);
   const int64_t blocks = (same_xcd ? ceil_div(groups, hpspmm::kXcds) * hpspmm::kXcds : groups) * row_tile_column_tiles(K, ldc);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
-  hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB, kLd>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
+  hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB, kLd, kSub>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent,
                      readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc, same_xcd);
   mark_launch(st, "spmm_rowtiles_wg_kernel");
@@ -372,16 +372,25 @@ int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, fl
 // one wavefront needs about 0.6 us per 64 nonzeros, which a 16k-nonzero row turns into 150 us.
 constexpr int64_t kRowTileSmallGrid = 1 << 15;
 
-template <int K, int kLd = 0>
+template <int K, int kLd = 0, int kSub = hpspmm::kSlot>
 int launch_row_tiles(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st,
                      uint32_t ldb = K, uint32_t ldc = K) {
   if (p->rt_wg > 0) {
-    if (p->max_row_nnz > 8192) return launch_row_tiles_wg<K, 16, kLd>(p, v, B, C, st, ldb, ldc);
-    return launch_row_tiles_wg<K, 8, kLd>(p, v, B, C, st, ldb, ldc);
+    if (p->max_row_nnz > 8192) return launch_row_tiles_wg<K, 16, kLd, kSub>(p, v, B, C, st, ldb, ldc);
+    return launch_row_tiles_wg<K, 8, kLd, kSub>(p, v, B, C, st, ldb, ldc);
   }
   if ((int64_t)p->rt_waves * row_tile_column_tiles(K, ldc) <= kRowTileSmallGrid)
-    return launch_row_tiles_w<K, 1, kLd>(p, v, B, C, st, ldb, ldc);
-  return launch_row_tiles_w<K, hpspmm::kWavesPerBlock, kLd>(p, v, B, C, st, ldb, ldc);
+    return launch_row_tiles_w<K, 1, kLd, kSub>(p, v, B, C, st, ldb, ldc);
+  return launch_row_tiles_w<K, hpspmm::kWavesPerBlock, kLd, kSub>(p, v, B, C, st, ldb, ldc);
+}
+
+// Lanes per entry of the row-tile kernels at a row length of its own: 8 (32 columns at a time), or 4 / 1
+// when there are at most 16 / 4 columns, so that a slot works on 2 / 8 of its entries at a time
+// (HPSPMM_ROW_TILES_SUB = 0 in the environment: always 8, for comparisons).
+inline int row_tile_sub_lanes(int64_t k) {
+  const char* e = std::getenv("HPSPMM_ROW_TILES_SUB");
+  if (e && std::atoi(e) == 0) return 8;
+  return k <= 4 ? 1 : k <= 16 ? 4 : 8;
 }
 
 template <int GP, bool kOdd>
@@ -2508,17 +2517,23 @@ int hpspmm_csr_spmm(hpspmm_plan* plan, const int32_t* d_rowptr, const int32_t* d
     }
   } else if (plan->d_tent && plan->rt_mode) {
     const uint32_t ldb = plan->rt_ldb, ldc = (uint32_t)plan->k;
+    const int sub = row_tile_sub_lanes(plan->k);
     if (plan->rt_mode == 2) {
       if (plan->nnz > 0) {  // (without nonzeros B is never read, and may be NULL)
         hipLaunchKernelGGL(hpspmm::pad_rows_kernel, dim3(grid_for(plan->cols * (int64_t)ldb, 1 << 16)),
                            dim3(hpspmm::kBlock), 0, st, plan->cols, plan->k, (int64_t)ldb, d_B, plan->d_bpad);
         mark_launch(st, "pad_rows_kernel");
       }
-      rc = launch_row_tiles<0, 2>(plan, d_val, plan->d_bpad, d_C, st, ldb, ldc);
+      rc = sub == 1   ? launch_row_tiles<0, 2, 1>(plan, d_val, plan->d_bpad, d_C, st, ldb, ldc)
+           : sub == 4 ? launch_row_tiles<0, 2, 4>(plan, d_val, plan->d_bpad, d_C, st, ldb, ldc)
+                      : launch_row_tiles<0, 2>(plan, d_val, plan->d_bpad, d_C, st, ldb, ldc);
     } else if (plan->rt_mode == 3) {
-      rc = launch_row_tiles<0, 3>(plan, d_val, d_B, d_C, st, ldb, ldc);
+      rc = sub == 4 ? launch_row_tiles<0, 3, 4>(plan, d_val, d_B, d_C, st, ldb, ldc)
+                    : launch_row_tiles<0, 3>(plan, d_val, d_B, d_C, st, ldb, ldc);
     } else {
-      rc = launch_row_tiles<0, 1>(plan, d_val, d_B, d_C, st, ldb, ldc);
+      rc = sub == 1   ? launch_row_tiles<0, 1, 1>(plan, d_val, d_B, d_C, st, ldb, ldc)
+           : sub == 4 ? launch_row_tiles<0, 1, 4>(plan, d_val, d_B, d_C, st, ldb, ldc)
+                      : launch_row_tiles<0, 1>(plan, d_val, d_B, d_C, st, ldb, ldc);
     }
   } else if (plan->d_tent) {
     switch (plan->k) {

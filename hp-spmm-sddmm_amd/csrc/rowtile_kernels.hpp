@@ -193,26 +193,44 @@ struct TileColumns {
   int lb;        // this lane's offset into the tile when it gathers (kLd = 3: may be as low as -3)
   int nv;        // how many of this lane's four columns exist in C (0 ... 4)
   bool aligned;  // C's rows start at multiples of 16 bytes
+  int sub;       // which of the entries that a slot works on at a time this lane is on (kSub < 8, see below)
 };
-template <int K, int kLd>
+// kSub = lanes per entry.  8: the slot's 8 lanes gather the 32 columns of one entry after the other.
+// 4 and 1, for row lengths of at most 16 and 4 columns (one column tile): the slot works on 2 or 8
+// of its entries at a time, lane l on entry l / kSub with columns 4 (l % kSub) ...; the partial sums
+// of the lanes that share columns are added up before the row's slots are (reduce_slot).
+template <int K, int kLd, int kSub>
 __device__ __forceinline__ TileColumns tile_columns(uint32_t ldb, uint32_t ldc, int tile, int l) {
   TileColumns tc;
   tc.k0 = tile * 32;
+  tc.sub = l / kSub;
+  const int lc = l % kSub;  // this lane's group of four columns
   if constexpr (kLd == 0) {
     tc.ldb = tc.ldc = (uint32_t)K;
-    tc.lb = 4 * l;
+    tc.lb = 4 * lc;
     tc.nv = 4;
     tc.aligned = true;
   } else {
     tc.ldb = ldb;
     tc.ldc = ldc;
     tc.aligned = kLd == 1 || (kLd == 2 && ldc % 4 == 0);
-    const int left = (int)ldc - (tc.k0 + 4 * l);
+    const int left = (int)ldc - (tc.k0 + 4 * lc);
     tc.nv = left < 0 ? 0 : left > 4 ? 4 : left;
-    if constexpr (kLd == 3) tc.lb = left >= 4 ? 4 * l : (int)ldb - 4 - tc.k0;  // (also a lane beyond the row: in bounds)
-    else tc.lb = left > 0 ? 4 * l : 0;
+    if constexpr (kLd == 3) tc.lb = left >= 4 ? 4 * lc : (int)ldb - 4 - tc.k0;  // (also a lane beyond the row: in bounds)
+    else tc.lb = left > 0 ? 4 * lc : 0;
   }
   return tc;
+}
+// Adds up the partial sums of the lanes of a slot that share columns (kSub < 8), in a fixed order.
+template <int kSub>
+__device__ __forceinline__ void reduce_slot(float4& acc) {
+#pragma unroll
+  for (int off = kSub; off < kSlot; off <<= 1) {
+    acc.x += __shfl_xor(acc.x, off);
+    acc.y += __shfl_xor(acc.y, off);
+    acc.z += __shfl_xor(acc.z, off);
+    acc.w += __shfl_xor(acc.w, off);
+  }
 }
 // Column tiles of a launch.
 template <int K, int kLd>
@@ -258,16 +276,18 @@ __device__ __forceinline__ void store_tile_row(float* __restrict__ C, int32_t ro
 // B (so that a non-finite value in an unreferenced row of B cannot leak in).  With `if (c >= 0)`
 // around the gathers the compiler copied a loaded register inside the batch and waited for it
 // there - one more dependent round trip in a kernel that is nothing but round trips.
-template <int N, bool kUnaligned>
+template <int N, bool kUnaligned, int kSub>
 __device__ __forceinline__ void gather_n(float4& acc, int32_t c, float v, int tid, int base, const TileColumns& tc,
                                          const int32_t* s_col, float* s_val, const float* __restrict__ B,
                                          const float* __restrict__ zrow) {
-  int32_t cc[N];
-  float4 b[N];
+  constexpr int R = kSlot / kSub;      // entries of the slot in work at a time
+  constexpr int S = (N + R - 1) / R;   // steps (an entry beyond the first N is padding in every slot of the tile)
+  int32_t cc[S];
+  float4 b[S];
 #pragma unroll
-  for (int i = 0; i < N; ++i) cc[i] = s_col[base + i];
+  for (int i = 0; i < S; ++i) cc[i] = s_col[base + i * R + tc.sub];
 #pragma unroll
-  for (int i = 0; i < N; ++i) {
+  for (int i = 0; i < S; ++i) {
     const float* src = cc[i] >= 0 ? B + (uint64_t)(uint32_t)cc[i] * (uint64_t)tc.ldb + (uint32_t)tc.k0 : zrow;
     if constexpr (kUnaligned) {
       const Float4Unaligned u = *reinterpret_cast<const Float4Unaligned*>(src + tc.lb);
@@ -279,7 +299,7 @@ __device__ __forceinline__ void gather_n(float4& acc, int32_t c, float v, int ti
   s_val[tid] = c >= 0 ? v : 0.f;
   wave_lds_fence();
 #pragma unroll
-  for (int i = 0; i < N; ++i) fma4(acc, s_val[base + i], b[i]);
+  for (int i = 0; i < S; ++i) fma4(acc, s_val[base + i * R + tc.sub], b[i]);
   wave_lds_fence();
 }
 
@@ -293,7 +313,7 @@ struct TileInfo {
 // Stages the tile's records (e = this lane's) in LDS, issues the load of this lane's value
 // (unconditionally: a padding entry reads val[0] and discards it) and gathers `depth` entries per
 // slot; depth < 0 = take the tile's own.
-template <bool kUnaligned>
+template <bool kUnaligned, int kSub>
 __device__ __forceinline__ TileInfo gather_tile(float4& acc, int2 e, int depth, int tid, int base, int l,
                                                 const TileColumns& tc, int32_t* s_col, int32_t* s_x, float* s_val,
                                                 const float* __restrict__ val, const float* __restrict__ B,
@@ -309,21 +329,21 @@ __device__ __forceinline__ TileInfo gather_tile(float4& acc, int2 e, int depth, 
   const float v = val[e.x >= 0 ? s_x[base + 1] + l : 0];
   switch (info.depth) {
     case 0: wave_lds_fence(); break;
-    case 1: gather_n<1, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
-    case 2: gather_n<2, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
-    case 3: gather_n<3, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
-    case 4: gather_n<4, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
-    case 5: gather_n<5, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
-    case 6: gather_n<6, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
-    case 7: gather_n<7, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
-    default: gather_n<8, kUnaligned>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 1: gather_n<1, kUnaligned, kSub>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 2: gather_n<2, kUnaligned, kSub>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 3: gather_n<3, kUnaligned, kSub>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 4: gather_n<4, kUnaligned, kSub>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 5: gather_n<5, kUnaligned, kSub>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 6: gather_n<6, kUnaligned, kSub>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    case 7: gather_n<7, kUnaligned, kSub>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
+    default: gather_n<8, kUnaligned, kSub>(acc, e.x, v, tid, base, tc, s_col, s_val, B, zrow); break;
   }
   return info;
 }
 
 // acc += the products of tiles [t0, t1) (t0 < t1) of one long row, worked through by one
 // wavefront; returns the row.
-template <bool kUnaligned>
+template <bool kUnaligned, int kSub>
 __device__ __forceinline__ int32_t gather_tiles(float4& acc, int32_t t0, int32_t t1, int lane, int l, int tid,
                                                 int base, const TileColumns& tc, int32_t* s_col, int32_t* s_x,
                                                 float* s_val,
@@ -334,16 +354,17 @@ __device__ __forceinline__ int32_t gather_tiles(float4& acc, int32_t t0, int32_t
   for (int32_t t = t0; t < t1; ++t) {
     const int2 e_now = e;
     if (t + 1 < t1) e = tent[(int64_t)(t + 1) * kRowTile + lane];  // on its way while this tile is gathered
-    row = gather_tile<kUnaligned>(acc, e_now, kSlot, tid, base, l, tc, s_col, s_x, s_val, val, B, zrow).row;
+    row = gather_tile<kUnaligned, kSub>(acc, e_now, kSlot, tid, base, l, tc, s_col, s_x, s_val, val, B, zrow).row;
   }
   return row;
 }
 
 // Sum over the 2^lg adjacent slots of a row (xor shuffles, in a fixed order), then the row's
 // first slot stores.
-template <int kLd>
+template <int kLd, int kSub>
 __device__ __forceinline__ void reduce_and_store(float4 acc, int lg, int32_t row, int s, int l, const TileColumns& tc,
                                                  float* __restrict__ C) {
+  reduce_slot<kSub>(acc);
 #pragma unroll
   for (int step = 0; step < 3; ++step) {
     if (lg > step) {
@@ -353,12 +374,12 @@ __device__ __forceinline__ void reduce_and_store(float4 acc, int lg, int32_t row
       acc.w += __shfl_xor(acc.w, kSlot << step);
     }
   }
-  if ((s & ((1 << lg) - 1)) == 0 && row >= 0) store_tile_row<kLd>(C, row, l, tc, acc);
+  if ((s & ((1 << lg) - 1)) == 0 && row >= 0 && l < kSub) store_tile_row<kLd>(C, row, l, tc, acc);
 }
 
 // Wavefront w < n_loop works through the tiles of long row w (ldesc[w] = first
 // tile, tile count); wavefront w >= n_loop owns tile loop_tiles + (w - n_loop).
-template <int K, int WPB, int kLd = 0>
+template <int K, int WPB, int kLd = 0, int kSub = kSlot>
 __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves, int32_t n_loop, int32_t loop_tiles,
                                                                const int2* __restrict__ ldesc,
                                                                const int2* __restrict__ tent,
@@ -379,7 +400,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
   int ctile;
   int32_t group;
   tile_of_workgroup<kLd>(blockIdx.x, T, same_xcd, ctile, group);
-  const TileColumns tc = tile_columns<K, kLd>(ldb, ldc, ctile, l);
+  const TileColumns tc = tile_columns<K, kLd, kSub>(ldb, ldc, ctile, l);
   const int32_t w = __builtin_amdgcn_readfirstlane(group * WPB + (tid >> 6));
   if (w >= n_waves) return;
 
@@ -387,13 +408,13 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
   if (w >= n_loop) {
     const int32_t tile = loop_tiles + (w - n_loop);
     const int2 e = tent[(int64_t)tile * kRowTile + lane];
-    const TileInfo info = gather_tile<kLd == 3>(acc, e, -1, tid, base, l, tc, s_col, s_x, s_val, val, B, zrow);
-    reduce_and_store<kLd>(acc, info.lg, info.row, s, l, tc, C);
+    const TileInfo info = gather_tile<kLd == 3, kSub>(acc, e, -1, tid, base, l, tc, s_col, s_x, s_val, val, B, zrow);
+    reduce_and_store<kLd, kSub>(acc, info.lg, info.row, s, l, tc, C);
   } else {
     const int2 ld = ldesc[w];
-    const int32_t row = gather_tiles<kLd == 3>(acc, ld.x, ld.x + ld.y, lane, l, tid, base, tc, s_col, s_x, s_val, tent, val,
+    const int32_t row = gather_tiles<kLd == 3, kSub>(acc, ld.x, ld.x + ld.y, lane, l, tid, base, tc, s_col, s_x, s_val, tent, val,
                                         B, zrow);
-    reduce_and_store<kLd>(acc, 3, row, s, l, tc, C);
+    reduce_and_store<kLd, kSub>(acc, 3, row, s, l, tc, C);
   }
 }
 
@@ -402,7 +423,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
 // shares, the shares' sums added in wavefront order through LDS), for matrices whose longest rows
 // would otherwise be the critical path of the launch.  The wavefronts of the other workgroups take
 // one remaining long row or one ordinary tile each, as above.
-template <int K, int WPB, int kLd = 0>
+template <int K, int WPB, int kLd = 0, int kSub = kSlot>
 __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_tiles, int32_t n_wg, int32_t n_loop,
                                                                     int32_t loop_tiles,
                                                                     const int2* __restrict__ ldesc,
@@ -427,7 +448,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
   int ctile;
   int32_t blk;
   tile_of_workgroup<kLd>(blockIdx.x, T, same_xcd, ctile, blk);
-  const TileColumns tc = tile_columns<K, kLd>(ldb, ldc, ctile, l);
+  const TileColumns tc = tile_columns<K, kLd, kSub>(ldb, ldc, ctile, l);
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 
   if (blk < n_wg) {  // uniform over the workgroup: every wavefront reaches the barrier
@@ -436,7 +457,8 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
     const int32_t t0 = ld.x + wave * per;
     const int32_t t1 = t0 + per < ld.x + ld.y ? t0 + per : ld.x + ld.y;
     int32_t row = -1;  // wavefront 0 always has tiles, the later ones may not
-    if (t0 < t1) row = gather_tiles<kLd == 3>(acc, t0, t1, lane, l, tid, base, tc, s_col, s_x, s_val, tent, val, B, zrow);
+    if (t0 < t1) row = gather_tiles<kLd == 3, kSub>(acc, t0, t1, lane, l, tid, base, tc, s_col, s_x, s_val, tent, val, B, zrow);
+    reduce_slot<kSub>(acc);
 #pragma unroll
     for (int off = kSlot; off < 64; off <<= 1) {
       acc.x += __shfl_xor(acc.x, off);
@@ -446,7 +468,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
     }
     if (lane < kSlot) s_part[wave][lane] = acc;
     __syncthreads();
-    if (tid < kSlot) {
+    if (tid < kSub) {
       float4 sum = s_part[0][tid];
       for (int j = 1; j < WPB; ++j) {
         const float4 p = s_part[j][tid];
@@ -463,15 +485,15 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
   const int32_t w = __builtin_amdgcn_readfirstlane(n_wg + (blk - n_wg) * WPB + wave);
   if (w < n_loop) {
     const int2 ld = ldesc[w];
-    const int32_t row = gather_tiles<kLd == 3>(acc, ld.x, ld.x + ld.y, lane, l, tid, base, tc, s_col, s_x, s_val, tent, val,
+    const int32_t row = gather_tiles<kLd == 3, kSub>(acc, ld.x, ld.x + ld.y, lane, l, tid, base, tc, s_col, s_x, s_val, tent, val,
                                         B, zrow);
-    reduce_and_store<kLd>(acc, 3, row, s, l, tc, C);
+    reduce_and_store<kLd, kSub>(acc, 3, row, s, l, tc, C);
   } else {
     const int32_t tile = loop_tiles + (w - n_loop);
     if (tile >= n_tiles) return;
     const int2 e = tent[(int64_t)tile * kRowTile + lane];
-    const TileInfo info = gather_tile<kLd == 3>(acc, e, -1, tid, base, l, tc, s_col, s_x, s_val, val, B, zrow);
-    reduce_and_store<kLd>(acc, info.lg, info.row, s, l, tc, C);
+    const TileInfo info = gather_tile<kLd == 3, kSub>(acc, e, -1, tid, base, l, tc, s_col, s_x, s_val, val, B, zrow);
+    reduce_and_store<kLd, kSub>(acc, info.lg, info.row, s, l, tc, C);
   }
 }
 

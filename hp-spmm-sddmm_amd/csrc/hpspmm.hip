@@ -2103,9 +2103,9 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
     const bool few_per_row = mean_row <= 8.0;
     // (K < 4, which row tiles read through a padded copy of B: 1.6 M nonzeros, K = 1: 30 against 18 us.)
     // On the largest matrices the segments kernel is level or ahead as well, unless the row lengths
-    // are very uneven (social graph, 115 M nonzeros, K = 8: 0.97 ms against 1.40 for row tiles, K = 1:
-    // 0.68 against 1.33; at 26 M nonzeros 0.38 against 0.30, 0.31 against 0.30; R-MAT at 31 M,
-    // K = 1: 1.05 against 0.38).
+    // are very uneven (social graph, 115 M nonzeros, K = 8: 0.97 ms against 1.12 for row tiles, K = 1:
+    // 0.68 against 1.01; at 26 M nonzeros 0.38 against 0.24, 0.31 against 0.22; R-MAT at 31 M,
+    // K = 1: 1.05 against 0.29).
     const bool uneven = (double)p->max_row_nnz >= 64.0 * mean_row;
     const bool any_k_range = !few_per_row  ? nnz < kRowTileMaxNnz && (uneven || nnz < (k < 4 ? kRowsAutoAnyKNnz / 4 : kRowsAutoAnyKNnz))
                              : k % 32 == 0 ? nnz < kRowsAutoMaxNnz && fits
@@ -2113,7 +2113,7 @@ static int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32
                                            : k <= 32 || nnz < kRowsAutoFewPerRowNnz;
     const bool in_range = fast_k(k) ? nnz < kRowsAutoMaxNnz && fits : any_k_range;
     // (a row gets at most one workgroup of 16 wavefronts; at K outside the tuned set that still beats
-    // the segments kernel with a row of 163k nonzeros - R-MAT, 128 M nonzeros, K = 8: 1.81 against 2.27 ms)
+    // the segments kernel with a row of 163k nonzeros - R-MAT, 128 M nonzeros, K = 8: 1.72 against 2.27 ms)
     const int64_t longest_ok = fast_k(k) || k < 4 ? kRowsAutoMaxRow : 4 * kRowsAutoMaxRow;
     const bool mid = in_range && p->max_row_nnz <= longest_ok && !(flags & HPSPMM_PLAN_NO_ROW_TILES);
     if (nnz == 0 || tiny || (mid && nnz < kClusterMinNnz)) {

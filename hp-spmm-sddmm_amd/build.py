@@ -1,4 +1,4 @@
-"""In-tree build of the native libraries (no cmake: three compiler lines).
+"""In-tree build of the native libraries (no cmake: a few compiler lines).
 
   libhpspmm.so           HIP kernels + C ABI (include/hpspmm.h), hipcc, gfx950
   libhpspmm_graphgen.so  seeded synthetic graph generators, g++ / OpenMP
@@ -37,9 +37,23 @@ def _run(cmd, verbose):
 
 
 def build_kernels(verbose=False):
+    """libhpspmm.so from csrc/*.hip: one object per translation unit (compiled side by side), one link.
+    Only the entry points of include/hpspmm.h are exported."""
+    from concurrent.futures import ThreadPoolExecutor
     out = os.path.join(HERE, "libhpspmm.so")
-    _run([HIPCC, *HIP_FLAGS, "-shared", "-I", INCLUDE, "-I", CSRC,
-          os.path.join(CSRC, "hpspmm.hip"), "-o", out], verbose)
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    srcs = sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
+    objs = [os.path.join(objdir, f[:-4] + ".o") for f in srcs]
+
+    def compile_one(pair):
+        src, obj = pair
+        _run([HIPCC, *HIP_FLAGS, "-fvisibility=hidden", "-c", "-I", INCLUDE, "-I", CSRC,
+              os.path.join(CSRC, src), "-o", obj], verbose)
+
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+        list(pool.map(compile_one, zip(srcs, objs)))
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out], verbose)
     return out
 
 

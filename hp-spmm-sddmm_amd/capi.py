@@ -65,7 +65,8 @@ EXPORTS = (
     "hpspmm_version", "hpspmm_last_error", "hpspmm_plan_create", "hpspmm_plan_get_info",
     "hpspmm_plan_destroy", "hpspmm_csr_spmm", "hpspmm_csr_spmm_noplan", "hpspmm_coo_spmm_accumulate",
     "hpspmm_fill_f32", "hpspmm_csr_spmm_timed", "hpspmm_plan_bind_values", "hpspmm_plan_create_ordered",
-    "hpspmm_csr_spmm_static", "hpspmm_csr_spmm_timed_launches",
+    "hpspmm_csr_spmm_static", "hpspmm_csr_spmm_timed_launches", "hpspmm_plan_create_ex",
+    "hpspmm_static_workspace_init", "hpspmm_csr_spmm_timed_min", "hpspmm_get_device_info",
 )
 
 _i64 = ctypes.c_int64
@@ -83,6 +84,31 @@ class PlanInfo(ctypes.Structure):
 
     def as_dict(self):
         return {name: getattr(self, name) for name, _ in self._fields_}
+
+
+class DeviceInfo(ctypes.Structure):
+    _fields_ = [
+        ("device", ctypes.c_int32), ("compute_units", ctypes.c_int32), ("clock_khz", ctypes.c_int32),
+        ("memory_clock_khz", ctypes.c_int32), ("l2_bytes", _i64), ("lds_bytes_per_cu", _i64), ("global_bytes", _i64),
+        ("xcd_dealing", ctypes.c_int32), ("arch", ctypes.c_char * 60),
+    ]
+
+
+class PlanOptions(ctypes.Structure):
+    """hpspmm_plan_options (include/hpspmm.h): zero in a field = the library's default."""
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32), ("flags", ctypes.c_uint32), ("d_row_order", ctypes.c_void_p),
+        ("segment_shift", ctypes.c_int32), ("hub_log2", ctypes.c_int32), ("routed_row_log2", ctypes.c_int32),
+        ("routed_phases", ctypes.c_int32), ("routed_tile_width", ctypes.c_int32),
+        ("routed_split_launch", ctypes.c_int32), ("xcd_dealing", ctypes.c_int32),
+        ("no_column_tiles", ctypes.c_int32), ("row_tiles_min_k", ctypes.c_int32), ("row_tiles_pad", ctypes.c_int32),
+        ("row_tiles_wide", ctypes.c_int32), ("row_tiles_round_robin", ctypes.c_int32),
+        ("sweep_window_log2", ctypes.c_int32), ("sweep_lead", ctypes.c_int32), ("sweep_spin", ctypes.c_int32),
+        ("sweep_limit", ctypes.c_int32), ("sweep_no_priorities", ctypes.c_int32), ("cluster_sweeps", ctypes.c_int32),
+        ("report", ctypes.c_int32),
+    ]
+
+    OPTION_NAMES = tuple(n for n, _ in _fields_[3:])
 
 
 class HpSpmmError(RuntimeError):
@@ -108,6 +134,12 @@ def lib():
                                          ctypes.POINTER(_p)]
         L.hpspmm_plan_create_ordered.argtypes = [_i64, _i64, _i64, _p, _p, _i64, ctypes.c_uint32, _p, _p,
                                                  ctypes.POINTER(_p)]
+        L.hpspmm_plan_create_ex.argtypes = [_i64, _i64, _i64, _p, _p, _i64, ctypes.POINTER(PlanOptions), _p,
+                                            ctypes.POINTER(_p)]
+        L.hpspmm_static_workspace_init.argtypes = []
+        L.hpspmm_get_device_info.argtypes = [ctypes.POINTER(DeviceInfo)]
+        L.hpspmm_csr_spmm_timed_min.argtypes = [_p, _p, _p, _p, _p, _p, _p, ctypes.c_int, ctypes.c_int, ctypes.c_float,
+                                                ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int64)]
         L.hpspmm_plan_get_info.argtypes = [_p, ctypes.POINTER(PlanInfo)]
         L.hpspmm_plan_destroy.argtypes = [_p]
         L.hpspmm_plan_bind_values.argtypes = [_p, _p, _p]
@@ -154,7 +186,8 @@ def _dev(t, dtype, name):
 class Plan:
     """Owns an hpspmm_plan (see hpspmm_plan_create in include/hpspmm.h)."""
 
-    def __init__(self, rows, cols, rowptr, col, k, flags=PLAN_DEFAULT, stream=None, row_order=None):
+    def __init__(self, rows, cols, rowptr, col, k, flags=PLAN_DEFAULT, stream=None, row_order=None, options=None):
+        """options: dict of hpspmm_plan_options fields (then the plan is made by hpspmm_plan_create_ex)."""
         import torch
         _dev(rowptr, torch.int32, "rowptr")
         _dev(col, torch.int32, "col")
@@ -162,7 +195,22 @@ class Plan:
             raise ValueError("rowptr must have rows + 1 entries")
         self._h = ctypes.c_void_p()
         self.rows, self.cols, self.nnz, self.k = int(rows), int(cols), int(col.numel()), int(k)
-        if row_order is None:
+        if options is not None:
+            o = PlanOptions()
+            o.struct_size = ctypes.sizeof(PlanOptions)
+            o.flags = flags
+            if row_order is not None:
+                _dev(row_order, torch.int32, "row_order")
+                if row_order.numel() != rows:
+                    raise ValueError("row_order must have rows entries")
+                o.d_row_order = row_order.data_ptr()
+            for name, value in options.items():
+                if name not in PlanOptions.OPTION_NAMES:
+                    raise KeyError(f"hpspmm_plan_options has no field {name!r}")
+                setattr(o, name, int(value))
+            check(lib().hpspmm_plan_create_ex(rows, cols, self.nnz, _ptr(rowptr), _ptr(col), k, ctypes.byref(o),
+                                              _stream(stream), ctypes.byref(self._h)))
+        elif row_order is None:
             check(lib().hpspmm_plan_create(rows, cols, self.nnz, _ptr(rowptr), _ptr(col), k, flags,
                                            _stream(stream), ctypes.byref(self._h)))
         else:
@@ -271,10 +319,36 @@ def csr_spmm_timed(plan, rowptr, col, val, B, C, warmup=20, iters=200, stream=No
     return float(ms.value)
 
 
+def csr_spmm_timed_min(plan, rowptr, col, val, B, C, warmup=20, iters=200, min_total_ms=10.0, stream=None):
+    """(mean ms per SpMM, launches timed): hpspmm_csr_spmm_timed_min - a region of `iters` launches, or of as
+    many as fill min_total_ms when those take less."""
+    _check_operands(plan.rows, plan.cols, plan.nnz, plan.k, rowptr, col, val, B, C)
+    ms = ctypes.c_float(0.0)
+    done = ctypes.c_int64(0)
+    check(lib().hpspmm_csr_spmm_timed_min(plan._h, _ptr(rowptr), _ptr(col), _ptr(val), _ptr(B), _ptr(C),
+                                          _stream(stream), warmup, iters, float(min_total_ms), ctypes.byref(ms),
+                                          ctypes.byref(done)))
+    return float(ms.value), int(done.value)
+
+
+def device_info():
+    """hpspmm_get_device_info as a dict."""
+    out = DeviceInfo()
+    check(lib().hpspmm_get_device_info(ctypes.byref(out)))
+    d = {name: getattr(out, name) for name, _ in DeviceInfo._fields_}
+    d["arch"] = d["arch"].decode()
+    return d
+
+
+def static_workspace_init():
+    """hpspmm_static_workspace_init: look up the static workspace of csr_spmm_static on the current device."""
+    check(lib().hpspmm_static_workspace_init())
+
+
 def csr_spmm_timed_launches(plan, rowptr, col, val, B, C, warmup=5, iters=50, stream=None):
     """[(kernel name, mean ms)] for every launch of one SpMM, in launch order (HIP events between the launches)."""
     _check_operands(plan.rows, plan.cols, plan.nnz, plan.k, rowptr, col, val, B, C)
-    cap = 8
+    cap = 40
     ms = (ctypes.c_float * cap)()
     names = (ctypes.c_char_p * cap)()
     n = ctypes.c_int(0)

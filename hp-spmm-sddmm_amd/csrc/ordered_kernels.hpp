@@ -109,7 +109,7 @@ __device__ __forceinline__ int32_t cluster_vote(int32_t lab, int32_t mine, int64
 // A sweep is a chain of three dependent round trips per row (row pointer, columns, labels) and
 // little else, so a half-wavefront takes kClusterRowsPerHalf pairs and issues each stage for all of
 // them before it needs any of the answers.
-__global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                const int32_t* __restrict__ col,
                                                                const int32_t* __restrict__ label_in,
                                                                int32_t* __restrict__ label_out, uint32_t sweep,
@@ -163,7 +163,7 @@ __global__ __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, con
 // columns also produce reuse inside a window, but that is the routed strategy's and the hub
 // cache's business; a graph without communities ends up in one giant cluster or in singletons and
 // scores nothing here.  One wavefront per row; intra[] has kClusterCounters entries.
-__global__ __launch_bounds__(kBlock) void cluster_intra_kernel(int64_t rows, int64_t stride,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void cluster_intra_kernel(int64_t rows, int64_t stride,
                                                                const int32_t* __restrict__ rowptr,
                                                                const int32_t* __restrict__ col,
                                                                const int32_t* __restrict__ label,
@@ -186,13 +186,13 @@ __global__ __launch_bounds__(kBlock) void cluster_intra_kernel(int64_t rows, int
 }
 
 // label[r] = r.
-__global__ __launch_bounds__(kBlock) void cluster_init_kernel(int64_t rows, int32_t* __restrict__ label) {
+HPSPMM_KERNEL __launch_bounds__(kBlock) void cluster_init_kernel(int64_t rows, int32_t* __restrict__ label) {
   const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (r < rows) label[r] = (int32_t)r;
 }
 
 // len[i] = number of nonzeros of the i-th row in processing order; len[rows] = 0.
-__global__ __launch_bounds__(kBlock) void ordered_len_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_len_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                              const int32_t* __restrict__ order,
                                                              uint32_t* __restrict__ len) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(kBlock) void ordered_len_kernel(int64_t rows, const
 }
 
 // seen[order[i]] += 1: a permutation leaves every counter at exactly one.
-__global__ __launch_bounds__(kBlock) void ordered_mark_kernel(int64_t rows, const int32_t* __restrict__ order,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_mark_kernel(int64_t rows, const int32_t* __restrict__ order,
                                                               int32_t* __restrict__ seen,
                                                               int32_t* __restrict__ bad) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(kBlock) void ordered_mark_kernel(int64_t rows, cons
 // Lays the nonzeros out in processing order.  One wavefront per position i:
 // row r = order[i] starts at pstart[i]; start[r] = pstart[i];
 // ocol / osrc / orow = column, original index and row of every nonzero.
-__global__ __launch_bounds__(kBlock) void ordered_fill_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_fill_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                               const int32_t* __restrict__ col,
                                                               const int32_t* __restrict__ order,
                                                               const uint32_t* __restrict__ pstart,
@@ -262,7 +262,7 @@ constexpr int kOrderedHistMax = 65;       // occurrence counts are told apart up
 constexpr int kOrderedBitmapWords = 1024;  // 32768 bits per bitmap
 constexpr int kOrderedMaxCap = 512;        // LDS slots a window can ask for, at most
 
-__global__ __launch_bounds__(kBlock) void ordered_hot_kernel(int64_t nnz, int window, int cap,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_hot_kernel(int64_t nnz, int window, int cap,
                                                              int32_t* __restrict__ ocol,
                                                              int32_t* __restrict__ wcols,
                                                              unsigned long long* __restrict__ served) {
@@ -367,7 +367,7 @@ __global__ __launch_bounds__(kBlock) void ordered_hot_kernel(int64_t nnz, int wi
 // in batches, and a batch is as slow as its slowest load.  One wavefront per
 // row; a row cut by a window boundary is left as it is (its slots belong to
 // two different windows).
-__global__ __launch_bounds__(kBlock) void ordered_partition_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_partition_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                    const int32_t* __restrict__ start, int window,
                                                                    int32_t* __restrict__ ocol,
                                                                    int32_t* __restrict__ osrc) {

@@ -1,0 +1,194 @@
+// Ordered strategy: clustering of the rows (label propagation) and the layout over a row order.
+#include "host.hpp"
+
+#include "ordered_kernels.hpp"
+#include "rank_kernels.hpp"
+
+namespace hpspmm_host {
+
+namespace {
+// LDS of one workgroup of the ordered strategy, staging tiles included: the most that still lets
+// three workgroups share a CU's 160 KB (measured on the co-purchase graph, K = 64: 3.14 ms with
+// 32 KB for the rows of B, 2.92 ms with 45 KB, 3.39 ms with 46 KB, where only two fit).
+constexpr int kOrderedBlockLdsBytes = 52992;
+}  // namespace
+
+// Builds the ordered layout for the processing order d_order (a permutation of
+// the row numbers, in device memory).  p->shift is chosen here.
+// With min_served > 0 the layout is kept only if at least that share of the nonzeros reads B from
+// LDS; otherwise everything built here is freed again and the plan is left as it was.
+int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, const int32_t* d_order,
+                  double min_served, hipStream_t st) {
+  const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
+  const int64_t subwaves = 64 / (k / 4);
+  // window = one workgroup's segments, at most kOrderedMaxWindow nonzeros
+  int shift = 9;
+  while (((int64_t)hpspmm::kWavesPerBlock * subwaves << shift) > hpspmm::kOrderedMaxWindow) --shift;
+  const int window = (int)((int64_t)hpspmm::kWavesPerBlock * subwaves << shift);
+  const int64_t staging_bytes = 3 * hpspmm::kWavesPerBlock * subwaves * hpspmm::kTileStride * 4;
+  const int cap = (int)((kOrderedBlockLdsBytes - staging_bytes) / (k * 4));
+  const int64_t windows = ceil_div(nnz, window);
+  const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
+
+  uint32_t* d_len = nullptr;   // [rows + 1] row lengths in processing order, then their scan
+  int32_t* d_seen = nullptr;   // [rows] + [1]: permutation check
+  unsigned long long* d_served = nullptr;
+  struct Guard {
+    void** q[3];
+    ~Guard() {
+      for (void** x : q)
+        if (*x) (void)hipFree(*x);
+    }
+  } guard{{(void**)&d_len, (void**)&d_seen, (void**)&d_served}};
+  HPSPMM_HIP(hipMalloc(&d_len, (size_t)(rows + 1) * sizeof(uint32_t)));
+  HPSPMM_HIP(hipMalloc(&d_seen, (size_t)(rows + 1) * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&d_served, sizeof(unsigned long long)));
+  HPSPMM_HIP(hipMemsetAsync(d_seen, 0, (size_t)(rows + 1) * sizeof(int32_t), st));
+  HPSPMM_HIP(hipMemsetAsync(d_served, 0, sizeof(unsigned long long), st));
+  const unsigned rgrid = (unsigned)ceil_div(rows + 1, hpspmm::kBlock);
+  hipLaunchKernelGGL(hpspmm::ordered_mark_kernel, dim3(rgrid), dim3(hpspmm::kBlock), 0, st, rows, d_order, d_seen,
+                     d_seen + rows);
+  int32_t bad = 0;
+  HPSPMM_HIP(hipMemcpyAsync(&bad, d_seen + rows, sizeof bad, hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  if (bad) return fail(HPSPMM_ERR_INVALID_ARG, "row order is not a permutation of [0, rows)");
+  hipLaunchKernelGGL(hpspmm::ordered_len_kernel, dim3(rgrid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_order,
+                     d_len);
+  if (int rc = exclusive_scan_u32(d_len, d_len, rows + 1, st)) return rc;
+
+  const size_t n_bytes = (size_t)std::max<int64_t>(nnz, 1) * sizeof(int32_t);
+  const size_t start_bytes = (size_t)std::max<int64_t>(rows, 1) * sizeof(int32_t);
+  const size_t wcols_bytes = (size_t)std::max<int64_t>(windows, 1) * (size_t)cap * sizeof(int32_t);
+  const size_t carry_bytes = (size_t)std::max<int64_t>(nseg, 1) * 2 * (size_t)k * sizeof(float);
+  float* d_new_carry = nullptr;
+  auto drop = [&]() {
+    for (void** q : {(void**)&p->d_ostart, (void**)&p->d_ocol, (void**)&p->d_osrc, (void**)&p->d_orow,
+                     (void**)&p->d_wcols, (void**)&d_new_carry}) {
+      if (*q) (void)hipFree(*q);
+      *q = nullptr;
+    }
+  };
+  if (hipMalloc(&p->d_ostart, start_bytes) != hipSuccess || hipMalloc(&p->d_ocol, n_bytes) != hipSuccess ||
+      hipMalloc(&p->d_osrc, n_bytes) != hipSuccess || hipMalloc(&p->d_orow, n_bytes) != hipSuccess ||
+      hipMalloc(&p->d_wcols, wcols_bytes) != hipSuccess || hipMalloc(&d_new_carry, carry_bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    drop();
+    return fail(HPSPMM_ERR_ALLOC, "device allocation for the ordered plan failed");
+  }
+  hipLaunchKernelGGL(hpspmm::ordered_fill_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
+                     dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_order, d_len, p->d_ostart, p->d_ocol,
+                     p->d_osrc, p->d_orow);
+  if (windows > INT32_MAX) {
+    drop();
+    return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  }
+  if (nnz > 0)
+    hipLaunchKernelGGL(hpspmm::ordered_hot_kernel, dim3((unsigned)windows), dim3(hpspmm::kBlock), 0, st, nnz, window,
+                       cap, p->d_ocol, p->d_wcols, d_served);
+  hipLaunchKernelGGL(hpspmm::ordered_partition_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
+                     dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, p->d_ostart, window, p->d_ocol, p->d_osrc);
+  unsigned long long served = 0;
+  hipError_t e = hipMemcpyAsync(&served, d_served, sizeof served, hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e == hipSuccess) e = hipGetLastError();
+  if (e != hipSuccess) {
+    drop();
+    return fail(HPSPMM_ERR_HIP, "construction of the ordered plan failed: %s", hipGetErrorString(e));
+  }
+  if ((double)served < min_served * (double)nnz) {
+    drop();
+    return HPSPMM_OK;
+  }
+  // accepted: the segments strategy's buffers are not needed any more
+  if (p->d_nnz_row) { (void)hipFree(p->d_nnz_row); p->d_nnz_row = nullptr; }
+  if (p->d_carry) (void)hipFree(p->d_carry);
+  p->d_carry = d_new_carry;
+  p->workspace_bytes = (int64_t)(start_bytes + 3 * n_bytes + wcols_bytes + carry_bytes);
+  p->shift = shift;
+  p->nseg = nseg;
+  p->ocap = cap;
+  p->owindows = windows;
+  p->oserved = (int64_t)served;
+  p->strategy = HPSPMM_STRATEGY_ORDERED;
+  return HPSPMM_OK;
+}
+
+// Finds a processing order for a square matrix by label propagation on its graph: rows of one
+// label next to each other, labels in increasing order, rows of a label in increasing order.
+// d_order_out receives a device array of `rows` entries (caller frees).
+constexpr int kClusterMaxSweeps = 16;
+constexpr int32_t kClusterMaxSize = 4096;  // rows of a cluster that still counts as one a window can profit from
+
+int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, const PlanOptions& opt,
+                 hipStream_t st, int32_t** d_order_out, double* intra_share_out) {
+  const int64_t rows = p->rows;
+  *d_order_out = nullptr;
+  *intra_share_out = 0.0;
+  int32_t* d_label = nullptr;
+  int32_t* d_label_next = nullptr;
+  uint32_t* d_changed = nullptr;
+  struct Guard {
+    void** q[3];
+    ~Guard() {
+      for (void** x : q)
+        if (*x) (void)hipFree(*x);
+    }
+  } guard{{(void**)&d_label, (void**)&d_label_next, (void**)&d_changed}};
+  HPSPMM_HIP(hipMalloc(&d_label, (size_t)rows * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&d_label_next, (size_t)rows * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&d_changed, hpspmm::kClusterCounters * sizeof(uint32_t)));
+  std::vector<uint32_t> counters((size_t)hpspmm::kClusterCounters);
+  hipLaunchKernelGGL(hpspmm::cluster_init_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                     0, st, rows, d_label);
+  const int max_sweeps = opt.cluster_sweeps > 0 ? opt.cluster_sweeps : kClusterMaxSweeps;
+  const bool debug = opt.report;
+  for (int sweep = 0; sweep < max_sweeps; ++sweep) {
+    HPSPMM_HIP(hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st));
+    hipLaunchKernelGGL(hpspmm::cluster_sweep_kernel,
+                       dim3((unsigned)ceil_div(ceil_div(rows, 2), hpspmm::kWavesPerBlock * 2 * hpspmm::kClusterRowsPerHalf)),
+                       dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_label, d_label_next, (uint32_t)sweep,
+                       d_changed);
+    std::swap(d_label, d_label_next);
+    HPSPMM_HIP(hipMemcpyAsync(counters.data(), d_changed, counters.size() * sizeof(uint32_t), hipMemcpyDeviceToHost,
+                              st));
+    HPSPMM_HIP(hipStreamSynchronize(st));
+    int64_t changed = 0;
+    for (uint32_t c : counters) changed += c;
+    if (debug) fprintf(stderr, "cluster sweep %d: %lld of %lld rows changed their label\n", sweep, (long long)changed, (long long)rows);
+    if (changed * 200 < rows) break;
+  }
+  // share of the nonzeros that stay inside a cluster small enough for a workgroup's window, from
+  // every 4th row when there are a million of them (a threshold decision: 1.4 -> 0.4 ms at 2.4 M rows)
+  const int64_t score_stride = rows >= ((int64_t)1 << 20) ? 4 : 1;
+  {
+    int32_t* d_size = nullptr;
+    hipError_t e = hipMalloc(&d_size, (size_t)rows * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMemsetAsync(d_size, 0, (size_t)rows * sizeof(int32_t), st);
+    if (e == hipSuccess) e = hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st);
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL(hpspmm::label_sizes_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                         0, st, rows, d_label, d_size);
+      hipLaunchKernelGGL(hpspmm::cluster_intra_kernel,
+                         dim3((unsigned)ceil_div(ceil_div(rows, score_stride), hpspmm::kWavesPerBlock)),
+                         dim3(hpspmm::kBlock), 0, st, rows, score_stride, d_rowptr, d_col, d_label, d_size,
+                         kClusterMaxSize, d_changed);
+      e = hipMemcpyAsync(counters.data(), d_changed, counters.size() * sizeof(uint32_t), hipMemcpyDeviceToHost, st);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (d_size) (void)hipFree(d_size);
+    if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "cluster scoring failed: %s", hipGetErrorString(e));
+    int64_t intra = 0;
+    for (uint32_t c : counters) intra += c;
+    intra *= score_stride;
+    *intra_share_out = p->nnz > 0 ? (double)intra / (double)p->nnz : 0.0;
+    if (debug) fprintf(stderr, "cluster: %.4f of the nonzeros inside clusters of at most %d rows\n", *intra_share_out, kClusterMaxSize);
+  }
+  // rows ordered by label, the rows of a label in increasing order: a stable sort, hence the same
+  // order on every run
+  int32_t* d_order = nullptr;
+  if (int rc = sort_rows_by_label(rows, d_label, st, &d_order)) return rc;
+  *d_order_out = d_order;
+  return HPSPMM_OK;
+}
+
+}  // namespace hpspmm_host

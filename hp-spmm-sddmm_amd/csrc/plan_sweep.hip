@@ -1,0 +1,297 @@
+// Sweep strategy: construction of the layout.
+#include "host.hpp"
+
+#include "rank_kernels.hpp"
+
+namespace hpspmm_host {
+
+namespace {
+
+constexpr int kSweepMaxBands = 64;
+constexpr int32_t kSweepMaxWindows = 8192;
+constexpr int32_t kSweepMaxLimit = 32768;  // piece lengths are sorted as 16-bit keys
+constexpr int kSweepWindowLog2 = 19;       // bytes of B per window
+constexpr int kSweepSpinLimit = 400;
+// Windows a wavefront may be ahead of the slowest of its CU.  Social graph, 233k vertices, ms at
+// K = 32 / 64 / 128: windows of 512 KB with lead 2: 1.09 / 1.68 / 3.17, lead 3: 1.11 / 1.70 / 2.86;
+// 1 MB with lead 2: 1.09 / 1.70 / 2.92, lead 4: 1.12 / 1.71 / 3.07; 256 KB with lead 4: 1.09 / 1.67 / 3.15.
+inline int sweep_lead(int64_t k) { return k >= 128 ? 3 : 2; }
+// Automatic choice: B beyond what the L2s hold between them without help, enough work to fill the device.
+constexpr double kSweepMinSpan = 0.5;  // mean distance from a row's first to its last column, as a share of the columns
+constexpr int64_t kSweepMinNnz = (int64_t)1 << 22;
+constexpr int64_t kSweepMinBBytes = (int64_t)5 << 20;  // social graph: 6 MB of B, sweep 103 / 127 us against 123 / 141; 3 MB: 90 / 65 against 87 / 63
+
+// Gives back what an abandoned attempt at the sweep layout has allocated in the plan so far.
+void drop_sweep_buffers(hpspmm_plan* p) {
+  for (void** q : {(void**)&p->d_sw_part_base, (void**)&p->d_sw_base, (void**)&p->d_sw_len, (void**)&p->d_sw_ends,
+                   (void**)&p->d_sw_slot_row, (void**)&p->d_vcol, (void**)&p->d_vsrc, (void**)&p->d_partial,
+                   (void**)&p->d_sw_split_rows, (void**)&p->d_zero_rows, (void**)&p->d_sw_zrow}) {
+    if (*q) (void)hipFree(*q);
+    *q = nullptr;
+  }
+}
+
+}  // namespace
+
+// Builds the sweep layout on top of a segments plan.  Returns HPSPMM_OK
+// with p->strategy left at SEGMENTS when the matrix does not qualify, cannot be laid out this way, or
+// the device has no room for the temporaries of the construction.  Diagnostics: the sweep_* fields of
+// hpspmm_plan_options (bytes of B per window, lead, spin limit, nonzeros per piece, priorities)
+// override the defaults.
+int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, const PlanOptions& opt,
+                hipStream_t st) {
+  const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
+  if (nnz <= 0) return HPSPMM_OK;
+  // gather offsets are 32-bit, stream entries keep the column in 24 bits
+  if (p->cols * p->k_full * 4 >= ((int64_t)1 << 32) || p->cols > ((int64_t)1 << hpspmm::kSweepColBits)) return HPSPMM_OK;
+  if (!forced && (nnz < kSweepMinNnz || p->cols * k * 4 < kSweepMinBBytes)) return HPSPMM_OK;
+  const int P = (int)(64 / (k / 4));
+  const int WS = P * hpspmm::kSweepSlots;
+  const int wpb = sweep_waves_for(k);
+
+  // one workgroup fills a CU, and a band fills the device exactly: every CU then runs the same
+  // load (a CU with less runs its wavefronts faster, and they leave the others behind)
+  int per_cu = 0;
+  if (int rc = sweep_prepare_kernels(k, &per_cu)) return rc;
+  if (per_cu < 1) return HPSPMM_OK;
+  int dev = 0;
+  hipDeviceProp_t prop;
+  HPSPMM_HIP(hipGetDevice(&dev));
+  HPSPMM_HIP(hipGetDeviceProperties(&prop, dev));
+  const int64_t band_blocks = prop.multiProcessorCount;
+  const int64_t band_waves = band_blocks * wpb;
+
+  // piece limit: a good half of what a sub-wave gets in all, so that the slots of a wavefront even out
+  const int64_t nonempty = std::max<int64_t>(1, rows - p->empty_rows);
+  const int64_t bands_guess = ceil_div(nonempty + nonempty / 8, band_waves * WS);
+  int64_t limit64 = nnz / (bands_guess * band_waves * P) * 6 / 10;
+  limit64 = std::max<int64_t>(64, std::min<int64_t>(limit64, kSweepMaxLimit));
+  const int32_t limit = std::max(1, std::min<int>(opt.sweep_limit > 0 ? opt.sweep_limit : (int)limit64, kSweepMaxLimit));
+
+  const int wlog2 = opt.sweep_window_log2 > 0 ? opt.sweep_window_log2 : kSweepWindowLog2;
+  int wshift = 0;  // log2 of the columns per window
+  while (wshift < 30 && (((int64_t)1 << (wshift + 1)) * k * 4) <= ((int64_t)1 << wlog2)) ++wshift;
+  const int64_t n_windows = ceil_div(p->cols, (int64_t)1 << wshift);
+  if (n_windows > kSweepMaxWindows) return HPSPMM_OK;
+  // every non-empty row is at least one piece: what the two criteria below come to at the very least
+  // (rules the layout out for a matrix of many short rows before any kernel has run)
+  if (!forced && (ceil_div(nonempty, band_waves * WS) * hpspmm::kXcds * p->cols > nnz / 4 || nonempty * n_windows * 3 > nnz * 2))
+    return HPSPMM_OK;
+  if (!columns_sorted(p, d_rowptr, d_col, st)) return HPSPMM_OK;  // a row must meet the windows in stored order
+  if (!forced) {
+    // rows that reach across most of the columns (a banded matrix is better off with whole rows or segments)
+    unsigned long long* d_span = nullptr;
+    unsigned long long span = 0;
+    HPSPMM_HIP(hipMalloc(&d_span, sizeof span));
+    hipError_t e = hipMemsetAsync(d_span, 0, sizeof span, st);
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL(hpspmm::sweep_row_span_kernel, dim3(grid_for(rows, 4096)), dim3(hpspmm::kBlock), 0, st, rows,
+                         d_rowptr, d_col, d_span);
+      e = hipMemcpyAsync(&span, d_span, sizeof span, hipMemcpyDeviceToHost, st);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    (void)hipFree(d_span);
+    if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "row span: %s", hipGetErrorString(e));
+    if ((double)span < kSweepMinSpan * (double)p->cols * (double)std::max<int64_t>(1, rows - p->empty_rows)) return HPSPMM_OK;
+  }
+
+  DeviceTemps tmp;
+  // pieces per row, their scans
+  uint32_t *d_pbase = nullptr, *d_part = nullptr, *d_scan0 = nullptr;
+  // (no room for a temporary or a buffer of the layout: the plan stays what it was, like any other
+  // matrix that cannot be laid out this way)
+  if (tmp.alloc(&d_pbase, (size_t)rows + 1 + (size_t)scan_scratch_words(rows + 1)) != HPSPMM_OK) return HPSPMM_OK;
+  d_scan0 = d_pbase + rows + 1;
+  if (hipMalloc(&p->d_sw_part_base, (size_t)(rows + 1) * sizeof(uint32_t)) != hipSuccess) {
+    (void)hipGetLastError();
+    p->d_sw_part_base = nullptr;
+    return HPSPMM_OK;
+  }
+  d_part = p->d_sw_part_base;
+  hipLaunchKernelGGL(hpspmm::sweep_row_pieces_kernel, dim3((unsigned)ceil_div(rows + 1, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, limit, d_pbase, d_part);
+  if (int rc = exclusive_scan_u32(d_pbase, d_pbase, rows + 1, st, d_scan0)) return rc;
+  if (int rc = exclusive_scan_u32(d_part, d_part, rows + 1, st, d_scan0)) return rc;
+  uint32_t n_pieces = 0, n_parts = 0;
+  HPSPMM_HIP(hipMemcpyAsync(&n_pieces, d_pbase + rows, sizeof n_pieces, hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipMemcpyAsync(&n_parts, d_part + rows, sizeof n_parts, hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  if (n_pieces == 0) {
+    drop_sweep_buffers(p);
+    return HPSPMM_OK;
+  }
+
+  const int64_t n_bands = ceil_div((int64_t)n_pieces, band_waves * WS);
+  // every band re-reads B once on every XCD: worth it while that stays well below the gather volume,
+  // and while a piece still finds one or two nonzeros in a window (the co-purchase graph at 6 M
+  // nonzeros has 0.85 on average and takes 251 us against 134 with the ordered strategy)
+  if (n_bands > kSweepMaxBands ||
+      (!forced && (n_bands * hpspmm::kXcds * p->cols > nnz / 4 || (int64_t)n_pieces * n_windows * 3 > nnz * 2))) {
+    drop_sweep_buffers(p);
+    return HPSPMM_OK;
+  }
+  const int64_t n_waves = n_bands * band_waves;
+  const int64_t n_slots = n_waves * WS;
+
+  // the other temporaries, one allocation
+  const int64_t n_tiles = ceil_div((int64_t)n_pieces, hpspmm::kSortTile);
+  const size_t scan_words = (size_t)std::max(scan_scratch_words(256 * n_tiles), scan_scratch_words(n_waves + 1));
+  for (int i = 0; i < 2; ++i) {
+    tmp.room<uint32_t>(n_pieces);
+    tmp.room<int32_t>(n_pieces);
+  }
+  tmp.room<uint32_t>((size_t)(256 * n_tiles + 1));
+  tmp.room<uint32_t>(scan_words);
+  tmp.room<int32_t>(n_pieces);
+  tmp.room<int32_t>((size_t)n_slots);
+  tmp.room<int32_t>((size_t)rows * (size_t)(n_windows + 1));
+  tmp.room<int32_t>((size_t)n_slots * (size_t)n_windows);
+  tmp.room<uint32_t>((size_t)n_waves + 1);
+  tmp.room<int32_t>(2);
+  // Where every row enters every window and where every slot's runs lie are tables of rows x windows
+  // and slots x windows words: a few words per nonzero on a matrix the layout suits, tens of gigabytes
+  // on one of millions of short rows (which only a forcing flag brings this far): 2 GiB + 64 bytes per
+  // nonzero is the most they may take.
+  if ((int64_t)rows * (n_windows + 1) + n_slots * n_windows > 16 * nnz + ((int64_t)1 << 29) || tmp.reserve() != HPSPMM_OK) {
+    drop_sweep_buffers(p);
+    return HPSPMM_OK;
+  }
+  uint32_t* d_keys[2];
+  int32_t* d_vals[2];
+  for (int i = 0; i < 2; ++i) {
+    d_keys[i] = tmp.take<uint32_t>(n_pieces);
+    d_vals[i] = tmp.take<int32_t>(n_pieces);
+  }
+  uint32_t* d_hist = tmp.take<uint32_t>((size_t)(256 * n_tiles + 1));
+  uint32_t* d_scan = tmp.take<uint32_t>(scan_words);
+  int32_t* d_piece_row = tmp.take<int32_t>(n_pieces);
+  int32_t* d_piece_of = tmp.take<int32_t>((size_t)n_slots);
+  int32_t* d_wstart = tmp.take<int32_t>((size_t)rows * (size_t)(n_windows + 1));
+  int32_t* d_run_at = tmp.take<int32_t>((size_t)n_slots * (size_t)n_windows);
+  uint32_t* d_stream_len = tmp.take<uint32_t>((size_t)n_waves + 1);
+  int32_t* d_counts = tmp.take<int32_t>(2);
+
+  // pieces by decreasing length, dealt to the wavefronts
+  hipLaunchKernelGGL(hpspmm::sweep_piece_keys_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, limit, d_pbase, d_keys[0], d_vals[0], d_piece_row);
+  int sorted = 0;
+  if (int rc = radix_sort_pairs(n_pieces, d_keys, d_vals, d_hist, d_scan, 16, st, &sorted)) return rc;
+  HPSPMM_HIP(hipMemsetAsync(d_piece_of, 0xFF, (size_t)n_slots * sizeof(int32_t), st));
+  hipLaunchKernelGGL(hpspmm::sweep_assign_kernel, dim3((unsigned)ceil_div((int64_t)n_pieces, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, (int64_t)n_pieces, d_vals[sorted], (int32_t)n_bands, (int32_t)band_waves,
+                     (int32_t)WS, d_piece_of);
+
+  // where every row enters every window
+  hipLaunchKernelGGL(hpspmm::sweep_row_windows_kernel, dim3((unsigned)ceil_div(nnz, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, nnz, p->d_nnz_row, d_rowptr, d_col, wshift, (int32_t)n_windows, d_wstart);
+
+  // chunk lengths, stream lengths, stream origins
+  if (hipMalloc(&p->d_sw_base, (size_t)(n_waves + 1) * sizeof(uint32_t)) != hipSuccess ||
+      hipMalloc(&p->d_sw_len, (size_t)n_waves * sizeof(uint32_t)) != hipSuccess ||
+      hipMalloc(&p->d_sw_ends, (size_t)n_waves * (size_t)n_windows * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&p->d_sw_slot_row, (size_t)n_slots * sizeof(int32_t)) != hipSuccess) {
+    (void)hipGetLastError();
+    drop_sweep_buffers(p);
+    return HPSPMM_OK;
+  }
+  const dim3 wave_grid((unsigned)n_waves);
+  switch (P) {
+    case 8:
+      hipLaunchKernelGGL(hpspmm::sweep_chunks_kernel<8>, wave_grid, dim3(hpspmm::kBlock), 0, st, (int32_t)n_windows, limit,
+                         d_piece_of, d_piece_row, d_pbase, d_rowptr, d_wstart, d_run_at, p->d_sw_ends, p->d_sw_len);
+      break;
+    case 4:
+      hipLaunchKernelGGL(hpspmm::sweep_chunks_kernel<4>, wave_grid, dim3(hpspmm::kBlock), 0, st, (int32_t)n_windows, limit,
+                         d_piece_of, d_piece_row, d_pbase, d_rowptr, d_wstart, d_run_at, p->d_sw_ends, p->d_sw_len);
+      break;
+    default:
+      hipLaunchKernelGGL(hpspmm::sweep_chunks_kernel<2>, wave_grid, dim3(hpspmm::kBlock), 0, st, (int32_t)n_windows, limit,
+                         d_piece_of, d_piece_row, d_pbase, d_rowptr, d_wstart, d_run_at, p->d_sw_ends, p->d_sw_len);
+      break;
+  }
+  hipLaunchKernelGGL(hpspmm::sweep_stream_lengths_kernel, dim3((unsigned)ceil_div(n_waves + 1, hpspmm::kBlock)),
+                     dim3(hpspmm::kBlock), 0, st, n_waves, P, p->d_sw_len, d_stream_len);
+  // the total must stay an int32 position: checked on the 64-bit sum of the lengths before the 32-bit scan
+  {
+    std::vector<uint32_t> lens((size_t)n_waves);
+    HPSPMM_HIP(hipMemcpyAsync(lens.data(), p->d_sw_len, (size_t)n_waves * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    HPSPMM_HIP(hipStreamSynchronize(st));
+    int64_t total = 0;
+    uint32_t longest = 0;
+    for (uint32_t v : lens) {
+      total += (int64_t)v * P;
+      longest = std::max(longest, v);
+    }
+    // (positions within a window's chunk are kept in 28 bits while the streams are laid out)
+    if (total >= INT32_MAX - 64 || longest >= (1u << 28)) {
+      drop_sweep_buffers(p);
+      return HPSPMM_OK;
+    }
+    p->sw_total = total;
+  }
+  if (int rc = exclusive_scan_u32(d_stream_len, p->d_sw_base, n_waves + 1, st, d_scan)) return rc;
+
+  // the streams
+  const int64_t total = p->sw_total;
+  if (hipMalloc(&p->d_vcol, (size_t)std::max<int64_t>(total, 1) * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&p->d_vsrc, (size_t)std::max<int64_t>(total, 1) * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&p->d_partial, (size_t)std::max<int64_t>(n_parts, 1) * (size_t)k * sizeof(float)) != hipSuccess ||
+      hipMalloc(&p->d_sw_split_rows, (size_t)std::max<int64_t>(n_parts / 2, 1) * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&p->d_zero_rows, (size_t)std::max<int64_t>(p->empty_rows, 1) * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&p->d_sw_zrow, 128 * sizeof(float)) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipStreamSynchronize(st);  // kernels of this attempt may still be reading its temporaries
+    drop_sweep_buffers(p);
+    return HPSPMM_OK;
+  }
+  hipLaunchKernelGGL(hpspmm::sweep_clear_stream_kernel, dim3(grid_for(total, 1 << 16)), dim3(hpspmm::kBlock), 0, st, total,
+                     p->d_vcol, p->d_vsrc);
+  hipLaunchKernelGGL(hpspmm::sweep_fill_kernel, wave_grid, dim3(hpspmm::kBlock), 0, st, (int32_t)n_windows, wshift, limit,
+                     (int32_t)WS, (int32_t)(k / 4), d_piece_of, d_piece_row, d_pbase, d_rowptr, d_col, d_wstart, d_run_at,
+                     p->d_sw_ends, p->d_sw_base, p->d_sw_len, p->d_vcol, p->d_vsrc);
+  hipLaunchKernelGGL(hpspmm::sweep_slot_rows_kernel, dim3((unsigned)ceil_div(n_slots, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                     0, st, n_slots, d_piece_of, d_piece_row, d_pbase, d_part, d_rowptr, limit, p->d_sw_slot_row);
+
+  // rows cut into pieces, rows without nonzeros
+  HPSPMM_HIP(hipMemsetAsync(d_counts, 0, 2 * sizeof(int32_t), st));
+  HPSPMM_HIP(hipMemsetAsync(p->d_sw_zrow, 0, 128 * sizeof(float), st));
+  const dim3 row_grid((unsigned)ceil_div(rows, hpspmm::kBlock));
+  hipLaunchKernelGGL(hpspmm::sweep_collect_rows_kernel, row_grid, dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, limit, 1,
+                     p->d_sw_split_rows, d_counts);
+  hipLaunchKernelGGL(hpspmm::sweep_collect_rows_kernel, row_grid, dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, limit, 0,
+                     p->d_zero_rows, d_counts + 1);
+  int32_t counts[2] = {0, 0};
+  HPSPMM_HIP(hipMemcpyAsync(counts, d_counts, sizeof counts, hipMemcpyDeviceToHost, st));
+  hipError_t e = hipStreamSynchronize(st);
+  if (e == hipSuccess) e = hipGetLastError();
+  if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "sweep layout failed: %s", hipGetErrorString(e));
+  if (counts[0] < 0 || counts[0] > (int32_t)(n_parts / 2) || counts[1] != p->empty_rows)
+    return fail(HPSPMM_ERR_HIP, "sweep layout: inconsistent row lists");
+  p->n_split = counts[0];
+  p->n_zero = counts[1];
+  p->sw_limit = limit;
+  p->sw_bands = (int32_t)n_bands;
+  p->sw.n_waves = n_waves;
+  p->sw.n_windows = (int32_t)n_windows;
+  p->sw.lead = std::max(1, opt.sweep_lead > 0 ? opt.sweep_lead : sweep_lead(k));
+  p->sw.spin_limit = opt.sweep_spin >= 0 ? opt.sweep_spin : kSweepSpinLimit;
+  p->sw.priorities = opt.sweep_priorities >= 0 ? opt.sweep_priorities : 1;
+  if (opt.report)
+    fprintf(stderr, "sweep plan: bands=%lld waves=%lld windows=%lld limit=%d pieces=%u split_rows=%d nnz=%lld stream=%lld (%.3f)\n",
+            (long long)n_bands, (long long)n_waves, (long long)n_windows, limit, n_pieces, counts[0], (long long)nnz,
+            (long long)total, (double)total / (double)nnz);
+  // the segments plan underneath is no longer needed
+  if (p->d_nnz_row) (void)hipFree(p->d_nnz_row);
+  if (p->d_carry) (void)hipFree(p->d_carry);
+  p->d_nnz_row = nullptr;
+  p->d_carry = nullptr;
+  p->workspace_bytes = 2 * total * 4 + (int64_t)std::max<int64_t>(n_parts, 1) * k * 4 + (n_waves + 1) * 4 + n_waves * 4 +
+                       n_waves * n_windows * 4 + n_slots * 4 + (rows + 1) * 4 + std::max<int64_t>(n_parts / 2, 1) * 4 +
+                       std::max<int64_t>(p->empty_rows, 1) * 4 + 512;
+  p->nseg = 0;
+  p->shift = 0;
+  p->strategy = HPSPMM_STRATEGY_SWEEP;
+  return HPSPMM_OK;
+}
+
+}  // namespace hpspmm_host

@@ -25,7 +25,7 @@ constexpr int kCountChunk = 1 << 15;
 constexpr int kCountSlots = 1 << 12;
 constexpr int kCountProbes = 4;
 
-__global__ __launch_bounds__(kBlock) void count_columns_strided_kernel(int64_t nnz, int64_t stride,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void count_columns_strided_kernel(int64_t nnz, int64_t stride,
                                                                        const int32_t* __restrict__ col,
                                                                        int32_t* __restrict__ count) {
   __shared__ int32_t s_key[kCountSlots];
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(kBlock) void count_columns_strided_kernel(int64_t n
 
 // hist[b] += number of counters whose bits above `shift + 8` equal those of `prefix` and whose byte
 // at `shift` is b (hist[256] zeroed by the caller).  With shift = 24 every counter takes part.
-__global__ __launch_bounds__(kBlock) void select_histogram_kernel(int64_t n, const int32_t* __restrict__ count,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void select_histogram_kernel(int64_t n, const int32_t* __restrict__ count,
                                                                   uint32_t prefix, int shift,
                                                                   uint32_t* __restrict__ hist) {
   __shared__ uint32_t s_hist[256];
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(kBlock) void select_histogram_kernel(int64_t n, con
 
 // above[i] = count[i] > threshold, equal[i] = count[i] == threshold (i < n); both get a trailing 0 at n
 // so that their exclusive scans end in the totals.
-__global__ __launch_bounds__(kBlock) void select_flags_kernel(int64_t n, const int32_t* __restrict__ count,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void select_flags_kernel(int64_t n, const int32_t* __restrict__ count,
                                                               int32_t threshold, uint32_t* __restrict__ above,
                                                               uint32_t* __restrict__ equal) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(kBlock) void select_flags_kernel(int64_t n, const i
 
 // The selected columns in index order: every column above the threshold, then the first `ties`
 // columns at the threshold.  key = (~count << 32) | index sorts by decreasing count, then index.
-__global__ __launch_bounds__(kBlock) void select_compact_kernel(int64_t n, const int32_t* __restrict__ count,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void select_compact_kernel(int64_t n, const int32_t* __restrict__ count,
                                                                 int32_t threshold,
                                                                 const uint32_t* __restrict__ above_scan,
                                                                 const uint32_t* __restrict__ equal_scan,
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kBlock) void select_compact_kernel(int64_t n, const
 
 // The selected keys taken apart for the radix sort: sort_key[i] = high word (the inverted count:
 // ascending = most referenced first), id[i] = low word (the column).  *served += the counts.
-__global__ __launch_bounds__(kBlock) void rank_split_kernel(int32_t m, const unsigned long long* __restrict__ keys,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void rank_split_kernel(int32_t m, const unsigned long long* __restrict__ keys,
                                                             uint32_t* __restrict__ sort_key, int32_t* __restrict__ id,
                                                             unsigned long long* __restrict__ served) {
   const int32_t i = (int32_t)blockIdx.x * kBlock + threadIdx.x;
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(kBlock) void rank_split_kernel(int32_t m, const uns
 
 // Popularity rank s -> compact-buffer slot (s % slices) * per_slice + s / slices:
 // colmap[ids[s]] = slot, slot_src[slot] = ids[s] (both preset to -1 by the caller).
-__global__ __launch_bounds__(kBlock) void hot_slots_kernel(int32_t m, const int32_t* __restrict__ ids, int slices,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void hot_slots_kernel(int32_t m, const int32_t* __restrict__ ids, int slices,
                                                            int32_t per_slice, int32_t* __restrict__ colmap,
                                                            int32_t* __restrict__ slot_src) {
   const int32_t s = (int32_t)blockIdx.x * kBlock + threadIdx.x;
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kBlock) void hot_slots_kernel(int32_t m, const int3
 }
 
 // colmap[ids[s]] = s.
-__global__ __launch_bounds__(kBlock) void hot_index_kernel(int32_t m, const int32_t* __restrict__ ids,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void hot_index_kernel(int32_t m, const int32_t* __restrict__ ids,
                                                            int32_t* __restrict__ colmap) {
   const int32_t s = (int32_t)blockIdx.x * kBlock + threadIdx.x;
   if (s < m) colmap[ids[s]] = s;
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(kBlock) void hot_index_kernel(int32_t m, const int3
 
 // Column ranges of equal nonzero count: range[c] = min(groups - 1, (nonzeros in columns < c) / target),
 // from the exclusive scan of the column counts.
-__global__ __launch_bounds__(kBlock) void column_range_kernel(int64_t cols, const uint32_t* __restrict__ before,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void column_range_kernel(int64_t cols, const uint32_t* __restrict__ before,
                                                               int64_t target, int groups,
                                                               uint8_t* __restrict__ range) {
   const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(kBlock) void column_range_kernel(int64_t cols, cons
 
 // hot[range[ids[s]]] += 1 (hot[] zeroed by the caller; at most 64 ranges), through a workgroup's LDS
 // histogram: a few dozen counters would otherwise take every increment one after the other.
-__global__ __launch_bounds__(kBlock) void range_hot_count_kernel(int32_t m, const int32_t* __restrict__ ids,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void range_hot_count_kernel(int32_t m, const int32_t* __restrict__ ids,
                                                                  const uint8_t* __restrict__ range,
                                                                  uint32_t* __restrict__ hot) {
   __shared__ uint32_t s_hot[64];
@@ -175,7 +175,7 @@ constexpr int kSortItems = 8;                     // elements per thread
 constexpr int kSortTile = kBlock * kSortItems;    // elements per workgroup
 
 // hist[d * n_tiles + tile] = elements of the tile whose digit is d.
-__global__ __launch_bounds__(kBlock) void sort_count_kernel(int64_t n, const uint32_t* __restrict__ keys, int shift,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sort_count_kernel(int64_t n, const uint32_t* __restrict__ keys, int shift,
                                                             int64_t n_tiles, uint32_t* __restrict__ hist) {
   __shared__ uint32_t s_hist[256];
   s_hist[threadIdx.x] = 0;
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(kBlock) void sort_count_kernel(int64_t n, const uin
 // elements of the tile before i with the same digit d).  That number is found round by round (256
 // consecutive elements a round), wavefront by wavefront within a round (running counts per digit in
 // LDS) and by ballots within a wavefront - in index order throughout, which is what keeps the sort stable.
-__global__ __launch_bounds__(kBlock) void sort_scatter_kernel(int64_t n, const uint32_t* __restrict__ keys_in,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sort_scatter_kernel(int64_t n, const uint32_t* __restrict__ keys_in,
                                                               const int32_t* __restrict__ vals_in, int shift,
                                                               int64_t n_tiles, const uint32_t* __restrict__ offsets,
                                                               uint32_t* __restrict__ keys_out,
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(kBlock) void sort_scatter_kernel(int64_t n, const u
 }
 
 // keys[r] = label[r], vals[r] = r.
-__global__ __launch_bounds__(kBlock) void label_pairs_kernel(int64_t rows, const int32_t* __restrict__ label,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void label_pairs_kernel(int64_t rows, const int32_t* __restrict__ label,
                                                              uint32_t* __restrict__ keys, int32_t* __restrict__ vals) {
   const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (r >= rows) return;
@@ -245,7 +245,7 @@ __global__ __launch_bounds__(kBlock) void label_pairs_kernel(int64_t rows, const
 }
 
 // size[label[r]] += 1 (size[] zeroed by the caller).
-__global__ __launch_bounds__(kBlock) void label_sizes_kernel(int64_t rows, const int32_t* __restrict__ label,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void label_sizes_kernel(int64_t rows, const int32_t* __restrict__ label,
                                                              int32_t* __restrict__ size) {
   const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (r < rows) atomicAdd(&size[label[r]], 1);

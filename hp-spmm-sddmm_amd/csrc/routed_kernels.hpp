@@ -106,7 +106,7 @@ __device__ __forceinline__ int range_class_of(int range, int nsub, bool single) 
 constexpr int kSinglePhaseFactor = 2;
 
 // *flag |= 1 if some row has a column index smaller than the one before it (row[] = row of every nonzero).
-__global__ __launch_bounds__(kBlock) void columns_unsorted_kernel(int64_t nnz, const int32_t* __restrict__ row,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void columns_unsorted_kernel(int64_t nnz, const int32_t* __restrict__ row,
                                                                   const int32_t* __restrict__ col,
                                                                   int32_t* __restrict__ flag) {
   bool bad = false;
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(kBlock) void columns_unsorted_kernel(int64_t nnz, c
 }
 
 // dst[q] = val[src[q]]: the values in the plan's order, once, for a caller who has declared them constant.
-__global__ __launch_bounds__(kBlock) void routed_gather_values_kernel(int64_t n, const int32_t* __restrict__ src,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_gather_values_kernel(int64_t n, const int32_t* __restrict__ src,
                                                                       const float* __restrict__ val,
                                                                       float* __restrict__ dst) {
   for (int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x; q < n; q += (int64_t)gridDim.x * kBlock)
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(kBlock) void routed_gather_values_kernel(int64_t n,
 }
 
 // flag[r] = 1 if row r is routed (r < rows), flag[rows] = 0.
-__global__ __launch_bounds__(kBlock) void routed_flag_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_flag_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                              int32_t min_row_nnz, uint32_t* __restrict__ flag) {
   const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (r > rows) return;
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(kBlock) void routed_flag_kernel(int64_t rows, const
 }
 
 // routed_rows[ridx[r]] = r for every routed row (ridx = exclusive scan of the routed flags).
-__global__ __launch_bounds__(kBlock) void routed_list_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_list_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                              int32_t min_row_nnz, const uint32_t* __restrict__ ridx,
                                                              int32_t* __restrict__ routed_rows) {
   const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(kBlock) void routed_list_kernel(int64_t rows, const
 
 // coldcnt[r] = nonzeros of row r if it is a short row, else 0 (r < rows); coldcnt[rows] = 0 (the
 // scan's total slot).  One thread per row: most rows of a large skewed matrix are short or empty.
-__global__ __launch_bounds__(kBlock) void routed_cold_count_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_cold_count_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                    int32_t min_row_nnz,
                                                                    uint32_t* __restrict__ coldcnt) {
   const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(kBlock) void routed_cold_count_kernel(int64_t rows,
 // whole plan.  nch[i] = chunks of routed row i (nch[n_routed] = 0: the scan's total slot).
 constexpr int kRoutedChunk = 4096;
 
-__global__ __launch_bounds__(kBlock) void routed_row_chunks_kernel(int64_t n_routed,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_row_chunks_kernel(int64_t n_routed,
                                                                    const int32_t* __restrict__ routed_rows,
                                                                    const int32_t* __restrict__ rowptr,
                                                                    uint32_t* __restrict__ nch) {
@@ -174,7 +174,7 @@ __global__ __launch_bounds__(kBlock) void routed_row_chunks_kernel(int64_t n_rou
 }
 
 // chunk_row[c] = routed-row number of chunk c (chunk_base = exclusive scan of nch).
-__global__ __launch_bounds__(kBlock) void routed_chunk_rows_kernel(int64_t n_routed,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_chunk_rows_kernel(int64_t n_routed,
                                                                    const uint32_t* __restrict__ chunk_base,
                                                                    int32_t* __restrict__ chunk_row) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -203,7 +203,7 @@ __device__ __forceinline__ RoutedChunk routed_chunk(int64_t c, const int32_t* __
 
 // One wavefront per chunk: cnt[x * n_chunks + c] = its nonzeros in hub class x.
 // cnt[nhub * n_chunks] = 0 (the scan's total slot) is written by the first wavefront.
-__global__ __launch_bounds__(kBlock) void routed_count_kernel(int64_t n_chunks, const int32_t* __restrict__ chunk_row,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_count_kernel(int64_t n_chunks, const int32_t* __restrict__ chunk_row,
                                                               const uint32_t* __restrict__ chunk_base,
                                                               const int32_t* __restrict__ routed_rows,
                                                               const int32_t* __restrict__ rowptr,
@@ -262,7 +262,7 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s
   return wave_off + incl - v;
 }
 
-__global__ __launch_bounds__(kBlock) void scan_tile_sums_kernel(int64_t n, const uint32_t* __restrict__ in,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void scan_tile_sums_kernel(int64_t n, const uint32_t* __restrict__ in,
                                                                 uint32_t* __restrict__ tile_sums) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
   const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(kBlock) void scan_tile_sums_kernel(int64_t n, const
 }
 
 // Exclusive scan of the tile sums in place, by one workgroup.
-__global__ __launch_bounds__(kBlock) void scan_tile_offsets_kernel(int64_t ntiles, uint32_t* __restrict__ tile_sums) {
+HPSPMM_KERNEL __launch_bounds__(kBlock) void scan_tile_offsets_kernel(int64_t ntiles, uint32_t* __restrict__ tile_sums) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
   uint32_t carry = 0;
   for (int64_t base = 0; base < ntiles; base += kBlock) {
@@ -290,7 +290,7 @@ __global__ __launch_bounds__(kBlock) void scan_tile_offsets_kernel(int64_t ntile
 }
 
 // (`out` may be `in`: every thread reads its items before it writes them.)
-__global__ __launch_bounds__(kBlock) void scan_apply_kernel(int64_t n, const uint32_t* in,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void scan_apply_kernel(int64_t n, const uint32_t* in,
                                                             const uint32_t* __restrict__ tile_offsets,
                                                             uint32_t* out) {
   __shared__ uint32_t s_wave[kWavesPerBlock];
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(kBlock) void scan_apply_kernel(int64_t n, const uin
 // row number r (r = n_routed: one past the class), from the exclusive scan of
 // the class-major chunk counts (scanned[x * n_chunks + c]) and the padded class
 // origins.  The end of the (r, x) run is rvptr[(r + 1) * nhub + x].
-__global__ __launch_bounds__(kBlock) void routed_vptr_kernel(RoutedLayout lay, int64_t n_chunks,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_vptr_kernel(RoutedLayout lay, int64_t n_chunks,
                                                              const uint32_t* __restrict__ chunk_base,
                                                              const uint32_t* __restrict__ scanned,
                                                              int32_t* __restrict__ rvptr) {
@@ -328,7 +328,7 @@ __global__ __launch_bounds__(kBlock) void routed_vptr_kernel(RoutedLayout lay, i
 }
 
 // coldptr[r] = virtual index of the first cold-class nonzero of row r (r = rows: one past the class).
-__global__ __launch_bounds__(kBlock) void routed_coldptr_kernel(int64_t rows, int64_t cold_begin,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_coldptr_kernel(int64_t rows, int64_t cold_begin,
                                                                 const uint32_t* __restrict__ scanned,
                                                                 int32_t* __restrict__ coldptr) {
   const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -339,7 +339,7 @@ __global__ __launch_bounds__(kBlock) void routed_coldptr_kernel(int64_t rows, in
 // Scatter the nonzeros of the routed rows into class-major order, keeping the stored order inside
 // every run.  One wavefront per chunk (its first slot in class x follows from the scan of the chunk
 // counts); positions within the chunk from ballots.
-__global__ __launch_bounds__(kBlock) void routed_fill_kernel(RoutedLayout lay, int64_t n_chunks,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_fill_kernel(RoutedLayout lay, int64_t n_chunks,
                                                              const int32_t* __restrict__ chunk_row,
                                                              const uint32_t* __restrict__ chunk_base,
                                                              const uint32_t* __restrict__ scanned,
@@ -390,7 +390,7 @@ __global__ __launch_bounds__(kBlock) void routed_fill_kernel(RoutedLayout lay, i
 
 // The nonzeros of the short rows go to the cold class in stored order.  One thread per nonzero
 // (nnz_row[j] = its row): a wavefront per row would idle on the millions of rows of a few nonzeros.
-__global__ __launch_bounds__(kBlock) void routed_fill_cold_kernel(int64_t nnz, const int32_t* __restrict__ nnz_row,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_fill_cold_kernel(int64_t nnz, const int32_t* __restrict__ nnz_row,
                                                                   const int32_t* __restrict__ rowptr,
                                                                   const int32_t* __restrict__ col,
                                                                   const int32_t* __restrict__ colmap,
@@ -416,7 +416,7 @@ __global__ __launch_bounds__(kBlock) void routed_fill_cold_kernel(int64_t nnz, c
 
 // What the final kernel has to do with every row: nothing (stored by the main kernel, or routed),
 // write zeros (no nonzeros), or add carry slots (a short row whose run crosses a segment boundary).
-__global__ __launch_bounds__(kBlock) void routed_action_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_action_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                int32_t min_row_nnz,
                                                                const int32_t* __restrict__ coldptr, int shift,
                                                                uint8_t* __restrict__ action) {
@@ -443,7 +443,7 @@ __global__ __launch_bounds__(kBlock) void routed_action_kernel(int64_t rows, con
 // sorted by position.  One workgroup per chunk.
 constexpr int kPermChunk = 4096;
 
-__global__ __launch_bounds__(kBlock) void routed_chunk_kernel(RoutedLayout lay, int64_t nnz,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_chunk_kernel(RoutedLayout lay, int64_t nnz,
                                                               const int32_t* __restrict__ vpos,
                                                               uint16_t* __restrict__ lslot,
                                                               int32_t* __restrict__ chunk_base,
@@ -696,7 +696,7 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
 }
 
 // list[] <- every row whose action byte equals `which` (order unspecified); *count must be zero on entry.
-__global__ __launch_bounds__(kBlock) void routed_collect_rows_kernel(int64_t rows, const uint8_t* __restrict__ action,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_collect_rows_kernel(int64_t rows, const uint8_t* __restrict__ action,
                                                                      uint8_t which, int32_t* __restrict__ list,
                                                                      int32_t* __restrict__ count) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;

@@ -69,7 +69,7 @@ __device__ __forceinline__ int rowtile_group(int32_t n) {
 // key[r] = group of row r, id[r] = r; count[g] += rows of group g; count[kRowTileGroups] += tiles
 // of the rows with tiles of their own; count[kRowTileGroups + 1] != 0 if rowptr is not a row
 // pointer array of a matrix with nnz nonzeros (unchecked input: the layout is then not built).
-__global__ __launch_bounds__(kBlock) void rowtile_classify_kernel(int64_t rows, int64_t nnz,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void rowtile_classify_kernel(int64_t rows, int64_t nnz,
                                                                   const int32_t* __restrict__ rowptr,
                                                                   uint32_t* __restrict__ key, int32_t* __restrict__ id,
                                                                   uint32_t* __restrict__ count) {
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kBlock) void rowtile_classify_kernel(int64_t rows, 
 }
 
 // tiles[i] = tiles of the i-th row with tiles of its own (order[] = rows sorted by group), [n] = 0.
-__global__ __launch_bounds__(kBlock) void rowtile_long_tiles_kernel(int64_t n, const int32_t* __restrict__ order,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void rowtile_long_tiles_kernel(int64_t n, const int32_t* __restrict__ order,
                                                                     const int32_t* __restrict__ rowptr,
                                                                     uint32_t* __restrict__ tiles) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(kBlock) void rowtile_long_tiles_kernel(int64_t n, c
 }
 
 // ldesc[i] = {first tile, tiles} of the i-th such row, from the scan of tiles[].
-__global__ __launch_bounds__(kBlock) void rowtile_ldesc_kernel(int64_t n, const uint32_t* __restrict__ first,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void rowtile_ldesc_kernel(int64_t n, const uint32_t* __restrict__ first,
                                                                int2* __restrict__ ldesc) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i < n) ldesc[i] = make_int2((int)first[i], (int)(first[i + 1] - first[i]));
@@ -126,7 +126,7 @@ struct RowTileLayout {
 // Every record of the layout, one thread each: record e of slot q belongs to slot j of some row, or
 // to no row (padding).  Lane 0 of a slot carries the row, lane 1 the index of the slot's first value,
 // lanes 2 and 3 of a tile's first slot the tile's depth and log2 of the slots per row.
-__global__ __launch_bounds__(kBlock) void rowtile_fill_kernel(RowTileLayout lay, const int32_t* __restrict__ order,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void rowtile_fill_kernel(RowTileLayout lay, const int32_t* __restrict__ order,
                                                               const int2* __restrict__ ldesc,
                                                               const int32_t* __restrict__ rowptr,
                                                               const int32_t* __restrict__ col, int2* __restrict__ tent) {

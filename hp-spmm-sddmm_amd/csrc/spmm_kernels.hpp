@@ -29,6 +29,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// A kernel that is not a template: defined in every translation unit that includes its header
+// (internal linkage), emitted only where it is launched.
+#define HPSPMM_KERNEL [[maybe_unused]] static __global__
+
 namespace hpspmm {
 
 constexpr int kBlock = 256;         // threads per workgroup = 4 wavefronts
@@ -608,7 +612,7 @@ __global__ __launch_bounds__(kBlock) void spmm_fixup_kernel(int64_t rows, const 
 
 // status[0] |= 1 rowptr[0] != 0, |= 2 rowptr decreases, |= 4 rowptr[rows] != nnz,
 //           |= 8 column index out of [0, cols).
-__global__ __launch_bounds__(kBlock) void validate_csr_kernel(int64_t rows, int64_t cols, int64_t nnz,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void validate_csr_kernel(int64_t rows, int64_t cols, int64_t nnz,
                                                               const int32_t* __restrict__ rowptr,
                                                               const int32_t* __restrict__ col,
                                                               int32_t* __restrict__ status) {
@@ -629,7 +633,7 @@ __global__ __launch_bounds__(kBlock) void validate_csr_kernel(int64_t rows, int6
 }
 
 // stats[0] = max row length, stats[1] = number of empty rows.
-__global__ __launch_bounds__(kBlock) void row_stats_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void row_stats_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                            int32_t* __restrict__ stats) {
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   int32_t mx = 0, empty = 0;
@@ -651,7 +655,7 @@ __global__ __launch_bounds__(kBlock) void row_stats_kernel(int64_t rows, const i
 
 // Appends every row longer than `threshold` to list[] (order unspecified);
 // *count must be zero on entry.
-__global__ __launch_bounds__(kBlock) void collect_long_rows_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void collect_long_rows_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                    int32_t threshold, int32_t* __restrict__ list,
                                                                    int32_t* __restrict__ count) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -666,7 +670,7 @@ __global__ __launch_bounds__(kBlock) void collect_long_rows_kernel(int64_t rows,
 }
 
 // out[j] = ~slot if column col[j] is cached in slot colmap[col[j]] >= 0, else col[j].
-__global__ __launch_bounds__(kBlock) void remap_columns_kernel(int64_t nnz, const int32_t* __restrict__ col,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void remap_columns_kernel(int64_t nnz, const int32_t* __restrict__ col,
                                                                const int32_t* __restrict__ colmap,
                                                                int32_t* __restrict__ out) {
   const int64_t stride = (int64_t)gridDim.x * kBlock;
@@ -704,7 +708,7 @@ __device__ __forceinline__ int64_t row_of_nonzero(const int32_t* __restrict__ ro
 // kExpandPerBlock consecutive nonzeros: two threads bisect all of rowptr for its first and last
 // one, the others only between those two rows (a handful of steps instead of log2(rows)).
 constexpr int kExpandPerBlock = 4 * kBlock;
-__global__ __launch_bounds__(kBlock) void expand_rows_kernel(int64_t rows, int64_t nnz,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void expand_rows_kernel(int64_t rows, int64_t nnz,
                                                              const int32_t* __restrict__ rowptr,
                                                              int32_t* __restrict__ nnz_row) {
   __shared__ int64_t s_ends[2];
@@ -719,13 +723,13 @@ __global__ __launch_bounds__(kBlock) void expand_rows_kernel(int64_t rows, int64
 
 // out[b] = id of the XCD that workgroup b runs on (hardware register XCC_ID, bits 3:0): lets the
 // plan verify the dealing of workgroups to XCDs that the routed strategy and xcd_remap assume.
-__global__ __launch_bounds__(64) void xcc_probe_kernel(int32_t* __restrict__ out) {
+HPSPMM_KERNEL __launch_bounds__(64) void xcc_probe_kernel(int32_t* __restrict__ out) {
   const unsigned v = __builtin_amdgcn_s_getreg(((4 - 1) << 11) | (0 << 6) | 20);
   if (threadIdx.x == 0) out[blockIdx.x] = (int32_t)(v & 0xFu);
 }
 
 // dst[r, 0:kp) = src[r, 0:k) followed by zeros: B with its rows padded to a multiple of 4 floats.
-__global__ __launch_bounds__(kBlock) void pad_rows_kernel(int64_t rows, int64_t k, int64_t kp,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void pad_rows_kernel(int64_t rows, int64_t k, int64_t kp,
                                                           const float* __restrict__ src, float* __restrict__ dst) {
   const int64_t total = rows * kp;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
@@ -734,7 +738,7 @@ __global__ __launch_bounds__(kBlock) void pad_rows_kernel(int64_t rows, int64_t 
   }
 }
 
-__global__ __launch_bounds__(kBlock) void fill_f32_kernel(float* __restrict__ x, int64_t n, float v) {
+HPSPMM_KERNEL __launch_bounds__(kBlock) void fill_f32_kernel(float* __restrict__ x, int64_t n, float v) {
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) x[i] = v;
 }

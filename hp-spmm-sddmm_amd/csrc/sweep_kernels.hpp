@@ -77,7 +77,7 @@ struct SweepLayout {
 // *sum += (last column - first column) of every row (sorted columns): how far the rows reach across
 // the columns.  The walk over B suits rows that reach all the way; a banded matrix would leave every
 // wavefront busy in a few windows of its own.
-__global__ __launch_bounds__(kBlock) void sweep_row_span_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_row_span_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                 const int32_t* __restrict__ col,
                                                                 unsigned long long* __restrict__ sum) {
   unsigned long long mine = 0;
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(kBlock) void sweep_row_span_kernel(int64_t rows, co
 
 // pieces[r] = number of pieces of row r (0 for an empty row), parts[r] = the same if the row is split,
 // else 0 (its partial-result rows); both get a trailing 0 for the scans' totals.
-__global__ __launch_bounds__(kBlock) void sweep_row_pieces_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_row_pieces_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                   int32_t limit, uint32_t* __restrict__ pieces,
                                                                   uint32_t* __restrict__ parts) {
   const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(kBlock) void sweep_row_pieces_kernel(int64_t rows, 
 
 // Sort keys: piece number pbase[r] + k (piece k of row r) gets key = limit - length, so that an
 // ascending stable sort lists the pieces by decreasing length, ties in row order.
-__global__ __launch_bounds__(kBlock) void sweep_piece_keys_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_piece_keys_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                   int32_t limit, const uint32_t* __restrict__ pbase,
                                                                   uint32_t* __restrict__ keys,
                                                                   int32_t* __restrict__ vals,
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kBlock) void sweep_piece_keys_kernel(int64_t rows, 
 // The i-th longest piece goes to band i % n_bands; within the band, pieces are dealt to the band's
 // wavefronts in rounds, alternately forwards and backwards; round j fills slot j of every wavefront.
 // piece_of[wavefront * slots + round] = piece (preset to -1).
-__global__ __launch_bounds__(kBlock) void sweep_assign_kernel(int64_t n_pieces, const int32_t* __restrict__ order,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_assign_kernel(int64_t n_pieces, const int32_t* __restrict__ order,
                                                               int32_t n_bands, int32_t band_waves, int32_t slots,
                                                               int32_t* __restrict__ piece_of) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(kBlock) void sweep_assign_kernel(int64_t n_pieces, 
 // wstart[r * (n_windows + 1) + p] = index of the first nonzero of row r whose column lies in window
 // p or beyond (p = n_windows: one past the row).  Columns must be sorted within a row.  One thread
 // per nonzero fills the entries between its predecessor's window and its own.
-__global__ __launch_bounds__(kBlock) void sweep_row_windows_kernel(int64_t nnz, const int32_t* __restrict__ nnz_row,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_row_windows_kernel(int64_t nnz, const int32_t* __restrict__ nnz_row,
                                                                    const int32_t* __restrict__ rowptr,
                                                                    const int32_t* __restrict__ col, int wshift,
                                                                    int32_t n_windows, int32_t* __restrict__ wstart) {
@@ -257,7 +257,7 @@ __global__ __launch_bounds__(kBlock) void sweep_chunks_kernel(int32_t n_windows,
 }
 
 // stream_len[w] = P * wave_len[w] (entries of the wavefront in the stream arrays); [n_waves] = 0.
-__global__ __launch_bounds__(kBlock) void sweep_stream_lengths_kernel(int64_t n_waves, int P,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_stream_lengths_kernel(int64_t n_waves, int P,
                                                                       const uint32_t* __restrict__ wave_len,
                                                                       uint32_t* __restrict__ stream_len) {
   const int64_t w = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(kBlock) void sweep_stream_lengths_kernel(int64_t n_
 }
 
 // Padding everywhere: the padding flag, value index -1 (= the value 0).
-__global__ __launch_bounds__(kBlock) void sweep_clear_stream_kernel(int64_t n, int32_t* __restrict__ vent,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_clear_stream_kernel(int64_t n, int32_t* __restrict__ vent,
                                                                     int32_t* __restrict__ vsrc) {
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
     vent[i] = kSweepPad;
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(kBlock) void sweep_clear_stream_kernel(int64_t n, i
 // is one wavefront's streams and nothing else, so the L2 sees every line of them completed within a
 // short time (one thread per nonzero of the matrix, in matrix order, wrote a few bytes here and a
 // few there all over the streams: 2-3 ms instead of well under one on 115 M nonzeros).
-__global__ __launch_bounds__(kBlock) void sweep_fill_kernel(int32_t n_windows, int wshift, int32_t limit, int32_t slots,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_fill_kernel(int32_t n_windows, int wshift, int32_t limit, int32_t slots,
                                                             int32_t lanes, const int32_t* __restrict__ piece_of,
                                                             const int32_t* __restrict__ piece_row,
                                                             const uint32_t* __restrict__ pbase,
@@ -358,7 +358,7 @@ __global__ __launch_bounds__(kBlock) void sweep_fill_kernel(int32_t n_windows, i
 
 // slot_row[slot] = what the slot's result is: row r >= 0 (a whole row, stored to C), ~i (partial
 // result row i of a split row) or kSweepUnused.
-__global__ __launch_bounds__(kBlock) void sweep_slot_rows_kernel(int64_t n_slots, const int32_t* __restrict__ piece_of,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_slot_rows_kernel(int64_t n_slots, const int32_t* __restrict__ piece_of,
                                                                  const int32_t* __restrict__ piece_row,
                                                                  const uint32_t* __restrict__ pbase,
                                                                  const uint32_t* __restrict__ part_base,
@@ -378,7 +378,7 @@ __global__ __launch_bounds__(kBlock) void sweep_slot_rows_kernel(int64_t n_slots
 
 // list[] <- every row with more than `limit` nonzeros (which = 1) or with none (which = 0), order
 // unspecified; *count must be zero on entry.
-__global__ __launch_bounds__(kBlock) void sweep_collect_rows_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_collect_rows_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                     int32_t limit, int which,
                                                                     int32_t* __restrict__ list,
                                                                     int32_t* __restrict__ count) {
@@ -399,7 +399,7 @@ __global__ __launch_bounds__(kBlock) void sweep_collect_rows_kernel(int64_t rows
 
 // dst[q] = val[vsrc[q]], 0 for padding: the values in the order of the index stream, once, for a
 // caller who has declared them constant.
-__global__ __launch_bounds__(kBlock) void sweep_gather_values_kernel(int64_t n, const int32_t* __restrict__ vsrc,
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_gather_values_kernel(int64_t n, const int32_t* __restrict__ vsrc,
                                                                      const float* __restrict__ val,
                                                                      float* __restrict__ dst) {
   for (int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x; q < n; q += (int64_t)gridDim.x * kBlock)

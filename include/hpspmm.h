@@ -99,6 +99,45 @@ typedef enum hpspmm_status {
 
 typedef struct hpspmm_plan hpspmm_plan;
 
+/*
+ * Everything hpspmm_plan_create_ex can be told, one struct per call: nothing about a plan depends
+ * on the environment or on other process-wide state (the reference's entry points have none either,
+ * include/spmm/mm/spmm_kernel.h:17-21).  Zero in a field means "the library's default", so
+ *     hpspmm_plan_options o = {0}; o.struct_size = sizeof o;
+ * is hpspmm_plan_create with flags 0.  struct_size lets a library newer than its caller see where
+ * the caller's struct ends (fields beyond are taken as zero).  The fields after d_row_order are
+ * for measurements and tests: they override choices the plan otherwise makes from the matrix.
+ */
+typedef struct hpspmm_plan_options {
+  uint32_t struct_size;       /* sizeof(hpspmm_plan_options) */
+  uint32_t flags;             /* HPSPMM_PLAN_* bits; a size field below, when not 0, replaces the same
+                                 size packed into the flag word */
+  const int32_t *d_row_order; /* NULL, or the processing order of hpspmm_plan_create_ordered */
+  int32_t segment_shift;      /* log2 of the segment length to force, 3..15 */
+  int32_t hub_log2;           /* log2 of the rows of B in the hub cache / the routed compact buffer, 4..24 */
+  int32_t routed_row_log2;    /* with FORCE_ROUTED: log2 of the shortest row that is routed */
+  int32_t routed_phases;      /* with FORCE_ROUTED: phases by column subset, 1..7 */
+  int32_t routed_tile_width;  /* routed strategy: 32 / 64 = work through B and C in column tiles of that
+                                 width, one after the other on all XCDs (k a multiple of it); -1 = never */
+  int32_t routed_split_launch; /* 1: hub phases and cold class as launches of their own (per-class timing) */
+  int32_t xcd_dealing;        /* 0: probe how workgroups are dealt to the XCDs (once per device and process);
+                                 1: take workgroup b to run on XCD b % 8; 2: take it not to */
+  int32_t no_column_tiles;    /* 1: a k outside 32 / 64 / 128 never gets the sweep / routed / ordered
+                                 layouts in column tiles */
+  int32_t row_tiles_min_k;    /* row tiles serve a k outside the tuned set only from this k up */
+  int32_t row_tiles_pad;      /* row tiles at such a k: 1 = never, 2 = whenever k is not a multiple of 32,
+                                 read B through the padded copy */
+  int32_t row_tiles_wide;     /* 1: 8 lanes per entry also at k <= 16 (instead of 4, or 1 at k <= 4) */
+  int32_t row_tiles_round_robin; /* 1: deal the column tiles of a group of row tiles round robin over the XCDs */
+  int32_t sweep_window_log2;  /* sweep strategy: log2 of the bytes of B per window */
+  int32_t sweep_lead;         /* windows a wavefront may run ahead of the slowest of its CU */
+  int32_t sweep_spin;         /* spin limit of its bounded wait; -1 = never wait */
+  int32_t sweep_limit;        /* nonzeros per piece */
+  int32_t sweep_no_priorities; /* 1: leave the wavefront priorities alone */
+  int32_t cluster_sweeps;     /* label-propagation sweeps, at most */
+  int32_t report;             /* 1: plan-time reports on stderr */
+} hpspmm_plan_options;
+
 typedef struct hpspmm_plan_info {
   int64_t rows, cols, nnz, k;
   int32_t strategy;        /* HPSPMM_STRATEGY_* */
@@ -116,6 +155,25 @@ typedef struct hpspmm_plan_info {
 
 /* Library version, major*10000 + minor*100 + patch. */
 int hpspmm_version(void);
+
+/*
+ * What the library sees of the current device (hipDeviceProp figures, and whether
+ * the probe of hpspmm_plan_create found workgroup b on XCD b % 8).  For reports:
+ * the benchmark prices the L2 -> CU path with the clock given here.  No
+ * counterpart in the reference.
+ */
+typedef struct hpspmm_device_info {
+  int32_t device;
+  int32_t compute_units;
+  int32_t clock_khz;         /* engine clock */
+  int32_t memory_clock_khz;
+  int64_t l2_bytes;          /* as hipDeviceProp reports it (one XCD's) */
+  int64_t lds_bytes_per_cu;
+  int64_t global_bytes;
+  int32_t xcd_dealing;       /* 1: workgroup b of a launch runs on XCD b % 8 */
+  char arch[60];
+} hpspmm_device_info;
+int hpspmm_get_device_info(hpspmm_device_info *info_out);
 
 /* Message of the last failure on the calling thread ("" if none). */
 const char *hpspmm_last_error(void);
@@ -170,8 +228,8 @@ const char *hpspmm_last_error(void);
  * dealing of the others) are used only if a probe launch, once per device and
  * process, has seen workgroup b run on XCD b % 8, which is how the whole
  * (unpartitioned) device deals them; otherwise the plan keeps to segments,
- * rows and ordered without that placement.  The environment variable
- * HPSPMM_XCD_DEALING=0 / 1 overrides the probe (diagnostics).
+ * rows and ordered without that placement (hpspmm_plan_options.xcd_dealing
+ * replaces the probe by the caller's word).
  */
 int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
                        const int32_t *d_col, int64_t k, uint32_t flags, void *stream,
@@ -191,6 +249,15 @@ int hpspmm_plan_create(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d
 int hpspmm_plan_create_ordered(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
                                const int32_t *d_col, int64_t k, uint32_t flags,
                                const int32_t *d_row_order, void *stream, hpspmm_plan **plan_out);
+
+/*
+ * hpspmm_plan_create / hpspmm_plan_create_ordered with every option in one struct (see
+ * hpspmm_plan_options; NULL = all defaults).  The two entry points above forward here.  A plan
+ * keeps what it was told: hpspmm_csr_spmm reads nothing but the plan and its arguments.
+ */
+int hpspmm_plan_create_ex(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
+                          const int32_t *d_col, int64_t k, const hpspmm_plan_options *options,
+                          void *stream, hpspmm_plan **plan_out);
 
 int hpspmm_plan_get_info(const hpspmm_plan *plan, hpspmm_plan_info *info_out);
 
@@ -261,10 +328,20 @@ int hpspmm_csr_spmm_noplan(int64_t rows, int64_t cols, int64_t nnz, const int32_
  * has written before), but all calls on one GPU share it: calls that overlap in
  * time on one GPU - two streams, two host threads - race.  The CSR arrays are
  * not validated.
+ * The first call on a device looks up where that device holds the array, which
+ * is not a thing to do on a capturing stream: call hpspmm_static_workspace_init
+ * (or make one ordinary call) on the device beforehand.
  */
 int hpspmm_csr_spmm_static(int64_t rows, int64_t cols, int64_t nnz, const int32_t *d_rowptr,
                            const int32_t *d_col, const float *d_val, const float *d_B, int64_t k,
                            float *d_C, void *stream);
+
+/*
+ * Looks up the static workspace of hpspmm_csr_spmm_static on the current
+ * device (once per device; later calls return at once).  No allocation, no
+ * launch.  It has no counterpart in the reference.
+ */
+int hpspmm_static_workspace_init(void);
 
 /*
  * C += A * B for A in COO (row-index per nonzero), the contract of one launch
@@ -294,13 +371,30 @@ int hpspmm_csr_spmm_timed(hpspmm_plan *plan, const int32_t *d_rowptr, const int3
                           int warmup, int iters, float *mean_ms_out);
 
 /*
+ * The same, for an SpMM of microseconds: when the `iters` launches take less
+ * than min_total_ms together, a second region of as many launches as fill
+ * min_total_ms at the rate just seen is timed and reported instead
+ * (*iters_done_out = the launches of the region reported; may be NULL).  The
+ * reference times 200 launches whatever they take
+ * (include/spmm/utils/timer_cuda.h:3-4); 200 launches of 4 us are 0.8 ms,
+ * within which clock ramps and launch jitter do not average out.
+ */
+int hpspmm_csr_spmm_timed_min(hpspmm_plan *plan, const int32_t *d_rowptr, const int32_t *d_col,
+                              const float *d_val, const float *d_B, float *d_C, void *stream,
+                              int warmup, int iters, float min_total_ms, float *mean_ms_out,
+                              int64_t *iters_done_out);
+
+/*
  * The same protocol with one more event after every kernel launch of an SpMM:
  * mean_ms_out[i] = mean duration of the i-th launch (i < *n_launches_out <=
- * max_launches, at most 8), names_out[i] = its kernel's name (a string owned by
- * the library).  For reporting which launch of a multi-launch strategy takes the
- * time; the extra events keep launches from overlapping their neighbours'
- * start-up, so the sum is slightly above hpspmm_csr_spmm_timed's mean.  The
- * reference has no counterpart (its launchers are single kernels).
+ * max_launches), names_out[i] = its kernel's name (a string owned by the
+ * library).  An SpMM of more launches than max_launches (or than the 32 the
+ * library records) gets the time of those beyond as one last entry named
+ * "(remaining launches)".  Every iteration ends with an event of its own that
+ * the host waits for.  For reporting which launch of a multi-launch strategy
+ * takes the time; the extra events keep launches from overlapping their
+ * neighbours' start-up, so the sum is slightly above hpspmm_csr_spmm_timed's
+ * mean.  The reference has no counterpart (its launchers are single kernels).
  */
 int hpspmm_csr_spmm_timed_launches(hpspmm_plan *plan, const int32_t *d_rowptr, const int32_t *d_col,
                                    const float *d_val, const float *d_B, float *d_C, void *stream,

@@ -19,13 +19,13 @@ def _to_dev(gpu, *arrays):
     return [torch.from_numpy(np.ascontiguousarray(a)).to(gpu) for a in arrays]
 
 
-def _run(pkg, gpu, g, B, flags=0, poison=True):
+def _run(pkg, gpu, g, B, flags=0, poison=True, options=None):
     import torch
     capi = pkg.capi
     k = B.shape[1]
     rp, ci, v, Bd = _to_dev(gpu, g.rowptr, g.col, g.val, B)
     C = torch.full((g.rows, k), float("nan") if poison else 0.0, device=gpu, dtype=torch.float32)
-    plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
+    plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags, options=options)
     info = plan.info
     capi.csr_spmm(plan, rp, ci, v, Bd, C)
     torch.cuda.synchronize()
@@ -490,20 +490,14 @@ def test_xcd_placement_is_verified_at_plan_time(pkg, oracle, gpu):
     per device; on the whole MI355X it holds and the social graph gets the routed strategy.  With the
     probe overridden to 'does not hold' the plan keeps to a strategy without XCD placement and the
     product is the same to rounding."""
-    import os
     capi = pkg.capi
     g = pkg.graphs.make_graph("c2_social", 0.1)
     k = 128
     B = pkg.graphs.make_dense("c2_social", g.cols, k)
-    assert "HPSPMM_XCD_DEALING" not in os.environ
     C, info = _run(pkg, gpu, g, B, capi.PLAN_NO_SWEEP)  # (the sweep strategy, which this graph gets by default, places nothing)
     assert info["strategy"] == capi.STRATEGY_ROUTED, info
     _check(oracle, g, B, C, "probe result")
-    os.environ["HPSPMM_XCD_DEALING"] = "0"
-    try:
-        C0, info0 = _run(pkg, gpu, g, B, capi.PLAN_NO_SWEEP)
-    finally:
-        del os.environ["HPSPMM_XCD_DEALING"]
+    C0, info0 = _run(pkg, gpu, g, B, capi.PLAN_NO_SWEEP, options={"xcd_dealing": 2})
     assert info0["strategy"] in (capi.STRATEGY_SEGMENTS, capi.STRATEGY_ROWS), info0
     _check(oracle, g, B, C0, "placement not available")
 
@@ -602,7 +596,7 @@ def test_random_matrices_all_strategies(pkg, oracle, gpu, seed):
 
 
 @pytest.mark.parametrize("seed", range(10))
-def test_random_matrices_column_tiles(pkg, oracle, gpu, monkeypatch, seed):
+def test_random_matrices_column_tiles(pkg, oracle, gpu, seed):
     """The same at row lengths outside the tuned set: from 16 columns up the forced sweep, routed and
     ordered plans run in column tiles; whole rows run over row tiles - B as it lies, then through the
     padded copy -, the others through the run-time-K kernels."""
@@ -629,8 +623,7 @@ def test_random_matrices_column_tiles(pkg, oracle, gpu, monkeypatch, seed):
         assert not bad.any(), f"seed {seed} rows={rows} cols={cols} k={k} {name}: {int(bad.sum())} elements off"
         assert not C[np.diff(rowptr) == 0].any()
     assert tiled >= 4 or col.size == 0 or k < 16, f"seed {seed}: only {tiled} plans ran in column tiles"
-    monkeypatch.setenv("HPSPMM_ROW_TILES_PAD", "1")
-    C, info = _run(pkg, gpu, g, B, pkg.capi.PLAN_FORCE_ROWS)
+    C, info = _run(pkg, gpu, g, B, pkg.capi.PLAN_FORCE_ROWS, options={"row_tiles_pad": 2})
     assert info["row_tiles"] > 0 or col.size == 0 or rows > 40 * col.size, info
     assert info["launches_per_spmm"] == (2 if info["row_tiles"] > 0 and k % 32 != 0 else 1), info
     bad = np.abs(C - want) > TOL * S
@@ -942,7 +935,7 @@ def test_row_tiles_layout_and_fallback(pkg, oracle, gpu):
 
 
 @pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 7, 20, 31, 33, 36, 41, 63, 65, 100, 130, 172, 259])
-def test_row_tiles_at_any_row_length(pkg, oracle, gpu, monkeypatch, k):
+def test_row_tiles_at_any_row_length(pkg, oracle, gpu, k):
     """Row tiles at a row length outside the tuned set: 32-column tiles, the last one narrower; B as it
     lies (K a multiple of 4: aligned gathers; else 16-byte gathers at 4-byte alignment, the lane of a
     row's last columns reading the row's last four floats) or through the plan's copy with rows padded
@@ -970,11 +963,10 @@ def test_row_tiles_at_any_row_length(pkg, oracle, gpu, monkeypatch, k):
     Cbig = torch.full((guard + rows * k + guard,), 12345.0, device=gpu)
     Bd, Cd = Bbig[guard:guard + cols * k].view(cols, k), Cbig[guard:guard + rows * k].view(rows, k)
     results = {}
-    for form, env in (("as it lies", "0"), ("padded copy", "1")):
-        monkeypatch.setenv("HPSPMM_ROW_TILES_PAD", env)
-        plan = capi.Plan(rows, cols, rp, ci, k, capi.PLAN_DEFAULT)
+    for form, pad in (("as it lies", 1), ("padded copy", 2)):
+        plan = capi.Plan(rows, cols, rp, ci, k, capi.PLAN_DEFAULT, options={"row_tiles_pad": pad})
         info = plan.info
-        padded = k < 4 or (env == "1" and k % 32 != 0)  # (a row of fewer than 4 floats is always read from a copy)
+        padded = k < 4 or (pad == 2 and k % 32 != 0)  # (a row of fewer than 4 floats is always read from a copy)
         assert info["strategy"] == capi.STRATEGY_ROWS and info["row_tiles"] * 64 >= col.size, info
         assert info["launches_per_spmm"] == (2 if padded else 1) and info["k"] == k, info
         for attempt in range(2):
@@ -989,7 +981,6 @@ def test_row_tiles_at_any_row_length(pkg, oracle, gpu, monkeypatch, k):
         plan.destroy()
     assert np.array_equal(results["as it lies"], results["padded copy"])
     # no row beyond 512 nonzeros: one wavefront per row tile, in workgroups of one (small grid) or four
-    monkeypatch.delenv("HPSPMM_ROW_TILES_PAD")
     for scale in (0.25, 4.0):
         g = pkg.graphs.make_graph("c1_citation", scale)
         B = pkg.graphs.dense_normal(g.cols, k, 5)
@@ -1061,7 +1052,6 @@ def test_sweep_layout_corners(pkg, oracle, gpu):
     """Forced sweep plans whose layout is all corners: windows of a few columns, pieces of 64 nonzeros
     (most rows split, several bands), a lead of one window; a matrix with empty rows and a row of
     every column; unsorted columns (the plan then keeps to segments)."""
-    import os
     capi = pkg.capi
     rng = np.random.default_rng(11)
     cases = []
@@ -1077,21 +1067,16 @@ def test_sweep_layout_corners(pkg, oracle, gpu):
     col = np.concatenate([np.sort(rng.choice(cols - 1 if d < cols else cols, int(d), replace=False)) for d in deg]).astype(np.int32)
     val = rng.uniform(-1, 1, col.size).astype(np.float32)
     cases.append(("ragged", pkg.graphs.CSR(rows, cols, rowptr, col, val)))
-    for env in ({}, {"HPSPMM_SWEEP_WINDOW_LOG2": "12", "HPSPMM_SWEEP_LIMIT": "64", "HPSPMM_SWEEP_LEAD": "1"},
-                {"HPSPMM_SWEEP_WINDOW_LOG2": "30", "HPSPMM_SWEEP_LIMIT": "1", "HPSPMM_SWEEP_SPIN": "0"}):
-        os.environ.update(env)
-        try:
-            for name, g in cases:
-                if env.get("HPSPMM_SWEEP_LIMIT") == "1" and name == "social":
-                    continue  # one piece per nonzero: only for the small matrix
-                for k in (32, 64, 128):
-                    B = pkg.graphs.dense_normal(g.cols, k, 5)
-                    C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SWEEP)
-                    assert info["strategy"] == capi.STRATEGY_SWEEP, (name, env, info)
-                    _check(oracle, g, B, C, f"sweep corners {name} k={k} {env}")
-        finally:
-            for key in env:
-                del os.environ[key]
+    for opts in ({}, {"sweep_window_log2": 12, "sweep_limit": 64, "sweep_lead": 1},
+                 {"sweep_window_log2": 30, "sweep_limit": 1, "sweep_spin": -1}):
+        for name, g in cases:
+            if opts.get("sweep_limit") == 1 and name == "social":
+                continue  # one piece per nonzero: only for the small matrix
+            for k in (32, 64, 128):
+                B = pkg.graphs.dense_normal(g.cols, k, 5)
+                C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SWEEP, options=opts)
+                assert info["strategy"] == capi.STRATEGY_SWEEP, (name, opts, info)
+                _check(oracle, g, B, C, f"sweep corners {name} k={k} {opts}")
     # columns out of order within the rows: no sweep layout, the forced flag falls back to segments
     rowptr, col, val = _random_csr(rng, 500, 700, 20, 1.5, 0.1, sorted_unique=False)
     g = pkg.graphs.CSR(500, 700, rowptr, col, val)

@@ -108,3 +108,36 @@ def test_static_entry_limits_and_edges(pkg, oracle, gpu):
     g = pkg.graphs.CSR(rows, cols, rowptr, col, val)
     assert g.nnz == 1 << 22
     _both(pkg, oracle, gpu, g, rng.standard_normal((cols, k)).astype(np.float32), "at the limit")
+
+
+def test_static_entry_under_graph_capture(pkg, oracle, gpu):
+    """After hpspmm_static_workspace_init the entry point is launches only, so it can be captured: the
+    replays (with the program's own eager calls between them) give the bits of the eager call."""
+    import torch
+    capi = pkg.capi
+    capi.static_workspace_init()
+    capi.static_workspace_init()  # later calls return at once
+    g = pkg.graphs.make_graph("c4_rmat", 0.004)
+    k = 64
+    B = pkg.graphs.make_dense("c4_rmat", g.cols, k)
+    rp, ci, v, Bd = [torch.from_numpy(np.ascontiguousarray(a)).to(gpu) for a in (g.rowptr, g.col, g.val, B)]
+    C = torch.full((g.rows, k), float("nan"), device=gpu)
+    eager = torch.empty_like(C)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            capi.csr_spmm_static(g.rows, g.cols, rp, ci, v, Bd, C, side)
+    torch.cuda.current_stream().wait_stream(side)
+    for scale in (1.0, -0.5, 2.0):
+        v.copy_(torch.from_numpy(g.val).to(gpu) * scale)
+        capi.csr_spmm_static(g.rows, g.cols, rp, ci, v, Bd, eager)
+        torch.cuda.synchronize()
+        C.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(C, eager), f"replay with values x{scale} differs from the eager call"
+    C64, S64 = oracle.csr_spmm_f64(g.rowptr, g.col, (g.val * 2.0).astype(np.float32), B)
+    err, pos = oracle.max_norm_err(C.cpu().numpy(), C64, S64)
+    assert err <= TOL, f"normalised error {err:.3e} at {pos}"

@@ -53,6 +53,26 @@ def plan_segment_shift(log2_len):
     return (int(log2_len) & 0xF) << 8
 
 
+class FlagsWithOptions(int):
+    """A plan-flag word that carries hpspmm_plan_options fields along (Plan then goes through
+    hpspmm_plan_create_ex): flags_with_options(PLAN_FORCE_ROUTED, routed_tile_width=32).  Or-ing further
+    flag bits onto it keeps the options."""
+
+    def __new__(cls, flags, options):
+        self = super().__new__(cls, flags)
+        self.options = dict(options)
+        return self
+
+    def __or__(self, other):
+        return FlagsWithOptions(int(self) | int(other), {**getattr(other, "options", {}), **self.options})
+
+    __ror__ = __or__
+
+
+def flags_with_options(flags=0, **options):
+    return FlagsWithOptions(flags, options)
+
+
 STRATEGY_ROWS = 1
 STRATEGY_SEGMENTS = 2
 STRATEGY_GENERIC_K = 3
@@ -100,7 +120,8 @@ class PlanOptions(ctypes.Structure):
         ("struct_size", ctypes.c_uint32), ("flags", ctypes.c_uint32), ("d_row_order", ctypes.c_void_p),
         ("segment_shift", ctypes.c_int32), ("hub_log2", ctypes.c_int32), ("routed_row_log2", ctypes.c_int32),
         ("routed_phases", ctypes.c_int32), ("routed_tile_width", ctypes.c_int32),
-        ("routed_split_launch", ctypes.c_int32), ("xcd_dealing", ctypes.c_int32),
+        ("routed_split_launch", ctypes.c_int32), ("routed_lds_rows", ctypes.c_int32),
+        ("xcd_dealing", ctypes.c_int32),
         ("no_column_tiles", ctypes.c_int32), ("row_tiles_min_k", ctypes.c_int32), ("row_tiles_pad", ctypes.c_int32),
         ("row_tiles_wide", ctypes.c_int32), ("row_tiles_round_robin", ctypes.c_int32),
         ("sweep_window_log2", ctypes.c_int32), ("sweep_lead", ctypes.c_int32), ("sweep_spin", ctypes.c_int32),
@@ -195,6 +216,9 @@ class Plan:
             raise ValueError("rowptr must have rows + 1 entries")
         self._h = ctypes.c_void_p()
         self.rows, self.cols, self.nnz, self.k = int(rows), int(cols), int(col.numel()), int(k)
+        if getattr(flags, "options", None):
+            options = {**flags.options, **(options or {})}
+        flags = int(flags)
         if options is not None:
             o = PlanOptions()
             o.struct_size = ctypes.sizeof(PlanOptions)

@@ -143,6 +143,7 @@ struct PlanOptions {
   int routed_row_log2 = 0, routed_phases = 0;
   int routed_tile_width = 0;  // 0 = automatic, -1 = never, 32 / 64
   bool routed_split_launch = false;
+  int routed_lds_rows = 0;    // column-tile phases: rows of B a workgroup keeps in LDS (0 = what fits, -1 = none)
   int xcd_dealing = -1;       // -1 probe, 0 / 1 assume
   bool column_tiles = true;   // a row length outside the tuned set may get the tiled layouts
   int64_t row_tiles_min_k = 1;
@@ -198,6 +199,10 @@ struct hpspmm_plan {
   float* d_vval = nullptr;        // [vtotal] the values in that order, rewritten by every SpMM (not with d_vsrc)
   int32_t* d_vsrc = nullptr;      // [vtotal] column-range slices: index of every position in the caller's arrays
   int32_t* d_vrow = nullptr;      // [vtotal] routed-row number (hub classes) or row (cold class)
+  // (column-tile phases keep the rows run by run instead: d_vcol then holds entry words, see kRunStart)
+  int32_t* d_run_row = nullptr;   // [n_runs] routed-row number or row of every run, in class-major order
+  int32_t* d_seg_run = nullptr;   // [nseg] run of every segment's first entry
+  int64_t n_runs = 0;
   int32_t* d_bhot_src = nullptr;  // [n_bhot] source column of every compact-buffer row (-1 = unused)
   int32_t* d_routed_rows = nullptr;  // [n_routed] row of every routed-row number
   int32_t* d_cross_rows = nullptr;   // short rows whose run crosses a segment boundary
@@ -375,6 +380,9 @@ int launch_coo_any(int64_t nnz, int64_t k, const int32_t* ri, const int32_t* ci,
 int launch_segments_workspace(int64_t rows, int64_t nnz, int64_t k, const int32_t* rp, const int32_t* ci,
                               const float* v, const float* B, float* C, int32_t* nnz_row, float* carry,
                               int64_t carry_floats, hipStream_t st);
+// Lets the routed strategy's column-tile kernel of that tile width have its LDS; *lds_rows = rows of B
+// that fit a workgroup's LDS next to its staging tiles.
+int routed_tiles_prepare(int tile_width, int* lds_rows);
 // Lets the sweep kernels for row length k have their LDS; *per_cu = workgroups of them one CU holds.
 int sweep_prepare_kernels(int64_t k, int* per_cu);
 // Wavefronts per workgroup of the sweep kernel for row length k.

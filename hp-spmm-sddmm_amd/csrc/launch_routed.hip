@@ -20,10 +20,38 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
   if (prep_blocks > 0) {
     hipLaunchKernelGGL((hpspmm::routed_prepare_kernel<K, kLd>), dim3((unsigned)prep_blocks), dim3(hpspmm::kBlock), 0, st,
                        p->n_bhot, gather_blocks, p->d_bhot_src, B, p->d_bhot, p->nnz, p->lay.nhub + 1, v, p->d_lslot,
-                       p->d_chunk_base, p->d_chunk_pref, p->d_vval, ld);
+                       p->d_chunk_base, p->d_chunk_pref, p->d_vval, ld, p->lay.tile_width);
     mark_launch(st, "routed_prepare_kernel");
   }
-  if (p->routed_grid > 0) {
+  if (p->lay.tile_width > 0 && p->routed_grid > 0) {
+    // Column-tile phases: one launch over all tiles; with routed_split_launch one per tile and part
+    // (hub classes, cold class).
+    if constexpr (kLd == 0) {
+      const bool split = p->routed_split_launch;
+      const int parts = split ? 2 * p->lay.tiles : 1;
+      for (int part = 0; part < parts; ++part) {
+        const int64_t tile0 = (int64_t)(part / 2) * p->lay.tile_grid;
+        const int64_t first = !split ? 0 : part % 2 ? tile0 + p->lay.hub_grid : tile0;
+        const int64_t last = !split ? p->routed_grid : part % 2 ? tile0 + p->lay.tile_grid : tile0 + p->lay.hub_grid;
+        if (last <= first) continue;
+        const dim3 grid((unsigned)(last - first));
+        constexpr int WPB = hpspmm::kRoutedTileWaves;
+        auto launch = [&](auto kernel, size_t lds) {
+          hipLaunchKernelGGL(kernel, grid, dim3(WPB * 64), lds, st, p->lay, p->d_rvptr, p->d_coldptr, p->d_vcol,
+                             p->d_vval, p->d_run_row, p->d_seg_run, p->d_zero_rows, B, p->d_bhot, p->d_partial,
+                             p->d_carry, C, first, (uint32_t)K, p->n_bhot);
+        };
+        if (p->lay.tile_width == 32)
+          launch(hpspmm::spmm_routed_tiles_kernel<32, WPB>, hpspmm::routed_tiles_lds_bytes<32, WPB>(p->lay.lds_rows));
+        else
+          launch(hpspmm::spmm_routed_tiles_kernel<64, WPB>, hpspmm::routed_tiles_lds_bytes<64, WPB>(p->lay.lds_rows));
+        mark_launch(st, !split ? "spmm_routed_tiles_kernel" : part % 2 ? "spmm_routed_tiles_kernel(cold class)"
+                                                                       : "spmm_routed_tiles_kernel(hub classes)");
+      }
+    } else {
+      return fail(HPSPMM_ERR_INVALID_ARG, "a plan of column-tile phases serves whole rows only");
+    }
+  } else if (p->routed_grid > 0) {
     // One launch; a plan created with hpspmm_plan_options.routed_split_launch (diagnostics: per-class
     // times and counters) issues one per phase of the hub classes and one for the cold class, each
     // from its first workgroup on.
@@ -52,17 +80,37 @@ int launch_routed(const hpspmm_plan* p, const float* v, const float* B, float* C
   }
   const int64_t routed_blocks = row_blocks(p->lay.n_routed, K);
   const int64_t cross_blocks = row_blocks(p->n_cross, K);
-  const int64_t fin_blocks = routed_blocks + cross_blocks + row_blocks(p->n_zero, K);
+  // (under column-tile phases the main kernel has written the rows without nonzeros)
+  const int64_t n_zero = p->lay.tile_width > 0 ? 0 : p->n_zero;
+  const int64_t fin_blocks = routed_blocks + cross_blocks + row_blocks(n_zero, K);
   if (fin_blocks > 0) {
     hipLaunchKernelGGL((hpspmm::spmm_routed_final_kernel<K, kLd>), dim3((unsigned)fin_blocks), dim3(hpspmm::kBlock), 0, st,
                        p->lay, p->d_rvptr, p->d_coldptr, p->d_routed_rows, routed_blocks, p->d_cross_rows, p->n_cross,
-                       cross_blocks, p->d_zero_rows, p->n_zero, p->d_partial, p->d_carry, C, ld);
+                       cross_blocks, p->d_zero_rows, n_zero, p->d_partial, p->d_carry, C, ld);
     mark_launch(st, "spmm_routed_final_kernel");
   }
   return HPSPMM_OK;
 }
 
 }  // namespace
+
+namespace {
+// LDS one workgroup of the column-tile kernel may use at most (of the CU's 160 KB).
+constexpr int kRoutedTilesLdsBudget = 152 << 10;
+template <int W>
+int routed_tiles_prepare_w(int* lds_rows) {
+  constexpr int WPB = hpspmm::kRoutedTileWaves;
+  const int rows = (int)((kRoutedTilesLdsBudget - hpspmm::routed_tiles_lds_bytes<W, WPB>(0)) / ((W + hpspmm::kTileLdsPad) * 4));
+  HPSPMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hpspmm::spmm_routed_tiles_kernel<W, WPB>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, kRoutedTilesLdsBudget));
+  *lds_rows = rows;
+  return HPSPMM_OK;
+}
+}  // namespace
+
+int routed_tiles_prepare(int tile_width, int* lds_rows) {
+  return tile_width == 32 ? routed_tiles_prepare_w<32>(lds_rows) : routed_tiles_prepare_w<64>(lds_rows);
+}
 
 int launch_routed_plan(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st, int ld_mode,
                        uint32_t ld, bool values_ready) {

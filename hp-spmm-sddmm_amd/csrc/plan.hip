@@ -502,6 +502,7 @@ HPSPMM_API int hpspmm_plan_create_ex(int64_t rows, int64_t cols, int64_t nnz, co
   if (!(o.routed_tile_width == 0 || o.routed_tile_width == -1 || o.routed_tile_width == 32 || o.routed_tile_width == 64))
     return fail(HPSPMM_ERR_INVALID_ARG, "routed_tile_width must be 0, -1, 32 or 64, got %d", o.routed_tile_width);
   o.routed_split_launch = in.routed_split_launch != 0;
+  o.routed_lds_rows = in.routed_lds_rows;
   if (in.xcd_dealing < 0 || in.xcd_dealing > 2) return fail(HPSPMM_ERR_INVALID_ARG, "xcd_dealing must be 0, 1 or 2");
   o.xcd_dealing = in.xcd_dealing == 0 ? -1 : in.xcd_dealing == 1 ? 1 : 0;
   o.column_tiles = in.no_column_tiles == 0;
@@ -560,7 +561,8 @@ HPSPMM_API int hpspmm_plan_destroy(hpspmm_plan* plan) {
   if (plan->d_bpad) (void)hipFree(plan->d_bpad);
   for (void* q : {(void*)plan->d_rvptr, (void*)plan->d_coldptr, (void*)plan->d_vcol, (void*)plan->d_lslot,
                   (void*)plan->d_chunk_base, (void*)plan->d_chunk_pref,
-                  (void*)plan->d_vval, (void*)plan->d_vsrc, (void*)plan->d_vrow, (void*)plan->d_bhot_src, (void*)plan->d_partial,
+                  (void*)plan->d_vval, (void*)plan->d_vsrc, (void*)plan->d_vrow, (void*)plan->d_run_row,
+                  (void*)plan->d_seg_run, (void*)plan->d_bhot_src, (void*)plan->d_partial,
                   (void*)plan->d_routed_rows, (void*)plan->d_cross_rows, (void*)plan->d_zero_rows,
                   (void*)plan->d_ostart, (void*)plan->d_ocol, (void*)plan->d_osrc, (void*)plan->d_orow,
                   (void*)plan->d_wcols, (void*)plan->d_tent, (void*)plan->d_ldesc, (void*)plan->d_zrow,

@@ -27,6 +27,12 @@ constexpr double kRoutedMinRoutedShare = 0.3;  // of the nonzeros in rows of at 
 // slice) 4.11 / 4.01 / 4.34 ms with 1 / 2 / 3 phases, K = 64 (7.5 MB a slice) 2.14 / 2.28 /
 // 2.51 ms; R-MAT scale 22, K = 128 (268 MB a slice) 6.63 / 6.23 / 6.32 ms.
 constexpr int64_t kRoutedPhaseBytes = (int64_t)8 << 20;
+// Column-tile phases (see spmm_routed_tiles_kernel), chosen where the slices would otherwise need two
+// phases: tiles of 32 columns; bytes of its slice's compact-buffer rows, within one tile, per XCD (what
+// the 4 MB L2 keeps of them is up to its replacement: R-MAT scale 22, K = 128: 5.74 ms with 2 MB,
+// 5.57 with 4 MB, 5.59 with 8 MB, against 6.08 ms for two phases over whole rows).
+constexpr int kRoutedTileWidth = 32;
+constexpr int64_t kRoutedTileHotBytes = (int64_t)4 << 20;
 
 }  // namespace
 
@@ -44,9 +50,17 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   const int64_t nonempty = std::max<int64_t>(1, rows - p->empty_rows);
   if (!forced && (double)nnz / (double)nonempty < kRoutedMinRowNnz) return HPSPMM_OK;
   if (nnz > INT32_MAX - ((int64_t)1 << 24)) return HPSPMM_OK;  // virtual indices stay int32
+  // Column-tile phases: all XCDs work through B and C one tile of tile_w columns after the other.
+  // For a plan of whole rows of a tuned length only (not for one that is itself a column tile of a
+  // wider product), and not with the values read in place (column-range slices).
+  int tile_w = opt.routed_tile_width > 0    ? opt.routed_tile_width
+               : opt.routed_tile_width == 0 ? (p->cols * k * 4 / hpspmm::kSlices > kRoutedPhaseBytes && !want_sub ? kRoutedTileWidth : 0)
+                                            : 0;
+  if (tile_w && (k % tile_w != 0 || k <= tile_w || p->k_full != k || p->cols >= ((int64_t)1 << 29))) tile_w = 0;
+  const int64_t kw = tile_w ? tile_w : k;  // row length the kernel's sub-waves are made for
   // cached rows per class
-  const int64_t h =
-      std::max<int64_t>(1, ((int64_t)1 << (log2_hubs ? log2_hubs : kRoutedLog2Cached)) / hpspmm::kSlices);
+  const int64_t default_cached = tile_w ? hpspmm::kSlices * kRoutedTileHotBytes / (tile_w * 4) : (int64_t)1 << kRoutedLog2Cached;
+  const int64_t h = std::max<int64_t>(1, (log2_hubs ? (int64_t)1 << log2_hubs : default_cached) / hpspmm::kSlices);
   if (int rc = rank_columns(p, d_col, h * hpspmm::kSlices, st, rk)) return rc;
   if (!forced && (double)rk.served < kRoutedMinShare * (double)nnz) return HPSPMM_OK;
   const int32_t n_ids = (int32_t)rk.n_ids;
@@ -54,6 +68,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   const int64_t slice_bytes = p->cols * k * 4 / hpspmm::kSlices;
   int nsub = slice_bytes > kRoutedPhaseBytes ? 2 : 1;
   if (want_sub) nsub = std::min(want_sub, hpspmm::kMaxSub);
+  if (tile_w) nsub = 1;  // the tiles are the phases
 
   const int64_t n_bhot = h * hpspmm::kSlices;
 
@@ -94,7 +109,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
            (void**)&d_chunk_base, (void**)&d_chunk_row}};
 
   bool inplace = false;
-  if (!sort_values && nsub == 1 && nnz > 0 && p->cols * p->k_full * 4 < ((int64_t)1 << 32) &&
+  if (!sort_values && !tile_w && nsub == 1 && nnz > 0 && p->cols * p->k_full * 4 < ((int64_t)1 << 32) &&
       columns_sorted(p, d_rowptr, d_col, st)) {
     const int groups = nhub;
     const int64_t target = ceil_div(rk.sampled, groups);  // the column counts are those of the sample
@@ -202,8 +217,24 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   lay.shift = p->shift;
   lay.nsub = nsub;
   lay.nhub = nhub;
-  const int64_t subwaves = 64 / (k / 4);
-  const int64_t quantum = ((int64_t)1 << p->shift) * subwaves * hpspmm::kWavesPerBlock;  // nonzeros per workgroup
+  lay.tile_width = tile_w;
+  lay.rows_of_b = p->cols;
+  lay.hub_rows_per_slice = h;
+  int tile_waves = hpspmm::kWavesPerBlock;
+  if (tile_w) {
+    // workgroups of 16 wavefronts, one per CU, whose LDS - what the staging tiles leave of it - holds
+    // the most referenced rows of the class (a multiple of 8 of them: the cold class takes an eighth per slice)
+    tile_waves = hpspmm::kRoutedTileWaves;
+    int room = 0;
+    if (int rc = routed_tiles_prepare(tile_w, &room)) return rc;
+    int lds_rows = opt.routed_lds_rows < 0 ? 0 : opt.routed_lds_rows > 0 ? std::min(opt.routed_lds_rows, room) : room;
+    lds_rows = (int)std::min<int64_t>(lds_rows, h) / hpspmm::kSlices * hpspmm::kSlices;
+    lay.tile_waves = tile_waves;
+    lay.lds_rows = lds_rows;
+  }
+  lay.tiles = tile_w ? (int)(k / tile_w) : 1;
+  const int64_t subwaves = 64 / (kw / 4);
+  const int64_t quantum = ((int64_t)1 << p->shift) * subwaves * tile_waves;  // nonzeros per workgroup
   int64_t at = 0;
   for (int x = 0; x <= nhub; ++x) {
     const int64_t n_x = x < nhub ? (int64_t)origin[x + 1] - (int64_t)origin[x] : (int64_t)cold_total;
@@ -223,6 +254,15 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   }
   lay.phase_begin[nsub] = grid;
   p->routed_grid = grid + lay.cls_blocks[nhub];
+  if (tile_w) {
+    // every tile's range of workgroups begins at a multiple of 8, so that workgroup -> XCD stays slice
+    lay.cold_grid = ceil_div(lay.cls_blocks[nhub], hpspmm::kXcds) * hpspmm::kXcds;
+    lay.n_zero = p->empty_rows;
+    const int64_t zero_per_block = (int64_t)tile_waves * subwaves * hpspmm::kTileZeroRows;
+    lay.hub_grid = grid;
+    lay.tile_grid = grid + lay.cold_grid + ceil_div(ceil_div(p->empty_rows, zero_per_block), hpspmm::kXcds) * hpspmm::kXcds;
+    p->routed_grid = lay.tile_grid * lay.tiles;
+  }
   if (vtotal >= INT32_MAX || p->routed_grid > INT32_MAX) return HPSPMM_OK;
 
   const int64_t nseg = vtotal >> p->shift;
@@ -241,7 +281,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   // the segments strategy's carry slots are not needed any more (the row of every nonzero is, for the fill)
   if (p->d_carry) { (void)hipFree(p->d_carry); p->d_carry = nullptr; }
   if (int rc = ensure_row_expansion(p, d_rowptr, st)) return rc;
-  const size_t total_bytes = rvptr_bytes + coldptr_bytes + 3 * v_bytes +
+  const size_t total_bytes = rvptr_bytes + coldptr_bytes + (tile_w ? 2 : 3) * v_bytes +
                              (inplace ? 0 : lslot_bytes + 2 * chunk_bytes) + partial_bytes + carry_bytes +
                              bhot_bytes + (size_t)n_bhot * 4 + 2 * list_bytes + routed_rows_bytes;
   // (the order of these allocations is felt: with the values allocated after the rows instead of
@@ -301,8 +341,37 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   HPSPMM_HIP(hipGetLastError());
   p->n_cross = counts[0];
   p->n_zero = counts[1];
+  p->lay.n_zero = std::min<int64_t>(counts[1], p->lay.n_zero);  // (the tile grid was sized for the latter)
   (void)hipFree(p->d_nnz_row);  // the row of every nonzero served the fill; the class-major arrays replace it
   p->d_nnz_row = nullptr;
+  if (tile_w) {
+    // The row of every entry becomes a flag in its entry word and one row per run; the row array goes.
+    DeviceTemps tmp;
+    uint32_t *d_flag = nullptr, *d_before = nullptr;
+    if (int rc = tmp.alloc(&d_flag, (size_t)vtotal + 1)) return rc;
+    if (int rc = tmp.alloc(&d_before, (size_t)vtotal + 1)) return rc;
+    hipLaunchKernelGGL(hpspmm::routed_run_flags_kernel, dim3(grid_for(vtotal + 1, 1 << 16)), dim3(hpspmm::kBlock), 0, st,
+                       lay, vtotal, p->d_vrow, d_flag);
+    if (int rc = exclusive_scan_u32(d_flag, d_before, vtotal + 1, st)) return rc;
+    uint32_t n_runs = 0;
+    HPSPMM_HIP(hipMemcpyAsync(&n_runs, d_before + vtotal, sizeof n_runs, hipMemcpyDeviceToHost, st));
+    HPSPMM_HIP(hipStreamSynchronize(st));
+    const size_t run_bytes = (size_t)std::max<uint32_t>(n_runs, 1) * sizeof(int32_t);
+    const size_t seg_bytes = (size_t)std::max<int64_t>(nseg, 1) * sizeof(int32_t);
+    if (hipMalloc(&p->d_run_row, run_bytes) != hipSuccess || hipMalloc(&p->d_seg_run, seg_bytes) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(HPSPMM_ERR_ALLOC, "device allocation for the routed plan failed (%zu bytes)", run_bytes + seg_bytes);
+    }
+    HPSPMM_HIP(hipMemsetAsync(p->d_seg_run, 0, seg_bytes, st));
+    hipLaunchKernelGGL(hpspmm::routed_runs_kernel, dim3(grid_for(vtotal, 1 << 16)), dim3(hpspmm::kBlock), 0, st, lay,
+                       vtotal, d_flag, d_before, p->d_vrow, p->d_vcol, p->d_run_row, p->d_seg_run);
+    HPSPMM_HIP(hipStreamSynchronize(st));
+    HPSPMM_HIP(hipGetLastError());
+    (void)hipFree(p->d_vrow);
+    p->d_vrow = nullptr;
+    p->n_runs = n_runs;
+    p->workspace_bytes += (int64_t)(run_bytes + seg_bytes);
+  }
   p->n_bhot = inplace ? 0 : n_bhot;
   p->n_hub = inplace ? 0 : (int64_t)n_ids;
   p->nseg = nseg;

@@ -69,7 +69,35 @@ struct RoutedLayout {
   int shift;  // log2(segment length)
   int nsub;   // phases
   int nhub;   // 8 * nsub
+  // Column-tile phases (tile_width > 0, then nsub = 1): B and C are worked through in `tiles` tiles of
+  // tile_width columns, one after the other on all XCDs; the workgroups of tile t are
+  // [t * tile_grid, (t + 1) * tile_grid), its first hub_grid (a multiple of 8) the hub classes, the
+  // next cold_grid the cold class, the rest write the tile's zeros of the rows without nonzeros.
+  int tile_width;
+  int tiles;
+  int64_t tile_grid;
+  int64_t hub_grid;
+  int64_t cold_grid;
+  int64_t n_zero;     // rows without nonzeros (listed in zero_rows[])
+  int64_t rows_of_b;  // = columns of A
+  // Its workgroups have tile_waves wavefronts and keep the lds_rows most referenced rows of their
+  // class (of the tile in hand) in LDS: in hub class x the first lds_rows compact-buffer rows of
+  // slice x, in the cold class the first lds_rows / 8 of every slice (ranks 0 .. lds_rows - 1 overall).
+  int tile_waves;
+  int lds_rows;
+  int64_t hub_rows_per_slice;
 };
+
+// Entry word of the class-major order under column-tile phases: bit 31 = the row of B is in the
+// compact buffer (bits 0..29 = its slot there) instead of B (bits 0..29 = the column); bit 30 = first
+// entry of its run (the nonzeros of one row in one class).  The rows of the runs are kept run by run
+// (run_row[]), not nonzero by nonzero, with the run of every segment's first entry (seg_run[]).
+constexpr int32_t kRunStart = 1 << 30;
+constexpr int32_t kInLds = 1 << 29;  // the row is among those the workgroup keeps in LDS (bits 0..28 = which)
+constexpr int32_t kEntryPayload = kInLds - 1;
+constexpr int kRoutedTileWaves = 16;  // wavefronts per workgroup of the column-tile kernel
+constexpr int kTileZeroRows = 8;  // rows without nonzeros written per sub-wave of a zero-writing workgroup
+constexpr int kTileLdsPad = 4;  // floats between the rows of the LDS copy: rows of different sub-waves on different banks
 
 // ---- plan-time kernels -----------------------------------------------------
 
@@ -233,6 +261,64 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_count_kernel(int64_t n_chunk
     }
   }
   if (lane < nhub) cnt[(int64_t)lane * n_chunks + c] = mine;
+}
+
+// Class of the class-major position q, or -1 for the padding between the classes.
+__device__ __forceinline__ int routed_class_of_position(const RoutedLayout& lay, int64_t q) {
+  for (int x = 0; x <= lay.nhub; ++x)
+    if (q >= lay.cls_begin[x] && q < lay.cls_end[x]) return x;
+  return -1;
+}
+
+// flag[q] = 1 if position q holds the first entry of a run (q < vtotal), flag[vtotal] = 0 (the
+// scan's total slot).  vrow[q] = routed-row number (hub classes) or row (cold class) of the entry.
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_run_flags_kernel(RoutedLayout lay, int64_t vtotal,
+                                                                     const int32_t* __restrict__ vrow,
+                                                                     uint32_t* __restrict__ flag) {
+  for (int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x; q <= vtotal; q += (int64_t)gridDim.x * kBlock) {
+    uint32_t f = 0;
+    if (q < vtotal) {
+      const int x = routed_class_of_position(lay, q);
+      if (x >= 0) f = q == lay.cls_begin[x] || vrow[q] != vrow[q - 1];
+    }
+    flag[q] = f;
+  }
+}
+
+// before[q] = run starts before position q (the exclusive scan of flag).  Every entry word gets its
+// final form (see kRunStart); run_row[r] = row of run r; seg_run[g] = run of the first entry of
+// segment g (segments that begin in the padding between classes are never read).
+HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_runs_kernel(RoutedLayout lay, int64_t vtotal,
+                                                                const uint32_t* __restrict__ flag,
+                                                                const uint32_t* __restrict__ before,
+                                                                const int32_t* __restrict__ vrow,
+                                                                int32_t* __restrict__ vent,
+                                                                int32_t* __restrict__ run_row,
+                                                                int32_t* __restrict__ seg_run) {
+  for (int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x; q < vtotal; q += (int64_t)gridDim.x * kBlock) {
+    const uint32_t f = flag[q];
+    const int32_t w = vent[q];  // column, or ~slot
+    const bool hot = w < 0;
+    const int x = routed_class_of_position(lay, q);
+    int32_t payload = hot ? ~w : w;
+    bool in_lds = false;
+    if (hot && x >= 0 && lay.lds_rows > 0) {
+      const int64_t h = lay.hub_rows_per_slice;
+      const int64_t slice = payload / h, place = payload - slice * h;
+      if (x < lay.nhub) {
+        in_lds = slice == x && place < lay.lds_rows;
+        if (in_lds) payload = (int32_t)place;
+      } else {
+        const int per = lay.lds_rows / kSlices;
+        in_lds = place < per;
+        if (in_lds) payload = (int32_t)(slice * per + place);
+      }
+    }
+    vent[q] = (hot ? INT32_MIN : 0) | (in_lds ? kInLds : 0) | (payload & kEntryPayload) | (f ? kRunStart : 0);
+    if (f) run_row[before[q]] = vrow[q];
+    if ((q & (((int64_t)1 << lay.shift) - 1)) == 0 && x >= 0)
+      seg_run[q >> lay.shift] = (int32_t)(before[q] + f) - 1;
+  }
 }
 
 // Three-pass exclusive scan of uint32 (n up to 2^32, total < 2^32).
@@ -510,7 +596,8 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
                                                                 const uint16_t* __restrict__ lslot,
                                                                 const int32_t* __restrict__ chunk_base,
                                                                 const int32_t* __restrict__ chunk_pref,
-                                                                float* __restrict__ vval, uint32_t ld_arg) {
+                                                                float* __restrict__ vval, uint32_t ld_arg,
+                                                                int tile_width = 0) {
   constexpr int G = K / 4;
   __shared__ float s_buf[kPermChunk];
   __shared__ int32_t s_base[kMaxClasses];
@@ -522,7 +609,12 @@ __global__ __launch_bounds__(kBlock) void routed_prepare_kernel(int64_t n_bhot, 
     if (s >= n_bhot) return;
     const int32_t c = src[s];
     if (c < 0) return;
-    *reinterpret_cast<float4*>(Bhot + (uint64_t)s * K + 4 * l) =
+    // column-tile phases keep the buffer tile by tile (tile t of every cached row, then tile t + 1),
+    // so that what one phase reads is one dense stretch of memory
+    const int tile = tile_width ? 4 * l / tile_width : 0;
+    float* dst = tile_width ? Bhot + ((uint64_t)tile * n_bhot + s) * tile_width + (4 * l - tile * tile_width)
+                            : Bhot + (uint64_t)s * K + 4 * l;
+    *reinterpret_cast<float4*>(dst) =
         lane_columns<K, kLd>(ld_arg, l) > 0 ? load_b_ld(B, c, l, row_length<K, kLd>(ld_arg)) : make_float4(0.f, 0.f, 0.f, 0.f);
     return;
   }
@@ -693,6 +785,157 @@ __global__ __launch_bounds__(kBlock) void spmm_routed_kernel(RoutedLayout lay, c
     wave_lds_fence();
   }
   flush_to((int64_t)vp[(int64_t)(cur + 1) * vstride] > e);
+}
+
+// The same work under column-tile phases (RoutedLayout::tile_width = W): workgroup b serves tile
+// b / tile_grid of B and C - W columns of rows that are `ld` floats long - and, within the tile's
+// range of workgroups, hub class (b % 8) - on XCD b % 8 - or the cold class.  All XCDs are on one
+// tile at a time, so an L2 has to hold W / ld of what it would of whole rows: four times as many of
+// its slice's hot rows of B stay resident at W = 32, ld = 128, for no partial-result row more (the
+// runs of a row in the 8 classes are what they were; every tile writes its W columns of them).  The
+// price: the streams are read once per tile - hence entry words that carry the run starts (8 bytes
+// per nonzero with the value, instead of 12 with a row word) - and every gather is W * 4 bytes.
+// Carry slots and partial-result rows are `ld` floats long, as the final kernel reads them.
+// WPB = wavefronts per workgroup (RoutedLayout::tile_waves).  Dynamic LDS: the staging tiles of the
+// workgroup's sub-waves, then lds_rows rows of W + kTileLdsPad floats: the most referenced rows of the
+// workgroup's class, copied from the compact buffer when the workgroup starts.  A gather is one flat
+// load whose address is selected between that copy, the compact buffer and B.  (What bounds the
+// kernel is how many requests a CU's L1 can have under way to the L2: with L2 hits and misses mixed
+// it sustains about 115 G lines/s, the fabric idling - every gather the LDS serves is one request fewer.)
+template <int W, int WPB>
+__global__ __launch_bounds__(WPB * 64) void spmm_routed_tiles_kernel(
+    RoutedLayout lay, const int32_t* __restrict__ rvptr, const int32_t* __restrict__ coldptr,
+    const int32_t* __restrict__ vent, const float* __restrict__ vval, const int32_t* __restrict__ run_row,
+    const int32_t* __restrict__ seg_run, const int32_t* __restrict__ zero_rows, const float* __restrict__ B,
+    const float* __restrict__ Bhot, float* __restrict__ partial, float* __restrict__ carry, float* __restrict__ C,
+    int64_t first_block, uint32_t ld, int64_t n_bhot) {
+  constexpr int G = W / 4;
+  constexpr int P = 64 / G;
+  constexpr int TL = kTile / G;
+  constexpr int kStage = WPB * P * kTileStride;
+  constexpr int kRow = W + kTileLdsPad;
+  extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
+  int32_t* s_col = reinterpret_cast<int32_t*>(s_raw);
+  float* s_val = reinterpret_cast<float*>(s_col + kStage);
+  int32_t* s_row = reinterpret_cast<int32_t*>(s_val + kStage);
+  float* s_b = reinterpret_cast<float*>(s_row + kStage);  // [lds_rows][kRow]
+
+  const int64_t bid = (int64_t)blockIdx.x + first_block;
+  const int64_t tile = bid / lay.tile_grid;
+  const int64_t rel = bid - tile * lay.tile_grid;
+  const int nhub = lay.nhub;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int l = lane % G;
+  const uint32_t k0 = (uint32_t)tile * W;  // first column of the tile
+  if (rel >= lay.hub_grid + lay.cold_grid) {
+    // The tile's columns of the rows without nonzeros, kTileZeroRows rows per sub-wave, after the
+    // tile's other work (as part of the final kernel these rows were half its time; spread among the
+    // hub workgroups instead, their lines pushed rows of B out of the L2s and cost more than they hid).
+    const int64_t first = ((rel - lay.hub_grid - lay.cold_grid) * (WPB * P) + (tid >> 6) * P + lane / G) * kTileZeroRows;
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int64_t j = first; j < first + kTileZeroRows && j < lay.n_zero; ++j)
+      store_result(C + (uint64_t)(uint32_t)zero_rows[j] * ld + k0 + 4 * l, zero);
+    return;
+  }
+  const bool hub = rel < lay.hub_grid;
+  const int x = hub ? (int)(rel % kSlices) : nhub;
+  const int64_t i = hub ? rel / kSlices : rel - lay.hub_grid;
+  if (i >= lay.cls_blocks[x]) return;
+
+  const float* hot_tile = Bhot + (uint64_t)tile * (uint64_t)n_bhot * W;
+
+  // the class's most referenced rows (of this tile) into LDS; every thread of the workgroup reaches the barrier
+  {
+    const int rows = lay.lds_rows;
+    const int per = rows / kSlices;
+    for (int j = tid; j < rows * G; j += WPB * 64) {
+      const int slot = j / G, part = j - slot * G;
+      const int64_t src = hub ? (int64_t)x * lay.hub_rows_per_slice + slot
+                              : (int64_t)(slot / per) * lay.hub_rows_per_slice + slot % per;
+      *reinterpret_cast<float4*>(s_b + slot * kRow + 4 * part) =
+          *reinterpret_cast<const float4*>(hot_tile + (uint64_t)src * W + 4 * part);
+    }
+    __syncthreads();
+  }
+
+  const int shift = lay.shift;
+  const int64_t g = (lay.cls_begin[x] >> shift) + (i * WPB + (tid >> 6)) * P + lane / G;
+  const int64_t s = g << shift;
+  const int64_t cls_end = lay.cls_end[x];
+  if (s >= cls_end) return;
+  const int64_t e = (s + ((int64_t)1 << shift)) < cls_end ? (s + ((int64_t)1 << shift)) : cls_end;
+  const int sbase = ((tid >> 6) * P + lane / G) * kTileStride;
+  const int32_t* vp = hub ? rvptr + x : coldptr;
+  const int64_t vstride = hub ? nhub : 1;
+  float* out = (hub ? partial + (uint64_t)x * ld : C) + k0 + 4 * l;
+  const uint64_t ostride = hub ? (uint64_t)nhub * ld : (uint64_t)ld;
+  float* cslot = carry + (uint64_t)(2 * g) * ld + k0 + 4 * l;
+  const float* bt = B + k0 + 4 * l;
+  const float* hot_t = hot_tile + 4 * l;
+  const float* lds_t = s_b + 4 * l;
+
+  // `run` = the run of the entry before the next tile to be fetched: to begin with, the run of the
+  // segment's first entry, less one if that entry starts it
+  const int32_t first_run = seg_run[g];
+  int32_t run = first_run - ((vent[s] & kRunStart) != 0);
+  int32_t cur = run_row[first_run];
+  bool head_pending = (int64_t)vp[(int64_t)cur * vstride] < s;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+
+  auto flush_to = [&](bool is_tail) {
+    float* dst = head_pending ? cslot : (is_tail ? cslot + ld : out + (uint64_t)(uint32_t)cur * ostride);
+    head_pending = false;
+    store_result(dst, acc);
+  };
+  auto flush = [&]() { flush_to(false); };
+  auto loadb = [&](int32_t c) {
+    const uint32_t idx = (uint32_t)(c & kEntryPayload);
+    const float* mem = c < 0 ? hot_t + (uint64_t)idx * W : bt + (uint64_t)idx * ld;
+    const float* src = (c & kInLds) ? lds_t + idx * kRow : mem;
+    return *reinterpret_cast<const float4*>(src);
+  };
+  // One tile of entries into registers: entry words and values as they lie, the row of every entry
+  // from the run starts - a lane counts those among its TL entries, the sub-wave scans the counts, and
+  // run_row[] (a few lines, reused by every tile of the segment) gives the rows.
+  auto fetch = [&](TileRegs<TL>& m, int64_t t) {
+    const int64_t q = t + l * TL;
+    load_run<TL>(m.c, vent, q, e, true);  // 0 beyond e: a plain entry of the run before
+    load_run<TL>(m.v, vval, q, e, true);
+    int32_t starts = 0;
+#pragma unroll
+    for (int j = 0; j < TL; ++j) starts += (m.c[j] & kRunStart) != 0;
+    int32_t incl = starts;
+#pragma unroll
+    for (int off = 1; off < G; off <<= 1) {
+      const int32_t o = __shfl_up(incl, off, G);
+      if (l >= off) incl += o;
+    }
+    int32_t at = run + incl - starts;
+#pragma unroll
+    for (int j = 0; j < TL; ++j) {
+      at += (m.c[j] & kRunStart) != 0;
+      m.r[j] = run_row[at];
+    }
+    run += __shfl(incl, G - 1, G);
+  };
+  TileRegs<TL> m;
+  fetch(m, s);
+  for (int64_t t = s; t < e; t += kTile) {
+    stage_tile<TL>(m, sbase + l * TL, s_col, s_val, s_row);
+    wave_lds_fence();
+    if (t + kTile < e) fetch(m, t + kTile);
+    const int cnt = (e - t) < kTile ? (int)(e - t) : kTile;
+    consume_tile(cnt, sbase, s_col, s_val, s_row, cur, acc, loadb, flush);
+    wave_lds_fence();
+  }
+  flush_to((int64_t)vp[(int64_t)(cur + 1) * vstride] > e);
+}
+
+// Bytes of dynamic LDS of one such workgroup.
+template <int W, int WPB>
+constexpr size_t routed_tiles_lds_bytes(int lds_rows) {
+  return (size_t)3 * WPB * (64 / (W / 4)) * kTileStride * 4 + (size_t)lds_rows * (W + kTileLdsPad) * 4;
 }
 
 // list[] <- every row whose action byte equals `which` (order unspecified); *count must be zero on entry.

@@ -120,6 +120,8 @@ typedef struct hpspmm_plan_options {
   int32_t routed_tile_width;  /* routed strategy: 32 / 64 = work through B and C in column tiles of that
                                  width, one after the other on all XCDs (k a multiple of it); -1 = never */
   int32_t routed_split_launch; /* 1: hub phases and cold class as launches of their own (per-class timing) */
+  int32_t routed_lds_rows;    /* column tiles of the routed strategy: rows of B a workgroup keeps in LDS (at most
+                                 what fits; -1 = none) */
   int32_t xcd_dealing;        /* 0: probe how workgroups are dealt to the XCDs (once per device and process);
                                  1: take workgroup b to run on XCD b % 8; 2: take it not to */
   int32_t no_column_tiles;    /* 1: a k outside 32 / 64 / 128 never gets the sweep / routed / ordered

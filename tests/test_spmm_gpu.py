@@ -66,7 +66,22 @@ def _strategies(capi):
             ("routed_3phases", capi.PLAN_FORCE_ROUTED | capi.plan_routed_phases(3) | capi.plan_routed_row_log2(4)),
             ("routed_7phases_tiny", capi.PLAN_FORCE_ROUTED | capi.plan_routed_phases(7) | capi.plan_hub_log2(5)
              | capi.plan_segment_shift(3) | capi.plan_routed_row_log2(1)),
-            ("sweep", capi.PLAN_FORCE_SWEEP)]
+            ("sweep", capi.PLAN_FORCE_SWEEP),
+            # routed in column-tile phases (only where K is a multiple of the tile width and wider; otherwise
+            # these are plain routed plans)
+            ("routed_tiles32", capi.flags_with_options(capi.PLAN_FORCE_ROUTED, routed_tile_width=32)),
+            ("routed_tiles64_tiny", capi.flags_with_options(
+                capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(5) | capi.plan_segment_shift(3) | capi.plan_routed_row_log2(1),
+                routed_tile_width=64)),
+            ("routed_tiles32_no_lds", capi.flags_with_options(
+                capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(7) | capi.plan_routed_row_log2(3),
+                routed_tile_width=32, routed_lds_rows=-1)),
+            ("routed_tiles32_lds16", capi.flags_with_options(
+                capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(12) | capi.plan_routed_row_log2(5),
+                routed_tile_width=32, routed_lds_rows=16)),
+            ("routed_tiles32_s16", capi.flags_with_options(
+                capi.PLAN_FORCE_ROUTED | capi.plan_hub_log2(10) | capi.plan_segment_shift(4) | capi.plan_routed_row_log2(3),
+                routed_tile_width=32))]
 
 
 @pytest.mark.parametrize("k", [32, 64, 128])

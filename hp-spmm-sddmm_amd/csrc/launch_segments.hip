@@ -107,15 +107,19 @@ int launch_ordered(const hpspmm_plan* p, const int32_t* rp, const float* v, cons
   if (grid > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   if (p->nnz > 0) {
     hipLaunchKernelGGL((hpspmm::spmm_ordered_kernel<K, kLd>), dim3((unsigned)grid), dim3(hpspmm::kBlock),
-                       (size_t)p->ocap * K * sizeof(float), st, rp, p->d_ostart, p->d_ocol, p->d_osrc, p->d_orow, v,
-                       p->d_wcols, p->ocap, B, C, p->d_carry, p->nnz, p->shift, nblocks, p->xcd_remap, ld);
+                       (size_t)p->ocap * K * sizeof(float), st, rp, p->d_ostart, p->d_ocol, p->d_run_row, p->d_run_delta,
+                       p->d_seg_run, v, p->d_wcols, p->ocap, B, C, p->d_carry, p->nnz, p->shift, nblocks, p->xcd_remap,
+                       ld);
     mark_launch(st, "spmm_ordered_kernel");
   }
-  const int rpw = fixup_rows_per_wave(p->rows, K);
-  const int64_t fix_blocks = ceil_div(ceil_div(p->rows, rpw), hpspmm::kWavesPerBlock);
-  hipLaunchKernelGGL((hpspmm::spmm_fixup_kernel<K, kLd>), dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0, st,
-                     p->rows, rp, p->d_ostart, p->d_carry, C, p->shift, rpw, ld);
-  mark_launch(st, "spmm_fixup_kernel");
+  const int64_t cross_blocks = row_blocks(p->n_cross, K);
+  const int64_t fix_blocks = cross_blocks + row_blocks(p->n_zero, K);
+  if (fix_blocks > 0) {
+    hipLaunchKernelGGL((hpspmm::spmm_ordered_fixup_kernel<K, kLd>), dim3((unsigned)fix_blocks), dim3(hpspmm::kBlock), 0,
+                       st, rp, p->d_ostart, p->d_cross_rows, p->n_cross, cross_blocks, p->d_zero_rows, p->n_zero,
+                       p->d_carry, C, p->shift, ld);
+    mark_launch(st, "spmm_ordered_fixup_kernel");
+  }
   return HPSPMM_OK;
 }
 

@@ -21,15 +21,21 @@
 //     the tile engine of the segments kernel, reading a slotted column from
 //     LDS and every other one from memory.
 //
-// The values are read in place through the nonzeros' original indices (a row's
-// nonzeros stay contiguous, so these loads remain coalesced).  Rows cut by a
-// segment boundary go through the carry slots exactly as in the segments
-// strategy; the fix-up kernel is shared.
+// A row's nonzeros keep their stored order, so what the kernel streams is one
+// entry word per nonzero - column or LDS slot, and a flag on the first entry of
+// every row (kRunStart, as in the routed strategy's column tiles) - and the
+// value, read where the caller keeps it: a row's values are contiguous there,
+// at the entry's position plus a per-row offset.  Rows and offsets are kept row
+// by row (run_row, run_delta).  8 bytes per nonzero; with a column, a source
+// index and a row per nonzero it was 16 (co-purchase graph, K = 64: 2.93 -> 2.8 ms).
+// Rows cut by a segment boundary go through the carry slots exactly as in the
+// segments strategy; a fix-up kernel adds them up from the plan's list of such rows.
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "routed_kernels.hpp"
 #include "spmm_kernels.hpp"
 
 namespace hpspmm {
@@ -191,10 +197,11 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void cluster_init_kernel(int64_t rows, i
   if (r < rows) label[r] = (int32_t)r;
 }
 
-// len[i] = number of nonzeros of the i-th row in processing order; len[rows] = 0.
+// len[i] = number of nonzeros of the i-th row in processing order, some[i] = 1 if it has any;
+// len[rows] = some[rows] = 0.
 HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_len_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                              const int32_t* __restrict__ order,
-                                                             uint32_t* __restrict__ len) {
+                                                             uint32_t* __restrict__ len, uint32_t* __restrict__ some) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i > rows) return;
   uint32_t n = 0;
@@ -203,6 +210,7 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_len_kernel(int64_t rows, co
     n = (uint32_t)(rowptr[r + 1] - rowptr[r]);
   }
   len[i] = n;
+  some[i] = n != 0;
 }
 
 // seen[order[i]] += 1: a permutation leaves every counter at exactly one.
@@ -219,16 +227,20 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_mark_kernel(int64_t rows, c
   if (atomicAdd(&seen[r], 1) != 0) atomicOr(bad, 2);
 }
 
-// Lays the nonzeros out in processing order.  One wavefront per position i:
-// row r = order[i] starts at pstart[i]; start[r] = pstart[i];
-// ocol / osrc / orow = column, original index and row of every nonzero.
+// Lays the nonzeros out in processing order.  One wavefront per position i: row r = order[i] starts
+// at pstart[i] and is run prun[i] (the scans of len and some); start[r] = pstart[i].  oent = the
+// column of every nonzero, a row's nonzeros in stored order, the first one flagged kRunStart;
+// run_row / run_delta of the row's run; seg_run[g] for every segment that begins within the row.
 HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_fill_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                               const int32_t* __restrict__ col,
                                                               const int32_t* __restrict__ order,
                                                               const uint32_t* __restrict__ pstart,
+                                                              const uint32_t* __restrict__ prun, int shift,
                                                               int32_t* __restrict__ start,
-                                                              int32_t* __restrict__ ocol, int32_t* __restrict__ osrc,
-                                                              int32_t* __restrict__ orow) {
+                                                              int32_t* __restrict__ oent,
+                                                              int32_t* __restrict__ run_row,
+                                                              int32_t* __restrict__ run_delta,
+                                                              int32_t* __restrict__ seg_run) {
   const int lane = threadIdx.x & 63;
   const int64_t i = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   if (i >= rows) return;
@@ -237,19 +249,23 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_fill_kernel(int64_t rows, c
   const int32_t hb = rowptr[r + 1];
   const int32_t p0 = (int32_t)pstart[i];
   if (lane == 0) start[r] = p0;
-  for (int32_t j = lb + lane; j < hb; j += 64) {
-    const int32_t p = p0 + (j - lb);
-    ocol[p] = col[j];
-    osrc[p] = j;
-    orow[p] = r;
+  if (hb == lb) return;
+  const int32_t run = (int32_t)prun[i];
+  if (lane == 0) {
+    run_row[run] = r;
+    run_delta[run] = lb - p0;
   }
+  const int64_t seg = (int64_t)1 << shift;
+  for (int64_t g = (p0 + seg - 1) / seg + lane; g * seg < (int64_t)p0 + (hb - lb); g += 64) seg_run[g] = run;
+  for (int32_t j = lb + lane; j < hb; j += 64) oent[p0 + (j - lb)] = col[j] | (j == lb ? kRunStart : 0);
 }
 
 // Per window of `window` consecutive nonzeros (in processing order; window <=
 // kOrderedMaxWindow): the columns that occur at least twice, the `cap` most
 // frequent of them (ties: an occurrence count is either kept whole or dropped
 // whole), in increasing column order -> wcols[w * cap + slot] (-1 = unused
-// slot); the nonzeros of those columns get ocol = ~slot.  One workgroup per
+// slot); the entry words of those columns (ocol: column in bits 0..28, kRunStart)
+// get bit 31 and the slot for the column.  One workgroup per
 // window.  Most columns of a window occur once, so two bitmaps first tell which
 // hash values were seen twice; only those nonzeros are counted exactly, in an LDS
 // hash table (as many slots as a window has nonzeros: it cannot overflow);
@@ -289,14 +305,14 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_hot_kernel(int64_t nnz, int
   __syncthreads();
   auto bit_of = [](int32_t c) { return ((uint32_t)c * 0x9E3779B1u) >> 17; };  // 15 bits
   for (int i = tid; i < n; i += kBlock) {
-    const uint32_t h = bit_of(ocol[p0 + i]);
+    const uint32_t h = bit_of(ocol[p0 + i] & kEntryPayload);
     const uint32_t m = 1u << (h & 31);
     if (atomicOr(&s_once[h >> 5], m) & m) atomicOr(&s_twice[h >> 5], m);
   }
   __syncthreads();
   // exact counts of the columns whose hash value was seen twice
   for (int i = tid; i < n; i += kBlock) {
-    const int32_t c = ocol[p0 + i];
+    const int32_t c = ocol[p0 + i] & kEntryPayload;
     const uint32_t h = bit_of(c);
     if (!((s_twice[h >> 5] >> (h & 31)) & 1u)) continue;
     uint32_t slot = ((uint32_t)c * 0x85EBCA6Bu) >> 19;  // 13 bits
@@ -346,7 +362,8 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_hot_kernel(int64_t nnz, int
   for (int i = tid; i < cap; i += kBlock) wcols[w * cap + i] = i < m ? s_sel[i] : -1;
   unsigned long long mine = 0;
   for (int i = tid; i < n; i += kBlock) {
-    const int32_t c = ocol[p0 + i];
+    const int32_t w = ocol[p0 + i];
+    const int32_t c = w & kEntryPayload;
     int lo = 0, hi = m;
     while (lo < hi) {
       const int mid = (lo + hi) >> 1;
@@ -354,7 +371,7 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_hot_kernel(int64_t nnz, int
       else hi = mid;
     }
     if (lo < m && s_sel[lo] == c) {
-      ocol[p0 + i] = ~lo;
+      ocol[p0 + i] = INT32_MIN | (w & kRunStart) | lo;  // the LDS slot, the first-of-row flag kept
       ++mine;
     }
   }
@@ -362,57 +379,32 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_hot_kernel(int64_t nnz, int
   if ((tid & 63) == 0 && mine) atomicAdd(served, mine);
 }
 
-// Within every row, the nonzeros that read B from memory first, those that read
-// it from LDS last (each group in its previous order): the gathers are issued
-// in batches, and a batch is as slow as its slowest load.  One wavefront per
-// row; a row cut by a window boundary is left as it is (its slots belong to
-// two different windows).
-HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_partition_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
-                                                                   const int32_t* __restrict__ start, int window,
-                                                                   int32_t* __restrict__ ocol,
-                                                                   int32_t* __restrict__ osrc) {
-  const int lane = threadIdx.x & 63;
-  const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+// What the fix-up kernel has to do with every row: write zeros (kActionZero: no nonzeros), add carry
+// slots (kActionCross: its nonzeros lie in more than one segment), or nothing.
+HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_action_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
+                                                                   const int32_t* __restrict__ start, int shift,
+                                                                   uint8_t* __restrict__ action) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (r >= rows) return;
-  const int32_t n = rowptr[r + 1] - rowptr[r];
-  if (n < 2) return;
-  const int32_t p0 = start[r];
-  if (p0 / window != (p0 + n - 1) / window) return;
-  // count the memory group, then place both groups; chunks of 64 keep their relative order
-  int32_t n_mem = 0;
-  for (int32_t i0 = 0; i0 < n; i0 += 64) {
-    const int32_t i = i0 + lane;
-    const bool mem = i < n && ocol[p0 + i] >= 0;
-    n_mem += (int32_t)__popcll(__ballot(mem));
-  }
-  if (n_mem == 0 || n_mem == n) return;
-  // rows longer than 64 would be overwritten while still being read: stage them through registers in
-  // chunks only when the whole row fits one chunk, else leave the row unchanged
-  if (n > 64) return;
-  const bool valid = lane < n;
-  const int32_t c = valid ? ocol[p0 + lane] : 0;
-  const int32_t sidx = valid ? osrc[p0 + lane] : 0;
-  const bool mem = valid && c >= 0;
-  const uint64_t m_mem = __ballot(mem);
-  const uint64_t m_lds = __ballot(valid && !mem);
-  const uint64_t below = (1ull << lane) - 1ull;
-  if (valid) {
-    const int32_t dst = mem ? (int32_t)__popcll(m_mem & below) : n_mem + (int32_t)__popcll(m_lds & below);
-    ocol[p0 + dst] = c;
-    osrc[p0 + dst] = sidx;
-  }
+  const int32_t len = rowptr[r + 1] - rowptr[r];
+  const int64_t p0 = start[r];
+  action[r] = len == 0 ? kActionZero : (p0 >> shift) != ((p0 + len - 1) >> shift) ? kActionCross : kActionNone;
 }
 
 // ---- SpMM kernel -----------------------------------------------------------
 
 // One workgroup per window = kWavesPerBlock * P segments of 2^shift nonzeros.
 // Dynamic LDS: cap * K floats, the window's slotted rows of B.
+// oent = entry words (bit 31: bits 0..29 are an LDS slot, else a column; kRunStart: first entry of
+// its row); run_row / run_delta per run (= non-empty row, in processing order); seg_run[g] = run of
+// segment g's first entry; start[r] = position of row r's first nonzero.
 template <int K, int kLd = 0>
 __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
-    const int32_t* __restrict__ rowptr, const int32_t* __restrict__ start, const int32_t* __restrict__ ocol,
-    const int32_t* __restrict__ osrc, const int32_t* __restrict__ orow, const float* __restrict__ val,
-    const int32_t* __restrict__ wcols, int cap, const float* __restrict__ B, float* __restrict__ C,
-    float* __restrict__ carry, int64_t nnz, int shift, int64_t nblocks, bool remap, uint32_t ld_arg) {
+    const int32_t* __restrict__ rowptr, const int32_t* __restrict__ start, const int32_t* __restrict__ oent,
+    const int32_t* __restrict__ run_row, const int32_t* __restrict__ run_delta, const int32_t* __restrict__ seg_run,
+    const float* __restrict__ val, const int32_t* __restrict__ wcols, int cap, const float* __restrict__ B,
+    float* __restrict__ C, float* __restrict__ carry, int64_t nnz, int shift, int64_t nblocks, bool remap,
+    uint32_t ld_arg) {
   constexpr int G = K / 4;
   constexpr int P = 64 / G;
   constexpr int TL = kTile / G;
@@ -447,7 +439,11 @@ __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
   const bool in_tile = nv > 0;
   const bool c_aligned = c_rows_aligned<kLd>(ld_arg);
   const uint32_t ldc = c_row_length<K, kLd>(ld_arg);
-  int32_t cur = orow[s];
+  // `run` = the run of the entry before the next tile whose rows are looked up: to begin with, the run
+  // of the segment's first entry, less one if that entry starts it
+  const int32_t first_run = seg_run[g];
+  int32_t run = first_run - ((oent[s] & kRunStart) != 0);
+  int32_t cur = run_row[first_run];
   bool head_pending = (int64_t)start[cur] < s;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 
@@ -469,39 +465,113 @@ __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
   // sums are never stored
   const int lg = in_tile ? l : 0;
   auto loadb = [&](int32_t c) {
-    const float* row = c < 0 ? lds_b + (uint32_t)(~c) * (uint32_t)K : B + (uint64_t)(uint32_t)c * (uint64_t)ld;
+    const uint32_t idx = (uint32_t)(c & kEntryPayload);
+    const float* row = c < 0 ? lds_b + idx * (uint32_t)K : B + (uint64_t)idx * (uint64_t)ld;
     return *reinterpret_cast<const float4*>(row + 4 * lg);
   };
 
-  // Two-deep prefetch: the original indices of tile t+2 and, through the indices
-  // fetched one iteration earlier, the values of tile t+1 (the plan's arrays
-  // are allocated by the library, hence always aligned for the vector loads).
-  TileRegs<TL> m;
-  int32_t src[TL];
-  const int64_t q0 = s + l * TL;
-  load_run<TL>(src, osrc, q0, e, true);
-  load_run<TL>(m.c, ocol, q0, e, true);
-  load_run<TL>(m.r, orow, q0, e, true);
+  // Two-deep prefetch.  look(t): the entry words of tile t and, from the run starts among them (a lane
+  // counts those of its TL entries, the sub-wave scans the counts), the row and the value offset of
+  // every entry.  take(t): the values of tile t through the offsets looked up one step earlier.  (The
+  // plan's arrays are allocated by the library, hence always aligned for the vector loads.)
+  int32_t ec[TL], er[TL], ed[TL];
+  auto look = [&](int64_t t) {
+    const int64_t q = t + l * TL;
+    load_run<TL>(ec, oent, q, e, true);  // 0 beyond e: a plain entry of the run before
+    int32_t starts = 0;
 #pragma unroll
-  for (int j = 0; j < TL; ++j) m.v[j] = q0 + j < e ? val[src[j]] : 0.f;
-  if (s + kTile < e) load_run<TL>(src, osrc, q0 + kTile, e, true);
-
+    for (int j = 0; j < TL; ++j) starts += (ec[j] & kRunStart) != 0;
+    int32_t incl = starts;
+#pragma unroll
+    for (int off = 1; off < G; off <<= 1) {
+      const int32_t o = __shfl_up(incl, off, G);
+      if (l >= off) incl += o;
+    }
+    int32_t at = run + incl - starts;
+#pragma unroll
+    for (int j = 0; j < TL; ++j) {
+      at += (ec[j] & kRunStart) != 0;
+      er[j] = run_row[at];
+      ed[j] = run_delta[at];
+    }
+    run += __shfl(incl, G - 1, G);
+  };
+  TileRegs<TL> m;
+  auto take = [&](int64_t t) {
+    const int64_t q = t + l * TL;
+#pragma unroll
+    for (int j = 0; j < TL; ++j) {
+      m.c[j] = ec[j];
+      m.r[j] = er[j];
+      m.v[j] = q + j < e ? val[q + j + ed[j]] : 0.f;
+    }
+  };
+  look(s);
+  take(s);
+  if (s + kTile < e) look(s + kTile);
   for (int64_t t = s; t < e; t += kTile) {
     stage_tile<TL>(m, sbase + l * TL, s_col, s_val, s_row);
     wave_lds_fence();
     if (t + kTile < e) {
-      const int64_t q = t + kTile + l * TL;
-      load_run<TL>(m.c, ocol, q, e, true);
-      load_run<TL>(m.r, orow, q, e, true);
-#pragma unroll
-      for (int j = 0; j < TL; ++j) m.v[j] = q + j < e ? val[src[j]] : 0.f;
-      if (t + 2 * kTile < e) load_run<TL>(src, osrc, q + kTile, e, true);
+      take(t + kTile);
+      if (t + 2 * kTile < e) look(t + 2 * kTile);
     }
     const int cnt = (e - t) < kTile ? (int)(e - t) : kTile;
     consume_tile(cnt, sbase, s_col, s_val, s_row, cur, acc, loadb, flush);
     wave_lds_fence();
   }
   flush_to((int64_t)start[cur] + (rowptr[cur + 1] - rowptr[cur]) > e);
+}
+
+// Fix-up after the ordered kernel, from the plan's lists: workgroups [0, cross_blocks) - one
+// sub-wave per row whose nonzeros lie in more than one segment: tail[ga] + head[ga + 1] + ... +
+// head[gb] from the carry slots, in that order; the others - one sub-wave per row without nonzeros:
+// zeros.  Every other row was stored by the main kernel.
+template <int K, int kLd = 0>
+__global__ __launch_bounds__(kBlock) void spmm_ordered_fixup_kernel(
+    const int32_t* __restrict__ rowptr, const int32_t* __restrict__ start, const int32_t* __restrict__ cross_rows,
+    int64_t n_cross, int64_t cross_blocks, const int32_t* __restrict__ zero_rows, int64_t n_zero,
+    const float* __restrict__ carry, float* __restrict__ C, int shift, uint32_t ld_arg) {
+  constexpr int G = K / 4;
+  constexpr int P = 64 / G;
+  const uint32_t ld = c_row_length<K, kLd>(ld_arg);
+  const bool c_aligned = c_rows_aligned<kLd>(ld_arg);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int l = lane % G;
+  const int nv = lane_columns<K, kLd>(ld_arg, l);
+  if (nv == 0) return;
+  const int sub = (tid >> 6) * P + lane / G;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  if ((int64_t)blockIdx.x >= cross_blocks) {
+    const int64_t idx = ((int64_t)blockIdx.x - cross_blocks) * (kWavesPerBlock * P) + sub;
+    if (idx < n_zero) store_c_row<kLd, false>(C + (uint64_t)(uint32_t)zero_rows[idx] * ld + 4 * l, acc, nv, c_aligned);
+    return;
+  }
+  const int64_t idx = (int64_t)blockIdx.x * (kWavesPerBlock * P) + sub;
+  if (idx >= n_cross) return;
+  const int64_t row = cross_rows[idx];
+  const int64_t p0 = start[row];
+  const int64_t ga = p0 >> shift;
+  const int64_t gb = (p0 + (rowptr[row + 1] - rowptr[row]) - 1) >> shift;
+  const float* cbase = carry + 4 * l;
+  auto add = [&](const float4& t) {
+    acc.x += t.x;
+    acc.y += t.y;
+    acc.z += t.z;
+    acc.w += t.w;
+  };
+  add(*reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * ga + 1) * K));
+  int64_t g = ga + 1;
+  for (; g + kBatch <= gb + 1; g += kBatch) {
+    float4 slot[kBatch];
+#pragma unroll
+    for (int t = 0; t < kBatch; ++t) slot[t] = *reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * (g + t)) * K);
+#pragma unroll
+    for (int t = 0; t < kBatch; ++t) add(slot[t]);
+  }
+  for (; g <= gb; ++g) add(*reinterpret_cast<const float4*>(cbase + (uint64_t)(2 * g) * K));
+  store_c_row<kLd, false>(C + (uint64_t)row * ld + 4 * l, acc, nv, c_aligned);
 }
 
 }  // namespace hpspmm

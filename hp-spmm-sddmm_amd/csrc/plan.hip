@@ -564,7 +564,7 @@ HPSPMM_API int hpspmm_plan_destroy(hpspmm_plan* plan) {
                   (void*)plan->d_vval, (void*)plan->d_vsrc, (void*)plan->d_vrow, (void*)plan->d_run_row,
                   (void*)plan->d_seg_run, (void*)plan->d_bhot_src, (void*)plan->d_partial,
                   (void*)plan->d_routed_rows, (void*)plan->d_cross_rows, (void*)plan->d_zero_rows,
-                  (void*)plan->d_ostart, (void*)plan->d_ocol, (void*)plan->d_osrc, (void*)plan->d_orow,
+                  (void*)plan->d_ostart, (void*)plan->d_ocol, (void*)plan->d_run_delta,
                   (void*)plan->d_wcols, (void*)plan->d_tent, (void*)plan->d_ldesc, (void*)plan->d_zrow,
                   (void*)plan->d_sw_base, (void*)plan->d_sw_len, (void*)plan->d_sw_ends, (void*)plan->d_sw_slot_row,
                   (void*)plan->d_sw_part_base, (void*)plan->d_sw_split_rows, (void*)plan->d_sw_zrow})

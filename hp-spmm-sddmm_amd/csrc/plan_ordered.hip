@@ -20,6 +20,7 @@ constexpr int kOrderedBlockLdsBytes = 52992;
 int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, const int32_t* d_order,
                   double min_served, hipStream_t st) {
   const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
+  if (p->cols > (int64_t)hpspmm::kEntryPayload) return HPSPMM_OK;  // an entry word keeps the column in 29 bits
   const int64_t subwaves = 64 / (k / 4);
   // window = one workgroup's segments, at most kOrderedMaxWindow nonzeros
   int shift = 9;
@@ -31,16 +32,18 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
   const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
 
   uint32_t* d_len = nullptr;   // [rows + 1] row lengths in processing order, then their scan
+  uint32_t* d_some = nullptr;  // [rows + 1] 1 for a row with nonzeros, then the scan: its run number
   int32_t* d_seen = nullptr;   // [rows] + [1]: permutation check
   unsigned long long* d_served = nullptr;
   struct Guard {
-    void** q[3];
+    void** q[4];
     ~Guard() {
       for (void** x : q)
         if (*x) (void)hipFree(*x);
     }
-  } guard{{(void**)&d_len, (void**)&d_seen, (void**)&d_served}};
+  } guard{{(void**)&d_len, (void**)&d_seen, (void**)&d_served, (void**)&d_some}};
   HPSPMM_HIP(hipMalloc(&d_len, (size_t)(rows + 1) * sizeof(uint32_t)));
+  HPSPMM_HIP(hipMalloc(&d_some, (size_t)(rows + 1) * sizeof(uint32_t)));
   HPSPMM_HIP(hipMalloc(&d_seen, (size_t)(rows + 1) * sizeof(int32_t)));
   HPSPMM_HIP(hipMalloc(&d_served, sizeof(unsigned long long)));
   HPSPMM_HIP(hipMemsetAsync(d_seen, 0, (size_t)(rows + 1) * sizeof(int32_t), st));
@@ -53,8 +56,13 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
   HPSPMM_HIP(hipStreamSynchronize(st));
   if (bad) return fail(HPSPMM_ERR_INVALID_ARG, "row order is not a permutation of [0, rows)");
   hipLaunchKernelGGL(hpspmm::ordered_len_kernel, dim3(rgrid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_order,
-                     d_len);
+                     d_len, d_some);
   if (int rc = exclusive_scan_u32(d_len, d_len, rows + 1, st)) return rc;
+  if (int rc = exclusive_scan_u32(d_some, d_some, rows + 1, st)) return rc;
+  uint32_t runs = 0;
+  HPSPMM_HIP(hipMemcpyAsync(&runs, d_some + rows, sizeof runs, hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  const int64_t n_runs = runs;
 
   const size_t n_bytes = (size_t)std::max<int64_t>(nnz, 1) * sizeof(int32_t);
   const size_t start_bytes = (size_t)std::max<int64_t>(rows, 1) * sizeof(int32_t);
@@ -62,22 +70,26 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
   const size_t carry_bytes = (size_t)std::max<int64_t>(nseg, 1) * 2 * (size_t)k * sizeof(float);
   float* d_new_carry = nullptr;
   auto drop = [&]() {
-    for (void** q : {(void**)&p->d_ostart, (void**)&p->d_ocol, (void**)&p->d_osrc, (void**)&p->d_orow,
-                     (void**)&p->d_wcols, (void**)&d_new_carry}) {
+    for (void** q : {(void**)&p->d_ostart, (void**)&p->d_ocol, (void**)&p->d_wcols,
+                     (void**)&d_new_carry, (void**)&p->d_run_row, (void**)&p->d_run_delta, (void**)&p->d_seg_run,
+                     (void**)&p->d_cross_rows, (void**)&p->d_zero_rows}) {
       if (*q) (void)hipFree(*q);
       *q = nullptr;
     }
   };
+  const size_t run_bytes = (size_t)std::max<int64_t>(n_runs, 1) * sizeof(int32_t);
+  const size_t seg_bytes = (size_t)std::max<int64_t>(nseg, 1) * sizeof(int32_t);
   if (hipMalloc(&p->d_ostart, start_bytes) != hipSuccess || hipMalloc(&p->d_ocol, n_bytes) != hipSuccess ||
-      hipMalloc(&p->d_osrc, n_bytes) != hipSuccess || hipMalloc(&p->d_orow, n_bytes) != hipSuccess ||
+      hipMalloc(&p->d_run_row, run_bytes) != hipSuccess || hipMalloc(&p->d_run_delta, run_bytes) != hipSuccess ||
+      hipMalloc(&p->d_seg_run, seg_bytes) != hipSuccess ||
       hipMalloc(&p->d_wcols, wcols_bytes) != hipSuccess || hipMalloc(&d_new_carry, carry_bytes) != hipSuccess) {
     (void)hipGetLastError();
     drop();
     return fail(HPSPMM_ERR_ALLOC, "device allocation for the ordered plan failed");
   }
   hipLaunchKernelGGL(hpspmm::ordered_fill_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
-                     dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_order, d_len, p->d_ostart, p->d_ocol,
-                     p->d_osrc, p->d_orow);
+                     dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_order, d_len, d_some, shift, p->d_ostart,
+                     p->d_ocol, p->d_run_row, p->d_run_delta, p->d_seg_run);
   if (windows > INT32_MAX) {
     drop();
     return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
@@ -85,8 +97,9 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
   if (nnz > 0)
     hipLaunchKernelGGL(hpspmm::ordered_hot_kernel, dim3((unsigned)windows), dim3(hpspmm::kBlock), 0, st, nnz, window,
                        cap, p->d_ocol, p->d_wcols, d_served);
-  hipLaunchKernelGGL(hpspmm::ordered_partition_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kWavesPerBlock)),
-                     dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, p->d_ostart, window, p->d_ocol, p->d_osrc);
+  // (A row's nonzeros stay in stored order.  Moving those that read B from LDS behind the others within
+  // every row - a batch of gathers is as slow as its slowest load - bought nothing: co-purchase graph,
+  // K = 64, 2.93 ms with that order, 2.92 without, and it cost an index per nonzero to find the values.)
   unsigned long long served = 0;
   hipError_t e = hipMemcpyAsync(&served, d_served, sizeof served, hipMemcpyDeviceToHost, st);
   if (e == hipSuccess) e = hipStreamSynchronize(st);
@@ -99,11 +112,43 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
     drop();
     return HPSPMM_OK;
   }
+  // the lists of the rows the fix-up kernel has to visit
+  {
+    DeviceTemps tmp;
+    uint8_t* d_action = nullptr;
+    int32_t* d_counts = nullptr;
+    int rc = tmp.alloc(&d_action, (size_t)std::max<int64_t>(rows, 1));
+    if (!rc) rc = tmp.alloc(&d_counts, 2);
+    if (rc || hipMalloc(&p->d_cross_rows, start_bytes) != hipSuccess || hipMalloc(&p->d_zero_rows, start_bytes) != hipSuccess) {
+      (void)hipGetLastError();
+      drop();
+      return rc ? rc : fail(HPSPMM_ERR_ALLOC, "device allocation for the ordered plan failed");
+    }
+    const unsigned row_grid = (unsigned)ceil_div(std::max<int64_t>(rows, 1), hpspmm::kBlock);
+    hipLaunchKernelGGL(hpspmm::ordered_action_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr,
+                       p->d_ostart, shift, d_action);
+    hipError_t e2 = hipMemsetAsync(d_counts, 0, 2 * sizeof(int32_t), st);
+    hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_action,
+                       hpspmm::kActionCross, p->d_cross_rows, d_counts);
+    hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_action,
+                       hpspmm::kActionZero, p->d_zero_rows, d_counts + 1);
+    int32_t counts[2] = {0, 0};
+    if (e2 == hipSuccess) e2 = hipMemcpyAsync(counts, d_counts, sizeof counts, hipMemcpyDeviceToHost, st);
+    if (e2 == hipSuccess) e2 = hipStreamSynchronize(st);
+    if (e2 == hipSuccess) e2 = hipGetLastError();
+    if (e2 != hipSuccess) {
+      drop();
+      return fail(HPSPMM_ERR_HIP, "construction of the ordered plan failed: %s", hipGetErrorString(e2));
+    }
+    p->n_cross = counts[0];
+    p->n_zero = counts[1];
+    p->n_runs = n_runs;
+  }
   // accepted: the segments strategy's buffers are not needed any more
   if (p->d_nnz_row) { (void)hipFree(p->d_nnz_row); p->d_nnz_row = nullptr; }
   if (p->d_carry) (void)hipFree(p->d_carry);
   p->d_carry = d_new_carry;
-  p->workspace_bytes = (int64_t)(start_bytes + 3 * n_bytes + wcols_bytes + carry_bytes);
+  p->workspace_bytes = (int64_t)(3 * start_bytes + n_bytes + wcols_bytes + carry_bytes + 2 * run_bytes + seg_bytes);
   p->shift = shift;
   p->nseg = nseg;
   p->ocap = cap;

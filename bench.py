@@ -198,6 +198,94 @@ def cpu_baseline(graphs, g, B, k, C_gpu_host_rows, budget_nnz):
     }
 
 
+# Forced strategies the plan's own choice is compared with (--held-out): column name, plan flags,
+# the strategy the plan must end up in for the column to count.
+def forced_strategies(capi):
+    return [("rows", capi.PLAN_FORCE_ROWS, capi.STRATEGY_ROWS),
+            ("segments", capi.PLAN_FORCE_SEGMENTS, capi.STRATEGY_SEGMENTS),
+            ("ordered", capi.PLAN_CLUSTER | capi.PLAN_FORCE_SEGMENTS | capi.PLAN_NO_HUB_CACHE, capi.STRATEGY_ORDERED),
+            ("routed", capi.PLAN_FORCE_ROUTED, capi.STRATEGY_ROUTED),
+            ("sweep", capi.PLAN_FORCE_SWEEP, capi.STRATEGY_SWEEP)]
+
+
+STRATEGY_NAMES = {1: "rows", 2: "segments", 4: "routed", 5: "ordered", 6: "sweep"}
+
+
+def strategy_times(capi, g, d_rp, d_ci, d_v, d_B, d_C, k, stream, regions=2, auto_options=None):
+    """Microseconds per SpMM of the default plan and of every forced strategy on one matrix: the
+    smaller of `regions` timed regions of at least MIN_TIMED_MS each.  A forced strategy the plan
+    could not build for this matrix (it falls back to another) reads None."""
+    import torch
+    out = {}
+    chosen = None
+    for name, flags, want in [("auto", 0, None)] + forced_strategies(capi):
+        plan = capi.Plan(g.rows, g.cols, d_rp, d_ci, k, flags, options=auto_options if want is None else None)
+        got = plan.info["strategy"]
+        if want is None:
+            chosen = got
+        if want is not None and got != want:
+            out[name] = None
+        else:
+            best = None
+            for r in range(regions):
+                ms, _ = capi.csr_spmm_timed_min(plan, d_rp, d_ci, d_v, d_B, d_C, warmup=3 if r == 0 else 0, iters=5,
+                                                min_total_ms=MIN_TIMED_MS, stream=stream)
+                best = ms if best is None else min(best, ms)
+            out[name] = best * 1e3
+        torch.cuda.synchronize()
+        plan.destroy()
+    return out, chosen
+
+
+def held_out(capi, graphs, dev, stream, args, plan_options=None):
+    """The plan's choice of strategy on generator families none of its thresholds was chosen on:
+    one table line per (family, size, K) with the default plan beside every forced strategy, and
+    rocSPARSE's best CSR/COO algorithm where --vendor-csv names what the host driver wrote for the
+    same matrices."""
+    import torch
+    vendor = {}
+    if args.vendor_csv:
+        import re
+        for line in open(args.vendor_csv):
+            f = line.strip().split(",")
+            if len(f) < 6 or "@" not in f[0]:
+                continue
+            name, sc = f[0].split("@")
+            # (rocSPARSE fills the reference's cuSPARSE columns: label, ms, GFLOPS)
+            ms = [float(m.group(1)) for m in re.finditer(r"cuSPARSE\([^)]*\):?\s*,([0-9.e+-]+),", line)]
+            ms = [m for m in ms if m > 0]
+            if ms:
+                vendor[(name, float(sc), int(f[4]))] = min(ms) * 1e3
+    scales = [float(x) for x in args.held_out_scales.split(",")]
+    ks = [int(x) for x in args.held_out_k.split(",")]
+    families = args.only.split(",") if args.only else list(graphs.HELD_OUT)
+    cols = [c[0] for c in forced_strategies(capi)]
+    print(f"{'family':14s} {'scale':>6s} {'rows':>9s} {'nnz':>10s} {'K':>4s} " + " ".join(f"{c:>9s}" for c in cols)
+          + f" {'auto':>9s}  {'chosen':9s} {'off':>6s} {'rocSPARSE':>10s}", flush=True)
+    worst = 0.0
+    for name in families:
+        for sc in scales:
+            g = graphs.make_graph(name, sc)
+            d_rp, d_ci, d_v = (torch.from_numpy(a).to(dev) for a in (g.rowptr, g.col, g.val))
+            for k in ks:
+                d_B = torch.from_numpy(graphs.make_dense(name, g.cols, k)).to(dev)
+                d_C = torch.empty((g.rows, k), device=dev, dtype=torch.float32)
+                t, chosen = strategy_times(capi, g, d_rp, d_ci, d_v, d_B, d_C, k, stream, auto_options=plan_options)
+                best = min(v for c, v in t.items() if c != "auto" and v is not None)
+                off = t["auto"] / best - 1
+                worst = max(worst, off)
+                v = vendor.get((name, sc, k))
+                print(f"{name:14s} {sc:6g} {g.rows:9d} {g.nnz:10d} {k:4d} "
+                      + " ".join(f"{t[c]:9.1f}" if t[c] is not None else f"{'-':>9s}" for c in cols)
+                      + f" {t['auto']:9.1f}  {STRATEGY_NAMES.get(chosen, str(chosen)):9s} {100 * off:+5.1f}%"
+                      + (f" {v:10.1f}" if v is not None else f" {'':>10s}"), flush=True)
+                del d_B, d_C
+            del d_rp, d_ci, d_v, g
+            torch.cuda.empty_cache()
+    print(f"largest gap between the plan's choice and the fastest forced strategy: {100 * worst:.1f} %")
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -219,6 +307,13 @@ def main():
                          "to the launches of the figure of merit)")
     ap.add_argument("--fabric-probe", action="store_true",
                     help="instead of the benchmark: the gather rate of the segments kernel against the size of B")
+    ap.add_argument("--held-out", action="store_true",
+                    help="instead of the benchmark: the default plan against every forced strategy on "
+                         "generator families none of the plan's thresholds was chosen on (microseconds)")
+    ap.add_argument("--held-out-scales", default="0.015,0.12,1.0", help="sizes for --held-out (1 = about 10^8 nonzeros)")
+    ap.add_argument("--held-out-k", default="32,64,128")
+    ap.add_argument("--vendor-csv", default="", help="--held-out: a csv written by spmm_test_all --synthetic ... --csv "
+                                                      "for the same matrices (name@scale), printed beside")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three 1 GiB device-to-device copies (a kernel of known traffic, "
                          "for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -266,6 +361,9 @@ def main():
     torch.cuda.synchronize()
     plan0.destroy()
     del w, g0
+
+    if args.held_out:
+        return held_out(capi, graphs, dev, stream, args, plan_options)
 
     workloads = WORKLOADS
     if args.only:

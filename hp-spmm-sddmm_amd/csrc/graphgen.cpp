@@ -253,6 +253,60 @@ struct RmatSampler {
   }
 };
 
+// Edges kept in arrays (a generator that builds its edge list one edge after the other).
+struct ListSampler {
+  const int32_t* us;
+  const int32_t* vs;
+  inline void operator()(int64_t e, int32_t& u, int32_t& v) const {
+    u = us[e];
+    v = vs[e];
+  }
+};
+
+// side x side grid, vertex = y * side + x: edges to the right, lower, lower-right and lower-left
+// neighbours (with their mirror images: the 8 neighbours of a 9-point stencil) and `noise` edges per
+// vertex to uniformly random vertices.  Edge e belongs to vertex e / (4 + noise).
+struct GridSampler {
+  int64_t side;
+  int noise;
+  uint64_t seed;
+  inline void operator()(int64_t e, int32_t& u, int32_t& v) const {
+    const int64_t per = 4 + noise, vert = e / per, which = e - vert * per;
+    const int64_t x = vert % side, y = vert / side;
+    u = (int32_t)vert;
+    int64_t nx = x, ny = y;
+    if (which == 0) nx = x + 1;
+    else if (which == 1) ny = y + 1;
+    else if (which == 2) { nx = x + 1; ny = y + 1; }
+    else if (which == 3) { nx = x - 1; ny = y + 1; }
+    else {
+      v = (int32_t)(((unsigned __int128)draw(seed, 51, (uint64_t)e) * (uint64_t)(side * side)) >> 64);
+      return;
+    }
+    v = (nx < 0 || nx >= side || ny >= side) ? u : (int32_t)(ny * side + nx);  // off the grid: a self-loop
+  }
+};
+
+// Communities of mixed sizes as consecutive vertex ranges: the second endpoint is uniform inside the
+// first one's community with probability p_intra, else uniform over all vertices.
+struct BlockSampler {
+  const int64_t* bstart;  // community -> first vertex; [n_blocks] = n
+  const int32_t* block;   // vertex -> community
+  int64_t n;
+  double p_intra;
+  uint64_t seed;
+  inline void operator()(int64_t e, int32_t& u, int32_t& v) const {
+    u = (int32_t)(((unsigned __int128)draw(seed, 61, (uint64_t)e) * (uint64_t)n) >> 64);
+    const uint64_t r = draw(seed, 62, (uint64_t)e);
+    if (u01(draw(seed, 63, (uint64_t)e)) < p_intra) {
+      const int64_t lo = bstart[block[u]], hi = bstart[block[u] + 1];
+      v = (int32_t)(lo + (int64_t)(((unsigned __int128)r * (uint64_t)(hi - lo)) >> 64));
+    } else {
+      v = (int32_t)(((unsigned __int128)r * (uint64_t)n) >> 64);
+    }
+  }
+};
+
 }  // namespace
 
 extern "C" {
@@ -403,6 +457,149 @@ hpspmm_graph* hpspmm_gen_rmat(int scale, int64_t n_edges, double a, double b, do
   return (hpspmm_graph*)build_symmetric((int64_t)1 << scale, n_edges, smp, false, kValSymUniformPM1, seed);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Families that none of the library's thresholds was chosen on: they exist to check that the plan's
+// choice of strategy holds up on matrices unlike the benchmark's four.
+// ---------------------------------------------------------------------------------------------
+
+// Preferential attachment (Barabasi-Albert): vertex t brings m edges whose other ends are drawn in
+// proportion to the degrees so far (an endpoint of a uniformly chosen earlier edge, or the vertex
+// before when there is none yet); vertices relabelled at random; values U(0,1).
+hpspmm_graph* hpspmm_gen_pref_attach(int64_t n, int64_t m, uint64_t seed) {
+  if (n < 2 || m < 1 || n * m > 0x3FFFFFFFll) {
+    g_err = "gen_pref_attach: bad arguments";
+    return nullptr;
+  }
+  const int64_t E = (n - 1) * m;
+  std::vector<int32_t> us((size_t)E), vs((size_t)E);
+  std::vector<int32_t> label((size_t)n);
+  {
+    std::vector<std::pair<uint64_t, int32_t>> key((size_t)n);
+    for (int64_t i = 0; i < n; ++i) key[i] = {draw(seed, 71, (uint64_t)i), (int32_t)i};
+    std::sort(key.begin(), key.end());
+    for (int64_t i = 0; i < n; ++i) label[key[i].second] = (int32_t)i;
+  }
+  // (sequential by nature: every draw looks at the edges before it; unlabelled vertices here)
+  for (int64_t e = 0; e < E; ++e) {
+    const int64_t t = 1 + e / m;
+    int32_t other = (int32_t)(t - 1);
+    if (e >= m) {  // an endpoint of one of the edges brought by earlier vertices
+      const int64_t before = (t - 1) * m;
+      const uint64_t r = draw(seed, 72, (uint64_t)e);
+      const int64_t pick = (int64_t)(((unsigned __int128)r * (uint64_t)(2 * before)) >> 64);
+      other = (pick & 1) ? vs[pick >> 1] : us[pick >> 1];
+    }
+    us[e] = (int32_t)t;
+    vs[e] = other;
+  }
+#pragma omp parallel for schedule(static)
+  for (int64_t e = 0; e < E; ++e) {
+    us[e] = label[us[e]];
+    vs[e] = label[vs[e]];
+  }
+  ListSampler smp{us.data(), vs.data()};
+  return (hpspmm_graph*)build_symmetric(n, E, smp, false, kValSymUniform01, seed);
+}
+
+// 9-point stencil on a side x side grid plus `noise` random long-range edges per vertex, symmetric,
+// a self-loop on every vertex; values 1 / (row length): an averaging operator.
+hpspmm_graph* hpspmm_gen_grid(int64_t side, int noise, uint64_t seed) {
+  if (side < 2 || noise < 0 || side * side * (4 + noise) > 0x3FFFFFFFll) {
+    g_err = "gen_grid: bad arguments";
+    return nullptr;
+  }
+  GridSampler smp{side, noise, seed};
+  return (hpspmm_graph*)build_symmetric(side * side, side * side * (4 + noise), smp, true, kValRowNormalised, seed);
+}
+
+// Rectangular users x items: every user (row) draws a lognormal(mu, sigma) number of items (columns)
+// from a Zipf(alpha)-weighted popularity, duplicates merged; values U(-1,1).  Not symmetric, not square.
+hpspmm_graph* hpspmm_gen_bipartite(int64_t users, int64_t items, double mu, double sigma, double alpha,
+                                   uint64_t seed) {
+  if (users < 1 || items < 1 || alpha <= 0) {
+    g_err = "gen_bipartite: bad arguments";
+    return nullptr;
+  }
+  std::vector<double> w((size_t)items);
+  {
+    // popularity rank -> item id shuffled, so that popular items are spread over the columns
+    std::vector<std::pair<uint64_t, int32_t>> key((size_t)items);
+    for (int64_t i = 0; i < items; ++i) key[i] = {draw(seed, 81, (uint64_t)i), (int32_t)i};
+    std::sort(key.begin(), key.end());
+    for (int64_t r = 0; r < items; ++r) w[key[r].second] = std::pow((double)r + 10.0, -alpha);
+  }
+  Alias table;
+  table.build(w);
+  std::vector<int64_t> off((size_t)users + 1, 0);
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < users; ++i) {
+    const double u1 = u01_open0(draw(seed, 82, (uint64_t)i));
+    const double u2 = u01(draw(seed, 83, (uint64_t)i));
+    const double z = std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586 * u2);
+    off[i + 1] = std::min<int64_t>(items, std::max<int64_t>(1, (int64_t)std::llround(std::exp(mu + sigma * z))));
+  }
+  for (int64_t i = 0; i < users; ++i) off[i + 1] += off[i];
+  if (off[users] > 0x7FFFFFFFll) {
+    g_err = "gen_bipartite: too many nonzeros";
+    return nullptr;
+  }
+  std::vector<int32_t> raw((size_t)off[users]);
+  std::vector<int64_t> newoff((size_t)users + 1, 0);
+#pragma omp parallel for schedule(dynamic, 256)
+  for (int64_t i = 0; i < users; ++i) {
+    int32_t* b = raw.data() + off[i];
+    const int64_t d = off[i + 1] - off[i];
+    for (int64_t j = 0; j < d; ++j) b[j] = table.sample(draw(seed, 84, (uint64_t)(off[i] + j)));
+    std::sort(b, b + d);
+    newoff[i + 1] = std::unique(b, b + d) - b;
+  }
+  for (int64_t i = 0; i < users; ++i) newoff[i + 1] += newoff[i];
+  Graph* g = new Graph;
+  g->rows = users;
+  g->cols = items;
+  g->nnz = newoff[users];
+  g->rowptr.resize((size_t)users + 1);
+  g->col.resize((size_t)g->nnz);
+  g->val.resize((size_t)g->nnz);
+#pragma omp parallel for schedule(dynamic, 256)
+  for (int64_t i = 0; i < users; ++i) {
+    g->rowptr[i] = (int32_t)newoff[i];
+    const int64_t len = newoff[i + 1] - newoff[i];
+    for (int64_t j = 0; j < len; ++j) {
+      const int32_t c = raw[off[i] + j];
+      g->col[newoff[i] + j] = c;
+      g->val[newoff[i] + j] = edge_value(kValUniformPM1, seed, i, c, items);
+    }
+  }
+  g->rowptr[users] = (int32_t)g->nnz;
+  return (hpspmm_graph*)g;
+}
+
+// Communities of mixed sizes (power law between min_size and max_size, exponent 2) as consecutive
+// vertex ranges; n_edges undirected samples of which p_intra stay inside a community; values U(0,1).
+hpspmm_graph* hpspmm_gen_blocks(int64_t n, int64_t min_size, int64_t max_size, double p_intra, int64_t n_edges,
+                                uint64_t seed) {
+  if (n < 1 || min_size < 1 || max_size < min_size || n_edges < 0 || p_intra < 0 || p_intra > 1) {
+    g_err = "gen_blocks: bad arguments";
+    return nullptr;
+  }
+  std::vector<int64_t> bstart{0};
+  while (bstart.back() < n) {
+    // inverse-CDF draw of a size with density ~ s^-2 on [min_size, max_size]
+    const double u = u01(draw(seed, 91, (uint64_t)bstart.size()));
+    const double a = 1.0 / (double)min_size, b = 1.0 / (double)max_size;
+    const int64_t size = std::max<int64_t>(min_size, (int64_t)(1.0 / (a - u * (a - b))));
+    bstart.push_back(std::min(n, bstart.back() + size));
+  }
+  const int64_t n_blocks = (int64_t)bstart.size() - 1;
+  std::vector<int32_t> block((size_t)n);
+#pragma omp parallel for schedule(dynamic, 64)
+  for (int64_t c = 0; c < n_blocks; ++c)
+    for (int64_t v = bstart[c]; v < bstart[c + 1]; ++v) block[v] = (int32_t)c;
+  BlockSampler smp{bstart.data(), block.data(), n, p_intra, seed};
+  return (hpspmm_graph*)build_symmetric(n, n_edges, smp, false, kValSymUniform01, seed);
+}
+
 // The benchmark configurations by name.  scale < 1 shrinks vertex and edge
 // counts together (tests); scale = 1 is the benchmark size.  Parameters were
 // calibrated so that the full-size graphs land on the configured statistics:
@@ -438,6 +635,28 @@ hpspmm_graph* hpspmm_gen_named(const char* name, double scale) {
   if (n == "c4_rmat") {
     const int sc = scale >= 1 ? 22 : std::max(6, 22 + (int)std::floor(std::log2(scale)));
     return hpspmm_gen_rmat(sc, (int64_t)16 << sc, 0.57, 0.19, 0.19, 4);
+  }
+  // Held-out families (scale 1 = about 10^8 nonzeros):
+  //   h1_prefattach  preferential attachment, 24 edges per new vertex
+  //   h2_rmat        R-MAT with a flatter quadrant law (0.45, 0.22, 0.22, 0.11), edge factor 24
+  //   h3_grid        9-point stencil + 2 random edges per vertex, about 13 nonzeros per row
+  //   h4_bipartite   users x items (8 : 1), lognormal basket sizes (mean ~60), Zipf(0.9) popularity
+  //   h5_blocks      communities of 8 to 4096 vertices, 90 % of the edges inside, mean degree ~40
+  //   h6_uniform100  100 uniformly placed nonzeros in every row
+  if (n == "h1_prefattach") return hpspmm_gen_pref_attach(scaled(2.1e6, 64), 24, 11);
+  if (n == "h2_rmat") {
+    const int sc = std::max(6, 21 + (int)std::lround(std::log2(scale)));
+    return hpspmm_gen_rmat(sc, (int64_t)24 << sc, 0.45, 0.22, 0.22, 12);
+  }
+  if (n == "h3_grid") return hpspmm_gen_grid(std::max<int64_t>(8, (int64_t)std::llround(2800.0 * std::sqrt(scale))), 2, 13);
+  if (n == "h4_bipartite") return hpspmm_gen_bipartite(scaled(1.7e6, 64), scaled(2.1e5, 64), 3.8, 0.8, 0.9, 14);
+  if (n == "h5_blocks") {
+    const int64_t v = scaled(2.5e6, 64);
+    return hpspmm_gen_blocks(v, 8, 4096, 0.9, (int64_t)std::llround(21.0 * (double)v), 15);
+  }
+  if (n == "h6_uniform100") {
+    const int64_t v = scaled(1.0e6, 128);
+    return hpspmm_gen_uniform_rows(v, v, 100, 16);
   }
   g_err = "gen_named: unknown configuration '" + n + "'";
   return nullptr;

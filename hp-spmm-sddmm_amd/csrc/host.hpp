@@ -343,6 +343,17 @@ int ensure_row_expansion(hpspmm_plan* p, const int32_t* d_rowptr, hipStream_t st
 // True if the column indices of every row are in non-decreasing order.  Errors count as "no".
 bool columns_sorted(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st);
 
+// Share of the gathers of rows of B that miss a cache of about 30k rows of B (one 32-column tile of
+// them: 4 MB, an L2) when the matrix is walked in stored order, every XCD taking one piece in eight:
+// 32 samples of the column stream, each walked until it has met 40k distinct columns (or 16 times as
+// many nonzeros).  Near 1 for columns without any order, 1 / (references per column within reach)
+// for a banded or block-structured matrix.  1.0 when the matrix is too small to sample or there is
+// no room for the bit tables.
+constexpr int kLocalitySamples = 32;
+constexpr int64_t kLocalityCapacity = 40960;
+constexpr int64_t kLocalityMaxWalk = 16;
+int stored_order_miss_share(const hpspmm_plan* p, const int32_t* d_col, hipStream_t st, double* share);
+
 // ---- layouts (plan_*.hip): each leaves p->strategy alone when the matrix does not qualify ----
 
 int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, hipStream_t st);
@@ -352,8 +363,8 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
                   double min_served, hipStream_t st);
 int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, const PlanOptions& opt,
                  hipStream_t st, int32_t** d_order_out, double* intra_share_out);
-int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, const PlanOptions& opt,
-                hipStream_t st);
+int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, double other_us,
+                const PlanOptions& opt, hipStream_t st);
 
 // ---- launches (launch_*.hip) ---------------------------------------------------------------
 

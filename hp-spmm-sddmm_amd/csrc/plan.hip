@@ -63,6 +63,15 @@ int choose_shift(int64_t nnz, int64_t k, int64_t max_row_nnz) {
 // Automatic clustering is tried for graphs of at least this size ...
 constexpr int64_t kClusterMinNnz = (int64_t)1 << 22;
 constexpr int64_t kClusterMinBBytes = (int64_t)24 << 20;
+// A matrix whose stored order is local already has its communities side by side; another order pays
+// only where B is far beyond every cache (blocks of 8 to 4096 vertices along the diagonal with 10 % of
+// the entries elsewhere, K = 32 / 64 / 128: at 10 M nonzeros (B = 38 / 77 / 154 MB) ordered 109 / 193 /
+// 377 us against 99 / 183 / 380 for whole rows; at 85 M (320 / 640 / 1280 MB) 0.95 / 1.66 / 3.17 ms
+// against 0.93 / 1.80 / 3.95).
+constexpr int64_t kClusterLocalMinBBytes = (int64_t)256 << 20;
+constexpr double kLocalMissShare = 0.3;  // stored order counts as local up to this share of missing gathers
+constexpr double kRowsFallbackMissShare = 0.85;
+constexpr double kRowsHitPs = 7.0, kRowsMissPs = 20.7;  // rows strategy: per nonzero and 32 columns of B
 constexpr double kClusterMinIntra = 0.15;   // share of the nonzeros inside such clusters for the order to be used
 constexpr int64_t kClusterMinMeanNnz = 8;
 // ... and its order is kept if this share of the nonzeros then reads B from LDS.
@@ -223,6 +232,9 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
   bool rows_need_tiles = false;  // rows strategy chosen on the strength of the row tiles
   bool rows_range = false;       // provisional segments; rows unless the ordered strategy qualifies
   bool want_row_tiles = true;    // rows strategy: over row tiles if they can be built
+  double miss = 1.0;             // share of the gathers that miss an L2 when the rows are taken in stored order
+  double rows_us = 0.0;          // what the rows strategy is expected to take (0: no estimate)
+  bool rows_fallback = false;    // whole rows rather than segments if no other layout qualifies
   if (!row_tiles_serve(k, opt)) {
     // a row length that not even the row tiles serve: whole rows over the CSR arrays for small
     // matrices (one launch), segments beyond (balanced over any degree distribution)
@@ -277,7 +289,37 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
     // (a row gets at most one workgroup of 16 wavefronts; at K outside the tuned set that still beats
     // the segments kernel with a row of 163k nonzeros - R-MAT, 128 M nonzeros, K = 8: 1.72 against 2.27 ms)
     const int64_t longest_ok = fast_k(k) || k < 4 ? kRowsAutoMaxRow : 4 * kRowsAutoMaxRow;
-    const bool mid = in_range && p->max_row_nnz <= longest_ok && !(flags & HPSPMM_PLAN_NO_ROW_TILES);
+    // How local the stored order is decides between strategies from here on.  The rows strategy over
+    // matrices of 25 to 200 uniformly placed nonzeros per row takes, per nonzero and 32 columns of B,
+    // 7.5 ps when the 32-column tile of B is 4 MB, 11.5 at 8 MB, 15.3 at 15 MB, 17.7 at 32 MB and
+    // 19.2 at 64 MB (the same for K = 32, 64 and 128): 7 ps for a gather that hits, 20.7 for one that
+    // does not.
+    if (!tiny && nnz > 0 && fast_k(k)) {
+      if (int rc = stored_order_miss_share(p, d_col, st, &miss)) return rc;
+      rows_us = (double)nnz * (double)(k / 32) * (kRowsHitPs + (kRowsMissPs - kRowsHitPs) * miss) * 1e-6;
+    }
+    // A matrix whose stored order is local (banded, a mesh, blocks along the diagonal) is served best
+    // by whole rows at any size: the gathers of neighbouring rows meet in the L2, and nothing is left
+    // for the other layouts to gain (9-point mesh with 2 random entries per row, 102 M nonzeros,
+    // K = 32 / 64 / 128: 1.27 / 2.58 / 5.75 ms against 1.81 / 3.31 / 6.44 for segments).
+    if (opt.report && rows_us > 0)
+      fprintf(stderr, "plan: %.3f of the gathers miss in stored order, whole rows expected to take %.1f us\n", miss, rows_us);
+    const bool short_rows = mean_row <= kRowsAutoLongMean;
+    const bool local = fast_k(k) && miss <= kLocalMissShare && short_rows && nnz < kRowTileMaxNnz;
+    const bool mid = (in_range || local) && p->max_row_nnz <= longest_ok && !(flags & HPSPMM_PLAN_NO_ROW_TILES);
+    // Beyond that range, when none of the other layouts qualifies, the choice is between whole rows
+    // and segments.  Row tiles are taken in stored order by all the CUs side by side, so that rows
+    // that share columns with their neighbours meet them in the L2; segments are long runs of
+    // nonzeros far apart from each other, which gain nothing from that order, but read the sparse
+    // matrix once instead of once per 32 columns.  Measured (rows against segments, K = 32 / 64 / 128):
+    // 9-point mesh with 2 / 8 random entries per row, 52 / 100 M nonzeros: 0.66 / 1.31 / 2.84 against
+    // 0.94 / 1.84 / 3.49 ms and 1.49 / 3.43 / 7.51 against 2.12 / 3.71 / 7.69; 20 uniformly placed
+    // nonzeros in each of 4 M rows: 1.61 / 3.70 / 8.33 against 1.69 / 3.68 / 7.98; preferential
+    // attachment, 101 M: 1.93 / 3.97 / 8.89 against 2.13 / 3.80 / 7.47.
+    // (a row is a chain of tiles on one wavefront: long rows only where they are all of a length)
+    const bool even_enough = (double)p->max_row_nnz < (short_rows ? 512.0 : 16.0) * mean_row;
+    rows_fallback = fast_k(k) && even_enough && nnz < kRowTileMaxNnz && p->max_row_nnz <= longest_ok &&
+                    !(flags & HPSPMM_PLAN_NO_ROW_TILES) && (miss <= kRowsFallbackMissShare || k == 32);
     if (nnz == 0 || tiny || (mid && nnz < kClusterMinNnz)) {
       p->strategy = HPSPMM_STRATEGY_ROWS;
       rows_need_tiles = !(nnz == 0 || tiny);
@@ -313,8 +355,8 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
   // the plan stays what it was.
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && nnz > 0 && !(flags & HPSPMM_PLAN_NO_SWEEP) &&
       ((flags & HPSPMM_PLAN_FORCE_SWEEP) ||
-       (!rows_range && !(flags & (HPSPMM_PLAN_FORCE_SEGMENTS | HPSPMM_PLAN_FORCE_ROUTED | HPSPMM_PLAN_CLUSTER))))) {
-    if (int rc = build_sweep(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_SWEEP) != 0, opt, st)) return rc;
+       !(flags & (HPSPMM_PLAN_FORCE_SEGMENTS | HPSPMM_PLAN_FORCE_ROUTED | HPSPMM_PLAN_CLUSTER)))) {
+    if (int rc = build_sweep(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_SWEEP) != 0, rows_us, opt, st)) return rc;
   }
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && !(flags & HPSPMM_PLAN_NO_ROUTED) && nnz > 0 &&
       !rows_range &&
@@ -331,7 +373,8 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && rows == cols && nnz > 0 &&
       !(flags & HPSPMM_PLAN_NO_CLUSTER) &&
       (want_cluster || (!(flags & HPSPMM_PLAN_FORCE_SEGMENTS) && nnz >= kClusterMinNnz &&
-                        cols * k * 4 >= kClusterMinBBytes && nnz >= rows * kClusterMinMeanNnz))) {
+                        cols * k * 4 >= (miss <= kLocalMissShare ? kClusterLocalMinBBytes : kClusterMinBBytes) &&
+                        nnz >= rows * kClusterMinMeanNnz))) {
     int32_t* d_order = nullptr;
     double intra_share = 0.0;
     int rc = cluster_rows(p, d_rowptr, d_col, opt, st, &d_order, &intra_share);
@@ -342,7 +385,7 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
       return rc;
     }
   }
-  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && rows_range && row_tiles_serve(k, opt)) {
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && (rows_range || rows_fallback) && row_tiles_serve(k, opt)) {
     // no communities: whole rows after all, if the row tiles get built
     if (int rc = build_row_tiles(p, d_rowptr, d_col, st)) {
       return rc;

@@ -17,8 +17,10 @@ constexpr int kSweepSpinLimit = 400;
 // 1 MB with lead 2: 1.09 / 1.70 / 2.92, lead 4: 1.12 / 1.71 / 3.07; 256 KB with lead 4: 1.09 / 1.67 / 3.15.
 inline int sweep_lead(int64_t k) { return k >= 128 ? 3 : 2; }
 // Automatic choice: B beyond what the L2s hold between them without help, enough work to fill the device.
-constexpr double kSweepMinSpan = 0.5;  // mean distance from a row's first to its last column, as a share of the columns
-constexpr int64_t kSweepMinNnz = (int64_t)1 << 22;
+// picoseconds per nonzero and microseconds per band and window at K = 32 / 64 / 128
+constexpr double kSweepPsPerNnz[3] = {6.5, 8.8, 13.4}, kSweepUsPerWindow[3] = {1.44, 1.72, 1.36};
+constexpr double kSweepMinGain = 0.9;  // expected time against that of whole rows for the sweep to be chosen
+constexpr int64_t kSweepMinNnz = (int64_t)1 << 21;
 constexpr int64_t kSweepMinBBytes = (int64_t)5 << 20;  // social graph: 6 MB of B, sweep 103 / 127 us against 123 / 141; 3 MB: 90 / 65 against 87 / 63
 
 // Gives back what an abandoned attempt at the sweep layout has allocated in the plan so far.
@@ -38,8 +40,8 @@ void drop_sweep_buffers(hpspmm_plan* p) {
 // the device has no room for the temporaries of the construction.  Diagnostics: the sweep_* fields of
 // hpspmm_plan_options (bytes of B per window, lead, spin limit, nonzeros per piece, priorities)
 // override the defaults.
-int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, const PlanOptions& opt,
-                hipStream_t st) {
+int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, double other_us,
+                const PlanOptions& opt, hipStream_t st) {
   const int64_t rows = p->rows, nnz = p->nnz, k = p->k;
   if (nnz <= 0) return HPSPMM_OK;
   // gather offsets are 32-bit, stream entries keep the column in 24 bits
@@ -73,27 +75,19 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   while (wshift < 30 && (((int64_t)1 << (wshift + 1)) * k * 4) <= ((int64_t)1 << wlog2)) ++wshift;
   const int64_t n_windows = ceil_div(p->cols, (int64_t)1 << wshift);
   if (n_windows > kSweepMaxWindows) return HPSPMM_OK;
-  // every non-empty row is at least one piece: what the two criteria below come to at the very least
-  // (rules the layout out for a matrix of many short rows before any kernel has run)
-  if (!forced && (ceil_div(nonempty, band_waves * WS) * hpspmm::kXcds * p->cols > nnz / 4 || nonempty * n_windows * 3 > nnz * 2))
-    return HPSPMM_OK;
+  // What a sweep takes: every gather hits, and every band walks all the windows at the pace of the
+  // slowest wavefront.  Over matrices of 25 to 200 uniformly placed nonzeros per row, 30k to 500k rows
+  // and columns, square and 16 : 1 either way: 6.5 / 8.8 / 13.4 ps per nonzero and 1.44 / 1.72 / 1.36 us
+  // per band and window at K = 32 / 64 / 128, within 25 % everywhere and 10 % rms.  Worth it where
+  // that is below what whole rows are expected to take in the stored order (`other_us`).  Every
+  // non-empty row is at least one piece: the first test rules the layout out for most matrices before
+  // any kernel has run.
+  const int ki = k == 32 ? 0 : k == 64 ? 1 : 2;
+  auto expected_us = [&](int64_t bands) {
+    return kSweepPsPerNnz[ki] * (double)nnz * 1e-6 + kSweepUsPerWindow[ki] * (double)(bands * n_windows);
+  };
+  if (!forced && (other_us <= 0 || expected_us(ceil_div(nonempty, band_waves * WS)) > kSweepMinGain * other_us)) return HPSPMM_OK;
   if (!columns_sorted(p, d_rowptr, d_col, st)) return HPSPMM_OK;  // a row must meet the windows in stored order
-  if (!forced) {
-    // rows that reach across most of the columns (a banded matrix is better off with whole rows or segments)
-    unsigned long long* d_span = nullptr;
-    unsigned long long span = 0;
-    HPSPMM_HIP(hipMalloc(&d_span, sizeof span));
-    hipError_t e = hipMemsetAsync(d_span, 0, sizeof span, st);
-    if (e == hipSuccess) {
-      hipLaunchKernelGGL(hpspmm::sweep_row_span_kernel, dim3(grid_for(rows, 4096)), dim3(hpspmm::kBlock), 0, st, rows,
-                         d_rowptr, d_col, d_span);
-      e = hipMemcpyAsync(&span, d_span, sizeof span, hipMemcpyDeviceToHost, st);
-    }
-    if (e == hipSuccess) e = hipStreamSynchronize(st);
-    (void)hipFree(d_span);
-    if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "row span: %s", hipGetErrorString(e));
-    if ((double)span < kSweepMinSpan * (double)p->cols * (double)std::max<int64_t>(1, rows - p->empty_rows)) return HPSPMM_OK;
-  }
 
   DeviceTemps tmp;
   // pieces per row, their scans
@@ -122,11 +116,8 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   }
 
   const int64_t n_bands = ceil_div((int64_t)n_pieces, band_waves * WS);
-  // every band re-reads B once on every XCD: worth it while that stays well below the gather volume,
-  // and while a piece still finds one or two nonzeros in a window (the co-purchase graph at 6 M
-  // nonzeros has 0.85 on average and takes 251 us against 134 with the ordered strategy)
-  if (n_bands > kSweepMaxBands ||
-      (!forced && (n_bands * hpspmm::kXcds * p->cols > nnz / 4 || (int64_t)n_pieces * n_windows * 3 > nnz * 2))) {
+  // (the same test with the bands there really are: long rows are several pieces)
+  if (n_bands > kSweepMaxBands || (!forced && expected_us(n_bands) > kSweepMinGain * other_us)) {
     drop_sweep_buffers(p);
     return HPSPMM_OK;
   }

@@ -359,4 +359,30 @@ bool columns_sorted(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
   return e == hipSuccess && unsorted == 0;
 }
 
+int stored_order_miss_share(const hpspmm_plan* p, const int32_t* d_col, hipStream_t st, double* share) {
+  *share = 1.0;
+  const int64_t nnz = p->nnz;
+  if (nnz < (int64_t)kLocalitySamples * hpspmm::kLocalityBlock) return HPSPMM_OK;
+  DeviceTemps tmp;
+  uint32_t* d_tables = nullptr;
+  const size_t table_words = (size_t)1 << (hpspmm::kLocalityBits - 5);
+  const size_t words = kLocalitySamples * table_words + 4 * kLocalitySamples;
+  if (tmp.alloc(&d_tables, words) != HPSPMM_OK) return HPSPMM_OK;  // no room: no estimate
+  uint32_t* d_out = d_tables + kLocalitySamples * table_words;
+  HPSPMM_HIP(hipMemsetAsync(d_tables, 0, words * sizeof(uint32_t), st));
+  hipLaunchKernelGGL(hpspmm::locality_walk_kernel, dim3(kLocalitySamples), dim3(hpspmm::kLocalityBlock), 0, st, nnz, d_col,
+                     nnz / kLocalitySamples, p->cols > ((int64_t)1 << hpspmm::kLocalityBits) ? 1 : 0,
+                     (uint32_t)kLocalityCapacity, (uint32_t)(kLocalityMaxWalk * kLocalityCapacity), d_tables, d_out);
+  uint32_t out[4 * kLocalitySamples];
+  HPSPMM_HIP(hipMemcpyAsync(out, d_out, sizeof out, hipMemcpyDeviceToHost, st));
+  HPSPMM_HIP(hipStreamSynchronize(st));
+  double fresh = 0, walked = 0;
+  for (int s = 0; s < kLocalitySamples; ++s) {
+    fresh += (double)out[4 * s + 3] - (double)out[4 * s + 1];
+    walked += (double)out[4 * s + 2] - (double)out[4 * s + 0];
+  }
+  if (walked > 0) *share = std::min(1.0, fresh / walked);
+  return HPSPMM_OK;
+}
+
 }  // namespace hpspmm_host

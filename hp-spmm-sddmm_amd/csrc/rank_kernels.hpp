@@ -251,4 +251,52 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void label_sizes_kernel(int64_t rows, co
   if (r < rows) atomicAdd(&size[label[r]], 1);
 }
 
+// Locality of the stored order: how often a gather of a row of B finds that row among the last
+// `capacity` distinct ones.  One workgroup per sample walks the column indices from its start
+// (wrapping at the end), one chunk of kLocalityBlock in every kLocalityDeal - what one XCD gets of
+// consecutive pieces of the matrix -, marks every column in a bit table of its own and counts the
+// columns it had not marked before.  The walk ends once `capacity` distinct columns have been seen
+// or after max_walk nonzeros.  out[4 s ..]: nonzeros walked and distinct columns when the count first
+// reached capacity / 2 (0, 0 if it never did), the same two at the end: the slope between the two
+// points is the share of the gathers that miss a cache of about 3/4 of that capacity.
+constexpr int kLocalityBlock = 1024;
+constexpr int kLocalityDeal = 8;
+constexpr int kLocalityBits = 22;  // bits per table; columns beyond that many are hashed into it
+HPSPMM_KERNEL __launch_bounds__(kLocalityBlock) void locality_walk_kernel(int64_t nnz, const int32_t* __restrict__ col,
+                                                                         int64_t sample_stride, int hashed,
+                                                                         uint32_t capacity, uint32_t max_walk,
+                                                                         uint32_t* __restrict__ tables,
+                                                                         uint32_t* __restrict__ out) {
+  __shared__ uint32_t s_new[3];
+  uint32_t* table = tables + ((size_t)blockIdx.x << (kLocalityBits - 5));
+  if (threadIdx.x < 3) s_new[threadIdx.x] = 0;
+  __syncthreads();
+  const int64_t base = (int64_t)blockIdx.x * sample_stride;
+  uint32_t walked = 0, distinct = 0, half_walked = 0, half_distinct = 0;
+  for (uint32_t it = 0; walked < max_walk && distinct < capacity; ++it) {
+    const int64_t q = (base + (int64_t)it * kLocalityDeal * kLocalityBlock + threadIdx.x) % nnz;
+    const uint32_t c = (uint32_t)col[q];
+    const uint32_t h = hashed ? (c * 2654435761u) >> (32 - kLocalityBits) : c;
+    const uint32_t bit = 1u << (h & 31);
+    const bool fresh = !(atomicOr(&table[h >> 5], bit) & bit);
+    const unsigned long long m = __ballot(fresh);
+    if ((threadIdx.x & 63) == 0 && m) atomicAdd(&s_new[it % 3], (uint32_t)__popcll(m));
+    __syncthreads();
+    distinct += s_new[it % 3];
+    walked += kLocalityBlock;
+    // the counter of the round after the next: last read before this barrier, next added to after the next one
+    if (threadIdx.x == 0) s_new[(it + 2) % 3] = 0;
+    if (half_walked == 0 && distinct >= capacity / 2) {
+      half_walked = walked;
+      half_distinct = distinct;
+    }
+  }
+  if (threadIdx.x == 0) {
+    out[4 * blockIdx.x + 0] = half_walked;
+    out[4 * blockIdx.x + 1] = half_distinct;
+    out[4 * blockIdx.x + 2] = walked;
+    out[4 * blockIdx.x + 3] = distinct;
+  }
+}
+
 }  // namespace hpspmm

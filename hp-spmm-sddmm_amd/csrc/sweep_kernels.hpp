@@ -74,21 +74,6 @@ struct SweepLayout {
 
 // ---- plan-time kernels -----------------------------------------------------
 
-// *sum += (last column - first column) of every row (sorted columns): how far the rows reach across
-// the columns.  The walk over B suits rows that reach all the way; a banded matrix would leave every
-// wavefront busy in a few windows of its own.
-HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_row_span_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
-                                                                const int32_t* __restrict__ col,
-                                                                unsigned long long* __restrict__ sum) {
-  unsigned long long mine = 0;
-  for (int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x; r < rows; r += (int64_t)gridDim.x * kBlock) {
-    const int32_t lb = rowptr[r], hb = rowptr[r + 1];
-    if (hb - lb >= 2) mine += (unsigned long long)(col[hb - 1] - col[lb]);
-  }
-  for (int off = 32; off > 0; off >>= 1) mine += __shfl_down(mine, off);
-  if ((threadIdx.x & 63) == 0 && mine) atomicAdd(sum, mine);
-}
-
 // pieces[r] = number of pieces of row r (0 for an empty row), parts[r] = the same if the row is split,
 // else 0 (its partial-result rows); both get a trailing 0 for the scans' totals.
 HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_row_pieces_kernel(int64_t rows, const int32_t* __restrict__ rowptr,

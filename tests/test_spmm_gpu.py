@@ -775,8 +775,8 @@ def test_hip_graph_capture_and_replay(pkg, oracle, gpu):
 
 
 def test_auto_strategy_leaves_short_rows_unrouted(pkg, oracle, gpu):
-    """Popular columns but no long rows: routing would move nothing, so the plan must stay with the
-    segments strategy; forced routing of the same matrix still gives the right result."""
+    """Popular columns but no long rows: routing would move nothing, so the plan must stay with
+    segments or whole rows; forced routing of the same matrix still gives the right result."""
     import torch
     capi = pkg.capi
     rng = np.random.default_rng(77)
@@ -788,7 +788,7 @@ def test_auto_strategy_leaves_short_rows_unrouted(pkg, oracle, gpu):
     g = pkg.graphs.CSR(rows, cols, rowptr, col, val)
     B = rng.standard_normal((cols, k)).astype(np.float32)
     C, info = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
-    assert info["strategy"] == capi.STRATEGY_SEGMENTS
+    assert info["strategy"] in (capi.STRATEGY_SEGMENTS, capi.STRATEGY_ROWS)
     lo, hi = 50_000, 54_000
     C64, S64 = oracle.csr_spmm_f64_rows(g.rowptr, g.col, g.val, B, lo, hi)
     err, _ = oracle.max_norm_err(C[lo:hi], C64, S64)
@@ -806,8 +806,10 @@ def test_auto_strategy_leaves_short_rows_unrouted(pkg, oracle, gpu):
     assert info_r["strategy"] == capi.STRATEGY_ROUTED
     err, _ = oracle.max_norm_err(Cr[lo:hi], C64, S64)
     assert err <= TOL
-    # the two strategies add every row's products in the same (stored) order here: no row is routed
-    assert np.array_equal(C, Cr)
+    # segments and routed add every row's products in the same (stored) order here: no row is routed
+    Cs, info_s = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SEGMENTS)
+    assert info_s["strategy"] == capi.STRATEGY_SEGMENTS
+    assert np.array_equal(Cs, Cr)
 
 
 @pytest.mark.parametrize("k", [32, 64, 128])

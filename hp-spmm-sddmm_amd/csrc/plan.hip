@@ -62,7 +62,11 @@ int choose_shift(int64_t nnz, int64_t k, int64_t max_row_nnz) {
 
 // Automatic clustering is tried for graphs of at least this size ...
 constexpr int64_t kClusterMinNnz = (int64_t)1 << 22;
-constexpr int64_t kClusterMinBBytes = (int64_t)24 << 20;
+constexpr int64_t kClusterMinBBytes = (int64_t)12 << 20;  // co-purchase graph, 6 M nonzeros, K = 32 (B = 16 MB): 65 us against 87 for whole rows
+// The sweep is chosen where it is expected to take this share of the time of whole rows: at once,
+// and once the ordered strategy has been tried.
+constexpr double kSweepSureGain = 0.7, kSweepMinGain = 0.9;
+constexpr int64_t kOtherLayoutsMinNnz = (int64_t)1 << 21;  // below: whole rows without looking further
 // A matrix whose stored order is local already has its communities side by side; another order pays
 // only where B is far beyond every cache (blocks of 8 to 4096 vertices along the diagonal with 10 % of
 // the entries elsewhere, K = 32 / 64 / 128: at 10 M nonzeros (B = 38 / 77 / 154 MB) ordered 109 / 193 /
@@ -320,7 +324,7 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
     const bool even_enough = (double)p->max_row_nnz < (short_rows ? 512.0 : 16.0) * mean_row;
     rows_fallback = fast_k(k) && even_enough && nnz < kRowTileMaxNnz && p->max_row_nnz <= longest_ok &&
                     !(flags & HPSPMM_PLAN_NO_ROW_TILES) && (miss <= kRowsFallbackMissShare || k == 32);
-    if (nnz == 0 || tiny || (mid && nnz < kClusterMinNnz)) {
+    if (nnz == 0 || tiny || (mid && nnz < kOtherLayoutsMinNnz)) {
       p->strategy = HPSPMM_STRATEGY_ROWS;
       rows_need_tiles = !(nnz == 0 || tiny);
       want_row_tiles = mid;
@@ -348,6 +352,11 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
     // what the segments kernels need (the row of every nonzero, the carry slots) is allocated at the
     // end, if the plan is still a segments plan then: the layouts tried below mostly replace both
   }
+  const bool want_cluster = (flags & HPSPMM_PLAN_CLUSTER) != 0;
+  // a graph (square) large enough for an order of its rows by community to pay, if it has communities
+  const bool cluster_candidate = rows == cols && nnz >= kClusterMinNnz && nnz >= rows * kClusterMinMeanNnz &&
+                                 cols * k * 4 >= (miss <= kLocalMissShare ? kClusterLocalMinBBytes : kClusterMinBBytes) &&
+                                 !(flags & HPSPMM_PLAN_NO_CLUSTER);
   // Long rows over a B that is small against the gather volume: every wavefront walks B window by
   // window (tried first: where it qualifies it beats the routed strategy - social graph, 233k
   // vertices, K = 32 / 64 / 128: 1.09 / 1.68 / 2.86 ms against 1.11 / 1.92 / 3.72).  When the matrix
@@ -356,7 +365,12 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && nnz > 0 && !(flags & HPSPMM_PLAN_NO_SWEEP) &&
       ((flags & HPSPMM_PLAN_FORCE_SWEEP) ||
        !(flags & (HPSPMM_PLAN_FORCE_SEGMENTS | HPSPMM_PLAN_FORCE_ROUTED | HPSPMM_PLAN_CLUSTER)))) {
-    if (int rc = build_sweep(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_SWEEP) != 0, rows_us, opt, st)) return rc;
+    // (where the gain expected is small, a matrix that may have communities is served better by the
+    // ordered strategy, which is tried first then: co-purchase graph at 6 M nonzeros, K = 32: sweep
+    // 87 us, whole rows 87, ordered 65)
+    if (int rc = build_sweep(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_SWEEP) != 0,
+                             (cluster_candidate ? kSweepSureGain : kSweepMinGain) * rows_us, opt, st))
+      return rc;
   }
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && !(flags & HPSPMM_PLAN_NO_ROUTED) && nnz > 0 &&
       !rows_range &&
@@ -369,12 +383,8 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
   // both popular columns and communities (the co-purchase graph at a quarter of its size: the 64k
   // most referenced columns take a quarter of the nonzeros there), and the ordered strategy is then
   // the faster of the two (0.73 ms against 1.15 ms for segments with the hub cache).
-  const bool want_cluster = (flags & HPSPMM_PLAN_CLUSTER) != 0;
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && rows == cols && nnz > 0 &&
-      !(flags & HPSPMM_PLAN_NO_CLUSTER) &&
-      (want_cluster || (!(flags & HPSPMM_PLAN_FORCE_SEGMENTS) && nnz >= kClusterMinNnz &&
-                        cols * k * 4 >= (miss <= kLocalMissShare ? kClusterLocalMinBBytes : kClusterMinBBytes) &&
-                        nnz >= rows * kClusterMinMeanNnz))) {
+      !(flags & HPSPMM_PLAN_NO_CLUSTER) && (want_cluster || (!(flags & HPSPMM_PLAN_FORCE_SEGMENTS) && cluster_candidate))) {
     int32_t* d_order = nullptr;
     double intra_share = 0.0;
     int rc = cluster_rows(p, d_rowptr, d_col, opt, st, &d_order, &intra_share);
@@ -384,6 +394,10 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
     if (rc) {
       return rc;
     }
+  }
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && nnz > 0 && rows_us > 0 &&
+      !(flags & (HPSPMM_PLAN_NO_SWEEP | HPSPMM_PLAN_FORCE_SEGMENTS | HPSPMM_PLAN_FORCE_ROUTED | HPSPMM_PLAN_CLUSTER))) {
+    if (int rc = build_sweep(p, d_rowptr, d_col, false, kSweepMinGain * rows_us, opt, st)) return rc;
   }
   if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && (rows_range || rows_fallback) && row_tiles_serve(k, opt)) {
     // no communities: whole rows after all, if the row tiles get built

@@ -19,7 +19,6 @@ inline int sweep_lead(int64_t k) { return k >= 128 ? 3 : 2; }
 // Automatic choice: B beyond what the L2s hold between them without help, enough work to fill the device.
 // picoseconds per nonzero and microseconds per band and window at K = 32 / 64 / 128
 constexpr double kSweepPsPerNnz[3] = {6.5, 8.8, 13.4}, kSweepUsPerWindow[3] = {1.44, 1.72, 1.36};
-constexpr double kSweepMinGain = 0.9;  // expected time against that of whole rows for the sweep to be chosen
 constexpr int64_t kSweepMinNnz = (int64_t)1 << 21;
 constexpr int64_t kSweepMinBBytes = (int64_t)5 << 20;  // social graph: 6 MB of B, sweep 103 / 127 us against 123 / 141; 3 MB: 90 / 65 against 87 / 63
 
@@ -78,15 +77,15 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
   // What a sweep takes: every gather hits, and every band walks all the windows at the pace of the
   // slowest wavefront.  Over matrices of 25 to 200 uniformly placed nonzeros per row, 30k to 500k rows
   // and columns, square and 16 : 1 either way: 6.5 / 8.8 / 13.4 ps per nonzero and 1.44 / 1.72 / 1.36 us
-  // per band and window at K = 32 / 64 / 128, within 25 % everywhere and 10 % rms.  Worth it where
-  // that is below what whole rows are expected to take in the stored order (`other_us`).  Every
+  // per band and window at K = 32 / 64 / 128, within 25 % everywhere and 10 % rms.  Chosen where
+  // that is below `other_us` (a share of what whole rows are expected to take in stored order).  Every
   // non-empty row is at least one piece: the first test rules the layout out for most matrices before
   // any kernel has run.
   const int ki = k == 32 ? 0 : k == 64 ? 1 : 2;
   auto expected_us = [&](int64_t bands) {
     return kSweepPsPerNnz[ki] * (double)nnz * 1e-6 + kSweepUsPerWindow[ki] * (double)(bands * n_windows);
   };
-  if (!forced && (other_us <= 0 || expected_us(ceil_div(nonempty, band_waves * WS)) > kSweepMinGain * other_us)) return HPSPMM_OK;
+  if (!forced && (other_us <= 0 || expected_us(ceil_div(nonempty, band_waves * WS)) > other_us)) return HPSPMM_OK;
   if (!columns_sorted(p, d_rowptr, d_col, st)) return HPSPMM_OK;  // a row must meet the windows in stored order
 
   DeviceTemps tmp;
@@ -117,7 +116,7 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
 
   const int64_t n_bands = ceil_div((int64_t)n_pieces, band_waves * WS);
   // (the same test with the bands there really are: long rows are several pieces)
-  if (n_bands > kSweepMaxBands || (!forced && expected_us(n_bands) > kSweepMinGain * other_us)) {
+  if (n_bands > kSweepMaxBands || (!forced && expected_us(n_bands) > other_us)) {
     drop_sweep_buffers(p);
     return HPSPMM_OK;
   }

@@ -600,6 +600,47 @@ hpspmm_graph* hpspmm_gen_blocks(int64_t n, int64_t min_size, int64_t max_size, d
   return (hpspmm_graph*)build_symmetric(n, n_edges, smp, false, kValSymUniform01, seed);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Cache model (CPU side, for traffic estimates): misses of a fully associative LRU cache of
+// `capacity` entries over a stream of n ids in [0, id_range).  Negative ids are skipped.
+// ---------------------------------------------------------------------------------------------
+int64_t hpspmm_model_lru_misses(const int32_t* ids, int64_t n, int64_t id_range, int64_t capacity) {
+  if (!ids || n < 0 || id_range <= 0 || capacity <= 0) return -1;
+  // doubly linked list over the ids, most recent at the head
+  std::vector<int32_t> prev((size_t)id_range, -1), next((size_t)id_range, -1);
+  std::vector<uint8_t> in((size_t)id_range, 0);
+  int32_t head = -1, tail = -1;
+  int64_t held = 0, misses = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    const int32_t c = ids[i];
+    if (c < 0 || c >= id_range) continue;
+    if (in[c]) {
+      if (head == c) continue;
+      // unlink
+      const int32_t p = prev[c], q = next[c];
+      next[p] = q;
+      if (q >= 0) prev[q] = p; else tail = p;
+    } else {
+      ++misses;
+      in[c] = 1;
+      if (held == capacity) {  // evict the least recent
+        const int32_t t = tail;
+        tail = prev[t];
+        if (tail >= 0) next[tail] = -1; else head = -1;
+        in[t] = 0;
+      } else {
+        ++held;
+      }
+    }
+    prev[c] = -1;
+    next[c] = head;
+    if (head >= 0) prev[head] = c;
+    head = c;
+    if (tail < 0) tail = c;
+  }
+  return misses;
+}
+
 // The benchmark configurations by name.  scale < 1 shrinks vertex and edge
 // counts together (tests); scale = 1 is the benchmark size.  Parameters were
 // calibrated so that the full-size graphs land on the configured statistics:

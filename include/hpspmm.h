@@ -184,8 +184,10 @@ const char *hpspmm_last_error(void);
  * Analyse the sparsity structure of A for a given k and build the device-side
  * work assignment.  The plan picks a strategy (reported by
  * hpspmm_plan_get_info): whole rows for small and medium matrices (below 2^24
- * nonzeros and nnz * k < 2^30, less when the rows are long; the rows cut into
- * 8-nonzero slots and packed, by length class, into one 64-entry tile per
+ * nonzeros and nnz * k < 2^30, less when the rows are long) and for matrices
+ * of any size whose stored order is local - rows that share columns with their
+ * neighbours, which the plan measures on a sample of the column stream (the
+ * rows cut into 8-nonzero slots and packed, by length class, into one 64-entry tile per
  * wavefront, so that a microsecond-scale SpMM is one launch with a two-step
  * dependent chain); fixed-length segments of nonzeros with a carry buffer;
  * for a large matrix of long rows whose B is small against the gather volume,

@@ -3,6 +3,7 @@
 #include "host.hpp"
 
 #include "rank_kernels.hpp"
+#include "routed_plan_kernels.hpp"
 #include "rowtile_kernels.hpp"
 
 #include <new>

@@ -3,6 +3,7 @@
 
 #include "ordered_kernels.hpp"
 #include "rank_kernels.hpp"
+#include "routed_plan_kernels.hpp"
 
 namespace hpspmm_host {
 

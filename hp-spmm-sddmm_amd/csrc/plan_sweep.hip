@@ -2,6 +2,7 @@
 #include "host.hpp"
 
 #include "rank_kernels.hpp"
+#include "routed_plan_kernels.hpp"
 
 namespace hpspmm_host {
 

@@ -7,6 +7,7 @@
 #include <string>
 
 #include "rank_kernels.hpp"
+#include "routed_plan_kernels.hpp"
 
 namespace hpspmm_host {
 

@@ -4,8 +4,15 @@
 // EXE_NUM_CUDA back-to-back launches (spmm/mm/spmm_kernel.cu:404-424).
 #pragma once
 
+#include <string>
+
 #include "spmm/spmm_common.h"
 #include "spmm/timer.h"
+
+// A field of hpspmm_plan_options (by its name in include/hpspmm.h) for every plan GESpMM and HPSpMM
+// build from here on; false if there is no such field.  Diagnostics and comparisons: no counterpart
+// in the reference, whose launchers have no plan.
+bool set_spmm_plan_option(const std::string& field, long value);
 
 // C = A * B for CSR A.  Stands in for GESpMM (spmm_kernel.cu:389-426): same
 // arguments, C overwritten.  Builds a plan (untimed, like the reference's host

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime_api.h>
 #include <rocsparse/rocsparse.h>
 
+#include <cstddef>
+#include <cstring>
 #include <iostream>
 
 #include "hpspmm.h"
@@ -28,6 +30,10 @@ Dims check_operands(int64_t rows, int64_t cols, const Matrix& idx_a, const Matri
   return d;
 }
 
+// Plan options of GESpMM / HPSpMM (set_spmm_plan_option); all zero = the library's own choices.
+hpspmm_plan_options g_plan_options{};
+bool g_have_plan_options = false;
+
 void check_status(int rc, const char* who) {
   if (rc != HPSPMM_OK) throw Error(std::string(who) + ": " + hpspmm_last_error());
 }
@@ -38,9 +44,16 @@ void csr_spmm_timed(const CSR_Matrix& a, const Matrix& mat2, Matrix& result, flo
   if (rp.size() != a.num_rows() + 1) throw Error(std::string(who) + ": row_offsets must have num_rows + 1 entries");
   const Dims d = check_operands(a.num_rows(), a.num_cols(), rp, ci, va, mat2, result, who);
   hpspmm_plan* plan = nullptr;
-  check_status(hpspmm_plan_create(d.m, d.n, d.nnz, rp.data<int32_t>(), ci.data<int32_t>(), d.k, HPSPMM_PLAN_DEFAULT,
-                                  nullptr, &plan),
-               who);
+  if (g_have_plan_options) {
+    g_plan_options.struct_size = sizeof(hpspmm_plan_options);
+    check_status(hpspmm_plan_create_ex(d.m, d.n, d.nnz, rp.data<int32_t>(), ci.data<int32_t>(), d.k, &g_plan_options,
+                                       nullptr, &plan),
+                 who);
+  } else {
+    check_status(hpspmm_plan_create(d.m, d.n, d.nnz, rp.data<int32_t>(), ci.data<int32_t>(), d.k, HPSPMM_PLAN_DEFAULT,
+                                    nullptr, &plan),
+                 who);
+  }
   if (bind_values) {
     const int rb = hpspmm_plan_bind_values(plan, va.data<float>(), nullptr);
     if (rb != HPSPMM_OK) {
@@ -57,6 +70,39 @@ void csr_spmm_timed(const CSR_Matrix& a, const Matrix& mat2, Matrix& result, flo
 }
 
 }  // namespace
+
+bool set_spmm_plan_option(const std::string& field, long value) {
+  struct Field {
+    const char* name;
+    size_t offset;
+    bool is_unsigned;
+  };
+#define HPSPMM_OPTION(f) {#f, offsetof(hpspmm_plan_options, f), false}
+  static const Field fields[] = {
+      {"flags", offsetof(hpspmm_plan_options, flags), true},
+      HPSPMM_OPTION(segment_shift), HPSPMM_OPTION(hub_log2), HPSPMM_OPTION(routed_row_log2),
+      HPSPMM_OPTION(routed_phases), HPSPMM_OPTION(routed_tile_width), HPSPMM_OPTION(routed_split_launch),
+      HPSPMM_OPTION(routed_lds_rows), HPSPMM_OPTION(xcd_dealing), HPSPMM_OPTION(no_column_tiles),
+      HPSPMM_OPTION(row_tiles_min_k), HPSPMM_OPTION(row_tiles_pad), HPSPMM_OPTION(row_tiles_wide),
+      HPSPMM_OPTION(row_tiles_round_robin), HPSPMM_OPTION(sweep_window_log2), HPSPMM_OPTION(sweep_lead),
+      HPSPMM_OPTION(sweep_spin), HPSPMM_OPTION(sweep_limit), HPSPMM_OPTION(sweep_no_priorities),
+      HPSPMM_OPTION(cluster_sweeps), HPSPMM_OPTION(report)};
+#undef HPSPMM_OPTION
+  for (const Field& f : fields) {
+    if (field != f.name) continue;
+    char* at = reinterpret_cast<char*>(&g_plan_options) + f.offset;
+    if (f.is_unsigned) {
+      const uint32_t v = (uint32_t)value;
+      std::memcpy(at, &v, sizeof v);
+    } else {
+      const int32_t v = (int32_t)value;
+      std::memcpy(at, &v, sizeof v);
+    }
+    g_have_plan_options = true;
+    return true;
+  }
+  return false;
+}
 
 void GESpMM(const CSR_Matrix& mat1, const Matrix& mat2, Matrix& result, float& time) {
   csr_spmm_timed(mat1, mat2, result, time, "GESpMM", false);

@@ -2,6 +2,8 @@
 //
 //   spmm_test_all <graph.smtx> <graph.reorder | -> <K> [--check] [--csv file] [--dump-c prefix]
 //   spmm_test_all --synthetic <name> <scale> <K> [--check] [--csv file] [--dump-c prefix]
+//   (either form: [--vendor-algs 2,3,-1,coo] [--plan-option FIELD=VALUE]..., a field of
+//   hpspmm_plan_options for the plans of GESpMM and HPSpMM, for comparisons)
 //
 // It loads (or generates) the graph, moves it to the GPU, times the vendor
 // comparator (rocSPARSE, in the slots the reference gives cuSPARSE), the CSR
@@ -46,12 +48,20 @@ int main(int argc, char** argv) {
       if (a == "--check") check = true;
       else if (a == "--synthetic") synthetic = true;
       else if (a == "--csv" && i + 1 < argc) csv = argv[++i];
+      else if (a == "--plan-option" && i + 1 < argc) {
+        const std::string kv = argv[++i];
+        const size_t eq = kv.find('=');
+        if (eq == std::string::npos || !set_spmm_plan_option(kv.substr(0, eq), std::stol(kv.substr(eq + 1)))) {
+          std::cerr << "error: --plan-option wants FIELD=VALUE with a field of hpspmm_plan_options, got '" << kv << "'\n";
+          return 2;
+        }
+      }
       else if (a == "--dump-c" && i + 1 < argc) dump = argv[++i];
       else if (a == "--vendor-algs" && i + 1 < argc) vendor = argv[++i];
       else pos.push_back(a);
     }
     if (pos.size() != 3) {
-      std::cerr << "usage: " << argv[0] << " <graph.smtx> <graph.reorder|-> <K> [--check] [--csv file] [--dump-c prefix] [--vendor-algs 2,3,-1,coo]\n"
+      std::cerr << "usage: " << argv[0] << " <graph.smtx> <graph.reorder|-> <K> [--check] [--csv file] [--dump-c prefix] [--vendor-algs 2,3,-1,coo] [--plan-option FIELD=VALUE]\n"
                 << "       " << argv[0] << " --synthetic <name> <scale> <K> [--check] [--csv file] [--dump-c prefix]\n";
       return 2;
     }

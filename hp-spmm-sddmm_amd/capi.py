@@ -100,6 +100,7 @@ class PlanInfo(ctypes.Structure):
         ("num_segments", _i64), ("max_row_nnz", _i64), ("empty_rows", _i64),
         ("workspace_bytes", _i64), ("launches_per_spmm", ctypes.c_int32), ("column_tiles", ctypes.c_int32),
         ("hub_rows", _i64), ("lds_served_nnz", _i64), ("row_tiles", _i64),
+        ("stored_order_miss_share", ctypes.c_double),
     ]
 
     def as_dict(self):

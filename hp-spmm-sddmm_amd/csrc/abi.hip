@@ -6,7 +6,7 @@
 
 using namespace hpspmm_host;
 
-HPSPMM_API int hpspmm_version(void) { return 200; }
+HPSPMM_API int hpspmm_version(void) { return 201; }
 
 HPSPMM_API const char* hpspmm_last_error(void) { return last_error_message(); }
 

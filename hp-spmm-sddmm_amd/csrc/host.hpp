@@ -161,6 +161,7 @@ struct PlanOptions {
 
 struct hpspmm_plan {
   int64_t rows = 0, cols = 0, nnz = 0, k = 0;
+  double stored_miss = -1.0;  // stored_order_miss_share() of the matrix, if the choice of strategy measured it
   // A row length that is a multiple of 4 but not a tuned one (256 = 2 x 128, 40 = one tile of 64 with
   // 10 of its 16 lanes) can be served by a layout built for a tuned length, one column tile after
   // the other: k is then the tile width, k_full the row length of B and C, tiles = ceil(k_full / k).

@@ -301,6 +301,7 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
     // does not.
     if (!tiny && nnz > 0 && fast_k(k)) {
       if (int rc = stored_order_miss_share(p, d_col, st, &miss)) return rc;
+      p->stored_miss = miss;
       rows_us = (double)nnz * (double)(k / 32) * (kRowsHitPs + (kRowsMissPs - kRowsHitPs) * miss) * 1e-6;
     }
     // A matrix whose stored order is local (banded, a mesh, blocks along the diagonal) is served best
@@ -605,6 +606,7 @@ HPSPMM_API int hpspmm_plan_get_info(const hpspmm_plan* plan, hpspmm_plan_info* o
   out->hub_rows = plan->n_hub;
   out->lds_served_nnz = plan->oserved;
   out->row_tiles = plan->d_tent ? plan->rt_tiles : 0;
+  out->stored_order_miss_share = plan->stored_miss;
   return HPSPMM_OK;
 }
 

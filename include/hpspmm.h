@@ -153,6 +153,9 @@ typedef struct hpspmm_plan_info {
   int64_t hub_rows;        /* rows of B kept in the hub cache (0 = none) */
   int64_t lds_served_nnz;  /* ordered strategy: nonzeros whose row of B comes from a workgroup's LDS copy */
   int64_t row_tiles;       /* rows strategy: 64-entry tiles of the plan's row-tile layout (0: the CSR arrays are walked) */
+  double stored_order_miss_share; /* share of the gathers of rows of B that miss an L2 when the nonzeros are taken
+                                     in stored order, as sampled for the choice of strategy (k = 32 / 64 / 128, from
+                                     2^21 nonzeros, no forcing flag); -1 when it was not measured */
 } hpspmm_plan_info;
 
 /* Library version, major*10000 + minor*100 + patch. */

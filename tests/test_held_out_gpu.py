@@ -70,3 +70,34 @@ def test_held_out_family(pkg, oracle, gpu, bench, family, scale):
             f"{family} x{scale} K={k}: default plan (strategy {chosen}) {t['auto']:.1f} us, "
             f"{best_name} forced {best:.1f} us; all: {t}")
         del Bd, C
+
+
+def test_locality_of_the_stored_order_is_measured(pkg, gpu):
+    """hpspmm_plan_info.stored_order_miss_share, the sampled share of the gathers that miss an L2 in
+    stored order, on matrices whose answer is known: columns without any order, a B that fits the
+    cache, a mesh (each row shares its columns with its neighbours), and no measurement for a small
+    matrix or under a forcing flag."""
+    import torch
+    capi, graphs = pkg.capi, pkg.graphs
+
+    def share(g, k=64, flags=0):
+        rp, ci = (torch.from_numpy(a).to(gpu) for a in (g.rowptr, g.col))
+        plan = capi.Plan(g.rows, g.cols, rp, ci, k, flags)
+        info = plan.info
+        plan.destroy()
+        return info["stored_order_miss_share"], info["strategy"]
+
+    uniform = graphs.uniform_rows(400_000, 400_000, 20, 5)      # 8 M nonzeros over 400k columns: nearly every gather misses
+    m, _ = share(uniform)
+    assert 0.85 <= m <= 1.0, m
+    fits = graphs.uniform_rows(400_000, 20_000, 20, 5)          # 20k columns: all of them within reach
+    m, _ = share(fits)
+    assert 0.0 <= m <= 0.05, m
+    mesh = graphs.make_graph("h3_grid", 0.12)                     # 9 of 13 entries per row shared with neighbouring rows
+    m, strategy = share(mesh, k=128)
+    assert 0.25 <= m <= 0.65, m
+    assert strategy == capi.STRATEGY_ROWS                          # 12 M nonzeros x 128 columns: whole rows all the same
+    m, _ = share(mesh, flags=capi.PLAN_FORCE_SEGMENTS)
+    assert m == -1.0
+    m, _ = share(graphs.make_graph("c1_citation"))
+    assert m == -1.0

@@ -276,7 +276,8 @@ HPSPMM_KERNEL __launch_bounds__(kLocalityBlock) void locality_walk_kernel(int64_
   for (uint32_t it = 0; walked < max_walk && distinct < capacity; ++it) {
     const int64_t q = (base + (int64_t)it * kLocalityDeal * kLocalityBlock + threadIdx.x) % nnz;
     const uint32_t c = (uint32_t)col[q];
-    const uint32_t h = hashed ? (c * 2654435761u) >> (32 - kLocalityBits) : c;
+    // (masked: the column indices of an unchecked matrix may be anything)
+    const uint32_t h = (hashed ? (c * 2654435761u) >> (32 - kLocalityBits) : c) & ((1u << kLocalityBits) - 1u);
     const uint32_t bit = 1u << (h & 31);
     const bool fresh = !(atomicOr(&table[h >> 5], bit) & bit);
     const unsigned long long m = __ballot(fresh);

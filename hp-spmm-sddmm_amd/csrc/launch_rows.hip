@@ -60,16 +60,33 @@ inline bool row_tiles_same_xcd(const hpspmm_plan* p, int kLd, uint32_t ldb) {
   return kLd != 0 && ldb % 32 != 0 && p->rt_same_xcd;
 }
 
+// Contiguous ranges of the groups of row tiles per XCD (tuned row lengths): how the groups are cut
+// and how many workgroups that takes.  `long_groups` = the groups at the front of the layout that
+// hold the long rows, which stay dealt round robin.
+hpspmm::TileRanges row_tile_ranges(const hpspmm_plan* p, int kLd, int64_t k_template, int64_t groups, int64_t long_groups,
+                                   int64_t* blocks) {
+  hpspmm::TileRanges tr{0, 0, 0, (int32_t)groups};
+  if (kLd != 0 || !p->rt_ranges || k_template <= 0 || groups < 4 * hpspmm::kXcds) return tr;
+  const int64_t ranges = hpspmm::kXcds / (k_template / 32);
+  long_groups = std::min(long_groups, groups);
+  tr.long_groups = (int32_t)long_groups;
+  tr.long_per = (int32_t)ceil_div(long_groups, ranges);
+  tr.per_range = (int32_t)std::max<int64_t>(1, ceil_div(groups - long_groups, ranges));
+  *blocks = (int64_t)hpspmm::kXcds * (tr.long_per + tr.per_range);
+  return tr;
+}
+
 template <int K, int WPB, int kLd, int kSub>
 int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, float* C, hipStream_t st, uint32_t ldb,
                        uint32_t ldc) {
   const bool same_xcd = row_tiles_same_xcd(p, kLd, ldb);
   const int64_t groups = ceil_div(p->rt_waves, WPB);
-  const int64_t blocks = (same_xcd ? ceil_div(groups, hpspmm::kXcds) * hpspmm::kXcds : groups) * row_tile_column_tiles(K, ldc);
+  int64_t blocks = (same_xcd ? ceil_div(groups, hpspmm::kXcds) * hpspmm::kXcds : groups) * row_tile_column_tiles(K, ldc);
+  const hpspmm::TileRanges ranges = row_tile_ranges(p, kLd, K, groups, ceil_div(p->rt_loop, WPB), &blocks);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB, kLd, kSub>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent, readable_values(p, v), B, C,
-                     p->d_zrow + 4, ldb, ldc, same_xcd);
+                     p->d_zrow + 4, ldb, ldc, same_xcd, ranges);
   mark_launch(st, "spmm_rowtiles_kernel");
   return HPSPMM_OK;
 }
@@ -80,11 +97,13 @@ int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, fl
   const int64_t wave_items = (p->rt_loop - p->rt_wg) + (p->rt_tiles - p->rt_loop_tiles);
   const bool same_xcd = row_tiles_same_xcd(p, kLd, ldb);
   const int64_t groups = p->rt_wg + ceil_div(wave_items, WPB);
-  const int64_t blocks = (same_xcd ? ceil_div(groups, hpspmm::kXcds) * hpspmm::kXcds : groups) * row_tile_column_tiles(K, ldc);
+  int64_t blocks = (same_xcd ? ceil_div(groups, hpspmm::kXcds) * hpspmm::kXcds : groups) * row_tile_column_tiles(K, ldc);
+  const hpspmm::TileRanges ranges =
+      row_tile_ranges(p, kLd, K, groups, p->rt_wg + ceil_div(p->rt_loop - p->rt_wg, WPB), &blocks);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB, kLd, kSub>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent,
-                     readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc, same_xcd);
+                     readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc, same_xcd, ranges);
   mark_launch(st, "spmm_rowtiles_wg_kernel");
   return HPSPMM_OK;
 }

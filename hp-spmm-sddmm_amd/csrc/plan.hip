@@ -417,6 +417,16 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
       p->strategy = HPSPMM_STRATEGY_ROWS;
     }
   }
+  if (p->d_tent && fast_k(k)) {
+    // Every XCD one contiguous range of the row tiles instead of every eighth group: only on request.
+    // It pays where neighbouring rows share columns (mesh with 2 random entries per row, 12 M nonzeros,
+    // K = 32 / 64 / 128: 151 / 269 / 599 -> 123 / 251 / 589 us; blocks along the diagonal, 10 M: 100 / 187 /
+    // 388 -> 86 / 173 / 381) and costs elsewhere, because the tiles lie sorted by the length class of
+    // their rows, so that the ranges are not equally heavy (citation graph x 16: 39 / 78 / 155 -> 50 / 94 /
+    // 187; R-MAT at 3.7 and 12 M nonzeros +4 to +7 %; preferential attachment +3 to +6 %; the mesh at
+    // 102 M +1 to +3 %).
+    p->rt_ranges = opt.row_tiles_ranges > 0;
+  }
   if (p->d_tent && !fast_k(k)) {
     // Row tiles at a row length of its own.  The gathers are fastest when every 32-column tile of a
     // row of B is one aligned 128-byte line (R-MAT graph, 3.7 M nonzeros: K = 96 131 us, K = 100
@@ -577,6 +587,8 @@ HPSPMM_API int hpspmm_plan_create_ex(int64_t rows, int64_t cols, int64_t nnz, co
   o.sweep_priorities = in.sweep_no_priorities ? 0 : -1;
   o.cluster_sweeps = std::max(0, in.cluster_sweeps);
   o.report = in.report != 0;
+  if (in.row_tiles_ranges < 0 || in.row_tiles_ranges > 2) return fail(HPSPMM_ERR_INVALID_ARG, "row_tiles_ranges must be 0, 1 or 2");
+  o.row_tiles_ranges = in.row_tiles_ranges == 0 ? -1 : in.row_tiles_ranges == 1 ? 0 : 1;
   return plan_create_guarded(rows, cols, nnz, d_rowptr, d_col, k, o, stream, plan_out);
 }
 

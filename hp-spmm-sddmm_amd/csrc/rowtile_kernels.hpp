@@ -242,9 +242,28 @@ __device__ __forceinline__ int column_tiles(uint32_t ldc) {
 // them).  same_xcd: the T tiles of a group go to workgroups b, b + 8, b + 16 ... - one XCD, one after
 // the other - for rows of B that are not a whole number of 128-byte lines: the line that two
 // neighbouring tiles share is then fetched into one L2 once instead of into two.
+//
+// ranges (tuned row lengths; per_range > 0): every XCD serves one column tile and one contiguous
+// range of the groups instead of every (8 / T)-th group, so that rows that share columns with their
+// neighbours (a mesh, a banded matrix, blocks along the diagonal) meet them in one L2 instead of
+// eight.  The first long_groups groups (the long rows, which come first in the layout) stay dealt
+// round robin - they are the heaviest -, the others are cut into 8 / T ranges of per_range groups.
+// A workgroup beyond the end of its range gets group n_groups, which has no work.
+struct TileRanges {
+  int32_t long_groups, long_per, per_range, n_groups;
+};
 template <int kLd>
-__device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, int& tile, int32_t& group) {
-  if (kLd != 0 && same_xcd) {
+__device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, const TileRanges& tr, int& tile,
+                                                  int32_t& group) {
+  if (kLd == 0 && tr.per_range > 0) {
+    const uint32_t xcd = b % (uint32_t)kXcds, j = b / (uint32_t)kXcds;
+    const uint32_t ranges = (uint32_t)kXcds / (uint32_t)T, r = xcd / (uint32_t)T;
+    tile = (int)(xcd % (uint32_t)T);
+    const uint32_t g = j < (uint32_t)tr.long_per ? j * ranges + r
+                                                 : (uint32_t)tr.long_groups + r * (uint32_t)tr.per_range + (j - (uint32_t)tr.long_per);
+    const bool idle = j < (uint32_t)tr.long_per ? g >= (uint32_t)tr.long_groups : g >= (uint32_t)tr.n_groups;
+    group = idle ? tr.n_groups : (int32_t)g;
+  } else if (kLd != 0 && same_xcd) {
     const uint32_t per = (uint32_t)kXcds * (uint32_t)T, r = b % per;
     tile = (int)(r / (uint32_t)kXcds);
     group = (int32_t)((b / per) * (uint32_t)kXcds + r % (uint32_t)kXcds);
@@ -386,7 +405,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
                                                                const float* __restrict__ val,
                                                                const float* __restrict__ B, float* __restrict__ C,
                                                                const float* __restrict__ zrow, uint32_t ldb,
-                                                               uint32_t ldc, bool same_xcd) {
+                                                               uint32_t ldc, bool same_xcd, TileRanges ranges) {
   const int T = column_tiles<K, kLd>(ldc);
   __shared__ int32_t s_col[WPB * 64];
   __shared__ int32_t s_x[WPB * 64];
@@ -399,7 +418,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
   const int base = tid - l;
   int ctile;
   int32_t group;
-  tile_of_workgroup<kLd>(blockIdx.x, T, same_xcd, ctile, group);
+  tile_of_workgroup<kLd>(blockIdx.x, T, same_xcd, ranges, ctile, group);
   const TileColumns tc = tile_columns<K, kLd, kSub>(ldb, ldc, ctile, l);
   const int32_t w = __builtin_amdgcn_readfirstlane(group * WPB + (tid >> 6));
   if (w >= n_waves) return;
@@ -432,7 +451,8 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
                                                                     const float* __restrict__ B,
                                                                     float* __restrict__ C,
                                                                     const float* __restrict__ zrow,
-                                                                    uint32_t ldb, uint32_t ldc, bool same_xcd) {
+                                                                    uint32_t ldb, uint32_t ldc, bool same_xcd,
+                                                                    TileRanges ranges) {
   const int T = column_tiles<K, kLd>(ldc);
   __shared__ int32_t s_col[WPB * 64];
   __shared__ int32_t s_x[WPB * 64];
@@ -447,7 +467,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
   const int base = tid - l;
   int ctile;
   int32_t blk;
-  tile_of_workgroup<kLd>(blockIdx.x, T, same_xcd, ctile, blk);
+  tile_of_workgroup<kLd>(blockIdx.x, T, same_xcd, ranges, ctile, blk);
   const TileColumns tc = tile_columns<K, kLd, kSub>(ldb, ldc, ctile, l);
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 

@@ -138,6 +138,8 @@ typedef struct hpspmm_plan_options {
   int32_t sweep_no_priorities; /* 1: leave the wavefront priorities alone */
   int32_t cluster_sweeps;     /* label-propagation sweeps, at most */
   int32_t report;             /* 1: plan-time reports on stderr */
+  int32_t row_tiles_ranges;   /* row tiles at k = 32 / 64 / 128: 2 = give every XCD one contiguous range of the row
+                                 tiles instead of every eighth group of them (0, 1: not) */
 } hpspmm_plan_options;
 
 typedef struct hpspmm_plan_info {

@@ -240,6 +240,7 @@ struct hpspmm_plan {
   int rt_sub = 8;            // lanes per entry of the row-tile kernels at such a row length: 8, 4 or 1
   bool rt_same_xcd = true;   // the column tiles of a group of row tiles on one XCD where rows of B share lines
   bool rt_ranges = false;    // tuned row lengths: every XCD serves one contiguous range of the row tiles
+  int32_t rt_cut[9] = {};    // ... cut where: first ordinary tile of every eighth of the work (build_row_tiles)
   // sweep strategy (its stream arrays are d_vcol = entry words, d_vsrc, d_vval when values are bound;
   // partial-result rows of split rows in d_partial; rows without nonzeros in d_zero_rows)
   hpspmm::SweepLayout sw{};

@@ -419,12 +419,14 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
   }
   if (p->d_tent && fast_k(k)) {
     // Every XCD one contiguous range of the row tiles instead of every eighth group: only on request.
-    // It pays where neighbouring rows share columns (mesh with 2 random entries per row, 12 M nonzeros,
-    // K = 32 / 64 / 128: 151 / 269 / 599 -> 123 / 251 / 589 us; blocks along the diagonal, 10 M: 100 / 187 /
-    // 388 -> 86 / 173 / 381) and costs elsewhere, because the tiles lie sorted by the length class of
-    // their rows, so that the ranges are not equally heavy (citation graph x 16: 39 / 78 / 155 -> 50 / 94 /
-    // 187; R-MAT at 3.7 and 12 M nonzeros +4 to +7 %; preferential attachment +3 to +6 %; the mesh at
-    // 102 M +1 to +3 %).
+    // It pays where neighbouring rows share columns (mesh with 2 random entries per row, 1.5 / 12 M
+    // nonzeros, K = 32 / 64 / 128: 30 / 45 / 64 -> 26 / 39 / 58 and 157 / 277 / 599 -> 134 / 264 / 593 us;
+    // blocks along the diagonal, 10 M: 111 / 200 / 380 -> 101 / 194 / 375) and costs elsewhere, although
+    // the ranges are cut by estimated work (the tiles lie sorted by the length class of their rows):
+    // citation graph x 16 and x 64: 46 / 82 / 154 -> 48 / 94 / 172 and 171 / 341 / 690 -> 219 / 422 / 743;
+    // R-MAT at 3.7 and 7.6 M nonzeros +1 to +12 %; preferential attachment, co-purchase graph, users x
+    // items +1 to +3 %; the mesh at 102 M +0 to +3 %; uniform rows, the social graph and the 20k-vertex
+    // citation graph +-1 %.
     p->rt_ranges = opt.row_tiles_ranges > 0;
   }
   if (p->d_tent && !fast_k(k)) {

@@ -247,10 +247,13 @@ __device__ __forceinline__ int column_tiles(uint32_t ldc) {
 // range of the groups instead of every (8 / T)-th group, so that rows that share columns with their
 // neighbours (a mesh, a banded matrix, blocks along the diagonal) meet them in one L2 instead of
 // eight.  The first long_groups groups (the long rows, which come first in the layout) stay dealt
-// round robin - they are the heaviest -, the others are cut into 8 / T ranges of per_range groups.
-// A workgroup beyond the end of its range gets group n_groups, which has no work.
+// round robin - they are the heaviest -, the others are cut into 8 / T ranges, range r = groups
+// [start[r], start[r + 1]), of about equal work (the tiles lie sorted by the length class of their
+// rows: equal counts would not be equal work).  A workgroup beyond the end of its range gets group
+// n_groups, which has no work.
 struct TileRanges {
-  int32_t long_groups, long_per, per_range, n_groups;
+  int32_t long_groups, long_per, per_range, n_groups;  // per_range = the longest range (0: no ranges)
+  int32_t start[kXcds + 1];
 };
 template <int kLd>
 __device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, const TileRanges& tr, int& tile,
@@ -259,9 +262,8 @@ __device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_x
     const uint32_t xcd = b % (uint32_t)kXcds, j = b / (uint32_t)kXcds;
     const uint32_t ranges = (uint32_t)kXcds / (uint32_t)T, r = xcd / (uint32_t)T;
     tile = (int)(xcd % (uint32_t)T);
-    const uint32_t g = j < (uint32_t)tr.long_per ? j * ranges + r
-                                                 : (uint32_t)tr.long_groups + r * (uint32_t)tr.per_range + (j - (uint32_t)tr.long_per);
-    const bool idle = j < (uint32_t)tr.long_per ? g >= (uint32_t)tr.long_groups : g >= (uint32_t)tr.n_groups;
+    const uint32_t g = j < (uint32_t)tr.long_per ? j * ranges + r : (uint32_t)tr.start[r] + (j - (uint32_t)tr.long_per);
+    const bool idle = j < (uint32_t)tr.long_per ? g >= (uint32_t)tr.long_groups : g >= (uint32_t)tr.start[r + 1];
     group = idle ? tr.n_groups : (int32_t)g;
   } else if (kLd != 0 && same_xcd) {
     const uint32_t per = (uint32_t)kXcds * (uint32_t)T, r = b % per;

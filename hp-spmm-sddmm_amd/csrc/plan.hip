@@ -230,9 +230,12 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
   const bool xcd_ok = xcd_dealing_holds(st, opt.xcd_dealing);
   p->xcd_remap = !(flags & HPSPMM_PLAN_NO_XCD_REMAP) && xcd_ok;
 
-  // Automatic choice, in this order: tiny matrix -> rows; a matrix in the rows strategy's range
-  // (`rows_range`) -> ordered if it has communities, else rows; beyond that range -> routed if a
-  // few columns take most of the nonzeros, else ordered if it has communities, else segments.
+  // Automatic choice, in this order: tiny matrix -> rows; sweep where its expected time is well
+  // below that of whole rows; a matrix in the rows strategy's range (`rows_range`: by size, or at any
+  // size when its stored order is local) -> ordered if it has communities, else sweep if that is
+  // still expected to pay, else rows; beyond that range -> routed if a few columns take most of the
+  // nonzeros, else ordered if it has communities, else sweep as before, else rows where the rows
+  // are even and not all gathers miss (`rows_fallback`), else segments.
   ColumnRanking ranking;         // column popularity, shared by the routed and the hub-cache decisions
   bool rows_need_tiles = false;  // rows strategy chosen on the strength of the row tiles
   bool rows_range = false;       // provisional segments; rows unless the ordered strategy qualifies
@@ -304,12 +307,12 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
       p->stored_miss = miss;
       rows_us = (double)nnz * (double)(k / 32) * (kRowsHitPs + (kRowsMissPs - kRowsHitPs) * miss) * 1e-6;
     }
+    if (opt.report && rows_us > 0)
+      fprintf(stderr, "plan: %.3f of the gathers miss in stored order, whole rows expected to take %.1f us\n", miss, rows_us);
     // A matrix whose stored order is local (banded, a mesh, blocks along the diagonal) is served best
     // by whole rows at any size: the gathers of neighbouring rows meet in the L2, and nothing is left
     // for the other layouts to gain (9-point mesh with 2 random entries per row, 102 M nonzeros,
     // K = 32 / 64 / 128: 1.27 / 2.58 / 5.75 ms against 1.81 / 3.31 / 6.44 for segments).
-    if (opt.report && rows_us > 0)
-      fprintf(stderr, "plan: %.3f of the gathers miss in stored order, whole rows expected to take %.1f us\n", miss, rows_us);
     const bool short_rows = mean_row <= kRowsAutoLongMean;
     const bool local = fast_k(k) && miss <= kLocalMissShare && short_rows && nnz < kRowTileMaxNnz;
     const bool mid = (in_range || local) && p->max_row_nnz <= longest_ok && !(flags & HPSPMM_PLAN_NO_ROW_TILES);

@@ -98,9 +98,18 @@ int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, flo
   int64_t blocks = (same_xcd ? ceil_div(groups, hpspmm::kXcds) * hpspmm::kXcds : groups) * row_tile_column_tiles(K, ldc);
   const hpspmm::TileRanges ranges = row_tile_ranges(p, kLd, K, groups, ceil_div(p->rt_loop, WPB), WPB, 0, &blocks);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  if constexpr (kLd == 0) {
+    if (ranges.per_range > 0) {
+      hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB, kLd, kSub, true>), dim3((unsigned)blocks), dim3(WPB * 64), 0,
+                         st, p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent, readable_values(p, v), B, C,
+                         p->d_zrow + 4, ldb, ldc, same_xcd, ranges);
+      mark_launch(st, "spmm_rowtiles_kernel");
+      return HPSPMM_OK;
+    }
+  }
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB, kLd, kSub>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent, readable_values(p, v), B, C,
-                     p->d_zrow + 4, ldb, ldc, same_xcd, ranges);
+                     p->d_zrow + 4, ldb, ldc, same_xcd, hpspmm::NoTileRanges{});
   mark_launch(st, "spmm_rowtiles_kernel");
   return HPSPMM_OK;
 }
@@ -115,9 +124,18 @@ int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, fl
   const hpspmm::TileRanges ranges =
       row_tile_ranges(p, kLd, K, groups, p->rt_wg + ceil_div(p->rt_loop - p->rt_wg, WPB), WPB, p->rt_wg, &blocks);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
+  if constexpr (kLd == 0) {
+    if (ranges.per_range > 0) {
+      hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB, kLd, kSub, true>), dim3((unsigned)blocks), dim3(WPB * 64),
+                         0, st, p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent,
+                         readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc, same_xcd, ranges);
+      mark_launch(st, "spmm_rowtiles_wg_kernel");
+      return HPSPMM_OK;
+    }
+  }
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB, kLd, kSub>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent,
-                     readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc, same_xcd, ranges);
+                     readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc, same_xcd, hpspmm::NoTileRanges{});
   mark_launch(st, "spmm_rowtiles_wg_kernel");
   return HPSPMM_OK;
 }

@@ -423,13 +423,13 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
   if (p->d_tent && fast_k(k)) {
     // Every XCD one contiguous range of the row tiles instead of every eighth group: only on request.
     // It pays where neighbouring rows share columns (mesh with 2 random entries per row, 1.5 / 12 M
-    // nonzeros, K = 32 / 64 / 128: 30 / 45 / 64 -> 26 / 39 / 58 and 157 / 277 / 599 -> 134 / 264 / 593 us;
-    // blocks along the diagonal, 10 M: 111 / 200 / 380 -> 101 / 194 / 375) and costs elsewhere, although
+    // nonzeros, K = 32 / 64 / 128: 20 / 36 / 64 -> 15 / 29 / 58 and 147 / 269 / 602 -> 124 / 253 / 592 us;
+    // blocks along the diagonal, 10 M: 98 / 182 / 382 -> 86 / 170 / 378) and costs elsewhere, although
     // the ranges are cut by estimated work (the tiles lie sorted by the length class of their rows):
-    // citation graph x 16 and x 64: 46 / 82 / 154 -> 48 / 94 / 172 and 171 / 341 / 690 -> 219 / 422 / 743;
-    // R-MAT at 3.7 and 7.6 M nonzeros +1 to +12 %; preferential attachment, co-purchase graph, users x
-    // items +1 to +3 %; the mesh at 102 M +0 to +3 %; uniform rows, the social graph and the 20k-vertex
-    // citation graph +-1 %.
+    // citation graph x 16 and x 64: 39 / 78 / 155 -> 46 / 90 / 172 and 168 / 338 / 697 -> 224 / 409 / 747;
+    // R-MAT at 3.7 and 7.6 M nonzeros +0 to +10 %; preferential attachment and the co-purchase graph
+    // +2 to +6 %; the mesh at 102 M +1 to +5 %; the 20k-vertex citation graph +1 to +10 %; uniform
+    // rows, users x items, the social graph +-1 %.
     p->rt_ranges = opt.row_tiles_ranges > 0;
   }
   if (p->d_tent && !fast_k(k)) {

@@ -251,21 +251,46 @@ __device__ __forceinline__ int column_tiles(uint32_t ldc) {
 // [start[r], start[r + 1]), of about equal work (the tiles lie sorted by the length class of their
 // rows: equal counts would not be equal work).  A workgroup beyond the end of its range gets group
 // n_groups, which has no work.
+// The kernels that deal ranges are instantiations of their own (kRanges): the others take an empty
+// argument in its place - the 13 words alone cost a launch of microseconds 0.2 us.
 struct TileRanges {
-  int32_t long_groups, long_per, per_range, n_groups;  // per_range = the longest range (0: no ranges)
+  int32_t long_groups, long_per, per_range, n_groups;  // per_range = the longest range
   int32_t start[kXcds + 1];
 };
+struct NoTileRanges {};
+template <bool kRanges>
+using TileRangesArg = typename std::conditional<kRanges, TileRanges, NoTileRanges>::type;
+template <int kLd>
+__device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, const NoTileRanges&, int& tile,
+                                                  int32_t& group);
 template <int kLd>
 __device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, const TileRanges& tr, int& tile,
                                                   int32_t& group) {
-  if (kLd == 0 && tr.per_range > 0) {
+  if (kLd == 0) {
     const uint32_t xcd = b % (uint32_t)kXcds, j = b / (uint32_t)kXcds;
     const uint32_t ranges = (uint32_t)kXcds / (uint32_t)T, r = xcd / (uint32_t)T;
     tile = (int)(xcd % (uint32_t)T);
-    const uint32_t g = j < (uint32_t)tr.long_per ? j * ranges + r : (uint32_t)tr.start[r] + (j - (uint32_t)tr.long_per);
-    const bool idle = j < (uint32_t)tr.long_per ? g >= (uint32_t)tr.long_groups : g >= (uint32_t)tr.start[r + 1];
+    // (start[r] by selects over constant indices: an index known only at run time would move the
+    // argument block into LDS and lengthen the start of every wavefront - 3.4 -> 16 us on a 100k-nonzero matrix)
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int i = 0; i < kXcds; ++i) {
+      if ((uint32_t)i == r) {
+        lo = (uint32_t)tr.start[i];
+        hi = (uint32_t)tr.start[i + 1];
+      }
+    }
+    const uint32_t g = j < (uint32_t)tr.long_per ? j * ranges + r : lo + (j - (uint32_t)tr.long_per);
+    const bool idle = j < (uint32_t)tr.long_per ? g >= (uint32_t)tr.long_groups : g >= hi;
     group = idle ? tr.n_groups : (int32_t)g;
-  } else if (kLd != 0 && same_xcd) {
+  } else {
+    tile_of_workgroup<kLd>(b, T, same_xcd, NoTileRanges{}, tile, group);
+  }
+}
+template <int kLd>
+__device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, const NoTileRanges&, int& tile,
+                                                  int32_t& group) {
+  if (kLd != 0 && same_xcd) {
     const uint32_t per = (uint32_t)kXcds * (uint32_t)T, r = b % per;
     tile = (int)(r / (uint32_t)kXcds);
     group = (int32_t)((b / per) * (uint32_t)kXcds + r % (uint32_t)kXcds);
@@ -400,14 +425,14 @@ __device__ __forceinline__ void reduce_and_store(float4 acc, int lg, int32_t row
 
 // Wavefront w < n_loop works through the tiles of long row w (ldesc[w] = first
 // tile, tile count); wavefront w >= n_loop owns tile loop_tiles + (w - n_loop).
-template <int K, int WPB, int kLd = 0, int kSub = kSlot>
+template <int K, int WPB, int kLd = 0, int kSub = kSlot, bool kRanges = false>
 __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves, int32_t n_loop, int32_t loop_tiles,
                                                                const int2* __restrict__ ldesc,
                                                                const int2* __restrict__ tent,
                                                                const float* __restrict__ val,
                                                                const float* __restrict__ B, float* __restrict__ C,
                                                                const float* __restrict__ zrow, uint32_t ldb,
-                                                               uint32_t ldc, bool same_xcd, TileRanges ranges) {
+                                                               uint32_t ldc, bool same_xcd, TileRangesArg<kRanges> ranges) {
   const int T = column_tiles<K, kLd>(ldc);
   __shared__ int32_t s_col[WPB * 64];
   __shared__ int32_t s_x[WPB * 64];
@@ -444,7 +469,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
 // shares, the shares' sums added in wavefront order through LDS), for matrices whose longest rows
 // would otherwise be the critical path of the launch.  The wavefronts of the other workgroups take
 // one remaining long row or one ordinary tile each, as above.
-template <int K, int WPB, int kLd = 0, int kSub = kSlot>
+template <int K, int WPB, int kLd = 0, int kSub = kSlot, bool kRanges = false>
 __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_tiles, int32_t n_wg, int32_t n_loop,
                                                                     int32_t loop_tiles,
                                                                     const int2* __restrict__ ldesc,
@@ -454,7 +479,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
                                                                     float* __restrict__ C,
                                                                     const float* __restrict__ zrow,
                                                                     uint32_t ldb, uint32_t ldc, bool same_xcd,
-                                                                    TileRanges ranges) {
+                                                                    TileRangesArg<kRanges> ranges) {
   const int T = column_tiles<K, kLd>(ldc);
   __shared__ int32_t s_col[WPB * 64];
   __shared__ int32_t s_x[WPB * 64];

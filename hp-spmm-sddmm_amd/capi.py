@@ -127,7 +127,7 @@ class PlanOptions(ctypes.Structure):
         ("row_tiles_wide", ctypes.c_int32), ("row_tiles_round_robin", ctypes.c_int32),
         ("sweep_window_log2", ctypes.c_int32), ("sweep_lead", ctypes.c_int32), ("sweep_spin", ctypes.c_int32),
         ("sweep_limit", ctypes.c_int32), ("sweep_no_priorities", ctypes.c_int32), ("cluster_sweeps", ctypes.c_int32),
-        ("report", ctypes.c_int32), ("row_tiles_ranges", ctypes.c_int32),
+        ("report", ctypes.c_int32), ("row_tiles_chunk_log2", ctypes.c_int32),
     ]
 
     OPTION_NAMES = tuple(n for n, _ in _fields_[3:])

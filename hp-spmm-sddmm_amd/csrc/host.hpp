@@ -150,7 +150,7 @@ struct PlanOptions {
   int row_tiles_pad = -1;     // -1 auto, 0 never, 1 whenever the length is not a multiple of 32
   bool row_tiles_narrow = true;    // 4 / 1 lanes per entry at <= 16 / <= 4 columns
   bool row_tiles_same_xcd = true;
-  int row_tiles_ranges = -1;  // tuned row lengths: 1 = one contiguous range of the row tiles per XCD (-1, 0: not)
+  int row_tiles_chunk_log2 = 0;  // tuned row lengths: 2^n consecutive groups of row tiles to an XCD at a time (0: the plan decides, -1: one)
   int sweep_window_log2 = 0, sweep_lead = 0, sweep_limit = 0;  // 0 = default
   int sweep_spin = -1;        // -1 = default, else the limit (0 = never wait)
   int sweep_priorities = -1;  // -1 = default (on), 0 = off
@@ -239,8 +239,7 @@ struct hpspmm_plan {
   uint32_t rt_ldb = 0;
   int rt_sub = 8;            // lanes per entry of the row-tile kernels at such a row length: 8, 4 or 1
   bool rt_same_xcd = true;   // the column tiles of a group of row tiles on one XCD where rows of B share lines
-  bool rt_ranges = false;    // tuned row lengths: every XCD serves one contiguous range of the row tiles
-  int32_t rt_cut[9] = {};    // ... cut where: first ordinary tile of every eighth of the work (build_row_tiles)
+  int rt_chunk_log2 = 0;     // tuned row lengths: 2^n consecutive groups of row tiles to an XCD at a time (0: one, -1: by the size)
   // sweep strategy (its stream arrays are d_vcol = entry words, d_vsrc, d_vval when values are bound;
   // partial-result rows of split rows in d_partial; rows without nonzeros in d_zero_rows)
   hpspmm::SweepLayout sw{};

@@ -60,34 +60,26 @@ inline bool row_tiles_same_xcd(const hpspmm_plan* p, int kLd, uint32_t ldb) {
   return kLd != 0 && ldb % 32 != 0 && p->rt_same_xcd;
 }
 
-// Contiguous ranges of the groups of row tiles per XCD (tuned row lengths): how the groups are cut
-// and how many workgroups that takes.  `long_groups` = the groups at the front of the layout that
-// hold the long rows, which stay dealt round robin.
-hpspmm::TileRanges row_tile_ranges(const hpspmm_plan* p, int kLd, int64_t k_template, int64_t groups, int64_t long_groups,
-                                   int64_t wpb, int64_t n_wg, int64_t* blocks) {
-  hpspmm::TileRanges tr{};
-  tr.n_groups = (int32_t)groups;
-  if (kLd != 0 || !p->rt_ranges || k_template <= 0 || groups < 4 * hpspmm::kXcds) return tr;
-  const int64_t ranges = hpspmm::kXcds / (k_template / 32);
+// Chunks of consecutive groups of row tiles per XCD (tuned row lengths): how large, and how many
+// workgroups that takes.  `long_groups` = the groups at the front of the layout that hold the long
+// rows, which stay dealt one at a time.  chunk_log2 = 0 in the result: no chunks.
+hpspmm::TileChunks row_tile_chunks(const hpspmm_plan* p, int kLd, int64_t k_template, int64_t groups, int64_t long_groups,
+                                   int64_t* blocks) {
+  hpspmm::TileChunks tc{0, 0, (int32_t)groups, 0};
+  if (kLd != 0 || k_template <= 0 || p->rt_chunk_log2 == 0) return tc;
+  const int64_t ways = hpspmm::kXcds / (k_template / 32);
   long_groups = std::min(long_groups, groups);
-  tr.long_groups = (int32_t)long_groups;
-  tr.long_per = (int32_t)ceil_div(long_groups, ranges);
-  // the plan's cuts are in ordinary tiles (rt_cut[i] = first tile, counted from the first ordinary
-  // one, of the i-th eighth of the work); a group is `wpb` consecutive wavefronts, after the n_wg rows
-  // that get a workgroup each; the long rows come first
-  const int64_t step = hpspmm::kXcds / ranges;
-  int64_t longest = 1;
-  for (int64_t r = 0; r <= ranges; ++r) {
-    const int64_t wave = (int64_t)p->rt_loop + p->rt_cut[r * step];
-    const int64_t g = r == 0        ? long_groups
-                      : r == ranges ? groups
-                                    : std::min(groups, std::max(long_groups, n_wg + (wave - n_wg) / wpb));
-    tr.start[r] = (int32_t)std::max<int64_t>(g, r ? tr.start[r - 1] : 0);
-    if (r) longest = std::max<int64_t>(longest, tr.start[r] - tr.start[r - 1]);
-  }
-  tr.per_range = (int32_t)longest;
-  *blocks = (int64_t)hpspmm::kXcds * (tr.long_per + tr.per_range);
-  return tr;
+  // the plan's own choice (-1): the largest n <= 9 that leaves every XCD 16 chunks - one chunk more
+  // or less is then 6 % of its work at most
+  int n = p->rt_chunk_log2 > 0 ? p->rt_chunk_log2 : 9;
+  if (p->rt_chunk_log2 < 0)
+    while (n > 0 && groups - long_groups < (16 * ways << n)) --n;
+  if (n <= 0 || groups - long_groups < (2 * ways << n)) return tc;
+  tc.chunk_log2 = n;
+  tc.long_groups = (int32_t)long_groups;
+  tc.long_per = (int32_t)ceil_div(long_groups, ways);
+  *blocks = (int64_t)hpspmm::kXcds * (tc.long_per + (ceil_div(groups - long_groups, ways << n) << n));
+  return tc;
 }
 
 template <int K, int WPB, int kLd, int kSub>
@@ -96,20 +88,20 @@ int launch_row_tiles_w(const hpspmm_plan* p, const float* v, const float* B, flo
   const bool same_xcd = row_tiles_same_xcd(p, kLd, ldb);
   const int64_t groups = ceil_div(p->rt_waves, WPB);
   int64_t blocks = (same_xcd ? ceil_div(groups, hpspmm::kXcds) * hpspmm::kXcds : groups) * row_tile_column_tiles(K, ldc);
-  const hpspmm::TileRanges ranges = row_tile_ranges(p, kLd, K, groups, ceil_div(p->rt_loop, WPB), WPB, 0, &blocks);
+  const hpspmm::TileChunks chunks = row_tile_chunks(p, kLd, K, groups, ceil_div(p->rt_loop, WPB), &blocks);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   if constexpr (kLd == 0) {
-    if (ranges.per_range > 0) {
+    if (chunks.chunk_log2 > 0) {
       hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB, kLd, kSub, true>), dim3((unsigned)blocks), dim3(WPB * 64), 0,
                          st, p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent, readable_values(p, v), B, C,
-                         p->d_zrow + 4, ldb, ldc, same_xcd, ranges);
+                         p->d_zrow + 4, ldb, ldc, same_xcd, chunks);
       mark_launch(st, "spmm_rowtiles_kernel");
       return HPSPMM_OK;
     }
   }
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_kernel<K, WPB, kLd, kSub>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_waves, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent, readable_values(p, v), B, C,
-                     p->d_zrow + 4, ldb, ldc, same_xcd, hpspmm::NoTileRanges{});
+                     p->d_zrow + 4, ldb, ldc, same_xcd, hpspmm::NoTileChunks{});
   mark_launch(st, "spmm_rowtiles_kernel");
   return HPSPMM_OK;
 }
@@ -121,21 +113,21 @@ int launch_row_tiles_wg(const hpspmm_plan* p, const float* v, const float* B, fl
   const bool same_xcd = row_tiles_same_xcd(p, kLd, ldb);
   const int64_t groups = p->rt_wg + ceil_div(wave_items, WPB);
   int64_t blocks = (same_xcd ? ceil_div(groups, hpspmm::kXcds) * hpspmm::kXcds : groups) * row_tile_column_tiles(K, ldc);
-  const hpspmm::TileRanges ranges =
-      row_tile_ranges(p, kLd, K, groups, p->rt_wg + ceil_div(p->rt_loop - p->rt_wg, WPB), WPB, p->rt_wg, &blocks);
+  const hpspmm::TileChunks chunks =
+      row_tile_chunks(p, kLd, K, groups, p->rt_wg + ceil_div(p->rt_loop - p->rt_wg, WPB), &blocks);
   if (blocks > INT32_MAX) return fail(HPSPMM_ERR_INVALID_ARG, "grid too large");
   if constexpr (kLd == 0) {
-    if (ranges.per_range > 0) {
+    if (chunks.chunk_log2 > 0) {
       hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB, kLd, kSub, true>), dim3((unsigned)blocks), dim3(WPB * 64),
                          0, st, p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent,
-                         readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc, same_xcd, ranges);
+                         readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc, same_xcd, chunks);
       mark_launch(st, "spmm_rowtiles_wg_kernel");
       return HPSPMM_OK;
     }
   }
   hipLaunchKernelGGL((hpspmm::spmm_rowtiles_wg_kernel<K, WPB, kLd, kSub>), dim3((unsigned)blocks), dim3(WPB * 64), 0, st,
                      p->rt_tiles, p->rt_wg, p->rt_loop, p->rt_loop_tiles, p->d_ldesc, p->d_tent,
-                     readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc, same_xcd, hpspmm::NoTileRanges{});
+                     readable_values(p, v), B, C, p->d_zrow + 4, ldb, ldc, same_xcd, hpspmm::NoTileChunks{});
   mark_launch(st, "spmm_rowtiles_wg_kernel");
   return HPSPMM_OK;
 }

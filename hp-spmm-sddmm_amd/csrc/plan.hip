@@ -68,6 +68,7 @@ constexpr int64_t kClusterMinBBytes = (int64_t)12 << 20;  // co-purchase graph, 
 // and once the ordered strategy has been tried.
 constexpr double kSweepSureGain = 0.7, kSweepMinGain = 0.9;
 constexpr int64_t kOtherLayoutsMinNnz = (int64_t)1 << 21;  // below: whole rows without looking further
+constexpr int64_t kRowTileChunksMinNnz = (int64_t)1 << 21;  // row tiles dealt to the XCDs in chunks from here up
 // A matrix whose stored order is local already has its communities side by side; another order pays
 // only where B is far beyond every cache (blocks of 8 to 4096 vertices along the diagonal with 10 % of
 // the entries elsewhere, K = 32 / 64 / 128: at 10 M nonzeros (B = 38 / 77 / 154 MB) ordered 109 / 193 /
@@ -421,16 +422,20 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
     }
   }
   if (p->d_tent && fast_k(k)) {
-    // Every XCD one contiguous range of the row tiles instead of every eighth group: only on request.
-    // It pays where neighbouring rows share columns (mesh with 2 random entries per row, 1.5 / 12 M
-    // nonzeros, K = 32 / 64 / 128: 20 / 36 / 64 -> 15 / 29 / 58 and 147 / 269 / 602 -> 124 / 253 / 592 us;
-    // blocks along the diagonal, 10 M: 98 / 182 / 382 -> 86 / 170 / 378) and costs elsewhere, although
-    // the ranges are cut by estimated work (the tiles lie sorted by the length class of their rows):
-    // citation graph x 16 and x 64: 39 / 78 / 155 -> 46 / 90 / 172 and 168 / 338 / 697 -> 224 / 409 / 747;
-    // R-MAT at 3.7 and 7.6 M nonzeros +0 to +10 %; preferential attachment and the co-purchase graph
-    // +2 to +6 %; the mesh at 102 M +1 to +5 %; the 20k-vertex citation graph +1 to +10 %; uniform
-    // rows, users x items, the social graph +-1 %.
-    p->rt_ranges = opt.row_tiles_ranges > 0;
+    // 2^n consecutive groups of row tiles to an XCD at a time instead of one (n by the size, at the
+    // launch): rows that share columns with their neighbours then share an L2.  Mesh with 2 random
+    // entries per row, 1.5 / 12 M nonzeros, K = 32 / 64 / 128: 20 / 36 / 64 -> 17 / 31 / 59 and 148 / 268 /
+    // 600 -> 127 / 253 / 589 us; blocks along the diagonal, 10 M: 98 / 178 / 377 -> 86 / 169 / 373; 85 M:
+    // -1 to -2 %.  Matrices without such an order pay up to 3 % (R-MAT at 0.9 to 7.6 M nonzeros +2 to
+    // +3 %, users x items +1 to +2 %, the mesh at 102 M +0 to +2 %, the others +-1 %), a launch of
+    // microseconds more (the 20k-vertex citation graph +2 to +5 %): from 2^21 nonzeros only.
+    // (One contiguous range of the tiles per XCD does the same for the mesh, -14 to -24 %, but costs
+    // the others up to 30 %: the tiles lie sorted by the length class of their rows, so the ranges
+    // are not equally heavy, also when cut by estimated work.)
+    p->rt_chunk_log2 = opt.row_tiles_chunk_log2 > 0   ? opt.row_tiles_chunk_log2
+                       : opt.row_tiles_chunk_log2 < 0 ? 0
+                       : nnz >= kRowTileChunksMinNnz  ? -1
+                                                      : 0;
   }
   if (p->d_tent && !fast_k(k)) {
     // Row tiles at a row length of its own.  The gathers are fastest when every 32-column tile of a
@@ -592,8 +597,9 @@ HPSPMM_API int hpspmm_plan_create_ex(int64_t rows, int64_t cols, int64_t nnz, co
   o.sweep_priorities = in.sweep_no_priorities ? 0 : -1;
   o.cluster_sweeps = std::max(0, in.cluster_sweeps);
   o.report = in.report != 0;
-  if (in.row_tiles_ranges < 0 || in.row_tiles_ranges > 2) return fail(HPSPMM_ERR_INVALID_ARG, "row_tiles_ranges must be 0, 1 or 2");
-  o.row_tiles_ranges = in.row_tiles_ranges == 0 ? -1 : in.row_tiles_ranges == 1 ? 0 : 1;
+  if (in.row_tiles_chunk_log2 < -1 || in.row_tiles_chunk_log2 > 16)
+    return fail(HPSPMM_ERR_INVALID_ARG, "row_tiles_chunk_log2 must be -1 .. 16");
+  o.row_tiles_chunk_log2 = in.row_tiles_chunk_log2;
   return plan_create_guarded(rows, cols, nnz, d_rowptr, d_col, k, o, stream, plan_out);
 }
 

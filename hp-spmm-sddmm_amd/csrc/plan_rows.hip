@@ -115,39 +115,6 @@ int build_row_tiles(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_co
   p->rt_wg = (int32_t)cnt[0];
   p->rt_loop_tiles = (int32_t)lay.loop_tiles;
   p->rt_waves = (int32_t)(n_loop + (tiles - lay.loop_tiles));
-  // Eighths of equal work over the ordinary tiles (for the dealing of contiguous ranges to the XCDs):
-  // a full tile of rows of 9 to 64 nonzeros weighs 1, a tile of one-slot rows a fixed part plus its
-  // depth, the length of its longest row, which is its first (the rows lie sorted by length there).
-  {
-    const int64_t ordinary = tiles - lay.loop_tiles;
-    std::vector<std::pair<int64_t, double>> pieces;  // consecutive tiles of one weight: (how many, weight each)
-    pieces.push_back({t3 + t2 + t1, 1.0});
-    int64_t rows_before = 0, tiles_before = 0;
-    for (int n = hpspmm::kSlot; n >= 0; --n) {  // one-slot tiles whose first row has n nonzeros
-      rows_before += cnt[5 + (hpspmm::kSlot - n)];
-      const int64_t upto = std::min(t0, ceil_div(rows_before, 8));
-      if (upto > tiles_before) pieces.push_back({upto - tiles_before, 0.35 + 0.65 * n / 8.0});
-      tiles_before = std::max(tiles_before, upto);
-    }
-    double total = 0;
-    for (const auto& pc : pieces) total += (double)pc.first * pc.second;
-    for (int i = 0; i <= 8; ++i) {
-      const double want = total * i / 8.0;
-      double acc = 0;
-      int64_t before = 0, cut = ordinary;
-      for (const auto& pc : pieces) {
-        const double all = (double)pc.first * pc.second;
-        if (acc + all >= want) {
-          cut = before + std::min<int64_t>(pc.first, (int64_t)((want - acc) / pc.second));
-          break;
-        }
-        acc += all;
-        before += pc.first;
-      }
-      p->rt_cut[i] = (int32_t)std::min(cut, ordinary);
-    }
-    p->rt_cut[8] = (int32_t)ordinary;
-  }
   return HPSPMM_OK;
 }
 

@@ -243,52 +243,38 @@ __device__ __forceinline__ int column_tiles(uint32_t ldc) {
 // the other - for rows of B that are not a whole number of 128-byte lines: the line that two
 // neighbouring tiles share is then fetched into one L2 once instead of into two.
 //
-// ranges (tuned row lengths; per_range > 0): every XCD serves one column tile and one contiguous
-// range of the groups instead of every (8 / T)-th group, so that rows that share columns with their
-// neighbours (a mesh, a banded matrix, blocks along the diagonal) meet them in one L2 instead of
-// eight.  The first long_groups groups (the long rows, which come first in the layout) stay dealt
-// round robin - they are the heaviest -, the others are cut into 8 / T ranges, range r = groups
-// [start[r], start[r + 1]), of about equal work (the tiles lie sorted by the length class of their
-// rows: equal counts would not be equal work).  A workgroup beyond the end of its range gets group
-// n_groups, which has no work.
-// The kernels that deal ranges are instantiations of their own (kRanges): the others take an empty
-// argument in its place - the 13 words alone cost a launch of microseconds 0.2 us.
-struct TileRanges {
-  int32_t long_groups, long_per, per_range, n_groups;  // per_range = the longest range
-  int32_t start[kXcds + 1];
+// chunks (tuned row lengths): the groups are dealt round robin all the same, but 2^chunk_log2
+// consecutive groups at a time.  All XCDs still work on the same stretch of the layout (the tiles lie
+// sorted by the length class of their rows: no XCD gets the heavier ones), and rows up to a chunk
+// apart share an L2 - what a mesh, a banded matrix or blocks along the diagonal need for the rows of
+// B that neighbouring rows have in common to be fetched into one L2 instead of eight.  The groups of
+// the long rows, the first long_groups of the layout, stay dealt one at a time: they are the heaviest.
+// A workgroup beyond the end gets group n_groups, which has no work.  The kernels that deal chunks
+// are instantiations of their own (kChunks): the others take an empty argument in its place - a few
+// more argument words alone cost a launch of microseconds 0.2 us.
+struct TileChunks {
+  int32_t long_groups, long_per, n_groups, chunk_log2;
 };
-struct NoTileRanges {};
-template <bool kRanges>
-using TileRangesArg = typename std::conditional<kRanges, TileRanges, NoTileRanges>::type;
+struct NoTileChunks {};
+template <bool kChunks>
+using TileChunksArg = typename std::conditional<kChunks, TileChunks, NoTileChunks>::type;
 template <int kLd>
-__device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, const NoTileRanges&, int& tile,
+__device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, const NoTileChunks&, int& tile,
                                                   int32_t& group);
 template <int kLd>
-__device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, const TileRanges& tr, int& tile,
-                                                  int32_t& group) {
-  if (kLd == 0) {
-    const uint32_t xcd = b % (uint32_t)kXcds, j = b / (uint32_t)kXcds;
-    const uint32_t ranges = (uint32_t)kXcds / (uint32_t)T, r = xcd / (uint32_t)T;
-    tile = (int)(xcd % (uint32_t)T);
-    // (start[r] by selects over constant indices: an index known only at run time would move the
-    // argument block into LDS and lengthen the start of every wavefront - 3.4 -> 16 us on a 100k-nonzero matrix)
-    uint32_t lo = 0, hi = 0;
-#pragma unroll
-    for (int i = 0; i < kXcds; ++i) {
-      if ((uint32_t)i == r) {
-        lo = (uint32_t)tr.start[i];
-        hi = (uint32_t)tr.start[i + 1];
-      }
-    }
-    const uint32_t g = j < (uint32_t)tr.long_per ? j * ranges + r : lo + (j - (uint32_t)tr.long_per);
-    const bool idle = j < (uint32_t)tr.long_per ? g >= (uint32_t)tr.long_groups : g >= hi;
-    group = idle ? tr.n_groups : (int32_t)g;
-  } else {
-    tile_of_workgroup<kLd>(b, T, same_xcd, NoTileRanges{}, tile, group);
-  }
+__device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool, const TileChunks& tc, int& tile, int32_t& group) {
+  static_assert(kLd == 0, "chunks are dealt at the tuned row lengths only");
+  const uint32_t xcd = b % (uint32_t)kXcds, j = b / (uint32_t)kXcds;
+  const uint32_t ways = (uint32_t)kXcds / (uint32_t)T, r = xcd / (uint32_t)T, L = (uint32_t)tc.chunk_log2;
+  tile = (int)(xcd % (uint32_t)T);
+  const uint32_t i = j - (uint32_t)tc.long_per;
+  const uint32_t g = j < (uint32_t)tc.long_per ? j * ways + r
+                                               : (uint32_t)tc.long_groups + (((i >> L) * ways + r) << L) + (i & ((1u << L) - 1u));
+  const bool idle = j < (uint32_t)tc.long_per ? g >= (uint32_t)tc.long_groups : g >= (uint32_t)tc.n_groups;
+  group = idle ? tc.n_groups : (int32_t)g;
 }
 template <int kLd>
-__device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, const NoTileRanges&, int& tile,
+__device__ __forceinline__ void tile_of_workgroup(uint32_t b, int T, bool same_xcd, const NoTileChunks&, int& tile,
                                                   int32_t& group) {
   if (kLd != 0 && same_xcd) {
     const uint32_t per = (uint32_t)kXcds * (uint32_t)T, r = b % per;
@@ -425,14 +411,14 @@ __device__ __forceinline__ void reduce_and_store(float4 acc, int lg, int32_t row
 
 // Wavefront w < n_loop works through the tiles of long row w (ldesc[w] = first
 // tile, tile count); wavefront w >= n_loop owns tile loop_tiles + (w - n_loop).
-template <int K, int WPB, int kLd = 0, int kSub = kSlot, bool kRanges = false>
+template <int K, int WPB, int kLd = 0, int kSub = kSlot, bool kChunks = false>
 __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves, int32_t n_loop, int32_t loop_tiles,
                                                                const int2* __restrict__ ldesc,
                                                                const int2* __restrict__ tent,
                                                                const float* __restrict__ val,
                                                                const float* __restrict__ B, float* __restrict__ C,
                                                                const float* __restrict__ zrow, uint32_t ldb,
-                                                               uint32_t ldc, bool same_xcd, TileRangesArg<kRanges> ranges) {
+                                                               uint32_t ldc, bool same_xcd, TileChunksArg<kChunks> chunks) {
   const int T = column_tiles<K, kLd>(ldc);
   __shared__ int32_t s_col[WPB * 64];
   __shared__ int32_t s_x[WPB * 64];
@@ -445,7 +431,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
   const int base = tid - l;
   int ctile;
   int32_t group;
-  tile_of_workgroup<kLd>(blockIdx.x, T, same_xcd, ranges, ctile, group);
+  tile_of_workgroup<kLd>(blockIdx.x, T, same_xcd, chunks, ctile, group);
   const TileColumns tc = tile_columns<K, kLd, kSub>(ldb, ldc, ctile, l);
   const int32_t w = __builtin_amdgcn_readfirstlane(group * WPB + (tid >> 6));
   if (w >= n_waves) return;
@@ -469,7 +455,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_kernel(int32_t n_waves
 // shares, the shares' sums added in wavefront order through LDS), for matrices whose longest rows
 // would otherwise be the critical path of the launch.  The wavefronts of the other workgroups take
 // one remaining long row or one ordinary tile each, as above.
-template <int K, int WPB, int kLd = 0, int kSub = kSlot, bool kRanges = false>
+template <int K, int WPB, int kLd = 0, int kSub = kSlot, bool kChunks = false>
 __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_tiles, int32_t n_wg, int32_t n_loop,
                                                                     int32_t loop_tiles,
                                                                     const int2* __restrict__ ldesc,
@@ -479,7 +465,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
                                                                     float* __restrict__ C,
                                                                     const float* __restrict__ zrow,
                                                                     uint32_t ldb, uint32_t ldc, bool same_xcd,
-                                                                    TileRangesArg<kRanges> ranges) {
+                                                                    TileChunksArg<kChunks> chunks) {
   const int T = column_tiles<K, kLd>(ldc);
   __shared__ int32_t s_col[WPB * 64];
   __shared__ int32_t s_x[WPB * 64];
@@ -494,7 +480,7 @@ __global__ __launch_bounds__(WPB * 64) void spmm_rowtiles_wg_kernel(int32_t n_ti
   const int base = tid - l;
   int ctile;
   int32_t blk;
-  tile_of_workgroup<kLd>(blockIdx.x, T, same_xcd, ranges, ctile, blk);
+  tile_of_workgroup<kLd>(blockIdx.x, T, same_xcd, chunks, ctile, blk);
   const TileColumns tc = tile_columns<K, kLd, kSub>(ldb, ldc, ctile, l);
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 

@@ -86,7 +86,7 @@ bool set_spmm_plan_option(const std::string& field, long value) {
       HPSPMM_OPTION(row_tiles_min_k), HPSPMM_OPTION(row_tiles_pad), HPSPMM_OPTION(row_tiles_wide),
       HPSPMM_OPTION(row_tiles_round_robin), HPSPMM_OPTION(sweep_window_log2), HPSPMM_OPTION(sweep_lead),
       HPSPMM_OPTION(sweep_spin), HPSPMM_OPTION(sweep_limit), HPSPMM_OPTION(sweep_no_priorities),
-      HPSPMM_OPTION(cluster_sweeps), HPSPMM_OPTION(report), HPSPMM_OPTION(row_tiles_ranges)};
+      HPSPMM_OPTION(cluster_sweeps), HPSPMM_OPTION(report), HPSPMM_OPTION(row_tiles_chunk_log2)};
 #undef HPSPMM_OPTION
   for (const Field& f : fields) {
     if (field != f.name) continue;

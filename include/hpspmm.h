@@ -138,8 +138,8 @@ typedef struct hpspmm_plan_options {
   int32_t sweep_no_priorities; /* 1: leave the wavefront priorities alone */
   int32_t cluster_sweeps;     /* label-propagation sweeps, at most */
   int32_t report;             /* 1: plan-time reports on stderr */
-  int32_t row_tiles_ranges;   /* row tiles at k = 32 / 64 / 128: 2 = give every XCD one contiguous range of the row
-                                 tiles instead of every eighth group of them (0, 1: not) */
+  int32_t row_tiles_chunk_log2; /* row tiles at k = 32 / 64 / 128: deal 2^n consecutive groups of tiles to an XCD at a
+                                 time instead of one (-1 = one; 0 = the library's choice, by the size) */
 } hpspmm_plan_options;
 
 typedef struct hpspmm_plan_info {

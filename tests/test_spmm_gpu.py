@@ -920,8 +920,8 @@ def test_row_tiles_layout_and_fallback(pkg, oracle, gpu):
         C2, info2 = _run(pkg, gpu, g, B, capi.PLAN_NO_ROW_TILES)
         assert info2["strategy"] == capi.STRATEGY_ROWS and info2["row_tiles"] == 0
         _check(oracle, g, B, C2, f"all row lengths k={k} csr")
-        # every XCD one contiguous range of the tiles instead of every eighth group: the same tiles, the same bits
-        Cr, info_r = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT, options={"row_tiles_ranges": 2})
+        # the groups of tiles dealt to the XCDs four at a time instead of one: the same tiles, the same bits
+        Cr, info_r = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT, options={"row_tiles_chunk_log2": 2})
         assert info_r["row_tiles"] == info["row_tiles"] and np.array_equal(C, Cr)
     # rows beyond 512 nonzeros get a workgroup each (8 wavefronts; 16 when a row exceeds 8192),
     # next to rows of 65..512 that one wavefront works through
@@ -940,8 +940,8 @@ def test_row_tiles_layout_and_fallback(pkg, oracle, gpu):
             _check(oracle, g, B, C, f"long rows up to {longest} k={k}")
             again, _ = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
             assert np.array_equal(C, again), "workgroup-per-row reduction must be bit-reproducible"
-            Cr, _ = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT, options={"row_tiles_ranges": 2})
-            assert np.array_equal(C, Cr), "tile ranges per XCD must not change the result"
+            Cr, _ = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT, options={"row_tiles_chunk_log2": 1})
+            assert np.array_equal(C, Cr), "dealing the tiles in chunks must not change the result"
     # 400k rows, 2k nonzeros: 50k tiles of padding for 2k entries - not built
     rows = 400_000
     lens = np.zeros(rows, np.int64)
@@ -956,20 +956,24 @@ def test_row_tiles_layout_and_fallback(pkg, oracle, gpu):
     _check(oracle, g, B, C, "mostly empty rows")
 
 
-@pytest.mark.parametrize("name,scale", [("h3_grid", 0.015), ("c4_rmat", 0.032), ("c1_citation", 4.0)])
-def test_row_tile_ranges_per_xcd(pkg, oracle, gpu, name, scale):
-    """hpspmm_plan_options.row_tiles_ranges = 2: every XCD serves one contiguous range of the row tiles
-    (long rows still dealt round robin).  Thousands of tiles, every class of row, the long rows of an
-    R-MAT graph on workgroups of their own: the oracle bar and the bits of the default dealing."""
+@pytest.mark.parametrize("name,scale", [("h3_grid", 0.03), ("c4_rmat", 0.1), ("c1_citation", 4.0)])
+def test_row_tile_chunks_per_xcd(pkg, oracle, gpu, name, scale):
+    """hpspmm_plan_options.row_tiles_chunk_log2: 2^n consecutive groups of row tiles go to an XCD at a
+    time (the groups of the long rows still one by one); from 2^21 nonzeros that is the default, with n
+    picked by the size.  Thousands of tiles, every class of row, the long rows of an R-MAT graph on
+    workgroups of their own, chunks of 2 to 512 groups: the oracle bar and the bits of the dealing
+    one by one."""
     capi = pkg.capi
     g = pkg.graphs.make_graph(name, scale)
     for k in (32, 64, 128):
         B = pkg.graphs.make_dense(name, g.cols, k)
-        C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_ROWS)
-        Cr, info_r = _run(pkg, gpu, g, B, capi.PLAN_FORCE_ROWS, options={"row_tiles_ranges": 2})
-        assert info_r["strategy"] == capi.STRATEGY_ROWS and info_r["row_tiles"] == info["row_tiles"] > 1000
-        _check(oracle, g, B, Cr, f"{name} k={k} tile ranges")
-        assert np.array_equal(C, Cr)
+        C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_ROWS, options={"row_tiles_chunk_log2": -1})
+        assert info["strategy"] == capi.STRATEGY_ROWS and info["row_tiles"] > 1000
+        _check(oracle, g, B, C, f"{name} k={k} one by one")
+        for n in (0, 1, 5, 9):
+            Cr, info_r = _run(pkg, gpu, g, B, capi.PLAN_FORCE_ROWS, options={"row_tiles_chunk_log2": n})
+            assert info_r["row_tiles"] == info["row_tiles"]
+            assert np.array_equal(C, Cr), f"{name} k={k} chunks of 2^{n}"
 
 
 @pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 7, 20, 31, 33, 36, 41, 63, 65, 100, 130, 172, 259])

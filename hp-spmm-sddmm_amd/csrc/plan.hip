@@ -310,15 +310,15 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
     }
     if (opt.report && rows_us > 0)
       fprintf(stderr, "plan: %.3f of the gathers miss in stored order, whole rows expected to take %.1f us\n", miss, rows_us);
-    // A matrix whose stored order is local (banded, a mesh, blocks along the diagonal) is served best
-    // by whole rows at any size: the gathers of neighbouring rows meet in the L2, and nothing is left
-    // for the other layouts to gain (9-point mesh with 2 random entries per row, 102 M nonzeros,
-    // K = 32 / 64 / 128: 1.27 / 2.58 / 5.75 ms against 1.81 / 3.31 / 6.44 for segments).
     const bool short_rows = mean_row <= kRowsAutoLongMean;
-    const bool local = fast_k(k) && miss <= kLocalMissShare && short_rows && nnz < kRowTileMaxNnz;
-    const bool mid = (in_range || local) && p->max_row_nnz <= longest_ok && !(flags & HPSPMM_PLAN_NO_ROW_TILES);
+    const bool mid = in_range && p->max_row_nnz <= longest_ok && !(flags & HPSPMM_PLAN_NO_ROW_TILES);
     // Beyond that range, when none of the other layouts qualifies, the choice is between whole rows
-    // and segments.  Row tiles are taken in stored order by all the CUs side by side, so that rows
+    // and segments.  A matrix whose stored order is local (banded, a mesh, blocks along the diagonal)
+    // is served best by whole rows at any size (9-point mesh with 2 random entries per row, 102 M
+    // nonzeros, K = 32 / 64 / 128: 1.27 / 2.58 / 5.75 ms against 1.81 / 3.31 / 6.44 for segments); a few
+    // missing gathers alone do not say that, though (R-MAT at 7.6 M nonzeros: 0.21 of them miss, for the
+    // popularity of its columns, and the routed strategy is 10 % ahead of whole rows at K = 128), so
+    // the other layouts are tried first.  Row tiles are taken in stored order by all the CUs side by side, so that rows
     // that share columns with their neighbours meet them in the L2; segments are long runs of
     // nonzeros far apart from each other, which gain nothing from that order, but read the sparse
     // matrix once instead of once per 32 columns.  Measured (rows against segments, K = 32 / 64 / 128):

@@ -18,8 +18,8 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 TOL = 1e-5           # |C - C64| <= TOL * (|A| |B|), the bar of every other parity test
 # The default plan against the fastest forced strategy.  The committed table has the default within
-# 10 % on every line of 12 M and 100 M nonzeros but one (blocks along the diagonal at 10 M, K = 32: 12 %)
-# and within 6 us on the lines of 1.5 M; the bound here is a guard against a wrong choice (those cost
+# 10 % on every line of 12 M and 100 M nonzeros and within 6 us on the lines of 1.5 M; the bound here
+# is a guard against a wrong choice (those cost
 # 25 to 90 %), with room for the 2-3 % that two timings of one plan differ by on top of that line.
 MAX_GAP = 0.20
 MAX_GAP_US = 8.0

@@ -16,7 +16,7 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-TOL = 1e-5           # |C - C64| <= TOL * (|A| |B|), the bar of every other parity test
+TOL = 1e-5           # |C - C64| <= TOL * (|A| |B|): ten times tighter than the bar of the other parity tests (1e-4)
 # The default plan against the fastest forced strategy: within 10 % (the committed table has it within
 # 7.5 % on every line of 12 M nonzeros), plus the 2 % that two timings of one plan differ by; on the
 # matrices of 1.5 M nonzeros, where an SpMM takes 12 to 60 us, within 8 us (largest in the table: 5.5).

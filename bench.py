@@ -425,9 +425,11 @@ def main():
                 wall = (time.perf_counter() - w0) * 1e3 / launches_issued
                 if ms_ < SHORT_SPMM_MS:
                     # an SpMM of microseconds: the median of five such regions (one region still moves
-                    # by 10-15 % with whatever the clocks were doing when it began)
-                    regions = [ms_]
-                    for _ in range(4):
+                    # by 10-15 % with whatever the clocks were doing when it began), the first one not
+                    # among them: the `warmup` launches before it are a fraction of a millisecond, and
+                    # the GPU has been idle while the host made the plan and the operands
+                    regions = []
+                    for _ in range(5):
                         m_, reps = capi.csr_spmm_timed_min(plan, d_rp, d_ci, d_v, d_B, d_C, warmup=0, iters=steps,
                                                            min_total_ms=MIN_TIMED_MS, stream=stream)
                         regions.append(m_)

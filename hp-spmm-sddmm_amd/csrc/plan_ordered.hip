@@ -129,9 +129,10 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
     hipLaunchKernelGGL(hpspmm::ordered_action_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr,
                        p->d_ostart, shift, d_action);
     hipError_t e2 = hipMemsetAsync(d_counts, 0, 2 * sizeof(int32_t), st);
-    hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_action,
+    const unsigned collect_grid = (unsigned)ceil_div(std::max<int64_t>(rows, 1), hpspmm::kCollectRows);
+    hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(collect_grid), dim3(hpspmm::kBlock), 0, st, rows, d_action,
                        hpspmm::kActionCross, p->d_cross_rows, d_counts);
-    hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_action,
+    hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(collect_grid), dim3(hpspmm::kBlock), 0, st, rows, d_action,
                        hpspmm::kActionZero, p->d_zero_rows, d_counts + 1);
     int32_t counts[2] = {0, 0};
     if (e2 == hipSuccess) e2 = hipMemcpyAsync(counts, d_counts, sizeof counts, hipMemcpyDeviceToHost, st);

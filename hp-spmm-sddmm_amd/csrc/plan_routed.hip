@@ -335,7 +335,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
     hipLaunchKernelGGL(hpspmm::routed_chunk_kernel, dim3((unsigned)nchunks), dim3(hpspmm::kBlock), 0, st, lay, nnz,
                        d_vpos, p->d_lslot, p->d_chunk_base, p->d_chunk_pref);
   // compact lists of the short rows the final kernel has to visit
-  const unsigned cgrid = (unsigned)ceil_div(rows, hpspmm::kBlock);
+  const unsigned cgrid = (unsigned)ceil_div(std::max<int64_t>(rows, 1), hpspmm::kCollectRows);
   hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(cgrid), dim3(hpspmm::kBlock), 0, st, rows, d_action,
                      hpspmm::kActionCross, p->d_cross_rows, d_counts);
   hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(cgrid), dim3(hpspmm::kBlock), 0, st, rows, d_action,

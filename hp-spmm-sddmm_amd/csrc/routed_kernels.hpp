@@ -478,18 +478,28 @@ constexpr size_t routed_tiles_lds_bytes(int lds_rows) {
 }
 
 // list[] <- every row whose action byte equals `which` (order unspecified); *count must be zero on entry.
+// A workgroup looks at kCollectRows consecutive rows, 8 per thread, and reserves its part of the list with
+// one atomic (one per wavefront of 64 rows took 0.44 ms over 2.4 M rows: 38k atomics on one address).
+constexpr int kCollectPerThread = 8;
+constexpr int kCollectRows = kBlock * kCollectPerThread;
 HPSPMM_KERNEL __launch_bounds__(kBlock) void routed_collect_rows_kernel(int64_t rows, const uint8_t* __restrict__ action,
                                                                      uint8_t which, int32_t* __restrict__ list,
                                                                      int32_t* __restrict__ count) {
-  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const bool hit = i < rows && action[i] == which;
-  const uint64_t mask = __ballot(hit);
-  if (mask == 0) return;
-  const int lane = threadIdx.x & 63;
-  int32_t base = 0;
-  if (lane == 0) base = atomicAdd(count, (int32_t)__popcll(mask));
-  base = __shfl(base, 0);
-  if (hit) list[base + __popcll(mask & ((1ull << lane) - 1ull))] = (int32_t)i;
+  __shared__ uint32_t s_wave[kWavesPerBlock];
+  __shared__ int32_t s_base;
+  const int64_t first = (int64_t)blockIdx.x * kCollectRows + (int64_t)threadIdx.x * kCollectPerThread;
+  uint32_t hits = 0;  // bit j: row first + j is wanted
+#pragma unroll
+  for (int j = 0; j < kCollectPerThread; ++j)
+    if (first + j < rows && action[first + j] == which) hits |= 1u << j;
+  uint32_t total;
+  const uint32_t before = block_exclusive_scan((uint32_t)__popc(hits), s_wave, total);
+  if (threadIdx.x == 0) s_base = total ? atomicAdd(count, (int32_t)total) : 0;
+  __syncthreads();
+  int32_t at = s_base + (int32_t)before;
+#pragma unroll
+  for (int j = 0; j < kCollectPerThread; ++j)
+    if (hits & (1u << j)) list[at++] = (int32_t)(first + j);
 }
 
 // Final pass, one sub-wave per listed row, three parts.

@@ -84,8 +84,9 @@ typedef enum hpspmm_status {
 #define HPSPMM_PLAN_NO_ROW_TILES 16384u /* rows strategy: walk the caller's CSR arrays instead of building row tiles */
 #define HPSPMM_PLAN_FORCE_SWEEP (1u << 22) /* use the sweep strategy (all wavefronts walk the columns of B window by
                                          window, the row accumulators stay in LDS) whatever the size of the matrix
-                                         (default: from 2^22 nonzeros and 8 MB of B up, when the rows are long
-                                         against the size of B).  It needs sorted columns within every row, at most
+                                         (default: from 2^21 nonzeros and 5 MB of B up, where a cost model of the
+                                         sweep is below the expected time of whole rows in stored order).  It needs
+                                         sorted columns within every row, at most
                                          2^24 columns and less than 4 GB of B; otherwise the plan keeps to segments */
 #define HPSPMM_PLAN_NO_SWEEP (1u << 23)    /* never use the sweep strategy */
 

@@ -58,6 +58,51 @@ def test_argument_validation_without_device(pkg):
     assert L.hpspmm_csr_spmm_timed(None, fake, fake, fake, fake, fake, None, 0, 0, ctypes.byref(ms)) == capi.ERR_INVALID_ARG
 
 
+def test_plan_options_are_validated_without_device(pkg):
+    """hpspmm_plan_create_ex: a struct size that is none, values outside a field's range and flags
+    that contradict each other are refused before any device is touched; the python mirror of the
+    struct has the header's fields in the header's order."""
+    capi = pkg.capi
+    L = capi.lib()
+    h = ctypes.c_void_p()
+    fake = ctypes.c_void_p(4096)
+
+    def create(**fields):
+        o = capi.PlanOptions()
+        o.struct_size = ctypes.sizeof(capi.PlanOptions)
+        for name, value in fields.items():
+            setattr(o, name, value)
+        rc = L.hpspmm_plan_create_ex(ctypes.c_int64(4), ctypes.c_int64(4), ctypes.c_int64(0), fake, fake,
+                                     ctypes.c_int64(32), ctypes.byref(o), None, ctypes.byref(h))
+        return rc, L.hpspmm_last_error()
+
+    for bad in ({"struct_size": 0}, {"struct_size": 6}, {"struct_size": 10},
+                {"routed_tile_width": 48}, {"xcd_dealing": 3}, {"xcd_dealing": -1}, {"row_tiles_pad": 3},
+                {"row_tiles_chunk_log2": 17}, {"row_tiles_chunk_log2": -2}):
+        rc, msg = create(**bad)
+        assert rc == capi.ERR_INVALID_ARG, (bad, rc, msg)
+        assert msg != b"" and not h.value
+    # the mirror of the struct: every field the header declares, in its order
+    header = open(capi.HEADER_PATH).read()
+    body = header[header.index("typedef struct hpspmm_plan_options {"):header.index("} hpspmm_plan_options;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    declared = re.findall(r"\b(?:uint32_t|int32_t|const int32_t \*)\s*([a-z0-9_]+);", body)
+    assert declared == [n for n, _ in capi.PlanOptions._fields_]
+
+
+def test_info_structs_mirror_the_header(pkg):
+    """hpspmm_plan_info and hpspmm_device_info in capi.py: the header's fields in the header's order."""
+    capi = pkg.capi
+    header = open(capi.HEADER_PATH).read()
+    for c_name, mirror in (("hpspmm_plan_info", capi.PlanInfo), ("hpspmm_device_info", capi.DeviceInfo)):
+        body = header[header.index("typedef struct %s {" % c_name):header.index("} %s;" % c_name)]
+        body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+        declared = []
+        for types, names in re.findall(r"\b(int64_t|int32_t|double|char)\s+([a-z0-9_,\s\[\]]+);", body):
+            declared += [n.strip().split("[")[0] for n in names.split(",")]
+        assert declared == [n for n, _ in mirror._fields_], c_name
+
+
 def test_no_device_is_an_error_not_a_fallback(pkg):
     import torch
     if torch.cuda.is_available():

@@ -42,7 +42,7 @@ int main(int argc, char** argv) {
   try {
     std::vector<std::string> pos;
     bool check = false, synthetic = false;
-    std::string csv = "./full_graph_res_reorder.csv", dump, vendor = "2,3,-1,coo";
+    std::string csv, dump, vendor = "2,3,-1,coo";
     for (int i = 1; i < argc; ++i) {
       const std::string a = argv[i];
       if (a == "--check") check = true;
@@ -70,6 +70,9 @@ int main(int argc, char** argv) {
     int64_t num = 0, dim = 0, nnz = 0;
     CSR_Matrix h_csr;
     COO_Matrix h_coo_reorder, h_coo;
+    // default result file: that of the reference driver whose input this is - test/main.cpp:112 without
+    // a reorder file, test/test_all.cpp:108 with one
+    if (csv.empty()) csv = !synthetic && pos[1] == "-" ? "./full_graph_res.csv" : "./full_graph_res_reorder.csv";
     if (synthetic) {
       info.filename_ = pos[0] + "@" + pos[1];
       h_csr = make_synthetic_csr(pos[0], std::stod(pos[1]));

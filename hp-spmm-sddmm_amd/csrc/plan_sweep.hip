@@ -87,9 +87,42 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
     return kSweepPsPerNnz[ki] * (double)nnz * 1e-6 + kSweepUsPerWindow[ki] * (double)(bands * n_windows);
   };
   if (!forced && (other_us <= 0 || expected_us(ceil_div(nonempty, band_waves * WS)) > other_us)) return HPSPMM_OK;
-  if (!columns_sorted(p, d_rowptr, d_col, st)) return HPSPMM_OK;  // a row must meet the windows in stored order
-
   DeviceTemps tmp;
+  // A row must meet the windows in the order of its entries.  Where the columns of the rows are not
+  // stored in increasing order the layout is built from a copy in which they are (two stable radix
+  // sorts of the nonzeros: by column, then by row), and the value indices of the streams lead back
+  // to where the caller has every entry.
+  const int32_t* d_stored_at = nullptr;
+  if (!columns_sorted(p, d_rowptr, d_col, st)) {
+    if (nnz >= ((int64_t)1 << 31) - hpspmm::kSortTile) return HPSPMM_OK;
+    if (int rc = ensure_row_expansion(p, d_rowptr, st)) return rc;
+    const int64_t sort_tiles = ceil_div(nnz, sort_tile());
+    uint32_t* keys[2] = {nullptr, nullptr};
+    int32_t* vals[2] = {nullptr, nullptr};
+    uint32_t *d_hist = nullptr, *d_sscan = nullptr;
+    int32_t* d_scol = nullptr;
+    if (tmp.alloc(&keys[0], (size_t)nnz) || tmp.alloc(&keys[1], (size_t)nnz) || tmp.alloc(&vals[0], (size_t)nnz) ||
+        tmp.alloc(&vals[1], (size_t)nnz) || tmp.alloc(&d_hist, (size_t)(256 * sort_tiles + 1)) ||
+        tmp.alloc(&d_sscan, (size_t)scan_scratch_words(256 * sort_tiles)) || tmp.alloc(&d_scol, (size_t)nnz))
+      return HPSPMM_OK;  // no room: the plan stays what it was
+    const dim3 g(grid_for(nnz, 1 << 16)), b(hpspmm::kBlock);
+    int col_bits = 1, row_bits = 1;
+    while (col_bits < 32 && ((int64_t)1 << col_bits) < p->cols) ++col_bits;
+    while (row_bits < 32 && ((int64_t)1 << row_bits) < rows) ++row_bits;
+    int cur = 0;
+    hipLaunchKernelGGL(hpspmm::sweep_sort_keys_kernel, g, b, 0, st, nnz, d_col, (const int32_t*)nullptr, keys[0], vals[0]);
+    if (int rc = radix_sort_pairs(nnz, keys, vals, d_hist, d_sscan, col_bits, st, &cur)) return rc;
+    if (cur != 0) std::swap(keys[0], keys[1]), std::swap(vals[0], vals[1]);
+    hipLaunchKernelGGL(hpspmm::sweep_sort_keys_kernel, g, b, 0, st, nnz, p->d_nnz_row, (const int32_t*)vals[0], keys[0],
+                       (int32_t*)nullptr);
+    if (int rc = radix_sort_pairs(nnz, keys, vals, d_hist, d_sscan, row_bits, st, &cur)) return rc;
+    // the columns in that order
+    hipLaunchKernelGGL(hpspmm::sweep_sort_keys_kernel, g, b, 0, st, nnz, d_col, (const int32_t*)vals[cur],
+                       reinterpret_cast<uint32_t*>(d_scol), (int32_t*)nullptr);
+    d_stored_at = vals[cur];
+    d_col = d_scol;
+  }
+
   // pieces per row, their scans
   uint32_t *d_pbase = nullptr, *d_part = nullptr, *d_scan0 = nullptr;
   // (no room for a temporary or a buffer of the layout: the plan stays what it was, like any other
@@ -239,7 +272,7 @@ int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, b
                      p->d_vcol, p->d_vsrc);
   hipLaunchKernelGGL(hpspmm::sweep_fill_kernel, wave_grid, dim3(hpspmm::kBlock), 0, st, (int32_t)n_windows, wshift, limit,
                      (int32_t)WS, (int32_t)(k / 4), d_piece_of, d_piece_row, d_pbase, d_rowptr, d_col, d_wstart, d_run_at,
-                     p->d_sw_ends, p->d_sw_base, p->d_sw_len, p->d_vcol, p->d_vsrc);
+                     p->d_sw_ends, p->d_sw_base, p->d_sw_len, d_stored_at, p->d_vcol, p->d_vsrc);
   hipLaunchKernelGGL(hpspmm::sweep_slot_rows_kernel, dim3((unsigned)ceil_div(n_slots, hpspmm::kBlock)), dim3(hpspmm::kBlock),
                      0, st, n_slots, d_piece_of, d_piece_row, d_pbase, d_part, d_rowptr, limit, p->d_sw_slot_row);
 

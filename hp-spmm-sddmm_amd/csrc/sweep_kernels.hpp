@@ -277,6 +277,7 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_fill_kernel(int32_t n_windows
                                                             const int32_t* __restrict__ chunk_end,
                                                             const uint32_t* __restrict__ wave_base,
                                                             const uint32_t* __restrict__ wave_len,
+                                                            const int32_t* __restrict__ stored_at,
                                                             int32_t* __restrict__ vent, int32_t* __restrict__ vsrc) {
   constexpr int kMaxSlots = 64;  // 8 slots for each of at most 8 sub-waves
   __shared__ int32_t s_row[kMaxSlots], s_lb[kMaxSlots], s_m[kMaxSlots], s_k[kMaxSlots], s_size[kMaxSlots];
@@ -337,7 +338,21 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_fill_kernel(int32_t n_windows
     // lanes, ... of the tile, so that one gather instruction of the values covers neighbouring entries
     // (mostly one line of the value array per piece instead of one per lane).
     const int32_t u = (int32_t)(pos % kTile);  // the streams start at multiples of 32
-    vsrc[pos - u + (u % lanes) * per_lane + u / lanes] = j;
+    // (col[] may be a copy with every row's columns in increasing order: stored_at[] then says where
+    // entry j of the copy lies in the caller's arrays)
+    vsrc[pos - u + (u % lanes) * per_lane + u / lanes] = stored_at ? stored_at[j] : j;
+  }
+}
+
+// Sort keys for bringing the columns of every row into increasing order: pass 1 sorts the nonzeros
+// by column (key = col[j], value = j), pass 2, stable, by row (key = row of the value).
+HPSPMM_KERNEL __launch_bounds__(kBlock) void sweep_sort_keys_kernel(int64_t nnz, const int32_t* __restrict__ key_of,
+                                                                 const int32_t* __restrict__ at,
+                                                                 uint32_t* __restrict__ keys, int32_t* __restrict__ vals) {
+  for (int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x; q < nnz; q += (int64_t)gridDim.x * kBlock) {
+    const int32_t j = at ? at[q] : (int32_t)q;
+    keys[q] = (uint32_t)key_of[j];
+    if (!at) vals[q] = j;
   }
 }
 

@@ -86,8 +86,9 @@ typedef enum hpspmm_status {
                                          window, the row accumulators stay in LDS) whatever the size of the matrix
                                          (default: from 2^21 nonzeros and 5 MB of B up, where a cost model of the
                                          sweep is below the expected time of whole rows in stored order).  It needs
-                                         sorted columns within every row, at most
-                                         2^24 columns and less than 4 GB of B; otherwise the plan keeps to segments */
+                                         at most 2^24 columns and less than 4 GB of B, otherwise the plan keeps to
+                                         segments; rows whose columns are not in increasing order are laid out from
+                                         a sorted copy made at plan time */
 #define HPSPMM_PLAN_NO_SWEEP (1u << 23)    /* never use the sweep strategy */
 
 /* strategy reported by hpspmm_plan_get_info */

@@ -1093,7 +1093,8 @@ def test_sweep_strategy(pkg, oracle, gpu):
 def test_sweep_layout_corners(pkg, oracle, gpu):
     """Forced sweep plans whose layout is all corners: windows of a few columns, pieces of 64 nonzeros
     (most rows split, several bands), a lead of one window; a matrix with empty rows and a row of
-    every column; unsorted columns (the plan then keeps to segments)."""
+    every column; columns out of order within the rows, duplicates included (the layout is then built
+    from a sorted copy, and the values are still read where the caller has them)."""
     capi = pkg.capi
     rng = np.random.default_rng(11)
     cases = []
@@ -1119,13 +1120,30 @@ def test_sweep_layout_corners(pkg, oracle, gpu):
                 C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SWEEP, options=opts)
                 assert info["strategy"] == capi.STRATEGY_SWEEP, (name, opts, info)
                 _check(oracle, g, B, C, f"sweep corners {name} k={k} {opts}")
-    # columns out of order within the rows: no sweep layout, the forced flag falls back to segments
+    # columns out of order within the rows (with duplicates): the sweep layout from a sorted copy
     rowptr, col, val = _random_csr(rng, 500, 700, 20, 1.5, 0.1, sorted_unique=False)
     g = pkg.graphs.CSR(500, 700, rowptr, col, val)
-    B = pkg.graphs.dense_normal(700, 64, 6)
-    C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SWEEP)
-    assert info["strategy"] == capi.STRATEGY_SEGMENTS, info
-    _check(oracle, g, B, C, "sweep forced on unsorted columns")
+    for k in (32, 64, 128):
+        B = pkg.graphs.dense_normal(700, k, 6)
+        for opts in ({}, {"sweep_window_log2": 12, "sweep_limit": 16, "sweep_lead": 1}):
+            C, info = _run(pkg, gpu, g, B, capi.PLAN_FORCE_SWEEP, options=opts)
+            assert info["strategy"] == capi.STRATEGY_SWEEP, info
+            _check(oracle, g, B, C, f"sweep forced on unsorted columns k={k} {opts}")
+    # the social graph with every row's entries shuffled: the same layout as from the sorted rows, so the
+    # same sums in the same order - bit for bit the product of the sorted matrix - and the default plan
+    # still picks the sweep
+    g = pkg.graphs.make_graph("c2_social", 0.1)
+    perm = np.arange(g.nnz)
+    for r in range(g.rows):
+        lo, hi = g.rowptr[r], g.rowptr[r + 1]
+        perm[lo:hi] = lo + rng.permutation(hi - lo)
+    shuffled = pkg.graphs.CSR(g.rows, g.cols, g.rowptr, g.col[perm], g.val[perm])
+    B = pkg.graphs.dense_normal(g.cols, 128, 7)
+    C_sorted, info_sorted = _run(pkg, gpu, g, B, capi.PLAN_DEFAULT)
+    C_shuffled, info_shuffled = _run(pkg, gpu, shuffled, B, capi.PLAN_DEFAULT)
+    assert info_sorted["strategy"] == info_shuffled["strategy"] == capi.STRATEGY_SWEEP
+    _check(oracle, shuffled, B, C_shuffled, "social graph with shuffled rows")
+    assert np.array_equal(C_sorted, C_shuffled)
 
 
 def test_sweep_is_not_chosen_for_a_banded_matrix(pkg, oracle, gpu):

@@ -81,6 +81,47 @@ def test_scaled_families_have_their_character(pkg):
     assert 35 < st["mean_degree"] < 65 and 0.5 < st["cv"] < 1.2
 
 
+HELD_OUT_SCALE = 0.004  # about 4e5 nonzeros each
+
+
+@pytest.mark.parametrize("name", ["h1_prefattach", "h2_rmat", "h3_grid", "h4_bipartite", "h5_blocks", "h6_uniform100"])
+def test_held_out_families(pkg, name):
+    """The families the plan's choice is checked on: valid CSR, sorted rows without duplicates, the same
+    matrix from the same name and scale, and the property each one is there for."""
+    graphs = pkg.graphs
+    assert name in graphs.HELD_OUT
+    g = graphs.make_graph(name, HELD_OUT_SCALE)
+    check_csr_invariants(g)
+    assert _digest(g) == _digest(graphs.make_graph(name, HELD_OUT_SCALE))
+    assert 3.0e5 <= g.nnz <= 4.5e5
+    deg = np.diff(g.rowptr)
+    if name == "h1_prefattach":      # 24 edges per new vertex, both directions stored; a few hubs
+        assert g.rows == g.cols and pattern_is_symmetric(g)
+        assert deg.min() >= 20 and 40 < deg.mean() < 50 and deg.max() > 20 * deg.mean()
+    elif name == "h2_rmat":           # 2^n vertices, skewed rows, some without any entry
+        assert g.rows == g.cols and g.rows & (g.rows - 1) == 0 and pattern_is_symmetric(g)
+        assert deg.max() > 20 * deg.mean() and (deg == 0).any()
+    elif name == "h3_grid":           # 9-point mesh + 2 long-range entries per row: near-constant short rows
+        side = int(round(g.rows ** 0.5))
+        assert side * side == g.rows == g.cols and pattern_is_symmetric(g)
+        assert 12.5 < deg.mean() < 13.5 and deg.max() <= 25
+        r = np.repeat(np.arange(g.rows), deg)
+        near = np.abs(g.col.astype(np.int64) - r) <= side + 1
+        assert 0.6 < near.mean() < 0.75   # the mesh neighbours lie within one mesh row of the diagonal
+    elif name == "h4_bipartite":      # users x items, 8 : 1, popular items
+        assert g.rows > 8 * g.cols * 0.95 and g.rows < 8 * g.cols * 1.1
+        hits = np.sort(np.bincount(g.col, minlength=g.cols))[::-1]
+        assert hits[: g.cols // 100].sum() > 0.05 * g.nnz      # the top 1 % of the items take > 5 % of the entries
+        assert deg.max() > 4 * deg.mean()
+    elif name == "h5_blocks":         # most entries inside diagonal blocks of mixed sizes
+        assert g.rows == g.cols and pattern_is_symmetric(g)
+        r = np.repeat(np.arange(g.rows), deg)
+        assert (np.abs(g.col.astype(np.int64) - r) < 4096).mean() > 0.85
+    else:                             # exactly 100 entries in every row, anywhere
+        assert (deg == 100).all()
+        assert np.bincount(g.col, minlength=g.cols).max() < 200
+
+
 def test_values_symmetric(pkg):
     import scipy.sparse as sp
     g = pkg.graphs.make_graph("c4_rmat", 0.002)

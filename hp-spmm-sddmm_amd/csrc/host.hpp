@@ -219,7 +219,8 @@ struct hpspmm_plan {
   int32_t* d_ostart = nullptr;  // [rows] first position of every row in processing order
   int32_t* d_ocol = nullptr;    // [nnz] entry words: column, or slot of the window's LDS copy of B; first-of-row flag
   int32_t* d_run_delta = nullptr;  // [n_runs] index of a row's first value in the caller's array - its position in the order
-  // (d_run_row: the non-empty rows in processing order; d_seg_run, d_cross_rows, d_zero_rows as above)
+  // (d_run_row: the non-empty rows in processing order; d_seg_run, d_zero_rows as above; d_cross_rows: the rows
+  // that cross a window boundary)
   int32_t* d_wcols = nullptr;   // [windows * ocap] columns held in LDS by each window's workgroup
   int ocap = 0;
   int64_t owindows = 0;

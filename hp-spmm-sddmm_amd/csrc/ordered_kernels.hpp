@@ -28,8 +28,11 @@
 // at the entry's position plus a per-row offset.  Rows and offsets are kept row
 // by row (run_row, run_delta).  8 bytes per nonzero; with a column, a source
 // index and a row per nonzero it was 16 (co-purchase graph, K = 64: 2.93 -> 2.8 ms).
-// Rows cut by a segment boundary go through the carry slots exactly as in the
-// segments strategy; a fix-up kernel adds them up from the plan's list of such rows.
+// A row cut by a segment boundary inside one window is added up by the window's workgroup itself
+// (the partial sums wait in registers and meet in LDS once the segments are done); only the rows
+// that cross a window boundary go through carry slots in memory as in the segments strategy, and a
+// fix-up kernel adds those up from the plan's list of such rows.  The order of the additions is the
+// same either way: the part in the row's first segment, then segment after segment.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -380,7 +383,8 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_hot_kernel(int64_t nnz, int
 }
 
 // What the fix-up kernel has to do with every row: write zeros (kActionZero: no nonzeros), add carry
-// slots (kActionCross: its nonzeros lie in more than one segment), or nothing.
+// slots (kActionCross: its nonzeros lie in more than one stretch of 2^shift positions - the ordered
+// plan passes the length of a window here, the main kernel adds up the rows cut inside one), or nothing.
 HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_action_kernel(int64_t rows, const int32_t* __restrict__ rowptr,
                                                                    const int32_t* __restrict__ start, int shift,
                                                                    uint8_t* __restrict__ action) {
@@ -429,104 +433,163 @@ __global__ __launch_bounds__(kBlock) void spmm_ordered_kernel(
   }
   __syncthreads();
 
-  const int64_t g = (blk * kWavesPerBlock + (tid >> 6)) * P + lane / G;
+  const int wseg = (tid >> 6) * P + lane / G;  // this sub-wave's segment within the window
+  const int64_t g = blk * (kWavesPerBlock * P) + wseg;
   const int64_t s = g << shift;
-  if (s >= nnz) return;
+  const bool active = s < nnz;  // (every thread stays for the barriers at the end)
   const int64_t e = (s + ((int64_t)1 << shift)) < nnz ? (s + ((int64_t)1 << shift)) : nnz;
-  const int sbase = ((tid >> 6) * P + lane / G) * kTileStride;
+  const int64_t wbeg = (blk * (kWavesPerBlock * P)) << shift;       // the window: positions [wbeg, wend)
+  const int64_t wend = wbeg + ((int64_t)(kWavesPerBlock * P) << shift);
+  const int sbase = wseg * kTileStride;
 
   const int nv = lane_columns<K, kLd>(ld_arg, l);
   const bool in_tile = nv > 0;
   const bool c_aligned = c_rows_aligned<kLd>(ld_arg);
   const uint32_t ldc = c_row_length<K, kLd>(ld_arg);
-  // `run` = the run of the entry before the next tile whose rows are looked up: to begin with, the run
-  // of the segment's first entry, less one if that entry starts it
-  const int32_t first_run = seg_run[g];
-  int32_t run = first_run - ((oent[s] & kRunStart) != 0);
-  int32_t cur = run_row[first_run];
-  bool head_pending = (int64_t)start[cur] < s;
+  // Partial sums of the rows this segment shares with its neighbours: of the row that began in an
+  // earlier segment (head) and of the row that goes on into the next one (tail).  They stay here when
+  // the whole row lies inside the window, and go to the carry slots in memory when it does not.
+  float4 head_acc = make_float4(0.f, 0.f, 0.f, 0.f), tail_acc = head_acc;
+  bool head_here = false, tail_here = false;
+  int32_t tail_row = 0;
+  int64_t tail_last = 0;  // last position of the tail row
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (active) {
+    // `run` = the run of the entry before the next tile whose rows are looked up: to begin with, the run
+    // of the segment's first entry, less one if that entry starts it
+    const int32_t first_run = seg_run[g];
+    int32_t run = first_run - ((oent[s] & kRunStart) != 0);
+    int32_t cur = run_row[first_run];
+    // (where the first row lies is looked up here, with the other loads of the start: inside the walk
+    // the two dependent loads would stall the wavefront at the first change of row)
+    const int64_t first_rs = start[cur];
+    const int64_t first_re = first_rs + (rowptr[cur + 1] - rowptr[cur]);
+    bool head_pending = first_rs < s;
+    const bool head_inside = first_rs >= wbeg && first_re <= wend;
 
-  auto flush_to = [&](bool is_tail) {
-    const bool to_c = !head_pending && !is_tail;  // a row of C; else a carry slot (aligned, K floats)
-    float* dst = head_pending ? carry + (uint64_t)(2 * g) * K
-                              : (is_tail ? carry + (uint64_t)(2 * g + 1) * K : C + (uint64_t)(uint32_t)cur * ldc);
-    head_pending = false;
-    if (in_tile) {  // (what a lane beyond the tile holds is never read)
-      if (to_c) store_c_row<kLd, true>(dst + 4 * l, acc, nv, c_aligned);
-      else store_result(dst + 4 * l, acc);
-    }
-  };
-  auto flush = [&]() { flush_to(false); };
-  // One flat load per gather, its address selected between the LDS copy and memory: a branch
-  // per gather would make every load of a batch wait for the one before it.
-  const float* lds_b = s_b;
-  // a lane beyond the tile gathers what lane 0 gathers (a valid address, no branch in the loop); its
-  // sums are never stored
-  const int lg = in_tile ? l : 0;
-  auto loadb = [&](int32_t c) {
-    const uint32_t idx = (uint32_t)(c & kEntryPayload);
-    const float* row = c < 0 ? lds_b + idx * (uint32_t)K : B + (uint64_t)idx * (uint64_t)ld;
-    return *reinterpret_cast<const float4*>(row + 4 * lg);
-  };
+    auto flush_to = [&](bool is_tail) {
+      if (head_pending) {
+        if (head_inside) {
+          head_acc = acc;
+          head_here = true;
+        } else if (in_tile) {
+          store_result(carry + (uint64_t)(2 * g) * K + 4 * l, acc);
+        }
+        head_pending = false;
+        return;
+      }
+      if (is_tail) {
+        const int64_t rs = start[cur];
+        const int64_t re = rs + (rowptr[cur + 1] - rowptr[cur]);
+        if (rs >= wbeg && re <= wend) {
+          tail_acc = acc;
+          tail_here = true;
+          tail_row = cur;
+          tail_last = re - 1;
+        } else if (in_tile) {
+          store_result(carry + (uint64_t)(2 * g + 1) * K + 4 * l, acc);
+        }
+        return;
+      }
+      // (what a lane beyond the tile holds is never read)
+      if (in_tile) store_c_row<kLd, true>(C + (uint64_t)(uint32_t)cur * ldc + 4 * l, acc, nv, c_aligned);
+    };
+    auto flush = [&]() { flush_to(false); };
+    // One flat load per gather, its address selected between the LDS copy and memory: a branch
+    // per gather would make every load of a batch wait for the one before it.
+    const float* lds_b = s_b;
+    // a lane beyond the tile gathers what lane 0 gathers (a valid address, no branch in the loop); its
+    // sums are never stored
+    const int lg = in_tile ? l : 0;
+    auto loadb = [&](int32_t c) {
+      const uint32_t idx = (uint32_t)(c & kEntryPayload);
+      const float* row = c < 0 ? lds_b + idx * (uint32_t)K : B + (uint64_t)idx * (uint64_t)ld;
+      return *reinterpret_cast<const float4*>(row + 4 * lg);
+    };
 
-  // Two-deep prefetch.  look(t): the entry words of tile t and, from the run starts among them (a lane
-  // counts those of its TL entries, the sub-wave scans the counts), the row and the value offset of
-  // every entry.  take(t): the values of tile t through the offsets looked up one step earlier.  (The
-  // plan's arrays are allocated by the library, hence always aligned for the vector loads.)
-  int32_t ec[TL], er[TL], ed[TL];
-  auto look = [&](int64_t t) {
-    const int64_t q = t + l * TL;
-    load_run<TL>(ec, oent, q, e, true);  // 0 beyond e: a plain entry of the run before
-    int32_t starts = 0;
+    // Two-deep prefetch.  look(t): the entry words of tile t and, from the run starts among them (a lane
+    // counts those of its TL entries, the sub-wave scans the counts), the row and the value offset of
+    // every entry.  take(t): the values of tile t through the offsets looked up one step earlier.  (The
+    // plan's arrays are allocated by the library, hence always aligned for the vector loads.)
+    int32_t ec[TL], er[TL], ed[TL];
+    auto look = [&](int64_t t) {
+      const int64_t q = t + l * TL;
+      load_run<TL>(ec, oent, q, e, true);  // 0 beyond e: a plain entry of the run before
+      int32_t starts = 0;
 #pragma unroll
-    for (int j = 0; j < TL; ++j) starts += (ec[j] & kRunStart) != 0;
-    int32_t incl = starts;
+      for (int j = 0; j < TL; ++j) starts += (ec[j] & kRunStart) != 0;
+      int32_t incl = starts;
 #pragma unroll
-    for (int off = 1; off < G; off <<= 1) {
-      const int32_t o = __shfl_up(incl, off, G);
-      if (l >= off) incl += o;
-    }
-    int32_t at = run + incl - starts;
+      for (int off = 1; off < G; off <<= 1) {
+        const int32_t o = __shfl_up(incl, off, G);
+        if (l >= off) incl += o;
+      }
+      int32_t at = run + incl - starts;
 #pragma unroll
-    for (int j = 0; j < TL; ++j) {
-      at += (ec[j] & kRunStart) != 0;
-      er[j] = run_row[at];
-      ed[j] = run_delta[at];
-    }
-    run += __shfl(incl, G - 1, G);
-  };
-  TileRegs<TL> m;
-  auto take = [&](int64_t t) {
-    const int64_t q = t + l * TL;
+      for (int j = 0; j < TL; ++j) {
+        at += (ec[j] & kRunStart) != 0;
+        er[j] = run_row[at];
+        ed[j] = run_delta[at];
+      }
+      run += __shfl(incl, G - 1, G);
+    };
+    TileRegs<TL> m;
+    auto take = [&](int64_t t) {
+      const int64_t q = t + l * TL;
 #pragma unroll
-    for (int j = 0; j < TL; ++j) {
-      m.c[j] = ec[j];
-      m.r[j] = er[j];
-      m.v[j] = q + j < e ? val[q + j + ed[j]] : 0.f;
+      for (int j = 0; j < TL; ++j) {
+        m.c[j] = ec[j];
+        m.r[j] = er[j];
+        m.v[j] = q + j < e ? val[q + j + ed[j]] : 0.f;
+      }
+    };
+    look(s);
+    take(s);
+    if (s + kTile < e) look(s + kTile);
+    for (int64_t t = s; t < e; t += kTile) {
+      stage_tile<TL>(m, sbase + l * TL, s_col, s_val, s_row);
+      wave_lds_fence();
+      if (t + kTile < e) {
+        take(t + kTile);
+        if (t + 2 * kTile < e) look(t + 2 * kTile);
+      }
+      const int cnt = (e - t) < kTile ? (int)(e - t) : kTile;
+      consume_tile(cnt, sbase, s_col, s_val, s_row, cur, acc, loadb, flush);
+      wave_lds_fence();
     }
-  };
-  look(s);
-  take(s);
-  if (s + kTile < e) look(s + kTile);
-  for (int64_t t = s; t < e; t += kTile) {
-    stage_tile<TL>(m, sbase + l * TL, s_col, s_val, s_row);
-    wave_lds_fence();
-    if (t + kTile < e) {
-      take(t + kTile);
-      if (t + 2 * kTile < e) look(t + 2 * kTile);
+    flush_to((int64_t)start[cur] + (rowptr[cur + 1] - rowptr[cur]) > e);
+  }  // active
+
+  // The rows cut inside the window.  The window's rows of B are not needed any more: their LDS takes
+  // the head sums, one row of K floats per segment of the window (cap >= kWavesPerBlock * P: the host
+  // checks).  Every thread of the workgroup reaches both barriers.
+  __syncthreads();
+  if (head_here && in_tile) *reinterpret_cast<float4*>(s_b + wseg * K + 4 * l) = head_acc;
+  __syncthreads();
+  if (tail_here && in_tile) {
+    // the part in the row's first segment, then the heads of the segments it goes on into, in that
+    // order - as the fix-up kernel adds the carry slots of a row
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+    sum.x += tail_acc.x;
+    sum.y += tail_acc.y;
+    sum.z += tail_acc.z;
+    sum.w += tail_acc.w;
+    const int last = (int)((tail_last - wbeg) >> shift);
+    for (int w = wseg + 1; w <= last; ++w) {
+      const float4 h = *reinterpret_cast<const float4*>(s_b + w * K + 4 * l);
+      sum.x += h.x;
+      sum.y += h.y;
+      sum.z += h.z;
+      sum.w += h.w;
     }
-    const int cnt = (e - t) < kTile ? (int)(e - t) : kTile;
-    consume_tile(cnt, sbase, s_col, s_val, s_row, cur, acc, loadb, flush);
-    wave_lds_fence();
+    store_c_row<kLd, true>(C + (uint64_t)(uint32_t)tail_row * ldc + 4 * l, sum, nv, c_aligned);
   }
-  flush_to((int64_t)start[cur] + (rowptr[cur + 1] - rowptr[cur]) > e);
 }
 
 // Fix-up after the ordered kernel, from the plan's lists: workgroups [0, cross_blocks) - one
-// sub-wave per row whose nonzeros lie in more than one segment: tail[ga] + head[ga + 1] + ... +
-// head[gb] from the carry slots, in that order; the others - one sub-wave per row without nonzeros:
-// zeros.  Every other row was stored by the main kernel.
+// sub-wave per row whose nonzeros lie in more than one window: tail[ga] + head[ga + 1] + ... +
+// head[gb] from the carry slots of its segments, in that order; the others - one sub-wave per row
+// without nonzeros: zeros.  Every other row was stored by the main kernel.
 template <int K, int kLd = 0>
 __global__ __launch_bounds__(kBlock) void spmm_ordered_fixup_kernel(
     const int32_t* __restrict__ rowptr, const int32_t* __restrict__ start, const int32_t* __restrict__ cross_rows,

@@ -29,6 +29,8 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
   const int window = (int)((int64_t)hpspmm::kWavesPerBlock * subwaves << shift);
   const int64_t staging_bytes = 3 * hpspmm::kWavesPerBlock * subwaves * hpspmm::kTileStride * 4;
   const int cap = (int)((kOrderedBlockLdsBytes - staging_bytes) / (k * 4));
+  // (at the end of a window the same LDS takes one row of K floats per segment, spmm_ordered_kernel)
+  if (cap < hpspmm::kWavesPerBlock * subwaves) return HPSPMM_OK;
   const int64_t windows = ceil_div(nnz, window);
   const int64_t nseg = ceil_div(nnz, (int64_t)1 << shift);
 
@@ -113,8 +115,11 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
     drop();
     return HPSPMM_OK;
   }
-  // the lists of the rows the fix-up kernel has to visit
+  // the lists of the rows the fix-up kernel has to visit: those without nonzeros and those that cross
+  // a window boundary (the main kernel adds up the rows cut inside a window)
   {
+    int window_shift = shift;
+    while (((int64_t)1 << window_shift) < window) ++window_shift;
     DeviceTemps tmp;
     uint8_t* d_action = nullptr;
     int32_t* d_counts = nullptr;
@@ -127,7 +132,7 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
     }
     const unsigned row_grid = (unsigned)ceil_div(std::max<int64_t>(rows, 1), hpspmm::kBlock);
     hipLaunchKernelGGL(hpspmm::ordered_action_kernel, dim3(row_grid), dim3(hpspmm::kBlock), 0, st, rows, d_rowptr,
-                       p->d_ostart, shift, d_action);
+                       p->d_ostart, window_shift, d_action);
     hipError_t e2 = hipMemsetAsync(d_counts, 0, 2 * sizeof(int32_t), st);
     const unsigned collect_grid = (unsigned)ceil_div(std::max<int64_t>(rows, 1), hpspmm::kCollectRows);
     hipLaunchKernelGGL(hpspmm::routed_collect_rows_kernel, dim3(collect_grid), dim3(hpspmm::kBlock), 0, st, rows, d_action,

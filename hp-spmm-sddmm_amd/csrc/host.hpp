@@ -207,7 +207,7 @@ struct hpspmm_plan {
   int64_t n_runs = 0;
   int32_t* d_bhot_src = nullptr;  // [n_bhot] source column of every compact-buffer row (-1 = unused)
   int32_t* d_routed_rows = nullptr;  // [n_routed] row of every routed-row number
-  int32_t* d_cross_rows = nullptr;   // short rows whose run crosses a segment boundary
+  int32_t* d_cross_rows = nullptr;   // routed: short rows whose run crosses a segment boundary
   int32_t* d_zero_rows = nullptr;    // rows without nonzeros
   int64_t n_cross = 0, n_zero = 0;
   float* d_partial = nullptr;     // [n_routed * nhub * k]

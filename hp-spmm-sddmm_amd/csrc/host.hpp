@@ -365,7 +365,7 @@ int build_routed(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
                  ColumnRanking& rk, hipStream_t st);
 int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, const int32_t* d_order,
                   double min_served, hipStream_t st);
-int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, const PlanOptions& opt,
+int cluster_rows(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, const PlanOptions& opt,
                  hipStream_t st, int32_t** d_order_out, double* intra_share_out);
 int build_sweep(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, bool forced, double other_us,
                 const PlanOptions& opt, hipStream_t st);

@@ -48,7 +48,8 @@ namespace hpspmm {
 // Label propagation, one sweep: every row takes the label that is most frequent
 // among (a sample of at most 32 of) its neighbours' labels - the rows whose
 // indices are its column indices; the matrix is taken as a graph, which is
-// meant for square, structurally symmetric A.  Ties are broken by a hash that
+// meant for square, structurally symmetric A (the host hands over the
+// bipartite graph of rows and columns for any other).  Ties are broken by a hash that
 // changes with the sweep, except that a row keeps its label when that is among
 // the most frequent.  A sweep reads label_in and writes label_out (two buffers,
 // so the outcome does not depend on the order in which the wavefronts run: two
@@ -154,7 +155,10 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void cluster_sweep_kernel(int64_t rows, 
     c[i] = hl * stride < n[i] ? col[lb[i] + hl * stride] : -1;
   }
 #pragma unroll
-  for (int i = 0; i < R; ++i) lab[i] = (c[i] >= 0 && (int64_t)c[i] < rows) ? label_in[c[i]] : INT32_MAX;  // sorts behind every label
+  // (an entry on the diagonal has no vote: with one, every row of A + I would find its own label among
+  // the most frequent ones in the first sweep and keep it, and nothing would ever move)
+  for (int i = 0; i < R; ++i)
+    lab[i] = (c[i] >= 0 && (int64_t)c[i] < rows && (int64_t)c[i] != r[i]) ? label_in[c[i]] : INT32_MAX;  // sorts behind every label
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int32_t next_label = cluster_vote(lab[i], mine[i], r[i], sweep, hl, half);
@@ -228,6 +232,29 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void ordered_mark_kernel(int64_t rows, c
     return;
   }
   if (atomicAdd(&seen[r], 1) != 0) atomicOr(bad, 2);
+}
+
+// A rows x cols pattern as a graph of rows + cols vertices (vertex rows + c stands for column c),
+// for the label propagation above: row r is adjacent to the columns it has an entry in, column c to
+// the rows that have one in it.
+// out[j] = col[j] + by: the neighbours of the row vertices.
+HPSPMM_KERNEL __launch_bounds__(kBlock) void bipartite_shift_kernel(int64_t nnz, const int32_t* __restrict__ col,
+                                                                 int32_t by, int32_t* __restrict__ out) {
+  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (j < nnz) out[j] = col[j] + by;
+}
+
+// colptr[c] = base + the number of entries in columns below c, for c in [0, cols], from the column
+// of every nonzero in increasing order (sorted[nnz]): thread q writes the pointers of the columns
+// that begin at position q (none for most q; every column up to `cols` for q = nnz).
+HPSPMM_KERNEL __launch_bounds__(kBlock) void bipartite_colptr_kernel(int64_t nnz, const uint32_t* __restrict__ sorted,
+                                                                  int64_t cols, int32_t base,
+                                                                  int32_t* __restrict__ colptr) {
+  const int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (q > nnz) return;
+  const int64_t a = q > 0 ? (int64_t)sorted[q - 1] : -1;
+  const int64_t b = q < nnz ? (int64_t)sorted[q] : cols;
+  for (int64_t c = a + 1; c <= b; ++c) colptr[c] = base + (int32_t)q;
 }
 
 // Lays the nonzeros out in processing order.  One wavefront per position i: row r = order[i] starts

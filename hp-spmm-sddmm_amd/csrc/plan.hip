@@ -79,7 +79,11 @@ constexpr double kLocalMissShare = 0.3;  // stored order counts as local up to t
 constexpr double kRowsFallbackMissShare = 0.85;
 constexpr double kRowsHitPs = 7.0, kRowsMissPs = 20.7;  // rows strategy: per nonzero and 32 columns of B
 constexpr double kClusterMinIntra = 0.15;   // share of the nonzeros inside such clusters for the order to be used
-constexpr int64_t kClusterMinMeanNnz = 8;
+// Rows of fewer nonzeros than this on average are left to the row tiles: what the ordered strategy spends per
+// row (a run's row and value offset, a store of C per ~13 gathers) outweighs the gathers it saves (9-point mesh
+// with two long-range entries per row, 12 M nonzeros, clusters found once the diagonal has no vote: 192 / 387 /
+// 742 us against 128 / 253 / 590 for whole rows in stored order).
+constexpr int64_t kClusterMinMeanNnz = 16;
 // ... and its order is kept if this share of the nonzeros then reads B from LDS.
 constexpr double kClusterMinServed = 0.15;
 
@@ -359,8 +363,9 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
     // end, if the plan is still a segments plan then: the layouts tried below mostly replace both
   }
   const bool want_cluster = (flags & HPSPMM_PLAN_CLUSTER) != 0;
-  // a graph (square) large enough for an order of its rows by community to pay, if it has communities
-  const bool cluster_candidate = rows == cols && nnz >= kClusterMinNnz && nnz >= rows * kClusterMinMeanNnz &&
+  // large enough for an order of its rows by community to pay, if it has communities (a square matrix
+  // is taken as a graph on its rows, any other as the bipartite graph of its rows and columns)
+  const bool cluster_candidate = nnz >= kClusterMinNnz && nnz >= rows * kClusterMinMeanNnz &&
                                  cols * k * 4 >= (miss <= kLocalMissShare ? kClusterLocalMinBBytes : kClusterMinBBytes) &&
                                  !(flags & HPSPMM_PLAN_NO_CLUSTER);
   // Long rows over a B that is small against the gather volume: every wavefront walks B window by
@@ -384,17 +389,17 @@ int plan_create_impl(int64_t rows, int64_t cols, int64_t nnz, const int32_t* d_r
       !(flags & HPSPMM_PLAN_FORCE_SEGMENTS && !(flags & HPSPMM_PLAN_FORCE_ROUTED))) {
     if (int rc = build_routed(p, d_rowptr, d_col, (flags & HPSPMM_PLAN_FORCE_ROUTED) != 0, opt, ranking, st)) return rc;
   }
-  // Community structure: not routed, the matrix is a graph (square) and B does not fit the L2s -
-  // look for clusters of rows that share columns.  Tried before the hub cache: a graph can have
+  // Community structure: not routed and B does not fit the L2s - look for clusters of rows that
+  // share columns.  Tried before the hub cache: a graph can have
   // both popular columns and communities (the co-purchase graph at a quarter of its size: the 64k
   // most referenced columns take a quarter of the nonzeros there), and the ordered strategy is then
   // the faster of the two (0.73 ms against 1.15 ms for segments with the hub cache).
-  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && rows == cols && nnz > 0 &&
+  if (p->strategy == HPSPMM_STRATEGY_SEGMENTS && fast_k(k) && nnz > 0 &&
       !(flags & HPSPMM_PLAN_NO_CLUSTER) && (want_cluster || (!(flags & HPSPMM_PLAN_FORCE_SEGMENTS) && cluster_candidate))) {
     int32_t* d_order = nullptr;
     double intra_share = 0.0;
     int rc = cluster_rows(p, d_rowptr, d_col, opt, st, &d_order, &intra_share);
-    if (rc == HPSPMM_OK && (want_cluster || intra_share >= kClusterMinIntra))
+    if (rc == HPSPMM_OK && d_order && (want_cluster || intra_share >= kClusterMinIntra))
       rc = build_ordered(p, d_rowptr, d_col, d_order, want_cluster ? 0.0 : kClusterMinServed, st);
     if (d_order) (void)hipFree(d_order);
     if (rc) {

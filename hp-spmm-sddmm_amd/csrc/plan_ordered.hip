@@ -165,16 +165,19 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
   return HPSPMM_OK;
 }
 
-// Finds a processing order for a square matrix by label propagation on its graph: rows of one
-// label next to each other, labels in increasing order, rows of a label in increasing order.
-// d_order_out receives a device array of `rows` entries (caller frees).
+// Label propagation over a graph of n vertices given as CSR adjacency (nnz entries): *d_label_out
+// receives the label of every vertex (a new device array, caller frees), *intra_share_out the share
+// of the entries whose two ends carry one label of at most kClusterMaxSize vertices.
 constexpr int kClusterMaxSweeps = 16;
-constexpr int32_t kClusterMaxSize = 4096;  // rows of a cluster that still counts as one a window can profit from
+constexpr int32_t kClusterMaxSize = 4096;  // vertices of a cluster that still counts as one a window can profit from
+constexpr int kClusterLookSweeps = 4;           // after this many sweeps the clusters found so far are scored once
+// ... and the propagation ends if their share of the entries is below this (graphs with communities: 0.12-0.18 by then,
+// on their way to 0.46-0.83; preferential attachment, R-MAT, users x items, uniform rows: 0.003-0.026, never beyond 0.03)
+constexpr double kClusterLookMinIntra = 0.05;
 
-int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, const PlanOptions& opt,
-                 hipStream_t st, int32_t** d_order_out, double* intra_share_out) {
-  const int64_t rows = p->rows;
-  *d_order_out = nullptr;
+static int cluster_graph(int64_t n, int64_t nnz, const int32_t* d_rowptr, const int32_t* d_col, const PlanOptions& opt,
+                         hipStream_t st, int32_t** d_label_out, double* intra_share_out) {
+  *d_label_out = nullptr;
   *intra_share_out = 0.0;
   int32_t* d_label = nullptr;
   int32_t* d_label_next = nullptr;
@@ -186,19 +189,50 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
         if (*x) (void)hipFree(*x);
     }
   } guard{{(void**)&d_label, (void**)&d_label_next, (void**)&d_changed}};
-  HPSPMM_HIP(hipMalloc(&d_label, (size_t)rows * sizeof(int32_t)));
-  HPSPMM_HIP(hipMalloc(&d_label_next, (size_t)rows * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&d_label, (size_t)n * sizeof(int32_t)));
+  HPSPMM_HIP(hipMalloc(&d_label_next, (size_t)n * sizeof(int32_t)));
   HPSPMM_HIP(hipMalloc(&d_changed, hpspmm::kClusterCounters * sizeof(uint32_t)));
   std::vector<uint32_t> counters((size_t)hpspmm::kClusterCounters);
-  hipLaunchKernelGGL(hpspmm::cluster_init_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock),
-                     0, st, rows, d_label);
+  hipLaunchKernelGGL(hpspmm::cluster_init_kernel, dim3((unsigned)ceil_div(n, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                     0, st, n, d_label);
   const int max_sweeps = opt.cluster_sweeps > 0 ? opt.cluster_sweeps : kClusterMaxSweeps;
   const bool debug = opt.report;
+  // share of the entries that stay inside a cluster small enough for a workgroup's window, from
+  // every 4th vertex when there are a million of them (a threshold decision: 1.4 -> 0.4 ms at 2.4 M rows)
+  const int64_t score_stride = n >= ((int64_t)1 << 20) ? 4 : 1;
+  int32_t* d_size = nullptr;
+  struct SizeGuard {
+    int32_t** q;
+    ~SizeGuard() {
+      if (*q) (void)hipFree(*q);
+    }
+  } size_guard{&d_size};
+  HPSPMM_HIP(hipMalloc(&d_size, (size_t)n * sizeof(int32_t)));
+  auto intra_share = [&](double* share) -> int {
+    hipError_t e = hipMemsetAsync(d_size, 0, (size_t)n * sizeof(int32_t), st);
+    if (e == hipSuccess) e = hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st);
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL(hpspmm::label_sizes_kernel, dim3((unsigned)ceil_div(n, hpspmm::kBlock)), dim3(hpspmm::kBlock),
+                         0, st, n, d_label, d_size);
+      hipLaunchKernelGGL(hpspmm::cluster_intra_kernel,
+                         dim3((unsigned)ceil_div(ceil_div(n, score_stride), hpspmm::kWavesPerBlock)),
+                         dim3(hpspmm::kBlock), 0, st, n, score_stride, d_rowptr, d_col, d_label, d_size,
+                         kClusterMaxSize, d_changed);
+      e = hipMemcpyAsync(counters.data(), d_changed, counters.size() * sizeof(uint32_t), hipMemcpyDeviceToHost, st);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "cluster scoring failed: %s", hipGetErrorString(e));
+    int64_t intra = 0;
+    for (uint32_t c : counters) intra += c;
+    intra *= score_stride;
+    *share = nnz > 0 ? (double)intra / (double)nnz : 0.0;
+    return HPSPMM_OK;
+  };
   for (int sweep = 0; sweep < max_sweeps; ++sweep) {
     HPSPMM_HIP(hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st));
     hipLaunchKernelGGL(hpspmm::cluster_sweep_kernel,
-                       dim3((unsigned)ceil_div(ceil_div(rows, 2), hpspmm::kWavesPerBlock * 2 * hpspmm::kClusterRowsPerHalf)),
-                       dim3(hpspmm::kBlock), 0, st, rows, d_rowptr, d_col, d_label, d_label_next, (uint32_t)sweep,
+                       dim3((unsigned)ceil_div(ceil_div(n, 2), hpspmm::kWavesPerBlock * 2 * hpspmm::kClusterRowsPerHalf)),
+                       dim3(hpspmm::kBlock), 0, st, n, d_rowptr, d_col, d_label, d_label_next, (uint32_t)sweep,
                        d_changed);
     std::swap(d_label, d_label_next);
     HPSPMM_HIP(hipMemcpyAsync(counters.data(), d_changed, counters.size() * sizeof(uint32_t), hipMemcpyDeviceToHost,
@@ -206,37 +240,77 @@ int cluster_rows(const hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d
     HPSPMM_HIP(hipStreamSynchronize(st));
     int64_t changed = 0;
     for (uint32_t c : counters) changed += c;
-    if (debug) fprintf(stderr, "cluster sweep %d: %lld of %lld rows changed their label\n", sweep, (long long)changed, (long long)rows);
-    if (changed * 200 < rows) break;
-  }
-  // share of the nonzeros that stay inside a cluster small enough for a workgroup's window, from
-  // every 4th row when there are a million of them (a threshold decision: 1.4 -> 0.4 ms at 2.4 M rows)
-  const int64_t score_stride = rows >= ((int64_t)1 << 20) ? 4 : 1;
-  {
-    int32_t* d_size = nullptr;
-    hipError_t e = hipMalloc(&d_size, (size_t)rows * sizeof(int32_t));
-    if (e == hipSuccess) e = hipMemsetAsync(d_size, 0, (size_t)rows * sizeof(int32_t), st);
-    if (e == hipSuccess) e = hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st);
-    if (e == hipSuccess) {
-      hipLaunchKernelGGL(hpspmm::label_sizes_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock),
-                         0, st, rows, d_label, d_size);
-      hipLaunchKernelGGL(hpspmm::cluster_intra_kernel,
-                         dim3((unsigned)ceil_div(ceil_div(rows, score_stride), hpspmm::kWavesPerBlock)),
-                         dim3(hpspmm::kBlock), 0, st, rows, score_stride, d_rowptr, d_col, d_label, d_size,
-                         kClusterMaxSize, d_changed);
-      e = hipMemcpyAsync(counters.data(), d_changed, counters.size() * sizeof(uint32_t), hipMemcpyDeviceToHost, st);
+    if (debug) fprintf(stderr, "cluster sweep %d: %lld of %lld vertices changed their label\n", sweep, (long long)changed, (long long)n);
+    if (changed * 200 < n) break;
+    if (debug || sweep + 1 == kClusterLookSweeps) {
+      // a look on the way: where no clusters are forming by now, none will
+      double so_far = 0.0;
+      if (int rc = intra_share(&so_far)) return rc;
+      if (debug) fprintf(stderr, "cluster: %.4f of the entries inside small clusters after sweep %d\n", so_far, sweep);
+      if (sweep + 1 == kClusterLookSweeps && so_far < kClusterLookMinIntra && opt.cluster_sweeps <= 0) break;
     }
-    if (e == hipSuccess) e = hipStreamSynchronize(st);
-    if (d_size) (void)hipFree(d_size);
-    if (e != hipSuccess) return fail(HPSPMM_ERR_HIP, "cluster scoring failed: %s", hipGetErrorString(e));
-    int64_t intra = 0;
-    for (uint32_t c : counters) intra += c;
-    intra *= score_stride;
-    *intra_share_out = p->nnz > 0 ? (double)intra / (double)p->nnz : 0.0;
-    if (debug) fprintf(stderr, "cluster: %.4f of the nonzeros inside clusters of at most %d rows\n", *intra_share_out, kClusterMaxSize);
+  }
+  if (int rc = intra_share(intra_share_out)) return rc;
+  if (debug) fprintf(stderr, "cluster: %.4f of the entries inside clusters of at most %d vertices\n", *intra_share_out, kClusterMaxSize);
+  *d_label_out = d_label;
+  d_label = nullptr;  // (the guard keeps what is still named here)
+  return HPSPMM_OK;
+}
+
+// Finds a processing order for the rows by label propagation: rows of one label next to each other,
+// labels in increasing order, rows of a label in increasing order.  A square matrix is taken as a
+// graph on its rows (row r adjacent to the rows whose numbers are its column indices); any other
+// as the bipartite graph of its rows and columns, whose column side (the transposed pattern) is
+// built here by a stable sort of the nonzeros by column.  d_order_out receives a device array of
+// `rows` entries (caller frees); no order (NULL, status OK) when the temporaries do not fit.
+int cluster_rows(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, const PlanOptions& opt,
+                 hipStream_t st, int32_t** d_order_out, double* intra_share_out) {
+  const int64_t rows = p->rows, cols = p->cols, nnz = p->nnz;
+  *d_order_out = nullptr;
+  *intra_share_out = 0.0;
+  int32_t* d_label = nullptr;
+  struct Guard {
+    int32_t** q;
+    ~Guard() {
+      if (*q) (void)hipFree(*q);
+    }
+  } guard{&d_label};
+  if (rows == cols) {
+    if (int rc = cluster_graph(rows, nnz, d_rowptr, d_col, opt, st, &d_label, intra_share_out)) return rc;
+  } else {
+    const int64_t n = rows + cols;
+    if (n >= ((int64_t)1 << 31) - 1 || 2 * nnz >= ((int64_t)1 << 31) - hpspmm::kSortTile) return HPSPMM_OK;
+    if (int rc = ensure_row_expansion(p, d_rowptr, st)) return rc;
+    DeviceTemps tmp;
+    const int64_t sort_tiles = ceil_div(nnz, sort_tile());
+    uint32_t* keys[2] = {nullptr, nullptr};
+    int32_t* vals[2] = {nullptr, nullptr};
+    uint32_t *d_hist = nullptr, *d_sscan = nullptr;
+    int32_t *d_rowptr2 = nullptr, *d_col2 = nullptr;
+    if (tmp.alloc(&keys[0], (size_t)nnz) || tmp.alloc(&keys[1], (size_t)nnz) || tmp.alloc(&vals[0], (size_t)nnz) ||
+        tmp.alloc(&vals[1], (size_t)nnz) || tmp.alloc(&d_hist, (size_t)(256 * sort_tiles + 1)) ||
+        tmp.alloc(&d_sscan, (size_t)scan_scratch_words(256 * sort_tiles)) || tmp.alloc(&d_rowptr2, (size_t)n + 1) ||
+        tmp.alloc(&d_col2, (size_t)(2 * nnz)))
+      return HPSPMM_OK;  // no room: no order
+    // the nonzeros by column (stable: the rows of a column in increasing order)
+    HPSPMM_HIP(hipMemcpyAsync(keys[0], d_col, (size_t)nnz * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
+    HPSPMM_HIP(hipMemcpyAsync(vals[0], p->d_nnz_row, (size_t)nnz * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
+    int col_bits = 1;
+    while (col_bits < 32 && ((int64_t)1 << col_bits) < cols) ++col_bits;
+    int cur = 0;
+    if (int rc = radix_sort_pairs(nnz, keys, vals, d_hist, d_sscan, col_bits, st, &cur)) return rc;
+    // (radix_sort_pairs leaves the sorted keys beside the sorted values)
+    const unsigned grid = (unsigned)ceil_div(nnz + 1, hpspmm::kBlock);
+    HPSPMM_HIP(hipMemcpyAsync(d_rowptr2, d_rowptr, (size_t)rows * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
+    hipLaunchKernelGGL(hpspmm::bipartite_colptr_kernel, dim3(grid), dim3(hpspmm::kBlock), 0, st, nnz, keys[cur], cols,
+                       (int32_t)nnz, d_rowptr2 + rows);
+    hipLaunchKernelGGL(hpspmm::bipartite_shift_kernel, dim3(grid), dim3(hpspmm::kBlock), 0, st, nnz, d_col, (int32_t)rows,
+                       d_col2);
+    HPSPMM_HIP(hipMemcpyAsync(d_col2 + nnz, vals[cur], (size_t)nnz * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
+    if (int rc = cluster_graph(n, 2 * nnz, d_rowptr2, d_col2, opt, st, &d_label, intra_share_out)) return rc;
   }
   // rows ordered by label, the rows of a label in increasing order: a stable sort, hence the same
-  // order on every run
+  // order on every run (the labels of the column vertices, behind those of the rows, are not looked at)
   int32_t* d_order = nullptr;
   if (int rc = sort_rows_by_label(rows, d_label, st, &d_order)) return rc;
   *d_order_out = d_order;

@@ -71,11 +71,12 @@ typedef enum hpspmm_status {
                                          structure); default: other addresses are HPSPMM_ERR_INVALID_ARG */
 /* bits 8..11: log2 of the segment length to force (0 = choose automatically) */
 #define HPSPMM_PLAN_SEGMENT_SHIFT(log2_len) (((uint32_t)(log2_len) & 0xFu) << 8)
-#define HPSPMM_PLAN_CLUSTER 4096u     /* square A: always look for clusters of rows that share columns and use the
+#define HPSPMM_PLAN_CLUSTER 4096u     /* always look for clusters of rows that share columns and use the
                                          ordered strategy on the order found (default: from 2^22 nonzeros and
-                                         24 MB of B up, when the graph is not routed, and only if >= 15 % of the
+                                         12 MB of B up, when the matrix is not routed, and only if >= 15 % of the
                                          nonzeros stay inside clusters of <= 4096 rows and >= 15 % then read B
-                                         from LDS).  The clustering is deterministic: two plans of one matrix
+                                         from LDS).  A square A is taken as a graph on its rows, any other as the
+                                         bipartite graph of its rows and columns.  The clustering is deterministic: two plans of one matrix
                                          order the rows alike and give the same bits of C */
 #define HPSPMM_PLAN_NO_CLUSTER 8192u  /* never */
 #define HPSPMM_PLAN_ROUTED_SORT_VALUES 32768u /* routed strategy: never cut the columns into consecutive ranges (which lets

@@ -867,6 +867,45 @@ def test_clustering_finds_planted_communities(pkg, oracle, gpu):
     _check(oracle, sq, Bs, C, "clustered unsymmetric square matrix")
 
 
+def test_clustering_of_rectangular_matrices_and_with_a_diagonal(pkg, oracle, gpu):
+    """The community structure must also be found when the matrix is not a plain graph: half the rows of
+    the co-purchase-style graph (users x items, taken as the bipartite graph of rows and columns) and the
+    same graph with a unit diagonal added (A + I, the form graph networks feed); a users x items matrix
+    without communities is not reordered, and the search for them ends early."""
+    import scipy.sparse as sp
+    capi, graphs = pkg.capi, pkg.graphs
+    g = graphs.make_graph("c3_copurchase", 0.1)          # 245k vertices, 12 M nonzeros
+    A = sp.csr_matrix((g.val, g.col, g.rowptr), shape=(g.rows, g.cols))
+    k = 64
+    B = graphs.make_dense("c3_copurchase", g.cols, k)
+
+    def csr_of(M):
+        M = M.tocsr()
+        M.sort_indices()
+        return graphs.CSR(M.shape[0], M.shape[1], M.indptr.astype(np.int32), M.indices.astype(np.int32),
+                          M.data.astype(np.float32))
+
+    half = csr_of(A[: g.rows // 2])
+    C, info = _run(pkg, gpu, half, B, capi.PLAN_DEFAULT)
+    assert info["strategy"] == capi.STRATEGY_ORDERED, info
+    assert info["lds_served_nnz"] >= 0.25 * half.nnz, info
+    _check(oracle, half, B, C, "half the rows of the co-purchase graph")
+    C2, _ = _run(pkg, gpu, half, B, capi.PLAN_DEFAULT)
+    assert np.array_equal(C.view(np.uint32), C2.view(np.uint32))  # two plans: same order, same bits
+
+    with_diag = csr_of(A + sp.identity(g.rows, dtype=np.float32, format="csr"))
+    C, info = _run(pkg, gpu, with_diag, B, capi.PLAN_DEFAULT)
+    assert info["strategy"] == capi.STRATEGY_ORDERED, info
+    assert info["lds_served_nnz"] >= 0.3 * with_diag.nnz, info
+    _check(oracle, with_diag, B, C, "co-purchase graph with a unit diagonal")
+
+    plain = graphs.make_graph("h4_bipartite", 0.12)      # users x items, popular items, no communities
+    Bp = graphs.make_dense("h4_bipartite", plain.cols, k)
+    C, info = _run(pkg, gpu, plain, Bp, capi.PLAN_DEFAULT)
+    assert info["strategy"] != capi.STRATEGY_ORDERED, info
+    _check(oracle, plain, Bp, C, "users x items")
+
+
 def test_extreme_shapes(pkg, oracle, gpu):
     """One dense row among singletons, a permutation matrix, a single column, a single row: the shapes
     that stress the carry chains, the row lists and the hot-column logic of every strategy."""

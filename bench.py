@@ -76,16 +76,16 @@ ROOFLINE_WORKLOAD = ("c2_social", 128)
 # measured on: same workload, K, strategy and number of launches, scale 1, default plan.
 MEASURED_TRAFFIC = {
     ("c2_social", 32): {"strategy": 6, "launches": 2, "profile": "profiles/spmm_sweep_kernel__c2_social.txt",
-                        "kernels": {"spmm_sweep_kernel": 3.929, "spmm_sweep_final_kernel": 0.012}},
+                        "kernels": {"spmm_sweep_kernel": 3.922, "spmm_sweep_final_kernel": 0.012}},
     ("c2_social", 64): {"strategy": 6, "launches": 2, "profile": "profiles/spmm_sweep_kernel__c2_social.txt",
                         "kernels": {"spmm_sweep_kernel": 3.998, "spmm_sweep_final_kernel": 0.010}},
     ("c2_social", 128): {"strategy": 6, "launches": 2, "profile": "profiles/spmm_sweep_kernel__c2_social.txt",
-                         "kernels": {"spmm_sweep_kernel": 6.379, "spmm_sweep_final_kernel": 0.019}},
+                         "kernels": {"spmm_sweep_kernel": 6.377, "spmm_sweep_final_kernel": 0.019}},
     ("c3_copurchase", 64): {"strategy": 5, "launches": 2, "profile": "profiles/spmm_ordered_kernel__c3_copurchase.txt",
-                            "kernels": {"spmm_ordered_kernel": 20.407, "spmm_ordered_fixup_kernel": 0.015}},
+                            "kernels": {"spmm_ordered_kernel": 20.428, "spmm_ordered_fixup_kernel": 0.015}},
     # (the main kernel of the routed strategy is instantiated by tile width and workgroup size, not by K)
     ("c4_rmat", 128): {"strategy": 4, "launches": 3, "profile": "profiles/spmm_routed_tiles_kernel__c4_rmat.txt",
-                       "kernels": {"routed_prepare_kernel": 1.573, "spmm_routed_tiles_kernel": 32.735,
+                       "kernels": {"routed_prepare_kernel": 1.573, "spmm_routed_tiles_kernel": 32.728,
                                    "spmm_routed_final_kernel": 0.715}},
 }
 

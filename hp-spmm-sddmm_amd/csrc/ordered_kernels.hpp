@@ -245,16 +245,20 @@ HPSPMM_KERNEL __launch_bounds__(kBlock) void bipartite_shift_kernel(int64_t nnz,
 }
 
 // colptr[c] = base + the number of entries in columns below c, for c in [0, cols], from the column
-// of every nonzero in increasing order (sorted[nnz]): thread q writes the pointers of the columns
-// that begin at position q (none for most q; every column up to `cols` for q = nnz).
+// of every nonzero in increasing order (sorted[nnz]): one thread per column bisects the sorted list
+// (the same work whatever the gaps between the columns that occur).
 HPSPMM_KERNEL __launch_bounds__(kBlock) void bipartite_colptr_kernel(int64_t nnz, const uint32_t* __restrict__ sorted,
                                                                   int64_t cols, int32_t base,
                                                                   int32_t* __restrict__ colptr) {
-  const int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (q > nnz) return;
-  const int64_t a = q > 0 ? (int64_t)sorted[q - 1] : -1;
-  const int64_t b = q < nnz ? (int64_t)sorted[q] : cols;
-  for (int64_t c = a + 1; c <= b; ++c) colptr[c] = base + (int32_t)q;
+  const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (c > cols) return;
+  int64_t lo = 0, hi = nnz;  // first position whose column is >= c
+  while (lo < hi) {
+    const int64_t mid = lo + ((hi - lo) >> 1);
+    if ((int64_t)sorted[mid] < c) lo = mid + 1;
+    else hi = mid;
+  }
+  colptr[c] = base + (int32_t)lo;
 }
 
 // Lays the nonzeros out in processing order.  One wavefront per position i: row r = order[i] starts

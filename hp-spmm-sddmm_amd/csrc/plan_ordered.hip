@@ -300,10 +300,10 @@ int cluster_rows(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
     int cur = 0;
     if (int rc = radix_sort_pairs(nnz, keys, vals, d_hist, d_sscan, col_bits, st, &cur)) return rc;
     // (radix_sort_pairs leaves the sorted keys beside the sorted values)
-    const unsigned grid = (unsigned)ceil_div(nnz + 1, hpspmm::kBlock);
+    const unsigned grid = (unsigned)ceil_div(nnz, hpspmm::kBlock);
     HPSPMM_HIP(hipMemcpyAsync(d_rowptr2, d_rowptr, (size_t)rows * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
-    hipLaunchKernelGGL(hpspmm::bipartite_colptr_kernel, dim3(grid), dim3(hpspmm::kBlock), 0, st, nnz, keys[cur], cols,
-                       (int32_t)nnz, d_rowptr2 + rows);
+    hipLaunchKernelGGL(hpspmm::bipartite_colptr_kernel, dim3((unsigned)ceil_div(cols + 1, hpspmm::kBlock)),
+                       dim3(hpspmm::kBlock), 0, st, nnz, keys[cur], cols, (int32_t)nnz, d_rowptr2 + rows);
     hipLaunchKernelGGL(hpspmm::bipartite_shift_kernel, dim3(grid), dim3(hpspmm::kBlock), 0, st, nnz, d_col, (int32_t)rows,
                        d_col2);
     HPSPMM_HIP(hipMemcpyAsync(d_col2 + nnz, vals[cur], (size_t)nnz * sizeof(int32_t), hipMemcpyDeviceToDevice, st));

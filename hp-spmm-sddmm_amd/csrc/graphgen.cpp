@@ -684,6 +684,8 @@ hpspmm_graph* hpspmm_gen_named(const char* name, double scale) {
   //   h4_bipartite   users x items (8 : 1), lognormal basket sizes (mean ~60), Zipf(0.9) popularity
   //   h5_blocks      communities of 8 to 4096 vertices, 90 % of the edges inside, mean degree ~40
   //   h6_uniform100  100 uniformly placed nonzeros in every row
+  //   h7_groups      users x items (1 : 2) with communities: the first half of the rows of a community graph
+  //                  (lognormal(3.2, 0.8) weights, communities of ~48, 70 % of the edges inside)
   if (n == "h1_prefattach") return hpspmm_gen_pref_attach(scaled(2.1e6, 64), 24, 11);
   if (n == "h2_rmat") {
     const int sc = std::max(6, 21 + (int)std::lround(std::log2(scale)));
@@ -698,6 +700,19 @@ hpspmm_graph* hpspmm_gen_named(const char* name, double scale) {
   if (n == "h6_uniform100") {
     const int64_t v = scaled(1.0e6, 128);
     return hpspmm_gen_uniform_rows(v, v, 100, 16);
+  }
+  if (n == "h7_groups") {
+    const int64_t v = scaled(3.2e6, 128);
+    hpspmm_graph* whole = hpspmm_gen_community(v, 3.2, 0.8, std::max<int64_t>(1, v / 48), 0.7,
+                                               (int64_t)std::llround(61.5 * (double)v), 17);
+    if (!whole) return nullptr;
+    Graph* g = (Graph*)whole;  // keep rows [0, v / 2): every community has members on both sides
+    g->rows = v / 2;
+    g->rowptr.resize((size_t)g->rows + 1);
+    g->nnz = g->rowptr[(size_t)g->rows];
+    g->col.resize((size_t)g->nnz);
+    g->val.resize((size_t)g->nnz);
+    return whole;
   }
   g_err = "gen_named: unknown configuration '" + n + "'";
   return nullptr;

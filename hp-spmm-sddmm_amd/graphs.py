@@ -140,10 +140,10 @@ CONFIG_K = {
 }
 CONFIG_SEED = {"c0_uniform": 0, "c1_citation": 1, "c2_social": 2, "c3_copurchase": 3, "c4_rmat": 4,
                "h1_prefattach": 11, "h2_rmat": 12, "h3_grid": 13, "h4_bipartite": 14, "h5_blocks": 15,
-               "h6_uniform100": 16}
+               "h6_uniform100": 16, "h7_groups": 17}
 # Families none of the library's thresholds was chosen on (scale 1 = about 10^8 nonzeros): they check
 # that the plan's choice of strategy holds up on matrices unlike the benchmark's four.
-HELD_OUT = ("h1_prefattach", "h2_rmat", "h3_grid", "h4_bipartite", "h5_blocks", "h6_uniform100")
+HELD_OUT = ("h1_prefattach", "h2_rmat", "h3_grid", "h4_bipartite", "h5_blocks", "h6_uniform100", "h7_groups")
 
 
 def make_graph(name, scale=1.0):

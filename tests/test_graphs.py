@@ -84,7 +84,8 @@ def test_scaled_families_have_their_character(pkg):
 HELD_OUT_SCALE = 0.004  # about 4e5 nonzeros each
 
 
-@pytest.mark.parametrize("name", ["h1_prefattach", "h2_rmat", "h3_grid", "h4_bipartite", "h5_blocks", "h6_uniform100"])
+@pytest.mark.parametrize("name", ["h1_prefattach", "h2_rmat", "h3_grid", "h4_bipartite", "h5_blocks", "h6_uniform100",
+                                  "h7_groups"])
 def test_held_out_families(pkg, name):
     """The families the plan's choice is checked on: valid CSR, sorted rows without duplicates, the same
     matrix from the same name and scale, and the property each one is there for."""
@@ -117,6 +118,15 @@ def test_held_out_families(pkg, name):
         assert g.rows == g.cols and pattern_is_symmetric(g)
         r = np.repeat(np.arange(g.rows), deg)
         assert (np.abs(g.col.astype(np.int64) - r) < 4096).mean() > 0.85
+    elif name == "h7_groups":         # users x items 1 : 2 out of a community graph: the rows kept are the first half
+        assert g.cols == 2 * g.rows and 55 < deg.mean() < 75
+        import scipy.sparse as sp
+        A = sp.csr_matrix((np.ones(g.nnz, np.float32), g.col, g.rowptr), shape=(g.rows, g.cols))
+        square = A[:, : g.rows]       # the kept rows against their own vertices: still a symmetric pattern
+        assert (square != square.T).nnz == 0
+        common = (A[:64] @ A.T).toarray()           # items shared between 64 users and all users
+        np.fill_diagonal(common[:, :64], 0)
+        assert (common.max(axis=1) >= 5).mean() > 0.8   # most users share several items with some other user
     else:                             # exactly 100 entries in every row, anywhere
         assert (deg == 100).all()
         assert np.bincount(g.col, minlength=g.cols).max() < 200

@@ -1,7 +1,7 @@
 """Generator families that none of the plan's thresholds was chosen on (preferential attachment,
 an R-MAT with a flatter quadrant law, a 9-point mesh with random long-range entries, a rectangular
 users x items matrix with Zipf popularity, blocks of mixed sizes along the diagonal, uniformly
-placed nonzeros): the default plan's product against the float64 oracle on slabs of rows, and the
+placed nonzeros, users x items with communities): the default plan's product against the float64 oracle on slabs of rows, and the
 default plan's time against every strategy forced on the same matrix.
 
 Sizes here: about 1.5 M and 12 M nonzeros (the 100 M size of every family is part of the committed
@@ -37,7 +37,8 @@ def bench():
 
 
 @pytest.mark.parametrize("scale", [0.015, 0.12])
-@pytest.mark.parametrize("family", ["h1_prefattach", "h2_rmat", "h3_grid", "h4_bipartite", "h5_blocks", "h6_uniform100"])
+@pytest.mark.parametrize("family", ["h1_prefattach", "h2_rmat", "h3_grid", "h4_bipartite", "h5_blocks", "h6_uniform100",
+                                    "h7_groups"])
 def test_held_out_family(pkg, oracle, gpu, bench, family, scale):
     import torch
     capi, graphs = pkg.capi, pkg.graphs

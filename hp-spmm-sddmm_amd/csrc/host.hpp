@@ -319,8 +319,9 @@ int64_t sort_tile();
 int radix_sort_pairs(int64_t n, uint32_t* d_keys[2], int32_t* d_vals[2], uint32_t* d_hist, uint32_t* d_scan_scratch,
                      int bits, hipStream_t st, int* result);
 // *d_order_out = the row numbers sorted by label[row], rows of one label in increasing order (a new
-// device array of `rows` entries, caller frees).
-int sort_rows_by_label(int64_t rows, const int32_t* d_label, hipStream_t st, int32_t** d_order_out);
+// device array of `rows` entries, caller frees).  Labels lie in [0, label_range).
+int sort_rows_by_label(int64_t rows, const int32_t* d_label, int64_t label_range, hipStream_t st,
+                       int32_t** d_order_out);
 
 // Column popularity, on the device: d_count[c] = nonzeros in column c, and d_ids = the `want` most
 // referenced columns in order of decreasing count (ties by lower index, so the choice is

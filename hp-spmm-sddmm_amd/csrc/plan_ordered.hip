@@ -166,8 +166,9 @@ int build_ordered(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col,
 }
 
 // Label propagation over a graph of n vertices given as CSR adjacency (nnz entries): *d_label_out
-// receives the label of every vertex (a new device array, caller frees), *intra_share_out the share
-// of the entries whose two ends carry one label of at most kClusterMaxSize vertices.
+// receives the label of every vertex (a new device array, caller frees; NULL with status OK when the
+// device has no room for the labels), *intra_share_out the share of the entries whose two ends carry
+// one label of at most kClusterMaxSize vertices.
 constexpr int kClusterMaxSweeps = 16;
 constexpr int32_t kClusterMaxSize = 4096;  // vertices of a cluster that still counts as one a window can profit from
 constexpr int kClusterLookSweeps = 4;           // after this many sweeps the clusters found so far are scored once
@@ -189,9 +190,20 @@ static int cluster_graph(int64_t n, int64_t nnz, const int32_t* d_rowptr, const 
         if (*x) (void)hipFree(*x);
     }
   } guard{{(void**)&d_label, (void**)&d_label_next, (void**)&d_changed}};
-  HPSPMM_HIP(hipMalloc(&d_label, (size_t)n * sizeof(int32_t)));
-  HPSPMM_HIP(hipMalloc(&d_label_next, (size_t)n * sizeof(int32_t)));
-  HPSPMM_HIP(hipMalloc(&d_changed, hpspmm::kClusterCounters * sizeof(uint32_t)));
+  int32_t* d_size = nullptr;
+  struct SizeGuard {
+    int32_t** q;
+    ~SizeGuard() {
+      if (*q) (void)hipFree(*q);
+    }
+  } size_guard{&d_size};
+  if (hipMalloc(&d_label, (size_t)n * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&d_label_next, (size_t)n * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&d_size, (size_t)n * sizeof(int32_t)) != hipSuccess ||
+      hipMalloc(&d_changed, hpspmm::kClusterCounters * sizeof(uint32_t)) != hipSuccess) {
+    (void)hipGetLastError();
+    return HPSPMM_OK;  // no room: no labels, the plan stays what it was
+  }
   std::vector<uint32_t> counters((size_t)hpspmm::kClusterCounters);
   hipLaunchKernelGGL(hpspmm::cluster_init_kernel, dim3((unsigned)ceil_div(n, hpspmm::kBlock)), dim3(hpspmm::kBlock),
                      0, st, n, d_label);
@@ -200,14 +212,6 @@ static int cluster_graph(int64_t n, int64_t nnz, const int32_t* d_rowptr, const 
   // share of the entries that stay inside a cluster small enough for a workgroup's window, from
   // every 4th vertex when there are a million of them (a threshold decision: 1.4 -> 0.4 ms at 2.4 M rows)
   const int64_t score_stride = n >= ((int64_t)1 << 20) ? 4 : 1;
-  int32_t* d_size = nullptr;
-  struct SizeGuard {
-    int32_t** q;
-    ~SizeGuard() {
-      if (*q) (void)hipFree(*q);
-    }
-  } size_guard{&d_size};
-  HPSPMM_HIP(hipMalloc(&d_size, (size_t)n * sizeof(int32_t)));
   auto intra_share = [&](double* share) -> int {
     hipError_t e = hipMemsetAsync(d_size, 0, (size_t)n * sizeof(int32_t), st);
     if (e == hipSuccess) e = hipMemsetAsync(d_changed, 0, counters.size() * sizeof(uint32_t), st);
@@ -311,8 +315,9 @@ int cluster_rows(hpspmm_plan* p, const int32_t* d_rowptr, const int32_t* d_col, 
   }
   // rows ordered by label, the rows of a label in increasing order: a stable sort, hence the same
   // order on every run (the labels of the column vertices, behind those of the rows, are not looked at)
+  if (!d_label) return HPSPMM_OK;
   int32_t* d_order = nullptr;
-  if (int rc = sort_rows_by_label(rows, d_label, st, &d_order)) return rc;
+  if (int rc = sort_rows_by_label(rows, d_label, rows == cols ? rows : rows + cols, st, &d_order)) return rc;
   *d_order_out = d_order;
   return HPSPMM_OK;
 }

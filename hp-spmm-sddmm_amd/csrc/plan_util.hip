@@ -140,7 +140,8 @@ int radix_sort_pairs(int64_t n, uint32_t* d_keys[2], int32_t* d_vals[2], uint32_
   return HPSPMM_OK;
 }
 
-int sort_rows_by_label(int64_t rows, const int32_t* d_label, hipStream_t st, int32_t** d_order_out) {
+int sort_rows_by_label(int64_t rows, const int32_t* d_label, int64_t label_range, hipStream_t st,
+                       int32_t** d_order_out) {
   *d_order_out = nullptr;
   const int64_t n_tiles = ceil_div(rows, hpspmm::kSortTile);
   uint32_t *d_keys[2] = {nullptr, nullptr}, *d_hist = nullptr;
@@ -160,7 +161,7 @@ int sort_rows_by_label(int64_t rows, const int32_t* d_label, hipStream_t st, int
   hipLaunchKernelGGL(hpspmm::label_pairs_kernel, dim3((unsigned)ceil_div(rows, hpspmm::kBlock)), dim3(hpspmm::kBlock), 0,
                      st, rows, d_label, d_keys[0], d_vals[0]);
   int bits = 1;
-  while (bits < 32 && ((int64_t)1 << bits) < rows) ++bits;
+  while (bits < 32 && ((int64_t)1 << bits) < label_range) ++bits;
   int cur = 0;
   for (int shift = 0; shift < bits; shift += 8) {
     hipLaunchKernelGGL(hpspmm::sort_count_kernel, dim3((unsigned)n_tiles), dim3(hpspmm::kBlock), 0, st, rows,

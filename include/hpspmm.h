@@ -139,7 +139,7 @@ typedef struct hpspmm_plan_options {
   int32_t sweep_spin;         /* spin limit of its bounded wait; -1 = never wait */
   int32_t sweep_limit;        /* nonzeros per piece */
   int32_t sweep_no_priorities; /* 1: leave the wavefront priorities alone */
-  int32_t cluster_sweeps;     /* label-propagation sweeps, at most */
+  int32_t cluster_sweeps;     /* label-propagation sweeps, at most (> 0 also keeps the search from ending after four sweeps where no clusters form) */
   int32_t report;             /* 1: plan-time reports on stderr */
   int32_t row_tiles_chunk_log2; /* row tiles at k = 32 / 64 / 128: deal 2^n consecutive groups of tiles to an XCD at a
                                  time instead of one (-1 = one; 0 = the library's choice, by the size) */
